@@ -1,0 +1,153 @@
+/*
+ * torchode_amd -- C ABI of the MI355X-native batch-parallel adaptive explicit
+ * Runge-Kutta solve loop.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream and
+ * allocates nothing.  All pointers are device pointers unless a comment says
+ * otherwise; every array is contiguous (row-major) in the layout given.  An
+ * entry point returns 0 on success and a negative TODE_E_* code otherwise;
+ * tode_last_error() returns a human-readable message for the last failure on
+ * the calling thread.  Work is enqueued on `stream` (a hipStream_t passed as
+ * void*) and is asynchronous with respect to the host.
+ *
+ * "Reference" below is the torchode source tree (martenlienen/torchode 1.0.1);
+ * each declaration names the Python interface it stands in for.
+ */
+#ifndef TORCHODE_AMD_H
+#define TORCHODE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TODE_ABI_VERSION 1
+
+/* floating point type of data (y) and time (t) arrays */
+enum { TODE_F32 = 0, TODE_F64 = 1 };
+/* single step methods: reference single_step_methods/dopri5.py, tsit5.py */
+enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1 };
+/* step size controllers: reference step_size_controllers.py:260 (integral), :554 (PID) */
+enum { TODE_CTRL_INTEGRAL = 0, TODE_CTRL_PID = 1 };
+/* right-hand sides the persistent kernel evaluates itself */
+enum { TODE_TERM_LINEAR_DECAY = 0, TODE_TERM_VAN_DER_POL = 1, TODE_TERM_LORENZ63 = 2 };
+/* per-sample status codes: reference status_codes.py:9-13 */
+enum {
+    TODE_SUCCESS = 0,
+    TODE_GENERAL_ERROR = 1,
+    TODE_REACHED_DT_MIN = 2,
+    TODE_REACHED_MAX_STEPS = 3,
+    TODE_INFINITE_NORM = 4
+};
+/* return codes */
+enum {
+    TODE_OK = 0,
+    TODE_E_INVALID = -1,     /* bad argument (null pointer, negative size, unknown enum) */
+    TODE_E_UNSUPPORTED = -2, /* valid request outside what the kernels are built for */
+    TODE_E_HIP = -3          /* a HIP runtime call failed */
+};
+
+/* Layout of the int32 flag block that tode_solve_builtin fills (device memory, 4 words). */
+enum {
+    TODE_FLAG_MAX_ITERATIONS = 0, /* max over samples of n_steps                        */
+    TODE_FLAG_FIRST_FAILURE = 1,  /* first loop iteration with a non-success status, or */
+                                  /* INT32_MAX                                          */
+    TODE_FLAG_NON_MONOTONE = 2,   /* 1 if some sample's t_eval row is not monotone in   */
+                                  /* its direction of time and no pending mask was given */
+    TODE_FLAG_WORDS = 4
+};
+
+/*
+ * Step size controller parameters.
+ * Replaces the constructor arguments of IntegralController / PIDController
+ * (reference step_size_controllers.py:263-287, 566-596).  atol and rtol are
+ * rounded to float32 before use, as the reference stores them in float32
+ * buffers.  The error norm is the RMS norm (reference :170-181).
+ */
+typedef struct tode_controller {
+    int32_t kind; /* TODE_CTRL_* */
+    int32_t has_dt_min;
+    int32_t has_dt_max;
+    int32_t reserved;
+    double atol, rtol;
+    double pcoeff, icoeff, dcoeff; /* PID only */
+    double safety, factor_min, factor_max;
+    double dt_min, dt_max;
+} tode_controller;
+
+/*
+ * One whole solve of a batch of initial value problems with a built-in
+ * right-hand side, in a single persistent kernel (one sample per lane).
+ *
+ * Replaces AutoDiffAdjoint.solve (reference adjoints.py:42-311) together with
+ * everything it calls per iteration: ExplicitRungeKutta.step
+ * (single_step_methods/runge_kutta.py:226-279), {Integral,PID}Controller.init /
+ * adapt_step_size / merge_states (step_size_controllers.py:333-490, 678-835),
+ * {Dopri5,Tsit5}.build_interpolation and FourthOrderPolynomialInterpolation.evaluate
+ * (dopri5.py:53-60, tsit5.py:123-139, interpolation.py:138-175).
+ *
+ * Each sample runs until it reaches t_end, reports a non-success status, or has
+ * taken `iteration_cap` steps.  The reference couples the samples of a batch in
+ * two ways -- every sample is stepped until the slowest has finished, and the
+ * first non-success status stops the whole batch -- which the caller restores
+ * from the flag block: L = min(first_failure, max_iterations) is the iteration
+ * at which the reference loop would have ended; if L < max_iterations the
+ * caller runs the solve again with iteration_cap = L, then passes L to
+ * tode_finalize_stats.
+ */
+typedef struct tode_solve_args {
+    int32_t dtype;  /* TODE_F32 | TODE_F64, for data and time alike */
+    int32_t method; /* TODE_DOPRI5 | TODE_TSIT5 */
+    int32_t term;   /* TODE_TERM_* */
+    int32_t n_features;        /* F */
+    int32_t n_eval;            /* E; 0 means "report y(t_end) only" */
+    int32_t n_params;          /* P: parameters per sample */
+    int64_t batch;             /* B */
+    int64_t max_steps;         /* < 0: unlimited (reference AutoDiffAdjoint max_steps) */
+    int64_t iteration_cap;     /* < 0: unlimited */
+    double term_scalars[4];    /* batch-uniform RHS constants (Lorenz: sigma, beta) */
+    const void *y0;            /* [B,F] */
+    const void *t_start;       /* [B]   */
+    const void *t_end;         /* [B]   */
+    const void *t_eval;        /* [B,E] or NULL when E == 0 */
+    const void *dt0;           /* [B] user initial step, or NULL to select one */
+    const void *params;        /* [B,P] */
+    void *ys;                  /* out [B,max(E,1),F] */
+    void *y_idle;              /* out [B,F], used only when E == 0: value the reference
+                                  reports for a sample that finished before iteration L */
+    uint8_t *pending;          /* scratch [B,E] bytes, or NULL; needed only for t_eval rows
+                                  that are not monotone in the direction of time */
+    int32_t *n_steps;          /* out [B] */
+    int32_t *n_accepted;       /* out [B] */
+    int32_t *n_initialized;    /* out [B] */
+    int32_t *status_last;      /* out [B] status at the sample's last own iteration */
+    int32_t *status_idle;      /* out [B] status the sample reports in later iterations */
+    int32_t *flags;            /* out [TODE_FLAG_WORDS] */
+} tode_solve_args;
+
+/* ABI version of the loaded library (== TODE_ABI_VERSION of the header it was built from). */
+int tode_abi_version(void);
+
+/* Message for the most recent non-zero return code on this host thread (host pointer). */
+const char *tode_last_error(void);
+
+/* See tode_solve_args. */
+int tode_solve_builtin(const tode_solve_args *args, const tode_controller *controller, void *stream);
+
+/*
+ * Turns the per-sample outputs of tode_solve_builtin into what the reference
+ * returns (adjoints.py:267-309): int64 stats and the final status of every
+ * sample at loop iteration `last_iteration` (L above).  status[b] is
+ * status_last[b] when n_steps[b] == L and status_idle[b] otherwise.  When
+ * n_eval == 0, ys[b] is replaced by y_idle[b] for samples with n_steps[b] < L.
+ */
+int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
+                        const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
+                        int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,
+                        int32_t dtype, int32_t n_features, int32_t n_eval, void *ys, const void *y_idle, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHODE_AMD_H */

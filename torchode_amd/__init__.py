@@ -1,0 +1,28 @@
+"""MI355X-native batch-parallel adaptive Runge-Kutta solver with torchode's API for that path."""
+
+__version__ = "0.1.0"
+
+from . import builtin_terms, workloads
+from .adjoints import AutoDiffAdjoint
+from .builtin_terms import LinearDecay, Lorenz63, VanDerPol
+from .problems import InitialValueProblem
+from .single_step_methods import Dopri5, Tsit5
+from .solution import Solution
+from .status_codes import Status
+from .step_size_controllers import IntegralController, PIDController
+from .terms import ODETerm
+
+__all__ = [
+    "AutoDiffAdjoint",
+    "InitialValueProblem",
+    "Dopri5",
+    "Tsit5",
+    "Solution",
+    "Status",
+    "IntegralController",
+    "PIDController",
+    "ODETerm",
+    "LinearDecay",
+    "VanDerPol",
+    "Lorenz63",
+]

@@ -1,0 +1,131 @@
+"""ctypes binding of libtorchode_amd.so (declared in include/torchode_amd.h).
+
+The library is loaded from this directory; if it is absent it is built once with
+hipcc.  There is no fallback: when the library cannot be loaded, or the tensors
+are not on a HIP device, the callers raise.
+"""
+import ctypes as C
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
+
+ABI_VERSION = 1
+F32, F64 = 0, 1
+DOPRI5, TSIT5 = 0, 1
+CTRL_INTEGRAL, CTRL_PID = 0, 1
+FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_WORDS = 0, 1, 2, 4
+INT32_MAX = 2**31 - 1
+
+DTYPES = {torch.float32: F32, torch.float64: F64}
+
+# every symbol include/torchode_amd.h declares
+EXPORTS = ("tode_abi_version", "tode_last_error", "tode_solve_builtin", "tode_finalize_stats")
+
+
+class Controller(C.Structure):
+    """struct tode_controller"""
+
+    _fields_ = [
+        ("kind", C.c_int32),
+        ("has_dt_min", C.c_int32),
+        ("has_dt_max", C.c_int32),
+        ("reserved", C.c_int32),
+        ("atol", C.c_double),
+        ("rtol", C.c_double),
+        ("pcoeff", C.c_double),
+        ("icoeff", C.c_double),
+        ("dcoeff", C.c_double),
+        ("safety", C.c_double),
+        ("factor_min", C.c_double),
+        ("factor_max", C.c_double),
+        ("dt_min", C.c_double),
+        ("dt_max", C.c_double),
+    ]
+
+
+class SolveArgs(C.Structure):
+    """struct tode_solve_args"""
+
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("method", C.c_int32),
+        ("term", C.c_int32),
+        ("n_features", C.c_int32),
+        ("n_eval", C.c_int32),
+        ("n_params", C.c_int32),
+        ("batch", C.c_int64),
+        ("max_steps", C.c_int64),
+        ("iteration_cap", C.c_int64),
+        ("term_scalars", C.c_double * 4),
+        ("y0", C.c_void_p),
+        ("t_start", C.c_void_p),
+        ("t_end", C.c_void_p),
+        ("t_eval", C.c_void_p),
+        ("dt0", C.c_void_p),
+        ("params", C.c_void_p),
+        ("ys", C.c_void_p),
+        ("y_idle", C.c_void_p),
+        ("pending", C.c_void_p),
+        ("n_steps", C.c_void_p),
+        ("n_accepted", C.c_void_p),
+        ("n_initialized", C.c_void_p),
+        ("status_last", C.c_void_p),
+        ("status_idle", C.c_void_p),
+        ("flags", C.c_void_p),
+    ]
+
+
+_lock = threading.Lock()
+_lib = None
+
+
+def load():
+    """Returns the loaded library, building it first if the file is missing."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            from . import build
+
+            build.build_library(force=True)
+        lib = C.CDLL(LIB_PATH)
+        lib.tode_abi_version.restype = C.c_int
+        lib.tode_last_error.restype = C.c_char_p
+        lib.tode_solve_builtin.restype = C.c_int
+        lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
+        lib.tode_finalize_stats.restype = C.c_int
+        lib.tode_finalize_stats.argtypes = [C.c_int64, C.c_int64] + [C.c_void_p] * 9 + [C.c_int32] * 3 + [C.c_void_p] * 3
+        got = lib.tode_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"libtorchode_amd.so has ABI version {got}, the Python package expects {ABI_VERSION}")
+        _lib = lib
+        return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = load().tode_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed with code {rc}: {msg}")
+
+
+def ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def require_device(*tensors):
+    """The kernels run on a HIP device only; anything else is an error, never a fallback."""
+    for t in tensors:
+        if t is not None and t.device.type != "cuda":
+            raise RuntimeError(
+                "torchode_amd runs on an AMD GPU (HIP device) only; got a tensor on "
+                f"'{t.device}'. There is no CPU implementation to fall back to."
+            )
+
+
+def stream_of(t) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)

@@ -1,0 +1,149 @@
+"""The solve driver (mirrors torchode/adjoints.py:26-319)."""
+from typing import Any, Dict, Optional
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .builtin_terms import BuiltinTerm
+from .problems import InitialValueProblem
+from .single_step_methods import ExplicitRungeKutta
+from .solution import Solution
+from .step_size_controllers import _AdaptiveController
+from .terms import ODETerm
+
+
+class AutoDiffAdjoint(nn.Module):
+    """Solves a batch of initial value problems with per-sample adaptive steps.
+
+    Same constructor and ``solve`` signature as the reference.  The forward solve
+    runs in HIP kernels; it does not record an autograd graph
+    (``backprop_through_step_size_control`` is accepted for compatibility), and
+    inputs that require grad are rejected rather than silently detached.
+    """
+
+    def __init__(
+        self,
+        step_method,
+        step_size_controller,
+        *,
+        max_steps: Optional[int] = None,
+        backprop_through_step_size_control: bool = True,
+    ):
+        super().__init__()
+        self.step_method = step_method
+        self.step_size_controller = step_size_controller
+        self.max_steps = max_steps
+        self.backprop_through_step_size_control = backprop_through_step_size_control
+
+    # ------------------------------------------------------------------ #
+    def solve(
+        self,
+        problem: InitialValueProblem,
+        term: Optional[ODETerm] = None,
+        dt0: Optional[torch.Tensor] = None,
+        args: Any = None,
+    ) -> Solution:
+        term_ = term if term is not None else self.step_method.term
+        assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
+        _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
+        if torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad for t in (problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
+        ):
+            raise RuntimeError(
+                "torchode_amd's solve loop is forward-only; call it under torch.no_grad() or detach the inputs"
+            )
+        if self._persistent_ok(problem, term_):
+            return self._solve_persistent(problem, term_, dt0)
+        raise NotImplementedError("only built-in terms are wired up so far")
+
+    # ------------------------------------------------------------------ #
+    def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
+        m, c = self.step_method, self.step_size_controller
+        return (
+            isinstance(term.f, BuiltinTerm)
+            and not term.with_args
+            and type(m).__name__ in ("Dopri5", "Tsit5")
+            and isinstance(m, ExplicitRungeKutta)
+            and isinstance(c, _AdaptiveController)
+            and c.fusable
+            and problem.data_dtype == problem.time_dtype
+            and problem.data_dtype in _lib.DTYPES
+        )
+
+    def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
+        lib = _lib.load()
+        f: BuiltinTerm = term.f
+        y0 = problem.y0.contiguous()
+        dev, dtype = y0.device, y0.dtype
+        B, F = y0.shape
+        E = problem.n_evaluation_points
+        t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
+        t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
+        params = f.builtin_params().to(device=dev, dtype=dtype)
+        assert params.shape[0] == B, "built-in term parameters do not match the batch size"
+        dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
+
+        ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
+        y_idle = torch.empty((B, F), dtype=dtype, device=dev) if E == 0 else None
+        counters = torch.empty((5, B), dtype=torch.int32, device=dev)
+        flags = torch.empty(_lib.FLAG_WORDS, dtype=torch.int32, device=dev)
+        ctrl = self.step_size_controller.c_struct()
+        stream = _lib.stream_of(y0)
+        scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
+
+        a = _lib.SolveArgs()
+        a.dtype, a.method, a.term = _lib.DTYPES[dtype], self.step_method.method_id, f.builtin_kind
+        a.n_features, a.n_eval, a.n_params, a.batch = F, E, params.shape[1], B
+        a.max_steps = -1 if self.max_steps is None else int(self.max_steps)
+        a.iteration_cap = -1
+        a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
+        a.y0, a.t_start, a.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
+        a.t_eval = None if t_eval is None else t_eval.data_ptr()
+        a.dt0 = None if dt0_ is None else dt0_.data_ptr()
+        a.params = params.data_ptr()
+        a.ys = ys.data_ptr()
+        a.y_idle = None if y_idle is None else y_idle.data_ptr()
+        a.pending = None
+        a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
+        a.flags = flags.data_ptr()
+
+        def run():
+            _lib.check(lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
+            return flags.tolist()  # the one host synchronisation of the solve
+
+        fl = run()
+        pending = None
+        if fl[_lib.FLAG_NON_MONOTONE]:
+            # some t_eval row is not monotone in its direction of time: redo with a pending mask
+            pending = torch.empty((B, E), dtype=torch.uint8, device=dev)
+            a.pending = pending.data_ptr()
+            fl = run()
+        max_iter, first_fail = fl[_lib.FLAG_MAX_ITERATIONS], fl[_lib.FLAG_FIRST_FAILURE]
+        last = min(max_iter, first_fail)
+        if last < max_iter:
+            # a non-success status stops the whole batch at iteration `last`
+            a.iteration_cap = last
+            run()
+
+        out = torch.empty((4, B), dtype=torch.int64, device=dev)
+        rc = lib.tode_finalize_stats(
+            B, last, *(_lib.ptr(counters[i]) for i in range(5)), *(_lib.ptr(out[i]) for i in range(4)),
+            _lib.DTYPES[dtype], F, E, _lib.ptr(ys), _lib.ptr(y_idle), stream,
+        )  # fmt: skip
+        _lib.check(rc, "tode_finalize_stats")
+
+        stats: Dict[str, Any] = {}
+        if term.with_stats:
+            n_init_evals = 2 if dt0 is None else 1
+            stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
+        stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
+        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+        return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+
+    def __repr__(self):
+        return (
+            f"AutoDiffAdjoint(step_method={self.step_method}, "
+            f"step_size_controller={self.step_size_controller}, max_steps={self.max_steps}, "
+            f"backprop_through_step_size_control={self.backprop_through_step_size_control})"
+        )

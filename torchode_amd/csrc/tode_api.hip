@@ -1,0 +1,98 @@
+// extern "C" surface of libtorchode_amd: argument validation, error reporting
+// and the small finalisation kernel.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/torchode_amd.h"
+#include "tode_internal.h"
+
+namespace tode {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t err, const char *what) {
+    if (err == hipSuccess) return TODE_OK;
+    return fail(TODE_E_HIP, "%s: %s", what, hipGetErrorString(err));
+}
+
+template <typename T>
+__global__ void finalize_kernel(long long batch, int last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
+                                const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
+                                int64_t *o_steps, int64_t *o_acc, int64_t *o_init, int64_t *o_status, int n_features,
+                                int n_eval, T *ys, const T *y_idle) {
+    const long long b = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= batch) return;
+    const int ns = n_steps[b];
+    const bool at_last = ns == last_iteration;
+    o_steps[b] = ns;
+    o_acc[b] = n_accepted[b];
+    o_init[b] = n_initialized[b];
+    o_status[b] = at_last ? status_last[b] : status_idle[b];
+    if (n_eval == 0 && !at_last) {
+        for (int f = 0; f < n_features; ++f) ys[b * n_features + f] = y_idle[b * n_features + f];
+    }
+}
+
+}  // namespace tode
+
+extern "C" {
+
+int tode_abi_version(void) { return TODE_ABI_VERSION; }
+
+const char *tode_last_error(void) { return tode::g_error; }
+
+int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void *stream) {
+    using namespace tode;
+    if (!a || !c) return fail(TODE_E_INVALID, "null argument struct");
+    if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
+        return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
+    if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->ys || (a->n_params > 0 && !a->params)))
+        return fail(TODE_E_INVALID, "null problem pointer");
+    if (a->n_eval > 0 && !a->t_eval) return fail(TODE_E_INVALID, "n_eval > 0 but t_eval is null");
+    if (a->n_eval == 0 && a->batch > 0 && !a->y_idle) return fail(TODE_E_INVALID, "n_eval == 0 needs y_idle");
+    if (!a->n_steps || !a->n_accepted || !a->n_initialized || !a->status_last || !a->status_idle || !a->flags)
+        return fail(TODE_E_INVALID, "null output pointer");
+    if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
+    if (a->batch > (int64_t)2147483647 * TODE_BLOCK) return fail(TODE_E_UNSUPPORTED, "batch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (a->dtype == TODE_F32) return solve_builtin_f32(*a, *c, s);
+    if (a->dtype == TODE_F64) return solve_builtin_f64(*a, *c, s);
+    return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+}
+
+int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
+                        const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
+                        int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,
+                        int32_t dtype, int32_t n_features, int32_t n_eval, void *ys, const void *y_idle, void *stream) {
+    using namespace tode;
+    if (batch < 0) return fail(TODE_E_INVALID, "negative batch");
+    if (batch == 0) return TODE_OK;
+    if (!n_steps || !n_accepted || !n_initialized || !status_last || !status_idle || !out_n_steps || !out_n_accepted ||
+        !out_n_initialized || !out_status)
+        return fail(TODE_E_INVALID, "null pointer");
+    if (n_eval == 0 && (!ys || !y_idle)) return fail(TODE_E_INVALID, "n_eval == 0 needs ys and y_idle");
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)((batch + 255) / 256);
+    if (dtype == TODE_F32)
+        hipLaunchKernelGGL(finalize_kernel<float>, dim3(blocks), dim3(256), 0, s, (long long)batch, (int)last_iteration, n_steps,
+                           n_accepted, n_initialized, status_last, status_idle, out_n_steps, out_n_accepted, out_n_initialized,
+                           out_status, n_features, n_eval, (float *)ys, (const float *)y_idle);
+    else if (dtype == TODE_F64)
+        hipLaunchKernelGGL(finalize_kernel<double>, dim3(blocks), dim3(256), 0, s, (long long)batch, (int)last_iteration, n_steps,
+                           n_accepted, n_initialized, status_last, status_idle, out_n_steps, out_n_accepted, out_n_initialized,
+                           out_status, n_features, n_eval, (double *)ys, (const double *)y_idle);
+    else
+        return fail(TODE_E_INVALID, "unknown dtype %d", dtype);
+    return check_hip(hipGetLastError(), "tode_finalize_stats launch");
+}
+
+}  // extern "C"

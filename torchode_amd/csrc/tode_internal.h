@@ -1,0 +1,24 @@
+// Host-side helpers shared by the translation units of libtorchode_amd.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../include/torchode_amd.h"
+
+#define TODE_BLOCK 64  // one wavefront per workgroup: B/64 workgroups spread over all CUs and XCDs
+
+#ifndef TODE_INSTANTIATE_F32
+#define TODE_INSTANTIATE_F32 0
+#endif
+#ifndef TODE_INSTANTIATE_F64
+#define TODE_INSTANTIATE_F64 0
+#endif
+
+namespace tode {
+// Records a formatted message for tode_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...);
+// Maps a HIP error to TODE_E_HIP (recording its string) or returns TODE_OK.
+int check_hip(hipError_t err, const char *what);
+
+int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+}  // namespace tode

@@ -1,0 +1,478 @@
+// Persistent whole-solve kernel: one sample per lane, the complete adaptive
+// Runge-Kutta loop (start step, stages, error estimate, step size control,
+// accept/reject, dense output, counters and status) runs in registers, and the
+// only HBM traffic is the problem in and the solution out.
+//
+// The reference steps the whole batch in lock step (torchode adjoints.py:135-260).
+// Samples are independent except for two batch-wide effects -- the loop runs
+// until the slowest sample has finished, and the first non-success status stops
+// everybody -- so each lane runs its own loop and reports, through the flag
+// block, what the caller needs to restore those two effects.
+#include <hip/hip_runtime.h>
+#include <limits.h>
+
+#include <type_traits>
+
+#include "../../include/torchode_amd.h"
+#include "tode_internal.h"
+#include "tode_math.h"
+
+namespace tode {
+
+// ---------------------------------------------------------------------------
+// Built-in right-hand sides.  Op order is part of the contract: each line is one
+// rounding, matching an eager evaluation of the torch expression in the comment.
+// ---------------------------------------------------------------------------
+template <typename T, int F_> struct LinearDecayTerm {  // (-k) * y
+    static constexpr int F = F_;
+    static constexpr int P = F_;
+    T nk[F_];
+    __device__ __forceinline__ void load(const T *par, const double *) {
+#pragma unroll
+        for (int f = 0; f < F; ++f) nk[f] = -par[f];
+    }
+    __device__ __forceinline__ void operator()(T, const T (&y)[F_], T (&dy)[F_]) const {
+#pragma unroll
+        for (int f = 0; f < F; ++f) dy[f] = nk[f] * y[f];
+    }
+};
+
+template <typename T> struct VanDerPolTerm {  // dx = v ; dv = ((mu*(1-(x*x)))*v)-x
+    static constexpr int F = 2;
+    static constexpr int P = 1;
+    T mu;
+    __device__ __forceinline__ void load(const T *par, const double *) { mu = par[0]; }
+    __device__ __forceinline__ void operator()(T, const T (&y)[2], T (&dy)[2]) const {
+        T x = y[0], v = y[1];
+        T xx = x * x;
+        T om = (T)1 - xx;
+        T m1 = mu * om;
+        T m2 = m1 * v;
+        dy[0] = v;
+        dy[1] = m2 - x;
+    }
+};
+
+template <typename T> struct Lorenz63Term {  // dx=sigma*(y-x); dy=(x*(rho-z))-y; dz=(x*y)-(beta*z)
+    static constexpr int F = 3;
+    static constexpr int P = 1;
+    T rho, sigma, beta;
+    __device__ __forceinline__ void load(const T *par, const double *sc) {
+        rho = par[0];
+        sigma = (T)sc[0];
+        beta = (T)sc[1];
+    }
+    __device__ __forceinline__ void operator()(T, const T (&y)[3], T (&dy)[3]) const {
+        T x = y[0], yy = y[1], z = y[2];
+        T d1 = yy - x;
+        T r1 = rho - z;
+        T xr = x * r1;
+        T xy = x * yy;
+        T bz = beta * z;
+        dy[0] = sigma * d1;
+        dy[1] = xr - yy;
+        dy[2] = xy - bz;
+    }
+};
+
+template <typename T> struct SolveParams {
+    const T *y0, *t_start, *t_end, *t_eval, *dt0, *params;
+    T *ys, *y_idle;
+    uint8_t *pending;
+    int32_t *n_steps, *n_accepted, *n_initialized, *status_last, *status_idle, *flags;
+    long long batch;
+    int n_eval;
+    int max_steps;  // INT_MAX: unlimited
+    int cap;        // INT_MAX: unlimited
+    double scalars[4];
+    CtrlParams<T> cp;
+};
+
+// Start step (step_size_controllers.py:431-490 integral, 776-835 PID; the integral
+// copy maps h0 == 0 to d2 = inf, the PID copy does not).
+template <typename T, int CTRL, typename Term>
+__device__ __forceinline__ T initial_step(const CtrlParams<T> &cp, const Term &rhs, T t0, const T (&y0)[Term::F], T dir, T span,
+                                          T (&f0)[Term::F]) {
+    constexpr int F = Term::F;
+    rhs(t0, y0, f0);
+    T inv[F], w[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) inv[f] = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol);
+#pragma unroll
+    for (int f = 0; f < F; ++f) w[f] = y0[f] * inv[f];
+    T d0 = rms<T, F>(w);
+#pragma unroll
+    for (int f = 0; f < F; ++f) w[f] = f0[f] * inv[f];
+    T d1 = rms<T, F>(w);
+    const T tiny = (T)1e-6;
+    T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? tiny : ((T)0.01 * d0) / d1;
+    h0 = tmin(h0, span);
+    T dh = dir * h0;
+    T y1[F], f1[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) y1[f] = fma_(dh, f0[f], y0[f]);
+    T t1 = fma_(dir, h0, t0);
+    rhs(t1, y1, f1);
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        T df = f1[f] - f0[f];
+        w[f] = df * inv[f];
+    }
+    T d2 = rms<T, F>(w) / h0;
+    if (CTRL == 0 && h0 == (T)0) d2 = (T)__builtin_huge_val();
+    T m = tmax(d1, d2);
+    T h1;
+    if (m <= (T)1e-15) {
+        h1 = tmax(tiny, h0 * (T)1e-3);
+    } else {
+        // python_float / tensor is evaluated by torch as reciprocal(tensor) * python_float
+        T rm = (T)1 / m;
+        h1 = rpow<T>(rm * (T)0.01, 1.0 / 5.0);
+    }
+    return dir * tmin((T)100 * h0, h1);
+}
+
+template <typename T, int METHOD, int CTRL, typename Term>
+__global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> p) {
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    constexpr int F = Term::F;
+    constexpr int P = Term::P;
+    const long long b = (long long)blockIdx.x * TODE_BLOCK + threadIdx.x;
+    const bool live = b < p.batch;
+    const CtrlParams<T> &cp = p.cp;
+    const int E = p.n_eval;
+
+    int my_fail = INT_MAX, my_steps = 0, my_nonmono = 0;
+
+    if (live) {
+        Term rhs;
+        rhs.load(p.params + b * P, p.scalars);
+        T y[F], k[7][F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) y[f] = p.y0[b * F + f];
+        const T ts = p.t_start[b], te = p.t_end[b];
+        const T dir = (te > ts) ? (T)1 : (T)-1;
+        const T tlo = tmin(ts, te), thi = tmax(te, ts);
+        const T *tev = p.t_eval ? p.t_eval + b * E : nullptr;
+        T *ys = p.ys + b * (long long)(E > 0 ? E : 1) * F;
+
+        // evaluation points: a cursor is equivalent to the reference's pending mask when
+        // the row is monotone in the direction of time; otherwise fall back to the mask
+        bool use_mask = false;
+        if (tev) {
+            T prev_te = tev[0];
+            for (int e = 1; e < E; ++e) {
+                T cur = tev[e];
+                if (!(dir > 0 ? cur >= prev_te : cur <= prev_te)) use_mask = true;
+                prev_te = cur;
+            }
+        }
+        uint8_t *pend = nullptr;
+        bool bail = false;
+        if (use_mask) {
+            if (p.pending) {
+                pend = p.pending + b * (long long)E;
+                for (int e = 0; e < E; ++e) pend[e] = 1;
+            } else {
+                my_nonmono = 1;
+                bail = true;
+            }
+        }
+
+        T t = ts, dt;
+        if (p.dt0) {
+            dt = p.dt0[b];
+            rhs(ts, y, k[0]);
+        } else {
+            dt = initial_step<T, CTRL, Term>(cp, rhs, ts, y, dir, abs_(te - ts), k[0]);
+        }
+        dt = tclamp(dt, tlo - t, thi - t);
+        T prev = (T)1, prev_prev = (T)1;
+        int cursor = 0;
+        if (tev && E > 0 && tev[0] == ts) {
+#pragma unroll
+            for (int f = 0; f < F; ++f) ys[f] = y[f];
+            if (pend)
+                pend[0] = 0;
+            else
+                cursor = 1;
+        }
+
+        // next pending evaluation time, kept in a register between iterations
+        T te_next = (tev && cursor < E) ? tev[cursor] : (T)0;
+
+        int n_steps = 0, n_acc = 0, status_last = 0, status_idle = 0;
+        bool idle_pass = false;
+        bool go = !bail && p.cap > 0;
+        while (go) {
+            // ---- stages (runge_kutta.py:255-263) ----
+            const T t0 = t;
+            T y1[F], err[F];
+#pragma unroll
+            for (int i = 1; i < 7; ++i) {
+                T tn = fma_((T)Tab::c[i], dt, t0);
+                T yi[F];
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    T s = 0;
+#pragma unroll
+                    for (int j = 0; j < i; ++j) s = fma_((T)Tab::a[i][j], k[j][f], s);
+                    yi[f] = fma_(dt, s, y[f]);
+                }
+                rhs(tn, yi, k[i]);
+                if (i == 6) {
+#pragma unroll
+                    for (int f = 0; f < F; ++f) y1[f] = yi[f];
+                }
+            }
+            weighted_k<T, F>(dt, Tab::b_err, k, err);
+
+            // ---- step size control (step_size_controllers.py:370-429, 715-774) ----
+            const T ratio = error_ratio<T, F>(cp, y, y1, err);
+            const bool accept = ratio < (T)1;
+            T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, prev_prev);
+            int status = limit_dt<T>(cp, ratio, dt_next);
+
+            const bool running = !idle_pass;
+            const bool move = accept && running;
+            const T t_new = move ? (t0 + dt) : t0;
+            const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+            if (running) {
+                n_steps += 1;
+                n_acc += move ? 1 : 0;
+            }
+            if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
+            const bool last_own = running && (status != 0 || !running_new || n_steps >= p.cap);
+
+            // ---- dense output (adjoints.py:215-234): points passed by the new t ----
+            bool have_q = false;
+            T q[5][F];
+            if (tev) {
+                if (pend) {
+                    for (int e = 0; e < E; ++e) {
+                        if (!pend[e]) continue;
+                        T te_e = tev[e];
+                        if (dir > 0 ? t_new >= te_e : t_new <= te_e) {
+                            if (!have_q) {
+                                quartic<T, F, METHOD>(dt, y, y1, k, q);
+                                have_q = true;
+                            }
+                            T out[F];
+                            quartic_eval<T, F>(q, t0, dt, te_e, out);
+#pragma unroll
+                            for (int f = 0; f < F; ++f) ys[(long long)e * F + f] = out[f];
+                            pend[e] = 0;
+                        }
+                    }
+                } else {
+                    while (cursor < E) {
+                        const T te_e = te_next;
+                        if (!(dir > 0 ? t_new >= te_e : t_new <= te_e)) break;
+                        if (!have_q) {
+                            quartic<T, F, METHOD>(dt, y, y1, k, q);
+                            have_q = true;
+                        }
+                        T out[F];
+                        quartic_eval<T, F>(q, t0, dt, te_e, out);
+#pragma unroll
+                        for (int f = 0; f < F; ++f) ys[(long long)cursor * F + f] = out[f];
+                        ++cursor;
+                        if (cursor < E) te_next = tev[cursor];
+                    }
+                }
+            } else if (last_own || idle_pass) {
+                // no evaluation points (adjoints.py:295-309): the interpolant of the loop's
+                // last iteration evaluated at t_end
+                quartic<T, F, METHOD>(dt, y, y1, k, q);
+                T out[F];
+                quartic_eval<T, F>(q, t0, dt, te, out);
+                T *dst = idle_pass ? (p.y_idle + b * F) : ys;
+#pragma unroll
+                for (int f = 0; f < F; ++f) dst[f] = out[f];
+            }
+
+            // ---- state update (adjoints.py:150-155, 247-255) ----
+            if (move) {
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    y[f] = y1[f];
+                    k[0][f] = k[6][f];
+                }
+            }
+            t = t_new;
+            const T dtn = running_new ? dt_next : dt;
+            dt = tclamp(dtn, tlo - t, thi - t);
+            if (CTRL == 1 && running_new && accept) {
+                prev_prev = prev;
+                prev = ratio;
+            }
+
+            if (idle_pass) {
+                status_idle = status;
+                if (status != 0 && n_steps + 1 < my_fail) my_fail = n_steps + 1;
+                break;
+            }
+            status_last = status;
+            if (status != 0) {
+                my_fail = n_steps;
+                break;
+            }
+            if (!running_new) {
+                // Finished.  Later iterations of the reference loop keep stepping this sample
+                // with the clamped dt; that is observable only through its status and, without
+                // evaluation points, through the end-point interpolant.  Both are trivial
+                // (status 0, value y) unless one of the following holds.
+                bool nontrivial = cp.has_dt_min || !(t == te);
+#pragma unroll
+                for (int f = 0; f < F; ++f) nontrivial = nontrivial || !finite_(k[0][f]) || !finite_(y[f]);
+                if (nontrivial) {
+                    idle_pass = true;
+                    continue;
+                }
+                if (!tev) {
+#pragma unroll
+                    for (int f = 0; f < F; ++f) p.y_idle[b * F + f] = y[f];
+                }
+                break;
+            }
+            if (n_steps >= p.cap) break;
+        }
+
+        int n_init = 1;
+        if (tev) {
+            if (pend) {
+                n_init = 0;
+                while (n_init < E && !pend[n_init]) ++n_init;
+            } else {
+                n_init = cursor;
+            }
+        }
+        p.n_steps[b] = n_steps;
+        p.n_accepted[b] = n_acc;
+        p.n_initialized[b] = n_init;
+        p.status_last[b] = status_last;
+        p.status_idle[b] = status_idle;
+        my_steps = n_steps;
+    }
+
+    // one atomic per wave for the batch-wide facts
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        my_fail = min(my_fail, __shfl_xor(my_fail, off));
+        my_steps = max(my_steps, __shfl_xor(my_steps, off));
+        my_nonmono = max(my_nonmono, __shfl_xor(my_nonmono, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        if (my_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], my_steps);
+        if (my_fail != INT_MAX) atomicMin(&p.flags[TODE_FLAG_FIRST_FAILURE], my_fail);
+        if (my_nonmono) atomicMax(&p.flags[TODE_FLAG_NON_MONOTONE], 1);
+    }
+}
+
+static __global__ void init_flags_kernel(int32_t *flags) {
+    if (threadIdx.x == 0) {
+        flags[TODE_FLAG_MAX_ITERATIONS] = 0;
+        flags[TODE_FLAG_FIRST_FAILURE] = INT_MAX;
+        flags[TODE_FLAG_NON_MONOTONE] = 0;
+        flags[3] = 0;
+    }
+}
+
+template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c) {
+    CtrlParams<T> cp;
+    cp.atol = (T)(float)c.atol;
+    cp.rtol = (T)(float)c.rtol;
+    cp.safety = (T)c.safety;
+    cp.fmin = (T)c.factor_min;
+    cp.fmax = (T)c.factor_max;
+    cp.dt_min = (T)c.dt_min;
+    cp.dt_max = (T)c.dt_max;
+    cp.has_dt_min = c.has_dt_min;
+    cp.has_dt_max = c.has_dt_max;
+    const double order = 5.0;  // convergence order of both pairs (dopri5.py:49-51, tsit5.py:119-121)
+    if (c.kind == TODE_CTRL_INTEGRAL) {
+        cp.e1 = -(1.0 / order);
+        cp.e2 = cp.e3 = 0.0;
+    } else {
+        double k_i = c.icoeff / order, k_p = c.pcoeff / order, k_d = c.dcoeff / order;
+        cp.e1 = -(k_i + k_p + k_d);
+        cp.e2 = k_p + 2 * k_d;
+        cp.e3 = -k_d;
+    }
+    cp.skip2 = ((double)(T)cp.e2 == 0.0);
+    cp.skip3 = ((double)(T)cp.e3 == 0.0);
+    return cp;
+}
+
+template <typename T, int METHOD, int CTRL, typename Term>
+static int launch(const tode_solve_args &a, const tode_controller &c, hipStream_t stream) {
+    SolveParams<T> p;
+    p.y0 = (const T *)a.y0;
+    p.t_start = (const T *)a.t_start;
+    p.t_end = (const T *)a.t_end;
+    p.t_eval = a.n_eval > 0 ? (const T *)a.t_eval : nullptr;
+    p.dt0 = (const T *)a.dt0;
+    p.params = (const T *)a.params;
+    p.ys = (T *)a.ys;
+    p.y_idle = (T *)a.y_idle;
+    p.pending = a.pending;
+    p.n_steps = a.n_steps;
+    p.n_accepted = a.n_accepted;
+    p.n_initialized = a.n_initialized;
+    p.status_last = a.status_last;
+    p.status_idle = a.status_idle;
+    p.flags = a.flags;
+    p.batch = a.batch;
+    p.n_eval = a.n_eval;
+    p.max_steps = (a.max_steps < 0 || a.max_steps >= INT_MAX) ? INT_MAX : (int)a.max_steps;
+    p.cap = (a.iteration_cap < 0 || a.iteration_cap >= INT_MAX) ? INT_MAX : (int)a.iteration_cap;
+    for (int i = 0; i < 4; ++i) p.scalars[i] = a.term_scalars[i];
+    p.cp = make_ctrl<T>(c);
+    const long long blocks = (a.batch + TODE_BLOCK - 1) / TODE_BLOCK;
+    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    if (blocks > 0) hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
+    return check_hip(hipGetLastError(), "tode_solve_builtin launch");
+}
+
+template <typename T, typename Term> static int dispatch_mc(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 0, 0, Term>(a, c, s);
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch<T, 0, 1, Term>(a, c, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 1, 0, Term>(a, c, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch<T, 1, 1, Term>(a, c, s);
+    return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
+}
+
+template <typename T> static int dispatch_term(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
+    switch (a.term) {
+    case TODE_TERM_VAN_DER_POL:
+        if (a.n_features != 2 || a.n_params != 1) return fail(TODE_E_INVALID, "Van der Pol needs F=2, P=1");
+        return dispatch_mc<T, VanDerPolTerm<T>>(a, c, s);
+    case TODE_TERM_LORENZ63:
+        if (a.n_features != 3 || a.n_params != 1) return fail(TODE_E_INVALID, "Lorenz-63 needs F=3, P=1");
+        return dispatch_mc<T, Lorenz63Term<T>>(a, c, s);
+    case TODE_TERM_LINEAR_DECAY:
+        if (a.n_params != a.n_features) return fail(TODE_E_INVALID, "linear decay needs P == F");
+        switch (a.n_features) {
+        case 1: return dispatch_mc<T, LinearDecayTerm<T, 1>>(a, c, s);
+        case 2: return dispatch_mc<T, LinearDecayTerm<T, 2>>(a, c, s);
+        case 3: return dispatch_mc<T, LinearDecayTerm<T, 3>>(a, c, s);
+        case 4: return dispatch_mc<T, LinearDecayTerm<T, 4>>(a, c, s);
+        case 8: return dispatch_mc<T, LinearDecayTerm<T, 8>>(a, c, s);
+        default: return fail(TODE_E_UNSUPPORTED, "linear decay is built for F in {1,2,3,4,8}, got %d", a.n_features);
+        }
+    default:
+        return fail(TODE_E_INVALID, "unknown built-in term %d", a.term);
+    }
+}
+
+int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+
+#if TODE_INSTANTIATE_F32
+int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float>(a, c, s); }
+#endif
+#if TODE_INSTANTIATE_F64
+int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double>(a, c, s); }
+#endif
+
+}  // namespace tode
