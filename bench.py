@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Benchmark of the batch-parallel adaptive RK solve loop on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vdp|lorenz|linear_decay] [--dtype f32|f64]
+
+A "step" is one full solve of the workload's batch (start step, adaptive loop,
+dense output, stats) with inputs resident in HBM.  Prints ONE JSON line.
+
+* value        RK sample-steps per second (sum over samples of attempted steps / wall time);
+               `ivps_per_s` and `equiv_hbm_gbps` are the other two figures of the metric.
+* roofline     dominant kernel = the persistent solve kernel.  `achieved` = algorithmic bytes
+               of one launch (sum_b n_steps[b] * bytes_step + B * bytes_dense) divided by the
+               kernel's average duration, measured with HIP events recorded around the kernel
+               on the stream it is launched on.
+* cpu_baseline the same loop issued as ATen CPU operations (oracle/torch_loop.py, the closest
+               stand-in for running the reference on the host), all host cores, on a bounded
+               prefix of the batch; `cpu_baseline_scalar_c` is the scalar C oracle with OpenMP.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="vdp", choices=["vdp", "lorenz", "linear_decay"])
+    ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
+    ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (samples would shard over the batch axis, see DESIGN.md)")
+
+    import torch
+
+    import torchode_amd as to
+    from torchode_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dtype = {None: None, "f32": torch.float32, "f64": torch.float64}[args.dtype]
+    w = to.workloads.make(args.workload, batch=args.batch, dtype=dtype, device="cuda")
+    dtype = w.y0.dtype
+    B, F = w.y0.shape
+    E = w.t_eval.shape[1]
+    spec = dict(w.controller)
+    kind = spec.pop("kind")
+    ctrl = to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
+    solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl)
+    problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
+    term = to.ODETerm(w.f)
+
+    for _ in range(args.warmup):
+        sol = solver.solve(problem, term)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sol = solver.solve(problem, term)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / args.steps
+
+    assert (sol.status == 0).all(), "benchmark solve did not succeed"
+    sample_steps = int(sol.stats["n_steps"].sum().item())
+    algo_bytes = sample_steps * w.bytes_step + B * w.bytes_dense
+
+    # kernel-only duration: HIP events recorded by the library around the solve kernel
+    _lib.set_kernel_timing(True)
+    kms = []
+    for _ in range(max(5, min(args.steps, 20))):
+        solver.solve(problem, term)
+        kms.append(_lib.last_solve_kernel_ms())
+    _lib.set_kernel_timing(False)
+    kernel_s = sum(kms) / len(kms) / 1e3
+    achieved = algo_bytes / kernel_s / 1e9
+
+    out = {
+        "metric": "RK sample-steps/s (adaptive Tsit5/Dopri5 solve, whole batch)",
+        "value": sample_steps / wall,
+        "unit": "sample-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.float32: "f32", torch.float64: "f64"}[dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name} B={B} F={F} E={E} {w.method}+{kind}",
+            "controller": w.controller,
+            "sample_steps_per_solve": sample_steps,
+            "max_steps_per_sample": int(sol.stats["n_steps"].max().item()),
+        },
+        "ivps_per_s": B / wall,
+        "equiv_hbm_gbps": algo_bytes / wall / 1e9,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "tode::solve_kernel",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
+            "algorithmic_bytes_per_launch": algo_bytes,
+            "bytes_per_sample_step": w.bytes_step,
+            "bytes_dense_per_sample": w.bytes_dense,
+            "kernel_ms": kernel_s * 1e3,
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        out.update(cpu_baselines(args, w, sol))
+    print(json.dumps(out))
+
+
+def cpu_baselines(args, w, sol):
+    """Host-core baselines on a bounded prefix of the same workload."""
+    import torch
+
+    import torchode_amd as to
+    from oracle import c_oracle, torch_loop
+
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    B = w.y0.shape[0]
+    n = min(B, 8192)
+    wc = to.workloads.make(w.name, batch=n, dtype=w.y0.dtype)
+    ctrl = torch_loop.Controller(**wc.controller)
+    ww = to.workloads.make(w.name, batch=min(256, n), dtype=w.y0.dtype)  # warm up
+    torch_loop.solve(ww.f, ww.y0, ww.t_eval, method=ww.method, controller=ctrl)
+    t0 = time.perf_counter()
+    ref = torch_loop.solve(wc.f, wc.y0, wc.t_eval, method=wc.method, controller=ctrl)
+    t_torch = time.perf_counter() - t0
+    steps_n = int(ref["n_steps"].sum())
+
+    name = {"vdp": "vdp", "lorenz": "lorenz", "linear_decay": "linear_decay"}[w.name]
+    nc = min(B, 65536)
+    wc2 = to.workloads.make(w.name, batch=nc, dtype=w.y0.dtype)
+    cfg = c_oracle.make_config(method=wc2.method, term=name, nthreads=cores, **wc2.controller)
+    c_oracle.solve(cfg, ww.f.builtin_params(), ww.y0, ww.t_eval)
+    t0 = time.perf_counter()
+    refc = c_oracle.solve(cfg, wc2.f.builtin_params(), wc2.y0, wc2.t_eval)
+    t_c = time.perf_counter() - t0
+    return {
+        "cpu_baseline": {
+            "value": steps_n / t_torch,
+            "unit": "sample-steps/s",
+            "cores": cores,
+            "kind": "port",
+            "sample": f"first {n} samples of the workload, one eager solve of the ATen-op restatement (torch {torch.__version__})",
+            "seconds": t_torch,
+        },
+        "cpu_baseline_scalar_c": {
+            "value": int(refc["n_steps"].sum()) / t_c,
+            "unit": "sample-steps/s",
+            "cores": cores,
+            "kind": "port",
+            "sample": f"first {nc} samples, one solve of the scalar C oracle (OpenMP over samples)",
+            "seconds": t_c,
+        },
+    }
+
+
+if __name__ == "__main__":
+    main()

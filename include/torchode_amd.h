@@ -147,6 +147,18 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
                         int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,
                         int32_t dtype, int32_t n_features, int32_t n_eval, void *ys, const void *y_idle, void *stream);
 
+/*
+ * Kernel timing for benchmarks and profiling; no counterpart in the reference.
+ * While enabled (per host thread), tode_solve_builtin records a HIP event on
+ * `stream` directly before and directly after its solve kernel.
+ * tode_last_solve_kernel_ms waits for the second event of the most recent
+ * launch made by the calling thread and writes the elapsed milliseconds of
+ * that one kernel; it returns TODE_E_INVALID if timing was off or nothing was
+ * launched.
+ */
+int tode_set_kernel_timing(int enable);
+int tode_last_solve_kernel_ms(float *out_ms);
+
 #ifdef __cplusplus
 }
 #endif

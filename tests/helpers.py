@@ -1,0 +1,66 @@
+"""Shared helpers for the parity tests: solver construction from a workload
+description and comparison against the CPU oracles."""
+import copy
+
+import torch
+
+import torchode_amd as to
+from oracle import c_oracle, torch_loop
+
+TERM_NAME = {to.LinearDecay: "linear_decay", to.VanDerPol: "vdp", to.Lorenz63: "lorenz"}
+
+
+def make_controller(spec: dict, **extra):
+    spec = dict(spec, **extra)
+    kind = spec.pop("kind")
+    return to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
+
+
+def make_method(name: str):
+    return {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[name]()
+
+
+def gpu_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, **ctrl_extra):
+    """Solve on cuda:0 through the public API.  All tensor arguments are CPU tensors."""
+    dev = "cuda"
+    mv = lambda x: None if x is None else x.to(dev)
+    solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **ctrl_extra), max_steps=max_steps)
+    problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
+    return solver.solve(problem, to.ODETerm(copy.deepcopy(f).to(dev)), dt0=mv(dt0))
+
+
+def c_oracle_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, nthreads=8, **ctrl_extra):
+    cfg = c_oracle.make_config(
+        method=method, term=TERM_NAME[type(f)], nthreads=nthreads, max_steps=max_steps, **dict(controller, **ctrl_extra)
+    )
+    return c_oracle.solve(cfg, f.builtin_params(), y0, t_eval, t_start=t_start, t_end=t_end, dt0=dt0)
+
+
+def torch_oracle_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, **ctrl_extra):
+    ctrl = torch_loop.Controller(**dict(controller, **ctrl_extra))
+    return torch_loop.solve(f, y0, t_eval, method=method, controller=ctrl, t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+
+
+def assert_identical(sol, ref, *, check_f_evals=True):
+    """Bit-for-bit: integer stats, status, and every initialised ys row."""
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        got = sol.stats[key].cpu()
+        assert got.dtype == torch.int64
+        assert torch.equal(got, ref[key]), f"{key}: {(got != ref[key]).sum().item()} of {got.numel()} samples differ"
+    assert torch.equal(sol.status.cpu(), ref["status"]), "status differs"
+    if check_f_evals:
+        assert sol.stats["n_f_evals"].device.type == "cpu"
+        assert torch.equal(sol.stats["n_f_evals"], ref["n_f_evals"])
+    ys, rys = sol.ys.cpu(), ref["ys"]
+    assert ys.shape == rys.shape
+    E = ys.shape[1]
+    init = torch.arange(E)[None, :] < ref["n_initialized"][:, None]  # rows the loop wrote
+    a, b = ys[init], rys[init]
+    same = (a == b) | (a.isnan() & b.isnan())
+    assert bool(same.all()), f"ys: {(~same).sum().item()} of {same.numel()} initialised values differ, max abs {(a - b).abs().nan_to_num().max().item():.3e}"
+
+
+def mixed_error(a, b):
+    """max over elements of min(abs error, rel error)."""
+    d = (a - b).abs()
+    return torch.minimum(d, d / b.abs().clamp_min(1e-300)).max().item()

@@ -23,7 +23,14 @@ INT32_MAX = 2**31 - 1
 DTYPES = {torch.float32: F32, torch.float64: F64}
 
 # every symbol include/torchode_amd.h declares
-EXPORTS = ("tode_abi_version", "tode_last_error", "tode_solve_builtin", "tode_finalize_stats")
+EXPORTS = (
+    "tode_abi_version",
+    "tode_last_error",
+    "tode_solve_builtin",
+    "tode_finalize_stats",
+    "tode_set_kernel_timing",
+    "tode_last_solve_kernel_ms",
+)
 
 
 class Controller(C.Structure):
@@ -100,6 +107,10 @@ def load():
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
         lib.tode_finalize_stats.restype = C.c_int
         lib.tode_finalize_stats.argtypes = [C.c_int64, C.c_int64] + [C.c_void_p] * 9 + [C.c_int32] * 3 + [C.c_void_p] * 3
+        lib.tode_set_kernel_timing.restype = C.c_int
+        lib.tode_set_kernel_timing.argtypes = [C.c_int]
+        lib.tode_last_solve_kernel_ms.restype = C.c_int
+        lib.tode_last_solve_kernel_ms.argtypes = [C.POINTER(C.c_float)]
         got = lib.tode_abi_version()
         if got != ABI_VERSION:
             raise RuntimeError(f"libtorchode_amd.so has ABI version {got}, the Python package expects {ABI_VERSION}")
@@ -129,3 +140,15 @@ def require_device(*tensors):
 
 def stream_of(t) -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def set_kernel_timing(enable: bool):
+    """Record HIP events around the solve kernel of subsequent solves made by this thread."""
+    check(load().tode_set_kernel_timing(int(enable)), "tode_set_kernel_timing")
+
+
+def last_solve_kernel_ms() -> float:
+    """Duration of the most recent solve kernel launched by this thread (waits for it)."""
+    out = C.c_float(0.0)
+    check(load().tode_last_solve_kernel_ms(C.byref(out)), "tode_last_solve_kernel_ms")
+    return out.value

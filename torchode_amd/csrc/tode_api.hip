@@ -24,6 +24,25 @@ int check_hip(hipError_t err, const char *what) {
     return fail(TODE_E_HIP, "%s: %s", what, hipGetErrorString(err));
 }
 
+static thread_local bool g_timing = false;
+static thread_local bool g_timed = false;
+static thread_local hipEvent_t g_ev[2] = {nullptr, nullptr};
+
+void timing_before(hipStream_t s) {
+    if (!g_timing) return;
+    if (!g_ev[0]) {
+        (void)hipEventCreate(&g_ev[0]);
+        (void)hipEventCreate(&g_ev[1]);
+    }
+    (void)hipEventRecord(g_ev[0], s);
+}
+
+void timing_after(hipStream_t s) {
+    if (!g_timing) return;
+    (void)hipEventRecord(g_ev[1], s);
+    g_timed = true;
+}
+
 template <typename T>
 __global__ void finalize_kernel(long long batch, int last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
                                 const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
@@ -50,6 +69,21 @@ int tode_abi_version(void) { return TODE_ABI_VERSION; }
 
 const char *tode_last_error(void) { return tode::g_error; }
 
+int tode_set_kernel_timing(int enable) {
+    tode::g_timing = enable != 0;
+    if (!enable) tode::g_timed = false;
+    return TODE_OK;
+}
+
+int tode_last_solve_kernel_ms(float *out_ms) {
+    using namespace tode;
+    if (!out_ms) return fail(TODE_E_INVALID, "null output pointer");
+    if (!g_timing || !g_timed) return fail(TODE_E_INVALID, "kernel timing is off or no solve was launched");
+    int rc = check_hip(hipEventSynchronize(g_ev[1]), "hipEventSynchronize");
+    if (rc) return rc;
+    return check_hip(hipEventElapsedTime(out_ms, g_ev[0], g_ev[1]), "hipEventElapsedTime");
+}
+
 int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void *stream) {
     using namespace tode;
     if (!a || !c) return fail(TODE_E_INVALID, "null argument struct");
@@ -57,9 +91,9 @@ int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void 
         return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
     if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->ys || (a->n_params > 0 && !a->params)))
         return fail(TODE_E_INVALID, "null problem pointer");
-    if (a->n_eval > 0 && !a->t_eval) return fail(TODE_E_INVALID, "n_eval > 0 but t_eval is null");
+    if (a->n_eval > 0 && a->batch > 0 && !a->t_eval) return fail(TODE_E_INVALID, "n_eval > 0 but t_eval is null");
     if (a->n_eval == 0 && a->batch > 0 && !a->y_idle) return fail(TODE_E_INVALID, "n_eval == 0 needs y_idle");
-    if (!a->n_steps || !a->n_accepted || !a->n_initialized || !a->status_last || !a->status_idle || !a->flags)
+    if (!a->flags || (a->batch > 0 && (!a->n_steps || !a->n_accepted || !a->n_initialized || !a->status_last || !a->status_idle)))
         return fail(TODE_E_INVALID, "null output pointer");
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (a->batch > (int64_t)2147483647 * TODE_BLOCK) return fail(TODE_E_UNSUPPORTED, "batch too large");

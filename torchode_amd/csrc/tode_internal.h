@@ -19,6 +19,10 @@ int fail(int code, const char *fmt, ...);
 // Maps a HIP error to TODE_E_HIP (recording its string) or returns TODE_OK.
 int check_hip(hipError_t err, const char *what);
 
+// Event pair around the solve kernel, active only while timing is enabled on this thread.
+void timing_before(hipStream_t s);
+void timing_after(hipStream_t s);
+
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 }  // namespace tode

@@ -430,7 +430,11 @@ static int launch(const tode_solve_args &a, const tode_controller &c, hipStream_
     p.cp = make_ctrl<T>(c);
     const long long blocks = (a.batch + TODE_BLOCK - 1) / TODE_BLOCK;
     hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
-    if (blocks > 0) hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
+    if (blocks > 0) {
+        timing_before(stream);
+        hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
+        timing_after(stream);
+    }
     return check_hip(hipGetLastError(), "tode_solve_builtin launch");
 }
 
