@@ -55,6 +55,8 @@ enum {
                                   /* INT32_MAX                                          */
     TODE_FLAG_NON_MONOTONE = 2,   /* 1 if some sample's t_eval row is not monotone in   */
                                   /* its direction of time and no pending mask was given */
+    TODE_FLAG_NEEDS_GENERAL = 3,  /* tode_solve_builtin_fast only: 1 if the batch needs the  */
+                                  /* general entry point (see there)                     */
     TODE_FLAG_WORDS = 4
 };
 
@@ -148,8 +150,29 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
                         int32_t dtype, int32_t n_features, int32_t n_eval, void *ys, const void *y_idle, void *stream);
 
 /*
+ * The same solve as tode_solve_builtin for the common case, in one kernel launch
+ * with no finalisation step: evaluation points given (n_eval > 0), no dt_min /
+ * dt_max, and a batch in which every sample succeeds.  Uses of `args`: all
+ * inputs, `ys` and `flags`; the int32 per-sample outputs, `y_idle`, `pending`
+ * and `iteration_cap` are ignored.  The reference's int64 stats and status are
+ * written directly (adjoints.py:267-294).
+ *
+ * On return (after stream synchronisation) flags[TODE_FLAG_MAX_ITERATIONS] is
+ * the loop's iteration count, and flags[TODE_FLAG_NEEDS_GENERAL] == 1 means the
+ * batch left the common case (a non-success status, max_steps reached, a t_eval
+ * row that is not monotone in its direction of time, or a sample that ended
+ * past t_end); every output is then unspecified and the caller must repeat the
+ * solve with tode_solve_builtin.  Results are bit-identical to
+ * tode_solve_builtin + tode_finalize_stats whenever the flag stays 0.
+ * Returns TODE_E_UNSUPPORTED for n_eval == 0, dt_min / dt_max, or n_eval too
+ * large for on-chip staging.
+ */
+int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
+                            int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream);
+
+/*
  * Kernel timing for benchmarks and profiling; no counterpart in the reference.
- * While enabled (per host thread), tode_solve_builtin records a HIP event on
+ * While enabled (per host thread), tode_solve_builtin and tode_solve_builtin_fast record a HIP event on
  * `stream` directly before and directly after its solve kernel.
  * tode_last_solve_kernel_ms waits for the second event of the most recent
  * launch made by the calling thread and writes the elapsed milliseconds of

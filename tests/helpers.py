@@ -20,11 +20,12 @@ def make_method(name: str):
     return {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[name]()
 
 
-def gpu_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, **ctrl_extra):
+def gpu_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, fast=True, **ctrl_extra):
     """Solve on cuda:0 through the public API.  All tensor arguments are CPU tensors."""
     dev = "cuda"
     mv = lambda x: None if x is None else x.to(dev)
     solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **ctrl_extra), max_steps=max_steps)
+    solver.use_fast_path = fast
     problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
     return solver.solve(problem, to.ODETerm(copy.deepcopy(f).to(dev)), dt0=mv(dt0))
 

@@ -16,11 +16,12 @@ pytestmark = pytest.mark.gpu
 F32, F64 = torch.float32, torch.float64
 
 
+@pytest.mark.parametrize("fast", [True, False], ids=["fast", "general"])
 @pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
 @pytest.mark.parametrize("name,batch", [("linear_decay", 256), ("vdp", 4096), ("lorenz", 4096)])
-def test_workload_matches_oracle_bit_for_bit(name, batch, dtype):
+def test_workload_matches_oracle_bit_for_bit(name, batch, dtype, fast):
     w = to.workloads.make(name, batch=batch, dtype=dtype)
-    sol = gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    sol = gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast=fast)
     ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
     assert_identical(sol, ref)
     assert sol.ts.data_ptr() != 0 and sol.ys.dtype == dtype
@@ -40,13 +41,23 @@ def test_workload_matches_oracle_bit_for_bit(name, batch, dtype):
 )
 def test_every_method_controller_pair(method, controller, dtype):
     w = to.workloads.make("vdp", batch=1024, dtype=dtype)
-    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller), c_oracle_solve(w.f, w.y0, w.t_eval, method, controller))
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, method, controller)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller, fast=False), ref)
 
 
 @pytest.mark.parametrize("batch", [1, 63, 65, 129])
 def test_ragged_batches(batch):
     w = to.workloads.make("lorenz", batch=batch, dtype=F32)
-    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller), c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller))
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast=False), ref)
+    w = to.workloads.make("vdp", batch=batch, dtype=F64)  # dense output staged through LDS vs written directly
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller), ref)
+    w = to.workloads.make("vdp", batch=batch, dtype=F32)
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller), ref)
 
 
 def test_ts_aliases_t_eval_and_inputs_untouched():

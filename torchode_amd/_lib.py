@@ -17,7 +17,7 @@ ABI_VERSION = 1
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
-FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_WORDS = 0, 1, 2, 4
+FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_NEEDS_GENERAL, FLAG_WORDS = 0, 1, 2, 3, 4
 INT32_MAX = 2**31 - 1
 
 DTYPES = {torch.float32: F32, torch.float64: F64}
@@ -27,6 +27,7 @@ EXPORTS = (
     "tode_abi_version",
     "tode_last_error",
     "tode_solve_builtin",
+    "tode_solve_builtin_fast",
     "tode_finalize_stats",
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
@@ -105,6 +106,8 @@ def load():
         lib.tode_last_error.restype = C.c_char_p
         lib.tode_solve_builtin.restype = C.c_int
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
+        lib.tode_solve_builtin_fast.restype = C.c_int
+        lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
         lib.tode_finalize_stats.restype = C.c_int
         lib.tode_finalize_stats.argtypes = [C.c_int64, C.c_int64] + [C.c_void_p] * 9 + [C.c_int32] * 3 + [C.c_void_p] * 3
         lib.tode_set_kernel_timing.restype = C.c_int

@@ -35,6 +35,9 @@ class AutoDiffAdjoint(nn.Module):
         self.step_size_controller = step_size_controller
         self.max_steps = max_steps
         self.backprop_through_step_size_control = backprop_through_step_size_control
+        # Set to False to route built-in terms through the general whole-solve kernel only
+        # (same results; used by the tests to compare the two kernels).
+        self.use_fast_path = True
 
     # ------------------------------------------------------------------ #
     def solve(
@@ -108,6 +111,26 @@ class AutoDiffAdjoint(nn.Module):
         a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
         a.flags = flags.data_ptr()
 
+        stats: Dict[str, Any] = {}
+        n_init_evals = 2 if dt0 is None else 1
+        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+
+        # Common case first: one kernel, int64 stats written directly.  It reports through the
+        # flag block when the batch needs the general kernel (which handles every case).
+        if self.use_fast_path and E > 0 and not ctrl.has_dt_min and not ctrl.has_dt_max and E * y0.element_size() <= 1024:
+            out = torch.empty((4, B), dtype=torch.int64, device=dev)
+            rc = lib.tode_solve_builtin_fast(
+                _lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream
+            )
+            _lib.check(rc, "tode_solve_builtin_fast")
+            fl = flags.tolist()  # the one host synchronisation of the solve
+            if not fl[_lib.FLAG_NEEDS_GENERAL]:
+                if term.with_stats:
+                    last = fl[_lib.FLAG_MAX_ITERATIONS]
+                    stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
+                stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
+                return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+
         def run():
             _lib.check(lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
             return flags.tolist()  # the one host synchronisation of the solve
@@ -133,12 +156,9 @@ class AutoDiffAdjoint(nn.Module):
         )  # fmt: skip
         _lib.check(rc, "tode_finalize_stats")
 
-        stats: Dict[str, Any] = {}
         if term.with_stats:
-            n_init_evals = 2 if dt0 is None else 1
             stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
-        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
         return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
 
     def __repr__(self):

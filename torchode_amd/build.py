@@ -37,6 +37,8 @@ UNITS = [
     ("tode_api.hip", "tode_api.o", []),
     ("tode_persistent.hip", "tode_persistent_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_persistent.hip", "tode_persistent_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
+    ("tode_fast.hip", "tode_fast_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
+    ("tode_fast.hip", "tode_fast_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
 ]
 
 

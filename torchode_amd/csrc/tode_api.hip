@@ -103,6 +103,25 @@ int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void 
     return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
 }
 
+int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,
+                            int64_t *st, void *stream) {
+    using namespace tode;
+    if (!a || !c) return fail(TODE_E_INVALID, "null argument struct");
+    if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
+        return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
+    if (a->n_eval == 0) return fail(TODE_E_UNSUPPORTED, "the fast entry point needs evaluation points");
+    if (c->has_dt_min || c->has_dt_max) return fail(TODE_E_UNSUPPORTED, "the fast entry point does not take dt_min / dt_max");
+    if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
+    if (!a->flags) return fail(TODE_E_INVALID, "null flags pointer");
+    if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->t_eval || !a->ys || (a->n_params > 0 && !a->params) || !ns || !na || !ni || !st))
+        return fail(TODE_E_INVALID, "null pointer");
+    if (a->batch > (int64_t)2147483647 * 64) return fail(TODE_E_UNSUPPORTED, "batch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (a->dtype == TODE_F32) return solve_fast_f32(*a, *c, ns, na, ni, st, s);
+    if (a->dtype == TODE_F64) return solve_fast_f64(*a, *c, ns, na, ni, st, s);
+    return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+}
+
 int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
                         const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
                         int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,

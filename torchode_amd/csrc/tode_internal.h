@@ -25,4 +25,6 @@ void timing_after(hipStream_t s);
 
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
+int solve_fast_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 }  // namespace tode

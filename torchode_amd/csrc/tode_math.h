@@ -97,6 +97,54 @@ __device__ __forceinline__ double pow_core(double x, double p) {
     return __builtin_ldexp(v, (int)n);
 }
 
+// The two halves of pow_core for arguments that need none of its special cases:
+// log2_normal(x) for a positive, finite, normal x, and exp2_of(y) for |y| <= 1016.
+// pow_core(x, p) == exp2_of(p * log2_normal(x)) bit for bit on that domain, which lets
+// a caller reuse one logarithm for several exponents.
+__device__ __forceinline__ double log2_normal(double x) {
+    const unsigned hi = (unsigned)__double2hiint(x);
+    int e = (int)((hi >> 20) & 0x7ff) - 1023;
+    double m = __hiloint2double((int)((hi & 0x000fffffu) | 0x3ff00000u), __double2loint(x));
+    const bool big = m > 1.4142135623730951;
+    m = big ? m * 0.5 : m;
+    e = big ? e + 1 : e;
+    double s = (m - 1.0) / (m + 1.0);
+    double z = s * s;
+    double q = 2.0 / 21.0;
+    q = __builtin_fma(q, z, 2.0 / 19.0);
+    q = __builtin_fma(q, z, 2.0 / 17.0);
+    q = __builtin_fma(q, z, 2.0 / 15.0);
+    q = __builtin_fma(q, z, 2.0 / 13.0);
+    q = __builtin_fma(q, z, 2.0 / 11.0);
+    q = __builtin_fma(q, z, 2.0 / 9.0);
+    q = __builtin_fma(q, z, 2.0 / 7.0);
+    q = __builtin_fma(q, z, 2.0 / 5.0);
+    q = __builtin_fma(q, z, 2.0 / 3.0);
+    double s3 = s * z;
+    double lnm = __builtin_fma(s3, q, 2.0 * s);
+    return __builtin_fma(lnm, 1.4426950408889634, (double)e);
+}
+
+__device__ __forceinline__ double exp2_of(double y) {
+    double n = __builtin_rint(y);
+    double r = (y - n) * 0.6931471805599453;
+    double v = 1.0 / 6227020800.0;
+    v = __builtin_fma(v, r, 1.0 / 479001600.0);
+    v = __builtin_fma(v, r, 1.0 / 39916800.0);
+    v = __builtin_fma(v, r, 1.0 / 3628800.0);
+    v = __builtin_fma(v, r, 1.0 / 362880.0);
+    v = __builtin_fma(v, r, 1.0 / 40320.0);
+    v = __builtin_fma(v, r, 1.0 / 5040.0);
+    v = __builtin_fma(v, r, 1.0 / 720.0);
+    v = __builtin_fma(v, r, 1.0 / 120.0);
+    v = __builtin_fma(v, r, 1.0 / 24.0);
+    v = __builtin_fma(v, r, 1.0 / 6.0);
+    v = __builtin_fma(v, r, 0.5);
+    v = __builtin_fma(v, r, 1.0);
+    v = __builtin_fma(v, r, 1.0);
+    return __builtin_ldexp(v, (int)n);
+}
+
 // Tensor ** python_float: the exponent is rounded to the tensor dtype first.
 template <typename T> __device__ __forceinline__ T rpow(T x, double p) { return (T)pow_core((double)x, (double)(T)p); }
 

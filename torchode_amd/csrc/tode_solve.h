@@ -1,0 +1,193 @@
+// Pieces shared by the whole-solve kernels: built-in right-hand sides, kernel
+// parameter block and the start-step selection.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <limits.h>
+
+#include <type_traits>
+
+#include "../../include/torchode_amd.h"
+#include "tode_internal.h"
+#include "tode_math.h"
+
+namespace tode {
+
+
+// ---------------------------------------------------------------------------
+// Built-in right-hand sides.  Op order is part of the contract: each line is one
+// rounding, matching an eager evaluation of the torch expression in the comment.
+// ---------------------------------------------------------------------------
+template <typename T, int F_> struct LinearDecayTerm {  // (-k) * y
+    static constexpr int F = F_;
+    static constexpr int P = F_;
+    T nk[F_];
+    __device__ __forceinline__ void load(const T *par, const double *) {
+#pragma unroll
+        for (int f = 0; f < F; ++f) nk[f] = -par[f];
+    }
+    __device__ __forceinline__ void operator()(T, const T (&y)[F_], T (&dy)[F_]) const {
+#pragma unroll
+        for (int f = 0; f < F; ++f) dy[f] = nk[f] * y[f];
+    }
+};
+
+template <typename T> struct VanDerPolTerm {  // dx = v ; dv = ((mu*(1-(x*x)))*v)-x
+    static constexpr int F = 2;
+    static constexpr int P = 1;
+    T mu;
+    __device__ __forceinline__ void load(const T *par, const double *) { mu = par[0]; }
+    __device__ __forceinline__ void operator()(T, const T (&y)[2], T (&dy)[2]) const {
+        T x = y[0], v = y[1];
+        T xx = x * x;
+        T om = (T)1 - xx;
+        T m1 = mu * om;
+        T m2 = m1 * v;
+        dy[0] = v;
+        dy[1] = m2 - x;
+    }
+};
+
+template <typename T> struct Lorenz63Term {  // dx=sigma*(y-x); dy=(x*(rho-z))-y; dz=(x*y)-(beta*z)
+    static constexpr int F = 3;
+    static constexpr int P = 1;
+    T rho, sigma, beta;
+    __device__ __forceinline__ void load(const T *par, const double *sc) {
+        rho = par[0];
+        sigma = (T)sc[0];
+        beta = (T)sc[1];
+    }
+    __device__ __forceinline__ void operator()(T, const T (&y)[3], T (&dy)[3]) const {
+        T x = y[0], yy = y[1], z = y[2];
+        T d1 = yy - x;
+        T r1 = rho - z;
+        T xr = x * r1;
+        T xy = x * yy;
+        T bz = beta * z;
+        dy[0] = sigma * d1;
+        dy[1] = xr - yy;
+        dy[2] = xy - bz;
+    }
+};
+
+template <typename T> struct SolveParams {
+    const T *y0, *t_start, *t_end, *t_eval, *dt0, *params;
+    T *ys, *y_idle;
+    uint8_t *pending;
+    int32_t *n_steps, *n_accepted, *n_initialized, *status_last, *status_idle, *flags;
+    long long batch;
+    int n_eval;
+    int max_steps;  // INT_MAX: unlimited
+    int cap;        // INT_MAX: unlimited
+    double scalars[4];
+    CtrlParams<T> cp;
+};
+
+// Start step (step_size_controllers.py:431-490 integral, 776-835 PID; the integral
+// copy maps h0 == 0 to d2 = inf, the PID copy does not).
+template <typename T, int CTRL, typename Term>
+__device__ __forceinline__ T initial_step(const CtrlParams<T> &cp, const Term &rhs, T t0, const T (&y0)[Term::F], T dir, T span,
+                                          T (&f0)[Term::F]) {
+    constexpr int F = Term::F;
+    rhs(t0, y0, f0);
+    T inv[F], w[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) inv[f] = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol);
+#pragma unroll
+    for (int f = 0; f < F; ++f) w[f] = y0[f] * inv[f];
+    T d0 = rms<T, F>(w);
+#pragma unroll
+    for (int f = 0; f < F; ++f) w[f] = f0[f] * inv[f];
+    T d1 = rms<T, F>(w);
+    const T tiny = (T)1e-6;
+    T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? tiny : ((T)0.01 * d0) / d1;
+    h0 = tmin(h0, span);
+    T dh = dir * h0;
+    T y1[F], f1[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) y1[f] = fma_(dh, f0[f], y0[f]);
+    T t1 = fma_(dir, h0, t0);
+    rhs(t1, y1, f1);
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        T df = f1[f] - f0[f];
+        w[f] = df * inv[f];
+    }
+    T d2 = rms<T, F>(w) / h0;
+    if (CTRL == 0 && h0 == (T)0) d2 = (T)__builtin_huge_val();
+    T m = tmax(d1, d2);
+    T h1;
+    if (m <= (T)1e-15) {
+        h1 = tmax(tiny, h0 * (T)1e-3);
+    } else {
+        // python_float / tensor is evaluated by torch as reciprocal(tensor) * python_float
+        T rm = (T)1 / m;
+        h1 = rpow<T>(rm * (T)0.01, 1.0 / 5.0);
+    }
+    return dir * tmin((T)100 * h0, h1);
+}
+
+
+// Controller parameters in the working type from the ABI struct.
+template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c) {
+    CtrlParams<T> cp;
+    cp.atol = (T)(float)c.atol;
+    cp.rtol = (T)(float)c.rtol;
+    cp.safety = (T)c.safety;
+    cp.fmin = (T)c.factor_min;
+    cp.fmax = (T)c.factor_max;
+    cp.dt_min = (T)c.dt_min;
+    cp.dt_max = (T)c.dt_max;
+    cp.has_dt_min = c.has_dt_min;
+    cp.has_dt_max = c.has_dt_max;
+    const double order = 5.0;  // convergence order of both pairs (dopri5.py:49-51, tsit5.py:119-121)
+    if (c.kind == TODE_CTRL_INTEGRAL) {
+        cp.e1 = -(1.0 / order);
+        cp.e2 = cp.e3 = 0.0;
+    } else {
+        double k_i = c.icoeff / order, k_p = c.pcoeff / order, k_d = c.dcoeff / order;
+        cp.e1 = -(k_i + k_p + k_d);
+        cp.e2 = k_p + 2 * k_d;
+        cp.e3 = -k_d;
+    }
+    cp.skip2 = ((double)(T)cp.e2 == 0.0);
+    cp.skip3 = ((double)(T)cp.e3 == 0.0);
+    return cp;
+}
+
+template <typename T> static SolveParams<T> make_params(const tode_solve_args &a, const tode_controller &c) {
+    SolveParams<T> p;
+    p.y0 = (const T *)a.y0;
+    p.t_start = (const T *)a.t_start;
+    p.t_end = (const T *)a.t_end;
+    p.t_eval = a.n_eval > 0 ? (const T *)a.t_eval : nullptr;
+    p.dt0 = (const T *)a.dt0;
+    p.params = (const T *)a.params;
+    p.ys = (T *)a.ys;
+    p.y_idle = (T *)a.y_idle;
+    p.pending = a.pending;
+    p.n_steps = a.n_steps;
+    p.n_accepted = a.n_accepted;
+    p.n_initialized = a.n_initialized;
+    p.status_last = a.status_last;
+    p.status_idle = a.status_idle;
+    p.flags = a.flags;
+    p.batch = a.batch;
+    p.n_eval = a.n_eval;
+    p.max_steps = (a.max_steps < 0 || a.max_steps >= INT_MAX) ? INT_MAX : (int)a.max_steps;
+    p.cap = (a.iteration_cap < 0 || a.iteration_cap >= INT_MAX) ? INT_MAX : (int)a.iteration_cap;
+    for (int i = 0; i < 4; ++i) p.scalars[i] = a.term_scalars[i];
+    p.cp = make_ctrl<T>(c);
+    return p;
+}
+
+// Resets the flag block; launched in front of every solve kernel.
+static __global__ void init_flags_kernel(int32_t *flags) {
+    if (threadIdx.x == 0) {
+        flags[TODE_FLAG_MAX_ITERATIONS] = 0;
+        flags[TODE_FLAG_FIRST_FAILURE] = INT_MAX;
+        flags[TODE_FLAG_NON_MONOTONE] = 0;
+        flags[TODE_FLAG_NEEDS_GENERAL] = 0;
+    }
+}
+
+}  // namespace tode
