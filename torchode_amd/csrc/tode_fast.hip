@@ -26,7 +26,8 @@ template <typename T> struct FastOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
 };
 
-template <typename T, int METHOD, int CTRL, typename Term, bool STAGE_YS>
+// NHIST: how many history factors the controller multiplies in (0 integral, 1 PI, 2 PID).
+template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_YS>
 __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, const FastOut<T> o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
@@ -91,8 +92,8 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         dt = initial_step<T, CTRL, Term>(cp, rhs, ts, y, dir, abs_(te - ts), k[0]);
     }
     dt = tclamp(dt, tlo - t, thi - t);
-    T prev = (T)1, prev_prev = (T)1;
-    double l2_prev = 0.0, l2_pprev = 0.0;  // log2 of prev / prev_prev (log2(1) = 0)
+    // log2 of the previous two accepted error ratios (both start at 1, log2(1) = 0)
+    double l2_prev = 0.0, l2_pprev = 0.0;
     int cursor = 0;
     T *ys_g = p.ys + bs * (long long)EF;
     if (te_s[lane] == ts) {
@@ -105,7 +106,10 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         }
         cursor = 1;
     }
-    T te_next = te_s[(cursor < E ? cursor : E - 1) * 64 + lane];
+    // direction-normalised times: multiplying by +-1 is exact, so dir*a >= dir*b decides
+    // "a has reached b in the direction of time" without a branch
+    T dte_next = dir * te_s[(cursor < E ? cursor : E - 1) * 64 + lane];
+    const T dte_end = dir * te;
 
     int n_steps = 0, n_acc = 0;
     bool active = live && !bail;
@@ -132,7 +136,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
                 for (int f = 0; f < F; ++f) y1[f] = yi[f];
             }
         }
-        weighted_k<T, F>(dt, Tab::b_err, k, err);
+        weighted_k<T, F, Tab, -1>(dt, k, err);
 
         // ---- step size control (step_size_controllers.py:370-429, 715-774) ----
         const T ratio = error_ratio<T, F>(cp, y, y1, err);
@@ -141,29 +145,26 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         const bool sane = ratio > (T)0 && ratio < (T)__builtin_huge_val();
         const double l2 = log2_normal(sane ? (double)ratio : 1.0);
         T factor = cp.safety * (T)exp2_of(e1 * l2);
-        if (CTRL == 1) {
-            T f2 = cp.skip2 ? (T)1 : (T)exp2_of(e2 * l2_prev);
-            T f3 = cp.skip3 ? (T)1 : (T)exp2_of(e3 * l2_pprev);
-            factor = factor * f2;
-            factor = factor * f3;
-        }
+        if (NHIST >= 1) factor = factor * (T)exp2_of(e2 * l2_prev);
+        if (NHIST >= 2) factor = factor * (T)exp2_of(e3 * l2_pprev);
         factor = tclamp(factor, cp.fmin, cp.fmax);
         const T dt_next = dt * factor;
 
         const bool move = accept && active;
         const T t_new = move ? (t0 + dt) : t0;
-        const bool running_new = fwd ? (t_new < te) : (t_new > te);
+        const T dt_new = dir * t_new;
+        const bool running_new = dt_new < dte_end;
         n_steps += active ? 1 : 0;
         n_acc += move ? 1 : 0;
 
         // ---- dense output (adjoints.py:215-234) ----
-        bool hit = active && cursor < E && (fwd ? t_new >= te_next : t_new <= te_next);
+        bool hit = active && cursor < E && dt_new >= dte_next;
         if (__any(hit)) {
             T q[5][F];
             quartic<T, F, METHOD>(dt, y, y1, k, q);
             do {
                 T out[F];
-                quartic_eval<T, F>(q, t0, dt, te_next, out);
+                quartic_eval<T, F>(q, t0, dt, dir * dte_next, out);
                 if (hit) {
 #pragma unroll
                     for (int f = 0; f < F; ++f) {
@@ -172,10 +173,11 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
                         else
                             ys_g[cursor * F + f] = out[f];
                     }
-                    cursor += 1;
-                    te_next = te_s[(cursor < E ? cursor : E - 1) * 64 + lane];
                 }
-                hit = hit && cursor < E && (fwd ? t_new >= te_next : t_new <= te_next);
+                cursor += hit ? 1 : 0;
+                const T nxt = dir * te_s[(cursor < E ? cursor : E - 1) * 64 + lane];
+                dte_next = hit ? nxt : dte_next;
+                hit = hit && cursor < E && dt_new >= dte_next;
             } while (__any(hit));
         }
 
@@ -186,30 +188,27 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
             k[0][f] = move ? k[6][f] : k[0][f];
         }
         t = t_new;
-        if (active) {
+        {
             const T dtn = running_new ? dt_next : dt;
-            dt = tclamp(dtn, tlo - t, thi - t);
+            const T dtc = tclamp(dtn, tlo - t, thi - t);
+            dt = active ? dtc : dt;
         }
-        if (CTRL == 1) {
+        if (NHIST >= 1) {
             const bool shift = active && running_new && accept;
-            prev_prev = shift ? prev : prev_prev;
-            l2_pprev = shift ? l2_prev : l2_pprev;
-            prev = shift ? ratio : prev;
+            if (NHIST >= 2) l2_pprev = shift ? l2_prev : l2_pprev;
             l2_prev = shift ? l2 : l2_prev;
         }
-        if (active) {
-            if (!sane || n_steps >= p.max_steps) {
-                bail = true;  // non-finite error ratio or max_steps reached
-                active = false;
-            } else if (!running_new) {
-                active = false;
-                // a sample that lands past t_end, or whose derivative at the end is not
-                // finite, shows up in later iterations of the reference loop
-                bool odd = !(t == te);
+        {
+            // non-finite error ratio or max_steps reached: not the common case
+            const bool failed = active && (!sane || n_steps >= p.max_steps);
+            const bool finished = active && !failed && !running_new;
+            // a sample that lands past t_end, or whose derivative at the end is not finite,
+            // shows up in later iterations of the reference loop
+            bool odd = !(t == te);
 #pragma unroll
-                for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
-                bail = bail || odd;
-            }
+            for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
+            bail = bail || failed || (finished && odd);
+            active = active && !failed && running_new;
         }
     }
 
@@ -270,11 +269,21 @@ static int launch_fast(const tode_solve_args &a, const tode_controller &c, const
     const size_t need_te = lds_bytes(a.n_eval, Term::F, sizeof(T), false);
     const size_t need_all = lds_bytes(a.n_eval, Term::F, sizeof(T), true);
     if (need_te > 64 * 1024) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the fast kernel", a.n_eval);
+    const CtrlParams<T> &cp = p.cp;
+    const int nhist = CTRL == 0 ? 0 : (cp.skip3 ? 1 : 2);
+    const bool stage = need_all <= budget;
+    const size_t lds = stage ? need_all : need_te;
+    const dim3 grid((unsigned)blocks), block(64);
     timing_before(stream);
-    if (need_all <= budget)
-        hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, Term, true>), dim3((unsigned)blocks), dim3(64), need_all, stream, p, o);
-    else
-        hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, Term, false>), dim3((unsigned)blocks), dim3(64), need_te, stream, p, o);
+#define TODE_FAST_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
+    if (nhist == 0) {
+        if (stage) TODE_FAST_LAUNCH(0, true); else TODE_FAST_LAUNCH(0, false);
+    } else if (nhist == 1) {
+        if (stage) TODE_FAST_LAUNCH(CTRL == 0 ? 0 : 1, true); else TODE_FAST_LAUNCH(CTRL == 0 ? 0 : 1, false);
+    } else {
+        if (stage) TODE_FAST_LAUNCH(CTRL == 0 ? 0 : 2, true); else TODE_FAST_LAUNCH(CTRL == 0 ? 0 : 2, false);
+    }
+#undef TODE_FAST_LAUNCH
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }

@@ -28,9 +28,17 @@ template <> __device__ __forceinline__ double abs_<double>(double a) { return __
 
 template <typename T> __device__ __forceinline__ bool finite_(T a) { return abs_(a) < __builtin_huge_val(); }
 
-// torch.maximum / torch.minimum / torch.clamp: NaN in any operand gives NaN.
-template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return (a != a) ? a : ((b != b) ? b : (a > b ? a : b)); }
-template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return (a != a) ? a : ((b != b) ? b : (a < b ? a : b)); }
+// torch.maximum / torch.minimum / torch.clamp: NaN in any operand gives NaN.  Written as
+// max/min plus one unordered-compare select so that it stays straight-line code.
+template <typename T> __device__ __forceinline__ T nan_();
+template <> __device__ __forceinline__ float nan_<float>() { return __builtin_nanf(""); }
+template <> __device__ __forceinline__ double nan_<double>() { return __builtin_nan(""); }
+__device__ __forceinline__ float hwmax(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double hwmax(double a, double b) { return __builtin_fmax(a, b); }
+__device__ __forceinline__ float hwmin(float a, float b) { return __builtin_fminf(a, b); }
+__device__ __forceinline__ double hwmin(double a, double b) { return __builtin_fmin(a, b); }
+template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return __builtin_isunordered(a, b) ? nan_<T>() : hwmax(a, b); }
+template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return __builtin_isunordered(a, b) ? nan_<T>() : hwmin(a, b); }
 template <typename T> __device__ __forceinline__ T tclamp(T x, T lo, T hi) { return tmin(tmax(x, lo), hi); }
 
 // pow(x, p) for x >= 0:  x = m 2^e with m in [1/sqrt2, sqrt2), s = (m-1)/(m+1),
@@ -239,13 +247,18 @@ template <typename T, int F> __device__ __forceinline__ T rms(const T (&v)[F]) {
 }
 
 // sum_s round(dt*w_s) * k_s, products rounded before they are added
-// (einsum "b, s, sbf -> bf" on the small-matrix path, F <= 57).
-template <typename T, int F> __device__ __forceinline__ void weighted_k(T dt, const double (&w)[7], const T (&k)[7][F], T (&out)[F]) {
+// (einsum "b, s, sbf -> bf" on the small-matrix path, F <= 57).  The weights are
+// row ROW of Tab::w, or Tab::b_err for ROW < 0; they are named by template
+// arguments so that the float64 -> T conversion happens at compile time.
+template <typename T, int F, typename Tab, int ROW>
+__device__ __forceinline__ void weighted_k(T dt, const T (&k)[7][F], T (&out)[F]) {
 #pragma unroll
     for (int f = 0; f < F; ++f) out[f] = 0;
 #pragma unroll
     for (int s = 0; s < 7; ++s) {
-        T p = dt * (T)w[s];
+        constexpr int R = ROW < 0 ? 0 : ROW;
+        const T ws = ROW < 0 ? (T)Tab::b_err[s] : (T)Tab::w[R][s];
+        T p = dt * ws;
 #pragma unroll
         for (int f = 0; f < F; ++f) {
             T pk = p * k[s][f];
@@ -304,12 +317,12 @@ __device__ __forceinline__ void quartic(T dt, const T (&y0)[F], const T (&y1)[F]
             q[0][f] = y0[f];
             q[1][f] = dt * k[0][f];
         }
-        weighted_k<T, F>(dt, Tsit5Tab::w[0], k, q[2]);
-        weighted_k<T, F>(dt, Tsit5Tab::w[1], k, q[3]);
-        weighted_k<T, F>(dt, Tsit5Tab::w[2], k, q[4]);
+        weighted_k<T, F, Tsit5Tab, 0>(dt, k, q[2]);
+        weighted_k<T, F, Tsit5Tab, 1>(dt, k, q[3]);
+        weighted_k<T, F, Tsit5Tab, 2>(dt, k, q[4]);
     } else {
         T ymid[F];
-        weighted_k<T, F>(dt, Dopri5Tab::w[0], k, ymid);
+        weighted_k<T, F, Dopri5Tab, 0>(dt, k, ymid);
 #pragma unroll
         for (int f = 0; f < F; ++f) {
             T f0 = dt * k[0][f], f1 = dt * k[6][f];

@@ -105,7 +105,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
                     for (int f = 0; f < F; ++f) y1[f] = yi[f];
                 }
             }
-            weighted_k<T, F>(dt, Tab::b_err, k, err);
+            weighted_k<T, F, Tab, -1>(dt, k, err);
 
             // ---- step size control (step_size_controllers.py:370-429, 715-774) ----
             const T ratio = error_ratio<T, F>(cp, y, y1, err);
