@@ -1,0 +1,151 @@
+"""CPU tests of the host side: problem validation, term bookkeeping, controller parameter
+marshalling, dispatch guards, the C ABI's exported symbols, the seeded workloads and the
+committed golden fixtures (checked here against the C oracle, on the GPU against the kernels)."""
+import glob
+import hashlib
+import json
+import os
+import re
+
+import pytest
+import torch
+
+import torchode_amd as to
+from oracle import c_oracle
+from torchode_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_problem_defaults_and_direction():
+    t_eval = torch.tensor([[0.0, 1.0, 2.0], [5.0, 4.0, 1.0], [3.0, 3.0, 3.0]])
+    p = to.InitialValueProblem(torch.zeros(3, 2), t_eval=t_eval)
+    assert torch.equal(p.t_start, t_eval[:, 0]) and torch.equal(p.t_end, t_eval[:, -1])
+    assert p.time_direction.tolist() == [1, -1, -1]  # t_end == t_start counts as backwards
+    assert (p.batch_size, p.n_features, p.n_evaluation_points) == (3, 2, 3)
+    p = to.InitialValueProblem(torch.zeros(2, 1, dtype=torch.float64), torch.zeros(2), torch.ones(2))
+    assert p.n_evaluation_points == 0 and p.data_dtype == torch.float64 and p.time_dtype == torch.float32
+
+
+@pytest.mark.parametrize(
+    "kwargs",
+    [
+        dict(y0=torch.zeros(3), t_start=torch.zeros(3), t_end=torch.ones(3)),  # y0 not 2-D
+        dict(y0=torch.zeros(3, 1), t_start=torch.zeros(2), t_end=torch.ones(2)),  # batch mismatch
+        dict(y0=torch.zeros(3, 1), t_start=torch.zeros(3), t_end=torch.ones(3, dtype=torch.float64)),  # time dtypes
+        dict(y0=torch.zeros(3, 1), t_eval=torch.zeros(3)),  # t_eval not 2-D
+    ],
+)
+def test_problem_rejects_bad_shapes(kwargs):
+    with pytest.raises((AssertionError, IndexError)):
+        to.InitialValueProblem(**kwargs)
+
+
+def test_term_counts_evaluations_on_cpu_tensor_and_passes_args_by_identity():
+    seen = []
+    term = to.ODETerm(lambda t, y, a: seen.append(a) or y, with_args=True)
+    problem = to.InitialValueProblem(torch.zeros(4, 1), t_eval=torch.zeros(4, 2))
+    stats = {}
+    term.init(problem, stats)
+    token = object()
+    for _ in range(3):
+        term.vf(problem.t_start, problem.y0, stats, token)
+    assert stats["n_f_evals"].tolist() == [3, 3, 3, 3] and stats["n_f_evals"].device.type == "cpu"
+    assert all(a is token for a in seen)
+    quiet = to.ODETerm(lambda t, y: y, with_stats=False)
+    stats = {}
+    quiet.init(problem, stats)
+    quiet.vf(problem.t_start, problem.y0, stats, None)
+    assert stats == {}
+
+
+def test_controller_struct_carries_float32_rounded_tolerances():
+    c = to.PIDController(1e-6, 1e-4, 0.2, 0.5, 0.0, dt_max=0.5).c_struct()
+    assert c.kind == _lib.CTRL_PID and c.has_dt_max == 1 and c.has_dt_min == 0 and c.dt_max == 0.5
+    assert c.atol == float(torch.tensor(1e-6)) != 1e-6 and c.rtol == float(torch.tensor(1e-4)) != 1e-4
+    assert (c.pcoeff, c.icoeff, c.dcoeff, c.safety, c.factor_min, c.factor_max) == (0.2, 0.5, 0.0, 0.9, 0.2, 10.0)
+    i = to.IntegralController(1e-3, 1e-3, safety=0.8)
+    assert i.c_struct().kind == _lib.CTRL_INTEGRAL and i.c_struct().safety == 0.8
+    assert i.atol.dtype == torch.float32 and "atol" in dict(i.named_buffers())
+    assert to.IntegralController(1e-3, 1e-3, norm=to.step_size_controllers.max_norm).fusable is False
+
+
+def test_solve_refuses_cpu_tensors_and_grad():
+    w = to.workloads.make("vdp", batch=4)
+    solver = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(1e-6, 1e-4, 0.2, 0.5, 0.0))
+    with pytest.raises(RuntimeError, match="AMD GPU"):
+        solver.solve(to.InitialValueProblem(w.y0, t_eval=w.t_eval), to.ODETerm(w.f))
+    assert solver.step_method.convergence_order() == 5 and solver.max_steps is None
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "torchode_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(tode_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _lib.load()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared in include/torchode_amd.h but not exported"
+    assert declared == set(_lib.EXPORTS)
+    assert lib.tode_abi_version() == _lib.ABI_VERSION == int(re.search(r"#define TODE_ABI_VERSION (\d+)", header).group(1))
+    assert lib.tode_last_error() is not None
+
+
+def test_abi_argument_validation_without_a_gpu():
+    """Null / inconsistent arguments are rejected before anything touches a device."""
+    lib = _lib.load()
+    a, c = _lib.SolveArgs(), _lib.Controller()
+    assert lib.tode_solve_builtin(None, None, None) == -1
+    a.batch, a.n_features, a.n_eval = 4, 2, 0
+    assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1
+    assert b"null" in lib.tode_last_error()
+    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -2  # n_eval == 0
+    a.n_features = 0
+    assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1
+    assert b"bad sizes" in lib.tode_last_error()
+    out = _lib.C.c_float()
+    assert lib.tode_last_solve_kernel_ms(_lib.C.byref(out)) == -1
+
+
+def test_workloads_are_deterministic_and_prefix_consistent():
+    a = to.workloads.make("vdp", batch=300, dtype=torch.float64)
+    b = to.workloads.make("vdp", batch=1000, dtype=torch.float64)
+    assert torch.equal(a.y0, b.y0[:300]) and torch.equal(a.t_eval, b.t_eval[:300]) and torch.equal(a.f.mu, b.f.mu[:300])
+    f32 = to.workloads.make("vdp", batch=300)
+    assert f32.y0.dtype == torch.float32 and torch.equal(f32.y0, a.y0.float())
+    assert torch.equal(a.t_eval[:, 0], torch.zeros(300, dtype=torch.float64))
+    assert (a.bytes_step, a.bytes_dense) == (160, 1200) and (f32.bytes_step, f32.bytes_dense) == (88, 600)
+    lz, ld = to.workloads.make("lorenz", batch=8), to.workloads.make("linear_decay")
+    assert (lz.bytes_step, lz.bytes_dense) == (88, 320) and (ld.bytes_step, ld.bytes_dense) == (216, 400)
+    assert ld.y0.shape == (256, 4) and ld.y0.dtype == torch.float64 and lz.t_eval.shape == (8, 20)
+
+
+def test_builtin_terms_are_plain_torch_callables():
+    w = to.workloads.make("lorenz", batch=5, dtype=torch.float64)
+    t = torch.zeros(5, dtype=torch.float64)
+    dy = w.f(t, w.y0)
+    x, y, z = w.y0.T
+    expect = torch.stack((10.0 * (y - x), x * (w.f.rho - z) - y, x * y - (8.0 / 3.0) * z), 1)
+    assert torch.equal(dy, expect)
+    assert w.f.builtin_params().shape == (5, 1) and w.f.builtin_kind == to.builtin_terms.TERM_LORENZ63
+
+
+def _sha(t):
+    return hashlib.sha256(t.contiguous().numpy().tobytes()).hexdigest()
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "*.json"))), ids=os.path.basename)
+def test_oracle_reproduces_golden_fixture(path):
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    assert {"y0": _sha(w.y0), "t_eval": _sha(w.t_eval), "params": _sha(w.f.builtin_params())} == g["inputs_sha256"]
+    cfg = c_oracle.make_config(method=g["method"], term=g["workload"], nthreads=4, **g["controller"])
+    out = c_oracle.solve(cfg, w.f.builtin_params(), w.y0, w.t_eval)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status"):
+        assert out[key].tolist() == g[key], key
+    assert int(out["n_f_evals"][0]) == g["n_f_evals"]
+    got = [float(v).hex() for v in out["ys"][g["subset"]].flatten().tolist()]
+    assert got == g["ys_subset"]
+    ys = out["ys"].double()
+    assert float(ys.sum()).hex() == g["ys_sum"] and float((ys * ys).sum()).hex() == g["ys_sum_sq"]

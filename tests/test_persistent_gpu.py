@@ -264,3 +264,29 @@ def test_against_aten_restatement_float64(name, dtype, tol):
     same = (sol.stats["n_steps"].cpu() == ref["n_steps"]) & (sol.stats["n_accepted"].cpu() == ref["n_accepted"])
     assert same.float().mean().item() >= 0.999
     assert mixed_error(sol.ys.cpu(), ref["ys"]) < tol
+
+
+# ---- committed golden fixtures (tests/golden/*.json, written by tests/golden/make_golden.py) ----
+
+import glob  # noqa: E402
+import json  # noqa: E402
+import os  # noqa: E402
+
+_GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")))
+
+
+@pytest.mark.parametrize("fast", [True, False], ids=["fast", "general"])
+@pytest.mark.parametrize("path", _GOLDEN, ids=os.path.basename)
+def test_gpu_matches_golden_fixture(path, fast):
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    sol = gpu_solve(w.f, w.y0, w.t_eval, g["method"], g["controller"], fast=fast)
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert sol.stats[key].cpu().tolist() == g[key], key
+    assert sol.status.cpu().tolist() == g["status"]
+    assert int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
+    ys = sol.ys.cpu()
+    assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
+    ysd = ys.double()
+    assert float(ysd.sum()).hex() == g["ys_sum"] and float((ysd * ysd).sum()).hex() == g["ys_sum_sq"]
