@@ -170,6 +170,105 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
 int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                             int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream);
 
+/* ------------------------------------------------------------------------- */
+/* Per-step kernels around a right-hand side that lives outside the library   */
+/* ------------------------------------------------------------------------- */
+
+/* Layout of the int32 flag block of a stepwise solve (device memory). */
+enum {
+    TODE_STEP_FLAG_STOPPED = 0,     /* 1 once the loop has ended on the device               */
+    TODE_STEP_FLAG_ITERATIONS = 1,  /* loop iterations completed before it ended             */
+    TODE_STEP_FLAG_ANY_RUNNING = 2, /* scratch of the current iteration                      */
+    TODE_STEP_FLAG_ANY_FAILURE = 3, /* 1 once any sample reported a non-success status       */
+    TODE_STEP_FLAG_WORDS = 4
+};
+
+/*
+ * Device-resident state of one solve whose right-hand side f is evaluated by
+ * the caller (any framework) between kernels.  The caller owns every buffer
+ * for the duration of the solve.  Data and time share one dtype.
+ *
+ * Replaces the locals of AutoDiffAdjoint.solve (reference adjoints.py:59-126),
+ * ERKState / ERKInterpolationData (single_step_methods/runge_kutta.py:161-172)
+ * and PIDState (step_size_controllers.py:493-551).
+ *
+ * Protocol of one solve on one stream (no host synchronisation required
+ * between calls):
+ *   k[0] <- f(t_start, y0)
+ *   tode_step_begin(phase 0)            with dt0 == NULL: ystage[1], tnode <- start-step probe
+ *   [ k[1] <- f(tnode, ystage[1]);  tode_step_begin(phase 1) ]      only when dt0 == NULL
+ *   repeat:  for s = 1..6:  tode_step_stage(s);  k[s] <- f(tnode, ystage[s])
+ *            tode_step_finish()
+ *   The caller reads `flags` whenever it likes; after TODE_STEP_FLAG_STOPPED is
+ *   set, further stage/finish calls are no-ops.  tode_step_stats converts the
+ *   counters.  k[0] must point at k0 from the first stage call on (begin
+ *   copies f(t_start, y0) there).
+ */
+typedef struct tode_step_state {
+    int32_t dtype;      /* TODE_F32 | TODE_F64 */
+    int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 */
+    int32_t n_features; /* F */
+    int32_t n_eval;     /* E; 0: report y(t_end) only */
+    int64_t batch;      /* B */
+    int64_t max_steps;  /* < 0: unlimited */
+    const void *y0;      /* [B,F] */
+    const void *t_start; /* [B] */
+    const void *t_end;   /* [B] */
+    const void *t_eval;  /* [B,E] or NULL */
+    void *t;             /* [B]   current time            */
+    void *dt;            /* [B]   current step            */
+    void *y;             /* [B,F] current state           */
+    void *k0;            /* [B,F] FSAL derivative f(t, y) */
+    double *l2_prev;     /* [B] log2 of the last accepted error ratio (PID history) */
+    double *l2_pprev;    /* [B] ... and of the one before                          */
+    int32_t *running;    /* [B] */
+    int32_t *cursor;     /* [B] index of the first evaluation point still pending  */
+    int32_t *n_steps;    /* [B] */
+    int32_t *n_accepted; /* [B] */
+    int32_t *status;     /* [B] status of the latest iteration */
+    int32_t *monotone;   /* [B] 1 if the sample's t_eval row is monotone in its direction */
+    uint8_t *pending;    /* [B,E] 1 while an evaluation point has not been written */
+    void *ys;            /* out [B,max(E,1),F] */
+    int32_t *flags;      /* [TODE_STEP_FLAG_WORDS] */
+    void *ystage[7];     /* [B,F] each: input of stage s (index 0 unused); ystage[6] is y1 */
+    const void *k[7];    /* [B,F] each: f at stage s, written by the caller; k[0] == k0   */
+    void *tnode;         /* [B] time of the stage that was just prepared */
+} tode_step_state;
+
+/*
+ * Start of a stepwise solve.  phase 0 resets the flag block and, with a user
+ * step dt0 ([B], may be NULL), initialises the loop state from k[0]; without
+ * dt0 it prepares the second evaluation of the start-step selection
+ * (reference step_size_controllers.py:431-490, 776-835).  phase 1 (only when
+ * dt0 == NULL) finishes the selection from k[1] and initialises the loop state
+ * (adjoints.py:59-126).
+ */
+int tode_step_begin(const tode_step_state *state, const tode_controller *controller, const void *dt0, int phase, void *stream);
+
+/*
+ * Stage `stage` (1..6): ystage[stage] = fma(dt, sum_j a[stage][j] k[j], y) and
+ * tnode = fma(c[stage], dt, t).  Replaces the body of the stage loop of
+ * ExplicitRungeKutta.step (reference single_step_methods/runge_kutta.py:259-262).
+ */
+int tode_step_stage(const tode_step_state *state, const tode_controller *controller, int stage, void *stream);
+
+/*
+ * Everything after the sixth stage of one loop iteration, fused into one pass
+ * per sample: error estimate (runge_kutta.py:265-272), error ratio, accept /
+ * reject, PI/PID proposal, dt_min / dt_max and status
+ * (step_size_controllers.py:370-429, 715-774), counters, dense output at the
+ * evaluation points the step passed (adjoints.py:215-234 with
+ * tsit5.py:123-139 / dopri5.py:53-60 / interpolation.py:25-40), state and FSAL
+ * update, running flag, dt clamp and controller history (adjoints.py:150-255),
+ * followed by the loop-continuation decision (adjoints.py:186-190).
+ */
+int tode_step_finish(const tode_step_state *state, const tode_controller *controller, void *stream);
+
+/* int32 counters of a stepwise solve -> the int64 stats and status the reference returns
+ * (adjoints.py:267-292). */
+int tode_step_stats(const tode_step_state *state, int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized,
+                    int64_t *out_status, void *stream);
+
 /*
  * Kernel timing for benchmarks and profiling; no counterpart in the reference.
  * While enabled (per host thread), tode_solve_builtin and tode_solve_builtin_fast record a HIP event on

@@ -1,0 +1,148 @@
+"""GPU tests of the per-step path (arbitrary Python f): fused stage / finish kernels around the
+user's torch right-hand side, loop state on the device.
+
+The right-hand sides here are the built-in terms hidden behind a plain Python callable, so the
+solver cannot recognise them and must take the per-step path; their torch ops round exactly like
+the scalar oracle's, which makes bit-for-bit comparison against the C oracle possible.
+"""
+import copy
+
+import pytest
+import torch
+
+import torchode_amd as to
+from helpers import assert_identical, c_oracle_solve, make_controller, make_method
+
+pytestmark = pytest.mark.gpu
+F32, F64 = torch.float32, torch.float64
+
+
+def stepwise_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, calls=None, **extra):
+    dev = "cuda"
+    mv = lambda x: None if x is None else x.to(dev)
+    fg = copy.deepcopy(f).to(dev)
+
+    def opaque(t, y):  # hides the built-in module from the dispatcher
+        if calls is not None:
+            calls.append((t, y))
+        return fg(t, y)
+
+    solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **extra), max_steps=max_steps)
+    problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
+    return solver.solve(problem, to.ODETerm(opaque), dt0=mv(dt0))
+
+
+@pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
+@pytest.mark.parametrize("name,batch", [("linear_decay", 256), ("vdp", 512), ("lorenz", 512)])
+def test_workload_matches_oracle_bit_for_bit(name, batch, dtype):
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller))
+
+
+@pytest.mark.parametrize("method", ["dopri5", "tsit5"])
+@pytest.mark.parametrize(
+    "controller",
+    [dict(kind="integral", atol=1e-6, rtol=1e-4), dict(kind="pid", atol=1e-5, rtol=1e-5, pcoeff=0.3, icoeff=0.4, dcoeff=0.1)],
+    ids=["I", "PID"],
+)
+def test_every_method_controller_pair(method, controller):
+    w = to.workloads.make("vdp", batch=200, dtype=F64)
+    assert_identical(stepwise_solve(w.f, w.y0, w.t_eval, method, controller), c_oracle_solve(w.f, w.y0, w.t_eval, method, controller))
+
+
+def test_loop_bookkeeping_cases():
+    w = to.workloads.make("vdp", batch=130, dtype=F32)
+    # non-monotone evaluation times (pending mask), points outside the range, user dt0
+    t_eval = w.t_eval.clone()
+    t_eval[5, [3, 7]] = t_eval[5, [7, 3]]
+    assert_identical(stepwise_solve(w.f, w.y0, t_eval, w.method, w.controller), c_oracle_solve(w.f, w.y0, t_eval, w.method, w.controller))
+    ts, te = torch.full((130,), 0.5), (w.t_eval[:, -1] * 0.9).contiguous()
+    kw = dict(t_start=ts, t_end=te, dt0=torch.full((130,), 0.02))
+    sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, **kw)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller, **kw))
+    assert sol.stats["n_f_evals"][0].item() == 1 + 6 * sol.stats["n_steps"].max().item()
+    # no evaluation points
+    sol = stepwise_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te))
+    assert sol.ys.shape == (130, 1, 2)
+
+
+def test_status_handling_matches_oracle():
+    w = to.workloads.make("lorenz", batch=100, dtype=F64)
+    full = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    cap = int(full["n_steps"].median())
+    sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, max_steps=cap)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller, max_steps=cap))
+    assert (sol.status == 3).any() and (sol.status == 0).any()
+    y0 = w.y0.clone()
+    y0[17, 1] = float("nan")
+    sol = stepwise_solve(w.f, y0, w.t_eval, w.method, w.controller)
+    assert_identical(sol, c_oracle_solve(w.f, y0, w.t_eval, w.method, w.controller))
+    assert sol.status[17].item() == 4 and sol.stats["n_steps"].max().item() == 1
+    t_eval = w.t_eval.clone()
+    t_eval[3] = t_eval[3] * 0.05
+    sol = stepwise_solve(w.f, w.y0, t_eval, w.method, w.controller, dt_min=1e-9)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, t_eval, w.method, w.controller, dt_min=1e-9))
+    assert sol.status[3].item() == 2
+
+
+def test_agrees_with_persistent_path_and_f_sees_fresh_tensors():
+    w = to.workloads.make("vdp", batch=300, dtype=F32, device="cuda")
+    ctrl = to.PIDController(1e-6, 1e-4, 0.2, 0.5, 0.0)
+    prob = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
+    a = to.AutoDiffAdjoint(to.Tsit5(), ctrl).solve(prob, to.ODETerm(w.f))
+    calls = []
+    b = to.AutoDiffAdjoint(to.Tsit5(), ctrl).solve(prob, to.ODETerm(lambda t, y: calls.append((t, y)) or w.f(t, y)))
+    assert torch.equal(a.ys, b.ys) and torch.equal(a.stats["n_steps"], b.stats["n_steps"]) and torch.equal(a.status, b.status)
+    assert torch.equal(a.stats["n_f_evals"], b.stats["n_f_evals"])
+    assert len(calls) >= b.stats["n_f_evals"][0].item()  # a few speculative calls after the loop ended
+    ptrs = {t.data_ptr() for t, _ in calls[:8]}
+    assert len(ptrs) == 8  # every evaluation got its own time tensor
+    t_min, t_max = w.t_eval.min(1).values, w.t_eval.max(1).values
+    for t, _ in calls[: b.stats["n_f_evals"][0].item()]:
+        assert (t >= t_min).all() and (t <= t_max).all()  # reference tests/adjoint_test.py:264-292
+
+
+def test_extra_args_are_passed_by_identity():
+    """reference tests/extra_args_test.py:10-22"""
+    seen = []
+
+    def f(t, y, args):
+        seen.append(args)
+        return torch.ones_like(y)
+
+    token = (0, True, "hello", torch.tensor([0.0, -1.0]))
+    term = to.ODETerm(f, with_args=True)
+    y0 = torch.tensor([[0.0, 1.0, 2.0]], device="cuda")
+    t_eval = torch.tensor([[0.0, 0.2, 0.6, 1.0]], device="cuda")
+    for method in (to.Dopri5, to.Tsit5):
+        sol = to.AutoDiffAdjoint(method(term), to.PIDController(1e-3, 1e-3, 0.0, 1.0, 0.0)).solve(
+            to.InitialValueProblem(y0, t_eval=t_eval), term, args=token
+        )
+        assert seen and all(a is token for a in seen)
+        assert torch.allclose(sol.ys[0, -1].cpu(), torch.tensor([1.0, 2.0, 3.0]), atol=1e-5)
+
+
+@pytest.mark.parametrize("ctrl", [to.PIDController(1e-5, 1e-5, 0.0, 1.0, 0.0), to.IntegralController(1e-5, 1e-5)])
+def test_constant_dynamics_in_opposite_directions(ctrl):
+    """reference tests/adjoint_test.py:357-368"""
+    term = to.ODETerm(lambda t, y: 2 * torch.ones_like(y))
+    y0 = torch.tensor([[1.0], [9.0]], device="cuda")
+    t_eval = torch.tensor([[0.0, 3.0, 5.0], [2.0, 0.5, -8.0]], device="cuda")
+    sol = to.AutoDiffAdjoint(to.Dopri5(), ctrl).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
+    assert torch.allclose(sol.ys.squeeze(-1).cpu(), torch.tensor([[1.0, 7.0, 11.0], [9.0, 6.0, -11.0]]), rtol=1e-6)
+    assert (sol.status == 0).all()
+
+
+def test_readme_example():
+    """reference README.md:42-59: exact stats of the documented example"""
+    y0 = torch.tensor([[1.2], [5.0]], device="cuda")
+    t_eval = torch.stack((torch.linspace(0, 5, 10), torch.linspace(3, 4, 10))).cuda()
+    term = to.ODETerm(lambda t, y: -0.5 * y)
+    solver = to.AutoDiffAdjoint(to.Dopri5(term=term), to.IntegralController(atol=1e-6, rtol=1e-3, term=term))
+    sol = solver.solve(to.InitialValueProblem(y0=y0, t_eval=t_eval))
+    assert sol.stats["n_f_evals"].tolist() == [26, 26]
+    assert sol.stats["n_steps"].tolist() == [4, 2] and sol.stats["n_accepted"].tolist() == [4, 2]
+    assert sol.stats["n_initialized"].tolist() == [10, 10]
+    assert torch.allclose(sol.ys[0, :, 0].cpu(), 1.2 * torch.exp(-0.5 * t_eval[0].cpu()), rtol=2e-3)

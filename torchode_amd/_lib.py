@@ -28,6 +28,10 @@ EXPORTS = (
     "tode_last_error",
     "tode_solve_builtin",
     "tode_solve_builtin_fast",
+    "tode_step_begin",
+    "tode_step_stage",
+    "tode_step_finish",
+    "tode_step_stats",
     "tode_finalize_stats",
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
@@ -87,6 +91,44 @@ class SolveArgs(C.Structure):
     ]
 
 
+STEP_FLAG_STOPPED, STEP_FLAG_ITERATIONS, STEP_FLAG_ANY_RUNNING, STEP_FLAG_ANY_FAILURE, STEP_FLAG_WORDS = 0, 1, 2, 3, 4
+
+
+class StepState(C.Structure):
+    """struct tode_step_state"""
+
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("method", C.c_int32),
+        ("n_features", C.c_int32),
+        ("n_eval", C.c_int32),
+        ("batch", C.c_int64),
+        ("max_steps", C.c_int64),
+        ("y0", C.c_void_p),
+        ("t_start", C.c_void_p),
+        ("t_end", C.c_void_p),
+        ("t_eval", C.c_void_p),
+        ("t", C.c_void_p),
+        ("dt", C.c_void_p),
+        ("y", C.c_void_p),
+        ("k0", C.c_void_p),
+        ("l2_prev", C.c_void_p),
+        ("l2_pprev", C.c_void_p),
+        ("running", C.c_void_p),
+        ("cursor", C.c_void_p),
+        ("n_steps", C.c_void_p),
+        ("n_accepted", C.c_void_p),
+        ("status", C.c_void_p),
+        ("monotone", C.c_void_p),
+        ("pending", C.c_void_p),
+        ("ys", C.c_void_p),
+        ("flags", C.c_void_p),
+        ("ystage", C.c_void_p * 7),
+        ("k", C.c_void_p * 7),
+        ("tnode", C.c_void_p),
+    ]
+
+
 _lock = threading.Lock()
 _lib = None
 
@@ -108,6 +150,14 @@ def load():
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
         lib.tode_solve_builtin_fast.restype = C.c_int
         lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
+        lib.tode_step_begin.restype = C.c_int
+        lib.tode_step_begin.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p, C.c_int, C.c_void_p]
+        lib.tode_step_stage.restype = C.c_int
+        lib.tode_step_stage.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_int, C.c_void_p]
+        lib.tode_step_finish.restype = C.c_int
+        lib.tode_step_finish.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p]
+        lib.tode_step_stats.restype = C.c_int
+        lib.tode_step_stats.argtypes = [C.POINTER(StepState)] + [C.c_void_p] * 5
         lib.tode_finalize_stats.restype = C.c_int
         lib.tode_finalize_stats.argtypes = [C.c_int64, C.c_int64] + [C.c_void_p] * 9 + [C.c_int32] * 3 + [C.c_void_p] * 3
         lib.tode_set_kernel_timing.restype = C.c_int

@@ -58,7 +58,13 @@ class AutoDiffAdjoint(nn.Module):
             )
         if self._persistent_ok(problem, term_):
             return self._solve_persistent(problem, term_, dt0)
-        raise NotImplementedError("only built-in terms are wired up so far")
+        if self._stepwise_ok(problem):
+            return self._solve_stepwise(problem, term_, dt0, args)
+        raise NotImplementedError(
+            "this combination of step method, controller and dtypes has no kernel path yet "
+            "(supported: Dopri5/Tsit5 with IntegralController/PIDController and the RMS norm, "
+            "time dtype equal to the data dtype)"
+        )
 
     # ------------------------------------------------------------------ #
     def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
@@ -73,6 +79,113 @@ class AutoDiffAdjoint(nn.Module):
             and problem.data_dtype == problem.time_dtype
             and problem.data_dtype in _lib.DTYPES
         )
+
+    def _stepwise_ok(self, problem: InitialValueProblem) -> bool:
+        m, c = self.step_method, self.step_size_controller
+        return (
+            type(m).__name__ in ("Dopri5", "Tsit5")
+            and isinstance(m, ExplicitRungeKutta)
+            and isinstance(c, _AdaptiveController)
+            and c.fusable
+            and problem.data_dtype == problem.time_dtype
+            and problem.data_dtype in _lib.DTYPES
+        )
+
+    # How many loop iterations are enqueued between two looks at the device flags.
+    poll_first, poll_max = 4, 32
+
+    def _solve_stepwise(self, problem: InitialValueProblem, term: ODETerm, dt0, args) -> Solution:
+        """Arbitrary Python ``f``: per-step kernels around the user's torch RHS, loop state on the
+        device, no host synchronisation per step (the host polls a flag every few iterations)."""
+        lib = _lib.load()
+        y0 = problem.y0.contiguous()
+        dev, dtype = y0.device, y0.dtype
+        B, F = y0.shape
+        E = problem.n_evaluation_points
+        t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
+        t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
+        dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
+        ctrl = self.step_size_controller.c_struct()
+        stream = _lib.stream_of(y0)
+        new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+
+        ys = new(B, max(E, 1), F)
+        t, dt = new(B), new(B)
+        y, k0 = new(B, F), new(B, F)
+        hist = new(2, B, dt=torch.float64)
+        ints = new(6, B, dt=torch.int32)
+        pending = new(B, max(E, 1), dt=torch.uint8)
+        flags = new(_lib.STEP_FLAG_WORDS, dt=torch.int32)
+
+        s = _lib.StepState()
+        s.dtype, s.method, s.n_features, s.n_eval = _lib.DTYPES[dtype], self.step_method.method_id, F, E
+        s.batch = B
+        s.max_steps = -1 if self.max_steps is None else int(self.max_steps)
+        s.y0, s.t_start, s.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
+        s.t_eval = None if t_eval is None else t_eval.data_ptr()
+        s.t, s.dt, s.y, s.k0 = t.data_ptr(), dt.data_ptr(), y.data_ptr(), k0.data_ptr()
+        s.l2_prev, s.l2_pprev = hist[0].data_ptr(), hist[1].data_ptr()
+        s.running, s.cursor, s.n_steps, s.n_accepted, s.status, s.monotone = (ints[i].data_ptr() for i in range(6))
+        s.pending, s.ys, s.flags = pending.data_ptr(), ys.data_ptr(), flags.data_ptr()
+        sref, cref = _lib.C.byref(s), _lib.C.byref(ctrl)
+
+        f, with_args = term.f, term.with_args
+
+        def rhs(tt, yy):
+            out = f(tt, yy, args) if with_args else f(tt, yy)
+            if out.dtype != dtype or not out.is_contiguous() or out.shape != yy.shape:
+                out = out.to(dtype).expand(yy.shape).contiguous()
+            return out
+
+        # Every evaluation of f gets freshly allocated (t, y) tensors, as in the reference, so a
+        # caller that keeps them (e.g. to log the evaluation times) sees what f saw.  `keep`
+        # holds the buffers of the current iteration alive while kernels still read them.
+        keep = {}
+
+        def stage_buffers(i):
+            keep["y", i], keep["t", i] = new(B, F), new(B)
+            s.ystage[i], s.tnode = keep["y", i].data_ptr(), keep["t", i].data_ptr()
+            return keep["t", i], keep["y", i]
+
+        def evaluate(i, tt, yy):
+            keep["k", i] = rhs(tt, yy)
+            s.k[i] = keep["k", i].data_ptr()
+
+        evaluate(0, t_start, y0)
+        n_init_evals = 1
+        if dt0_ is None:
+            tt, yy = stage_buffers(1)
+            _lib.check(lib.tode_step_begin(sref, cref, None, 0, stream), "tode_step_begin")
+            evaluate(1, tt, yy)
+            _lib.check(lib.tode_step_begin(sref, cref, None, 1, stream), "tode_step_begin")
+            n_init_evals = 2
+        else:
+            s.tnode = t.data_ptr()  # unused by this phase, but must be a valid pointer
+            _lib.check(lib.tode_step_begin(sref, cref, _lib.ptr(dt0_), 0, stream), "tode_step_begin")
+        s.k[0] = k0.data_ptr()  # from here on the FSAL slot is the state's own buffer
+
+        chunk = self.poll_first
+        while True:
+            for _ in range(chunk):
+                for i in range(1, 7):
+                    tt, yy = stage_buffers(i)
+                    _lib.check(lib.tode_step_stage(sref, cref, i, stream), "tode_step_stage")
+                    evaluate(i, tt, yy)
+                _lib.check(lib.tode_step_finish(sref, cref, stream), "tode_step_finish")
+            fl = flags.tolist()  # host/device synchronisation, once per chunk of iterations
+            if fl[_lib.STEP_FLAG_STOPPED]:
+                break
+            chunk = min(2 * chunk, self.poll_max)
+
+        out = new(4, B, dt=torch.int64)
+        _lib.check(lib.tode_step_stats(sref, *(_lib.ptr(out[i]) for i in range(4)), stream), "tode_step_stats")
+        stats: Dict[str, Any] = {}
+        if term.with_stats:
+            n = n_init_evals + 6 * fl[_lib.STEP_FLAG_ITERATIONS]
+            stats["n_f_evals"] = torch.full((B,), n, dtype=torch.long, device="cpu")
+        stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
+        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+        return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
 
     def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
         lib = _lib.load()

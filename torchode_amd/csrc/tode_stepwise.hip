@@ -1,0 +1,549 @@
+// Per-step kernels for right-hand sides that live outside the library (any Python
+// f): the loop state stays on the device, the host enqueues
+//     6 x (stage kernel, user f)  ->  finish kernel  ->  loop-control kernel
+// per iteration and never waits for a step; it polls the flag block every few
+// iterations.  Once the loop has ended on the device, kernels of iterations
+// that were enqueued speculatively return immediately.
+//
+// One thread per sample; features are walked with run-time loops in the same
+// order as a scalar evaluation (this path is meant for small F, where a
+// sample's row is a few contiguous values; the stage arrays necessarily go
+// through HBM because f is external).
+#include "tode_solve.h"
+
+namespace tode {
+
+template <typename T> struct StepParams {
+    // problem
+    const T *y0, *t_start, *t_end, *t_eval;
+    long long batch;
+    int F, E;
+    int max_steps;
+    // loop state (device, owned by the caller for the duration of a solve)
+    T *t, *dt, *y, *k0;          // [B], [B], [B,F], [B,F] (FSAL derivative)
+    double *l2_prev, *l2_pprev;  // [B] log2 of the last two accepted error ratios
+    int32_t *running, *cursor, *n_steps, *n_accepted, *status, *monotone;
+    uint8_t *pending;  // [B,E]
+    T *ys;             // [B,max(E,1),F]
+    int32_t *flags;    // TODE_STEP_FLAG_*
+    // per-iteration buffers
+    T *ystage[7];    // [B,F] stage inputs; ystage[6] is y1
+    const T *k[7];   // [B,F] stage derivatives; k[0] aliases k0
+    T *tnode;        // [B]
+    CtrlParams<T> cp;
+};
+
+template <typename T> __device__ __forceinline__ T tab_a(int method, int i, int j) {
+    return method == 1 ? (T)Tsit5Tab::a[i][j] : (T)Dopri5Tab::a[i][j];
+}
+
+// ystage[s] = fma(dt, sum_j a_sj k_j, y); tnode = fma(c_s, dt, t)   (runge_kutta.py:259-262)
+template <typename T, int METHOD, int S> __global__ void __launch_bounds__(256) stage_kernel(const StepParams<T> p) {
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long n = p.batch * p.F;
+    if (i >= n) return;
+    const long long b = i / p.F;
+    const T dt = p.dt[b];
+    T s = 0;
+#pragma unroll
+    for (int j = 0; j < S; ++j) s = fma_((T)Tab::a[S][j], p.k[j][i], s);
+    p.ystage[S][i] = fma_(dt, s, p.y[i]);
+    if (i - b * p.F == 0) p.tnode[b] = fma_((T)Tab::c[S], dt, p.t[b]);
+}
+
+// Start step, first half (step_size_controllers.py:459-479): from f0 = f(t0, y0) compute h0,
+// y1 = y0 + dir*h0*f0 -> ystage[1], t1 -> tnode; h0 is parked in dt.
+template <typename T> __global__ void __launch_bounds__(256) init_a_kernel(const StepParams<T> p) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= p.batch) return;
+    const int F = p.F;
+    const CtrlParams<T> &cp = p.cp;
+    const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
+    const T sf = (T)__builtin_sqrt((double)F);
+    T a0 = 0, a1 = 0;
+    for (int f = 0; f < F; ++f) {
+        T inv = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol);
+        T x0 = (y0[f] * inv) / sf, x1 = (f0[f] * inv) / sf;
+        if (F <= 3) {
+            a0 = fma_(x0, x0, a0);
+            a1 = fma_(x1, x1, a1);
+        } else {
+            T s0 = x0 * x0, s1 = x1 * x1;
+            a0 = a0 + s0;
+            a1 = a1 + s1;
+        }
+    }
+    const T d0 = sqrt_(a0), d1 = sqrt_(a1);
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
+    h0 = tmin(h0, abs_(te - ts));
+    const T dh = dir * h0;
+    T *y1 = p.ystage[1] + b * F;
+    for (int f = 0; f < F; ++f) y1[f] = fma_(dh, f0[f], y0[f]);
+    p.tnode[b] = fma_(dir, h0, ts);
+    p.dt[b] = h0;
+}
+
+// Loop state at t_start; with FROM_F1 also the second half of the start step
+// (step_size_controllers.py:481-490 integral, 826-835 PID) from f1 = k[1].
+template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(256) init_b_kernel(const StepParams<T> p, const T *dt0) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= p.batch) return;
+    const int F = p.F, E = p.E;
+    const CtrlParams<T> &cp = p.cp;
+    const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    T dt;
+    if (FROM_F1) {
+        const T *f1 = p.k[1] + b * F;
+        const T sf = (T)__builtin_sqrt((double)F);
+        const T h0 = p.dt[b];
+        T a1 = 0, a2 = 0;
+        for (int f = 0; f < F; ++f) {
+            T inv = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol);
+            T x1 = (f0[f] * inv) / sf;
+            T df = f1[f] - f0[f];
+            T x2 = (df * inv) / sf;
+            if (F <= 3) {
+                a1 = fma_(x1, x1, a1);
+                a2 = fma_(x2, x2, a2);
+            } else {
+                T s1 = x1 * x1, s2 = x2 * x2;
+                a1 = a1 + s1;
+                a2 = a2 + s2;
+            }
+        }
+        const T d1 = sqrt_(a1);
+        T d2 = sqrt_(a2) / h0;
+        if (CTRL == 0 && h0 == (T)0) d2 = (T)__builtin_huge_val();
+        const T m = tmax(d1, d2);
+        T h1;
+        if (m <= (T)1e-15) {
+            h1 = tmax((T)1e-6, h0 * (T)1e-3);
+        } else {
+            T rm = (T)1 / m;
+            h1 = rpow<T>(rm * (T)0.01, 1.0 / 5.0);
+        }
+        dt = dir * tmin((T)100 * h0, h1);
+    } else {
+        dt = dt0[b];
+    }
+    const T tlo = tmin(ts, te), thi = tmax(te, ts);
+    p.t[b] = ts;
+    p.dt[b] = tclamp(dt, tlo - ts, thi - ts);
+    for (int f = 0; f < F; ++f) {
+        p.y[b * F + f] = y0[f];
+        p.k0[b * F + f] = f0[f];
+    }
+    p.l2_prev[b] = 0.0;
+    p.l2_pprev[b] = 0.0;
+    p.running[b] = 1;
+    p.n_steps[b] = 0;
+    p.n_accepted[b] = 0;
+    p.status[b] = 0;
+    int cursor = 0, mono = 1;
+    if (E > 0) {
+        const T *tev = p.t_eval + b * E;
+        T prev_te = tev[0];
+        for (int e = 0; e < E; ++e) {
+            T cur = tev[e];
+            if (e > 0 && !(dir > 0 ? cur >= prev_te : cur <= prev_te)) mono = 0;
+            prev_te = cur;
+            p.pending[b * E + e] = 1;
+        }
+        if (tev[0] == ts) {
+            for (int f = 0; f < F; ++f) p.ys[(b * E) * F + f] = y0[f];
+            p.pending[b * E] = 0;
+            cursor = 1;
+        }
+    }
+    p.cursor[b] = cursor;
+    p.monotone[b] = mono;
+}
+
+// Quartic of the attempted step for one feature, evaluated at time te (tsit5.py:123-139,
+// dopri5.py:53-60, interpolation.py:25-40, 138-175).  ks[s] = k_s[b,f].
+template <typename T, int METHOD> __device__ __forceinline__ T dense_value(T t0, T dt, T y0, T y1, const T (&ks)[7], bool fused, T te) {
+    T q[5][1], yy0[1] = {y0}, yy1[1] = {y1}, kk[7][1];
+#pragma unroll
+    for (int s = 0; s < 7; ++s) kk[s][0] = ks[s];
+    if (!fused) {
+        quartic<T, 1, METHOD>(dt, yy0, yy1, kk, q);
+    } else {
+        // F >= 58: the weighted sums are fused chains (large-matrix product path)
+        using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+        T w[3] = {0, 0, 0};
+#pragma unroll
+        for (int r = 0; r < Tab::n_other; ++r)
+#pragma unroll
+            for (int s = 0; s < 7; ++s) w[r] = fma_(dt * (T)Tab::w[r][s], ks[s], w[r]);
+        if (METHOD == 1) {
+            q[0][0] = y0;
+            q[1][0] = dt * ks[0];
+            q[2][0] = w[0];
+            q[3][0] = w[1];
+            q[4][0] = w[2];
+        } else {
+            T f0 = dt * ks[0], f1 = dt * ks[6];
+            T ym = y0 + w[0];
+            T a = (T)2 * (f1 - f0);
+            a = fma_((T)-8, y1 + y0, a);
+            a = fma_((T)16, ym, a);
+            T bq = (T)5 * f0;
+            bq = fma_((T)-3, f1, bq);
+            bq = fma_((T)18, y0, bq);
+            bq = fma_((T)14, y1, bq);
+            bq = fma_((T)-32, ym, bq);
+            T c = fma_((T)-4, f0, f1);
+            c = fma_((T)-11, y0, c);
+            c = fma_((T)-5, y1, c);
+            c = fma_((T)16, ym, c);
+            q[0][0] = y0;
+            q[1][0] = f0;
+            q[2][0] = c;
+            q[3][0] = bq;
+            q[4][0] = a;
+        }
+    }
+    T out[1];
+    quartic_eval<T, 1>(q, t0, dt, te, out);
+    return out[0];
+}
+
+// Everything after the last stage of one loop iteration, for one sample per thread:
+// error estimate, error ratio, accept/reject, PI/PID proposal, dt_min/dt_max, status,
+// counters, dense output at the evaluation points the step passed, state update, running
+// flag, dt clamp (runge_kutta.py:265-272, step_size_controllers.py:370-429 / 715-774,
+// adjoints.py:150-255).
+template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<T> p) {
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= p.batch) return;
+    const int F = p.F, E = p.E;
+    const CtrlParams<T> &cp = p.cp;
+    const bool fused = F >= 58;
+    const T sf = (T)__builtin_sqrt((double)F);
+    const T t0 = p.t[b], dt = p.dt[b];
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
+
+    // ---- error estimate and error ratio ----
+    T acc = 0;
+    for (int f = 0; f < F; ++f) {
+        T err = 0;
+#pragma unroll
+        for (int s = 0; s < 7; ++s) {
+            T ps = dt * (T)Tab::b_err[s];
+            T ks = p.k[s][b * F + f];
+            if (fused)
+                err = fma_(ps, ks, err);
+            else {
+                T pk = ps * ks;
+                err = err + pk;
+            }
+        }
+        T m = tmax(abs_(y[f]), abs_(y1[f]));
+        T eb = fma_(cp.rtol, m, cp.atol);
+        T x = (abs_(err) / eb) / sf;
+        if (F <= 3)
+            acc = fma_(x, x, acc);
+        else {
+            T sq = x * x;
+            acc = acc + sq;
+        }
+    }
+    const T ratio = tmax(sqrt_(acc), (T)1e-38);
+    const bool accept = ratio < (T)1;
+
+    // ---- step size proposal ----
+    const double l2p = p.l2_prev[b], l2pp = p.l2_pprev[b];
+    T factor = cp.safety * rpow<T>(ratio, cp.e1);
+    if (CTRL == 1) {
+        // prev ** e2 and prev_prev ** e3 from the stored logarithms (identical bits to pow)
+        T f2 = cp.skip2 ? (T)1 : (T)exp2_of((double)(T)cp.e2 * l2p);
+        T f3 = cp.skip3 ? (T)1 : (T)exp2_of((double)(T)cp.e3 * l2pp);
+        factor = factor * f2;
+        factor = factor * f3;
+    }
+    factor = tclamp(factor, cp.fmin, cp.fmax);
+    T dt_next = dt * factor;
+    int status = limit_dt<T>(cp, ratio, dt_next);
+
+    const bool running = p.running[b] != 0;
+    const bool move = accept && running;
+    const T t_new = move ? (t0 + dt) : t0;
+    const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+    const int n_steps = p.n_steps[b] + (running ? 1 : 0);
+    p.n_steps[b] = n_steps;
+    if (move) p.n_accepted[b] += 1;
+    if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
+    p.status[b] = status;
+
+    // ---- dense output with the interpolant of the attempted step ----
+    if (E > 0) {
+        const T *tev = p.t_eval + b * E;
+        T *ys = p.ys + b * (long long)E * F;
+        uint8_t *pend = p.pending + b * (long long)E;
+        const bool mono = p.monotone[b] != 0;
+        int cursor = p.cursor[b];
+        int e = mono ? cursor : 0;
+        for (; e < E; ++e) {
+            if (!pend[e]) continue;
+            const T te_e = tev[e];
+            const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+            if (!passed) {
+                if (mono) break;
+                continue;
+            }
+            for (int f = 0; f < F; ++f) {
+                T ks[7];
+#pragma unroll
+                for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+                ys[(long long)e * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
+            }
+            pend[e] = 0;
+        }
+        while (cursor < E && !pend[cursor]) ++cursor;  // first still-pending point
+        p.cursor[b] = cursor;
+    } else {
+        // no evaluation points: the end-point value of the loop's last interpolant
+        // (adjoints.py:295-309); rewritten every iteration, the last one stays
+        for (int f = 0; f < F; ++f) {
+            T ks[7];
+#pragma unroll
+            for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+            p.ys[b * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+        }
+    }
+
+    // ---- state update ----
+    if (move) {
+        for (int f = 0; f < F; ++f) {
+            p.y[b * F + f] = y1[f];
+            p.k0[b * F + f] = p.k[6][b * F + f];
+        }
+    }
+    p.t[b] = t_new;
+    const T tlo = tmin(ts, te), thi = tmax(te, ts);
+    const T dtn = running_new ? dt_next : dt;
+    p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
+    if (CTRL == 1 && running_new && accept) {
+        // log2 of the accepted ratio; anything outside (0, inf) ends the loop with status 4,
+        // after which the history is never read again
+        const bool sane = ratio > (T)0 && ratio < (T)__builtin_huge_val();
+        p.l2_pprev[b] = l2p;
+        p.l2_prev[b] = log2_normal(sane ? (double)ratio : 1.0);
+    }
+    p.running[b] = running_new ? 1 : 0;
+    if (running_new) p.flags[TODE_STEP_FLAG_ANY_RUNNING] = 1;
+    if (status != 0) p.flags[TODE_STEP_FLAG_ANY_FAILURE] = 1;
+}
+
+// One thread: closes the iteration.  The loop goes on iff some sample is still running and
+// every status is SUCCESS (adjoints.py:186-190).
+static __global__ void loop_control_kernel(int32_t *flags) {
+    if (threadIdx.x != 0 || flags[TODE_STEP_FLAG_STOPPED]) return;
+    flags[TODE_STEP_FLAG_ITERATIONS] += 1;
+    if (!flags[TODE_STEP_FLAG_ANY_RUNNING] || flags[TODE_STEP_FLAG_ANY_FAILURE]) flags[TODE_STEP_FLAG_STOPPED] = 1;
+    flags[TODE_STEP_FLAG_ANY_RUNNING] = 0;
+}
+
+static __global__ void step_flags_init_kernel(int32_t *flags) {
+    if (threadIdx.x < TODE_STEP_FLAG_WORDS) flags[threadIdx.x] = 0;
+}
+
+// int32 device state -> the reference's int64 stats (adjoints.py:267-292)
+static __global__ void step_stats_kernel(long long batch, const int32_t *n_steps, const int32_t *n_accepted, const int32_t *cursor,
+                                         const int32_t *status, int n_eval, int64_t *o_steps, int64_t *o_acc, int64_t *o_init,
+                                         int64_t *o_status) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= batch) return;
+    o_steps[b] = n_steps[b];
+    o_acc[b] = n_accepted[b];
+    o_init[b] = n_eval > 0 ? cursor[b] : 1;
+    o_status[b] = status[b];
+}
+
+template <typename T> static StepParams<T> make_step_params(const tode_step_state &s, const tode_controller &c) {
+    StepParams<T> p;
+    p.y0 = (const T *)s.y0;
+    p.t_start = (const T *)s.t_start;
+    p.t_end = (const T *)s.t_end;
+    p.t_eval = (const T *)s.t_eval;
+    p.batch = s.batch;
+    p.F = s.n_features;
+    p.E = s.n_eval;
+    p.max_steps = (s.max_steps < 0 || s.max_steps >= INT_MAX) ? INT_MAX : (int)s.max_steps;
+    p.t = (T *)s.t;
+    p.dt = (T *)s.dt;
+    p.y = (T *)s.y;
+    p.k0 = (T *)s.k0;
+    p.l2_prev = s.l2_prev;
+    p.l2_pprev = s.l2_pprev;
+    p.running = s.running;
+    p.cursor = s.cursor;
+    p.n_steps = s.n_steps;
+    p.n_accepted = s.n_accepted;
+    p.status = s.status;
+    p.monotone = s.monotone;
+    p.pending = s.pending;
+    p.ys = (T *)s.ys;
+    p.flags = s.flags;
+    for (int i = 0; i < 7; ++i) {
+        p.ystage[i] = (T *)s.ystage[i];
+        p.k[i] = (const T *)s.k[i];
+    }
+    p.tnode = (T *)s.tnode;
+    p.cp = make_ctrl<T>(c);
+    return p;
+}
+
+static int check_state(const tode_step_state *s, const tode_controller *c) {
+    if (!s || !c) return fail(TODE_E_INVALID, "null argument struct");
+    if (s->batch < 0 || s->n_features <= 0 || s->n_eval < 0) return fail(TODE_E_INVALID, "bad sizes");
+    if (s->dtype != TODE_F32 && s->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", s->dtype);
+    if (s->method != TODE_DOPRI5 && s->method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", s->method);
+    if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
+    if (!s->flags) return fail(TODE_E_INVALID, "null flags pointer");
+    if (s->batch > 0 && (!s->y0 || !s->t_start || !s->t_end || !s->t || !s->dt || !s->y || !s->k0 || !s->l2_prev || !s->l2_pprev ||
+                         !s->running || !s->cursor || !s->n_steps || !s->n_accepted || !s->status || !s->monotone || !s->ys || !s->tnode))
+        return fail(TODE_E_INVALID, "null state pointer");
+    if (s->batch > 0 && s->n_eval > 0 && (!s->t_eval || !s->pending)) return fail(TODE_E_INVALID, "n_eval > 0 needs t_eval and pending");
+    return TODE_OK;
+}
+
+#define TODE_DISPATCH_T(dtype, EXPR)    \
+    do {                                \
+        if ((dtype) == TODE_F32) {      \
+            using T = float;            \
+            EXPR;                       \
+        } else {                        \
+            using T = double;           \
+            EXPR;                       \
+        }                               \
+    } while (0)
+
+}  // namespace tode
+
+extern "C" {
+
+int tode_step_begin(const tode_step_state *s, const tode_controller *c, const void *dt0, int phase, void *stream) {
+    using namespace tode;
+    int rc = check_state(s, c);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)((s->batch + 255) / 256);
+    if (phase == 0) {
+        hipLaunchKernelGGL(step_flags_init_kernel, dim3(1), dim3(64), 0, st, s->flags);
+        if (blocks == 0) return check_hip(hipGetLastError(), "tode_step_begin");
+        if (dt0) {
+            if (!s->k[0]) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
+            TODE_DISPATCH_T(s->dtype, {
+                auto p = make_step_params<T>(*s, *c);
+                if (c->kind == TODE_CTRL_INTEGRAL)
+                    hipLaunchKernelGGL((init_b_kernel<T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
+                else
+                    hipLaunchKernelGGL((init_b_kernel<T, 1, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
+            });
+        } else {
+            if (!s->k[0] || !s->ystage[1]) return fail(TODE_E_INVALID, "k[0] or ystage[1] is null");
+            TODE_DISPATCH_T(s->dtype, {
+                auto p = make_step_params<T>(*s, *c);
+                hipLaunchKernelGGL(init_a_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
+            });
+        }
+    } else {
+        if (blocks == 0) return TODE_OK;
+        if (!s->k[0] || !s->k[1]) return fail(TODE_E_INVALID, "k[0] or k[1] is null");
+        TODE_DISPATCH_T(s->dtype, {
+            auto p = make_step_params<T>(*s, *c);
+            if (c->kind == TODE_CTRL_INTEGRAL)
+                hipLaunchKernelGGL((init_b_kernel<T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+            else
+                hipLaunchKernelGGL((init_b_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+        });
+    }
+    return check_hip(hipGetLastError(), "tode_step_begin");
+}
+
+int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stage, void *stream) {
+    using namespace tode;
+    int rc = check_state(s, c);
+    if (rc) return rc;
+    if (stage < 1 || stage > 6) return fail(TODE_E_INVALID, "stage must be 1..6, got %d", stage);
+    for (int j = 0; j < stage; ++j)
+        if (s->batch > 0 && !s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
+    if (s->batch > 0 && !s->ystage[stage]) return fail(TODE_E_INVALID, "ystage[%d] is null", stage);
+    const long long n = s->batch * s->n_features;
+    if (n == 0) return TODE_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+#define TODE_STAGE_CASE(M, S) \
+    case S: hipLaunchKernelGGL((stage_kernel<T, M, S>), dim3(blocks), dim3(256), 0, st, p); break;
+#define TODE_STAGE_SWITCH(M)                                                                  \
+    switch (stage) {                                                                          \
+        TODE_STAGE_CASE(M, 1) TODE_STAGE_CASE(M, 2) TODE_STAGE_CASE(M, 3) TODE_STAGE_CASE(M, 4) \
+        TODE_STAGE_CASE(M, 5) TODE_STAGE_CASE(M, 6)                                           \
+    }
+    TODE_DISPATCH_T(s->dtype, {
+        auto p = make_step_params<T>(*s, *c);
+        if (s->method == TODE_TSIT5) {
+            TODE_STAGE_SWITCH(1)
+        } else {
+            TODE_STAGE_SWITCH(0)
+        }
+    });
+#undef TODE_STAGE_SWITCH
+#undef TODE_STAGE_CASE
+    return check_hip(hipGetLastError(), "tode_step_stage");
+}
+
+int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *stream) {
+    using namespace tode;
+    int rc = check_state(s, c);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)((s->batch + 255) / 256);
+    if (blocks > 0) {
+        for (int j = 0; j < 7; ++j)
+            if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
+        if (!s->ystage[6]) return fail(TODE_E_INVALID, "ystage[6] is null");
+        TODE_DISPATCH_T(s->dtype, {
+            auto p = make_step_params<T>(*s, *c);
+            const bool pid = c->kind == TODE_CTRL_PID;
+            if (s->method == TODE_TSIT5) {
+                if (pid)
+                    hipLaunchKernelGGL((finish_kernel<T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
+                else
+                    hipLaunchKernelGGL((finish_kernel<T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
+            } else {
+                if (pid)
+                    hipLaunchKernelGGL((finish_kernel<T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
+                else
+                    hipLaunchKernelGGL((finish_kernel<T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
+            }
+        });
+    }
+    hipLaunchKernelGGL(loop_control_kernel, dim3(1), dim3(64), 0, st, s->flags);
+    return check_hip(hipGetLastError(), "tode_step_finish");
+}
+
+int tode_step_stats(const tode_step_state *s, int64_t *n_steps, int64_t *n_accepted, int64_t *n_initialized, int64_t *status, void *stream) {
+    using namespace tode;
+    if (!s) return fail(TODE_E_INVALID, "null state");
+    if (s->batch == 0) return TODE_OK;
+    if (!n_steps || !n_accepted || !n_initialized || !status || !s->n_steps || !s->n_accepted || !s->cursor || !s->status)
+        return fail(TODE_E_INVALID, "null pointer");
+    const unsigned blocks = (unsigned)((s->batch + 255) / 256);
+    hipLaunchKernelGGL(step_stats_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (long long)s->batch, s->n_steps, s->n_accepted,
+                       s->cursor, s->status, s->n_eval, n_steps, n_accepted, n_initialized, status);
+    return check_hip(hipGetLastError(), "tode_step_stats");
+}
+
+}  // extern "C"
