@@ -28,7 +28,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/solve_fast_kernel_vdp_f32_b65536_hbm_traffic.txt: (7120.1 KiB x 2.000 + 27680 KiB x 1.000) x 1024
+    ("vdp", "torch.float32", 65536): 42.93e6,
+}
 
 
 def main():
@@ -40,6 +43,12 @@ def main():
     ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
     ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument(
+        "--calibration-copy-mib",
+        type=int,
+        default=0,
+        help="also run one plain device copy of this many MiB (a known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (samples would shard over the batch axis, see DESIGN.md)")
@@ -61,6 +70,14 @@ def main():
     solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl)
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
     term = to.ODETerm(w.f)
+
+    if args.calibration_copy_mib:
+        src = torch.ones(args.calibration_copy_mib * 2**20 // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads and writes exactly calibration_copy_mib MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         sol = solver.solve(problem, term)
@@ -108,7 +125,7 @@ def main():
         "equiv_hbm_gbps": algo_bytes / wall / 1e9,
         "roofline": {
             "bound": "hbm",
-            "kernel": "tode::solve_kernel",
+            "kernel": "tode::solve_fast_kernel",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
