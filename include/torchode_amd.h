@@ -219,8 +219,8 @@ typedef struct tode_step_state {
     void *dt;            /* [B]   current step            */
     void *y;             /* [B,F] current state           */
     void *k0;            /* [B,F] FSAL derivative f(t, y) */
-    double *l2_prev;     /* [B] log2 of the last accepted error ratio (PID history) */
-    double *l2_pprev;    /* [B] ... and of the one before                          */
+    void *ratio_prev;    /* [B] last accepted error ratio (PID history, data dtype) */
+    void *ratio_pprev;   /* [B] ... and the one before                             */
     int32_t *running;    /* [B] */
     int32_t *cursor;     /* [B] index of the first evaluation point still pending  */
     int32_t *n_steps;    /* [B] */

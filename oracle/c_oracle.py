@@ -55,8 +55,10 @@ def lib():
     global _lib
     if _lib is None:
         _lib = C.CDLL(build())
-        _lib.oracle_pow_core.restype = C.c_double
-        _lib.oracle_pow_core.argtypes = [C.c_double, C.c_double]
+        _lib.oracle_pow.restype = C.c_double
+        _lib.oracle_pow.argtypes = [C.c_double, C.c_double]
+        _lib.oracle_powf.restype = C.c_float
+        _lib.oracle_powf.argtypes = [C.c_float, C.c_float]
         _lib.oracle_initial_step_f32.restype = C.c_float
         _lib.oracle_initial_step_f64.restype = C.c_double
     return _lib
@@ -113,8 +115,20 @@ def _real(dtype):
     return C.c_float if dtype == torch.float32 else C.c_double
 
 
-def pow_core(x: float, p: float) -> float:
-    return lib().oracle_pow_core(x, p)
+def pow_scalar(x: float, p: float, dtype=torch.float64) -> float:
+    """pow(x, p) of the oracle in `dtype` (one value)."""
+    return lib().oracle_powf(x, p) if dtype == torch.float32 else lib().oracle_pow(x, p)
+
+
+def pow_array(x: torch.Tensor, p: float) -> torch.Tensor:
+    """Elementwise x ** p of the oracle (p is rounded to x's dtype, as ATen does)."""
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    if x.dtype == torch.float32:
+        lib().oracle_powf_array(_p(x), C.c_float(p), _p(out), C.c_int64(x.numel()))
+    else:
+        lib().oracle_pow_array(_p(x), C.c_double(p), _p(out), C.c_int64(x.numel()))
+    return out
 
 
 def solve(cfg: Config, params, y0, t_eval=None, *, t_start=None, t_end=None, dt0=None, trace_iters=0, trace_B=0):

@@ -15,12 +15,12 @@
  * erk_oracle_impl.h), with explicit fma() and floating point contraction
  * switched off at compile time.
  *
- * Deviations from an ATen evaluation, both on purpose and both harmless at
- * the stated tolerances:
- *   - pow() is oracle_pow_core below, a fixed sequence of IEEE double
- *     operations (so that an independent implementation can reproduce it
- *     bit for bit), not the vectorised library pow ATen calls;
- *   - Tsit5's dense output weights come from an exact rational expansion.
+ * Third-party arithmetic: the reference's pow runs in ATen, which calls the
+ * SLEEF library's vectorised pow (vendored in PyTorch 2.10's third_party/sleef).
+ * Its published algorithm is restated below and reproduces torch.pow bit for
+ * bit (tests/test_oracle_pins.py).  Remaining deliberate deviation: Tsit5's
+ * dense output weights come from an exact rational expansion (the reference
+ * expands in floating point with sympy; last-ulp differences at most).
  *
  * Reference sites (torchode source tree):
  *   loop                adjoints.py:50-309
@@ -45,74 +45,168 @@
 #include "erk_oracle.h"
 
 /* ------------------------------------------------------------------------- */
-/* pow(x, p) for x >= 0 as a fixed sequence of double operations:            */
-/*   x = m 2^e, m in [1/sqrt2, sqrt2);  s = (m-1)/(m+1);                      */
-/*   ln m = 2 s + s^3 (2/3 + 2 s^2/5 + ... + 2 s^18/21)                        */
-/*   y = p (e + ln m / ln 2);  n = rint(y);  r = (y - n) ln 2                  */
-/*   result = ldexp(sum_{i<=13} r^i / i!, n)                                   */
-/* Relative error about 2e-15 for |y| < 20.                                   */
+/* pow.  ATen's CPU kernels evaluate tensor ** scalar with the vectorised pow  */
+/* of the SLEEF library (Sleef_powf*_u10 / Sleef_powd*_u10, FMA variants):     */
+/* pow(x, y) = expk(logk(|x|) * y) in double-word arithmetic.  The published   */
+/* algorithm is restated here operation by operation (every product, sum and   */
+/* fused multiply-add is one IEEE operation in the working type), so that the  */
+/* oracle reproduces ATen's results bit for bit and an independent             */
+/* implementation can reproduce the oracle's.  Special cases are restated for  */
+/* x >= 0 or NaN, which is all the solver produces.                            */
 /* ------------------------------------------------------------------------- */
-double oracle_pow_core(double x, double p) {
-    if (p == 0.0) return 1.0;
-    if (x != x || p != p) return NAN;
-    if (x == 1.0) return 1.0;
-    if (x < 0.0) return NAN;
-    if (x == 0.0) return p > 0.0 ? 0.0 : INFINITY;
-    if (isinf(x)) return p > 0.0 ? INFINITY : 0.0;
-    if (isinf(p)) return ((x < 1.0) == (p > 0.0)) ? 0.0 : INFINITY;
+#define DW_DEFINE(T, P, FMA)                                                                                        \
+    typedef struct { T x, y; } P##2;                                                                                \
+    static inline P##2 P##mk(T x, T y) { P##2 r = {x, y}; return r; }                                               \
+    static inline T P##fmapn(T x, T y, T z) { return FMA(x, y, -z); }                                               \
+    static inline T P##fmanp(T x, T y, T z) { return FMA(-x, y, z); }                                               \
+    static inline P##2 P##add2_s_s(T x, T y) { T s = x + y; T v = s - x; return P##mk(s, (x - (s - v)) + (y - v)); } \
+    static inline P##2 P##add2_d_s(P##2 x, T y) { T s = x.x + y; T v = s - x.x; T t = (x.x - (s - v)) + (y - v); return P##mk(s, t + x.y); } \
+    static inline P##2 P##add_s_d(T x, P##2 y) { T s = x + y.x; return P##mk(s, ((x - s) + y.x) + y.y); }            \
+    static inline P##2 P##add_d_d(P##2 x, P##2 y) { T s = x.x + y.x; return P##mk(s, (((x.x - s) + y.x) + x.y) + y.y); } \
+    static inline P##2 P##add2_d_d(P##2 x, P##2 y) { T s = x.x + y.x; T v = s - x.x; T t = (x.x - (s - v)) + (y.x - v); return P##mk(s, t + (x.y + y.y)); } \
+    static inline P##2 P##scale(P##2 d, T s) { return P##mk(d.x * s, d.y * s); }                                    \
+    static inline P##2 P##normalize(P##2 t) { T s = t.x + t.y; return P##mk(s, (t.x - s) + t.y); }                  \
+    static inline P##2 P##div(P##2 n, P##2 d) {                                                                     \
+        T t = (T)1 / d.x; T s = n.x * t; T u = P##fmapn(t, n.x, s);                                                 \
+        T v = P##fmanp(d.y, t, P##fmanp(d.x, t, (T)1));                                                             \
+        return P##mk(s, FMA(s, v, FMA(n.y, t, u)));                                                                 \
+    }                                                                                                               \
+    static inline P##2 P##squ(P##2 x) { T s = x.x * x.x; return P##mk(s, FMA(x.x + x.x, x.y, P##fmapn(x.x, x.x, s))); } \
+    static inline P##2 P##mul_d_s(P##2 x, T y) { T s = x.x * y; return P##mk(s, FMA(x.y, y, P##fmapn(x.x, y, s))); }  \
+    static inline P##2 P##mul_d_d(P##2 x, P##2 y) { T s = x.x * y.x; return P##mk(s, FMA(x.x, y.y, FMA(x.y, y.x, P##fmapn(x.x, y.x, s)))); }
 
-    uint64_t bits;
-    memcpy(&bits, &x, 8);
-    int e = (int)((bits >> 52) & 0x7ff);
-    if (e == 0) { /* subnormal: renormalise */
-        x = x * 18014398509481984.0; /* 2^54 */
-        memcpy(&bits, &x, 8);
-        e = (int)((bits >> 52) & 0x7ff) - 54;
-    }
-    e -= 1023;
-    bits = (bits & 0x000fffffffffffffULL) | 0x3ff0000000000000ULL;
+DW_DEFINE(float, df, fmaf)
+DW_DEFINE(double, dd, fma)
+
+/* ---- float ---- */
+static inline float f_pow2i(int q) { int32_t i = (int32_t)(q + 0x7f) << 23; float f; memcpy(&f, &i, 4); return f; }
+static inline float f_ldexp2k(float d, int e) { return d * f_pow2i(e >> 1) * f_pow2i(e - (e >> 1)); }
+
+static df2 f_logk(float d) {
+    int o = d < 1.17549435e-38f;
+    if (o) d = d * ((float)(INT64_C(1) << 32) * (float)(INT64_C(1) << 32));
+    float d43 = d * (1.0f / 0.75f);
+    int32_t bits;
+    memcpy(&bits, &d43, 4);
+    int e = ((bits >> 23) & 0xff) - 0x7f;
+    memcpy(&bits, &d, 4);
+    bits -= e << 23; /* d * 2^-e by exponent arithmetic */
+    float m;
+    memcpy(&m, &bits, 4);
+    if (o) e -= 64;
+    df2 x = dfdiv(dfadd2_s_s(-1.0f, m), dfadd2_s_s(1.0f, m));
+    df2 x2 = dfsqu(x);
+    float t = 0.240320354700088500976562f;
+    t = fmaf(t, x2.x, 0.285112679004669189453125f);
+    t = fmaf(t, x2.x, 0.400007992982864379882812f);
+    df2 c = dfmk(0.66666662693023681640625f, 3.69183861259614332084311e-09f);
+    df2 s = dfmul_d_s(dfmk(0.69314718246459960938f, -1.904654323148236017e-09f), (float)e);
+    s = dfadd_d_d(s, dfscale(x, 2.0f));
+    s = dfadd_d_d(s, dfmul_d_d(dfmul_d_d(x2, x), dfadd2_d_d(dfmul_d_s(x2, t), c)));
+    return s;
+}
+
+static float f_expk(df2 d) {
+    float u = (d.x + d.y) * 1.442695040888963407359924681001892137426645954152985934135449406931f;
+    float fq = rintf(u);
+    int q = (int)fq;
+    df2 s = dfadd2_d_s(d, fq * -0.693145751953125f);
+    s = dfadd2_d_s(s, fq * -1.428606765330187045e-06f);
+    s = dfnormalize(s);
+    u = 0.00136324646882712841033936f;
+    u = fmaf(u, s.x, 0.00836596917361021041870117f);
+    u = fmaf(u, s.x, 0.0416710823774337768554688f);
+    u = fmaf(u, s.x, 0.166665524244308471679688f);
+    u = fmaf(u, s.x, 0.499999850988388061523438f);
+    df2 t = dfadd_d_d(s, dfmul_d_s(dfsqu(s), u));
+    t = dfadd_s_d(1.0f, t);
+    u = t.x + t.y;
+    u = f_ldexp2k(u, q);
+    if (d.x < -104.0f) u = 0.0f;
+    return u;
+}
+
+float oracle_powf(float x, float y) {
+    if (y == 0.0f || x == 1.0f) return 1.0f;
+    if (x != x || y != y) return NAN;
+    if (x < 0.0f) return NAN; /* not produced by the solver (negative base, non-integer exponent) */
+    if (isinf(x) || x == 0.0f) return (((x == 0.0f) ? -y : y) < 0.0f) ? 0.0f : INFINITY;
+    if (isinf(y)) { float efx = (y < 0 ? -1.0f : 1.0f) * (x - 1.0f); return efx < 0 ? 0.0f : (efx == 0 ? 1.0f : INFINITY); }
+    float r = f_expk(dfmul_d_s(f_logk(x), y));
+    return (r != r) ? INFINITY : r;
+}
+
+/* ---- double ---- */
+static inline double d_pow2i(int q) { int64_t i = (int64_t)(q + 0x3ff) << 52; double f; memcpy(&f, &i, 8); return f; }
+static inline double d_ldexp2k(double d, int e) { return d * d_pow2i(e >> 1) * d_pow2i(e - (e >> 1)); }
+
+static dd2 d_logk(double d) {
+    int o = d < 2.2250738585072014e-308;
+    if (o) d = d * ((double)(INT64_C(1) << 32) * (double)(INT64_C(1) << 32));
+    double d43 = d * (1.0 / 0.75);
+    int64_t bits;
+    memcpy(&bits, &d43, 8);
+    int e = (int)((bits >> 52) & 0x7ff) - 0x3ff;
+    memcpy(&bits, &d, 8);
+    bits -= (int64_t)e << 52;
     double m;
     memcpy(&m, &bits, 8);
-    if (m > 1.4142135623730951) {
-        m = m * 0.5;
-        e += 1;
-    }
-    double s = (m - 1.0) / (m + 1.0);
-    double z = s * s;
-    double q = 2.0 / 21.0;
-    q = fma(q, z, 2.0 / 19.0);
-    q = fma(q, z, 2.0 / 17.0);
-    q = fma(q, z, 2.0 / 15.0);
-    q = fma(q, z, 2.0 / 13.0);
-    q = fma(q, z, 2.0 / 11.0);
-    q = fma(q, z, 2.0 / 9.0);
-    q = fma(q, z, 2.0 / 7.0);
-    q = fma(q, z, 2.0 / 5.0);
-    q = fma(q, z, 2.0 / 3.0);
-    double s3 = s * z;
-    double lnm = fma(s3, q, 2.0 * s);
-    double l2 = fma(lnm, 1.4426950408889634, (double)e);
-    double y = p * l2;
-    if (y > 1100.0) return INFINITY;
-    if (y < -1100.0) return 0.0;
-    double n = rint(y);
-    double r = (y - n) * 0.6931471805599453;
-    double v = 1.0 / 6227020800.0;
-    v = fma(v, r, 1.0 / 479001600.0);
-    v = fma(v, r, 1.0 / 39916800.0);
-    v = fma(v, r, 1.0 / 3628800.0);
-    v = fma(v, r, 1.0 / 362880.0);
-    v = fma(v, r, 1.0 / 40320.0);
-    v = fma(v, r, 1.0 / 5040.0);
-    v = fma(v, r, 1.0 / 720.0);
-    v = fma(v, r, 1.0 / 120.0);
-    v = fma(v, r, 1.0 / 24.0);
-    v = fma(v, r, 1.0 / 6.0);
-    v = fma(v, r, 0.5);
-    v = fma(v, r, 1.0);
-    v = fma(v, r, 1.0);
-    return ldexp(v, (int)n);
+    if (o) e -= 64;
+    dd2 x = dddiv(ddadd2_s_s(-1.0, m), ddadd2_s_s(1.0, m));
+    dd2 x2 = ddsqu(x);
+    double z = x2.x, z2 = z * z, z4 = z2 * z2, z8 = z4 * z4;
+    /* Estrin evaluation of a degree-8 polynomial in z */
+    double p01 = fma(z, 0.285714285714249172087875, 0.400000000000000077715612);
+    double p23 = fma(z, 0.181818180850050775676507, 0.222222222230083560345903);
+    double p45 = fma(z, 0.13332981086846273921509, 0.153846227114512262845736);
+    double p67 = fma(z, 0.103239680901072952701192, 0.117754809412463995466069);
+    double lo = fma(z2, p23, p01), hi = fma(z2, p67, p45);
+    double t = fma(z8, 0.116255524079935043668677, fma(z4, hi, lo));
+    dd2 c = ddmk(0.666666666666666629659233, 3.80554962542412056336616e-17);
+    dd2 s = ddmul_d_s(ddmk(0.693147180559945286226764, 2.319046813846299558417771e-17), (double)e);
+    s = ddadd_d_d(s, ddscale(x, 2.0));
+    x = ddmul_d_d(x2, x);
+    s = ddadd_d_d(s, ddmul_d_d(x, c));
+    x = ddmul_d_d(x2, x);
+    s = ddadd_d_d(s, ddmul_d_s(x, t));
+    return s;
 }
+
+static double d_expk(dd2 d) {
+    double u = (d.x + d.y) * 1.442695040888963407359924681001892137426645954152985934135449406931;
+    double dq = rint(u);
+    int q = (int)dq;
+    dd2 s = ddadd2_d_s(d, dq * -.69314718055966295651160180568695068359375);
+    s = ddadd2_d_s(s, dq * -.28235290563031577122588448175013436025525412068e-12);
+    s = ddnormalize(s);
+    double z = s.x, z2 = z * z, z4 = z2 * z2, z8 = z4 * z4;
+    double p01 = fma(z, 0.166666666666666740681535, 0.500000000000000999200722);
+    double p23 = fma(z, 0.00833333333332371417601081, 0.0416666666665409524128449);
+    double p45 = fma(z, 0.000198412698809069797676111, 0.0013888888939977128960529);
+    double p67 = fma(z, 2.75572496725023574143864e-06, 2.48014973989819794114153e-05);
+    double p89 = fma(z, 2.51069683420950419527139e-08, 2.76286166770270649116855e-07);
+    double lo = fma(z2, p23, p01), hi = fma(z2, p67, p45);
+    u = fma(z8, p89, fma(z4, hi, lo));
+    dd2 t = ddadd_s_d(1.0, s);
+    t = ddadd_d_d(t, ddmul_d_s(ddsqu(s), u));
+    u = t.x + t.y;
+    u = d_ldexp2k(u, q);
+    if (d.x < -1000.0) u = 0.0;
+    return u;
+}
+
+double oracle_pow(double x, double y) {
+    if (y == 0.0 || x == 1.0) return 1.0;
+    if (x != x || y != y) return NAN;
+    if (x < 0.0) return NAN;
+    if (isinf(x) || x == 0.0) return (((x == 0.0) ? -y : y) < 0.0) ? 0.0 : INFINITY;
+    if (isinf(y)) { double efx = (y < 0 ? -1.0 : 1.0) * (x - 1.0); return efx < 0 ? 0.0 : (efx == 0 ? 1.0 : INFINITY); }
+    double r = d_expk(ddmul_d_s(d_logk(x), y));
+    return (r != r) ? INFINITY : r;
+}
+
+void oracle_powf_array(const float *x, float y, float *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = oracle_powf(x[i], y); }
+void oracle_pow_array(const double *x, double y, double *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = oracle_pow(x[i], y); }
 
 /* ------------------------------------------------------------------------- */
 /* Butcher tableaux (float64, cast per use)                                   */
@@ -199,7 +293,9 @@ const oracle_tableau *oracle_get_tableau(int method) {
 #define R_SQRT(a) sqrtf(a)
 #define R_ABS(a) fabsf(a)
 #define R_ISFINITE(a) isfinite(a)
+#define R_POW(x, p) oracle_powf((x), (float)(p))
 #include "erk_oracle_impl.h"
+#undef R_POW
 #undef REAL
 #undef SFX
 #undef R_FMA
@@ -213,4 +309,5 @@ const oracle_tableau *oracle_get_tableau(int method) {
 #define R_SQRT(a) sqrt(a)
 #define R_ABS(a) fabs(a)
 #define R_ISFINITE(a) isfinite(a)
+#define R_POW(x, p) oracle_pow((x), (double)(p))
 #include "erk_oracle_impl.h"

@@ -36,7 +36,10 @@ typedef struct {
     int64_t max_steps; /* < 0: none */
 } oracle_config;
 
-double oracle_pow_core(double x, double p);
+float oracle_powf(float x, float y);
+double oracle_pow(double x, double y);
+void oracle_powf_array(const float *x, float y, float *out, int64_t n);
+void oracle_pow_array(const double *x, double y, double *out, int64_t n);
 const oracle_tableau *oracle_get_tableau(int method);
 
 #define ORACLE_DECLARE(REAL, SFX)                                                                                      \

@@ -10,8 +10,8 @@ static inline REAL SFX(tmin)(REAL a, REAL b) { return (a != a) ? a : ((b != b) ?
 static inline REAL SFX(tclamp)(REAL x, REAL lo, REAL hi) { return SFX(tmin)(SFX(tmax)(x, lo), hi); }
 
 /* pow in the tensor dtype with the exponent rounded to that dtype first
- * (ATen pow(Tensor, Scalar)); evaluated through oracle_pow_core in double. */
-static inline REAL SFX(rpow)(REAL x, double p) { return (REAL)oracle_pow_core((double)x, (double)(REAL)p); }
+ * (ATen pow(Tensor, Scalar)). */
+static inline REAL SFX(rpow)(REAL x, double p) { return R_POW(x, (REAL)p); }
 
 /* ---- built-in right-hand sides, canonical op order, every op rounded on its own ---- */
 static void SFX(rhs)(const oracle_config *cfg, const REAL *par, REAL t, const REAL *y, REAL *dy, int F) {

@@ -143,9 +143,12 @@ def test_oracle_reproduces_golden_fixture(path):
     cfg = c_oracle.make_config(method=g["method"], term=g["workload"], nthreads=4, **g["controller"])
     out = c_oracle.solve(cfg, w.f.builtin_params(), w.y0, w.t_eval)
     for key in ("n_steps", "n_accepted", "n_initialized", "status"):
-        assert out[key].tolist() == g[key], key
+        if isinstance(g[key], dict):
+            assert _sha(out[key]) == g[key]["sha256_int64"] and int(out[key].sum()) == g[key]["sum"], key
+        else:
+            assert out[key].tolist() == g[key], key
+    assert _sha(out["ys"]) == g["ys_sha256"]
     assert int(out["n_f_evals"][0]) == g["n_f_evals"]
     got = [float(v).hex() for v in out["ys"][g["subset"]].flatten().tolist()]
     assert got == g["ys_subset"]
-    ys = out["ys"].double()
-    assert float(ys.sum()).hex() == g["ys_sum"] and float((ys * ys).sum()).hex() == g["ys_sum_sq"]
+    assert float(out["ys"].double().abs().max()).hex() == g["ys_max_abs"]

@@ -253,17 +253,25 @@ def test_time_reversal_round_trip():
 # ---- against the ATen-op restatement (closest stand-in for the reference itself) -----
 
 
-@pytest.mark.parametrize("name,dtype,tol", [("linear_decay", F64, 1e-10), ("lorenz", F64, 1e-8), ("vdp", F64, 1e-7)])
-def test_against_aten_restatement_float64(name, dtype, tol):
-    """The only arithmetic difference to an ATen evaluation is pow (fixed double sequence here,
-    vectorised library pow there); it perturbs dt in the last ulp, which the noise-dominated
-    first error ratios amplify.  Integer stats must still agree on >= 99.9 % of samples."""
-    w = to.workloads.make(name, batch=1024 if name != "linear_decay" else 256, dtype=dtype)
+@pytest.mark.parametrize("name,batch,dtype", [("vdp", 2048, F32), ("lorenz", 1024, F64)])
+def test_against_live_aten_restatement(name, batch, dtype):
+    """On a host whose ATen CPU kernels round like the one the oracle was pinned on, the loop
+    issued as ATen operations and the kernels agree bit for bit (bar: 1e-4 / 1e-10, stats on
+    99.9 % of samples).  On other hosts ATen itself computes different bits (its BLAS picks other
+    kernels), so only a loose sanity bound is checked there; the pinned values are in the golden
+    fixtures below."""
+    from helpers import aten_host_matches
+
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
     sol = gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
     ref = torch_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
-    same = (sol.stats["n_steps"].cpu() == ref["n_steps"]) & (sol.stats["n_accepted"].cpu() == ref["n_accepted"])
-    assert same.float().mean().item() >= 0.999
-    assert mixed_error(sol.ys.cpu(), ref["ys"]) < tol
+    if aten_host_matches():
+        assert_identical(sol, ref)
+    else:
+        close = (sol.stats["n_steps"].cpu() - ref["n_steps"]).abs() <= 3
+        assert close.float().mean().item() > 0.9
+        err = (sol.ys.cpu() - ref["ys"]).abs()
+        assert (err <= 5e-2 * (1 + ref["ys"].abs())).float().mean().item() > 0.999
 
 
 # ---- committed golden fixtures (tests/golden/*.json, written by tests/golden/make_golden.py) ----
@@ -278,15 +286,23 @@ _GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__
 @pytest.mark.parametrize("fast", [True, False], ids=["fast", "general"])
 @pytest.mark.parametrize("path", _GOLDEN, ids=os.path.basename)
 def test_gpu_matches_golden_fixture(path, fast):
+    """Golden vectors of the ATen-op restatement, written in the authoring container."""
+    import hashlib
+
     g = json.load(open(path))
     dtype = getattr(torch, g["dtype"])
     w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    sha = lambda t: hashlib.sha256(t.contiguous().numpy().tobytes()).hexdigest()
+    assert {"y0": sha(w.y0), "t_eval": sha(w.t_eval), "params": sha(w.f.builtin_params())} == g["inputs_sha256"]
     sol = gpu_solve(w.f, w.y0, w.t_eval, g["method"], g["controller"], fast=fast)
-    for key in ("n_steps", "n_accepted", "n_initialized"):
-        assert sol.stats[key].cpu().tolist() == g[key], key
-    assert sol.status.cpu().tolist() == g["status"]
+    got = dict(sol.stats, status=sol.status)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status"):
+        if isinstance(g[key], dict):
+            assert sha(got[key].cpu()) == g[key]["sha256_int64"] and int(got[key].sum()) == g[key]["sum"], key
+        else:
+            assert got[key].cpu().tolist() == g[key], key
+    assert sha(sol.ys.cpu()) == g["ys_sha256"]
     assert int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
     ys = sol.ys.cpu()
     assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
-    ysd = ys.double()
-    assert float(ysd.sum()).hex() == g["ys_sum"] and float((ysd * ysd).sum()).hex() == g["ys_sum_sq"]
+    assert float(ys.double().abs().max()).hex() == g["ys_max_abs"]

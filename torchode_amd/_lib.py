@@ -112,8 +112,8 @@ class StepState(C.Structure):
         ("dt", C.c_void_p),
         ("y", C.c_void_p),
         ("k0", C.c_void_p),
-        ("l2_prev", C.c_void_p),
-        ("l2_pprev", C.c_void_p),
+        ("ratio_prev", C.c_void_p),
+        ("ratio_pprev", C.c_void_p),
         ("running", C.c_void_p),
         ("cursor", C.c_void_p),
         ("n_steps", C.c_void_p),

@@ -112,7 +112,7 @@ class AutoDiffAdjoint(nn.Module):
         ys = new(B, max(E, 1), F)
         t, dt = new(B), new(B)
         y, k0 = new(B, F), new(B, F)
-        hist = new(2, B, dt=torch.float64)
+        hist = new(2, B)
         ints = new(6, B, dt=torch.int32)
         pending = new(B, max(E, 1), dt=torch.uint8)
         flags = new(_lib.STEP_FLAG_WORDS, dt=torch.int32)
@@ -124,7 +124,7 @@ class AutoDiffAdjoint(nn.Module):
         s.y0, s.t_start, s.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
         s.t_eval = None if t_eval is None else t_eval.data_ptr()
         s.t, s.dt, s.y, s.k0 = t.data_ptr(), dt.data_ptr(), y.data_ptr(), k0.data_ptr()
-        s.l2_prev, s.l2_pprev = hist[0].data_ptr(), hist[1].data_ptr()
+        s.ratio_prev, s.ratio_pprev = hist[0].data_ptr(), hist[1].data_ptr()
         s.running, s.cursor, s.n_steps, s.n_accepted, s.status, s.monotone = (ints[i].data_ptr() for i in range(6))
         s.pending, s.ys, s.flags = pending.data_ptr(), ys.data_ptr(), flags.data_ptr()
         sref, cref = _lib.C.byref(s), _lib.C.byref(ctrl)

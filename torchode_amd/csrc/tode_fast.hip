@@ -11,7 +11,7 @@
 //     lane's reads hit its own bank) instead of being fetched from HBM inside
 //     the loop, and -- when it fits -- the dense output is collected in LDS and
 //     written back at the end as one contiguous, fully coalesced block per wave;
-//   * the controller's powers share one logarithm per step.
+//   * the controller's powers share one double-word logarithm per step.
 // The arithmetic is the same sequence of IEEE operations as in the general
 // kernel (tode_persistent.hip), so the two produce identical bits.
 //
@@ -92,8 +92,8 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         dt = initial_step<T, CTRL, Term>(cp, rhs, ts, y, dir, abs_(te - ts), k[0]);
     }
     dt = tclamp(dt, tlo - t, thi - t);
-    // log2 of the previous two accepted error ratios (both start at 1, log2(1) = 0)
-    double l2_prev = 0.0, l2_pprev = 0.0;
+    // logarithms of the previous two accepted error ratios (both start at 1, log 1 = 0)
+    DW<T> lg_prev = dw((T)0, (T)0), lg_pprev = dw((T)0, (T)0);
     int cursor = 0;
     T *ys_g = p.ys + bs * (long long)EF;
     if (te_s[lane] == ts) {
@@ -113,7 +113,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
 
     int n_steps = 0, n_acc = 0;
     bool active = live && !bail;
-    const double e1 = (double)(T)cp.e1, e2 = (double)(T)cp.e2, e3 = (double)(T)cp.e3;
+    const T e1 = (T)cp.e1, e2 = (T)cp.e2, e3 = (T)cp.e3;
 
     while (__any(active)) {
         // ---- stages (runge_kutta.py:255-263) ----
@@ -143,10 +143,10 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         const bool accept = ratio < (T)1;
         // any ratio outside (0, inf) is a non-success status: leave it to the general kernel
         const bool sane = ratio > (T)0 && ratio < (T)__builtin_huge_val();
-        const double l2 = log2_normal(sane ? (double)ratio : 1.0);
-        T factor = cp.safety * (T)exp2_of(e1 * l2);
-        if (NHIST >= 1) factor = factor * (T)exp2_of(e2 * l2_prev);
-        if (NHIST >= 2) factor = factor * (T)exp2_of(e3 * l2_pprev);
+        const DW<T> lg = logk(sane ? ratio : (T)1);
+        T factor = cp.safety * powk<T>(lg, e1);
+        if (NHIST >= 1) factor = factor * powk<T>(lg_prev, e2);
+        if (NHIST >= 2) factor = factor * powk<T>(lg_pprev, e3);
         factor = tclamp(factor, cp.fmin, cp.fmax);
         const T dt_next = dt * factor;
 
@@ -195,8 +195,12 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         }
         if (NHIST >= 1) {
             const bool shift = active && running_new && accept;
-            if (NHIST >= 2) l2_pprev = shift ? l2_prev : l2_pprev;
-            l2_prev = shift ? l2 : l2_prev;
+            if (NHIST >= 2) {
+                lg_pprev.x = shift ? lg_prev.x : lg_pprev.x;
+                lg_pprev.y = shift ? lg_prev.y : lg_pprev.y;
+            }
+            lg_prev.x = shift ? lg.x : lg_prev.x;
+            lg_prev.y = shift ? lg.y : lg_prev.y;
         }
         {
             // non-finite error ratio or max_steps reached: not the common case

@@ -41,120 +41,185 @@ template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return __bui
 template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return __builtin_isunordered(a, b) ? nan_<T>() : hwmin(a, b); }
 template <typename T> __device__ __forceinline__ T tclamp(T x, T lo, T hi) { return tmin(tmax(x, lo), hi); }
 
-// pow(x, p) for x >= 0:  x = m 2^e with m in [1/sqrt2, sqrt2), s = (m-1)/(m+1),
-// ln m = 2s + s^3 (2/3 + 2 s^2/5 + ... + 2 s^18/21), y = p (e + ln m / ln 2),
-// n = rint(y), r = (y-n) ln 2, result = ldexp(sum_{i<=13} r^i/i!, n).
-// Relative error about 2e-15 for |y| < 20.
-__device__ __forceinline__ double pow_core(double x, double p) {
-    if (p == 0.0) return 1.0;
-    if (x != x || p != p) return __builtin_nan("");
-    if (x == 1.0) return 1.0;
-    if (x < 0.0) return __builtin_nan("");
-    if (x == 0.0) return p > 0.0 ? 0.0 : __builtin_huge_val();
-    if (x == __builtin_huge_val()) return p > 0.0 ? __builtin_huge_val() : 0.0;
-    if (__builtin_fabs(p) == __builtin_huge_val()) return ((x < 1.0) == (p > 0.0)) ? 0.0 : __builtin_huge_val();
+// ---------------------------------------------------------------------------
+// pow.  The reference's `tensor ** python_float` is evaluated by ATen's CPU kernels with
+// the SLEEF library's vectorised pow (u10, FMA variants): pow(x, y) = expk(logk(|x|) * y)
+// in double-word arithmetic.  That published algorithm is written out here operation by
+// operation -- every sum, product and fma below is one IEEE operation in the working
+// type -- which makes the device result identical, bit for bit, to what the reference
+// computes on the host.  logk() and expk() are exposed separately so that a caller can
+// reuse one logarithm for several exponents.  Special cases are covered for x >= 0 or
+// NaN, which is all the step size controllers produce.
+// ---------------------------------------------------------------------------
+template <typename T> struct DW { T x, y; };  // unevaluated sum x + y, |y| <= ulp(x)/2
 
-    uint64_t bits = (uint64_t)__double_as_longlong(x);
-    int e = (int)((bits >> 52) & 0x7ff);
-    if (e == 0) {
-        x = x * 18014398509481984.0;
-        bits = (uint64_t)__double_as_longlong(x);
-        e = (int)((bits >> 52) & 0x7ff) - 54;
-    }
-    e -= 1023;
-    bits = (bits & 0x000fffffffffffffULL) | 0x3ff0000000000000ULL;
-    double m = __longlong_as_double((long long)bits);
-    if (m > 1.4142135623730951) {
-        m = m * 0.5;
-        e += 1;
-    }
-    double s = (m - 1.0) / (m + 1.0);
-    double z = s * s;
-    double q = 2.0 / 21.0;
-    q = __builtin_fma(q, z, 2.0 / 19.0);
-    q = __builtin_fma(q, z, 2.0 / 17.0);
-    q = __builtin_fma(q, z, 2.0 / 15.0);
-    q = __builtin_fma(q, z, 2.0 / 13.0);
-    q = __builtin_fma(q, z, 2.0 / 11.0);
-    q = __builtin_fma(q, z, 2.0 / 9.0);
-    q = __builtin_fma(q, z, 2.0 / 7.0);
-    q = __builtin_fma(q, z, 2.0 / 5.0);
-    q = __builtin_fma(q, z, 2.0 / 3.0);
-    double s3 = s * z;
-    double lnm = __builtin_fma(s3, q, 2.0 * s);
-    double l2 = __builtin_fma(lnm, 1.4426950408889634, (double)e);
-    double y = p * l2;
-    if (y > 1100.0) return __builtin_huge_val();
-    if (y < -1100.0) return 0.0;
-    double n = __builtin_rint(y);
-    double r = (y - n) * 0.6931471805599453;
-    double v = 1.0 / 6227020800.0;
-    v = __builtin_fma(v, r, 1.0 / 479001600.0);
-    v = __builtin_fma(v, r, 1.0 / 39916800.0);
-    v = __builtin_fma(v, r, 1.0 / 3628800.0);
-    v = __builtin_fma(v, r, 1.0 / 362880.0);
-    v = __builtin_fma(v, r, 1.0 / 40320.0);
-    v = __builtin_fma(v, r, 1.0 / 5040.0);
-    v = __builtin_fma(v, r, 1.0 / 720.0);
-    v = __builtin_fma(v, r, 1.0 / 120.0);
-    v = __builtin_fma(v, r, 1.0 / 24.0);
-    v = __builtin_fma(v, r, 1.0 / 6.0);
-    v = __builtin_fma(v, r, 0.5);
-    v = __builtin_fma(v, r, 1.0);
-    v = __builtin_fma(v, r, 1.0);
-    return __builtin_ldexp(v, (int)n);
+template <typename T> __device__ __forceinline__ DW<T> dw(T x, T y) { return DW<T>{x, y}; }
+template <typename T> __device__ __forceinline__ T fmapn(T x, T y, T z) { return fma_(x, y, -z); }
+template <typename T> __device__ __forceinline__ T fmanp(T x, T y, T z) { return fma_(-x, y, z); }
+template <typename T> __device__ __forceinline__ DW<T> dw_add2(T x, T y) {
+    T s = x + y, v = s - x;
+    return dw(s, (x - (s - v)) + (y - v));
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_add2(DW<T> x, T y) {
+    T s = x.x + y, v = s - x.x;
+    T t = (x.x - (s - v)) + (y - v);
+    return dw(s, t + x.y);
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_add(T x, DW<T> y) {
+    T s = x + y.x;
+    return dw(s, ((x - s) + y.x) + y.y);
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_add(DW<T> x, DW<T> y) {
+    T s = x.x + y.x;
+    return dw(s, (((x.x - s) + y.x) + x.y) + y.y);
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_add2(DW<T> x, DW<T> y) {
+    T s = x.x + y.x, v = s - x.x;
+    T t = (x.x - (s - v)) + (y.x - v);
+    return dw(s, t + (x.y + y.y));
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_scale(DW<T> d, T s) { return dw(d.x * s, d.y * s); }
+template <typename T> __device__ __forceinline__ DW<T> dw_normalize(DW<T> t) {
+    T s = t.x + t.y;
+    return dw(s, (t.x - s) + t.y);
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_div(DW<T> n, DW<T> d) {
+    T t = (T)1 / d.x;
+    T s = n.x * t;
+    T u = fmapn(t, n.x, s);
+    T v = fmanp(d.y, t, fmanp(d.x, t, (T)1));
+    return dw(s, fma_(s, v, fma_(n.y, t, u)));
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_squ(DW<T> x) {
+    T s = x.x * x.x;
+    return dw(s, fma_(x.x + x.x, x.y, fmapn(x.x, x.x, s)));
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_mul(DW<T> x, T y) {
+    T s = x.x * y;
+    return dw(s, fma_(x.y, y, fmapn(x.x, y, s)));
+}
+template <typename T> __device__ __forceinline__ DW<T> dw_mul(DW<T> x, DW<T> y) {
+    T s = x.x * y.x;
+    return dw(s, fma_(x.x, y.y, fma_(x.y, y.x, fmapn(x.x, y.x, s))));
 }
 
-// The two halves of pow_core for arguments that need none of its special cases:
-// log2_normal(x) for a positive, finite, normal x, and exp2_of(y) for |y| <= 1016.
-// pow_core(x, p) == exp2_of(p * log2_normal(x)) bit for bit on that domain, which lets
-// a caller reuse one logarithm for several exponents.
-__device__ __forceinline__ double log2_normal(double x) {
-    const unsigned hi = (unsigned)__double2hiint(x);
-    int e = (int)((hi >> 20) & 0x7ff) - 1023;
-    double m = __hiloint2double((int)((hi & 0x000fffffu) | 0x3ff00000u), __double2loint(x));
-    const bool big = m > 1.4142135623730951;
-    m = big ? m * 0.5 : m;
-    e = big ? e + 1 : e;
-    double s = (m - 1.0) / (m + 1.0);
-    double z = s * s;
-    double q = 2.0 / 21.0;
-    q = __builtin_fma(q, z, 2.0 / 19.0);
-    q = __builtin_fma(q, z, 2.0 / 17.0);
-    q = __builtin_fma(q, z, 2.0 / 15.0);
-    q = __builtin_fma(q, z, 2.0 / 13.0);
-    q = __builtin_fma(q, z, 2.0 / 11.0);
-    q = __builtin_fma(q, z, 2.0 / 9.0);
-    q = __builtin_fma(q, z, 2.0 / 7.0);
-    q = __builtin_fma(q, z, 2.0 / 5.0);
-    q = __builtin_fma(q, z, 2.0 / 3.0);
-    double s3 = s * z;
-    double lnm = __builtin_fma(s3, q, 2.0 * s);
-    return __builtin_fma(lnm, 1.4426950408889634, (double)e);
+// ---- float ----
+__device__ __forceinline__ float pow2i(float, int q) { return __int_as_float((q + 0x7f) << 23); }
+__device__ __forceinline__ double pow2i(double, int q) { return __longlong_as_double((long long)(q + 0x3ff) << 52); }
+template <typename T> __device__ __forceinline__ T ldexp2k(T d, int e) { return d * pow2i(T(0), e >> 1) * pow2i(T(0), e - (e >> 1)); }
+
+// log of a positive finite d as a double-word
+__device__ __forceinline__ DW<float> logk(float d) {
+    const bool o = d < 1.17549435e-38f;
+    d = o ? d * 18446744073709551616.0f : d;  // 2^64
+    const float d43 = d * (1.0f / 0.75f);
+    int e = ((__float_as_int(d43) >> 23) & 0xff) - 0x7f;
+    const float m = __int_as_float(__float_as_int(d) - (e << 23));  // d * 2^-e
+    e = o ? e - 64 : e;
+    DW<float> x = dw_div(dw_add2(-1.0f, m), dw_add2(1.0f, m));
+    DW<float> x2 = dw_squ(x);
+    float t = 0.240320354700088500976562f;
+    t = fma_(t, x2.x, 0.285112679004669189453125f);
+    t = fma_(t, x2.x, 0.400007992982864379882812f);
+    const DW<float> c = dw(0.66666662693023681640625f, 3.69183861259614332084311e-09f);
+    DW<float> s = dw_mul(dw(0.69314718246459960938f, -1.904654323148236017e-09f), (float)e);
+    s = dw_add(s, dw_scale(x, 2.0f));
+    s = dw_add(s, dw_mul(dw_mul(x2, x), dw_add2(dw_mul(x2, t), c)));
+    return s;
 }
 
-__device__ __forceinline__ double exp2_of(double y) {
-    double n = __builtin_rint(y);
-    double r = (y - n) * 0.6931471805599453;
-    double v = 1.0 / 6227020800.0;
-    v = __builtin_fma(v, r, 1.0 / 479001600.0);
-    v = __builtin_fma(v, r, 1.0 / 39916800.0);
-    v = __builtin_fma(v, r, 1.0 / 3628800.0);
-    v = __builtin_fma(v, r, 1.0 / 362880.0);
-    v = __builtin_fma(v, r, 1.0 / 40320.0);
-    v = __builtin_fma(v, r, 1.0 / 5040.0);
-    v = __builtin_fma(v, r, 1.0 / 720.0);
-    v = __builtin_fma(v, r, 1.0 / 120.0);
-    v = __builtin_fma(v, r, 1.0 / 24.0);
-    v = __builtin_fma(v, r, 1.0 / 6.0);
-    v = __builtin_fma(v, r, 0.5);
-    v = __builtin_fma(v, r, 1.0);
-    v = __builtin_fma(v, r, 1.0);
-    return __builtin_ldexp(v, (int)n);
+// exp of a double-word
+__device__ __forceinline__ float expk(DW<float> d) {
+    float u = (d.x + d.y) * 1.442695040888963407359924681001892137426645954152985934135449406931f;
+    const float fq = __builtin_rintf(u);
+    const int q = (int)fq;
+    DW<float> s = dw_add2(d, fq * -0.693145751953125f);
+    s = dw_add2(s, fq * -1.428606765330187045e-06f);
+    s = dw_normalize(s);
+    u = 0.00136324646882712841033936f;
+    u = fma_(u, s.x, 0.00836596917361021041870117f);
+    u = fma_(u, s.x, 0.0416710823774337768554688f);
+    u = fma_(u, s.x, 0.166665524244308471679688f);
+    u = fma_(u, s.x, 0.499999850988388061523438f);
+    DW<float> t = dw_add(s, dw_mul(dw_squ(s), u));
+    t = dw_add(1.0f, t);
+    u = t.x + t.y;
+    u = ldexp2k(u, q);
+    return d.x < -104.0f ? 0.0f : u;
+}
+
+// ---- double ----
+__device__ __forceinline__ DW<double> logk(double d) {
+    const bool o = d < 2.2250738585072014e-308;
+    d = o ? d * 18446744073709551616.0 : d;
+    const double d43 = d * (1.0 / 0.75);
+    int e = (int)((__double2hiint(d43) >> 20) & 0x7ff) - 0x3ff;
+    const double m = __hiloint2double(__double2hiint(d) - (e << 20), __double2loint(d));
+    e = o ? e - 64 : e;
+    DW<double> x = dw_div(dw_add2(-1.0, m), dw_add2(1.0, m));
+    DW<double> x2 = dw_squ(x);
+    const double z = x2.x, z2 = z * z, z4 = z2 * z2, z8 = z4 * z4;
+    const double p01 = fma_(z, 0.285714285714249172087875, 0.400000000000000077715612);
+    const double p23 = fma_(z, 0.181818180850050775676507, 0.222222222230083560345903);
+    const double p45 = fma_(z, 0.13332981086846273921509, 0.153846227114512262845736);
+    const double p67 = fma_(z, 0.103239680901072952701192, 0.117754809412463995466069);
+    const double lo = fma_(z2, p23, p01), hi = fma_(z2, p67, p45);
+    const double t = fma_(z8, 0.116255524079935043668677, fma_(z4, hi, lo));
+    const DW<double> c = dw(0.666666666666666629659233, 3.80554962542412056336616e-17);
+    DW<double> s = dw_mul(dw(0.693147180559945286226764, 2.319046813846299558417771e-17), (double)e);
+    s = dw_add(s, dw_scale(x, 2.0));
+    x = dw_mul(x2, x);
+    s = dw_add(s, dw_mul(x, c));
+    x = dw_mul(x2, x);
+    s = dw_add(s, dw_mul(x, t));
+    return s;
+}
+
+__device__ __forceinline__ double expk(DW<double> d) {
+    double u = (d.x + d.y) * 1.442695040888963407359924681001892137426645954152985934135449406931;
+    const double dq = __builtin_rint(u);
+    const int q = (int)dq;
+    DW<double> s = dw_add2(d, dq * -.69314718055966295651160180568695068359375);
+    s = dw_add2(s, dq * -.28235290563031577122588448175013436025525412068e-12);
+    s = dw_normalize(s);
+    const double z = s.x, z2 = z * z, z4 = z2 * z2, z8 = z4 * z4;
+    const double p01 = fma_(z, 0.166666666666666740681535, 0.500000000000000999200722);
+    const double p23 = fma_(z, 0.00833333333332371417601081, 0.0416666666665409524128449);
+    const double p45 = fma_(z, 0.000198412698809069797676111, 0.0013888888939977128960529);
+    const double p67 = fma_(z, 2.75572496725023574143864e-06, 2.48014973989819794114153e-05);
+    const double p89 = fma_(z, 2.51069683420950419527139e-08, 2.76286166770270649116855e-07);
+    const double lo = fma_(z2, p23, p01), hi = fma_(z2, p67, p45);
+    u = fma_(z8, p89, fma_(z4, hi, lo));
+    DW<double> t = dw_add(1.0, s);
+    t = dw_add(t, dw_mul(dw_squ(s), u));
+    u = t.x + t.y;
+    u = ldexp2k(u, q);
+    return d.x < -1000.0 ? 0.0 : u;
+}
+
+// exp(lg * y) with the library's "NaN result means overflow" rule; lg = logk(x) of a
+// positive finite x.  pow_(x, y) == powk(logk(x), y) on that domain.
+template <typename T> __device__ __forceinline__ T powk(DW<T> lg, T y) {
+    T r = expk(dw_mul(lg, y));
+    return (r != r) ? (T)__builtin_huge_val() : r;
+}
+
+// x ** y for x >= 0 or NaN, all special cases included.
+template <typename T> __device__ __forceinline__ T pow_(T x, T y) {
+    if (y == (T)0 || x == (T)1) return (T)1;
+    if (x != x || y != y) return nan_<T>();
+    if (x < (T)0) return nan_<T>();
+    const T inf = (T)__builtin_huge_val();
+    if (x == inf || x == (T)0) return (((x == (T)0) ? -y : y) < (T)0) ? (T)0 : inf;
+    if (abs_(y) == inf) {
+        T efx = (y < (T)0 ? (T)-1 : (T)1) * (x - (T)1);
+        return efx < (T)0 ? (T)0 : (efx == (T)0 ? (T)1 : inf);
+    }
+    return powk<T>(logk(x), y);
 }
 
 // Tensor ** python_float: the exponent is rounded to the tensor dtype first.
-template <typename T> __device__ __forceinline__ T rpow(T x, double p) { return (T)pow_core((double)x, (double)(T)p); }
+template <typename T> __device__ __forceinline__ T rpow(T x, double p) { return pow_<T>(x, (T)p); }
 
 // ---------------------------------------------------------------------------
 // Butcher tableaux, float64 literals cast to the working type where used

@@ -21,7 +21,7 @@ template <typename T> struct StepParams {
     int max_steps;
     // loop state (device, owned by the caller for the duration of a solve)
     T *t, *dt, *y, *k0;          // [B], [B], [B,F], [B,F] (FSAL derivative)
-    double *l2_prev, *l2_pprev;  // [B] log2 of the last two accepted error ratios
+    T *ratio_prev, *ratio_pprev;  // [B] the last two accepted error ratios (PID history)
     int32_t *running, *cursor, *n_steps, *n_accepted, *status, *monotone;
     uint8_t *pending;  // [B,E]
     T *ys;             // [B,max(E,1),F]
@@ -139,8 +139,8 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
         p.y[b * F + f] = y0[f];
         p.k0[b * F + f] = f0[f];
     }
-    p.l2_prev[b] = 0.0;
-    p.l2_pprev[b] = 0.0;
+    p.ratio_prev[b] = (T)1;
+    p.ratio_pprev[b] = (T)1;
     p.running[b] = 1;
     p.n_steps[b] = 0;
     p.n_accepted[b] = 0;
@@ -262,17 +262,9 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     const bool accept = ratio < (T)1;
 
     // ---- step size proposal ----
-    const double l2p = p.l2_prev[b], l2pp = p.l2_pprev[b];
-    T factor = cp.safety * rpow<T>(ratio, cp.e1);
-    if (CTRL == 1) {
-        // prev ** e2 and prev_prev ** e3 from the stored logarithms (identical bits to pow)
-        T f2 = cp.skip2 ? (T)1 : (T)exp2_of((double)(T)cp.e2 * l2p);
-        T f3 = cp.skip3 ? (T)1 : (T)exp2_of((double)(T)cp.e3 * l2pp);
-        factor = factor * f2;
-        factor = factor * f3;
-    }
-    factor = tclamp(factor, cp.fmin, cp.fmax);
-    T dt_next = dt * factor;
+    const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
+    const T factor0 = dt_factor<T, CTRL>(cp, ratio, prev, pprev);
+    T dt_next = dt * factor0;
     int status = limit_dt<T>(cp, ratio, dt_next);
 
     const bool running = p.running[b] != 0;
@@ -334,11 +326,8 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     const T dtn = running_new ? dt_next : dt;
     p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
     if (CTRL == 1 && running_new && accept) {
-        // log2 of the accepted ratio; anything outside (0, inf) ends the loop with status 4,
-        // after which the history is never read again
-        const bool sane = ratio > (T)0 && ratio < (T)__builtin_huge_val();
-        p.l2_pprev[b] = l2p;
-        p.l2_prev[b] = log2_normal(sane ? (double)ratio : 1.0);
+        p.ratio_pprev[b] = prev;
+        p.ratio_prev[b] = ratio;
     }
     p.running[b] = running_new ? 1 : 0;
     if (running_new) p.flags[TODE_STEP_FLAG_ANY_RUNNING] = 1;
@@ -384,8 +373,8 @@ template <typename T> static StepParams<T> make_step_params(const tode_step_stat
     p.dt = (T *)s.dt;
     p.y = (T *)s.y;
     p.k0 = (T *)s.k0;
-    p.l2_prev = s.l2_prev;
-    p.l2_pprev = s.l2_pprev;
+    p.ratio_prev = (T *)s.ratio_prev;
+    p.ratio_pprev = (T *)s.ratio_pprev;
     p.running = s.running;
     p.cursor = s.cursor;
     p.n_steps = s.n_steps;
@@ -411,7 +400,7 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     if (s->method != TODE_DOPRI5 && s->method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", s->method);
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (!s->flags) return fail(TODE_E_INVALID, "null flags pointer");
-    if (s->batch > 0 && (!s->y0 || !s->t_start || !s->t_end || !s->t || !s->dt || !s->y || !s->k0 || !s->l2_prev || !s->l2_pprev ||
+    if (s->batch > 0 && (!s->y0 || !s->t_start || !s->t_end || !s->t || !s->dt || !s->y || !s->k0 || !s->ratio_prev || !s->ratio_pprev ||
                          !s->running || !s->cursor || !s->n_steps || !s->n_accepted || !s->status || !s->monotone || !s->ys || !s->tnode))
         return fail(TODE_E_INVALID, "null state pointer");
     if (s->batch > 0 && s->n_eval > 0 && (!s->t_eval || !s->pending)) return fail(TODE_E_INVALID, "n_eval > 0 needs t_eval and pending");

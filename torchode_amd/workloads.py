@@ -31,7 +31,15 @@ def _uniform(g, a, b, shape):
 
 
 def _log_uniform(g, a, b, shape):
-    return torch.exp(_uniform(g, math.log(a), math.log(b), shape))
+    """exp(U(ln a, ln b)).  The exponential is evaluated with mpmath and rounded once, because
+    torch.exp / libm may differ in the last bit between hosts and the workloads have to be
+    identical everywhere (parity fixtures identify their inputs by hash)."""
+    import mpmath
+
+    u = _uniform(g, math.log(a), math.log(b), shape)
+    with mpmath.workprec(100):
+        vals = [float(mpmath.exp(mpmath.mpf(v))) for v in u.flatten().tolist()]
+    return torch.tensor(vals, dtype=torch.float64).reshape(shape)
 
 
 def _t_eval(t0, t1, E):
