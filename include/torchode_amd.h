@@ -40,6 +40,10 @@ enum {
     TODE_REACHED_MAX_STEPS = 3,
     TODE_INFINITE_NORM = 4
 };
+/* Safety limit, not in the reference: a sample that reaches 2^22 steps stops with
+ * TODE_GENERAL_ERROR (the reference's loop would never end; a kernel must). */
+#define TODE_HARD_STEP_LIMIT (1 << 22)
+
 /* return codes */
 enum {
     TODE_OK = 0,
@@ -268,6 +272,15 @@ int tode_step_finish(const tode_step_state *state, const tode_controller *contro
  * (adjoints.py:267-292). */
 int tode_step_stats(const tode_step_state *state, int64_t *out_n_steps, int64_t *out_n_accepted, int64_t *out_n_initialized,
                     int64_t *out_status, void *stream);
+
+/*
+ * Which kernel tode_solve_builtin_fast launches (per host thread); no counterpart in the
+ * reference.  0 (default): two wavefronts per 64 samples (a stepper and a dense-output
+ * evaluator) while the batch would otherwise leave SIMDs with at most two wavefronts, one
+ * wavefront per 64 samples above that; 1: always one wavefront; 2: two wavefronts or
+ * TODE_E_UNSUPPORTED.  All variants produce identical bits.
+ */
+int tode_set_fast_kernel_variant(int variant);
 
 /*
  * Kernel timing for benchmarks and profiling; no counterpart in the reference.

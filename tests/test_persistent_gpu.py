@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 F32, F64 = torch.float32, torch.float64
 
 
-@pytest.mark.parametrize("fast", [True, False], ids=["fast", "general"])
+@pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])
 @pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
 @pytest.mark.parametrize("name,batch", [("linear_decay", 256), ("vdp", 4096), ("lorenz", 4096)])
 def test_workload_matches_oracle_bit_for_bit(name, batch, dtype, fast):
@@ -42,7 +42,8 @@ def test_workload_matches_oracle_bit_for_bit(name, batch, dtype, fast):
 def test_every_method_controller_pair(method, controller, dtype):
     w = to.workloads.make("vdp", batch=1024, dtype=dtype)
     ref = c_oracle_solve(w.f, w.y0, w.t_eval, method, controller)
-    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller, fast="one"), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller, fast="two"), ref)
     assert_identical(gpu_solve(w.f, w.y0, w.t_eval, method, controller, fast=False), ref)
 
 
@@ -50,7 +51,8 @@ def test_every_method_controller_pair(method, controller, dtype):
 def test_ragged_batches(batch):
     w = to.workloads.make("lorenz", batch=batch, dtype=F32)
     ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
-    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast="one"), ref)
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast="two"), ref)
     assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast=False), ref)
     w = to.workloads.make("vdp", batch=batch, dtype=F64)  # dense output staged through LDS vs written directly
     ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
@@ -283,7 +285,7 @@ import os  # noqa: E402
 _GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")))
 
 
-@pytest.mark.parametrize("fast", [True, False], ids=["fast", "general"])
+@pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])
 @pytest.mark.parametrize("path", _GOLDEN, ids=os.path.basename)
 def test_gpu_matches_golden_fixture(path, fast):
     """Golden vectors of the ATen-op restatement, written in the authoring container."""

@@ -33,6 +33,7 @@ EXPORTS = (
     "tode_step_finish",
     "tode_step_stats",
     "tode_finalize_stats",
+    "tode_set_fast_kernel_variant",
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
 )
@@ -160,6 +161,8 @@ def load():
         lib.tode_step_stats.argtypes = [C.POINTER(StepState)] + [C.c_void_p] * 5
         lib.tode_finalize_stats.restype = C.c_int
         lib.tode_finalize_stats.argtypes = [C.c_int64, C.c_int64] + [C.c_void_p] * 9 + [C.c_int32] * 3 + [C.c_void_p] * 3
+        lib.tode_set_fast_kernel_variant.restype = C.c_int
+        lib.tode_set_fast_kernel_variant.argtypes = [C.c_int]
         lib.tode_set_kernel_timing.restype = C.c_int
         lib.tode_set_kernel_timing.argtypes = [C.c_int]
         lib.tode_last_solve_kernel_ms.restype = C.c_int
@@ -205,3 +208,8 @@ def last_solve_kernel_ms() -> float:
     out = C.c_float(0.0)
     check(load().tode_last_solve_kernel_ms(C.byref(out)), "tode_last_solve_kernel_ms")
     return out.value
+
+
+def set_fast_kernel_variant(variant: int):
+    """0: automatic, 1: one wavefront per 64 samples, 2: stepper + evaluator wavefronts."""
+    check(load().tode_set_fast_kernel_variant(int(variant)), "tode_set_fast_kernel_variant")

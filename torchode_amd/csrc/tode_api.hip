@@ -24,6 +24,7 @@ int check_hip(hipError_t err, const char *what) {
     return fail(TODE_E_HIP, "%s: %s", what, hipGetErrorString(err));
 }
 
+static thread_local int g_fast_variant = 0;
 static thread_local bool g_timing = false;
 static thread_local bool g_timed = false;
 static thread_local hipEvent_t g_ev[2] = {nullptr, nullptr};
@@ -68,6 +69,12 @@ extern "C" {
 int tode_abi_version(void) { return TODE_ABI_VERSION; }
 
 const char *tode_last_error(void) { return tode::g_error; }
+
+int tode_set_fast_kernel_variant(int variant) {
+    if (variant < 0 || variant > 2) return tode::fail(TODE_E_INVALID, "variant must be 0 (auto), 1 (one wavefront) or 2 (two wavefronts)");
+    tode::g_fast_variant = variant;
+    return TODE_OK;
+}
 
 int tode_set_kernel_timing(int enable) {
     tode::g_timing = enable != 0;
@@ -117,9 +124,16 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         return fail(TODE_E_INVALID, "null pointer");
     if (a->batch > (int64_t)2147483647 * 64) return fail(TODE_E_UNSUPPORTED, "batch too large");
     hipStream_t s = (hipStream_t)stream;
+    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (g_fast_variant != 1) {
+        // small batches: two wavefronts per group of 64 samples (stepper + dense-output evaluator)
+        bool used = false;
+        int rc = a->dtype == TODE_F32 ? solve_pair_f32(*a, *c, ns, na, ni, st, s, &used) : solve_pair_f64(*a, *c, ns, na, ni, st, s, &used);
+        if (rc || used) return rc;
+        if (g_fast_variant == 2) return fail(TODE_E_UNSUPPORTED, "the two-wavefront kernel does not cover this problem size");
+    }
     if (a->dtype == TODE_F32) return solve_fast_f32(*a, *c, ns, na, ni, st, s);
-    if (a->dtype == TODE_F64) return solve_fast_f64(*a, *c, ns, na, ni, st, s);
-    return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    return solve_fast_f64(*a, *c, ns, na, ni, st, s);
 }
 
 int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,

@@ -204,7 +204,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         }
         {
             // non-finite error ratio or max_steps reached: not the common case
-            const bool failed = active && (!sane || n_steps >= p.max_steps);
+            const bool failed = active && (!sane || n_steps >= p.max_steps || n_steps >= TODE_HARD_STEP_LIMIT);
             const bool finished = active && !failed && !running_new;
             // a sample that lands past t_end, or whose derivative at the end is not finite,
             // shows up in later iterations of the reference loop

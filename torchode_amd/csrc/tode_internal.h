@@ -4,6 +4,14 @@
 
 #include "../../include/torchode_amd.h"
 
+// No sample may take more than this many steps.  The reference has no such limit (without
+// max_steps a step size that has underflowed to zero makes its loop spin forever); a kernel
+// that never ends would take the whole GPU with it, so the loop is cut here: the fast kernels
+// hand the batch to the general one, which reports TODE_GENERAL_ERROR for the sample.
+#ifndef TODE_HARD_STEP_LIMIT
+#define TODE_HARD_STEP_LIMIT (1 << 22)
+#endif
+
 #define TODE_BLOCK 64  // one wavefront per workgroup: B/64 workgroups spread over all CUs and XCDs
 
 #ifndef TODE_INSTANTIATE_F32
@@ -26,5 +34,7 @@ void timing_after(hipStream_t s);
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
+int solve_pair_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
+int solve_pair_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
 int solve_fast_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 }  // namespace tode

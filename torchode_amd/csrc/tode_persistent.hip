@@ -122,6 +122,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
                 n_acc += move ? 1 : 0;
             }
             if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
+            if (status == 0 && n_steps >= TODE_HARD_STEP_LIMIT) status = TODE_GENERAL_ERROR;
             const bool last_own = running && (status != 0 || !running_new || n_steps >= p.cap);
 
             // ---- dense output (adjoints.py:215-234): points passed by the new t ----

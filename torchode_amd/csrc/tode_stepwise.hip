@@ -275,6 +275,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     p.n_steps[b] = n_steps;
     if (move) p.n_accepted[b] += 1;
     if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
+    if (status == 0 && n_steps >= TODE_HARD_STEP_LIMIT) status = TODE_GENERAL_ERROR;
     p.status[b] = status;
 
     // ---- dense output with the interpolant of the attempted step ----
