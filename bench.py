@@ -29,8 +29,10 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/solve_fast_kernel_vdp_f32_b65536_hbm_traffic.txt: (7120.1 KiB x 2.000 + 27680 KiB x 1.000) x 1024
-    ("vdp", "torch.float32", 65536): 42.93e6,
+    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6869.1 KiB x 2.000 + 32540.4 KiB x 1.000) x 1024
+    ("vdp", "torch.float32", 65536): 47.39e6,
+    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (77468.9 KiB x 2.000 + 895940 KiB x 1.000) x 1024
+    ("lorenz", "torch.float32", 1048576): 1076.1e6,
 }
 
 
@@ -125,7 +127,7 @@ def main():
         "equiv_hbm_gbps": algo_bytes / wall / 1e9,
         "roofline": {
             "bound": "hbm",
-            "kernel": "tode::solve_fast_kernel",
+            "kernel": _lib.last_solve_kernel_name(),
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

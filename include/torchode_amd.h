@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 1
+#define TODE_ABI_VERSION 2
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -114,8 +114,10 @@ typedef struct tode_solve_args {
     int64_t iteration_cap;     /* < 0: unlimited */
     double term_scalars[4];    /* batch-uniform RHS constants (Lorenz: sigma, beta) */
     const void *y0;            /* [B,F] */
-    const void *t_start;       /* [B]   */
-    const void *t_end;         /* [B]   */
+    const void *t_start;       /* [B], sample b at element b * t_start_stride */
+    const void *t_end;         /* [B], sample b at element b * t_end_stride   */
+    int64_t t_start_stride;    /* >= 1; 1 for a dense array, E for column 0 of t_eval */
+    int64_t t_end_stride;      /* >= 1 */
     const void *t_eval;        /* [B,E] or NULL when E == 0 */
     const void *dt0;           /* [B] user initial step, or NULL to select one */
     const void *params;        /* [B,P] */
@@ -293,6 +295,9 @@ int tode_set_fast_kernel_variant(int variant);
  */
 int tode_set_kernel_timing(int enable);
 int tode_last_solve_kernel_ms(float *out_ms);
+/* Name of the solve kernel most recently launched by the calling thread ("" if none), e.g.
+ * "tode::solve_pair_kernel"; the same for every template instance of a kernel. */
+const char *tode_last_solve_kernel_name(void);
 
 #ifdef __cplusplus
 }

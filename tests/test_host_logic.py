@@ -99,6 +99,11 @@ def test_abi_argument_validation_without_a_gpu():
     a.batch, a.n_features, a.n_eval = 4, 2, 0
     assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1
     assert b"null" in lib.tode_last_error()
+    dummy = (_lib.C.c_double * 64)()
+    for name in ("y0", "t_start", "t_end", "ys", "y_idle"):
+        setattr(a, name, _lib.C.addressof(dummy))
+    assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1  # strides left at zero
+    assert b"stride" in lib.tode_last_error()
     assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -2  # n_eval == 0
     a.n_features = 0
     assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1

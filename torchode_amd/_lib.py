@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -36,6 +36,7 @@ EXPORTS = (
     "tode_set_fast_kernel_variant",
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
+    "tode_last_solve_kernel_name",
 )
 
 
@@ -77,6 +78,8 @@ class SolveArgs(C.Structure):
         ("y0", C.c_void_p),
         ("t_start", C.c_void_p),
         ("t_end", C.c_void_p),
+        ("t_start_stride", C.c_int64),
+        ("t_end_stride", C.c_int64),
         ("t_eval", C.c_void_p),
         ("dt0", C.c_void_p),
         ("params", C.c_void_p),
@@ -166,6 +169,8 @@ def load():
         lib.tode_set_kernel_timing.restype = C.c_int
         lib.tode_set_kernel_timing.argtypes = [C.c_int]
         lib.tode_last_solve_kernel_ms.restype = C.c_int
+        lib.tode_last_solve_kernel_name.restype = C.c_char_p
+        lib.tode_last_solve_kernel_name.argtypes = []
         lib.tode_last_solve_kernel_ms.argtypes = [C.POINTER(C.c_float)]
         got = lib.tode_abi_version()
         if got != ABI_VERSION:
@@ -208,6 +213,11 @@ def last_solve_kernel_ms() -> float:
     out = C.c_float(0.0)
     check(load().tode_last_solve_kernel_ms(C.byref(out)), "tode_last_solve_kernel_ms")
     return out.value
+
+
+def last_solve_kernel_name() -> str:
+    """Name of the solve kernel most recently launched by this thread (as a profiler shows it)."""
+    return load().tode_last_solve_kernel_name().decode()
 
 
 def set_fast_kernel_variant(variant: int):

@@ -194,7 +194,8 @@ class AutoDiffAdjoint(nn.Module):
         dev, dtype = y0.device, y0.dtype
         B, F = y0.shape
         E = problem.n_evaluation_points
-        t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
+        # t_start / t_end are usually columns of t_eval: hand them over with their stride
+        t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
         t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
         params = f.builtin_params().to(device=dev, dtype=dtype)
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
@@ -202,7 +203,6 @@ class AutoDiffAdjoint(nn.Module):
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
         y_idle = torch.empty((B, F), dtype=dtype, device=dev) if E == 0 else None
-        counters = torch.empty((5, B), dtype=torch.int32, device=dev)
         flags = torch.empty(_lib.FLAG_WORDS, dtype=torch.int32, device=dev)
         ctrl = self.step_size_controller.c_struct()
         stream = _lib.stream_of(y0)
@@ -215,13 +215,13 @@ class AutoDiffAdjoint(nn.Module):
         a.iteration_cap = -1
         a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
         a.y0, a.t_start, a.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
+        a.t_start_stride, a.t_end_stride = t_start.stride(0), t_end.stride(0)
         a.t_eval = None if t_eval is None else t_eval.data_ptr()
         a.dt0 = None if dt0_ is None else dt0_.data_ptr()
         a.params = params.data_ptr()
         a.ys = ys.data_ptr()
         a.y_idle = None if y_idle is None else y_idle.data_ptr()
         a.pending = None
-        a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
         a.flags = flags.data_ptr()
 
         stats: Dict[str, Any] = {}
@@ -243,6 +243,9 @@ class AutoDiffAdjoint(nn.Module):
                     stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
                 stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
                 return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+
+        counters = torch.empty((5, B), dtype=torch.int32, device=dev)
+        a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
 
         def run():
             _lib.check(lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(ctrl), stream), "tode_solve_builtin")

@@ -29,7 +29,10 @@ static thread_local bool g_timing = false;
 static thread_local bool g_timed = false;
 static thread_local hipEvent_t g_ev[2] = {nullptr, nullptr};
 
-void timing_before(hipStream_t s) {
+static thread_local const char *g_kernel_name = "";
+
+void timing_before(hipStream_t s, const char *kernel_name) {
+    g_kernel_name = kernel_name;
     if (!g_timing) return;
     if (!g_ev[0]) {
         (void)hipEventCreate(&g_ev[0]);
@@ -82,6 +85,8 @@ int tode_set_kernel_timing(int enable) {
     return TODE_OK;
 }
 
+const char *tode_last_solve_kernel_name(void) { return tode::g_kernel_name; }
+
 int tode_last_solve_kernel_ms(float *out_ms) {
     using namespace tode;
     if (!out_ms) return fail(TODE_E_INVALID, "null output pointer");
@@ -98,6 +103,8 @@ int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void 
         return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
     if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->ys || (a->n_params > 0 && !a->params)))
         return fail(TODE_E_INVALID, "null problem pointer");
+    if (a->t_start_stride < 1 || a->t_end_stride < 1)
+        return fail(TODE_E_INVALID, "t_start_stride / t_end_stride must be >= 1 (got %lld, %lld)", (long long)a->t_start_stride, (long long)a->t_end_stride);
     if (a->n_eval > 0 && a->batch > 0 && !a->t_eval) return fail(TODE_E_INVALID, "n_eval > 0 but t_eval is null");
     if (a->n_eval == 0 && a->batch > 0 && !a->y_idle) return fail(TODE_E_INVALID, "n_eval == 0 needs y_idle");
     if (!a->flags || (a->batch > 0 && (!a->n_steps || !a->n_accepted || !a->n_initialized || !a->status_last || !a->status_idle)))
@@ -122,6 +129,8 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (!a->flags) return fail(TODE_E_INVALID, "null flags pointer");
     if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->t_eval || !a->ys || (a->n_params > 0 && !a->params) || !ns || !na || !ni || !st))
         return fail(TODE_E_INVALID, "null pointer");
+    if (a->t_start_stride < 1 || a->t_end_stride < 1)
+        return fail(TODE_E_INVALID, "t_start_stride / t_end_stride must be >= 1 (got %lld, %lld)", (long long)a->t_start_stride, (long long)a->t_end_stride);
     if (a->batch > (int64_t)2147483647 * 64) return fail(TODE_E_UNSUPPORTED, "batch too large");
     hipStream_t s = (hipStream_t)stream;
     if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);

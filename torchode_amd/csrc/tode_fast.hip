@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
     T y[F], k[7][F];
 #pragma unroll
     for (int f = 0; f < F; ++f) y[f] = p.y0[bs * F + f];
-    const T ts = p.t_start[bs], te = p.t_end[bs];
+    const T ts = p.t_start[bs * p.ts_stride], te = p.t_end[bs * p.te_stride];
     const bool fwd = te > ts;
     const T dir = fwd ? (T)1 : (T)-1;
     const T tlo = tmin(ts, te), thi = tmax(te, ts);
@@ -278,7 +278,7 @@ static int launch_fast(const tode_solve_args &a, const tode_controller &c, const
     const bool stage = need_all <= budget;
     const size_t lds = stage ? need_all : need_te;
     const dim3 grid((unsigned)blocks), block(64);
-    timing_before(stream);
+    timing_before(stream, "tode::solve_fast_kernel");
 #define TODE_FAST_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
     if (nhist == 0) {
         if (stage) TODE_FAST_LAUNCH(0, true); else TODE_FAST_LAUNCH(0, false);

@@ -28,7 +28,7 @@ int fail(int code, const char *fmt, ...);
 int check_hip(hipError_t err, const char *what);
 
 // Event pair around the solve kernel, active only while timing is enabled on this thread.
-void timing_before(hipStream_t s);
+void timing_before(hipStream_t s, const char *kernel_name);
 void timing_after(hipStream_t s);
 
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);

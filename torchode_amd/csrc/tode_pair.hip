@@ -49,7 +49,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
     int *ctl = reinterpret_cast<int *>(rec + 2 * NF * 64);   // [2] "stepper is done" per phase
     T *te_s = reinterpret_cast<T *>(ctl + 4);                // [E][64] when STAGE_TE
 
-    const T ts = p.t_start[bs], te = p.t_end[bs];
+    const T ts = p.t_start[bs * p.ts_stride], te = p.t_end[bs * p.te_stride];
     const bool fwd = te > ts;
     const T dir = fwd ? (T)1 : (T)-1;
 
@@ -289,7 +289,7 @@ static int launch_pair(const tode_solve_args &a, const tode_controller &c, const
     const int nhist = CTRL == 0 ? 0 : (p.cp.skip3 ? 1 : 2);
     const dim3 grid((unsigned)blocks), block(128);
     hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
-    timing_before(stream);
+    timing_before(stream, "tode::solve_pair_kernel");
 #define TODE_PAIR_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_pair_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
     if (nhist == 0) {
         if (stage_te) TODE_PAIR_LAUNCH(0, true); else TODE_PAIR_LAUNCH(0, false);

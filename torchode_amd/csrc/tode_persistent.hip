@@ -30,7 +30,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
         T y[F], k[7][F];
 #pragma unroll
         for (int f = 0; f < F; ++f) y[f] = p.y0[b * F + f];
-        const T ts = p.t_start[b], te = p.t_end[b];
+        const T ts = p.t_start[b * p.ts_stride], te = p.t_end[b * p.te_stride];
         const T dir = (te > ts) ? (T)1 : (T)-1;
         const T tlo = tmin(ts, te), thi = tmax(te, ts);
         const T *tev = p.t_eval ? p.t_eval + b * E : nullptr;
@@ -256,7 +256,7 @@ static int launch(const tode_solve_args &a, const tode_controller &c, hipStream_
     const long long blocks = (a.batch + TODE_BLOCK - 1) / TODE_BLOCK;
     hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
     if (blocks > 0) {
-        timing_before(stream);
+        timing_before(stream, "tode::solve_kernel");
         hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
         timing_after(stream);
     }

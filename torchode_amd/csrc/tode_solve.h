@@ -74,7 +74,7 @@ template <typename T> struct SolveParams {
     T *ys, *y_idle;
     uint8_t *pending;
     int32_t *n_steps, *n_accepted, *n_initialized, *status_last, *status_idle, *flags;
-    long long batch;
+    long long batch, ts_stride, te_stride;
     int n_eval;
     int max_steps;  // INT_MAX: unlimited
     int cap;        // INT_MAX: unlimited
@@ -172,6 +172,8 @@ template <typename T> static SolveParams<T> make_params(const tode_solve_args &a
     p.status_idle = a.status_idle;
     p.flags = a.flags;
     p.batch = a.batch;
+    p.ts_stride = a.t_start_stride;
+    p.te_stride = a.t_end_stride;
     p.n_eval = a.n_eval;
     p.max_steps = (a.max_steps < 0 || a.max_steps >= INT_MAX) ? INT_MAX : (int)a.max_steps;
     p.cap = (a.iteration_cap < 0 || a.iteration_cap >= INT_MAX) ? INT_MAX : (int)a.iteration_cap;
