@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 2
+#define TODE_ABI_VERSION 3
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -298,6 +298,131 @@ int tode_last_solve_kernel_ms(float *out_ms);
 /* Name of the solve kernel most recently launched by the calling thread ("" if none), e.g.
  * "tode::solve_pair_kernel"; the same for every template instance of a kernel. */
 const char *tode_last_solve_kernel_name(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Protocol operators.
+ *
+ * The reference's solve loop is written against plug-in protocols (SingleStepMethod,
+ * StepSizeController, LocalInterpolation; reference single_step_methods/base.py:20-89,
+ * step_size_controllers.py:16-113, interpolation.py:43-45), and users may supply their own
+ * implementation of any of them.  The operators below are what the package's own
+ * implementations of those protocol methods call, one kernel each, so that any mix of
+ * library and user-supplied parts runs through the same loop.  Time and data share `dtype`.
+ * All pointers are device pointers except the `const double *` coefficient arrays, which are
+ * host arrays read before the call returns.  Arrays are dense row-major.
+ * ------------------------------------------------------------------------------------------ */
+#define TODE_MAX_STAGES 16
+enum { TODE_NORM_RMS = 0, TODE_NORM_MAX = 1 }; /* reference step_size_controllers.py:170-186 */
+
+/* Stage input of an explicit Runge-Kutta step (reference runge_kutta.py:258-262):
+ *   y_out[b,f] = fma(dt[b], sum_{j<n_terms} a[j] * k[j,b,f], y0[b,f])   (the sum is a chain of fma)
+ *   t_out[b]   = fma(c, dt[b], t0[b])                                   (skipped if t_out is NULL)
+ * k is [n_stages_total, B, F]; only its first n_terms slices are read. */
+int tode_erk_stage(int32_t dtype, int64_t batch, int32_t n_features, int32_t n_terms, const double *a, double c,
+                   const void *t0, const void *dt, const void *y0, const void *k, void *y_out, void *t_out, void *stream);
+
+/* Weighted stage sum (reference runge_kutta.py:264-267, einsum "b,s,sbf->bf"):
+ *   out[b,f] = sum_{s<n_stages} (dt[b] * w[s]) * k[s,b,f]   (+ y0[b,f] when y0 is not NULL)
+ * used for the error estimate (w = b_err) and for y1 of methods whose last stage is not the solution. */
+int tode_erk_combine(int32_t dtype, int64_t batch, int32_t n_features, int32_t n_stages, const double *w, const void *dt,
+                     const void *k, const void *y0, void *out, void *stream);
+
+/* out[b,f] = |err[b,f]| / (atol + rtol * max(|y0[b,f]|, |y1[b,f]|))   (reference step_size_controllers.py:389-393, 734-738);
+ * atol and rtol are rounded to float32 first, as the reference's buffers are. */
+int tode_error_scale(int32_t dtype, int64_t batch, int32_t n_features, double atol, double rtol, const void *y0, const void *y1,
+                     const void *err, void *out, void *stream);
+
+/* Row norms of x [B,F] -> out [B]: TODE_NORM_RMS or TODE_NORM_MAX (reference step_size_controllers.py:170-186). */
+int tode_row_norm(int32_t dtype, int32_t norm, int64_t batch, int32_t n_features, const void *x, void *out, void *stream);
+
+/* From the error norm to the decision (reference step_size_controllers.py:394-429, 739-774, dt_factor :289-294, :598-621,
+ * PID update_state :640-671):  ratio = max(norm, 1e-38); accept = ratio < 1; dt_next = dt * clamp(factor);
+ * status = INFINITE_NORM if ratio is not finite, REACHED_DT_MIN if |dt_next| < dt_min; dt_min/dt_max applied.
+ * PID: prev / prev_prev are the history in (NULL for the integral controller), prev_out / prev_prev_out the history
+ * after update_state (shifted where accept).  accept is one byte per sample, status int64. */
+int tode_control(int32_t dtype, const tode_controller *c, int32_t method_order, int64_t batch, const void *norm, const void *dt,
+                 const void *prev, const void *prev_prev, uint8_t *accept, void *dt_next, void *ratio, int64_t *status,
+                 void *prev_out, void *prev_prev_out, void *stream);
+
+/* tode_error_scale + tode_row_norm + tode_control in one kernel: {Integral,PID}Controller.adapt_step_size
+ * with a built-in norm (reference step_size_controllers.py:370-429, 715-774). */
+int tode_adapt_step(int32_t dtype, const tode_controller *c, int32_t method_order, int32_t norm, int64_t batch, int32_t n_features,
+                    const void *dt, const void *y0, const void *y1, const void *err, const void *prev, const void *prev_prev,
+                    uint8_t *accept, void *dt_next, void *ratio, int64_t *status, void *prev_out, void *prev_prev_out,
+                    void *stream);
+
+/* Start step selection, first half (reference step_size_controllers.py:459-479, 804-824): from f0 = f(t_start, y0)
+ *   h0[b], y1 = y0 + direction * h0 * f0 [B,F], t1 = t_start + direction * h0 [B]
+ * and second half (:481-490, :826-835) from f1 = f(t1, y1): dt0[b] (signed).  `kind` is the controller kind: the
+ * integral controller maps h0 == 0 to d2 = inf, the PID controller does not (:481 against :826). */
+int tode_initial_step_a(int32_t dtype, int32_t norm, int64_t batch, int32_t n_features, double atol, double rtol, const void *t_start,
+                        const void *t_end, const void *y0, const void *f0, void *h0, void *y1, void *t1, void *stream);
+int tode_initial_step_b(int32_t dtype, int32_t kind, int32_t norm, int32_t method_order, int64_t batch, int32_t n_features, double atol,
+                        double rtol, const void *t_start, const void *t_end, const void *y0, const void *f0, const void *f1,
+                        const void *h0, void *dt0, void *stream);
+
+/* Quartic dense-output coefficients of a Dopri5 / Tsit5 step, lowest power first: coeff [5,B,F]
+ * (reference tsit5.py:123-139; dopri5.py:53-60 -> interpolation.py:138-170).  k is [7,B,F]. */
+int tode_quartic_build(int32_t dtype, int32_t method, int64_t batch, int32_t n_features, const void *dt, const void *y0,
+                       const void *y1, const void *k, void *coeff, void *stream);
+
+/* Polynomial evaluation (reference interpolation.py:8-40, 103-106, 172-175): for n = 0..count-1, b = idx[n],
+ *   x = (t[n] - t0[b]) / (t1[b] - t0[b])  (denominator 1 where it is 0);  out[n,f] = Horner(coeff[degree..0, b, f], x)
+ * coeff is [degree+1,B,F], degree in 1..4. */
+int tode_poly_eval(int32_t dtype, int32_t degree, int64_t batch, int32_t n_features, int64_t count, const void *coeff,
+                   const void *t0, const void *t1, const void *t, const int64_t *idx, void *out, void *stream);
+
+/* The same evaluation for every set entry of a [B,E] byte mask, written to ys[b,e,:]
+ * (reference adjoints.py:227-233 without materialising the index list). */
+int tode_poly_eval_masked(int32_t dtype, int32_t degree, int64_t batch, int32_t n_features, int32_t n_eval, const void *coeff,
+                          const void *t0, const void *t1, const void *t_eval, const uint8_t *mask, void *ys, void *stream);
+
+/* out[b,:] = mask[b] ? a[b,:] : b[b,:] for rows of `width` values (merge_states, reference runge_kutta.py:216-224,
+ * step_size_controllers.py:628-638). */
+int tode_select_rows(int32_t dtype, int64_t batch, int32_t width, const uint8_t *mask, const void *a, const void *b, void *out,
+                     void *stream);
+
+/*
+ * Bookkeeping of one loop iteration (reference adjoints.py:150-255) in one call.
+ * Given the step's proposal (y_new, accept, dt_next, optional status of method and controller) it computes
+ *   to_update = accept & running;  t, y where to_update;  n_steps += running;  n_accepted += to_update;
+ *   running_out = direction * (t_out - t_end) < 0;  status (max of the two, REACHED_MAX_STEPS at max_steps);
+ *   to_evaluate[b,e] = pending[b,e] & (direction * (t_out - t_eval[b,e]) >= 0), pending ^= to_evaluate;
+ *   dt_out = clamp(running_out ? dt_next : dt, t_min - t_out, t_max - t_out)
+ * and the flag block {any sample running, any status != SUCCESS, number of set to_evaluate entries}.
+ * Outputs never alias inputs (callers of the protocols may keep earlier t / y / dt tensors).
+ * n_steps, n_accepted and pending are updated in place.
+ */
+enum { TODE_LOOP_ANY_RUNNING = 0, TODE_LOOP_ANY_FAILURE = 1, TODE_LOOP_N_TO_EVALUATE = 2, TODE_LOOP_FLAG_WORDS = 4 };
+typedef struct tode_loop_args {
+    int32_t dtype, n_features, n_eval, reserved;
+    int64_t batch;
+    int64_t max_steps;            /* < 0: none */
+    const void *t_start, *t_end;  /* [B] */
+    const void *t_eval;           /* [B,E] or NULL */
+    const void *t, *dt, *y;       /* state before the step: [B], [B], [B,F] */
+    const uint8_t *running;       /* [B] */
+    const void *y_new;            /* [B,F] step result */
+    const uint8_t *accept;        /* [B] */
+    const void *dt_next;          /* [B] */
+    const int64_t *method_status, *controller_status; /* [B] or NULL */
+    void *t_out, *dt_out, *y_out; /* state after the step */
+    uint8_t *running_out, *to_update; /* [B] */
+    int64_t *status;              /* [B] */
+    int64_t *n_steps, *n_accepted; /* [B], in place */
+    uint8_t *pending;             /* [B,E], in place, or NULL */
+    uint8_t *to_evaluate;         /* [B,E] or NULL */
+    int32_t *flags;               /* [TODE_LOOP_FLAG_WORDS] */
+} tode_loop_args;
+int tode_loop_advance(const tode_loop_args *a, void *stream);
+
+/* Start of the loop (reference adjoints.py:76-79, 107, 121-126): pending[b,e] = 1; where t_eval[b,0] == t_start[b]
+ * ys[b,0,:] = y0[b,:] and pending[b,0] = 0; dt_out = clamp(dt, t_min - t_start, t_max - t_start). */
+int tode_loop_begin(int32_t dtype, int64_t batch, int32_t n_features, int32_t n_eval, const void *t_start, const void *t_end,
+                    const void *t_eval, const void *y0, const void *dt, void *dt_out, uint8_t *pending, void *ys, void *stream);
+
+/* n_initialized[b] = number of leading zeros of pending[b,:] (reference adjoints.py:284-292). */
+int tode_count_initialized(int64_t batch, int32_t n_eval, const uint8_t *pending, int64_t *n_initialized, void *stream);
 
 #ifdef __cplusplus
 }

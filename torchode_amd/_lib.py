@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -37,7 +37,26 @@ EXPORTS = (
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
     "tode_last_solve_kernel_name",
+    "tode_erk_stage",
+    "tode_erk_combine",
+    "tode_error_scale",
+    "tode_row_norm",
+    "tode_control",
+    "tode_adapt_step",
+    "tode_initial_step_a",
+    "tode_initial_step_b",
+    "tode_quartic_build",
+    "tode_poly_eval",
+    "tode_poly_eval_masked",
+    "tode_select_rows",
+    "tode_loop_advance",
+    "tode_loop_begin",
+    "tode_count_initialized",
 )
+
+NORM_RMS, NORM_MAX = 0, 1
+MAX_STAGES = 16
+LOOP_ANY_RUNNING, LOOP_ANY_FAILURE, LOOP_N_TO_EVALUATE, LOOP_FLAG_WORDS = 0, 1, 2, 4
 
 
 class Controller(C.Structure):
@@ -133,6 +152,42 @@ class StepState(C.Structure):
     ]
 
 
+class LoopArgs(C.Structure):
+    """struct tode_loop_args"""
+
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("n_features", C.c_int32),
+        ("n_eval", C.c_int32),
+        ("reserved", C.c_int32),
+        ("batch", C.c_int64),
+        ("max_steps", C.c_int64),
+        ("t_start", C.c_void_p),
+        ("t_end", C.c_void_p),
+        ("t_eval", C.c_void_p),
+        ("t", C.c_void_p),
+        ("dt", C.c_void_p),
+        ("y", C.c_void_p),
+        ("running", C.c_void_p),
+        ("y_new", C.c_void_p),
+        ("accept", C.c_void_p),
+        ("dt_next", C.c_void_p),
+        ("method_status", C.c_void_p),
+        ("controller_status", C.c_void_p),
+        ("t_out", C.c_void_p),
+        ("dt_out", C.c_void_p),
+        ("y_out", C.c_void_p),
+        ("running_out", C.c_void_p),
+        ("to_update", C.c_void_p),
+        ("status", C.c_void_p),
+        ("n_steps", C.c_void_p),
+        ("n_accepted", C.c_void_p),
+        ("pending", C.c_void_p),
+        ("to_evaluate", C.c_void_p),
+        ("flags", C.c_void_p),
+    ]
+
+
 _lock = threading.Lock()
 _lib = None
 
@@ -172,6 +227,27 @@ def load():
         lib.tode_last_solve_kernel_name.restype = C.c_char_p
         lib.tode_last_solve_kernel_name.argtypes = []
         lib.tode_last_solve_kernel_ms.argtypes = [C.POINTER(C.c_float)]
+        V, I32, I64, D = C.c_void_p, C.c_int32, C.c_int64, C.c_double
+        DP, CP = C.POINTER(C.c_double), C.POINTER(Controller)
+        for name, argtypes in {
+            "tode_erk_stage": [I32, I64, I32, I32, DP, D] + [V] * 7,
+            "tode_erk_combine": [I32, I64, I32, I32, DP] + [V] * 5,
+            "tode_error_scale": [I32, I64, I32, D, D] + [V] * 5,
+            "tode_row_norm": [I32, I32, I64, I32] + [V] * 3,
+            "tode_control": [I32, CP, I32, I64] + [V] * 11,
+            "tode_adapt_step": [I32, CP, I32, I32, I64, I32] + [V] * 13,
+            "tode_initial_step_a": [I32, I32, I64, I32, D, D] + [V] * 8,
+            "tode_initial_step_b": [I32, I32, I32, I32, I64, I32, D, D] + [V] * 8,
+            "tode_quartic_build": [I32, I32, I64, I32] + [V] * 6,
+            "tode_poly_eval": [I32, I32, I64, I32, I64] + [V] * 7,
+            "tode_poly_eval_masked": [I32, I32, I64, I32, I32] + [V] * 7,
+            "tode_select_rows": [I32, I64, I32] + [V] * 5,
+            "tode_loop_advance": [C.POINTER(LoopArgs), V],
+            "tode_loop_begin": [I32, I64, I32, I32] + [V] * 9,
+            "tode_count_initialized": [I64, I32, V, V, V],
+        }.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = C.c_int, argtypes
         got = lib.tode_abi_version()
         if got != ABI_VERSION:
             raise RuntimeError(f"libtorchode_amd.so has ABI version {got}, the Python package expects {ABI_VERSION}")

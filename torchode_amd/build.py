@@ -42,6 +42,7 @@ UNITS = [
     ("tode_pair.hip", "tode_pair_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_pair.hip", "tode_pair_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
     ("tode_stepwise.hip", "tode_stepwise.o", []),
+    ("tode_ops.hip", "tode_ops.o", []),
 ]
 
 

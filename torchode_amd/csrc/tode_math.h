@@ -432,4 +432,51 @@ template <typename T, int F> __device__ __forceinline__ void quartic_eval(const 
     }
 }
 
+// Quartic coefficients for a single feature with run-time choice of ATen's two
+// summation forms: products rounded and then added (F <= 57), or one fused chain
+// (F >= 58, where the contraction runs as a matrix product).  ks[s] = k_s[b,f].
+template <typename T, int METHOD>
+__device__ __forceinline__ void quartic_elem(T dt, T y0, T y1, const T (&ks)[7], bool fused, T (&q)[5][1]) {
+    if (!fused) {
+        T yy0[1] = {y0}, yy1[1] = {y1}, kk[7][1];
+#pragma unroll
+        for (int s = 0; s < 7; ++s) kk[s][0] = ks[s];
+        quartic<T, 1, METHOD>(dt, yy0, yy1, kk, q);
+        return;
+    }
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    T w[3] = {0, 0, 0};
+#pragma unroll
+    for (int r = 0; r < Tab::n_other; ++r)
+#pragma unroll
+        for (int s = 0; s < 7; ++s) w[r] = fma_(dt * (T)Tab::w[r][s], ks[s], w[r]);
+    if (METHOD == 1) {
+        q[0][0] = y0;
+        q[1][0] = dt * ks[0];
+        q[2][0] = w[0];
+        q[3][0] = w[1];
+        q[4][0] = w[2];
+    } else {
+        T f0 = dt * ks[0], f1 = dt * ks[6];
+        T ym = y0 + w[0];
+        T a = (T)2 * (f1 - f0);
+        a = fma_((T)-8, y1 + y0, a);
+        a = fma_((T)16, ym, a);
+        T bq = (T)5 * f0;
+        bq = fma_((T)-3, f1, bq);
+        bq = fma_((T)18, y0, bq);
+        bq = fma_((T)14, y1, bq);
+        bq = fma_((T)-32, ym, bq);
+        T c = fma_((T)-4, f0, f1);
+        c = fma_((T)-11, y0, c);
+        c = fma_((T)-5, y1, c);
+        c = fma_((T)16, ym, c);
+        q[0][0] = y0;
+        q[1][0] = f0;
+        q[2][0] = c;
+        q[3][0] = bq;
+        q[4][0] = a;
+    }
+}
+
 }  // namespace tode

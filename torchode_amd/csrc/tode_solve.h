@@ -128,7 +128,7 @@ __device__ __forceinline__ T initial_step(const CtrlParams<T> &cp, const Term &r
 
 
 // Controller parameters in the working type from the ABI struct.
-template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c) {
+template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c, double order = 5.0) {
     CtrlParams<T> cp;
     cp.atol = (T)(float)c.atol;
     cp.rtol = (T)(float)c.rtol;
@@ -139,7 +139,7 @@ template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c) {
     cp.dt_max = (T)c.dt_max;
     cp.has_dt_min = c.has_dt_min;
     cp.has_dt_max = c.has_dt_max;
-    const double order = 5.0;  // convergence order of both pairs (dopri5.py:49-51, tsit5.py:119-121)
+    // order: convergence order of the step method; 5 for both pairs (dopri5.py:49-51, tsit5.py:119-121)
     if (c.kind == TODE_CTRL_INTEGRAL) {
         cp.e1 = -(1.0 / order);
         cp.e2 = cp.e3 = 0.0;

@@ -168,47 +168,8 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
 // Quartic of the attempted step for one feature, evaluated at time te (tsit5.py:123-139,
 // dopri5.py:53-60, interpolation.py:25-40, 138-175).  ks[s] = k_s[b,f].
 template <typename T, int METHOD> __device__ __forceinline__ T dense_value(T t0, T dt, T y0, T y1, const T (&ks)[7], bool fused, T te) {
-    T q[5][1], yy0[1] = {y0}, yy1[1] = {y1}, kk[7][1];
-#pragma unroll
-    for (int s = 0; s < 7; ++s) kk[s][0] = ks[s];
-    if (!fused) {
-        quartic<T, 1, METHOD>(dt, yy0, yy1, kk, q);
-    } else {
-        // F >= 58: the weighted sums are fused chains (large-matrix product path)
-        using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
-        T w[3] = {0, 0, 0};
-#pragma unroll
-        for (int r = 0; r < Tab::n_other; ++r)
-#pragma unroll
-            for (int s = 0; s < 7; ++s) w[r] = fma_(dt * (T)Tab::w[r][s], ks[s], w[r]);
-        if (METHOD == 1) {
-            q[0][0] = y0;
-            q[1][0] = dt * ks[0];
-            q[2][0] = w[0];
-            q[3][0] = w[1];
-            q[4][0] = w[2];
-        } else {
-            T f0 = dt * ks[0], f1 = dt * ks[6];
-            T ym = y0 + w[0];
-            T a = (T)2 * (f1 - f0);
-            a = fma_((T)-8, y1 + y0, a);
-            a = fma_((T)16, ym, a);
-            T bq = (T)5 * f0;
-            bq = fma_((T)-3, f1, bq);
-            bq = fma_((T)18, y0, bq);
-            bq = fma_((T)14, y1, bq);
-            bq = fma_((T)-32, ym, bq);
-            T c = fma_((T)-4, f0, f1);
-            c = fma_((T)-11, y0, c);
-            c = fma_((T)-5, y1, c);
-            c = fma_((T)16, ym, c);
-            q[0][0] = y0;
-            q[1][0] = f0;
-            q[2][0] = c;
-            q[3][0] = bq;
-            q[4][0] = a;
-        }
-    }
+    T q[5][1];
+    quartic_elem<T, METHOD>(dt, y0, y1, ks, fused, q);
     T out[1];
     quartic_eval<T, 1>(q, t0, dt, te, out);
     return out[0];
