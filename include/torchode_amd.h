@@ -314,6 +314,11 @@ const char *tode_last_solve_kernel_name(void);
 #define TODE_MAX_STAGES 16
 enum { TODE_NORM_RMS = 0, TODE_NORM_MAX = 1 }; /* reference step_size_controllers.py:170-186 */
 
+/* Coefficients the kernels use for Dopri5 / Tsit5 (reference dopri5.py:11-44, tsit5.py:11-114), as doubles:
+ * c [7], a [7*7] row-major (strictly lower triangle; row 6 is b), b_err [7], b_other [3*7] with *n_other rows set
+ * (Dopri5: the mid-point weights; Tsit5: the theta^2..theta^4 dense output weights).  Host arrays. */
+int tode_tableau(int32_t method, double *c, double *a, double *b_err, double *b_other, int32_t *n_other);
+
 /* Stage input of an explicit Runge-Kutta step (reference runge_kutta.py:258-262):
  *   y_out[b,f] = fma(dt[b], sum_{j<n_terms} a[j] * k[j,b,f], y0[b,f])   (the sum is a chain of fma)
  *   t_out[b]   = fma(c, dt[b], t0[b])                                   (skipped if t_out is NULL)
@@ -365,6 +370,16 @@ int tode_initial_step_b(int32_t dtype, int32_t kind, int32_t norm, int32_t metho
  * (reference tsit5.py:123-139; dopri5.py:53-60 -> interpolation.py:138-170).  k is [7,B,F]. */
 int tode_quartic_build(int32_t dtype, int32_t method, int64_t batch, int32_t n_features, const void *dt, const void *y0,
                        const void *y1, const void *k, void *coeff, void *stream);
+
+/* The same quartic from a given mid-point value y_mid = y(t0 + dt/2) and the first / last stage derivatives
+ * (reference FourthOrderPolynomialInterpolation.from_k, interpolation.py:138-170): coeff [5,B,F]. */
+int tode_quartic_from_mid(int32_t dtype, int64_t batch, int32_t n_features, const void *dt, const void *y0, const void *y1,
+                          const void *k_first, const void *k_last, const void *y_mid, void *coeff, void *stream);
+
+/* Hermite cubic from the end points and end-point derivatives (reference ThirdOrderPolynomialInterpolation.from_k,
+ * interpolation.py:84-106): coeff [4,B,F], lowest power first. */
+int tode_cubic_build(int32_t dtype, int64_t batch, int32_t n_features, const void *dt, const void *y0, const void *y1,
+                     const void *k_first, const void *k_last, void *coeff, void *stream);
 
 /* Polynomial evaluation (reference interpolation.py:8-40, 103-106, 172-175): for n = 0..count-1, b = idx[n],
  *   x = (t[n] - t0[b]) / (t1[b] - t0[b])  (denominator 1 where it is 0);  out[n,f] = Horner(coeff[degree..0, b, f], x)

@@ -1,0 +1,613 @@
+"""GPU tests of the protocol path: the loop driven through SingleStepMethod /
+StepSizeController / LocalInterpolation objects, the library's and user-defined ones.
+
+Part one restates the loop-bookkeeping cases of the reference's own test suite
+(tests/adjoint_test.py:26-319, with scripted step methods and controllers written for
+this suite) against the kernels.  Part two restates its controller, Runge-Kutta and
+interpolation unit tests (tests/step_size_controllers_test.py,
+tests/single_step_methods_test.py, tests/interpolation_test.py).  Part three checks
+that the protocol path reproduces the C oracle bit for bit.
+"""
+import copy
+from itertools import chain, repeat
+
+import numpy as np
+import pytest
+import torch
+
+import torchode_amd as to
+from helpers import assert_identical, c_oracle_solve, make_controller
+from torchode_amd.interpolation import (
+    FourthOrderPolynomialInterpolation,
+    LinearInterpolation,
+    LocalInterpolation,
+    ThirdOrderPolynomialInterpolation,
+)
+from torchode_amd.single_step_methods import ButcherTableau, ERKInterpolationData, ExplicitRungeKutta, SingleStepMethod, StepResult
+from torchode_amd.step_size_controllers import PIDState, StepSizeController, max_norm, rms_norm
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+OK, FAILED, DT_MIN, MAX_STEPS, INF_NORM = 0, 1, 2, 3, 4
+
+
+def dev(x, dtype=torch.float32):
+    return torch.as_tensor(x, dtype=dtype, device=DEV)
+
+
+# ---------------------------------------------------------------------------------------------
+# scripted plug-ins
+# ---------------------------------------------------------------------------------------------
+
+
+def curve(t, *idx):
+    """A known solution curve with one feature; evaluate(t, idx) ignores the sample index."""
+    return (torch.sin(3 * t) + 0.5 * t**2)[..., None]
+
+
+def script(values):
+    """Iterator over per-call values; the last one repeats."""
+    values = list(values)
+    return chain(values[:-1], repeat(values[-1]))
+
+
+class ExactInterpolation(LocalInterpolation):
+    def __init__(self, fn):
+        self.fn = fn
+
+    def evaluate(self, t, idx):
+        return self.fn(t, idx)
+
+
+class ScriptedMethod(SingleStepMethod):
+    """Returns ``fn(t0)`` as the step result and ``fn`` itself as the dense output."""
+
+    def __init__(self, fn, status=(None,), error=None):
+        super().__init__()
+        self.fn, self.status, self.error = fn, script(status), error
+        self.seen_t, self.seen_dt = [], []
+
+    def init(self, term, problem, f0, *, stats, args):
+        return "method-state"
+
+    def step(self, term, running, y0, t0, dt, state, *, stats, args):
+        self.seen_t.append(t0)
+        self.seen_dt.append(dt)
+        y1 = self.fn(t0)
+        err = torch.zeros_like(y1) if self.error is None else self.error(t0)
+        st = next(self.status)
+        return StepResult(y1, err), self.fn, state, None if st is None else dev(st, torch.long)
+
+    def merge_states(self, accept, current, previous):
+        return current
+
+    def build_interpolation(self, data):
+        return ExactInterpolation(data)
+
+    def convergence_order(self):
+        return 3
+
+
+class ScriptedController(StepSizeController):
+    def __init__(self, dt0, dt, accept=(True,), status=(None,)):
+        super().__init__()
+        self.dt0, self.dt, self.accept, self.status = dt0, script(dt), script(accept), script(status)
+
+    def init(self, term, problem, method_order, dt0, *, stats, args):
+        return dev(self.dt0).expand(problem.batch_size), {}, None
+
+    def adapt_step_size(self, t0, dt, y0, step_result, state, stats):
+        B = t0.shape[0]
+        st = next(self.status)
+        return (
+            dev(next(self.accept), torch.bool).expand(B),
+            dev(next(self.dt)).expand(B),
+            state,
+            None if st is None else dev(st, torch.long).expand(B),
+        )
+
+    def merge_states(self, running, current, previous):
+        return current
+
+
+def curve_problem(t_eval, t_start=None, t_end=None, fn=curve):
+    t_eval = dev(t_eval)
+    t_start = t_eval[:, 0] if t_start is None else dev(t_start)
+    t_end = t_eval[:, -1] if t_end is None else dev(t_end)
+    return to.InitialValueProblem(fn(t_start), t_start, t_end, t_eval)
+
+
+def no_rhs(t, y):
+    raise AssertionError("the right-hand side must not be called")
+
+
+def solve(method, controller, problem, **kw):
+    solver_kw = {k: kw.pop(k) for k in ("max_steps",) if k in kw}
+    return to.AutoDiffAdjoint(method, controller, **solver_kw).solve(problem, to.ODETerm(no_rhs), **kw)
+
+
+# ---------------------------------------------------------------------------------------------
+# part one: loop bookkeeping (reference tests/adjoint_test.py)
+# ---------------------------------------------------------------------------------------------
+
+
+def test_solution_is_evaluated_at_the_evaluation_points():
+    problem = curve_problem([[0.0, 2.0], [2.0, 4.0], [0.5, 2.5]])
+    sol = solve(ScriptedMethod(curve), ScriptedController(0.3, [0.3]), problem)
+    assert sol.status.tolist() == [OK] * 3
+    assert sol.stats["n_steps"].tolist() == [7, 7, 7] and sol.stats["n_accepted"].tolist() == [7, 7, 7]
+    assert sol.stats["n_initialized"].tolist() == [2, 2, 2]
+    assert sol.ts is problem.t_eval
+    assert torch.equal(sol.ys, curve(problem.t_eval))
+
+
+def test_samples_step_independently():
+    problem = curve_problem([[0.0, 0.15, 1.0], [1.0, 1.9, 2.0]])
+    sol = solve(ScriptedMethod(curve), ScriptedController([0.1, 0.3], [[0.5, 0.125]]), problem)
+    assert sol.status.tolist() == [OK, OK]
+    assert sol.stats["n_steps"].tolist() == [3, 7] and sol.stats["n_accepted"].tolist() == [3, 7]
+    assert sol.stats["n_initialized"].tolist() == [3, 3]
+    assert torch.equal(sol.ys, curve(problem.t_eval))
+
+
+def test_several_evaluation_points_inside_one_step():
+    problem = curve_problem([[0.0, 0.25, 0.33, 1.0]])
+    sol = solve(ScriptedMethod(curve), ScriptedController(0.1, [0.5]), problem)
+    assert sol.stats["n_steps"].tolist() == [3] and sol.stats["n_initialized"].tolist() == [4]
+    assert torch.equal(sol.ys, curve(problem.t_eval))
+
+
+def test_several_evaluation_points_on_the_last_step():
+    problem = curve_problem([[0.0, 1.0], [0.9, 1.0], [0.9, 1.0]], t_start=[0.0] * 3, t_end=[1.0] * 3)
+    sol = solve(ScriptedMethod(curve), ScriptedController([1.1, 1.1, 0.6], [0.6]), problem)
+    assert sol.stats["n_steps"].tolist() == [1, 1, 2] and sol.stats["n_accepted"].tolist() == [1, 1, 2]
+    assert sol.stats["n_initialized"].tolist() == [2, 2, 2]
+    assert torch.equal(sol.ys, curve(problem.t_eval))
+
+
+class ForwardEuler(SingleStepMethod):
+    """A user-defined method: y1 = y0 + dt f(t0, y0), no error estimate, linear dense output."""
+
+    def __init__(self, term=None):
+        super().__init__()
+        self.term = term
+
+    def init(self, term, problem, f0, *, stats, args):
+        return None
+
+    def step(self, term, running, y0, t0, dt, state, *, stats, args):
+        term = term if term is not None else self.term
+        y1 = y0 + dt[:, None] * term.vf(t0, y0, stats, args)
+        return StepResult(y1, None), (t0, dt, y0, y1), None, None
+
+    def merge_states(self, accept, current, previous):
+        return current
+
+    def build_interpolation(self, data):
+        return LinearInterpolation(*data)
+
+    def convergence_order(self):
+        return 1
+
+
+def test_without_evaluation_points_the_end_point_is_reported():
+    y0 = dev([[0.0], [1.0], [2.0]])
+    t_start, t_end = dev([0.0, 5.0, 2.0]), dev([10.0, 9.0, 4.5])
+    problem = to.InitialValueProblem(y0, t_start, t_end)
+    dt = [0.5001, 0.2501, 1.0]
+    term = to.ODETerm(lambda t, y: torch.ones_like(y))
+    sol = to.AutoDiffAdjoint(ForwardEuler(), ScriptedController(dt, [dt])).solve(problem, term)
+    assert sol.status.tolist() == [OK] * 3
+    assert sol.stats["n_steps"].tolist() == [20, 16, 3] and sol.stats["n_accepted"].tolist() == [20, 16, 3]
+    assert sol.stats["n_initialized"].tolist() == [1, 1, 1]
+    assert sol.stats["n_f_evals"].tolist() == [20] * 3 and sol.stats["n_f_evals"].device.type == "cpu"
+    assert sol.ts[:, 0].tolist() == t_end.tolist()
+    assert torch.allclose(sol.ys[:, 0], y0 + (t_end - t_start)[:, None], rtol=1e-5)
+
+
+def test_max_steps_stops_the_batch():
+    y0 = torch.zeros((2, 1), device=DEV)
+    t_eval = dev([[1.0, 4.9], [2.0, 13.0]])
+    problem = to.InitialValueProblem(y0, t_eval[:, 0], t_eval[:, -1], t_eval)
+    const = lambda t, *idx: y0[idx[0]] if idx else y0
+    sol = solve(ScriptedMethod(const), to.FixedStepController(), problem, max_steps=7, dt0=torch.ones(2, device=DEV))
+    assert sol.status.tolist() == [OK, MAX_STEPS]
+    assert sol.stats["n_steps"].tolist() == [4, 7] and sol.stats["n_initialized"].tolist() == [2, 1]
+
+
+def test_a_rejected_step_is_retried_from_the_same_time():
+    problem = curve_problem([[0.0, 1.0], [1.0, 2.0]])
+    method = ScriptedMethod(curve)
+    accept = [True, [True, False], [True, False], True]
+    sol = solve(method, ScriptedController(0.1, [0.5], accept), problem)
+    expected = [[0.0, 1.0], [0.1, 1.1], [0.6, 1.1], [1.0, 1.1], [1.0, 1.6]]
+    assert torch.stack(method.seen_t).cpu().numpy() == pytest.approx(np.array(expected))
+    assert sol.status.tolist() == [OK, OK]
+    assert sol.stats["n_steps"].tolist() == [3, 5] and sol.stats["n_accepted"].tolist() == [3, 3]
+    assert sol.stats["n_initialized"].tolist() == [2, 2]
+    assert torch.equal(sol.ys, curve(problem.t_eval))
+
+
+def test_a_value_is_stored_only_when_its_step_is_accepted():
+    problem = curve_problem([[0.6]] * 3, t_start=[0.0] * 3, t_end=[1.0] * 3)
+    calls = iter(range(3))
+
+    def fn(t, *idx):
+        if torch.all(t == dev(0.6)):  # the dense output: a different value on every call
+            out = torch.full((3, 1), float(next(calls)), device=DEV)
+            return out[idx[0]] if idx else out
+        return curve(t)
+
+    accept = [[False, True, True], [False, True, True], [True, True, True]]
+    dt = [[1.1, 0.0, 0.5], [1.1, 0.0, 0.0], [0.0] * 3]
+    sol = solve(ScriptedMethod(fn), ScriptedController([1.1, 1.1, 0.55], dt, accept), problem)
+    assert sol.stats["n_steps"].tolist() == [3, 1, 2] and sol.stats["n_accepted"].tolist() == [1, 1, 2]
+    assert sol.stats["n_initialized"].tolist() == [1, 1, 1]
+    assert sol.ys.tolist() == [[[2.0]], [[0.0]], [[1.0]]]
+
+
+def test_rejecting_the_first_step_keeps_the_value_at_t_start():
+    y0 = dev([[1.3], [2.5]])
+    const = lambda t, *idx: y0[idx[0]] if idx else y0
+    problem = to.InitialValueProblem(y0, dev([0.0, 0.0]), dev([1.0, 2.0]), dev([[0.0], [0.0]]))
+    sol = solve(ScriptedMethod(const), ScriptedController(0.6, [0.6], [[False, False], True]), problem)
+    assert sol.stats["n_steps"].tolist() == [3, 5] and sol.stats["n_accepted"].tolist() == [2, 4]
+    assert sol.stats["n_initialized"].tolist() == [1, 1]
+    assert torch.equal(sol.ys, y0[:, None])
+
+
+def test_a_failing_step_method_stops_every_sample():
+    problem = curve_problem([[0.0, 2.0], [2.0, 4.0]])
+    method = ScriptedMethod(curve, status=[[OK, OK]] * 3 + [[OK, FAILED]])
+    sol = solve(method, ScriptedController(0.2, [0.2]), problem)
+    assert sol.status.tolist() == [OK, FAILED]
+    assert sol.stats["n_steps"].tolist() == [4, 4] and sol.stats["n_accepted"].tolist() == [4, 4]
+    assert sol.stats["n_initialized"].tolist() == [1, 1]
+
+
+def test_a_failing_controller_stops_every_sample():
+    problem = curve_problem([[0.0, 2.0], [2.0, 4.0]])
+    ctrl = ScriptedController(0.2, [0.2], status=[[OK, OK]] * 5 + [[FAILED, OK]])
+    sol = solve(ScriptedMethod(curve), ctrl, problem)
+    assert sol.status.tolist() == [FAILED, OK]
+    assert sol.stats["n_steps"].tolist() == [6, 6] and sol.stats["n_initialized"].tolist() == [1, 1]
+
+
+def test_a_finished_sample_keeps_its_step_size():
+    # sample 1 finishes after one step with a tiny error; an adaptive controller must not keep
+    # growing its dt while sample 0 is still running
+    y0 = torch.zeros((2, 1), device=DEV)
+    const = lambda t, *idx: y0[idx[0]] if idx else y0
+    method = ScriptedMethod(const, error=lambda t: dev([[0.9], [1e-10]]))
+    problem = to.InitialValueProblem(y0, t_eval=dev([[0.0, 5.0], [0.0, 0.9]]))
+    sol = solve(method, to.IntegralController(atol=1.0, rtol=0.0), problem, dt0=torch.ones(2, device=DEV))
+    assert sol.status.tolist() == [OK, OK]
+    assert (torch.stack(method.seen_dt)[:, 1] < 1.1).all()
+
+
+def test_the_right_hand_side_is_only_evaluated_inside_the_time_range():
+    t_eval = dev([[0.1, 1.0], [1.0, 2.0], [1.0, 0.95]])  # long run / dt overshoots / backwards
+    seen = []
+
+    def rhs(t, y):
+        seen.append(t)
+        return -y
+
+    problem = to.InitialValueProblem(torch.ones((3, 1), device=DEV), t_eval=t_eval)
+    dt = [0.1, 0.4, -0.02]
+    sol = to.AutoDiffAdjoint(to.Dopri5(), ScriptedController(dt, [dt])).solve(problem, to.ODETerm(rhs))
+    times = torch.stack(seen)
+    lo, hi = torch.minimum(t_eval[:, 0], t_eval[:, 1]), torch.maximum(t_eval[:, 0], t_eval[:, 1])
+    assert (times >= lo).all() and (times <= hi).all()
+    assert sol.status.tolist() == [OK] * 3 and sol.ts.tolist() == t_eval.tolist()
+    assert torch.allclose(sol.ys[:, -1, 0], torch.exp(-(t_eval[:, 1] - t_eval[:, 0])), atol=1e-5)
+
+
+def test_extra_args_reach_the_right_hand_side_by_identity():
+    marker = object()
+    got = []
+
+    def rhs(t, y, args):
+        got.append(args)
+        return -y
+
+    problem = to.InitialValueProblem(torch.ones((2, 1), device=DEV), t_eval=dev([[0.0, 1.0], [0.0, 2.0]]))
+
+    class MyDopri5(to.Dopri5):  # a subclass is not recognised by the fused paths
+        pass
+
+    sol = to.AutoDiffAdjoint(MyDopri5(), to.IntegralController(1e-6, 1e-4)).solve(problem, to.ODETerm(rhs, with_args=True), args=marker)
+    assert sol.status.tolist() == [OK, OK] and got and all(a is marker for a in got)
+
+
+def test_user_defined_controller_can_wrap_a_library_controller():
+    class Logging(StepSizeController):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner, self.ratios = inner, []
+
+        def init(self, *a, **kw):
+            return self.inner.init(*a, **kw)
+
+        def adapt_step_size(self, t0, dt, y0, step_result, state, stats):
+            out = self.inner.adapt_step_size(t0, dt, y0, step_result, state, stats)
+            stats["n_adapt"] = stats.get("n_adapt", 0) + 1
+            return out
+
+        def merge_states(self, running, current, previous):
+            return self.inner.merge_states(running, current, previous)
+
+    w = to.workloads.make("vdp", batch=64, dtype=torch.float64, device=DEV)
+    inner = make_controller(w.controller)
+    sol = to.AutoDiffAdjoint(to.Tsit5(), Logging(inner)).solve(to.InitialValueProblem(w.y0, t_eval=w.t_eval), to.ODETerm(w.f))
+    ref = to.AutoDiffAdjoint(to.Tsit5(), inner).solve(to.InitialValueProblem(w.y0, t_eval=w.t_eval), to.ODETerm(w.f))
+    assert sol.stats["n_adapt"] == int(ref.stats["n_steps"].max())
+    assert torch.equal(sol.ys, ref.ys) and torch.equal(sol.stats["n_steps"], ref.stats["n_steps"])
+
+
+# ---------------------------------------------------------------------------------------------
+# part two: controllers, Runge-Kutta step, interpolation (reference unit tests)
+# ---------------------------------------------------------------------------------------------
+
+BOTH = [
+    lambda **kw: to.PIDController(atol=1.0, rtol=0.0, pcoeff=0, icoeff=1, dcoeff=0, **kw),
+    lambda **kw: to.IntegralController(atol=1.0, rtol=0.0, **kw),
+]
+
+
+def unit_problem(y0, t0, dt):
+    return to.InitialValueProblem(y0, t0, t0 + dt, t0.reshape((-1, 1)))
+
+
+@pytest.mark.parametrize("make", [lambda: to.PIDController(1, 1, 1, 1, 1), lambda: to.IntegralController(1.0, 0.0)])
+def test_no_error_estimate_keeps_the_step_size(make):
+    c = make()
+    t0, dt, y0 = dev([0.0]), dev([1.0]), dev([[1.0, 2.0, 3.0]])
+    state = c.initial_state(method_order=5, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    accept, dt_next, _, status = c.adapt_step_size(t0, dt, y0, StepResult(y0, None), state, stats={})
+    assert accept.tolist() == [True] and dt_next.tolist() == dt.tolist() and status is None
+
+
+@pytest.mark.parametrize("make", [lambda: to.PIDController(1, 1, 1, 1, 1), lambda: to.IntegralController(1.0, 0.0)])
+def test_zero_error_gives_a_finite_step_size(make):
+    c = make()
+    t0, dt, y0 = dev([0.0]), dev([1.0]), dev([[1.0, 2.0, 3.0]])
+    state = c.initial_state(method_order=5, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    _, dt_next, _, _ = c.adapt_step_size(t0, dt, y0, StepResult(y0, torch.zeros_like(y0)), state, stats={})
+    assert torch.isfinite(dt_next).all() and dt_next.item() == pytest.approx(10.0)
+
+
+@pytest.mark.parametrize("make", BOTH)
+def test_infinite_error_norm_is_reported(make):
+    c = make(norm=rms_norm)
+    t0, dt, y0 = torch.zeros(3, device=DEV), torch.ones(3, device=DEV), torch.ones((3, 2), device=DEV)
+    state = c.initial_state(method_order=5, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    err = dev([[1.0, 1.0], [torch.finfo(torch.float32).max, 1.0], [0.5, 1.25]])
+    _, _, _, status = c.adapt_step_size(t0, dt, y0, StepResult(y0, err), state, stats={})
+    assert status.tolist() == [OK, INF_NORM, OK]
+
+
+@pytest.mark.parametrize("make", BOTH)
+def test_nan_state_is_reported(make):
+    c = make(norm=max_norm)
+    t0, dt = torch.zeros(2, device=DEV), torch.ones(2, device=DEV)
+    y0 = dev([[float("nan"), 1.0], [1.5, 1.0]])
+    state = c.initial_state(method_order=5, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    _, _, _, status = c.adapt_step_size(t0, dt, y0, StepResult(y0, torch.ones((2, 2), device=DEV)), state, stats={})
+    assert status.tolist() == [INF_NORM, OK]
+
+
+@pytest.mark.parametrize("make", BOTH)
+def test_small_error_is_accepted_and_the_step_grows(make):
+    c = make(norm=max_norm)
+    t0, dt, y0 = dev([0.0, 1.5]), dev([1.0, 0.5]), dev([[1.0, 2.0], [3.0, 4.0]])
+    state = c.initial_state(method_order=5, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    result = StepResult(y0, torch.full_like(y0, 0.5))
+    accept, dt_next, state_next, status = c.adapt_step_size(t0, dt, y0, result, state, stats={})
+    assert accept.all() and (dt_next > dt).all() and (status == OK).all()
+    # hand value: ratio 0.5, factor 0.9 * 0.5**(-1/5)
+    assert dt_next.tolist() == pytest.approx([0.9 * 0.5**-0.2, 0.45 * 0.5**-0.2], rel=1e-6)
+    if isinstance(state, PIDState):
+        assert (state_next.prev_error_ratio != 1.0).all()
+        assert torch.equal(state_next.prev_prev_error_ratio, state.prev_error_ratio)
+    accept, dt_final, state_final, status = c.adapt_step_size(t0 + dt, dt_next, y0, result, state_next, stats={})
+    assert accept.all() and (dt_final > dt_next).all() and (status == OK).all()
+    if isinstance(state, PIDState):
+        assert torch.equal(state_final.prev_prev_error_ratio, state_final.prev_error_ratio)
+
+
+@pytest.mark.parametrize("make", BOTH)
+def test_dt_min_sets_the_status(make):
+    c = make(norm=max_norm, factor_min=0.0)
+    dt_min = dev(0.5)
+    t0, dt, y0 = dev([0.0, 0.0]), dev([1.0, 1.0]), dev([[1.0, 2.0], [3.0, 4.0]])
+    state = c.initial_state(2, unit_problem(y0, t0, dt), dt_min, dt_max=None)
+    result = StepResult(y0, dev([[0.9, 0.7], [0.0, 100.0]]))
+    accept, dt_next, state_next, status = c.adapt_step_size(t0, dt, y0, result, state, stats={})
+    assert accept.tolist() == [True, False] and dt_next[1] == dt_min and status.tolist() == [OK, DT_MIN]
+    if isinstance(state, PIDState):
+        assert state_next.prev_error_ratio[1] == state.prev_error_ratio[1]
+        assert state_next.prev_error_ratio[0] != state.prev_error_ratio[0]
+        assert state_next.prev_prev_error_ratio[1] == state.prev_prev_error_ratio[1]
+        assert state_next.prev_prev_error_ratio[0] == state.prev_error_ratio[0]
+
+
+def test_pid_history_is_kept_when_the_step_is_rejected():
+    t0, dt, y0 = dev([0.0, 2.5]), dev([1.0, 1.0]), dev([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    c = to.PIDController(atol=0.75, rtol=0, pcoeff=0, icoeff=1, dcoeff=0, norm=max_norm, safety=1.0)
+    state = c.initial_state(method_order=3, problem=unit_problem(y0, t0, dt), dt_min=None, dt_max=None)
+    state.prev_error_ratio = torch.rand((2,), device=DEV)
+    state.prev_prev_error_ratio = torch.rand((2,), device=DEV)
+    result = StepResult(y0, dev([[0.0, 0.8, 0.0], [0.0, 0.0, 0.0]]))
+    accept, dt_next, state_next, status = c.adapt_step_size(t0, dt, y0, result, state, stats={})
+    assert accept.tolist() == [False, True] and dt_next[0] < dt[0] and dt_next[1] > dt[1] and status.tolist() == [OK, OK]
+    assert state_next.prev_error_ratio[0] == state.prev_error_ratio[0]
+    assert state_next.prev_prev_error_ratio[0] == state.prev_prev_error_ratio[0]
+    assert state_next.prev_prev_error_ratio[1] == state.prev_error_ratio[1]
+
+
+@pytest.mark.parametrize("make", BOTH)
+def test_dt_max_limits_the_step(make):
+    c = make(norm=max_norm)
+    t0, dt, y0 = dev([0.0, 1.5]), dev([1.0, 0.5]), dev([[1.0, 2.0], [3.0, 4.0]])
+    problem = unit_problem(y0, t0, dt)
+    result = StepResult(y0, torch.full_like(y0, 0.5))
+    free = c.adapt_step_size(t0, dt, y0, result, c.initial_state(5, problem, None, None), stats={})[1]
+    assert (free > 0.4).any()
+    limited = c.adapt_step_size(t0, dt, y0, result, c.initial_state(5, problem, None, 0.4), stats={})[1]
+    assert (limited <= 0.4).all()
+
+
+def test_a_user_defined_norm_is_called_on_the_scaled_error():
+    seen = []
+
+    def l1(x):
+        seen.append(x)
+        return x.abs().mean(dim=1)
+
+    c = to.IntegralController(atol=0.5, rtol=0.5, norm=l1)
+    t0, dt = dev([0.0]), dev([1.0])
+    y0, y1, err = dev([[1.0, -3.0]]), dev([[2.0, 1.0]]), dev([[0.3, -0.4]])
+    state = c.initial_state(4, unit_problem(y0, t0, dt), None, None)
+    accept, dt_next, _, status = c.adapt_step_size(t0, dt, y0, StepResult(y1, err), state, stats={})
+    scaled = [0.3 / (0.5 + 0.5 * 2.0), 0.4 / (0.5 + 0.5 * 3.0)]
+    assert seen[0][0].tolist() == pytest.approx(scaled)
+    ratio = sum(scaled) / 2
+    assert accept.tolist() == [True] and status.tolist() == [OK]
+    assert dt_next.item() == pytest.approx(0.9 * ratio**-0.25, rel=1e-6)
+    assert c.dt_factor(state, dev([ratio])).item() == pytest.approx(0.9 * ratio**-0.25, rel=1e-6)
+
+
+class ThreeStage(ExplicitRungeKutta):
+    TABLEAU = ButcherTableau.from_lists(c=[0, 0.5, 1.0], a=[[], [1], [0.5, 0.5]], b=[1 / 3, 1 / 3, 1 / 3], b_low_order=[1 / 2, 0, 1 / 2])
+
+    def __init__(self, term):
+        super().__init__(term, ThreeStage.TABLEAU)
+
+
+def test_runge_kutta_step_with_a_user_tableau():
+    calls = []
+
+    def rhs(t, y):
+        calls.append((t, y))
+        return y
+
+    term = to.ODETerm(rhs)
+    problem = to.InitialValueProblem(dev([[1.0], [2.0]]), t_eval=dev([[0.0], [0.0]]))
+    method = ThreeStage(term)
+    assert not method.tableau.fsal and not method.tableau.ssal
+    stats = {}
+    term.init(problem, stats)
+    state = method.init(None, problem, None, stats=stats, args=None)
+    dt = dev([1.0, 1.0])
+    result, _, _, status = method.step(None, torch.ones(2, dtype=torch.bool, device=DEV), problem.y0, problem.t_start, dt, state, stats=stats, args=None)
+    assert status is None and len(calls) == 3 and stats["n_f_evals"].tolist() == [3, 3]
+    f_t, f_y = torch.stack([c[0] for c in calls]), torch.stack([c[1] for c in calls])
+    y0 = problem.y0
+    assert torch.allclose(f_t[0], problem.t_start) and torch.allclose(f_t[1], problem.t_start + 0.5 * dt) and torch.allclose(f_t[2], problem.t_start + dt)
+    assert torch.allclose(f_y[0], y0) and torch.allclose(f_y[1], y0 + dt[:, None] * y0)
+    assert torch.allclose(f_y[2], y0 + dt[:, None] * (y0 + f_y[1]) / 2)
+    assert torch.allclose(result.y, y0 + dt[:, None] * f_y.sum(dim=0) / 3)
+    assert torch.allclose(result.error_estimate, dt[:, None] * (-f_y[0] / 6 + f_y[1] / 3 - f_y[2] / 6))
+
+
+def test_library_tableaux_are_fsal_and_consistent():
+    for cls in (to.Dopri5, to.Tsit5):
+        tab = cls.TABLEAU
+        assert tab.fsal and tab.ssal and tab.n_stages == 7
+        assert torch.allclose(tab.a.sum(dim=1), tab.c, atol=1e-14) and abs(tab.b.sum().item() - 1) < 1e-14
+        assert abs(tab.b_err.sum().item()) < 1e-15
+    assert to.Dopri5.TABLEAU.b_other.shape == (1, 7) and to.Tsit5.TABLEAU.b_other.shape == (3, 7)
+    assert torch.allclose(to.Tsit5.TABLEAU.b_other.sum(dim=0)[1:], to.Tsit5.TABLEAU.b[1:], atol=1e-13)
+
+
+@pytest.mark.parametrize("cls,coef", [(ThirdOrderPolynomialInterpolation, [1.1, 0.2, -0.7, -2.8]), (FourthOrderPolynomialInterpolation, [1, -2, 5, 2.5, 3.7])])
+def test_polynomial_evaluation_on_a_batch(cls, coef):
+    t0, t1 = dev([2.5, 1.0, 5.0]), dev([5.0, 3.0, 6.0])
+    coefficients = [torch.full((3, 5), c, device=DEV) for c in coef]
+    interp = cls(t0, t1, coefficients)
+    out = interp.evaluate((t0 + t1) * 0.5, torch.arange(3, device=DEV))
+    assert np.allclose(out.cpu().numpy(), np.polynomial.Polynomial(coef)(0.5))
+    out = interp.evaluate(dev([3.0, 3.0]), dev([1, 0], torch.long))  # any order, any subset
+    assert np.allclose(out[0].cpu().numpy(), np.polynomial.Polynomial(coef)(1.0)) and np.allclose(out[1].cpu().numpy(), np.polynomial.Polynomial(coef)(0.2))
+
+
+def test_zero_length_step_does_not_produce_nan():
+    t0 = dev([1.0])
+    idx = torch.zeros(1, dtype=torch.long, device=DEV)
+    y0 = torch.rand((1, 5), device=DEV)
+    assert not torch.isnan(LinearInterpolation(t0, torch.zeros(1, device=DEV), y0, y0).evaluate(t0, idx)).any()
+    assert not torch.isnan(ThirdOrderPolynomialInterpolation(t0, t0, torch.rand((4, 1, 2), device=DEV)).evaluate(t0, idx)).any()
+    assert not torch.isnan(FourthOrderPolynomialInterpolation(t0, t0, torch.rand((5, 1, 2), device=DEV)).evaluate(t0, idx)).any()
+
+
+def test_cubic_and_quartic_from_stage_derivatives_recover_the_polynomial():
+    P = np.polynomial.Polynomial
+    t0, dt = np.array([0.3]), np.array([1.9])
+    p = P([1.1, 0.2, -0.7, -2.8], domain=(t0[0], (t0 + dt)[0]), window=(0, 1))
+    col = lambda x: dev(x)[:, None]
+    k = dev(np.stack([p.deriv()(t0), p.deriv()(t0 + dt)]))[..., None]
+    interp = ThirdOrderPolynomialInterpolation.from_k(dev(t0), dev(dt), col(p(t0)), col(p(t0 + dt)), k)
+    assert interp.t0.allclose(dev(t0)) and interp.t1.allclose(dev(t0 + dt))
+    assert torch.cat(interp.coefficients)[:, 0].cpu().numpy() == pytest.approx(p.coef, abs=1e-4)
+
+    t0, dt = np.array([1.0]), np.array([1.5])
+    p = P([1, -0.5, 1.2, 3.3, 0.5], domain=(t0[0], (t0 + dt)[0]), window=(0, 1))
+    k = dev(np.stack([p.deriv()(t0), (p(t0 + dt / 2) - p(t0)) / dt, p.deriv()(t0 + dt)]))[..., None]
+    interp = FourthOrderPolynomialInterpolation.from_k(dev(t0), dev(dt), col(p(t0)), col(p(t0 + dt)), k, torch.tensor([0.0, 1.0, 0.0]))
+    assert torch.cat(interp.coefficients)[:, 0].cpu().numpy() == pytest.approx(p.coef, abs=1e-5)
+
+    # Tsit5's free dense output recovers a quartic from its stage derivatives
+    c = to.Tsit5.TABLEAU.c.numpy()
+    k = dev(np.stack([p.deriv()(t0 + ci * dt) for ci in c]))[..., None]
+    interp = to.Tsit5.build_interpolation(None, ERKInterpolationData(to.Tsit5.TABLEAU, dev(t0), dev(dt), col(p(t0)), col(p(t0 + dt)), k))
+    assert torch.cat(interp.coefficients)[:, 0].cpu().numpy() == pytest.approx(p.coef, abs=5e-4)
+
+
+# ---------------------------------------------------------------------------------------------
+# part three: the protocol path against the C oracle
+# ---------------------------------------------------------------------------------------------
+
+
+class OwnTsit5(to.Tsit5):
+    """Not recognised by the fused paths: every protocol call goes through its own kernel."""
+
+
+class OwnDopri5(to.Dopri5):
+    pass
+
+
+def protocol_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, **extra):
+    mv = lambda x: None if x is None else x.to(DEV)
+    m = {"tsit5": OwnTsit5, "dopri5": OwnDopri5}[method]()
+    solver = to.AutoDiffAdjoint(m, make_controller(controller, **extra), max_steps=max_steps)
+    problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
+    return solver.solve(problem, to.ODETerm(copy.deepcopy(f).to(DEV)), dt0=mv(dt0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("name,batch", [("linear_decay", 256), ("vdp", 512), ("lorenz", 512)])
+def test_protocol_path_matches_oracle_bit_for_bit(name, batch, dtype):
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    sol = protocol_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller))
+
+
+@pytest.mark.parametrize("method", ["dopri5", "tsit5"])
+@pytest.mark.parametrize("kind", ["integral", "pid"])
+def test_protocol_path_other_pairs_and_limits(method, kind):
+    w = to.workloads.make("vdp", batch=300, dtype=torch.float32)
+    ctrl = dict(kind=kind, atol=1e-5, rtol=1e-3)
+    if kind == "pid":
+        ctrl.update(pcoeff=0.3, icoeff=0.4, dcoeff=0.1)
+    sol = protocol_solve(w.f, w.y0, w.t_eval, method, ctrl, dt_max=0.25, max_steps=60)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, method, ctrl, dt_max=0.25, max_steps=60))
+
+
+def test_protocol_path_without_evaluation_points_and_backwards():
+    w = to.workloads.make("linear_decay", batch=200, dtype=torch.float64)
+    t0, t1 = w.t_eval[:, 0].clone(), w.t_eval[:, -1].clone()
+    flip = torch.arange(200) % 3 == 0
+    t0[flip], t1[flip] = t1[flip], t0[flip].clone()
+    sol = protocol_solve(w.f, w.y0, None, w.method, w.controller, t_start=t0, t_end=t1)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=t0, t_end=t1))

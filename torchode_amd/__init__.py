@@ -9,7 +9,7 @@ from .problems import InitialValueProblem
 from .single_step_methods import Dopri5, Tsit5
 from .solution import Solution
 from .status_codes import Status
-from .step_size_controllers import IntegralController, PIDController
+from .step_size_controllers import FixedStepController, IntegralController, PIDController
 from .terms import ODETerm
 
 __all__ = [
@@ -19,6 +19,7 @@ __all__ = [
     "Tsit5",
     "Solution",
     "Status",
+    "FixedStepController",
     "IntegralController",
     "PIDController",
     "ODETerm",

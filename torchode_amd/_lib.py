@@ -37,6 +37,7 @@ EXPORTS = (
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
     "tode_last_solve_kernel_name",
+    "tode_tableau",
     "tode_erk_stage",
     "tode_erk_combine",
     "tode_error_scale",
@@ -46,6 +47,8 @@ EXPORTS = (
     "tode_initial_step_a",
     "tode_initial_step_b",
     "tode_quartic_build",
+    "tode_quartic_from_mid",
+    "tode_cubic_build",
     "tode_poly_eval",
     "tode_poly_eval_masked",
     "tode_select_rows",
@@ -230,6 +233,7 @@ def load():
         V, I32, I64, D = C.c_void_p, C.c_int32, C.c_int64, C.c_double
         DP, CP = C.POINTER(C.c_double), C.POINTER(Controller)
         for name, argtypes in {
+            "tode_tableau": [I32, DP, DP, DP, DP, C.POINTER(I32)],
             "tode_erk_stage": [I32, I64, I32, I32, DP, D] + [V] * 7,
             "tode_erk_combine": [I32, I64, I32, I32, DP] + [V] * 5,
             "tode_error_scale": [I32, I64, I32, D, D] + [V] * 5,
@@ -239,6 +243,8 @@ def load():
             "tode_initial_step_a": [I32, I32, I64, I32, D, D] + [V] * 8,
             "tode_initial_step_b": [I32, I32, I32, I32, I64, I32, D, D] + [V] * 8,
             "tode_quartic_build": [I32, I32, I64, I32] + [V] * 6,
+            "tode_quartic_from_mid": [I32, I64, I32] + [V] * 8,
+            "tode_cubic_build": [I32, I64, I32] + [V] * 7,
             "tode_poly_eval": [I32, I32, I64, I32, I64] + [V] * 7,
             "tode_poly_eval_masked": [I32, I32, I64, I32, I32] + [V] * 7,
             "tode_select_rows": [I32, I64, I32] + [V] * 5,

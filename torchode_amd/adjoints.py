@@ -7,10 +7,22 @@ import torch.nn as nn
 from . import _lib
 from .builtin_terms import BuiltinTerm
 from .problems import InitialValueProblem
-from .single_step_methods import ExplicitRungeKutta
+from .interpolation import _PolynomialInterpolation
+from .single_step_methods import Dopri5, Tsit5
 from .solution import Solution
-from .step_size_controllers import _AdaptiveController
+from .step_size_controllers import IntegralController, PIDController
 from .terms import ODETerm
+
+_PROTOCOL_NAMES = (
+    "init", "step", "merge_states", "build_interpolation", "convergence_order", "adapt_step_size", "update_state",
+    "initial_state", "dt_factor", "_select_initial_step",
+)  # fmt: skip
+
+
+def _library_object(obj, classes) -> bool:
+    """True if ``obj`` is exactly one of the library's classes with no protocol method replaced on
+    the instance; only then may a fused kernel stand in for the calls the loop would make."""
+    return type(obj) in classes and not any(name in vars(obj) for name in _PROTOCOL_NAMES)
 
 
 class AutoDiffAdjoint(nn.Module):
@@ -47,7 +59,7 @@ class AutoDiffAdjoint(nn.Module):
         dt0: Optional[torch.Tensor] = None,
         args: Any = None,
     ) -> Solution:
-        term_ = term if term is not None else self.step_method.term
+        term_ = term if term is not None else getattr(self.step_method, "term", None)
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
         if torch.is_grad_enabled() and any(
@@ -58,38 +70,145 @@ class AutoDiffAdjoint(nn.Module):
             )
         if self._persistent_ok(problem, term_):
             return self._solve_persistent(problem, term_, dt0)
-        if self._stepwise_ok(problem):
+        if self._stepwise_ok(problem, term_):
             return self._solve_stepwise(problem, term_, dt0, args)
-        raise NotImplementedError(
-            "this combination of step method, controller and dtypes has no kernel path yet "
-            "(supported: Dopri5/Tsit5 with IntegralController/PIDController and the RMS norm, "
-            "time dtype equal to the data dtype)"
-        )
+        if problem.data_dtype != problem.time_dtype or problem.data_dtype not in _lib.DTYPES:
+            raise NotImplementedError(
+                "the solve loop needs time and data in one dtype, float32 or float64 "
+                f"(got time {problem.time_dtype}, data {problem.data_dtype})"
+            )
+        return self._solve_protocol(problem, term, term_, dt0, args)
 
     # ------------------------------------------------------------------ #
-    def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
+    def _fused_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
         m, c = self.step_method, self.step_size_controller
         return (
-            isinstance(term.f, BuiltinTerm)
-            and not term.with_args
-            and type(m).__name__ in ("Dopri5", "Tsit5")
-            and isinstance(m, ExplicitRungeKutta)
-            and isinstance(c, _AdaptiveController)
+            _library_object(m, (Dopri5, Tsit5))
+            and _library_object(c, (IntegralController, PIDController))
             and c.fusable
+            and type(term) is ODETerm
+            and "vf" not in vars(term)
             and problem.data_dtype == problem.time_dtype
             and problem.data_dtype in _lib.DTYPES
         )
 
-    def _stepwise_ok(self, problem: InitialValueProblem) -> bool:
-        m, c = self.step_method, self.step_size_controller
-        return (
-            type(m).__name__ in ("Dopri5", "Tsit5")
-            and isinstance(m, ExplicitRungeKutta)
-            and isinstance(c, _AdaptiveController)
-            and c.fusable
-            and problem.data_dtype == problem.time_dtype
-            and problem.data_dtype in _lib.DTYPES
-        )
+    def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
+        return self._fused_ok(problem, term) and isinstance(term.f, BuiltinTerm) and not term.with_args
+
+    def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
+        return self._fused_ok(problem, term)
+
+    # ------------------------------------------------------------------ #
+    def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args) -> Solution:
+        """The loop of the reference (adjoints.py:50-311) against the plug-in protocols: any step
+        method, controller and interpolant, the library's or the user's.  The protocol methods are
+        called in the reference's order with the reference's arguments; the bookkeeping between them
+        is one kernel per iteration, and the host reads one small flag block per iteration (the
+        reference synchronises there as well)."""
+        lib = _lib.load()
+        method, controller = self.step_method, self.step_size_controller
+        dev, dtype, code = problem.device, problem.data_dtype, _lib.DTYPES[problem.data_dtype]
+        B, F, E = problem.batch_size, problem.n_features, problem.n_evaluation_points
+        stream = _lib.stream_of(problem.y0)
+        t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
+        t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
+        y = problem.y0.contiguous()
+        t = t_start
+        new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+
+        def as_float(x, shape):
+            x = torch.as_tensor(x, device=dev)
+            return x.to(dtype).expand(shape).contiguous()
+
+        def as_status(x):
+            return None if x is None else torch.as_tensor(x, device=dev).to(torch.long).expand((B,)).contiguous()
+
+        stats: Dict[str, Any] = {}
+        term_.init(problem, stats)
+        order = method.convergence_order()
+        dt, controller_state, f0 = controller.init(term, problem, order, dt0, stats=stats, args=args)
+        method_state = method.init(term, problem, f0, stats=stats, args=args)
+
+        ys = new(B, max(E, 1), F)
+        pending = new(B, E, dt=torch.uint8) if E > 0 else None
+        dt_in, dt = as_float(dt, (B,)), new(B)
+        rc = lib.tode_loop_begin(
+            code, B, F, E, _lib.ptr(t_start), _lib.ptr(t_end), _lib.ptr(t_eval), _lib.ptr(y), _lib.ptr(dt_in), _lib.ptr(dt),
+            _lib.ptr(pending), _lib.ptr(ys), stream,
+        )  # fmt: skip
+        _lib.check(rc, "tode_loop_begin")
+
+        running = torch.ones(B, dtype=torch.bool, device=dev)
+        n_steps = torch.zeros(B, dtype=torch.long, device=dev)
+        n_accepted = torch.zeros(B, dtype=torch.long, device=dev)
+        flags = new(_lib.LOOP_FLAG_WORDS, dt=torch.int32)
+
+        a = _lib.LoopArgs()
+        a.dtype, a.n_features, a.n_eval, a.batch = code, F, E, B
+        a.max_steps = -1 if self.max_steps is None else int(self.max_steps)
+        a.t_start, a.t_end = t_start.data_ptr(), t_end.data_ptr()
+        a.t_eval = None if t_eval is None else t_eval.data_ptr()
+        a.n_steps, a.n_accepted = n_steps.data_ptr(), n_accepted.data_ptr()
+        a.pending = None if pending is None else pending.data_ptr()
+        a.flags = flags.data_ptr()
+
+        while True:
+            step_result, interp_data, method_state_next, method_status = method.step(
+                term, running, y, t, dt, method_state, stats=stats, args=args
+            )
+            accept, dt_next, controller_state_next, controller_status = controller.adapt_step_size(
+                t, dt, y, step_result, controller_state, stats
+            )
+
+            # ---- one kernel: state update, counters, running, status, evaluation mask, next dt ----
+            y_new = as_float(step_result.y, (B, F))
+            accept_ = torch.as_tensor(accept, device=dev).to(torch.bool).expand((B,)).contiguous()
+            dt_next_ = as_float(dt_next, (B,))
+            m_status, c_status = as_status(method_status), as_status(controller_status)
+            t_out, dt_out, y_out = new(B), new(B), new(B, F)
+            running_out, to_update = new(B, dt=torch.bool), new(B, dt=torch.bool)
+            status = new(B, dt=torch.long)
+            to_evaluate = new(B, E, dt=torch.uint8) if E > 0 else None
+            a.t, a.dt, a.y, a.running = t.data_ptr(), dt.data_ptr(), y.data_ptr(), running.data_ptr()
+            a.y_new, a.accept, a.dt_next = y_new.data_ptr(), accept_.data_ptr(), dt_next_.data_ptr()
+            a.method_status = None if m_status is None else m_status.data_ptr()
+            a.controller_status = None if c_status is None else c_status.data_ptr()
+            a.t_out, a.dt_out, a.y_out = t_out.data_ptr(), dt_out.data_ptr(), y_out.data_ptr()
+            a.running_out, a.to_update, a.status = running_out.data_ptr(), to_update.data_ptr(), status.data_ptr()
+            a.to_evaluate = None if to_evaluate is None else to_evaluate.data_ptr()
+            _lib.check(lib.tode_loop_advance(_lib.C.byref(a), stream), "tode_loop_advance")
+            fl = flags.tolist()  # the iteration's host synchronisation
+
+            method_state = method.merge_states(to_update, method_state_next, method_state)
+
+            # ---- dense output at the evaluation points this step passed ----
+            if E > 0 and fl[_lib.LOOP_N_TO_EVALUATE] > 0:
+                interpolation = method.build_interpolation(interp_data)
+                if isinstance(interpolation, _PolynomialInterpolation) and type(interpolation).evaluate is _PolynomialInterpolation.evaluate:
+                    interpolation.evaluate_masked(t_eval, to_evaluate, ys)
+                else:
+                    hit = to_evaluate.view(torch.bool).nonzero()
+                    sample_idx, eval_idx = hit[:, 0], hit[:, 1]
+                    ys[sample_idx, eval_idx] = interpolation.evaluate(t_eval[sample_idx, eval_idx], sample_idx).to(dtype)
+
+            controller_state = controller.merge_states(running_out, controller_state_next, controller_state)
+            t, dt, y, running = t_out, dt_out, y_out, running_out
+
+            if fl[_lib.LOOP_ANY_RUNNING] and not fl[_lib.LOOP_ANY_FAILURE]:
+                continue
+
+            if m_status is None and c_status is None and self.max_steps is None:
+                status = torch.tensor(0, dtype=torch.long, device=dev).expand(B)
+            stats["n_steps"], stats["n_accepted"] = n_steps, n_accepted
+            if E > 0:
+                n_init = new(B, dt=torch.long)
+                _lib.check(lib.tode_count_initialized(B, E, _lib.ptr(pending), _lib.ptr(n_init), stream), "tode_count_initialized")
+                stats["n_initialized"] = n_init
+                return Solution(ts=problem.t_eval, ys=ys, stats=stats, status=status)
+            interpolation = method.build_interpolation(interp_data)
+            y_end = interpolation.evaluate(problem.t_end, torch.arange(B, device=dev))
+            stats["n_initialized"] = torch.ones(B, dtype=torch.long, device=dev)
+            return Solution(ts=problem.t_end[:, None], ys=y_end[:, None], stats=stats, status=status)
 
     # How many loop iterations are enqueued between two looks at the device flags.
     poll_first, poll_max = 4, 32

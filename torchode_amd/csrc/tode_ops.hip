@@ -299,6 +299,52 @@ __global__ void __launch_bounds__(256) quartic_build_kernel(long long batch, int
     for (int p = 0; p < 5; ++p) coeff[p * bf + i] = q[p][0];
 }
 
+// Quartic through y0, y1, the end-point slopes and a mid-point value (interpolation.py:138-170).
+template <typename T>
+__global__ void __launch_bounds__(256) quartic_from_mid_kernel(long long batch, int F, const T *dt, const T *y0, const T *y1, const T *k_first,
+                                                               const T *k_last, const T *y_mid, T *coeff) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long bf = batch * F;
+    if (i >= bf) return;
+    const T h = dt[i / F];
+    const T f0 = h * k_first[i], f1 = h * k_last[i], ym = y_mid[i], a0 = y0[i], a1 = y1[i];
+    T a = (T)2 * (f1 - f0);
+    a = fma_((T)-8, a1 + a0, a);
+    a = fma_((T)16, ym, a);
+    T b = (T)5 * f0;
+    b = fma_((T)-3, f1, b);
+    b = fma_((T)18, a0, b);
+    b = fma_((T)14, a1, b);
+    b = fma_((T)-32, ym, b);
+    T c = fma_((T)-4, f0, f1);
+    c = fma_((T)-11, a0, c);
+    c = fma_((T)-5, a1, c);
+    c = fma_((T)16, ym, c);
+    coeff[i] = a0;
+    coeff[bf + i] = f0;
+    coeff[2 * bf + i] = c;
+    coeff[3 * bf + i] = b;
+    coeff[4 * bf + i] = a;
+}
+
+// Hermite cubic through y0, y1 and the end-point slopes (interpolation.py:84-106).
+template <typename T>
+__global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F, const T *dt, const T *y0, const T *y1, const T *k_first,
+                                                          const T *k_last, T *coeff) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long bf = batch * F;
+    if (i >= bf) return;
+    const T h = dt[i / F];
+    const T f0 = k_first[i], f1 = k_last[i];
+    const T d01 = y0[i] - y1[i];
+    const T a = fma_((T)2, d01, h * (f0 + f1));            // add(dt*(f0+f1), y0-y1, alpha=2)
+    const T b = fma_((T)-3, d01, h * fma_((T)-2, f0, -f1));  // add(dt*add(-f1, f0, alpha=-2), y0-y1, alpha=-3)
+    coeff[i] = y0[i];
+    coeff[bf + i] = h * f0;
+    coeff[2 * bf + i] = b;
+    coeff[3 * bf + i] = a;
+}
+
 // x = (t - t0) / (t1 - t0) with a zero interval mapped to 1 (interpolation.py:8-40)
 template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) {
     T den = t1 - t0;
@@ -502,6 +548,27 @@ using namespace tode;
 
 extern "C" {
 
+int tode_tableau(int32_t method, double *c, double *a, double *b_err, double *b_other, int32_t *n_other) {
+    if (method != TODE_DOPRI5 && method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", method);
+    if (!c || !a || !b_err || !b_other || !n_other) return fail(TODE_E_INVALID, "null pointer");
+    auto fill = [&](auto tab) {
+        using Tab = decltype(tab);
+        for (int i = 0; i < 7; ++i) {
+            c[i] = Tab::c[i];
+            b_err[i] = Tab::b_err[i];
+            for (int j = 0; j < 7; ++j) a[i * 7 + j] = Tab::a[i][j];
+        }
+        *n_other = Tab::n_other;
+        for (int r = 0; r < 3; ++r)
+            for (int j = 0; j < 7; ++j) b_other[r * 7 + j] = r < Tab::n_other ? Tab::w[r][j] : 0.0;
+    };
+    if (method == TODE_TSIT5)
+        fill(Tsit5Tab{});
+    else
+        fill(Dopri5Tab{});
+    return TODE_OK;
+}
+
 int tode_erk_stage(int32_t dtype, int64_t batch, int32_t F, int32_t n_terms, const double *a, double c, const void *t0, const void *dt,
                    const void *y0, const void *k, void *y_out, void *t_out, void *stream) {
     if (int rc = check_common(dtype, batch, F)) return rc;
@@ -653,6 +720,26 @@ int tode_quartic_build(int32_t dtype, int32_t method, int64_t batch, int32_t F, 
                                (const T *)k, (T *)coeff);
     });
     return done("tode_quartic_build launch");
+}
+
+int tode_quartic_from_mid(int32_t dtype, int64_t batch, int32_t F, const void *dt, const void *y0, const void *y1, const void *k_first,
+                          const void *k_last, const void *y_mid, void *coeff, void *stream) {
+    if (int rc = check_common(dtype, batch, F)) return rc;
+    if (batch == 0) return TODE_OK;
+    if (!dt || !y0 || !y1 || !k_first || !k_last || !y_mid || !coeff) return fail(TODE_E_INVALID, "null pointer");
+    TODE_T(dtype, hipLaunchKernelGGL(quartic_from_mid_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
+                                     (const T *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (const T *)y_mid, (T *)coeff));
+    return done("tode_quartic_from_mid launch");
+}
+
+int tode_cubic_build(int32_t dtype, int64_t batch, int32_t F, const void *dt, const void *y0, const void *y1, const void *k_first,
+                     const void *k_last, void *coeff, void *stream) {
+    if (int rc = check_common(dtype, batch, F)) return rc;
+    if (batch == 0) return TODE_OK;
+    if (!dt || !y0 || !y1 || !k_first || !k_last || !coeff) return fail(TODE_E_INVALID, "null pointer");
+    TODE_T(dtype, hipLaunchKernelGGL(cubic_build_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
+                                     (const T *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (T *)coeff));
+    return done("tode_cubic_build launch");
 }
 
 int tode_poly_eval(int32_t dtype, int32_t degree, int64_t batch, int32_t F, int64_t count, const void *coeff, const void *t0, const void *t1,

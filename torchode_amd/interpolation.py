@@ -1,0 +1,155 @@
+"""Local interpolants of a single step (mirror torchode/interpolation.py).
+
+An interpolant answers ``evaluate(t, idx)``: the value of sample ``idx[n]``'s step
+polynomial at time ``t[n]``.  The polynomial classes keep their coefficients as one
+``[degree+1, B, F]`` device tensor and evaluate with one kernel; any other object with
+an ``evaluate`` method can be returned by a user-defined step method instead.
+"""
+from typing import Sequence, Union
+
+import torch
+
+from . import _lib
+
+
+class LocalInterpolation:
+    """Protocol (reference interpolation.py:43-45)."""
+
+    def evaluate(self, t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError()
+
+
+def _stack(coefficients: Union[torch.Tensor, Sequence[torch.Tensor]]) -> torch.Tensor:
+    if isinstance(coefficients, torch.Tensor):
+        return coefficients.contiguous()
+    return torch.stack(list(coefficients)).contiguous()
+
+
+class _PolynomialInterpolation(LocalInterpolation):
+    """Polynomial on [t0, t1] in x = (t - t0) / (t1 - t0); ``coefficients[i]`` belongs to x**i."""
+
+    degree = -1
+
+    def __init__(self, t0: torch.Tensor, t1: torch.Tensor, coefficients):
+        self.t0 = t0
+        self.t1 = t1
+        self._coeff = _stack(coefficients)
+        assert self._coeff.ndim == 3 and self._coeff.shape[0] == self.degree + 1
+        self.coefficients = tuple(self._coeff.unbind(0))
+
+    def _check(self, *times):
+        c = self._coeff
+        _lib.require_device(c, self.t0, self.t1, *times)
+        if c.dtype not in _lib.DTYPES or any(t.dtype != c.dtype for t in (self.t0, self.t1, *times)):
+            raise NotImplementedError("polynomial evaluation needs time and data in one dtype (float32 or float64)")
+
+    def evaluate(self, t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+        """reference interpolation.py:103-106, 172-175"""
+        self._check(t)
+        c = self._coeff
+        _, B, F = c.shape
+        t, idx = t.contiguous(), idx.to(torch.long).contiguous()
+        t0, t1 = self.t0.contiguous(), self.t1.contiguous()
+        out = c.new_empty((t.shape[0], F))
+        rc = _lib.load().tode_poly_eval(
+            _lib.DTYPES[c.dtype], self.degree, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
+            _lib.ptr(idx), _lib.ptr(out), _lib.stream_of(c),
+        )  # fmt: skip
+        _lib.check(rc, "tode_poly_eval")
+        return out
+
+    def evaluate_masked(self, t_eval: torch.Tensor, mask: torch.Tensor, ys: torch.Tensor) -> None:
+        """``ys[b, e] = p_b(t_eval[b, e])`` wherever ``mask[b, e]`` is set (one byte per entry);
+        the index list of reference adjoints.py:227-233 is never materialised."""
+        self._check(t_eval)
+        c = self._coeff
+        _, B, F = c.shape
+        assert t_eval.is_contiguous() and mask.is_contiguous() and ys.is_contiguous() and mask.element_size() == 1
+        t0, t1 = self.t0.contiguous(), self.t1.contiguous()
+        rc = _lib.load().tode_poly_eval_masked(
+            _lib.DTYPES[c.dtype], self.degree, B, F, t_eval.shape[1], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1),
+            _lib.ptr(t_eval), _lib.ptr(mask), _lib.ptr(ys), _lib.stream_of(c),
+        )  # fmt: skip
+        _lib.check(rc, "tode_poly_eval_masked")
+
+    def __repr__(self):
+        return f"{type(self).__name__}(t0={self.t0}, t1={self.t1}, coefficients={self.coefficients})"
+
+
+def _build_args(dt, y0, y1, *more):
+    _lib.require_device(dt, y0, y1, *more)
+    if y0.dtype not in _lib.DTYPES or dt.dtype != y0.dtype:
+        raise NotImplementedError("interpolant construction needs time and data in one dtype (float32 or float64)")
+    return [x.contiguous() for x in (dt, y0, y1, *more)]
+
+
+class LinearInterpolation(_PolynomialInterpolation):
+    """y0 + (y1 - y0) x (reference interpolation.py:48-62; x is taken over (t0 + dt) - t0)."""
+
+    degree = 1
+
+    def __init__(self, t0: torch.Tensor, dt: torch.Tensor, y0: torch.Tensor, y1: torch.Tensor):
+        super().__init__(t0, t0 + dt, (y0, y1 - y0))
+        self.dt = dt
+        self.y0 = y0
+        self.dy = self.coefficients[1]
+
+
+class ThirdOrderPolynomialInterpolation(_PolynomialInterpolation):
+    """reference interpolation.py:65-118"""
+
+    degree = 3
+
+    @staticmethod
+    def from_k(t0, dt, y0, y1, k):
+        """Hermite cubic from the first and last stage derivative (reference interpolation.py:84-106)."""
+        dt_, y0_, y1_, kf, kl = _build_args(dt, y0, y1, k[0], k[-1])
+        B, F = y0_.shape
+        coeff = y0_.new_empty((4, B, F))
+        rc = _lib.load().tode_cubic_build(
+            _lib.DTYPES[y0_.dtype], B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl),
+            _lib.ptr(coeff), _lib.stream_of(y0_),
+        )  # fmt: skip
+        _lib.check(rc, "tode_cubic_build")
+        return ThirdOrderPolynomialInterpolation(t0, t0 + dt, coeff)
+
+
+class FourthOrderPolynomialInterpolation(_PolynomialInterpolation):
+    """reference interpolation.py:121-181"""
+
+    degree = 4
+
+    @staticmethod
+    def from_k(t0, dt, y0, y1, k, b_mid):
+        """Quartic through both end points, their derivatives and the mid-point value
+        ``y0 + dt * sum_s b_mid[s] k[s]`` (reference interpolation.py:138-170)."""
+        dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+        S, B, F = k_.shape
+        lib, code, stream = _lib.load(), _lib.DTYPES[y0_.dtype], _lib.stream_of(y0_)
+        w = [float(x) for x in (b_mid.tolist() if isinstance(b_mid, torch.Tensor) else b_mid)]
+        assert len(w) == S <= _lib.MAX_STAGES
+        y_mid = torch.empty_like(y0_)
+        rc = lib.tode_erk_combine(code, B, F, S, (_lib.C.c_double * S)(*w), _lib.ptr(dt_), _lib.ptr(k_), _lib.ptr(y0_), _lib.ptr(y_mid), stream)
+        _lib.check(rc, "tode_erk_combine")
+        coeff = y0_.new_empty((5, B, F))
+        rc = lib.tode_quartic_from_mid(
+            code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_[0]), _lib.ptr(k_[-1]), _lib.ptr(y_mid),
+            _lib.ptr(coeff), stream,
+        )  # fmt: skip
+        _lib.check(rc, "tode_quartic_from_mid")
+        return FourthOrderPolynomialInterpolation(t0, t0 + dt, coeff)
+
+    @staticmethod
+    def from_erk_step(method_id: int, t0, dt, y0, y1, k):
+        """Dense output of a Dopri5 / Tsit5 step with the pair's own weights, one kernel
+        (reference tsit5.py:123-139, dopri5.py:53-60)."""
+        dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+        S, B, F = k_.shape
+        assert S == 7
+        coeff = y0_.new_empty((5, B, F))
+        rc = _lib.load().tode_quartic_build(
+            _lib.DTYPES[y0_.dtype], method_id, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_), _lib.ptr(coeff),
+            _lib.stream_of(y0_),
+        )  # fmt: skip
+        _lib.check(rc, "tode_quartic_build")
+        return FourthOrderPolynomialInterpolation(t0, t0 + dt, coeff)

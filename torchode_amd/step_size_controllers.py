@@ -1,17 +1,19 @@
-"""Adaptive step size controllers (mirror torchode/step_size_controllers.py:260-835).
+"""Step size controllers (mirror torchode/step_size_controllers.py).
 
-The classes keep the reference's constructor signatures and protocol methods.
-Their arithmetic runs in HIP kernels: inside the persistent whole-solve kernel
-when ``AutoDiffAdjoint`` recognises the whole configuration, and in the per-step
-kernels otherwise.
+The classes keep the reference's constructor signatures and protocol methods
+(``init``, ``adapt_step_size``, ``merge_states`` ...).  Their arithmetic runs in HIP
+kernels: inside the whole-solve kernel when ``AutoDiffAdjoint`` recognises the whole
+configuration, and one kernel per protocol call otherwise.  A user-defined controller
+subclasses ``StepSizeController``.
 """
 from math import sqrt
-from typing import Callable, Optional
+from typing import Any, Callable, Dict, NamedTuple, Optional, Tuple
 
 import torch
 import torch.nn as nn
 
 from . import _lib
+from .problems import InitialValueProblem
 from .terms import ODETerm
 
 
@@ -27,7 +29,102 @@ def max_norm(y: torch.Tensor) -> torch.Tensor:
     return torch.linalg.vector_norm(y, dim=1, ord=torch.inf)
 
 
-class _AdaptiveController(nn.Module):
+class StepSizeController(nn.Module):
+    """Protocol (reference step_size_controllers.py:16-113)."""
+
+    def init(self, term: Optional[ODETerm], problem: InitialValueProblem, method_order: int, dt0: Optional[torch.Tensor], *, stats: Dict[str, Any], args: Any):
+        """Returns ``(dt0, controller state, f(t_start, y0) or None)``; a step size suggested by the user wins."""
+        raise NotImplementedError()
+
+    def adapt_step_size(self, t0, dt, y0, step_result, state, stats: Dict[str, Any]):
+        """Returns ``(accept [B] bool, next dt [B], next state, status int64 [B] or None)``."""
+        raise NotImplementedError()
+
+    def merge_states(self, running: torch.Tensor, current, previous):
+        """State that is ``current`` for samples still running and ``previous`` for finished ones."""
+        raise NotImplementedError()
+
+
+class FixedStepState(NamedTuple):
+    accept_all: torch.Tensor
+    dt0: torch.Tensor
+
+
+class FixedStepController(StepSizeController):
+    """Accepts every step and keeps the step size (reference step_size_controllers.py:116-167)."""
+
+    def init(self, term, problem, method_order, dt0, *, stats, args):
+        assert dt0 is not None, "Fixed step size solving requires you to configure dt0"
+        accept_all = torch.ones(problem.batch_size, device=problem.device, dtype=torch.bool)
+        return dt0, FixedStepState(accept_all=accept_all, dt0=dt0), None
+
+    def adapt_step_size(self, t0, dt, y0, step_result, state: FixedStepState, stats):
+        return state.accept_all, state.dt0, state, None
+
+    def merge_states(self, running, current: FixedStepState, previous: FixedStepState):
+        return current
+
+
+def _almost_zero(dtype, device):
+    # lower bound of the error ratio (reference step_size_controllers.py:243-249)
+    return torch.tensor(1e-5 if dtype == torch.float16 else 1e-38, dtype=dtype, device=device)
+
+
+def _limit(x):
+    return None if x is None else float(x)
+
+
+class IntegralState:
+    """reference step_size_controllers.py:215-257"""
+
+    def __init__(self, method_order: int, almost_zero: torch.Tensor, dt_min=None, dt_max=None):
+        self.method_order = method_order
+        self.almost_zero = almost_zero
+        self.dt_min = dt_min
+        self.dt_max = dt_max
+
+    def update_error_ratios(self, prev_error_ratio, prev_prev_error_ratio):
+        return self
+
+    def __repr__(self):
+        return f"IState(method_order={self.method_order}, almost_zero={self.almost_zero}, dt_min={self.dt_min}, dt_max={self.dt_max})"
+
+    @staticmethod
+    def default(*, method_order: int, batch_size: int, dtype, device, dt_min, dt_max):
+        return IntegralState(method_order, _almost_zero(dtype, device), dt_min, dt_max)
+
+
+class PIDState:
+    """reference step_size_controllers.py:493-551: the error ratios of the last two accepted steps"""
+
+    def __init__(self, method_order: int, prev_error_ratio, prev_prev_error_ratio, almost_zero, dt_min=None, dt_max=None):
+        self.method_order = method_order
+        self.prev_error_ratio = prev_error_ratio
+        self.prev_prev_error_ratio = prev_prev_error_ratio
+        self.almost_zero = almost_zero
+        self.dt_min = dt_min
+        self.dt_max = dt_max
+
+    def update_error_ratios(self, prev_error_ratio, prev_prev_error_ratio):
+        return PIDState(self.method_order, prev_error_ratio, prev_prev_error_ratio, self.almost_zero, self.dt_min, self.dt_max)
+
+    def __repr__(self):
+        return (
+            f"PIDState(method_order={self.method_order}, prev_error_ratio={self.prev_error_ratio}, "
+            f"prev_prev_error_ratio={self.prev_prev_error_ratio}, almost_zero={self.almost_zero}, "
+            f"dt_min={self.dt_min}, dt_max={self.dt_max})"
+        )
+
+    @staticmethod
+    def default(*, method_order: int, batch_size: int, dtype, device, dt_min, dt_max):
+        ones = torch.ones(batch_size, dtype=dtype, device=device)
+        return PIDState(method_order, ones, ones, _almost_zero(dtype, device), dt_min, dt_max)
+
+
+class AdaptiveStepSizeController(StepSizeController):
+    """Error-ratio based control shared by the integral and the PID controller
+    (reference step_size_controllers.py:189-213, 333-490, 678-835)."""
+
     _kind = -1
 
     def __init__(self, atol, rtol, pcoeff, icoeff, dcoeff, term, norm, dt_min, dt_max, safety, factor_min, factor_max):
@@ -49,32 +146,152 @@ class _AdaptiveController(nn.Module):
         self._atol_f = float(torch.tensor(atol))
         self._rtol_f = float(torch.tensor(rtol))
 
+    # ------------------------------------------------------------------ #
     @property
     def fusable(self) -> bool:
-        """True when the device kernels implement this controller exactly (RMS norm)."""
+        """True when the whole-solve kernels implement this controller exactly (RMS norm)."""
         return self.norm is rms_norm
 
-    def c_struct(self) -> "_lib.Controller":
-        """Parameters in the layout of ``struct tode_controller``."""
+    def _norm_id(self) -> Optional[int]:
+        return {rms_norm: _lib.NORM_RMS, max_norm: _lib.NORM_MAX}.get(self.norm)
+
+    def c_struct(self, limits=None) -> "_lib.Controller":
+        """Parameters in the layout of ``struct tode_controller``.  ``limits`` is a
+        ``(dt_min, dt_max)`` pair of floats or ``None``s; by default the constructor's."""
+        dt_min, dt_max = (self.dt_min, self.dt_max) if limits is None else limits
         return _lib.Controller(
-            self._kind,
-            self.dt_min is not None,
-            self.dt_max is not None,
-            0,
-            self._atol_f,
-            self._rtol_f,
-            float(self.pcoeff),
-            float(self.icoeff),
-            float(self.dcoeff),
-            float(self.safety),
-            float(self.factor_min),
-            float(self.factor_max),
-            float(self.dt_min or 0.0),
-            float(self.dt_max or 0.0),
-        )
+            self._kind, dt_min is not None, dt_max is not None, 0, self._atol_f, self._rtol_f,
+            float(self.pcoeff), float(self.icoeff), float(self.dcoeff), float(self.safety),
+            float(self.factor_min), float(self.factor_max), float(dt_min or 0.0), float(dt_max or 0.0),
+        )  # fmt: skip
+
+    # ------------------------------------------------------------------ #
+    def initial_state(self, method_order: int, problem: InitialValueProblem, dt_min, dt_max):
+        raise NotImplementedError()
+
+    def update_state(self, state, y0, dt, error_ratio, accept):
+        raise NotImplementedError()
+
+    def _decide(self, state, dt, *, norm=None, y0=None, y1=None, err=None, limits=True):
+        """Runs the decision kernel: fused with the error norm when ``norm`` is None, from a
+        precomputed norm otherwise.  Returns (accept, dt_next, ratio, status, prev, prev_prev)."""
+        ref = dt if y0 is None else y0
+        _lib.require_device(dt, norm, y0, y1, err)
+        if ref.dtype not in _lib.DTYPES or dt.dtype != ref.dtype:
+            raise NotImplementedError("the step size controllers need time and data in one dtype (float32 or float64)")
+        dt = dt.contiguous()
+        B = dt.shape[0]
+        pid = self._kind == _lib.CTRL_PID
+        prev = state.prev_error_ratio.to(ref.dtype).contiguous() if pid else None
+        pprev = state.prev_prev_error_ratio.to(ref.dtype).contiguous() if pid else None
+        accept = torch.empty(B, dtype=torch.bool, device=dt.device)
+        dt_next, ratio = torch.empty_like(dt), torch.empty_like(dt)
+        status = torch.empty(B, dtype=torch.long, device=dt.device)
+        prev_o = torch.empty_like(dt) if pid else None
+        pprev_o = torch.empty_like(dt) if pid else None
+        # the limits in force are the state's (reference step_size_controllers.py:406-408)
+        c = self.c_struct((_limit(state.dt_min), _limit(state.dt_max)) if limits else (None, None))
+        lib, code, stream = _lib.load(), _lib.DTYPES[ref.dtype], _lib.stream_of(dt)
+        tail = (_lib.ptr(prev), _lib.ptr(pprev), _lib.ptr(accept), _lib.ptr(dt_next), _lib.ptr(ratio), _lib.ptr(status),
+                _lib.ptr(prev_o), _lib.ptr(pprev_o), stream)  # fmt: skip
+        if norm is None:
+            y0, y1, err = (x.contiguous() for x in (y0, y1, err))
+            assert y1.dtype == y0.dtype == err.dtype and y0.shape == y1.shape == err.shape
+            rc = lib.tode_adapt_step(
+                code, _lib.C.byref(c), int(state.method_order), self._norm_id(), B, y0.shape[1],
+                _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(y1), _lib.ptr(err), *tail,
+            )  # fmt: skip
+            _lib.check(rc, "tode_adapt_step")
+        else:
+            norm = norm.to(ref.dtype).contiguous()
+            rc = lib.tode_control(code, _lib.C.byref(c), int(state.method_order), B, _lib.ptr(norm), _lib.ptr(dt), *tail)
+            _lib.check(rc, "tode_control")
+        return accept, dt_next, ratio, status, prev_o, pprev_o
+
+    def dt_factor(self, state, error_ratio: torch.Tensor) -> torch.Tensor:
+        """Growth factor of the step size for a given error ratio, clipped to
+        ``[factor_min, factor_max]`` (reference step_size_controllers.py:289-294, 598-621)."""
+        ones = torch.ones_like(error_ratio)
+        return self._decide(state, ones, norm=error_ratio, limits=False)[1]
+
+    # ------------------------------------------------------------------ #
+    def init(self, term, problem: InitialValueProblem, method_order: int, dt0, *, stats, args):
+        """reference step_size_controllers.py:333-368, 678-713"""
+        if dt0 is None:
+            dt0, f0 = self._select_initial_step(term, problem, method_order, stats, args)
+        else:
+            f0 = None
+        dt_min, dt_max = self.dt_min, self.dt_max
+        if dt_min is not None:
+            dt_min = torch.tensor(dt_min, dtype=problem.time_dtype, device=problem.device)
+        if dt_max is not None:
+            dt_max = torch.tensor(dt_max, dtype=problem.time_dtype, device=problem.device)
+        return dt0, self.initial_state(method_order, problem, dt_min, dt_max), f0
+
+    def adapt_step_size(self, t0, dt, y0, step_result, state, stats):
+        """reference step_size_controllers.py:370-429, 715-774"""
+        y1, error_estimate = step_result.y, step_result.error_estimate
+        if error_estimate is None:
+            # no error estimate: accept and keep the step size
+            return torch.ones_like(dt, dtype=torch.bool), dt, self.update_state(state, y0, dt, None, None), None
+        if self._norm_id() is not None:
+            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, y0=y0, y1=y1, err=error_estimate)
+        else:
+            # user-defined norm: scale on the device, call the norm, decide on the device
+            _lib.require_device(y0, y1, error_estimate)
+            a, b, e = y0.contiguous(), y1.contiguous(), error_estimate.contiguous()
+            if a.dtype not in _lib.DTYPES or not (a.dtype == b.dtype == e.dtype):
+                raise NotImplementedError("the step size controllers need float32 or float64 data of one dtype")
+            scaled = torch.empty_like(a)
+            rc = _lib.load().tode_error_scale(
+                _lib.DTYPES[a.dtype], a.shape[0], a.shape[1], self._atol_f, self._rtol_f, _lib.ptr(a), _lib.ptr(b), _lib.ptr(e),
+                _lib.ptr(scaled), _lib.stream_of(a),
+            )  # fmt: skip
+            _lib.check(rc, "tode_error_scale")
+            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, norm=self.norm(scaled))
+        if self._kind == _lib.CTRL_PID and type(self).update_state is PIDController.update_state:
+            state = state.update_error_ratios(prev, pprev)  # the decision kernel has already shifted the history
+        else:
+            state = self.update_state(state, y0, dt, ratio, accept)
+        return accept, dt_next, state, status
+
+    def _select_initial_step(self, term, problem: InitialValueProblem, method_order: int, stats, args):
+        """Hairer, Norsett & Wanner I, Sec. II.4, with the tolerances applied to the norms
+        (reference step_size_controllers.py:431-490, 776-835).  Two kernels around the two
+        evaluations of ``f``."""
+        term_ = term if term is not None else self.term
+        assert term_ is not None
+        norm = self._norm_id()
+        if norm is None:
+            raise NotImplementedError("automatic selection of the first step needs rms_norm or max_norm; pass dt0 with a custom norm")
+        y0, t0, t1 = problem.y0.contiguous(), problem.t_start.contiguous(), problem.t_end.contiguous()
+        _lib.require_device(y0, t0, t1)
+        if y0.dtype not in _lib.DTYPES or t0.dtype != y0.dtype:
+            raise NotImplementedError("the step size controllers need time and data in one dtype (float32 or float64)")
+        B, F = y0.shape
+        lib, code, stream = _lib.load(), _lib.DTYPES[y0.dtype], _lib.stream_of(y0)
+        f0 = term_.vf(t0, y0, stats, args).contiguous()
+        h0, y1, tn = torch.empty_like(t0), torch.empty_like(y0), torch.empty_like(t0)
+        rc = lib.tode_initial_step_a(
+            code, norm, B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0),
+            _lib.ptr(h0), _lib.ptr(y1), _lib.ptr(tn), stream,
+        )  # fmt: skip
+        _lib.check(rc, "tode_initial_step_a")
+        f1 = term_.vf(tn, y1, stats, args).contiguous()
+        dt0 = torch.empty_like(t0)
+        rc = lib.tode_initial_step_b(
+            code, self._kind, norm, int(method_order), B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1),
+            _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(f1), _lib.ptr(h0), _lib.ptr(dt0), stream,
+        )  # fmt: skip
+        _lib.check(rc, "tode_initial_step_b")
+        return dt0, f0
 
 
-class IntegralController(_AdaptiveController):
+# name kept for the dispatch in adjoints.py
+_AdaptiveController = AdaptiveStepSizeController
+
+
+class IntegralController(AdaptiveStepSizeController):
     """Scales the step by ``safety * ratio**(-1/order)`` clipped to ``[factor_min, factor_max]``
     (reference step_size_controllers.py:260-294)."""
 
@@ -95,8 +312,20 @@ class IntegralController(_AdaptiveController):
     ):
         super().__init__(atol, rtol, 0.0, 1.0, 0.0, term, norm, dt_min, dt_max, safety, factor_min, factor_max)
 
+    def initial_state(self, method_order: int, problem: InitialValueProblem, dt_min, dt_max) -> IntegralState:
+        return IntegralState.default(
+            method_order=method_order, batch_size=problem.batch_size, dtype=problem.data_dtype, device=problem.device,
+            dt_min=dt_min, dt_max=dt_max,
+        )  # fmt: skip
 
-class PIDController(_AdaptiveController):
+    def merge_states(self, running, current: IntegralState, previous: IntegralState) -> IntegralState:
+        return current
+
+    def update_state(self, state: IntegralState, y0, dt, error_ratio, accept) -> IntegralState:
+        return state
+
+
+class PIDController(AdaptiveStepSizeController):
     """PID step size control after Soederlind (2003), eq. (34), with the coefficients divided by
     the method order (reference step_size_controllers.py:554-620)."""
 
@@ -119,3 +348,39 @@ class PIDController(_AdaptiveController):
         factor_max: float = 10.0,
     ):
         super().__init__(atol, rtol, pcoeff, icoeff, dcoeff, term, norm, dt_min, dt_max, safety, factor_min, factor_max)
+
+    def initial_state(self, method_order: int, problem: InitialValueProblem, dt_min, dt_max) -> PIDState:
+        return PIDState.default(
+            method_order=method_order, batch_size=problem.batch_size, dtype=problem.data_dtype, device=problem.device,
+            dt_min=dt_min, dt_max=dt_max,
+        )  # fmt: skip
+
+    def merge_states(self, running, current: PIDState, previous: PIDState) -> PIDState:
+        """reference step_size_controllers.py:628-638"""
+        mask = running.contiguous()
+        assert mask.element_size() == 1
+        outs = []
+        for cur, prev in ((current.prev_error_ratio, previous.prev_error_ratio), (current.prev_prev_error_ratio, previous.prev_prev_error_ratio)):
+            _lib.require_device(cur, prev, mask)
+            cur, prev = cur.contiguous(), prev.contiguous()
+            assert cur.dtype == prev.dtype and cur.dtype in _lib.DTYPES
+            out = torch.empty_like(cur)
+            rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], cur.shape[0], 1, _lib.ptr(mask), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
+            _lib.check(rc, "tode_select_rows")
+            outs.append(out)
+        return current.update_error_ratios(*outs)
+
+    def update_state(self, state: PIDState, y0, dt, error_ratio, accept) -> PIDState:
+        """reference step_size_controllers.py:640-671"""
+        if error_ratio is None:
+            return state.update_error_ratios(prev_error_ratio=y0.new_ones(dt.shape), prev_prev_error_ratio=state.prev_error_ratio)
+        assert accept is not None
+        mask = accept.contiguous()
+        outs = []
+        for cur, prev in ((error_ratio, state.prev_error_ratio), (state.prev_error_ratio, state.prev_prev_error_ratio)):
+            cur, prev = cur.contiguous(), prev.contiguous()
+            out = torch.empty_like(cur)
+            rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], cur.shape[0], 1, _lib.ptr(mask), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
+            _lib.check(rc, "tode_select_rows")
+            outs.append(out)
+        return state.update_error_ratios(*outs)
