@@ -385,6 +385,107 @@ def quartic_eval(coeff, t0, t1, t, idx):
 # --------------------------------------------------------------------------- #
 
 
+def run_loop(
+    y0: torch.Tensor,
+    t_start: torch.Tensor,
+    t_end: torch.Tensor,
+    t_eval: Optional[torch.Tensor],
+    dt: torch.Tensor,
+    step: Callable,
+    adapt: Callable,
+    merge_method: Callable,
+    merge_controller: Callable,
+    dense: Callable,
+    method_state,
+    controller_state,
+    *,
+    max_steps: Optional[int] = None,
+    on_iteration: Optional[Callable] = None,
+):
+    """The loop of adjoints.py:50-309 with the step method and the controller as callables:
+
+      step(running, y, t, dt, method_state) -> (y1, interp_data, method_state_next, status | None)
+      adapt(t, dt, y, y1, interp_data, controller_state) -> (accept, dt_next, controller_state_next, status | None)
+      merge_method(move, new, old), merge_controller(running, new, old) -> state
+      dense(interp_data) -> evaluate(t[n], idx[n]) -> [n, F]
+
+    Returns (ys, status | None, n_steps, n_accepted, n_initialized, iterations).
+
+    pinned by: the loop cases of tests/adjoint_test.py:26-319 restated with scripted
+    callables (evaluation points hit exactly, independent stepping, several points in
+    one step / on the last step, end-point evaluation, max_steps, retry after rejection,
+    values stored on accept only, first-step rejection, method / controller failure,
+    finished samples keep dt).
+    """
+    B = y0.shape[0]
+    direction = torch.where(t_end > t_start, 1, -1).to(dtype=t_start.dtype)
+    t, y = t_start, y0
+    n_steps = torch.zeros(B, dtype=torch.long)
+    n_accepted = torch.zeros(B, dtype=torch.long)
+    t_min, t_max = torch.minimum(t_start, t_end), torch.maximum(t_end, t_start)
+    if t_eval is not None:
+        ys = y0.new_empty((B, t_eval.shape[1], y0.shape[1]))
+        pending = torch.ones_like(t_eval, dtype=torch.bool)
+        neg_eval = -direction[:, None] * t_eval
+    neg_end = -direction * t_end
+    running = torch.ones(B, dtype=torch.bool)
+    dt = torch.clamp(dt, t_min - t, t_max - t)
+
+    if t_eval is not None:
+        at_start = t_eval[:, 0] == t_start
+        ys[at_start, 0] = y[at_start]
+        pending[at_start, 0] = False
+
+    iterations = 0
+    while True:
+        iterations += 1
+        y1, interp_data, method_state_next, method_status = step(running, y, t, dt, method_state)
+        accept, dt_next, controller_state_next, controller_status = adapt(t, dt, y, y1, interp_data, controller_state)
+
+        move = accept & running
+        if on_iteration is not None:
+            on_iteration(t, dt, accept, running, controller_state_next)
+        t = torch.where(move, t + dt, t)
+        y = torch.where(move[:, None], y1, y)
+        method_state = merge_method(move, method_state_next, method_state)
+        n_steps.add_(running)
+        n_accepted.add_(move)
+
+        running = torch.addcmul(neg_end, direction, t) < 0.0
+        status = method_status
+        if status is None:
+            status = controller_status
+        elif controller_status is not None:
+            status = torch.maximum(status, controller_status)
+        if max_steps is not None:
+            status = torch.where(n_steps >= max_steps, REACHED_MAX_STEPS, status if status is not None else SUCCESS)
+        go_on = torch.any(running)
+        if status is not None:
+            go_on = go_on & torch.all(status == SUCCESS)
+
+        if t_eval is not None:
+            hit = (torch.addcmul(neg_eval, direction[:, None], t[:, None]) >= 0.0) & pending
+            if hit.any():
+                evaluate = dense(interp_data)
+                nz = hit.nonzero()
+                si, ei = nz[:, 0], nz[:, 1]
+                ys[si, ei] = evaluate(t_eval[si, ei], si)
+                pending = torch.logical_xor(hit, pending)
+
+        dt = torch.where(running, dt_next, dt)
+        dt = torch.clamp(dt, t_min - t, t_max - t)
+        controller_state = merge_controller(running, controller_state_next, controller_state)
+
+        if bool(go_on):
+            continue
+
+        if t_eval is not None:
+            n_init = torch.searchsorted(pending.int(), torch.ones((B, 1), dtype=torch.int)).squeeze(dim=1)
+            return ys, status, n_steps, n_accepted, n_init, iterations
+        y_end = dense(interp_data)(t_end, torch.arange(B))
+        return y_end[:, None], status, n_steps, n_accepted, torch.ones(B, dtype=torch.long), iterations
+
+
 def solve(
     f: Callable,
     y0: torch.Tensor,
@@ -398,7 +499,8 @@ def solve(
     max_steps: Optional[int] = None,
     trace: Optional[list] = None,
 ) -> Dict[str, torch.Tensor]:
-    """adjoints.py:50-309 for (Dopri5|Tsit5) x (Integral|PID, rms norm).
+    """adjoints.py:50-309 for (Dopri5|Tsit5) x (Integral|PID, rms norm): ``run_loop`` with
+    the Runge-Kutta step, the error-ratio controller and the quartic dense output plugged in.
 
     ``f(t, y)`` is any torch callable.  Returns a dict with ys, ts, status and
     the four stats (n_f_evals is the batch-uniform CPU counter of terms.py).
@@ -417,7 +519,6 @@ def solve(
     order = ORDER[method]
     tab = TABLEAUX[method].cast(t_start.dtype, y0.dtype)
     direction_i = torch.where(t_end > t_start, 1, -1)
-    direction = direction_i.to(dtype=t_start.dtype)
 
     calls = [0]
 
@@ -425,80 +526,44 @@ def solve(
         calls[0] += 1
         return f(t, y)
 
-    t, y = t_start, y0
-    n_steps = torch.zeros(B, dtype=torch.long)
-    n_accepted = torch.zeros(B, dtype=torch.long)
-    t_min, t_max = torch.minimum(t_start, t_end), torch.maximum(t_end, t_start)
-    if t_eval is not None:
-        ys = y0.new_empty((B, t_eval.shape[1], y0.shape[1]))
-        pending = torch.ones_like(t_eval, dtype=torch.bool)
-        neg_eval = -direction[:, None] * t_eval
-    neg_end = -direction * t_end
-    running = torch.ones(B, dtype=torch.bool)
-
     if dt0 is None:
         dt, k0 = initial_step(vf, controller, order, t_start, y0, direction_i, (t_end - t_start).abs())
     else:
         dt, k0 = dt0, vf(t_start, y0)
-    prev = prev_prev = torch.ones(B, dtype=y0.dtype)
-    dt = torch.clamp(dt, t_min - t, t_max - t)
+    ones = torch.ones(B, dtype=y0.dtype)
 
-    if t_eval is not None:
-        at_start = t_eval[:, 0] == t_start
-        ys[at_start, 0] = y[at_start]
-        pending[at_start, 0] = False
-
-    while True:
+    def step(running, y, t, dt, k0):
         y1, err, k = erk_step(vf, tab, t, dt, y, k0)
-        accept, dt_next, status, ratio, prev_n, prev_prev_n = adapt(controller, order, dt, y, y1, err, prev, prev_prev)
-        step_t0, step_dt, step_y0 = t, dt, y
+        return y1, (t, dt, y, y1, err, k), k[-1], None
 
-        move = accept & running
-        t = torch.where(move, t + dt, t)
-        y = torch.where(move[:, None], y1, y)
-        k0 = torch.where(move[:, None], k[-1], k0)
-        n_steps.add_(running)
-        n_accepted.add_(move)
+    def adapt_(t, dt, y, y1, data, state):
+        accept, dt_next, status, ratio, prev_n, prev_prev_n = adapt(controller, order, dt, y, y1, data[4], *state)
+        return accept, dt_next, (prev_n, prev_prev_n, ratio), status
+
+    def merge_method(move, new, old):
+        return torch.where(move[:, None], new, old)
+
+    def merge_controller(running, new, old):
+        return torch.where(running, new[0], old[0]), torch.where(running, new[1], old[1])
+
+    def dense(data):
+        t0, dt, y, y1, _, k = data
+        coeff = quartic_tsit5(tab, dt, y, k) if method == "tsit5" else quartic_dopri5(tab, dt, y, y1, k)
+        return lambda tt, idx: quartic_eval(coeff, t0, t0 + dt, tt, idx)
+
+    def on_iteration(t, dt, accept, running, state_next):
         if trace is not None:
-            trace.append(dict(t=step_t0.clone(), dt=step_dt.clone(), ratio=ratio.clone(), accept=accept.clone(), running=running.clone()))
+            trace.append(dict(t=t.clone(), dt=dt.clone(), ratio=state_next[2].clone(), accept=accept.clone(), running=running.clone()))
 
-        running = torch.addcmul(neg_end, direction, t) < 0.0
-        if max_steps is not None:
-            status = torch.where(n_steps >= max_steps, REACHED_MAX_STEPS, status)
-        go_on = bool(torch.any(running) & torch.all(status == SUCCESS))
-
-        if t_eval is not None:
-            hit = (torch.addcmul(neg_eval, direction[:, None], t[:, None]) >= 0.0) & pending
-            if hit.any():
-                if method == "tsit5":
-                    coeff = quartic_tsit5(tab, step_dt, step_y0, k)
-                else:
-                    coeff = quartic_dopri5(tab, step_dt, step_y0, y1, k)
-                nz = hit.nonzero()
-                si, ei = nz[:, 0], nz[:, 1]
-                ys[si, ei] = quartic_eval(coeff, step_t0, step_t0 + step_dt, t_eval[si, ei], si)
-                pending = torch.logical_xor(hit, pending)
-
-        dt = torch.where(running, dt_next, dt)
-        dt = torch.clamp(dt, t_min - t, t_max - t)
-        prev = torch.where(running, prev_n, prev)
-        prev_prev = torch.where(running, prev_prev_n, prev_prev)
-
-        if go_on:
-            continue
-
-        stats = {
-            "n_f_evals": torch.full((B,), calls[0], dtype=torch.long),
-            "n_steps": n_steps,
-            "n_accepted": n_accepted,
-        }
-        if t_eval is not None:
-            stats["n_initialized"] = torch.searchsorted(pending.int(), torch.ones((B, 1), dtype=torch.int)).squeeze(dim=1)
-            return dict(ts=t_eval, ys=ys, status=status, **stats)
-        if method == "tsit5":
-            coeff = quartic_tsit5(tab, step_dt, step_y0, k)
-        else:
-            coeff = quartic_dopri5(tab, step_dt, step_y0, y1, k)
-        y_end = quartic_eval(coeff, step_t0, step_t0 + step_dt, t_end, torch.arange(B))
-        stats["n_initialized"] = torch.ones(B, dtype=torch.long)
-        return dict(ts=t_end[:, None], ys=y_end[:, None], status=status, **stats)
+    ys, status, n_steps, n_accepted, n_init, _ = run_loop(
+        y0, t_start, t_end, t_eval, dt, step, adapt_, merge_method, merge_controller, dense, k0, (ones, ones),
+        max_steps=max_steps, on_iteration=on_iteration,
+    )  # fmt: skip
+    stats = {
+        "n_f_evals": torch.full((B,), calls[0], dtype=torch.long),
+        "n_steps": n_steps,
+        "n_accepted": n_accepted,
+        "n_initialized": n_init,
+    }
+    ts = t_eval if t_eval is not None else t_end[:, None]
+    return dict(ts=ts, ys=ys, status=status, **stats)
