@@ -31,7 +31,13 @@ enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1 };
 /* step size controllers: reference step_size_controllers.py:260 (integral), :554 (PID) */
 enum { TODE_CTRL_INTEGRAL = 0, TODE_CTRL_PID = 1 };
 /* right-hand sides the persistent kernel evaluates itself */
-enum { TODE_TERM_LINEAR_DECAY = 0, TODE_TERM_VAN_DER_POL = 1, TODE_TERM_LORENZ63 = 2 };
+enum {
+    TODE_TERM_LINEAR_DECAY = 0,       /* dy/dt = -k y, k [B,F] */
+    TODE_TERM_VAN_DER_POL = 1,        /* F = 2, mu [B] */
+    TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
+    TODE_TERM_REACTION_DIFFUSION = 3  /* F = N*N periodic grid (N = 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
+                                         float32, tode_solve_builtin_fast only */
+};
 /* per-sample status codes: reference status_codes.py:9-13 */
 enum {
     TODE_SUCCESS = 0,

@@ -4,7 +4,7 @@ __version__ = "0.1.0"
 
 from . import builtin_terms, workloads
 from .adjoints import AutoDiffAdjoint
-from .builtin_terms import LinearDecay, Lorenz63, VanDerPol
+from .builtin_terms import LinearDecay, Lorenz63, MLPField, ReactionDiffusion, VanDerPol
 from .problems import InitialValueProblem
 from .single_step_methods import Dopri5, Tsit5
 from .solution import Solution
@@ -26,4 +26,6 @@ __all__ = [
     "LinearDecay",
     "VanDerPol",
     "Lorenz63",
+    "ReactionDiffusion",
+    "MLPField",
 ]

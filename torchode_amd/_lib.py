@@ -17,6 +17,8 @@ ABI_VERSION = 3
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
+PERSISTENT_TERMS = (0, 1, 2, 3)  # TODE_TERM_* that a whole-solve kernel evaluates itself
+GENERAL_TERMS = (0, 1, 2)  # ... of which these also have the general kernel (every case, not only the common one)
 FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_NEEDS_GENERAL, FLAG_WORDS = 0, 1, 2, 3, 4
 INT32_MAX = 2**31 - 1
 

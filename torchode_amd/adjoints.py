@@ -69,7 +69,9 @@ class AutoDiffAdjoint(nn.Module):
                 "torchode_amd's solve loop is forward-only; call it under torch.no_grad() or detach the inputs"
             )
         if self._persistent_ok(problem, term_):
-            return self._solve_persistent(problem, term_, dt0)
+            sol = self._solve_persistent(problem, term_, dt0)
+            if sol is not None:
+                return sol
         if self._stepwise_ok(problem, term_):
             return self._solve_stepwise(problem, term_, dt0, args)
         if problem.data_dtype != problem.time_dtype or problem.data_dtype not in _lib.DTYPES:
@@ -93,10 +95,12 @@ class AutoDiffAdjoint(nn.Module):
         )
 
     def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        return self._fused_ok(problem, term) and isinstance(term.f, BuiltinTerm) and not term.with_args
+        f = term.f
+        return self._fused_ok(problem, term) and isinstance(f, BuiltinTerm) and f.builtin_kind in _lib.PERSISTENT_TERMS and not term.with_args
 
     def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        return self._fused_ok(problem, term)
+        # the per-step kernels walk a sample's row in one thread: small rows only
+        return self._fused_ok(problem, term) and problem.n_features < 64
 
     # ------------------------------------------------------------------ #
     def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args) -> Solution:
@@ -349,13 +353,23 @@ class AutoDiffAdjoint(nn.Module):
 
         # Common case first: one kernel, int64 stats written directly.  It reports through the
         # flag block when the batch needs the general kernel (which handles every case).
-        if self.use_fast_path and E > 0 and not ctrl.has_dt_min and not ctrl.has_dt_max and E * y0.element_size() <= 1024:
+        has_general = f.builtin_kind in _lib.GENERAL_TERMS
+        fast_ok = E > 0 and not ctrl.has_dt_min and not ctrl.has_dt_max
+        if has_general:
+            fast_ok = fast_ok and self.use_fast_path and E * y0.element_size() <= 1024
+        else:
+            fast_ok = fast_ok and dtype == torch.float32 and F in (32 * 32, 64 * 64) and E <= 8192
+            if not fast_ok:
+                return None  # no whole-solve kernel for this case: the caller takes the protocol path
+        if fast_ok:
             out = torch.empty((4, B), dtype=torch.int64, device=dev)
             rc = lib.tode_solve_builtin_fast(
                 _lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream
             )
             _lib.check(rc, "tode_solve_builtin_fast")
             fl = flags.tolist()  # the one host synchronisation of the solve
+            if fl[_lib.FLAG_NEEDS_GENERAL] and not has_general:
+                return None
             if not fl[_lib.FLAG_NEEDS_GENERAL]:
                 if term.with_stats:
                     last = fl[_lib.FLAG_MAX_ITERATIONS]

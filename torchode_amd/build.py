@@ -43,6 +43,7 @@ UNITS = [
     ("tode_pair.hip", "tode_pair_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
     ("tode_stepwise.hip", "tode_stepwise.o", []),
     ("tode_ops.hip", "tode_ops.o", []),
+    ("tode_grid.hip", "tode_grid.o", []),
 ]
 
 

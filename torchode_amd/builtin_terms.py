@@ -14,6 +14,8 @@ import torch.nn as nn
 TERM_LINEAR_DECAY = 0
 TERM_VAN_DER_POL = 1
 TERM_LORENZ63 = 2
+TERM_REACTION_DIFFUSION = 3
+TERM_MLP = 4
 
 
 class BuiltinTerm(nn.Module):
@@ -89,3 +91,48 @@ class Lorenz63(BuiltinTerm):
 
     def builtin_scalars(self):
         return (self.sigma, self.beta)
+
+
+class ReactionDiffusion(BuiltinTerm):
+    """Fisher-KPP reaction-diffusion on a periodic ``n x n`` grid with unit spacing, one
+    diffusivity per sample (``D`` of shape ``[B]``); the state is the flattened grid, ``F = n*n``:
+    ``du/dt = D * lap(u) + u * (1 - u)`` with the five-point Laplacian summed as
+    ``(((up + down) + left) + right) - 4u``."""
+
+    builtin_kind = TERM_REACTION_DIFFUSION
+
+    def __init__(self, D: torch.Tensor, n: int = 64):
+        super().__init__()
+        assert D.ndim == 1
+        self.register_buffer("D", D)
+        self.n = int(n)
+        self.n_features = self.n * self.n
+
+    def forward(self, t, y):
+        u = y.view(y.shape[0], self.n, self.n)
+        lap = (((torch.roll(u, 1, 1) + torch.roll(u, -1, 1)) + torch.roll(u, 1, 2)) + torch.roll(u, -1, 2)) - (4 * u)
+        return (self.D[:, None, None] * lap + u * (1 - u)).flatten(1)
+
+    def builtin_params(self):
+        return self.D.reshape(-1, 1).contiguous()
+
+
+class MLPField(BuiltinTerm):
+    """Time-dependent two-layer perceptron shared by the whole batch:
+    ``f(t, y) = tanh(cat([y, t], 1) @ W1.T + b1) @ W2.T + b2`` with ``W1 [H, F+1]``, ``W2 [F, H]``."""
+
+    builtin_kind = TERM_MLP
+
+    def __init__(self, W1: torch.Tensor, b1: torch.Tensor, W2: torch.Tensor, b2: torch.Tensor):
+        super().__init__()
+        assert W1.ndim == 2 and W2.ndim == 2 and W1.shape[0] == W2.shape[1] and W1.shape[1] == W2.shape[0] + 1
+        for name, w in (("W1", W1), ("b1", b1), ("W2", W2), ("b2", b2)):
+            self.register_buffer(name, w)
+        self.n_features = W2.shape[0]
+
+    def forward(self, t, y):
+        h = torch.tanh(torch.cat([y, t[:, None]], 1) @ self.W1.T + self.b1)
+        return h @ self.W2.T + self.b2
+
+    def builtin_params(self):
+        return torch.empty((0, 0), dtype=self.W1.dtype, device=self.W1.device)

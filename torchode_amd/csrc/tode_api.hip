@@ -134,6 +134,10 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (a->batch > (int64_t)2147483647 * 64) return fail(TODE_E_UNSUPPORTED, "batch too large");
     hipStream_t s = (hipStream_t)stream;
     if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (a->term == TODE_TERM_REACTION_DIFFUSION) {
+        if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for float32");
+        return solve_grid_f32(*a, *c, ns, na, ni, st, s);
+    }
     if (g_fast_variant != 1) {
         // small batches: two wavefronts per group of 64 samples (stepper + dense-output evaluator)
         bool used = false;

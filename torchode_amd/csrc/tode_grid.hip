@@ -1,0 +1,296 @@
+// Whole-solve kernel for right-hand sides on a periodic N x N grid (reaction-diffusion,
+// F = N*N state values per sample): one workgroup per sample.
+//
+// Thread t owns the four consecutive cells 4t..4t+3 of the row-major grid and keeps
+// their state (y, the seven stage derivatives, the dense-output coefficients) in
+// registers for the whole solve.  Only the stage input travels through LDS, double
+// buffered, so that the five-point stencil can read its neighbours: one barrier per
+// right-hand side evaluation.  Norms over the row are block reductions in a fixed
+// order (the order of wave_row_norm in tode_ops.hip: per-thread chain over its four
+// values, butterfly over the wavefront, wavefront sums added in order), so that this
+// kernel and the per-call operators produce the same bits.  Every thread of the
+// workgroup carries the same scalar state (t, dt, error ratio, counters), computed
+// redundantly from the same reduced values: there is no divergence inside a sample.
+//
+// The dense output is what this kernel is bound by: every evaluation point is one
+// coalesced 4*F-byte row of ys, written with 16-byte stores straight from registers.
+//
+// Same contract as the fast kernels: the common case only; anything else (a
+// non-success status, max_steps reached, evaluation times that are not monotone in
+// the direction of time, a sample that does not land on t_end) raises
+// TODE_FLAG_NEEDS_GENERAL and leaves the outputs unspecified.
+#include <limits.h>
+
+#include "tode_solve.h"
+
+namespace tode {
+
+struct GridOut {
+    int64_t *n_steps, *n_accepted, *n_initialized, *status;
+};
+
+template <int NW> struct GridShared {
+    float xch[2][NW * 256];  // stage input, double buffered
+    float red[2][NW][2];     // wavefront sums of up to two reductions, double buffered
+};
+
+// Sum over the workgroup of two per-thread partial sums, in the fixed order.
+template <int NW> __device__ __forceinline__ void block_sum2(GridShared<NW> &sh, int &slot, float a, float b, float &A, float &B) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a = a + __shfl_xor(a, off);
+        b = b + __shfl_xor(b, off);
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+        sh.red[slot][wave][0] = a;
+        sh.red[slot][wave][1] = b;
+    }
+    __syncthreads();
+    A = 0;
+    B = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        A = A + sh.red[slot][w][0];
+        B = B + sh.red[slot][w][1];
+    }
+    slot ^= 1;
+}
+
+// du/dt = D * lap(u) + u * (1 - u) on the periodic grid; each operation rounds on its own, in the
+// order of the torch expression  (((up + down) + left) + right) - 4u,  D * lap + u * (1 - u).
+template <int N, int NW>
+__device__ __forceinline__ void grid_rhs(GridShared<NW> &sh, int &buf, float D, const float (&u)[4], float (&out)[4]) {
+    const int t = threadIdx.x;
+    constexpr int PER_ROW = N / 4;
+    const int r = t / PER_ROW, c0 = 4 * (t - r * PER_ROW);
+    float *x = sh.xch[buf];
+    *reinterpret_cast<float4 *>(x + 4 * t) = make_float4(u[0], u[1], u[2], u[3]);
+    __syncthreads();
+    const int ru = (r + N - 1) & (N - 1), rd = (r + 1) & (N - 1);
+    const float4 up = *reinterpret_cast<const float4 *>(x + ru * N + c0);
+    const float4 dn = *reinterpret_cast<const float4 *>(x + rd * N + c0);
+    const float lf = x[r * N + ((c0 + N - 1) & (N - 1))];
+    const float rt = x[r * N + ((c0 + 4) & (N - 1))];
+    const float ups[4] = {up.x, up.y, up.z, up.w}, dns[4] = {dn.x, dn.y, dn.z, dn.w};
+    const float lfs[4] = {lf, u[0], u[1], u[2]}, rts[4] = {u[1], u[2], u[3], rt};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lap = (((ups[j] + dns[j]) + lfs[j]) + rts[j]) - (4.0f * u[j]);
+        const float diff = D * lap;
+        const float react = u[j] * (1.0f - u[j]);
+        out[j] = diff + react;
+    }
+    buf ^= 1;
+}
+
+template <int METHOD, int CTRL, int N>
+__global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<float> p, const GridOut o) {
+    using T = float;
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    constexpr int F = N * N, NT = F / 4, NW = NT / 64;
+    __shared__ GridShared<NW> sh;
+    extern __shared__ __align__(16) unsigned char dyn[];
+    T *te_s = reinterpret_cast<T *>(dyn);  // [E] evaluation times of this sample
+
+    const int tid = threadIdx.x;
+    const long long b = blockIdx.x;
+    const int E = p.n_eval;
+    const CtrlParams<T> &cp = p.cp;
+    const T sf = (T)__builtin_sqrt((double)F);
+    int buf = 0, slot = 0;
+
+    for (int e = tid; e < E; e += NT) te_s[e] = p.t_eval[b * E + e];
+    const T ts = p.t_start[b * p.ts_stride], te = p.t_end[b * p.te_stride];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const T tlo = tmin(ts, te), thi = tmax(te, ts);
+    const T D = p.params[b];
+    T y[4], k[7][4];
+    {
+        const float4 v = *reinterpret_cast<const float4 *>(p.y0 + b * F + 4 * tid);
+        y[0] = v.x, y[1] = v.y, y[2] = v.z, y[3] = v.w;
+    }
+    __syncthreads();  // te_s
+
+    bool bail = false;
+    for (int e = 1; e < E; ++e) bail = bail || !(dir * te_s[e] >= dir * te_s[e - 1]);  // not monotone
+
+    // ---- first step size (step_size_controllers.py:431-490, 776-835) ----
+    T t = ts, dt;
+    grid_rhs<N, NW>(sh, buf, D, y, k[0]);
+    if (p.dt0) {
+        dt = p.dt0[b];
+    } else {
+        T inv[4], a0 = 0, a1 = 0, A0, A1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            inv[j] = inv_scale(cp.atol, cp.rtol, y[j]);
+            const T x0 = (y[j] * inv[j]) / sf, x1 = (k[0][j] * inv[j]) / sf;
+            a0 = fma_(x0, x0, a0);
+            a1 = fma_(x1, x1, a1);
+        }
+        block_sum2<NW>(sh, slot, a0, a1, A0, A1);
+        const T d0 = sqrt_(A0), d1 = sqrt_(A1);
+        T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
+        h0 = tmin(h0, abs_(te - ts));
+        T y1[4], f1[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) y1[j] = fma_(dir * h0, k[0][j], y[j]);
+        grid_rhs<N, NW>(sh, buf, D, y1, f1);
+        T a2 = 0, A2, unused;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const T df = f1[j] - k[0][j];
+            const T x2 = (df * inv[j]) / sf;
+            a2 = fma_(x2, x2, a2);
+        }
+        block_sum2<NW>(sh, slot, a2, (T)0, A2, unused);
+        dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, h0, d1, sqrt_(A2));
+    }
+    dt = tclamp(dt, tlo - t, thi - t);
+
+    int cursor = 0, n_steps = 0, n_acc = 0;
+    if (E > 0 && te_s[0] == ts) {
+        *reinterpret_cast<float4 *>(p.ys + (b * E) * F + 4 * tid) = make_float4(y[0], y[1], y[2], y[3]);
+        cursor = 1;
+    }
+    T prev = 1, pprev = 1;
+
+    while (!bail) {
+        // ---- stages (runge_kutta.py:255-263) ----
+        const T t0 = t;
+        T y1[4];
+#pragma unroll
+        for (int i = 1; i < 7; ++i) {
+            T yi[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                T s = 0;
+#pragma unroll
+                for (int jj = 0; jj < i; ++jj) s = fma_((T)Tab::a[i][jj], k[jj][j], s);
+                yi[j] = fma_(dt, s, y[j]);
+            }
+            grid_rhs<N, NW>(sh, buf, D, yi, k[i]);
+            if (i == 6) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) y1[j] = yi[j];
+            }
+        }
+
+        // ---- error ratio (runge_kutta.py:267, step_size_controllers.py:389-395); long rows: fused sums ----
+        T part = 0, total, unused;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            T err = 0;
+#pragma unroll
+            for (int s = 0; s < 7; ++s) err = fma_(dt * (T)Tab::b_err[s], k[s][j], err);
+            const T m = tmax(abs_(y[j]), abs_(y1[j]));
+            const T x = (abs_(err) / fma_(cp.rtol, m, cp.atol)) / sf;
+            part = fma_(x, x, part);
+        }
+        block_sum2<NW>(sh, slot, part, (T)0, total, unused);
+        const T ratio = tmax(sqrt_(total), (T)1e-38);
+        const bool accept = ratio < (T)1;
+        T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
+        const int status = limit_dt<T>(cp, ratio, dt_next);
+
+        const T t_new = accept ? (t0 + dt) : t0;
+        const bool running_new = fma_(dir, t_new, -dir * te) < (T)0;
+        n_steps += 1;
+        n_acc += accept ? 1 : 0;
+
+        // ---- dense output at the evaluation points this step passed (adjoints.py:215-234) ----
+        if (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0) {
+            T q[4][5][1];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                T ks[7];
+#pragma unroll
+                for (int s = 0; s < 7; ++s) ks[s] = k[s][j];
+                quartic_elem<T, METHOD>(dt, y[j], y1[j], ks, true, q[j]);
+            }
+            const T t1 = t0 + dt;
+            do {
+                const T x = unit_time(te_s[cursor], t0, t1);
+                T out[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    T v = q[j][4][0];
+#pragma unroll
+                    for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
+                    out[j] = v;
+                }
+                *reinterpret_cast<float4 *>(p.ys + (b * E + cursor) * F + 4 * tid) = make_float4(out[0], out[1], out[2], out[3]);
+                ++cursor;
+            } while (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0);
+        }
+
+        // ---- state update (adjoints.py:150-155, 247-255) ----
+        if (accept) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                y[j] = y1[j];
+                k[0][j] = k[6][j];
+            }
+        }
+        t = t_new;
+        dt = tclamp(running_new ? dt_next : dt, tlo - t, thi - t);
+        if (CTRL == 1 && running_new && accept) {
+            pprev = prev;
+            prev = ratio;
+        }
+        if (status != 0 || n_steps >= p.max_steps || n_steps >= TODE_HARD_STEP_LIMIT) {
+            bail = true;
+            break;
+        }
+        if (!running_new) {
+            // a sample that does not land on t_end, or ends on a non-finite value, shows up in later
+            // iterations of the reference loop: not the common case
+            int odd = !(t == te);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) odd |= !finite_(y[j]) || !finite_(k[0][j]);
+            if (__syncthreads_or(odd)) bail = true;
+            break;
+        }
+    }
+
+    if (tid == 0) {
+        o.n_steps[b] = n_steps;
+        o.n_accepted[b] = n_acc;
+        o.n_initialized[b] = cursor;
+        o.status[b] = 0;
+        if (n_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], n_steps);
+        if (bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
+    }
+}
+
+template <int METHOD, int CTRL, int N> static int launch_grid(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t stream) {
+    SolveParams<float> p = make_params<float>(a, c);
+    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
+    const size_t lds = (size_t)a.n_eval * sizeof(float);
+    timing_before(stream, "tode::solve_grid_kernel");
+    hipLaunchKernelGGL((solve_grid_kernel<METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4), lds, stream, p, o);
+    timing_after(stream);
+    return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
+}
+
+template <int N> static int grid_mc(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t s) {
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<0, 0, N>(a, c, o, s);
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch_grid<0, 1, N>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<1, 0, N>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch_grid<1, 1, N>(a, c, o, s);
+    return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
+}
+
+int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+    if (a.n_params != 1) return fail(TODE_E_INVALID, "reaction-diffusion needs one parameter (the diffusivity) per sample");
+    if (a.n_eval > 8192) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the grid kernel", a.n_eval);
+    if (a.batch > INT_MAX) return fail(TODE_E_UNSUPPORTED, "batch too large");
+    GridOut o{ns, na, ni, st};
+    if (a.n_features == 64 * 64) return grid_mc<64>(a, c, o, s);
+    if (a.n_features == 32 * 32) return grid_mc<32>(a, c, o, s);
+    return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 32 x 32 and 64 x 64 grids, got F=%d", a.n_features);
+}
+
+}  // namespace tode

@@ -95,27 +95,37 @@ template <typename T, int NORM> struct RowNorm {
     __device__ __forceinline__ T get() const { return NORM == TODE_NORM_MAX ? acc : sqrt_(acc); }
 };
 
-// One wavefront reduces one row (F >= 64): lanes walk the row with stride 64, partial
-// results are combined with a butterfly.
+// One wavefront reduces one row (F >= 64).  The order of summation is fixed, so that every kernel
+// that forms such a norm gets the same bits: the row is cut into chunks of 256 values; within a
+// chunk lane l accumulates values 4l..4l+3 in order (fused multiply-add from zero), the 64 partial
+// sums are combined by a butterfly (xor 32, 16, .., 1), and the chunk sums are added in order.
 template <typename T, int NORM, typename Load> __device__ __forceinline__ T wave_row_norm(int F, Load load) {
     const int lane = threadIdx.x & 63;
     const T sf = (T)__builtin_sqrt((double)F);
-    T acc = 0;
-    for (int f = lane; f < F; f += 64) {
-        const T v = load(f);
-        if (NORM == TODE_NORM_MAX)
-            acc = tmax(acc, abs_(v));
-        else {
-            const T x = v / sf;
-            acc = fma_(x, x, acc);
-        }
-    }
+    T total = 0;
+    for (int base = 0; base < F; base += 256) {
+        T p = 0;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const T o = __shfl_xor(acc, off);
-        acc = NORM == TODE_NORM_MAX ? tmax(acc, o) : acc + o;
+        for (int j = 0; j < 4; ++j) {
+            const int f = base + 4 * lane + j;
+            if (f < F) {
+                const T v = load(f);
+                if (NORM == TODE_NORM_MAX)
+                    p = tmax(p, abs_(v));
+                else {
+                    const T x = v / sf;
+                    p = fma_(x, x, p);
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const T o = __shfl_xor(p, off);
+            p = NORM == TODE_NORM_MAX ? tmax(p, o) : p + o;
+        }
+        total = NORM == TODE_NORM_MAX ? tmax(total, p) : total + p;
     }
-    return NORM == TODE_NORM_MAX ? acc : sqrt_(acc);
+    return NORM == TODE_NORM_MAX ? total : sqrt_(total);
 }
 
 template <typename T, int NORM> __global__ void __launch_bounds__(256) row_norm_thread_kernel(long long batch, int F, const T *x, T *out) {
@@ -189,8 +199,6 @@ __global__ void __launch_bounds__(256) adapt_wave_kernel(CtrlParams<T> cp, long 
 // start step (step_size_controllers.py:431-490, 776-835)
 // ------------------------------------------------------------------------------------------
 
-template <typename T> __device__ __forceinline__ T inv_scale(T atol, T rtol, T y0) { return (T)1 / fma_(rtol, abs_(y0), atol); }
-
 template <typename T, int NORM>
 __global__ void __launch_bounds__(256) initial_a_thread_kernel(long long batch, int F, T atol, T rtol, const T *t_start, const T *t_end, const T *y0,
                                                                const T *f0, T *h0_out) {
@@ -232,20 +240,6 @@ __global__ void __launch_bounds__(256) initial_probe_kernel(long long batch, int
     const T h = h0[b];
     y1[i] = fma_(dir * h, f0[i], y0[i]);
     if (i - b * F == 0) t1[b] = fma_(dir, h, t_start[b]);
-}
-
-template <typename T> __device__ __forceinline__ T initial_finish(int kind, double inv_order, T dir, T h0, T d1, T d2n) {
-    T d2 = d2n / h0;
-    if (kind == TODE_CTRL_INTEGRAL && h0 == (T)0) d2 = (T)__builtin_huge_val();
-    const T m = tmax(d1, d2);
-    T h1;
-    if (m <= (T)1e-15) {
-        h1 = tmax((T)1e-6, h0 * (T)1e-3);
-    } else {
-        const T rm = (T)1 / m;  // python_float / tensor runs as reciprocal(tensor) * python_float
-        h1 = rpow<T>(rm * (T)0.01, inv_order);
-    }
-    return dir * tmin((T)100 * h0, h1);
 }
 
 template <typename T, int NORM>
@@ -343,19 +337,6 @@ __global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F
     coeff[bf + i] = h * f0;
     coeff[2 * bf + i] = b;
     coeff[3 * bf + i] = a;
-}
-
-// x = (t - t0) / (t1 - t0) with a zero interval mapped to 1 (interpolation.py:8-40)
-template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) {
-    T den = t1 - t0;
-    if (!(abs_(den) > (T)0)) den = (T)1;
-    return (t - t0) / den;
-}
-
-template <typename T> __device__ __forceinline__ T horner(const T *coeff, long long bf, long long at, int degree, T x) {
-    T y = coeff[degree * bf + at];
-    for (int p = degree - 1; p >= 0; --p) y = fma_(y, x, coeff[p * bf + at]);
-    return y;
 }
 
 template <typename T>

@@ -127,6 +127,37 @@ __device__ __forceinline__ T initial_step(const CtrlParams<T> &cp, const Term &r
 }
 
 
+// Pieces of the start step and of the dense output shared by the per-call operators and the
+// whole-solve kernels for long rows.
+template <typename T> __device__ __forceinline__ T inv_scale(T atol, T rtol, T y0) { return (T)1 / fma_(rtol, abs_(y0), atol); }
+
+template <typename T> __device__ __forceinline__ T initial_finish(int kind, double inv_order, T dir, T h0, T d1, T d2n) {
+    T d2 = d2n / h0;
+    if (kind == TODE_CTRL_INTEGRAL && h0 == (T)0) d2 = (T)__builtin_huge_val();
+    const T m = tmax(d1, d2);
+    T h1;
+    if (m <= (T)1e-15) {
+        h1 = tmax((T)1e-6, h0 * (T)1e-3);
+    } else {
+        const T rm = (T)1 / m;  // python_float / tensor runs as reciprocal(tensor) * python_float
+        h1 = rpow<T>(rm * (T)0.01, inv_order);
+    }
+    return dir * tmin((T)100 * h0, h1);
+}
+
+// x = (t - t0) / (t1 - t0) with a zero interval mapped to 1 (interpolation.py:8-40)
+template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) {
+    T den = t1 - t0;
+    if (!(abs_(den) > (T)0)) den = (T)1;
+    return (t - t0) / den;
+}
+
+template <typename T> __device__ __forceinline__ T horner(const T *coeff, long long bf, long long at, int degree, T x) {
+    T y = coeff[degree * bf + at];
+    for (int p = degree - 1; p >= 0; --p) y = fma_(y, x, coeff[p * bf + at]);
+    return y;
+}
+
 // Controller parameters in the working type from the ABI struct.
 template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c, double order = 5.0) {
     CtrlParams<T> cp;

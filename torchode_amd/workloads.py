@@ -42,6 +42,23 @@ def _log_uniform(g, a, b, shape):
     return torch.tensor(vals, dtype=torch.float64).reshape(shape)
 
 
+def _blur_periodic(u, sigma: float, radius: int):
+    """One separable Gaussian blur with periodic boundaries over the last two dims, float64,
+    kernel normalised to one (weights through mpmath, for the same reason as above)."""
+    import mpmath
+
+    with mpmath.workprec(100):
+        w = [float(mpmath.exp(-mpmath.mpf(i * i) / (2 * sigma * sigma))) for i in range(-radius, radius + 1)]
+    total = math.fsum(w)
+    w = [x / total for x in w]
+    for dim in (1, 2):
+        acc = torch.zeros_like(u)
+        for i, wi in zip(range(-radius, radius + 1), w):
+            acc = acc + wi * torch.roll(u, i, dim)
+        u = acc
+    return u
+
+
 def _t_eval(t0, t1, E):
     frac = torch.arange(E, dtype=torch.float64) / (E - 1)
     return t0[:, None] + (t1 - t0)[:, None] * frac[None, :]
@@ -58,7 +75,7 @@ def _algorithmic_bytes(F, P, C, E, itemsize):
 
 
 def make(name: str, *, batch: Optional[int] = None, dtype=None, device="cpu") -> Workload:
-    """Build workload ``name`` in {"linear_decay", "vdp", "lorenz"}.
+    """Build workload ``name`` in {"linear_decay", "vdp", "lorenz", "reaction_diffusion", "mlp"}.
 
     ``batch`` draws the full-size tensors and keeps the first ``batch`` samples
     (samples are independent, so a prefix is a valid smaller instance of the same
@@ -92,6 +109,34 @@ def make(name: str, *, batch: Optional[int] = None, dtype=None, device="cpu") ->
         t_eval = _t_eval(torch.zeros(B, dtype=torch.float64), torch.full((B,), 2.0, dtype=torch.float64), E)
         params, cls = rho, bt.Lorenz63
         method, ctrl, P, C = "dopri5", dict(kind="integral", atol=1e-5, rtol=1e-3), 1, 0
+    elif name == "reaction_diffusion":
+        B, n, E, seed = 512, 64, 100, 105
+        F = n * n
+        dtype = dtype or torch.float32
+        g = torch.Generator("cpu").manual_seed(seed)
+        D = _log_uniform(g, 1e-3, 1e-1, (B,))
+        u0 = _blur_periodic(_uniform(g, 0.0, 1.0, (B, n, n)), sigma=2.0, radius=6)
+        y0 = u0.reshape(B, F)
+        t_eval = _t_eval(torch.zeros(B, dtype=torch.float64), torch.ones(B, dtype=torch.float64), E)
+        params, cls = D, bt.ReactionDiffusion
+        method = "tsit5"
+        ctrl, P, C = dict(kind="pid", atol=1e-5, rtol=1e-3, pcoeff=0.2, icoeff=0.5, dcoeff=0.0), 1, 2
+    elif name == "mlp":
+        B, F, H, E, seed = 4096, 64, 256, 20, 104
+        dtype = dtype or torch.float32
+        g = torch.Generator("cpu").manual_seed(seed)
+        b1, b2 = math.sqrt(6.0 / (F + 1 + H)), math.sqrt(6.0 / (H + F))
+        W1 = _uniform(g, -b1, b1, (H, F + 1))
+        W2 = _uniform(g, -b2, b2, (F, H))
+        y0 = torch.randn((B, F), generator=g, dtype=torch.float64)
+        t_eval = _t_eval(torch.zeros(B, dtype=torch.float64), torch.ones(B, dtype=torch.float64), E)
+        method, ctrl, P, C = "dopri5", dict(kind="integral", atol=1e-5, rtol=1e-3), 0, 0
+        n = B if batch is None else int(batch)
+        assert 0 < n <= B
+        w = lambda x: x.to(dtype).contiguous().to(device)
+        f = bt.MLPField(w(W1), w(torch.zeros(H, dtype=torch.float64)), w(W2), w(torch.zeros(F, dtype=torch.float64)))
+        step, dense = _algorithmic_bytes(F, P, C, E, torch.empty((), dtype=dtype).element_size())
+        return Workload(name, f, w(y0[:n]), w(t_eval[:n]), method, ctrl, step, dense)
     else:
         raise ValueError(f"unknown workload {name!r}")
 
