@@ -33,6 +33,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("vdp", "torch.float32", 65536): 47.39e6,
     # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (77468.9 KiB x 2.000 + 895940 KiB x 1.000) x 1024
     ("lorenz", "torch.float32", 1048576): 1076.1e6,
+    # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4363 KiB x 2.000 + 819284 KiB x 1.000) x 1024
+    ("reaction_diffusion", "torch.float32", 512): 847.9e6,
 }
 
 

@@ -143,3 +143,26 @@ def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():
     sol = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-6, 1e-4)).solve(to.InitialValueProblem(y0, t_eval[:, 0], t_eval[:, -1], t_bad), to.ODETerm(f))
     ref = to.AutoDiffAdjoint(OwnTsit5(), to.IntegralController(1e-6, 1e-4)).solve(to.InitialValueProblem(y0, t_eval[:, 0], t_eval[:, -1], t_bad), to.ODETerm(f))
     assert_same(sol, ref)
+
+
+@pytest.mark.parametrize("name,batch", [("reaction_diffusion", 16), ("mlp", 128)])
+def test_against_the_committed_vectors(name, batch):
+    """tests/golden/*_tolerance.json: ATen-op oracle results written in the authoring container."""
+    import hashlib
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(__file__), "golden", f"{name}_float32_b{batch}_tolerance.json")
+    gold = json.load(open(path))
+    w = to.workloads.make(name, batch=batch)
+    digest = lambda t: hashlib.sha256(t.contiguous().numpy().tobytes()).hexdigest()
+    assert digest(w.y0) == gold["inputs_sha256"]["y0"] and digest(w.t_eval) == gold["inputs_sha256"]["t_eval"]
+    sol = device_solve(w)
+    assert sol.status.tolist() == gold["status"] and sol.stats["n_f_evals"].tolist() == [gold["n_f_evals"]] * batch
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        differ = sum(a != b for a, b in zip(sol.stats[key].tolist(), gold[key]))
+        assert differ <= 0.001 * batch, f"{key}: {differ} of {batch} samples differ"
+    pts = torch.tensor(gold["ys_points"])
+    want = torch.tensor([float.fromhex(v) for v in gold["ys_values"]], dtype=torch.float64)
+    got = sol.ys.cpu()[pts[:, 0], pts[:, 1], pts[:, 2]].double()
+    assert mixed_error(got, want) < 1e-4
