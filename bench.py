@@ -26,6 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
 MEASURED_TRAFFIC_BYTES = {
@@ -111,6 +112,39 @@ def main():
         kernel_name, kernel_s = "protocol path (one kernel per protocol call + torch right-hand side)", wall
     _lib.set_kernel_timing(False)
     achieved = algo_bytes / kernel_s / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": kernel_name,
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBPS,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
+        "algorithmic_bytes_per_launch": algo_bytes,
+        "bytes_per_sample_step": w.bytes_step,
+        "bytes_dense_per_sample": w.bytes_dense,
+        "kernel_ms": kernel_s * 1e3,
+    }
+    if w.name == "mlp":
+        # dense contractions: the matrix cores bound this workload, not HBM.  Per evaluation of f and
+        # sample 2*(65*256 + 256*64) flops; a sample evaluates f twice for the first step size and six
+        # times per step; about 5000 flops per step for the Runge-Kutta sums, error norm and control.
+        H, Fin = w.f.W1.shape
+        flops_f = 2 * (Fin * H + H * F)
+        flops = (2 * B + 6 * sample_steps) * flops_f + 5000 * sample_steps
+        tflops = flops / kernel_s / 1e12
+        roofline = {
+            "bound": "mfma",
+            "kernel": kernel_name,
+            "achieved": tflops,
+            "peak": MFMA_FP32_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
+            "algorithmic_flops_per_launch": flops,
+            "flops_per_rhs_evaluation_per_sample": flops_f,
+            "kernel_ms": kernel_s * 1e3,
+        }
 
     out = {
         "metric": "RK sample-steps/s (adaptive Tsit5/Dopri5 solve, whole batch)",
@@ -133,19 +167,7 @@ def main():
         },
         "ivps_per_s": B / wall,
         "equiv_hbm_gbps": algo_bytes / wall / 1e9,
-        "roofline": {
-            "bound": "hbm",
-            "kernel": kernel_name,
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
-            "algorithmic_bytes_per_launch": algo_bytes,
-            "bytes_per_sample_step": w.bytes_step,
-            "bytes_dense_per_sample": w.bytes_dense,
-            "kernel_ms": kernel_s * 1e3,
-        },
+        "roofline": roofline,
     }
 
     if not args.no_cpu_baseline:

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 3
+#define TODE_ABI_VERSION 4
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -35,8 +35,10 @@ enum {
     TODE_TERM_LINEAR_DECAY = 0,       /* dy/dt = -k y, k [B,F] */
     TODE_TERM_VAN_DER_POL = 1,        /* F = 2, mu [B] */
     TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
-    TODE_TERM_REACTION_DIFFUSION = 3  /* F = N*N periodic grid (N = 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
+    TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
                                          float32, tode_solve_builtin_fast only */
+    TODE_TERM_MLP = 4                 /* F = 64: tanh([y, t] W1^T + b1) W2^T + b2 with 256 hidden units, weights in
+                                         shared_params; float32, tode_solve_builtin_fast only */
 };
 /* per-sample status codes: reference status_codes.py:9-13 */
 enum {
@@ -127,6 +129,8 @@ typedef struct tode_solve_args {
     const void *t_eval;        /* [B,E] or NULL when E == 0 */
     const void *dt0;           /* [B] user initial step, or NULL to select one */
     const void *params;        /* [B,P] */
+    const void *shared_params; /* [n_shared_params] right-hand side parameters shared by the batch, or NULL */
+    int64_t n_shared_params;   /* TODE_TERM_MLP: W1 [256,65] | b1 [256] | W2 [64,256] | b2 [64], row-major, concatenated */
     void *ys;                  /* out [B,max(E,1),F] */
     void *y_idle;              /* out [B,F], used only when E == 0: value the reference
                                   reports for a sample that finished before iteration L */

@@ -27,15 +27,17 @@ def device_solve(w):
 
 
 def compare(sol, ref, min_agree):
+    """integer stats equal and ys within 1e-4 (mixed absolute / relative) on at least `min_agree` of the samples"""
     assert sol.status.tolist() == ref["status"].tolist()
     B = sol.ys.shape[0]
+    ys, rys = sol.ys.cpu().double(), ref["ys"].double()
+    d = (ys - rys).abs()
+    good = torch.minimum(d, d / rys.abs().clamp_min(1e-300)).flatten(1).amax(dim=1) < 1e-4
     for key in ("n_steps", "n_accepted", "n_initialized"):
-        differ = int((sol.stats[key].cpu() != ref[key]).sum())
-        print(f"{key}: {differ} of {B} samples differ")
-        assert differ <= (1 - min_agree) * B, key
-    err = mixed_error(sol.ys.cpu().double(), ref["ys"].double())
-    print(f"ys mixed error {err:.3e}")
-    assert err < 1e-4
+        good &= sol.stats[key].cpu() == ref[key]
+    print(f"{int((~good).sum())} of {B} samples differ in stats or by more than 1e-4")
+    assert int((~good).sum()) <= (1 - min_agree) * B
+    assert mixed_error(ys, rys) < 1e-2
 
 
 def test_reaction_diffusion_against_the_aten_oracle():
@@ -166,3 +168,68 @@ def test_against_the_committed_vectors(name, batch):
     want = torch.tensor([float.fromhex(v) for v in gold["ys_values"]], dtype=torch.float64)
     got = sol.ys.cpu()[pts[:, 0], pts[:, 1], pts[:, 2]].double()
     assert mixed_error(got, want) < 1e-4
+
+
+# ---------------------------------------------------------------------------------------------
+# the whole-solve MLP kernel (matrix cores) against the protocol path (torch matrix products)
+# ---------------------------------------------------------------------------------------------
+
+
+def mlp_both_paths(w, method, ctrl, **kw):
+    from torchode_amd import _lib
+
+    lib_m, own_m = {"tsit5": (to.Tsit5, OwnTsit5), "dopri5": (to.Dopri5, OwnDopri5)}[method]
+    problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
+    fused = to.AutoDiffAdjoint(lib_m(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f), **kw)
+    assert _lib.last_solve_kernel_name() == "tode::solve_mlp_kernel"
+    return fused, to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f), **kw)
+
+
+def per_sample_error(a, b):
+    """max over a sample's values of min(abs error, rel error)"""
+    d = (a - b).abs()
+    return torch.minimum(d, d / b.abs().clamp_min(1e-300)).flatten(1).amax(dim=1)
+
+
+def assert_close_solutions(a, b, min_agree=0.98, loose=1e-2):
+    """Two float32 pipelines whose matrix products round differently.  The first step of a solve is
+    tiny, its error estimate (a sum that cancels to ~1e-9) lies below the ~1e-7 rounding noise of a
+    256-term float32 dot product, and the next step size is 0.9 * ratio**-0.2 of that noise: a few
+    samples take visibly different (equally valid) steps and then differ by the solver's own
+    truncation error.  Asked for: integer stats equal and ys within 1e-4 on at least `min_agree` of
+    the samples, every sample within `loose`."""
+    B = a.ys.shape[0]
+    assert torch.equal(a.status, b.status)
+    good = per_sample_error(a.ys.double(), b.ys.double()) < 1e-4
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        good &= a.stats[key] == b.stats[key]
+    print(f"{int((~good).sum())} of {B} samples took other steps")
+    assert int((~good).sum()) <= (1 - min_agree) * B
+    assert mixed_error(a.ys.double().cpu(), b.ys.double().cpu()) < loose
+
+
+@pytest.mark.parametrize("batch", [256, 250, 7])
+def test_mlp_kernel_on_the_benchmark_workload(batch):
+    w = to.workloads.make("mlp", batch=batch, device="cuda")
+    fused, proto = mlp_both_paths(w, w.method, w.controller)
+    assert fused.ys.shape == (batch, 20, 64) and (fused.stats["n_initialized"] == 20).all()
+    assert fused.stats["n_f_evals"].tolist() == proto.stats["n_f_evals"].tolist()
+    assert_close_solutions(fused, proto)
+
+
+@pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "pid"), ("tsit5", "integral")])
+def test_mlp_kernel_with_tight_tolerances(method, kind):
+    """At rtol 1e-6 every error estimate sits at the rounding noise of the float32 matrix products, so
+    the two pipelines accept and reject differently; both then solve the problem to the tolerance, and
+    that is what is compared: the solutions, and the amount of work."""
+    w = to.workloads.make("mlp", batch=96, device="cuda")
+    ctrl = dict(kind=kind, atol=1e-7, rtol=1e-6)
+    if kind == "pid":
+        ctrl.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    for kw in ({}, {"dt0": torch.full((96,), 0.05, device="cuda")}):
+        fused, proto = mlp_both_paths(w, method, ctrl, **kw)
+        assert (fused.stats["n_steps"] >= 4).all() and torch.equal(fused.status, proto.status)
+        assert (fused.stats["n_initialized"] == 20).all()
+        assert mixed_error(fused.ys.double().cpu(), proto.ys.double().cpu()) < 2e-5
+        work = fused.stats["n_steps"].sum().item() / proto.stats["n_steps"].sum().item()
+        assert 0.8 < work < 1.25, work

@@ -13,11 +13,12 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
-PERSISTENT_TERMS = (0, 1, 2, 3)  # TODE_TERM_* that a whole-solve kernel evaluates itself
+TERM_REACTION_DIFFUSION, TERM_MLP = 3, 4
+PERSISTENT_TERMS = (0, 1, 2, 3, 4)  # TODE_TERM_* that a whole-solve kernel evaluates itself
 GENERAL_TERMS = (0, 1, 2)  # ... of which these also have the general kernel (every case, not only the common one)
 FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_NEEDS_GENERAL, FLAG_WORDS = 0, 1, 2, 3, 4
 INT32_MAX = 2**31 - 1
@@ -107,6 +108,8 @@ class SolveArgs(C.Structure):
         ("t_eval", C.c_void_p),
         ("dt0", C.c_void_p),
         ("params", C.c_void_p),
+        ("shared_params", C.c_void_p),
+        ("n_shared_params", C.c_int64),
         ("ys", C.c_void_p),
         ("y_idle", C.c_void_p),
         ("pending", C.c_void_p),

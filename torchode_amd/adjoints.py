@@ -321,7 +321,10 @@ class AutoDiffAdjoint(nn.Module):
         t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
         t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
         params = f.builtin_params().to(device=dev, dtype=dtype)
+        if params.numel() == 0:
+            params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
+        shared = f.builtin_shared().to(device=dev, dtype=dtype) if hasattr(f, "builtin_shared") else None
         dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
@@ -341,7 +344,9 @@ class AutoDiffAdjoint(nn.Module):
         a.t_start_stride, a.t_end_stride = t_start.stride(0), t_end.stride(0)
         a.t_eval = None if t_eval is None else t_eval.data_ptr()
         a.dt0 = None if dt0_ is None else dt0_.data_ptr()
-        a.params = params.data_ptr()
+        a.params = params.data_ptr() if params.numel() else None
+        a.shared_params = None if shared is None else shared.data_ptr()
+        a.n_shared_params = 0 if shared is None else shared.numel()
         a.ys = ys.data_ptr()
         a.y_idle = None if y_idle is None else y_idle.data_ptr()
         a.pending = None
@@ -358,7 +363,11 @@ class AutoDiffAdjoint(nn.Module):
         if has_general:
             fast_ok = fast_ok and self.use_fast_path and E * y0.element_size() <= 1024
         else:
-            fast_ok = fast_ok and dtype == torch.float32 and F in (32 * 32, 64 * 64) and E <= 8192
+            fast_ok = fast_ok and dtype == torch.float32
+            if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
+                fast_ok = fast_ok and F in (32 * 32, 64 * 64) and E <= 8192
+            else:
+                fast_ok = fast_ok and F == 64 and tuple(f.W1.shape) == (256, 65) and E <= 512
             if not fast_ok:
                 return None  # no whole-solve kernel for this case: the caller takes the protocol path
         if fast_ok:

@@ -44,6 +44,7 @@ UNITS = [
     ("tode_stepwise.hip", "tode_stepwise.o", []),
     ("tode_ops.hip", "tode_ops.o", []),
     ("tode_grid.hip", "tode_grid.o", []),
+    ("tode_mlp.hip", "tode_mlp.o", []),
 ]
 
 

@@ -136,3 +136,7 @@ class MLPField(BuiltinTerm):
 
     def builtin_params(self):
         return torch.empty((0, 0), dtype=self.W1.dtype, device=self.W1.device)
+
+    def builtin_shared(self) -> torch.Tensor:
+        """W1 | b1 | W2 | b2, row-major and concatenated: the layout the whole-solve kernel reads."""
+        return torch.cat([self.W1.reshape(-1), self.b1.reshape(-1), self.W2.reshape(-1), self.b2.reshape(-1)]).contiguous()

@@ -138,6 +138,10 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for float32");
         return solve_grid_f32(*a, *c, ns, na, ni, st, s);
     }
+    if (a->term == TODE_TERM_MLP) {
+        if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the MLP kernel is built for float32");
+        return solve_mlp_f32(*a, *c, ns, na, ni, st, s);
+    }
     if (g_fast_variant != 1) {
         // small batches: two wavefronts per group of 64 samples (stepper + dense-output evaluator)
         bool used = false;
