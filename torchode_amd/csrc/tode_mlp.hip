@@ -33,10 +33,12 @@ struct MlpOut {
 };
 
 constexpr int MLP_F = 64, MLP_H = 256, MLP_K1 = 68;  // 65 inputs padded to a multiple of 4
-constexpr int MLP_XS = 69, MLP_HS = 261;             // LDS row strides of the two A operands
+// LDS rows of the two A operands, stored so that what a lane feeds to the matrix cores is contiguous:
+// lane (q, c) needs row c, columns 4 kk + q for all kk; column k sits at (k % 4) * (K / 4) + k / 4.
+constexpr int MLP_XS = 4 * 17 + 4, MLP_HS = 4 * 64 + 4;  // row strides (floats), multiples of 4 for 16-byte reads
 constexpr int MLP_TILE = 16;
 
-struct MlpShared {
+struct __align__(16) MlpShared {
     float x[MLP_TILE * MLP_XS];
     float hid[MLP_TILE * MLP_HS];
     float red[2][4][MLP_TILE][2];  // per-wavefront partial sums of up to two per-sample reductions
@@ -60,36 +62,55 @@ __device__ __forceinline__ float mlp_tanh(float x) {
 // out[r] = f(tn[r], yi[r]) for the lane's four (sample, feature) pairs.
 __device__ __forceinline__ void mlp_rhs(MlpShared &sh, const MlpWeights &W, const float (&tn)[4], const float (&yi)[4], float (&out)[4]) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, q = lane >> 4, c = lane & 15;
+    {
+        const int k = 16 * w + c;  // this lane's feature is input column k
 #pragma unroll
-    for (int r = 0; r < 4; ++r) sh.x[(4 * q + r) * MLP_XS + 16 * w + c] = yi[r];
-    if (w == 0 && c == 0) {
+        for (int r = 0; r < 4; ++r) sh.x[(4 * q + r) * MLP_XS + (k & 3) * 17 + (k >> 2)] = yi[r];
+        if (w == 0 && c == 0) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sh.x[(4 * q + r) * MLP_XS + MLP_F] = tn[r];
+            for (int r = 0; r < 4; ++r) sh.x[(4 * q + r) * MLP_XS + (MLP_F & 3) * 17 + (MLP_F >> 2)] = tn[r];
+        }
     }
     __syncthreads();
+    // all A operands of the layer into registers first, so that the matrix cores never wait for LDS
+    float a1[20];
+    {
+        const float *row = sh.x + c * MLP_XS + q * 17;  // 17 contiguous values (read as 20)
+#pragma unroll
+        for (int j = 0; j < 20; ++j) a1[j] = row[j];
+    }
+    asm volatile("" ::: "memory");
     mfma_acc acc1[4];
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) acc1[tile] = {W.b1[tile], W.b1[tile], W.b1[tile], W.b1[tile]};
 #pragma unroll
     for (int kk = 0; kk < 17; ++kk) {
-        const float a = sh.x[c * MLP_XS + 4 * kk + q];
 #pragma unroll
-        for (int tile = 0; tile < 4; ++tile) acc1[tile] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, W.w1[kk][tile], acc1[tile], 0, 0, 0);
+        for (int tile = 0; tile < 4; ++tile) acc1[tile] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[kk], W.w1[kk][tile], acc1[tile], 0, 0, 0);
     }
 #pragma unroll
-    for (int tile = 0; tile < 4; ++tile)
+    for (int tile = 0; tile < 4; ++tile) {
+        const int h = 64 * w + 16 * tile + c;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sh.hid[(4 * q + r) * MLP_HS + 64 * w + 16 * tile + c] = mlp_tanh(acc1[tile][r]);
+        for (int r = 0; r < 4; ++r) sh.hid[(4 * q + r) * MLP_HS + (h & 3) * 64 + (h >> 2)] = mlp_tanh(acc1[tile][r]);
+    }
     __syncthreads();
+    float a2[64];
+    {
+        const float4 *row = reinterpret_cast<const float4 *>(sh.hid + c * MLP_HS + q * 64);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float4 v = row[j];
+            a2[4 * j] = v.x, a2[4 * j + 1] = v.y, a2[4 * j + 2] = v.z, a2[4 * j + 3] = v.w;
+        }
+    }
+    asm volatile("" ::: "memory");
     mfma_acc acc2[4];
     acc2[0] = {W.b2, W.b2, W.b2, W.b2};
 #pragma unroll
     for (int i = 1; i < 4; ++i) acc2[i] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int kk = 0; kk < 64; ++kk) {
-        const float a = sh.hid[c * MLP_HS + 4 * kk + q];
-        acc2[kk & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, W.w2[kk], acc2[kk & 3], 0, 0, 0);
-    }
+    for (int kk = 0; kk < 64; ++kk) acc2[kk & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a2[kk], W.w2[kk], acc2[kk & 3], 0, 0, 0);
 #pragma unroll
     for (int r = 0; r < 4; ++r) out[r] = (acc2[0][r] + acc2[1][r]) + (acc2[2][r] + acc2[3][r]);
 }
