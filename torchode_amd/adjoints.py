@@ -321,7 +321,7 @@ class AutoDiffAdjoint(nn.Module):
         t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
         t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
         params = f.builtin_params().to(device=dev, dtype=dtype)
-        if params.numel() == 0:
+        if params.numel() == 0 and params.shape[0] != B:  # a term without per-sample parameters
             params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
         shared = f.builtin_shared().to(device=dev, dtype=dtype) if hasattr(f, "builtin_shared") else None
