@@ -56,7 +56,7 @@ def main():
     )
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (samples would shard over the batch axis, see DESIGN.md)")
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (with more GPUs the batch axis would be split, every GPU solving its own samples)")
 
     import torch
 

@@ -19,6 +19,13 @@ _PROTOCOL_NAMES = (
 )  # fmt: skip
 
 
+def _f_evals(count: int, batch: int) -> torch.Tensor:
+    """``stats["n_f_evals"]``: int64 ``[B]`` on the CPU, every sample carrying the same count (the
+    reference counts evaluations of ``f`` on the whole batch, terms.py:41-63).  One stored value
+    viewed ``B`` times: filling half a megabyte per solve costs more than the kernel launch."""
+    return torch.tensor(count, dtype=torch.long).expand(batch)
+
+
 def _library_object(obj, classes) -> bool:
     """True if ``obj`` is exactly one of the library's classes with no protocol method replaced on
     the instance; only then may a fused kernel stand in for the calls the loop would make."""
@@ -305,7 +312,7 @@ class AutoDiffAdjoint(nn.Module):
         stats: Dict[str, Any] = {}
         if term.with_stats:
             n = n_init_evals + 6 * fl[_lib.STEP_FLAG_ITERATIONS]
-            stats["n_f_evals"] = torch.full((B,), n, dtype=torch.long, device="cpu")
+            stats["n_f_evals"] = _f_evals(n, B)
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
         ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
         return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
@@ -382,7 +389,7 @@ class AutoDiffAdjoint(nn.Module):
             if not fl[_lib.FLAG_NEEDS_GENERAL]:
                 if term.with_stats:
                     last = fl[_lib.FLAG_MAX_ITERATIONS]
-                    stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
+                    stats["n_f_evals"] = _f_evals(n_init_evals + 6 * last, B)
                 stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
                 return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
 
@@ -415,7 +422,7 @@ class AutoDiffAdjoint(nn.Module):
         _lib.check(rc, "tode_finalize_stats")
 
         if term.with_stats:
-            stats["n_f_evals"] = torch.full((B,), n_init_evals + 6 * last, dtype=torch.long, device="cpu")
+            stats["n_f_evals"] = _f_evals(n_init_evals + 6 * last, B)
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
         return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
 
