@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 4
+#define TODE_ABI_VERSION 5
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -317,11 +317,17 @@ const char *tode_last_solve_kernel_name(void);
  * step_size_controllers.py:16-113, interpolation.py:43-45), and users may supply their own
  * implementation of any of them.  The operators below are what the package's own
  * implementations of those protocol methods call, one kernel each, so that any mix of
- * library and user-supplied parts runs through the same loop.  Time and data share `dtype`.
+ * library and user-supplied parts runs through the same loop.  Time and data may have different
+ * floating point types (reference problems.py:44-56, tests/dtype_stability_test.py), see TODE_DTYPES.
  * All pointers are device pointers except the `const double *` coefficient arrays, which are
  * host arrays read before the call returns.  Arrays are dense row-major.
  * ------------------------------------------------------------------------------------------ */
 #define TODE_MAX_STAGES 16
+/* dtype argument of the operators when time and data differ: TODE_DTYPES(data, time); a plain
+ * TODE_F32 / TODE_F64 means both.  Time: t, dt, t_start, t_end, t_eval and everything derived
+ * (node times, next step size).  Data: y, derivatives, coefficients, error norms and ratios. */
+#define TODE_DTYPE_PAIR 0x100
+#define TODE_DTYPES(data, time) (TODE_DTYPE_PAIR | (data) | ((time) << 4))
 enum { TODE_NORM_RMS = 0, TODE_NORM_MAX = 1 }; /* reference step_size_controllers.py:170-186 */
 
 /* Coefficients the kernels use for Dopri5 / Tsit5 (reference dopri5.py:11-44, tsit5.py:11-114), as doubles:

@@ -611,3 +611,66 @@ def test_protocol_path_without_evaluation_points_and_backwards():
     t0[flip], t1[flip] = t1[flip], t0[flip].clone()
     sol = protocol_solve(w.f, w.y0, None, w.method, w.controller, t_start=t0, t_end=t1)
     assert_identical(sol, c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=t0, t_end=t1))
+
+
+# ---------------------------------------------------------------------------------------------
+# part four: time and data in different dtypes (reference tests/dtype_stability_test.py)
+# ---------------------------------------------------------------------------------------------
+
+MIXED = [(torch.float64, torch.float32), (torch.float32, torch.float64)]
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", MIXED, ids=["t64-y32", "t32-y64"])
+@pytest.mark.parametrize("method", [to.Dopri5, to.Tsit5])
+def test_time_and_data_dtypes_are_kept_apart(time_dtype, data_dtype, method):
+    seen = []
+
+    def rhs(t, y):
+        assert t.dtype == time_dtype and y.dtype == data_dtype
+        seen.append(t)
+        return torch.zeros_like(y)
+
+    y0 = torch.tensor([[0.33, 1.2, -0.4]], dtype=data_dtype, device=DEV)
+    t_eval = torch.tensor([[0.0, 1.77, 3.0]], dtype=time_dtype, device=DEV)
+    problem = to.InitialValueProblem(y0, t_start=t_eval[:, 0], t_end=t_eval[:, -1], t_eval=t_eval)
+    sol = to.AutoDiffAdjoint(method(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0)).solve(problem, to.ODETerm(rhs))
+    assert sol.stats["n_steps"].item() > 3 and sol.status.item() == OK and len(seen) > 20
+    assert sol.ts.dtype == time_dtype and sol.ys.dtype == data_dtype
+    assert torch.equal(sol.ys, y0[:, None].expand(1, 3, 3))  # zero dynamics: exact
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", MIXED, ids=["t64-y32", "t32-y64"])
+def test_mixed_dtypes_solve_the_same_problem(time_dtype, data_dtype):
+    w = to.workloads.make("vdp", batch=96, dtype=torch.float64, device=DEV)
+    f64 = to.VanDerPol(w.f.mu)
+    fd = to.VanDerPol(w.f.mu.to(data_dtype))
+    ctrl = dict(kind="pid", atol=1e-7, rtol=1e-6, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)
+    ref = to.AutoDiffAdjoint(to.Tsit5(), make_controller(ctrl)).solve(to.InitialValueProblem(w.y0, t_eval=w.t_eval), to.ODETerm(f64))
+    problem = to.InitialValueProblem(w.y0.to(data_dtype), t_eval=w.t_eval.to(time_dtype))
+    sol = to.AutoDiffAdjoint(to.Tsit5(), make_controller(ctrl)).solve(problem, to.ODETerm(lambda t, y: fd(t, y)))
+    assert sol.ys.dtype == data_dtype and sol.ts.dtype == time_dtype and (sol.status == OK).all()
+    assert (sol.stats["n_initialized"] == w.t_eval.shape[1]).all()
+    err = (sol.ys.double() - ref.ys).abs().max().item()
+    assert err < (2e-3 if torch.float32 in (time_dtype, data_dtype) else 1e-9), err
+    work = sol.stats["n_steps"].sum().item() / ref.stats["n_steps"].sum().item()
+    assert 0.7 < work < 1.4, work
+
+
+def test_user_defined_method_with_mixed_dtypes():
+    y0 = torch.tensor([[0.0], [1.0]], dtype=torch.float32, device=DEV)
+    t_start, t_end = dev([0.0, 1.0], torch.float64), dev([2.0, 4.0], torch.float64)
+    term = to.ODETerm(lambda t, y: torch.ones_like(y))
+    dt = [0.25, 0.5]
+
+    class Euler64(ForwardEuler):
+        def step(self, term, running, y0, t0, dt, state, *, stats, args):
+            assert t0.dtype == dt.dtype == torch.float64 and y0.dtype == torch.float32
+            y1 = y0 + dt.to(y0.dtype)[:, None] * term.vf(t0, y0, stats, args)
+            return StepResult(y1, None), (t0, dt, y0, y1), None, None
+
+    ctrl = ScriptedController(dt, [dt])
+    ctrl.init = lambda term, problem, order, dt0, *, stats, args: (dev(dt, torch.float64), {}, None)
+    ctrl.adapt_step_size = lambda t0, dt_, y0, sr, state, stats: (torch.ones(2, dtype=torch.bool, device=DEV), dev(dt, torch.float64), state, None)
+    sol = to.AutoDiffAdjoint(Euler64(), ctrl).solve(to.InitialValueProblem(y0, t_start, t_end), term)
+    assert sol.stats["n_steps"].tolist() == [8, 6] and sol.ys.dtype == torch.float32 and sol.ts.dtype == torch.float64
+    assert torch.allclose(sol.ys[:, 0, 0], dev([2.0, 4.0]))

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -270,6 +270,15 @@ def check(rc: int, what: str):
     if rc != 0:
         msg = load().tode_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"{what} failed with code {rc}: {msg}")
+
+
+def dtype_code(data_dtype, time_dtype=None) -> int:
+    """``dtype`` argument of the operator entry points (TODE_DTYPES in the header)."""
+    if data_dtype not in DTYPES or (time_dtype is not None and time_dtype not in DTYPES):
+        raise NotImplementedError(f"the kernels are built for float32 and float64 (got data {data_dtype}, time {time_dtype})")
+    if time_dtype is None or time_dtype == data_dtype:
+        return DTYPES[data_dtype]
+    return 0x100 | DTYPES[data_dtype] | (DTYPES[time_dtype] << 4)
 
 
 def ptr(t):

@@ -81,11 +81,6 @@ class AutoDiffAdjoint(nn.Module):
                 return sol
         if self._stepwise_ok(problem, term_):
             return self._solve_stepwise(problem, term_, dt0, args)
-        if problem.data_dtype != problem.time_dtype or problem.data_dtype not in _lib.DTYPES:
-            raise NotImplementedError(
-                "the solve loop needs time and data in one dtype, float32 or float64 "
-                f"(got time {problem.time_dtype}, data {problem.data_dtype})"
-            )
         return self._solve_protocol(problem, term, term_, dt0, args)
 
     # ------------------------------------------------------------------ #
@@ -118,7 +113,8 @@ class AutoDiffAdjoint(nn.Module):
         reference synchronises there as well)."""
         lib = _lib.load()
         method, controller = self.step_method, self.step_size_controller
-        dev, dtype, code = problem.device, problem.data_dtype, _lib.DTYPES[problem.data_dtype]
+        dev, dtype, ttype = problem.device, problem.data_dtype, problem.time_dtype
+        code = _lib.dtype_code(dtype, ttype)  # time and data may differ (float32 / float64 each)
         B, F, E = problem.batch_size, problem.n_features, problem.n_evaluation_points
         stream = _lib.stream_of(problem.y0)
         t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
@@ -127,9 +123,9 @@ class AutoDiffAdjoint(nn.Module):
         t = t_start
         new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
 
-        def as_float(x, shape):
+        def as_float(x, shape, to=dtype):
             x = torch.as_tensor(x, device=dev)
-            return x.to(dtype).expand(shape).contiguous()
+            return x.to(to).expand(shape).contiguous()
 
         def as_status(x):
             return None if x is None else torch.as_tensor(x, device=dev).to(torch.long).expand((B,)).contiguous()
@@ -142,7 +138,7 @@ class AutoDiffAdjoint(nn.Module):
 
         ys = new(B, max(E, 1), F)
         pending = new(B, E, dt=torch.uint8) if E > 0 else None
-        dt_in, dt = as_float(dt, (B,)), new(B)
+        dt_in, dt = as_float(dt, (B,), ttype), new(B, dt=ttype)
         rc = lib.tode_loop_begin(
             code, B, F, E, _lib.ptr(t_start), _lib.ptr(t_end), _lib.ptr(t_eval), _lib.ptr(y), _lib.ptr(dt_in), _lib.ptr(dt),
             _lib.ptr(pending), _lib.ptr(ys), stream,
@@ -174,9 +170,9 @@ class AutoDiffAdjoint(nn.Module):
             # ---- one kernel: state update, counters, running, status, evaluation mask, next dt ----
             y_new = as_float(step_result.y, (B, F))
             accept_ = torch.as_tensor(accept, device=dev).to(torch.bool).expand((B,)).contiguous()
-            dt_next_ = as_float(dt_next, (B,))
+            dt_next_ = as_float(dt_next, (B,), ttype)
             m_status, c_status = as_status(method_status), as_status(controller_status)
-            t_out, dt_out, y_out = new(B), new(B), new(B, F)
+            t_out, dt_out, y_out = new(B, dt=ttype), new(B, dt=ttype), new(B, F)
             running_out, to_update = new(B, dt=torch.bool), new(B, dt=torch.bool)
             status = new(B, dt=torch.long)
             to_evaluate = new(B, E, dt=torch.uint8) if E > 0 else None

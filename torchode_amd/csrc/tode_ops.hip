@@ -4,6 +4,10 @@
 // iteration.  The package's Python classes call these, so that library parts and
 // user-supplied parts can be mixed freely in one solve.
 //
+// Time (t, dt, evaluation times) and data (y, derivatives, error ratios) may have different
+// floating point types, TT and T below; every formula converts where the reference does
+// (dt to the data type for the stage sums, the step factor to the time type for the new step).
+//
 // Elementwise kernels use one thread per value of [B,F].  Per-sample kernels use
 // one thread per sample and walk the row in order when F < 64 (the summation
 // order of a scalar evaluation), and one wavefront per sample when F >= 64.
@@ -22,28 +26,28 @@ struct Coeffs {
 // ------------------------------------------------------------------------------------------
 
 // y_out = fma(dt, sum_j a_j k_j, y0), t_out = fma(c, dt, t0)   (runge_kutta.py:258-262)
-template <typename T>
-__global__ void __launch_bounds__(256) erk_stage_kernel(long long batch, int F, int n, Coeffs a, double c, const T *t0, const T *dt,
-                                                        const T *y0, const T *k, T *y_out, T *t_out) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) erk_stage_kernel(long long batch, int F, int n, Coeffs a, double c, const TT *t0, const TT *dt,
+                                                        const T *y0, const T *k, T *y_out, TT *t_out) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long bf = batch * F;
     if (i >= bf) return;
     const long long b = i / F;
-    const T h = dt[b];
+    const T h = (T)dt[b];
     T s = 0;
     for (int j = 0; j < n; ++j) s = fma_((T)a.v[j], k[j * bf + i], s);
     y_out[i] = fma_(h, s, y0[i]);
-    if (t_out && i - b * F == 0) t_out[b] = fma_((T)c, h, t0[b]);
+    if (t_out && i - b * F == 0) t_out[b] = fma_((TT)c, dt[b], t0[b]);
 }
 
 // out = sum_s (dt * w_s) * k_s (+ y0)   (runge_kutta.py:264-267).  ATen rounds the products
 // before adding them for F <= 57 and runs one fused chain for F >= 58.
-template <typename T>
-__global__ void __launch_bounds__(256) erk_combine_kernel(long long batch, int F, int S, Coeffs w, const T *dt, const T *k, const T *y0, T *out) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) erk_combine_kernel(long long batch, int F, int S, Coeffs w, const TT *dt, const T *k, const T *y0, T *out) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long bf = batch * F;
     if (i >= bf) return;
-    const T h = dt[i / F];
+    const T h = (T)dt[i / F];
     const bool fused = F >= 58;
     T acc = 0;
     for (int s = 0; s < S; ++s) {
@@ -150,17 +154,32 @@ struct ControlOut {
     int64_t *status;
 };
 
-// ratio -> accept, dt_next, status, PID history (step_size_controllers.py:394-429, 640-671, 739-774)
-template <typename T, int CTRL>
-__device__ __forceinline__ void control_one(const CtrlParams<T> &cp, long long b, T norm, T dt, const T *prev, const T *pprev, const ControlOut &o) {
+// ratio -> accept, dt_next, status, PID history (step_size_controllers.py:394-429, 640-671, 739-774).
+// The factor is formed in the data type and converted; the new step and its limits live in the time type.
+template <typename TT> struct StepLimits {
+    TT dt_min, dt_max;
+};
+
+template <typename TT, typename T, int CTRL>
+__device__ __forceinline__ void control_one(const CtrlParams<T> &cp, const StepLimits<TT> &lim, long long b, T norm, TT dt, const T *prev, const T *pprev,
+                                            const ControlOut &o) {
     const T ratio = tmax(norm, (T)1e-38);
     const bool accept = ratio < (T)1;
     const T p1 = CTRL == 1 ? prev[b] : (T)1, p2 = CTRL == 1 ? pprev[b] : (T)1;
     const T factor = dt_factor<T, CTRL>(cp, ratio, p1, p2);
-    T dt_next = dt * factor;
-    const int status = limit_dt<T>(cp, ratio, dt_next);
+    TT dt_next = dt * (TT)factor;
+    int status = finite_(ratio) ? 0 : 4;
+    if (cp.has_dt_min || cp.has_dt_max) {
+        const TT mag = abs_(dt_next);
+        TT c = mag;
+        if (cp.has_dt_min) c = tmax(c, lim.dt_min);
+        if (cp.has_dt_max) c = tmin(c, lim.dt_max);
+        const TT sg = (dt_next > 0) ? (TT)1 : ((dt_next < 0) ? (TT)-1 : dt_next);
+        dt_next = sg * c;
+        if (cp.has_dt_min && mag < lim.dt_min) status = 2;
+    }
     o.accept[b] = accept ? 1 : 0;
-    ((T *)o.dt_next)[b] = dt_next;
+    ((TT *)o.dt_next)[b] = dt_next;
     if (o.ratio) ((T *)o.ratio)[b] = ratio;
     o.status[b] = status;
     if (CTRL == 1) {
@@ -169,38 +188,39 @@ __device__ __forceinline__ void control_one(const CtrlParams<T> &cp, long long b
     }
 }
 
-template <typename T, int CTRL>
-__global__ void __launch_bounds__(256) control_kernel(CtrlParams<T> cp, long long batch, const T *norm, const T *dt, const T *prev, const T *pprev, ControlOut o) {
+template <typename TT, typename T, int CTRL>
+__global__ void __launch_bounds__(256) control_kernel(CtrlParams<T> cp, StepLimits<TT> lim, long long batch, const T *norm, const TT *dt, const T *prev,
+                                                      const T *pprev, ControlOut o) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (b < batch) control_one<T, CTRL>(cp, b, norm[b], dt[b], prev, pprev, o);
+    if (b < batch) control_one<TT, T, CTRL>(cp, lim, b, norm[b], dt[b], prev, pprev, o);
 }
 
-template <typename T, int CTRL, int NORM>
-__global__ void __launch_bounds__(256) adapt_thread_kernel(CtrlParams<T> cp, long long batch, int F, const T *dt, const T *y0, const T *y1, const T *err,
-                                                           const T *prev, const T *pprev, ControlOut o) {
+template <typename TT, typename T, int CTRL, int NORM>
+__global__ void __launch_bounds__(256) adapt_thread_kernel(CtrlParams<T> cp, StepLimits<TT> lim, long long batch, int F, const TT *dt, const T *y0,
+                                                           const T *y1, const T *err, const T *prev, const T *pprev, ControlOut o) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
     RowNorm<T, NORM> r(F);
     for (int f = 0; f < F; ++f) r.add(scaled_error(cp.atol, cp.rtol, y0[b * F + f], y1[b * F + f], err[b * F + f]));
-    control_one<T, CTRL>(cp, b, r.get(), dt[b], prev, pprev, o);
+    control_one<TT, T, CTRL>(cp, lim, b, r.get(), dt[b], prev, pprev, o);
 }
 
-template <typename T, int CTRL, int NORM>
-__global__ void __launch_bounds__(256) adapt_wave_kernel(CtrlParams<T> cp, long long batch, int F, const T *dt, const T *y0, const T *y1, const T *err,
-                                                         const T *prev, const T *pprev, ControlOut o) {
+template <typename TT, typename T, int CTRL, int NORM>
+__global__ void __launch_bounds__(256) adapt_wave_kernel(CtrlParams<T> cp, StepLimits<TT> lim, long long batch, int F, const TT *dt, const T *y0,
+                                                         const T *y1, const T *err, const T *prev, const T *pprev, ControlOut o) {
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= batch) return;
     const T *r0 = y0 + b * F, *r1 = y1 + b * F, *re = err + b * F;
     const T norm = wave_row_norm<T, NORM>(F, [&](int f) { return scaled_error(cp.atol, cp.rtol, r0[f], r1[f], re[f]); });
-    if ((threadIdx.x & 63) == 0) control_one<T, CTRL>(cp, b, norm, dt[b], prev, pprev, o);
+    if ((threadIdx.x & 63) == 0) control_one<TT, T, CTRL>(cp, lim, b, norm, dt[b], prev, pprev, o);
 }
 
 // ------------------------------------------------------------------------------------------
 // start step (step_size_controllers.py:431-490, 776-835)
 // ------------------------------------------------------------------------------------------
 
-template <typename T, int NORM>
-__global__ void __launch_bounds__(256) initial_a_thread_kernel(long long batch, int F, T atol, T rtol, const T *t_start, const T *t_end, const T *y0,
+template <typename TT, typename T, int NORM>
+__global__ void __launch_bounds__(256) initial_a_thread_kernel(long long batch, int F, T atol, T rtol, const TT *t_start, const TT *t_end, const T *y0,
                                                                const T *f0, T *h0_out) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
@@ -212,11 +232,11 @@ __global__ void __launch_bounds__(256) initial_a_thread_kernel(long long batch, 
     }
     const T d0 = n0.get(), d1 = n1.get();
     T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
-    h0_out[b] = tmin(h0, abs_(t_end[b] - t_start[b]));
+    h0_out[b] = tmin(h0, (T)abs_(t_end[b] - t_start[b]));
 }
 
-template <typename T, int NORM>
-__global__ void __launch_bounds__(256) initial_a_wave_kernel(long long batch, int F, T atol, T rtol, const T *t_start, const T *t_end, const T *y0,
+template <typename TT, typename T, int NORM>
+__global__ void __launch_bounds__(256) initial_a_wave_kernel(long long batch, int F, T atol, T rtol, const TT *t_start, const TT *t_end, const T *y0,
                                                              const T *f0, T *h0_out) {
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= batch) return;
@@ -225,26 +245,26 @@ __global__ void __launch_bounds__(256) initial_a_wave_kernel(long long batch, in
     const T d1 = wave_row_norm<T, NORM>(F, [&](int f) { return rf[f] * inv_scale(atol, rtol, ry[f]); });
     if ((threadIdx.x & 63) == 0) {
         T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
-        h0_out[b] = tmin(h0, abs_(t_end[b] - t_start[b]));
+        h0_out[b] = tmin(h0, (T)abs_(t_end[b] - t_start[b]));
     }
 }
 
 // y1 = y0 + (direction * h0) * f0, t1 = t_start + direction * h0   (:474-479)
-template <typename T>
-__global__ void __launch_bounds__(256) initial_probe_kernel(long long batch, int F, const T *t_start, const T *t_end, const T *y0, const T *f0, const T *h0,
-                                                            T *y1, T *t1) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) initial_probe_kernel(long long batch, int F, const TT *t_start, const TT *t_end, const T *y0, const T *f0,
+                                                            const T *h0, T *y1, TT *t1) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i >= batch * F) return;
     const long long b = i / F;
-    const T dir = (t_end[b] > t_start[b]) ? (T)1 : (T)-1;
+    const bool fwd = t_end[b] > t_start[b];
     const T h = h0[b];
-    y1[i] = fma_(dir * h, f0[i], y0[i]);
-    if (i - b * F == 0) t1[b] = fma_(dir, h, t_start[b]);
+    y1[i] = fma_((fwd ? (T)1 : (T)-1) * h, f0[i], y0[i]);
+    if (i - b * F == 0) t1[b] = fma_(fwd ? (TT)1 : (TT)-1, (TT)h, t_start[b]);
 }
 
-template <typename T, int NORM>
-__global__ void __launch_bounds__(256) initial_b_thread_kernel(int kind, double inv_order, long long batch, int F, T atol, T rtol, const T *t_start,
-                                                               const T *t_end, const T *y0, const T *f0, const T *f1, const T *h0, T *dt0) {
+template <typename TT, typename T, int NORM>
+__global__ void __launch_bounds__(256) initial_b_thread_kernel(int kind, double inv_order, long long batch, int F, T atol, T rtol, const TT *t_start,
+                                                               const TT *t_end, const T *y0, const T *f0, const T *f1, const T *h0, TT *dt0) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
     RowNorm<T, NORM> n1(F), n2(F);
@@ -255,12 +275,12 @@ __global__ void __launch_bounds__(256) initial_b_thread_kernel(int kind, double 
         n2.add(df * inv);
     }
     const T dir = (t_end[b] > t_start[b]) ? (T)1 : (T)-1;
-    dt0[b] = initial_finish<T>(kind, inv_order, dir, h0[b], n1.get(), n2.get());
+    dt0[b] = (TT)initial_finish<T>(kind, inv_order, dir, h0[b], n1.get(), n2.get());
 }
 
-template <typename T, int NORM>
-__global__ void __launch_bounds__(256) initial_b_wave_kernel(int kind, double inv_order, long long batch, int F, T atol, T rtol, const T *t_start,
-                                                             const T *t_end, const T *y0, const T *f0, const T *f1, const T *h0, T *dt0) {
+template <typename TT, typename T, int NORM>
+__global__ void __launch_bounds__(256) initial_b_wave_kernel(int kind, double inv_order, long long batch, int F, T atol, T rtol, const TT *t_start,
+                                                             const TT *t_end, const T *y0, const T *f0, const T *f1, const T *h0, TT *dt0) {
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= batch) return;
     const T *ry = y0 + b * F, *r0 = f0 + b * F, *r1 = f1 + b * F;
@@ -271,7 +291,7 @@ __global__ void __launch_bounds__(256) initial_b_wave_kernel(int kind, double in
     });
     if ((threadIdx.x & 63) == 0) {
         const T dir = (t_end[b] > t_start[b]) ? (T)1 : (T)-1;
-        dt0[b] = initial_finish<T>(kind, inv_order, dir, h0[b], d1, d2n);
+        dt0[b] = (TT)initial_finish<T>(kind, inv_order, dir, h0[b], d1, d2n);
     }
 }
 
@@ -279,8 +299,8 @@ __global__ void __launch_bounds__(256) initial_b_wave_kernel(int kind, double in
 // dense output
 // ------------------------------------------------------------------------------------------
 
-template <typename T, int METHOD>
-__global__ void __launch_bounds__(256) quartic_build_kernel(long long batch, int F, const T *dt, const T *y0, const T *y1, const T *k, T *coeff) {
+template <typename TT, typename T, int METHOD>
+__global__ void __launch_bounds__(256) quartic_build_kernel(long long batch, int F, const TT *dt, const T *y0, const T *y1, const T *k, T *coeff) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long bf = batch * F;
     if (i >= bf) return;
@@ -288,19 +308,19 @@ __global__ void __launch_bounds__(256) quartic_build_kernel(long long batch, int
 #pragma unroll
     for (int s = 0; s < 7; ++s) ks[s] = k[s * bf + i];
     T q[5][1];
-    quartic_elem<T, METHOD>(dt[i / F], y0[i], y1[i], ks, F >= 58, q);
+    quartic_elem<T, METHOD>((T)dt[i / F], y0[i], y1[i], ks, F >= 58, q);
 #pragma unroll
     for (int p = 0; p < 5; ++p) coeff[p * bf + i] = q[p][0];
 }
 
 // Quartic through y0, y1, the end-point slopes and a mid-point value (interpolation.py:138-170).
-template <typename T>
-__global__ void __launch_bounds__(256) quartic_from_mid_kernel(long long batch, int F, const T *dt, const T *y0, const T *y1, const T *k_first,
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) quartic_from_mid_kernel(long long batch, int F, const TT *dt, const T *y0, const T *y1, const T *k_first,
                                                                const T *k_last, const T *y_mid, T *coeff) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long bf = batch * F;
     if (i >= bf) return;
-    const T h = dt[i / F];
+    const T h = (T)dt[i / F];
     const T f0 = h * k_first[i], f1 = h * k_last[i], ym = y_mid[i], a0 = y0[i], a1 = y1[i];
     T a = (T)2 * (f1 - f0);
     a = fma_((T)-8, a1 + a0, a);
@@ -322,13 +342,13 @@ __global__ void __launch_bounds__(256) quartic_from_mid_kernel(long long batch, 
 }
 
 // Hermite cubic through y0, y1 and the end-point slopes (interpolation.py:84-106).
-template <typename T>
-__global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F, const T *dt, const T *y0, const T *y1, const T *k_first,
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F, const TT *dt, const T *y0, const T *y1, const T *k_first,
                                                           const T *k_last, T *coeff) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long bf = batch * F;
     if (i >= bf) return;
-    const T h = dt[i / F];
+    const T h = (T)dt[i / F];
     const T f0 = k_first[i], f1 = k_last[i];
     const T d01 = y0[i] - y1[i];
     const T a = fma_((T)2, d01, h * (f0 + f1));            // add(dt*(f0+f1), y0-y1, alpha=2)
@@ -339,39 +359,39 @@ __global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F
     coeff[3 * bf + i] = a;
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) poly_eval_kernel(int degree, long long batch, int F, long long count, const T *coeff, const T *t0, const T *t1,
-                                                        const T *t, const int64_t *idx, T *out) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) poly_eval_kernel(int degree, long long batch, int F, long long count, const T *coeff, const TT *t0, const TT *t1,
+                                                        const TT *t, const int64_t *idx, T *out) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i >= count * F) return;
     const long long n = i / F;
     const int f = (int)(i - n * F);
     const long long b = idx[n];
     if (b < 0 || b >= batch) return;
-    out[i] = horner(coeff, batch * F, b * F + f, degree, unit_time(t[n], t0[b], t1[b]));
+    out[i] = horner(coeff, batch * F, b * F + f, degree, (T)unit_time(t[n], t0[b], t1[b]));
 }
 
 // small F: one thread per sample walks its mask row
-template <typename T>
-__global__ void __launch_bounds__(256) poly_eval_masked_thread_kernel(int degree, long long batch, int F, int E, const T *coeff, const T *t0, const T *t1,
-                                                                      const T *t_eval, const uint8_t *mask, T *ys) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) poly_eval_masked_thread_kernel(int degree, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
+                                                                      const TT *t_eval, const uint8_t *mask, T *ys) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
     for (int e = 0; e < E; ++e) {
         if (!mask[b * E + e]) continue;
-        const T x = unit_time(t_eval[b * E + e], t0[b], t1[b]);
+        const T x = (T)unit_time(t_eval[b * E + e], t0[b], t1[b]);
         for (int f = 0; f < F; ++f) ys[(b * E + e) * F + f] = horner(coeff, batch * F, b * F + f, degree, x);
     }
 }
 
 // large F: one workgroup per sample, threads over features
-template <typename T>
-__global__ void __launch_bounds__(256) poly_eval_masked_block_kernel(int degree, long long batch, int F, int E, const T *coeff, const T *t0, const T *t1,
-                                                                     const T *t_eval, const uint8_t *mask, T *ys) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) poly_eval_masked_block_kernel(int degree, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
+                                                                     const TT *t_eval, const uint8_t *mask, T *ys) {
     const long long b = blockIdx.x;
     for (int e = 0; e < E; ++e) {
         if (!mask[b * E + e]) continue;  // uniform over the workgroup
-        const T x = unit_time(t_eval[b * E + e], t0[b], t1[b]);
+        const T x = (T)unit_time(t_eval[b * E + e], t0[b], t1[b]);
         for (int f = threadIdx.x; f < F; f += 256) ys[(b * E + e) * F + f] = horner(coeff, batch * F, b * F + f, degree, x);
     }
 }
@@ -447,13 +467,13 @@ template <typename T> __global__ void __launch_bounds__(256) loop_advance_kernel
     }
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) loop_begin_kernel(long long batch, int F, int E, const T *t_start, const T *t_end, const T *t_eval, const T *y0,
-                                                         const T *dt, T *dt_out, uint8_t *pending, T *ys) {
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) loop_begin_kernel(long long batch, int F, int E, const TT *t_start, const TT *t_end, const TT *t_eval, const T *y0,
+                                                         const TT *dt, TT *dt_out, uint8_t *pending, T *ys) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
-    const T ts = t_start[b], te = t_end[b];
-    const T tlo = tmin(ts, te), thi = tmax(te, ts);
+    const TT ts = t_start[b], te = t_end[b];
+    const TT tlo = tmin(ts, te), thi = tmax(te, ts);
     dt_out[b] = tclamp(dt[b], tlo - ts, thi - ts);
     if (E > 0) {
         const bool at_start = t_eval[b * E] == ts;
@@ -477,8 +497,13 @@ static __global__ void __launch_bounds__(256) count_initialized_kernel(long long
 
 static unsigned blocks_for(long long n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
+static int data_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? (dtype & 0xF) : dtype; }
+static int time_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? ((dtype >> 4) & 0xF) : dtype; }
+
 static int check_common(int32_t dtype, int64_t batch, int32_t F) {
-    if (dtype != TODE_F32 && dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", dtype);
+    const int d = data_type(dtype), t = time_type(dtype);
+    if ((d != TODE_F32 && d != TODE_F64) || (t != TODE_F32 && t != TODE_F64) || (dtype & ~(TODE_DTYPE_PAIR | 0xFF)))
+        return fail(TODE_E_INVALID, "unknown dtype %d", dtype);
     if (batch < 0 || F <= 0) return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d", (long long)batch, F);
     if (batch * (long long)F > (long long)INT_MAX * 256) return fail(TODE_E_UNSUPPORTED, "batch * features too large");
     return TODE_OK;
@@ -495,6 +520,18 @@ static int done(const char *what) { return check_hip(hipGetLastError(), what); }
             using T = double;      \
             __VA_ARGS__;           \
         }                          \
+    } while (0)
+
+// TT = time type, T = data type
+#define TODE_TT(dtype, ...)                      \
+    do {                                         \
+        if (time_type(dtype) == TODE_F32) {      \
+            using TT = float;                    \
+            TODE_T(data_type(dtype), __VA_ARGS__); \
+        } else {                                 \
+            using TT = double;                   \
+            TODE_T(data_type(dtype), __VA_ARGS__); \
+        }                                        \
     } while (0)
 
 // dispatch on (controller kind, norm) at compile time
@@ -558,8 +595,8 @@ int tode_erk_stage(int32_t dtype, int64_t batch, int32_t F, int32_t n_terms, con
     if ((n_terms > 0 && (!a || !k)) || !dt || !y0 || !y_out || (t_out && !t0)) return fail(TODE_E_INVALID, "null pointer");
     Coeffs co{};
     for (int j = 0; j < n_terms; ++j) co.v[j] = a[j];
-    TODE_T(dtype, hipLaunchKernelGGL(erk_stage_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F, n_terms,
-                                     co, c, (const T *)t0, (const T *)dt, (const T *)y0, (const T *)k, (T *)y_out, (T *)t_out));
+    TODE_TT(dtype, hipLaunchKernelGGL((erk_stage_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
+                                      n_terms, co, c, (const TT *)t0, (const TT *)dt, (const T *)y0, (const T *)k, (T *)y_out, (TT *)t_out));
     return done("tode_erk_stage launch");
 }
 
@@ -571,8 +608,8 @@ int tode_erk_combine(int32_t dtype, int64_t batch, int32_t F, int32_t S, const d
     if (!w || !dt || !k || !out) return fail(TODE_E_INVALID, "null pointer");
     Coeffs co{};
     for (int j = 0; j < S; ++j) co.v[j] = w[j];
-    TODE_T(dtype, hipLaunchKernelGGL(erk_combine_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F, S, co,
-                                     (const T *)dt, (const T *)k, (const T *)y0, (T *)out));
+    TODE_TT(dtype, hipLaunchKernelGGL((erk_combine_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F, S,
+                                      co, (const TT *)dt, (const T *)k, (const T *)y0, (T *)out));
     return done("tode_erk_combine launch");
 }
 
@@ -581,8 +618,8 @@ int tode_error_scale(int32_t dtype, int64_t batch, int32_t F, double atol, doubl
     if (int rc = check_common(dtype, batch, F)) return rc;
     if (batch == 0) return TODE_OK;
     if (!y0 || !y1 || !err || !out) return fail(TODE_E_INVALID, "null pointer");
-    TODE_T(dtype, hipLaunchKernelGGL(error_scale_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch * F,
-                                     (T)(float)atol, (T)(float)rtol, (const T *)y0, (const T *)y1, (const T *)err, (T *)out));
+    TODE_T(data_type(dtype), hipLaunchKernelGGL(error_scale_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream,
+                                                (long long)batch * F, (T)(float)atol, (T)(float)rtol, (const T *)y0, (const T *)y1, (const T *)err, (T *)out));
     return done("tode_error_scale launch");
 }
 
@@ -592,7 +629,7 @@ int tode_row_norm(int32_t dtype, int32_t norm, int64_t batch, int32_t F, const v
     if (batch == 0) return TODE_OK;
     if (!x || !out) return fail(TODE_E_INVALID, "null pointer");
     hipStream_t s = (hipStream_t)stream;
-    TODE_T(dtype, TODE_CN(0, norm, {
+    TODE_T(data_type(dtype), TODE_CN(0, norm, {
                (void)CTRL;
                if (F < 64)
                    hipLaunchKernelGGL((row_norm_thread_kernel<T, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, (long long)batch, F, (const T *)x, (T *)out);
@@ -609,11 +646,12 @@ int tode_control(int32_t dtype, const tode_controller *c, int32_t order, int64_t
     if (batch == 0) return TODE_OK;
     if (!norm || !dt || !accept || !dt_next || !status) return fail(TODE_E_INVALID, "null pointer");
     ControlOut o{accept, dt_next, ratio, prev_out, pprev_out, status};
-    TODE_T(dtype, TODE_CN(c->kind, TODE_NORM_RMS, {
-               (void)NORM;
-               hipLaunchKernelGGL((control_kernel<T, CTRL>), dim3(blocks_for(batch, 256)), dim3(256), 0, (hipStream_t)stream, make_ctrl<T>(*c, (double)order),
-                                  (long long)batch, (const T *)norm, (const T *)dt, (const T *)prev, (const T *)pprev, o);
-           }));
+    TODE_TT(dtype, TODE_CN(c->kind, TODE_NORM_RMS, {
+                (void)NORM;
+                const StepLimits<TT> lim{(TT)c->dt_min, (TT)c->dt_max};
+                hipLaunchKernelGGL((control_kernel<TT, T, CTRL>), dim3(blocks_for(batch, 256)), dim3(256), 0, (hipStream_t)stream,
+                                   make_ctrl<T>(*c, (double)order), lim, (long long)batch, (const T *)norm, (const TT *)dt, (const T *)prev, (const T *)pprev, o);
+            }));
     return done("tode_control launch");
 }
 
@@ -627,15 +665,16 @@ int tode_adapt_step(int32_t dtype, const tode_controller *c, int32_t order, int3
     if (!dt || !y0 || !y1 || !err || !accept || !dt_next || !status) return fail(TODE_E_INVALID, "null pointer");
     ControlOut o{accept, dt_next, ratio, prev_out, pprev_out, status};
     hipStream_t s = (hipStream_t)stream;
-    TODE_T(dtype, TODE_CN(c->kind, norm, {
-               const CtrlParams<T> cp = make_ctrl<T>(*c, (double)order);
-               if (F < 64)
-                   hipLaunchKernelGGL((adapt_thread_kernel<T, CTRL, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, cp, (long long)batch, F, (const T *)dt,
-                                      (const T *)y0, (const T *)y1, (const T *)err, (const T *)prev, (const T *)pprev, o);
-               else
-                   hipLaunchKernelGGL((adapt_wave_kernel<T, CTRL, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, cp, (long long)batch, F, (const T *)dt,
-                                      (const T *)y0, (const T *)y1, (const T *)err, (const T *)prev, (const T *)pprev, o);
-           }));
+    TODE_TT(dtype, TODE_CN(c->kind, norm, {
+                const CtrlParams<T> cp = make_ctrl<T>(*c, (double)order);
+                const StepLimits<TT> lim{(TT)c->dt_min, (TT)c->dt_max};
+                if (F < 64)
+                    hipLaunchKernelGGL((adapt_thread_kernel<TT, T, CTRL, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, cp, lim, (long long)batch, F,
+                                       (const TT *)dt, (const T *)y0, (const T *)y1, (const T *)err, (const T *)prev, (const T *)pprev, o);
+                else
+                    hipLaunchKernelGGL((adapt_wave_kernel<TT, T, CTRL, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, cp, lim, (long long)batch, F,
+                                       (const TT *)dt, (const T *)y0, (const T *)y1, (const T *)err, (const T *)prev, (const T *)pprev, o);
+            }));
     return done("tode_adapt_step launch");
 }
 
@@ -646,18 +685,18 @@ int tode_initial_step_a(int32_t dtype, int32_t norm, int64_t batch, int32_t F, d
     if (batch == 0) return TODE_OK;
     if (!t_start || !t_end || !y0 || !f0 || !h0 || !y1 || !t1) return fail(TODE_E_INVALID, "null pointer");
     hipStream_t s = (hipStream_t)stream;
-    TODE_T(dtype, TODE_CN(0, norm, {
-               (void)CTRL;
-               const T at = (T)(float)atol, rt = (T)(float)rtol;
-               if (F < 64)
-                   hipLaunchKernelGGL((initial_a_thread_kernel<T, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, (long long)batch, F, at, rt,
-                                      (const T *)t_start, (const T *)t_end, (const T *)y0, (const T *)f0, (T *)h0);
-               else
-                   hipLaunchKernelGGL((initial_a_wave_kernel<T, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, (long long)batch, F, at, rt,
-                                      (const T *)t_start, (const T *)t_end, (const T *)y0, (const T *)f0, (T *)h0);
-               hipLaunchKernelGGL(initial_probe_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, s, (long long)batch, F, (const T *)t_start,
-                                  (const T *)t_end, (const T *)y0, (const T *)f0, (const T *)h0, (T *)y1, (T *)t1);
-           }));
+    TODE_TT(dtype, TODE_CN(0, norm, {
+                (void)CTRL;
+                const T at = (T)(float)atol, rt = (T)(float)rtol;
+                if (F < 64)
+                    hipLaunchKernelGGL((initial_a_thread_kernel<TT, T, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, (long long)batch, F, at, rt,
+                                       (const TT *)t_start, (const TT *)t_end, (const T *)y0, (const T *)f0, (T *)h0);
+                else
+                    hipLaunchKernelGGL((initial_a_wave_kernel<TT, T, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, (long long)batch, F, at, rt,
+                                       (const TT *)t_start, (const TT *)t_end, (const T *)y0, (const T *)f0, (T *)h0);
+                hipLaunchKernelGGL((initial_probe_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, s, (long long)batch, F, (const TT *)t_start,
+                                   (const TT *)t_end, (const T *)y0, (const T *)f0, (const T *)h0, (T *)y1, (TT *)t1);
+            }));
     return done("tode_initial_step_a launch");
 }
 
@@ -671,16 +710,16 @@ int tode_initial_step_b(int32_t dtype, int32_t kind, int32_t norm, int32_t order
     if (!t_start || !t_end || !y0 || !f0 || !f1 || !h0 || !dt0) return fail(TODE_E_INVALID, "null pointer");
     hipStream_t s = (hipStream_t)stream;
     const double inv_order = 1.0 / (double)order;
-    TODE_T(dtype, TODE_CN(0, norm, {
-               (void)CTRL;
-               const T at = (T)(float)atol, rt = (T)(float)rtol;
-               if (F < 64)
-                   hipLaunchKernelGGL((initial_b_thread_kernel<T, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, kind, inv_order, (long long)batch, F, at,
-                                      rt, (const T *)t_start, (const T *)t_end, (const T *)y0, (const T *)f0, (const T *)f1, (const T *)h0, (T *)dt0);
-               else
-                   hipLaunchKernelGGL((initial_b_wave_kernel<T, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, kind, inv_order, (long long)batch, F, at, rt,
-                                      (const T *)t_start, (const T *)t_end, (const T *)y0, (const T *)f0, (const T *)f1, (const T *)h0, (T *)dt0);
-           }));
+    TODE_TT(dtype, TODE_CN(0, norm, {
+                (void)CTRL;
+                const T at = (T)(float)atol, rt = (T)(float)rtol;
+                if (F < 64)
+                    hipLaunchKernelGGL((initial_b_thread_kernel<TT, T, NORM>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, kind, inv_order, (long long)batch, F,
+                                       at, rt, (const TT *)t_start, (const TT *)t_end, (const T *)y0, (const T *)f0, (const T *)f1, (const T *)h0, (TT *)dt0);
+                else
+                    hipLaunchKernelGGL((initial_b_wave_kernel<TT, T, NORM>), dim3(blocks_for(batch, 4)), dim3(256), 0, s, kind, inv_order, (long long)batch, F,
+                                       at, rt, (const TT *)t_start, (const TT *)t_end, (const T *)y0, (const T *)f0, (const T *)f1, (const T *)h0, (TT *)dt0);
+            }));
     return done("tode_initial_step_b launch");
 }
 
@@ -692,12 +731,12 @@ int tode_quartic_build(int32_t dtype, int32_t method, int64_t batch, int32_t F, 
     if (!dt || !y0 || !y1 || !k || !coeff) return fail(TODE_E_INVALID, "null pointer");
     const dim3 grid(blocks_for(batch * F, 256));
     hipStream_t s = (hipStream_t)stream;
-    TODE_T(dtype, {
+    TODE_TT(dtype, {
         if (method == TODE_TSIT5)
-            hipLaunchKernelGGL((quartic_build_kernel<T, 1>), grid, dim3(256), 0, s, (long long)batch, F, (const T *)dt, (const T *)y0, (const T *)y1,
+            hipLaunchKernelGGL((quartic_build_kernel<TT, T, 1>), grid, dim3(256), 0, s, (long long)batch, F, (const TT *)dt, (const T *)y0, (const T *)y1,
                                (const T *)k, (T *)coeff);
         else
-            hipLaunchKernelGGL((quartic_build_kernel<T, 0>), grid, dim3(256), 0, s, (long long)batch, F, (const T *)dt, (const T *)y0, (const T *)y1,
+            hipLaunchKernelGGL((quartic_build_kernel<TT, T, 0>), grid, dim3(256), 0, s, (long long)batch, F, (const TT *)dt, (const T *)y0, (const T *)y1,
                                (const T *)k, (T *)coeff);
     });
     return done("tode_quartic_build launch");
@@ -708,8 +747,8 @@ int tode_quartic_from_mid(int32_t dtype, int64_t batch, int32_t F, const void *d
     if (int rc = check_common(dtype, batch, F)) return rc;
     if (batch == 0) return TODE_OK;
     if (!dt || !y0 || !y1 || !k_first || !k_last || !y_mid || !coeff) return fail(TODE_E_INVALID, "null pointer");
-    TODE_T(dtype, hipLaunchKernelGGL(quartic_from_mid_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
-                                     (const T *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (const T *)y_mid, (T *)coeff));
+    TODE_TT(dtype, hipLaunchKernelGGL((quartic_from_mid_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch,
+                                      F, (const TT *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (const T *)y_mid, (T *)coeff));
     return done("tode_quartic_from_mid launch");
 }
 
@@ -718,8 +757,8 @@ int tode_cubic_build(int32_t dtype, int64_t batch, int32_t F, const void *dt, co
     if (int rc = check_common(dtype, batch, F)) return rc;
     if (batch == 0) return TODE_OK;
     if (!dt || !y0 || !y1 || !k_first || !k_last || !coeff) return fail(TODE_E_INVALID, "null pointer");
-    TODE_T(dtype, hipLaunchKernelGGL(cubic_build_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
-                                     (const T *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (T *)coeff));
+    TODE_TT(dtype, hipLaunchKernelGGL((cubic_build_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F,
+                                      (const TT *)dt, (const T *)y0, (const T *)y1, (const T *)k_first, (const T *)k_last, (T *)coeff));
     return done("tode_cubic_build launch");
 }
 
@@ -731,8 +770,8 @@ int tode_poly_eval(int32_t dtype, int32_t degree, int64_t batch, int32_t F, int6
     if (count == 0) return TODE_OK;
     if (batch == 0) return fail(TODE_E_INVALID, "evaluation points but an empty batch");
     if (!coeff || !t0 || !t1 || !t || !idx || !out) return fail(TODE_E_INVALID, "null pointer");
-    TODE_T(dtype, hipLaunchKernelGGL(poly_eval_kernel<T>, dim3(blocks_for(count * F, 256)), dim3(256), 0, (hipStream_t)stream, degree, (long long)batch, F,
-                                     (long long)count, (const T *)coeff, (const T *)t0, (const T *)t1, (const T *)t, idx, (T *)out));
+    TODE_TT(dtype, hipLaunchKernelGGL((poly_eval_kernel<TT, T>), dim3(blocks_for(count * F, 256)), dim3(256), 0, (hipStream_t)stream, degree, (long long)batch,
+                                      F, (long long)count, (const T *)coeff, (const TT *)t0, (const TT *)t1, (const TT *)t, idx, (T *)out));
     return done("tode_poly_eval launch");
 }
 
@@ -744,13 +783,13 @@ int tode_poly_eval_masked(int32_t dtype, int32_t degree, int64_t batch, int32_t 
     if (batch == 0 || E == 0) return TODE_OK;
     if (!coeff || !t0 || !t1 || !t_eval || !mask || !ys) return fail(TODE_E_INVALID, "null pointer");
     hipStream_t s = (hipStream_t)stream;
-    TODE_T(dtype, {
+    TODE_TT(dtype, {
         if (F < 64)
-            hipLaunchKernelGGL(poly_eval_masked_thread_kernel<T>, dim3(blocks_for(batch, 256)), dim3(256), 0, s, degree, (long long)batch, F, E,
-                               (const T *)coeff, (const T *)t0, (const T *)t1, (const T *)t_eval, mask, (T *)ys);
+            hipLaunchKernelGGL((poly_eval_masked_thread_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, degree, (long long)batch, F, E,
+                               (const T *)coeff, (const TT *)t0, (const TT *)t1, (const TT *)t_eval, mask, (T *)ys);
         else
-            hipLaunchKernelGGL(poly_eval_masked_block_kernel<T>, dim3((unsigned)batch), dim3(256), 0, s, degree, (long long)batch, F, E, (const T *)coeff,
-                               (const T *)t0, (const T *)t1, (const T *)t_eval, mask, (T *)ys);
+            hipLaunchKernelGGL((poly_eval_masked_block_kernel<TT, T>), dim3((unsigned)batch), dim3(256), 0, s, degree, (long long)batch, F, E, (const T *)coeff,
+                               (const TT *)t0, (const TT *)t1, (const TT *)t_eval, mask, (T *)ys);
     });
     return done("tode_poly_eval_masked launch");
 }
@@ -759,8 +798,8 @@ int tode_select_rows(int32_t dtype, int64_t batch, int32_t width, const uint8_t 
     if (int rc = check_common(dtype, batch, width)) return rc;
     if (batch == 0) return TODE_OK;
     if (!mask || !a || !b || !out) return fail(TODE_E_INVALID, "null pointer");
-    TODE_T(dtype, hipLaunchKernelGGL(select_rows_kernel<T>, dim3(blocks_for(batch * width, 256)), dim3(256), 0, (hipStream_t)stream,
-                                     (long long)batch * width, width, mask, (const T *)a, (const T *)b, (T *)out));
+    TODE_T(data_type(dtype), hipLaunchKernelGGL(select_rows_kernel<T>, dim3(blocks_for(batch * width, 256)), dim3(256), 0, (hipStream_t)stream,
+                                                (long long)batch * width, width, mask, (const T *)a, (const T *)b, (T *)out));
     return done("tode_select_rows launch");
 }
 
@@ -779,12 +818,10 @@ int tode_loop_advance(const tode_loop_args *a, void *stream) {
     if (a->t_out == a->t || a->dt_out == a->dt || a->y_out == a->y || a->y_out == a->y_new)
         return fail(TODE_E_INVALID, "outputs must not alias inputs");
     const long long n = a->batch * a->n_features;
-    TODE_T(a->dtype, {
-        hipLaunchKernelGGL(loop_advance_kernel<T>, dim3(blocks_for(a->batch, 256)), dim3(256), 0, s, *a);
-        // y where to_update (written by the kernel above, same stream)
-        hipLaunchKernelGGL(select_rows_kernel<T>, dim3(blocks_for(n, 256)), dim3(256), 0, s, n, a->n_features, (const uint8_t *)a->to_update,
-                           (const T *)a->y_new, (const T *)a->y, (T *)a->y_out);
-    });
+    // the time side of the bookkeeping, then y where to_update (written by the first kernel, same stream)
+    TODE_T(time_type(a->dtype), hipLaunchKernelGGL(loop_advance_kernel<T>, dim3(blocks_for(a->batch, 256)), dim3(256), 0, s, *a));
+    TODE_T(data_type(a->dtype), hipLaunchKernelGGL(select_rows_kernel<T>, dim3(blocks_for(n, 256)), dim3(256), 0, s, n, a->n_features,
+                                                   (const uint8_t *)a->to_update, (const T *)a->y_new, (const T *)a->y, (T *)a->y_out));
     return done("tode_loop_advance launch");
 }
 
@@ -795,8 +832,9 @@ int tode_loop_begin(int32_t dtype, int64_t batch, int32_t F, int32_t E, const vo
     if (batch == 0) return TODE_OK;
     if (!t_start || !t_end || !y0 || !dt || !dt_out) return fail(TODE_E_INVALID, "null pointer");
     if (E > 0 && (!t_eval || !pending || !ys)) return fail(TODE_E_INVALID, "n_eval > 0 needs t_eval, pending and ys");
-    TODE_T(dtype, hipLaunchKernelGGL(loop_begin_kernel<T>, dim3(blocks_for(batch, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F, E,
-                                     (const T *)t_start, (const T *)t_end, (const T *)t_eval, (const T *)y0, (const T *)dt, (T *)dt_out, pending, (T *)ys));
+    TODE_TT(dtype, hipLaunchKernelGGL((loop_begin_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, (hipStream_t)stream, (long long)batch, F, E,
+                                      (const TT *)t_start, (const TT *)t_end, (const TT *)t_eval, (const T *)y0, (const TT *)dt, (TT *)dt_out, pending,
+                                      (T *)ys));
     return done("tode_loop_begin launch");
 }
 

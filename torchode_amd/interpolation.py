@@ -37,22 +37,22 @@ class _PolynomialInterpolation(LocalInterpolation):
         assert self._coeff.ndim == 3 and self._coeff.shape[0] == self.degree + 1
         self.coefficients = tuple(self._coeff.unbind(0))
 
-    def _check(self, *times):
+    def _code(self, *times) -> int:
         c = self._coeff
         _lib.require_device(c, self.t0, self.t1, *times)
-        if c.dtype not in _lib.DTYPES or any(t.dtype != c.dtype for t in (self.t0, self.t1, *times)):
-            raise NotImplementedError("polynomial evaluation needs time and data in one dtype (float32 or float64)")
+        assert all(t.dtype == self.t0.dtype for t in (self.t1, *times)), "time tensors of different dtypes"
+        return _lib.dtype_code(c.dtype, self.t0.dtype)
 
     def evaluate(self, t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
         """reference interpolation.py:103-106, 172-175"""
-        self._check(t)
+        code = self._code(t)
         c = self._coeff
         _, B, F = c.shape
         t, idx = t.contiguous(), idx.to(torch.long).contiguous()
         t0, t1 = self.t0.contiguous(), self.t1.contiguous()
         out = c.new_empty((t.shape[0], F))
         rc = _lib.load().tode_poly_eval(
-            _lib.DTYPES[c.dtype], self.degree, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
+            code, self.degree, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
             _lib.ptr(idx), _lib.ptr(out), _lib.stream_of(c),
         )  # fmt: skip
         _lib.check(rc, "tode_poly_eval")
@@ -61,13 +61,13 @@ class _PolynomialInterpolation(LocalInterpolation):
     def evaluate_masked(self, t_eval: torch.Tensor, mask: torch.Tensor, ys: torch.Tensor) -> None:
         """``ys[b, e] = p_b(t_eval[b, e])`` wherever ``mask[b, e]`` is set (one byte per entry);
         the index list of reference adjoints.py:227-233 is never materialised."""
-        self._check(t_eval)
+        code = self._code(t_eval)
         c = self._coeff
         _, B, F = c.shape
         assert t_eval.is_contiguous() and mask.is_contiguous() and ys.is_contiguous() and mask.element_size() == 1
         t0, t1 = self.t0.contiguous(), self.t1.contiguous()
         rc = _lib.load().tode_poly_eval_masked(
-            _lib.DTYPES[c.dtype], self.degree, B, F, t_eval.shape[1], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1),
+            code, self.degree, B, F, t_eval.shape[1], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1),
             _lib.ptr(t_eval), _lib.ptr(mask), _lib.ptr(ys), _lib.stream_of(c),
         )  # fmt: skip
         _lib.check(rc, "tode_poly_eval_masked")
@@ -77,10 +77,10 @@ class _PolynomialInterpolation(LocalInterpolation):
 
 
 def _build_args(dt, y0, y1, *more):
+    """Contiguous operands and the dtype code (dt in the time dtype, the rest in the data dtype)."""
     _lib.require_device(dt, y0, y1, *more)
-    if y0.dtype not in _lib.DTYPES or dt.dtype != y0.dtype:
-        raise NotImplementedError("interpolant construction needs time and data in one dtype (float32 or float64)")
-    return [x.contiguous() for x in (dt, y0, y1, *more)]
+    assert all(x.dtype == y0.dtype for x in (y1, *more)), "data tensors of different dtypes"
+    return [_lib.dtype_code(y0.dtype, dt.dtype)] + [x.contiguous() for x in (dt, y0, y1, *more)]
 
 
 class LinearInterpolation(_PolynomialInterpolation):
@@ -89,7 +89,7 @@ class LinearInterpolation(_PolynomialInterpolation):
     degree = 1
 
     def __init__(self, t0: torch.Tensor, dt: torch.Tensor, y0: torch.Tensor, y1: torch.Tensor):
-        super().__init__(t0, t0 + dt, (y0, y1 - y0))
+        super().__init__(t0, t0 + dt, (y0, y1 - y0))  # x is taken over (t0 + dt) - t0
         self.dt = dt
         self.y0 = y0
         self.dy = self.coefficients[1]
@@ -103,11 +103,11 @@ class ThirdOrderPolynomialInterpolation(_PolynomialInterpolation):
     @staticmethod
     def from_k(t0, dt, y0, y1, k):
         """Hermite cubic from the first and last stage derivative (reference interpolation.py:84-106)."""
-        dt_, y0_, y1_, kf, kl = _build_args(dt, y0, y1, k[0], k[-1])
+        code, dt_, y0_, y1_, kf, kl = _build_args(dt, y0, y1, k[0], k[-1])
         B, F = y0_.shape
         coeff = y0_.new_empty((4, B, F))
         rc = _lib.load().tode_cubic_build(
-            _lib.DTYPES[y0_.dtype], B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl),
+            code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl),
             _lib.ptr(coeff), _lib.stream_of(y0_),
         )  # fmt: skip
         _lib.check(rc, "tode_cubic_build")
@@ -123,9 +123,9 @@ class FourthOrderPolynomialInterpolation(_PolynomialInterpolation):
     def from_k(t0, dt, y0, y1, k, b_mid):
         """Quartic through both end points, their derivatives and the mid-point value
         ``y0 + dt * sum_s b_mid[s] k[s]`` (reference interpolation.py:138-170)."""
-        dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+        code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
         S, B, F = k_.shape
-        lib, code, stream = _lib.load(), _lib.DTYPES[y0_.dtype], _lib.stream_of(y0_)
+        lib, stream = _lib.load(), _lib.stream_of(y0_)
         w = [float(x) for x in (b_mid.tolist() if isinstance(b_mid, torch.Tensor) else b_mid)]
         assert len(w) == S <= _lib.MAX_STAGES
         y_mid = torch.empty_like(y0_)
@@ -143,12 +143,12 @@ class FourthOrderPolynomialInterpolation(_PolynomialInterpolation):
     def from_erk_step(method_id: int, t0, dt, y0, y1, k):
         """Dense output of a Dopri5 / Tsit5 step with the pair's own weights, one kernel
         (reference tsit5.py:123-139, dopri5.py:53-60)."""
-        dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+        code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
         S, B, F = k_.shape
         assert S == 7
         coeff = y0_.new_empty((5, B, F))
         rc = _lib.load().tode_quartic_build(
-            _lib.DTYPES[y0_.dtype], method_id, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_), _lib.ptr(coeff),
+            code, method_id, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_), _lib.ptr(coeff),
             _lib.stream_of(y0_),
         )  # fmt: skip
         _lib.check(rc, "tode_quartic_build")

@@ -159,14 +159,13 @@ class ExplicitRungeKutta(SingleStepMethod):
         term_ = term if term is not None else self.term
         assert term_ is not None
         _lib.require_device(y0, t0, dt)
-        if y0.dtype not in _lib.DTYPES or t0.dtype != y0.dtype or dt.dtype != y0.dtype:
-            raise NotImplementedError("the Runge-Kutta kernels need time and data in one dtype (float32 or float64)")
+        assert dt.dtype == t0.dtype, "t and dt of different dtypes"
         tab = state.tableau
         h = tab.host()
         y0, t0, dt = y0.contiguous(), t0.contiguous(), dt.contiguous()
         B, F = y0.shape
         S = h.n_stages
-        lib, code, stream = _lib.load(), _lib.DTYPES[y0.dtype], _lib.stream_of(y0)
+        lib, code, stream = _lib.load(), _lib.dtype_code(y0.dtype, t0.dtype), _lib.stream_of(y0)
 
         vf0 = state.prev_vf1 if tab.fsal and state.prev_vf1 is not None else term_.vf(t0, y0, stats, args)
         k = y0.new_empty((S, B, F))

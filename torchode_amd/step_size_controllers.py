@@ -172,26 +172,25 @@ class AdaptiveStepSizeController(StepSizeController):
     def update_state(self, state, y0, dt, error_ratio, accept):
         raise NotImplementedError()
 
-    def _decide(self, state, dt, *, norm=None, y0=None, y1=None, err=None, limits=True):
+    def _decide(self, state, dt, *, norm=None, y0=None, y1=None, err=None, limits=True, data_dtype=None):
         """Runs the decision kernel: fused with the error norm when ``norm`` is None, from a
         precomputed norm otherwise.  Returns (accept, dt_next, ratio, status, prev, prev_prev)."""
-        ref = dt if y0 is None else y0
         _lib.require_device(dt, norm, y0, y1, err)
-        if ref.dtype not in _lib.DTYPES or dt.dtype != ref.dtype:
-            raise NotImplementedError("the step size controllers need time and data in one dtype (float32 or float64)")
+        data_dtype = data_dtype if y0 is None else y0.dtype
+        code = _lib.dtype_code(data_dtype, dt.dtype)
         dt = dt.contiguous()
         B = dt.shape[0]
         pid = self._kind == _lib.CTRL_PID
-        prev = state.prev_error_ratio.to(ref.dtype).contiguous() if pid else None
-        pprev = state.prev_prev_error_ratio.to(ref.dtype).contiguous() if pid else None
+        prev = state.prev_error_ratio.to(data_dtype).contiguous() if pid else None
+        pprev = state.prev_prev_error_ratio.to(data_dtype).contiguous() if pid else None
         accept = torch.empty(B, dtype=torch.bool, device=dt.device)
-        dt_next, ratio = torch.empty_like(dt), torch.empty_like(dt)
+        dt_next, ratio = torch.empty_like(dt), torch.empty(B, dtype=data_dtype, device=dt.device)
         status = torch.empty(B, dtype=torch.long, device=dt.device)
-        prev_o = torch.empty_like(dt) if pid else None
-        pprev_o = torch.empty_like(dt) if pid else None
+        prev_o = torch.empty_like(ratio) if pid else None
+        pprev_o = torch.empty_like(ratio) if pid else None
         # the limits in force are the state's (reference step_size_controllers.py:406-408)
         c = self.c_struct((_limit(state.dt_min), _limit(state.dt_max)) if limits else (None, None))
-        lib, code, stream = _lib.load(), _lib.DTYPES[ref.dtype], _lib.stream_of(dt)
+        lib, stream = _lib.load(), _lib.stream_of(dt)
         tail = (_lib.ptr(prev), _lib.ptr(pprev), _lib.ptr(accept), _lib.ptr(dt_next), _lib.ptr(ratio), _lib.ptr(status),
                 _lib.ptr(prev_o), _lib.ptr(pprev_o), stream)  # fmt: skip
         if norm is None:
@@ -203,7 +202,7 @@ class AdaptiveStepSizeController(StepSizeController):
             )  # fmt: skip
             _lib.check(rc, "tode_adapt_step")
         else:
-            norm = norm.to(ref.dtype).contiguous()
+            norm = norm.to(data_dtype).contiguous()
             rc = lib.tode_control(code, _lib.C.byref(c), int(state.method_order), B, _lib.ptr(norm), _lib.ptr(dt), *tail)
             _lib.check(rc, "tode_control")
         return accept, dt_next, ratio, status, prev_o, pprev_o
@@ -212,7 +211,7 @@ class AdaptiveStepSizeController(StepSizeController):
         """Growth factor of the step size for a given error ratio, clipped to
         ``[factor_min, factor_max]`` (reference step_size_controllers.py:289-294, 598-621)."""
         ones = torch.ones_like(error_ratio)
-        return self._decide(state, ones, norm=error_ratio, limits=False)[1]
+        return self._decide(state, ones, norm=error_ratio, limits=False, data_dtype=error_ratio.dtype)[1]
 
     # ------------------------------------------------------------------ #
     def init(self, term, problem: InitialValueProblem, method_order: int, dt0, *, stats, args):
@@ -248,7 +247,7 @@ class AdaptiveStepSizeController(StepSizeController):
                 _lib.ptr(scaled), _lib.stream_of(a),
             )  # fmt: skip
             _lib.check(rc, "tode_error_scale")
-            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, norm=self.norm(scaled))
+            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, norm=self.norm(scaled), data_dtype=a.dtype)
         if self._kind == _lib.CTRL_PID and type(self).update_state is PIDController.update_state:
             state = state.update_error_ratios(prev, pprev)  # the decision kernel has already shifted the history
         else:
@@ -266,12 +265,10 @@ class AdaptiveStepSizeController(StepSizeController):
             raise NotImplementedError("automatic selection of the first step needs rms_norm or max_norm; pass dt0 with a custom norm")
         y0, t0, t1 = problem.y0.contiguous(), problem.t_start.contiguous(), problem.t_end.contiguous()
         _lib.require_device(y0, t0, t1)
-        if y0.dtype not in _lib.DTYPES or t0.dtype != y0.dtype:
-            raise NotImplementedError("the step size controllers need time and data in one dtype (float32 or float64)")
         B, F = y0.shape
-        lib, code, stream = _lib.load(), _lib.DTYPES[y0.dtype], _lib.stream_of(y0)
+        lib, code, stream = _lib.load(), _lib.dtype_code(y0.dtype, t0.dtype), _lib.stream_of(y0)
         f0 = term_.vf(t0, y0, stats, args).contiguous()
-        h0, y1, tn = torch.empty_like(t0), torch.empty_like(y0), torch.empty_like(t0)
+        h0, y1, tn = y0.new_empty(B), torch.empty_like(y0), torch.empty_like(t0)
         rc = lib.tode_initial_step_a(
             code, norm, B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0),
             _lib.ptr(h0), _lib.ptr(y1), _lib.ptr(tn), stream,
