@@ -382,6 +382,18 @@ int tode_initial_step_b(int32_t dtype, int32_t kind, int32_t norm, int32_t metho
                         double rtol, const void *t_start, const void *t_end, const void *y0, const void *f0, const void *f1,
                         const void *h0, void *dt0, void *stream);
 
+/* The start step with a user-defined norm, whose evaluations happen between the calls:
+ *   out = v * (1 / (atol + rtol * |y_ref|))                                 (tode_tolerance_scale: the norm's argument)
+ *   d0 = norm(scale(y0)), d1 = norm(scale(f0))  ->  h0, y1, t1              (tode_initial_step_a_norms)
+ *   d2n = norm(scale(f1 - f0))                  ->  dt0                      (tode_initial_step_b_norms)
+ * d0, d1, d2n, h0 are [B] in the data type. */
+int tode_tolerance_scale(int32_t dtype, int64_t batch, int32_t n_features, double atol, double rtol, const void *y_ref, const void *v,
+                         void *out, void *stream);
+int tode_initial_step_a_norms(int32_t dtype, int64_t batch, int32_t n_features, const void *t_start, const void *t_end, const void *y0,
+                              const void *f0, const void *d0, const void *d1, void *h0, void *y1, void *t1, void *stream);
+int tode_initial_step_b_norms(int32_t dtype, int32_t kind, int32_t method_order, int64_t batch, const void *t_start, const void *t_end,
+                              const void *h0, const void *d1, const void *d2n, void *dt0, void *stream);
+
 /* Quartic dense-output coefficients of a Dopri5 / Tsit5 step, lowest power first: coeff [5,B,F]
  * (reference tsit5.py:123-139; dopri5.py:53-60 -> interpolation.py:138-170).  k is [7,B,F]. */
 int tode_quartic_build(int32_t dtype, int32_t method, int64_t batch, int32_t n_features, const void *dt, const void *y0,

@@ -674,3 +674,20 @@ def test_user_defined_method_with_mixed_dtypes():
     sol = to.AutoDiffAdjoint(Euler64(), ctrl).solve(to.InitialValueProblem(y0, t_start, t_end), term)
     assert sol.stats["n_steps"].tolist() == [8, 6] and sol.ys.dtype == torch.float32 and sol.ts.dtype == torch.float64
     assert torch.allclose(sol.ys[:, 0, 0], dev([2.0, 4.0]))
+
+
+def test_user_defined_norm_also_selects_the_first_step():
+    calls = []
+
+    def my_rms(x):  # the RMS norm again, but not the library's function object
+        calls.append(x.shape)
+        return torch.linalg.vector_norm(x / x.shape[1] ** 0.5, dim=1)
+
+    w = to.workloads.make("vdp", batch=128, dtype=torch.float64, device=DEV)
+    problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
+    ctrl = dict(atol=1e-8, rtol=1e-7, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)
+    ref = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(**ctrl)).solve(problem, to.ODETerm(w.f))
+    sol = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(**ctrl, norm=my_rms)).solve(problem, to.ODETerm(w.f))
+    assert len(calls) == 3 + int(ref.stats["n_steps"].max()) and (sol.status == OK).all()
+    assert (sol.stats["n_steps"] == ref.stats["n_steps"]).float().mean() > 0.95
+    assert (sol.ys - ref.ys).abs().max().item() < 1e-6

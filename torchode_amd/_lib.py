@@ -49,6 +49,9 @@ EXPORTS = (
     "tode_adapt_step",
     "tode_initial_step_a",
     "tode_initial_step_b",
+    "tode_tolerance_scale",
+    "tode_initial_step_a_norms",
+    "tode_initial_step_b_norms",
     "tode_quartic_build",
     "tode_quartic_from_mid",
     "tode_cubic_build",
@@ -247,6 +250,9 @@ def load():
             "tode_adapt_step": [I32, CP, I32, I32, I64, I32] + [V] * 13,
             "tode_initial_step_a": [I32, I32, I64, I32, D, D] + [V] * 8,
             "tode_initial_step_b": [I32, I32, I32, I32, I64, I32, D, D] + [V] * 8,
+            "tode_tolerance_scale": [I32, I64, I32, D, D] + [V] * 4,
+            "tode_initial_step_a_norms": [I32, I64, I32] + [V] * 10,
+            "tode_initial_step_b_norms": [I32, I32, I32, I64] + [V] * 7,
             "tode_quartic_build": [I32, I32, I64, I32] + [V] * 6,
             "tode_quartic_from_mid": [I32, I64, I32] + [V] * 8,
             "tode_cubic_build": [I32, I64, I32] + [V] * 7,

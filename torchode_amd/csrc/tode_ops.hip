@@ -249,6 +249,31 @@ __global__ void __launch_bounds__(256) initial_a_wave_kernel(long long batch, in
     }
 }
 
+// The same two halves with the norms supplied by the caller (a user-defined norm): scaling for the
+// norm's argument, h0 from (d0, d1), the final step from (d1, d2n).
+template <typename T>
+__global__ void __launch_bounds__(256) tolerance_scale_kernel(long long n, T atol, T rtol, const T *y_ref, const T *v, T *out) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = v[i] * inv_scale(atol, rtol, y_ref[i]);
+}
+
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) initial_h0_kernel(long long batch, const TT *t_start, const TT *t_end, const T *d0, const T *d1, T *h0_out) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= batch) return;
+    T h0 = (d0[b] < (T)1e-5 || d1[b] < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0[b]) / d1[b];
+    h0_out[b] = tmin(h0, (T)abs_(t_end[b] - t_start[b]));
+}
+
+template <typename TT, typename T>
+__global__ void __launch_bounds__(256) initial_dt_kernel(int kind, double inv_order, long long batch, const TT *t_start, const TT *t_end, const T *h0,
+                                                         const T *d1, const T *d2n, TT *dt0) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= batch) return;
+    const T dir = (t_end[b] > t_start[b]) ? (T)1 : (T)-1;
+    dt0[b] = (TT)initial_finish<T>(kind, inv_order, dir, h0[b], d1[b], d2n[b]);
+}
+
 // y1 = y0 + (direction * h0) * f0, t1 = t_start + direction * h0   (:474-479)
 template <typename TT, typename T>
 __global__ void __launch_bounds__(256) initial_probe_kernel(long long batch, int F, const TT *t_start, const TT *t_end, const T *y0, const T *f0,
@@ -698,6 +723,42 @@ int tode_initial_step_a(int32_t dtype, int32_t norm, int64_t batch, int32_t F, d
                                    (const TT *)t_end, (const T *)y0, (const T *)f0, (const T *)h0, (T *)y1, (TT *)t1);
             }));
     return done("tode_initial_step_a launch");
+}
+
+int tode_tolerance_scale(int32_t dtype, int64_t batch, int32_t F, double atol, double rtol, const void *y_ref, const void *v, void *out, void *stream) {
+    if (int rc = check_common(dtype, batch, F)) return rc;
+    if (batch == 0) return TODE_OK;
+    if (!y_ref || !v || !out) return fail(TODE_E_INVALID, "null pointer");
+    TODE_T(data_type(dtype), hipLaunchKernelGGL(tolerance_scale_kernel<T>, dim3(blocks_for(batch * F, 256)), dim3(256), 0, (hipStream_t)stream,
+                                                (long long)batch * F, (T)(float)atol, (T)(float)rtol, (const T *)y_ref, (const T *)v, (T *)out));
+    return done("tode_tolerance_scale launch");
+}
+
+int tode_initial_step_a_norms(int32_t dtype, int64_t batch, int32_t F, const void *t_start, const void *t_end, const void *y0, const void *f0,
+                              const void *d0, const void *d1, void *h0, void *y1, void *t1, void *stream) {
+    if (int rc = check_common(dtype, batch, F)) return rc;
+    if (batch == 0) return TODE_OK;
+    if (!t_start || !t_end || !y0 || !f0 || !d0 || !d1 || !h0 || !y1 || !t1) return fail(TODE_E_INVALID, "null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    TODE_TT(dtype, {
+        hipLaunchKernelGGL((initial_h0_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, (long long)batch, (const TT *)t_start, (const TT *)t_end,
+                           (const T *)d0, (const T *)d1, (T *)h0);
+        hipLaunchKernelGGL((initial_probe_kernel<TT, T>), dim3(blocks_for(batch * F, 256)), dim3(256), 0, s, (long long)batch, F, (const TT *)t_start,
+                           (const TT *)t_end, (const T *)y0, (const T *)f0, (const T *)h0, (T *)y1, (TT *)t1);
+    });
+    return done("tode_initial_step_a_norms launch");
+}
+
+int tode_initial_step_b_norms(int32_t dtype, int32_t kind, int32_t order, int64_t batch, const void *t_start, const void *t_end, const void *h0,
+                              const void *d1, const void *d2n, void *dt0, void *stream) {
+    if (int rc = check_common(dtype, batch, 1)) return rc;
+    if (kind != TODE_CTRL_INTEGRAL && kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", kind);
+    if (order <= 0) return fail(TODE_E_INVALID, "method order must be positive, got %d", order);
+    if (batch == 0) return TODE_OK;
+    if (!t_start || !t_end || !h0 || !d1 || !d2n || !dt0) return fail(TODE_E_INVALID, "null pointer");
+    TODE_TT(dtype, hipLaunchKernelGGL((initial_dt_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, (hipStream_t)stream, kind, 1.0 / (double)order,
+                                      (long long)batch, (const TT *)t_start, (const TT *)t_end, (const T *)h0, (const T *)d1, (const T *)d2n, (TT *)dt0));
+    return done("tode_initial_step_b_norms launch");
 }
 
 int tode_initial_step_b(int32_t dtype, int32_t kind, int32_t norm, int32_t order, int64_t batch, int32_t F, double atol, double rtol,

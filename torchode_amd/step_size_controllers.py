@@ -261,20 +261,41 @@ class AdaptiveStepSizeController(StepSizeController):
         term_ = term if term is not None else self.term
         assert term_ is not None
         norm = self._norm_id()
-        if norm is None:
-            raise NotImplementedError("automatic selection of the first step needs rms_norm or max_norm; pass dt0 with a custom norm")
         y0, t0, t1 = problem.y0.contiguous(), problem.t_start.contiguous(), problem.t_end.contiguous()
         _lib.require_device(y0, t0, t1)
         B, F = y0.shape
         lib, code, stream = _lib.load(), _lib.dtype_code(y0.dtype, t0.dtype), _lib.stream_of(y0)
-        f0 = term_.vf(t0, y0, stats, args).contiguous()
+        f0 = term_.vf(t0, y0, stats, args).to(y0.dtype).contiguous()
         h0, y1, tn = y0.new_empty(B), torch.empty_like(y0), torch.empty_like(t0)
+        if norm is None:
+            # user-defined norm: its arguments are scaled on the device, it is called three times
+            def scaled_norm(v):
+                out = torch.empty_like(y0)
+                rc = lib.tode_tolerance_scale(code, B, F, self._atol_f, self._rtol_f, _lib.ptr(y0), _lib.ptr(v), _lib.ptr(out), stream)
+                _lib.check(rc, "tode_tolerance_scale")
+                return self.norm(out).to(y0.dtype).contiguous()
+
+            d0, d1 = scaled_norm(y0), scaled_norm(f0)
+            rc = lib.tode_initial_step_a_norms(
+                code, B, F, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(d0), _lib.ptr(d1), _lib.ptr(h0),
+                _lib.ptr(y1), _lib.ptr(tn), stream,
+            )  # fmt: skip
+            _lib.check(rc, "tode_initial_step_a_norms")
+            f1 = term_.vf(tn, y1, stats, args).to(y0.dtype).contiguous()
+            d2n = scaled_norm(f1 - f0)
+            dt0 = torch.empty_like(t0)
+            rc = lib.tode_initial_step_b_norms(
+                code, self._kind, int(method_order), B, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(h0), _lib.ptr(d1), _lib.ptr(d2n),
+                _lib.ptr(dt0), stream,
+            )  # fmt: skip
+            _lib.check(rc, "tode_initial_step_b_norms")
+            return dt0, f0
         rc = lib.tode_initial_step_a(
             code, norm, B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0),
             _lib.ptr(h0), _lib.ptr(y1), _lib.ptr(tn), stream,
         )  # fmt: skip
         _lib.check(rc, "tode_initial_step_a")
-        f1 = term_.vf(tn, y1, stats, args).contiguous()
+        f1 = term_.vf(tn, y1, stats, args).to(y0.dtype).contiguous()
         dt0 = torch.empty_like(t0)
         rc = lib.tode_initial_step_b(
             code, self._kind, norm, int(method_order), B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1),
