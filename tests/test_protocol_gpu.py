@@ -691,3 +691,88 @@ def test_user_defined_norm_also_selects_the_first_step():
     assert len(calls) == 3 + int(ref.stats["n_steps"].max()) and (sol.status == OK).all()
     assert (sol.stats["n_steps"] == ref.stats["n_steps"]).float().mean() > 0.95
     assert (sol.ys - ref.ys).abs().max().item() < 1e-6
+
+
+# ---------------------------------------------------------------------------------------------
+# part five: Heun, Euler, fixed steps and solve_ivp (reference tests/interface_test.py,
+# tests/fixed_step_controller_test.py, tests/adjoint_test.py:98-118, tests/extra_args_test.py)
+# ---------------------------------------------------------------------------------------------
+
+
+def sine_solution(t, *idx):
+    return (-0.5 * t**4 * torch.cos(2 * t) + 0.5 * t**3 * torch.sin(2 * t) + 0.25 * t**2 * torch.cos(2 * t) - t**3 + 2 * t**4 + (torch.pi - 0.25) * t**2)[..., None]
+
+
+def sine_dynamics(t, y):
+    return (2 * y[:, 0] / t + t**4 * torch.sin(2 * t) - t**2 + 4 * t**3)[..., None]
+
+
+def test_solve_ivp_with_defaults():
+    t_eval = dev([[0.1, 0.15, 1.0], [1.0, 1.9, 2.0]])
+    sol = to.solve_ivp(to.ODETerm(sine_dynamics), sine_solution(t_eval[:, 0]), t_eval)
+    assert sol.status.tolist() == [OK, OK]
+    assert sol.ys.cpu().numpy() == pytest.approx(sine_solution(sol.ts).cpu().numpy(), rel=1e-5)
+    # a plain callable, a registered name, a shared 1-d t_eval, a t_span and extra arguments
+    seen = []
+
+    def rhs(t, y, args):
+        seen.append(args)
+        return -y
+
+    y0 = torch.ones((3, 2), device=DEV)
+    sol = to.solve_ivp(rhs, y0, dev([0.5, 1.0]), t_span=(dev(0.0), dev(1.0)), method="heun", args="tag",
+                       controller=to.IntegralController(1e-6, 1e-5))  # fmt: skip
+    assert all(a == "tag" for a in seen) and sol.ys.shape == (3, 2, 2)
+    assert torch.allclose(sol.ys[:, :, 0], torch.exp(-dev([0.5, 1.0])).expand(3, 2), rtol=1e-4)
+    to.register_method("euler", to.Euler)
+    sol = to.solve_ivp(lambda t, y: -y, y0, dev([0.0, 1.0]), method="euler", controller=to.FixedStepController(), dt0=torch.full((3,), 1e-3, device=DEV))
+    assert torch.allclose(sol.ys[:, 1], torch.full((3, 2), 0.999**1000, device=DEV), rtol=1e-4)
+
+
+@pytest.mark.parametrize("method", [to.Dopri5, to.Heun, to.Tsit5])
+def test_fixed_step_controller(method):
+    t_eval = dev([[0.1, 0.7, 2.0], [0.5, 1.2, 4.0]])
+    problem = to.InitialValueProblem(sine_solution(t_eval[:, 0]), t_eval=t_eval)
+    sol = to.AutoDiffAdjoint(method(), to.FixedStepController()).solve(problem, to.ODETerm(sine_dynamics), dt0=dev([0.01, 0.005]))
+    assert sol.status.tolist() == [OK, OK] and sol.ts is t_eval
+    assert sol.ys.cpu().numpy() == pytest.approx(sine_solution(t_eval).cpu().numpy(), rel=1e-2)
+    n = sol.stats["n_steps"].tolist()  # 1.9 / 0.01 and 3.5 / 0.005 steps, plus one where float32 sums fall short of t_end
+    assert n[0] in (190, 191) and n[1] in (700, 701) and sol.stats["n_accepted"].tolist() == n
+
+
+def test_euler_reports_the_end_point_without_evaluation_points():
+    y0 = dev([[0.0], [1.0], [2.0]])
+    t_start, t_end = dev([0.0, 5.0, 2.0]), dev([10.0, 9.0, 4.5])
+    dt = [0.5001, 0.2501, 1.0]
+    term = to.ODETerm(lambda t, y: torch.ones_like(y))
+    sol = to.AutoDiffAdjoint(to.Euler(term), ScriptedController(dt, [dt])).solve(to.InitialValueProblem(y0, t_start, t_end))
+    assert sol.stats["n_steps"].tolist() == [20, 16, 3] and sol.stats["n_initialized"].tolist() == [1, 1, 1]
+    assert torch.allclose(sol.ys[:, 0], y0 + (t_end - t_start)[:, None], rtol=1e-5)
+
+
+@pytest.mark.parametrize("method", [to.Dopri5, to.Heun, to.Tsit5])
+def test_extra_args_reach_the_dynamics(method):
+    static = (0, True, "hello", torch.tensor([0.0, -1.0]))
+    got = []
+
+    def rhs(t, y, args):
+        got.append(args)
+        return torch.ones_like(y)
+
+    term = to.ODETerm(rhs, with_args=True)
+    problem = to.InitialValueProblem(dev([[0.0, 1.0, 2.0]]), t_eval=dev([[0.0, 0.2, 0.6, 1.0]]))
+    sol = to.AutoDiffAdjoint(method(term), to.PIDController(1e-3, 1e-3, 0.0, 1.0, 0.0)).solve(problem, term, args=static)
+    assert got and all(a is static for a in got) and sol.status.tolist() == [OK]
+    assert torch.allclose(sol.ys[0, -1], dev([1.0, 2.0, 3.0]))
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", MIXED, ids=["t64-y32", "t32-y64"])
+def test_heun_keeps_time_and_data_dtypes_apart(time_dtype, data_dtype):
+    def rhs(t, y):
+        assert t.dtype == time_dtype and y.dtype == data_dtype
+        return torch.zeros_like(y)
+
+    y0 = torch.tensor([[0.33, 1.2, -0.4]], dtype=data_dtype, device=DEV)
+    t_eval = torch.tensor([[0.0, 1.77, 3.0]], dtype=time_dtype, device=DEV)
+    sol = to.AutoDiffAdjoint(to.Heun(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0)).solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(rhs))
+    assert sol.stats["n_steps"].item() > 3 and sol.ts.dtype == time_dtype and sol.ys.dtype == data_dtype

@@ -6,16 +6,25 @@ from . import builtin_terms, workloads
 from .adjoints import AutoDiffAdjoint
 from .builtin_terms import LinearDecay, Lorenz63, MLPField, ReactionDiffusion, VanDerPol
 from .problems import InitialValueProblem
-from .single_step_methods import Dopri5, Tsit5
+from .interface import register_method, solve_ivp
+from .single_step_methods import Dopri5, Euler, Heun, Tsit5
 from .solution import Solution
 from .status_codes import Status
 from .step_size_controllers import FixedStepController, IntegralController, PIDController
 from .terms import ODETerm
 
+register_method("heun", Heun)
+register_method("dopri5", Dopri5)
+register_method("tsit5", Tsit5)
+
 __all__ = [
     "AutoDiffAdjoint",
     "InitialValueProblem",
+    "register_method",
+    "solve_ivp",
     "Dopri5",
+    "Euler",
+    "Heun",
     "Tsit5",
     "Solution",
     "Status",

@@ -1,0 +1,53 @@
+"""Forward Euler (mirrors torchode/single_step_methods/euler.py)."""
+from typing import Any, Dict, NamedTuple, Optional
+
+import torch
+
+from .. import _lib
+from ..interpolation import LinearInterpolation
+from ..terms import ODETerm
+from .base import SingleStepMethod, StepResult
+
+
+class LinearInterpolationData(NamedTuple):
+    t0: torch.Tensor
+    dt: torch.Tensor
+    y0: torch.Tensor
+    y1: torch.Tensor
+
+
+class Euler(SingleStepMethod):
+    """``y1 = y0 + dt f(t0, y0)``, no error estimate (a controller then keeps the step size), linear
+    dense output."""
+
+    def __init__(self, term: Optional[ODETerm] = None):
+        super().__init__()
+        self.term = term
+
+    def init(self, term, problem, f0, *, stats: Dict[str, Any], args: Any):
+        return None
+
+    def step(self, term, running, y0, t0, dt, state, *, stats, args):
+        term_ = term if term is not None else self.term
+        assert term_ is not None
+        _lib.require_device(y0, t0, dt)
+        y0, dt = y0.contiguous(), dt.contiguous()
+        B, F = y0.shape
+        k = term_.vf(t0, y0, stats, args).to(y0.dtype).contiguous()
+        y1 = torch.empty_like(y0)
+        one = (_lib.C.c_double * 1)(1.0)
+        rc = _lib.load().tode_erk_stage(
+            _lib.dtype_code(y0.dtype, dt.dtype), B, F, 1, one, 0.0, None, _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(k), _lib.ptr(y1), None,
+            _lib.stream_of(y0),
+        )  # fmt: skip
+        _lib.check(rc, "tode_erk_stage")
+        return StepResult(y1, None), LinearInterpolationData(t0, dt, y0, y1), state, None
+
+    def merge_states(self, accept, current, previous):
+        return None
+
+    def convergence_order(self) -> int:
+        return 1
+
+    def build_interpolation(self, data: LinearInterpolationData):
+        return LinearInterpolation(data.t0, data.dt, data.y0, data.y1)
