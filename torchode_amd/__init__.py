@@ -4,6 +4,7 @@ __version__ = "0.1.0"
 
 from . import builtin_terms, workloads
 from .adjoints import AutoDiffAdjoint
+from .backsolve import BacksolveAdjoint, JointBacksolveAdjoint
 from .builtin_terms import LinearDecay, Lorenz63, MLPField, ReactionDiffusion, VanDerPol
 from .problems import InitialValueProblem
 from .interface import register_method, solve_ivp
@@ -19,6 +20,8 @@ register_method("tsit5", Tsit5)
 
 __all__ = [
     "AutoDiffAdjoint",
+    "BacksolveAdjoint",
+    "JointBacksolveAdjoint",
     "InitialValueProblem",
     "register_method",
     "solve_ivp",

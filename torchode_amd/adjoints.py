@@ -90,8 +90,10 @@ class AutoDiffAdjoint(nn.Module):
             _library_object(m, (Dopri5, Tsit5))
             and _library_object(c, (IntegralController, PIDController))
             and c.fusable
-            and type(term) is ODETerm
-            and "vf" not in vars(term)
+            and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
+            and type(term).vf is ODETerm.vf
+            and type(term).init is ODETerm.init
+            and not any(name in vars(term) for name in ("vf", "init"))
             and problem.data_dtype == problem.time_dtype
             and problem.data_dtype in _lib.DTYPES
         )
