@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the batch-parallel adaptive RK solve loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vdp|lorenz|linear_decay] [--dtype f32|f64]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|f64] [--path auto|per-step]
+                    [--workload vdp|lorenz|linear_decay|reaction_diffusion|mlp]
 
 A "step" is one full solve of the workload's batch (start step, adaptive loop,
 dense output, stats) with inputs resident in HBM.  Prints ONE JSON line.
@@ -36,6 +37,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("lorenz", "torch.float32", 1048576): 1076.1e6,
     # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4363 KiB x 2.000 + 819284 KiB x 1.000) x 1024
     ("reaction_diffusion", "torch.float32", 512): 847.9e6,
+    # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1578 KiB x 2.000 + 20616 KiB x 1.000) x 1024
+    ("mlp", "torch.float32", 4096): 24.34e6,
 }
 
 
@@ -48,6 +51,13 @@ def main():
     ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
     ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument(
+        "--path",
+        default="auto",
+        choices=["auto", "per-step"],
+        help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
+    )
+    ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the baseline's sample is sized to")
     ap.add_argument(
         "--calibration-copy-mib",
         type=int,
@@ -74,7 +84,7 @@ def main():
     ctrl = to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
     solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl)
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
-    term = to.ODETerm(w.f)
+    term = to.ODETerm(w.f if args.path == "auto" else (lambda t, y, f=w.f: f(t, y)))
 
     if args.calibration_copy_mib:
         src = torch.ones(args.calibration_copy_mib * 2**20 // 4, dtype=torch.float32, device="cuda")
@@ -109,7 +119,9 @@ def main():
     except RuntimeError:
         # no whole-solve kernel for this workload: the solve is a sequence of per-call kernels
         # around the torch right-hand side, and the figure below is over the whole solve
-        kernel_name, kernel_s = "protocol path (one kernel per protocol call + torch right-hand side)", wall
+        per_step = args.path == "per-step" and F < 64
+        kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
+        kernel_s = wall
     _lib.set_kernel_timing(False)
     achieved = algo_bytes / kernel_s / 1e9
     roofline = {
@@ -125,6 +137,11 @@ def main():
         "bytes_dense_per_sample": w.bytes_dense,
         "kernel_ms": kernel_s * 1e3,
     }
+    if args.path == "per-step":
+        # with an external f the stages go through HBM: per sample-step the stage kernels read 27 and
+        # write 6 rows, f reads and writes a row six times, the finishing kernel reads 9 and writes 2
+        sd = w.y0.element_size()
+        roofline["own_compulsory_bytes_per_launch"] = sample_steps * (56 * F * sd + w.bytes_step - 4 * F * sd)
     if w.name == "mlp":
         # dense contractions: the matrix cores bound this workload, not HBM.  Per evaluation of f and
         # sample 2*(65*256 + 256*64) flops; a sample evaluates f twice for the first step size and six
@@ -185,15 +202,23 @@ def cpu_baselines(args, w, sol):
     cores = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
     B = w.y0.shape[0]
-    n = min(B, {"reaction_diffusion": 32, "mlp": 1024}.get(w.name, 8192))
-    wc = to.workloads.make(w.name, batch=n, dtype=w.y0.dtype)
-    ctrl = torch_loop.Controller(**wc.controller)
-    ww = to.workloads.make(w.name, batch=min(256, max(n // 4, 1)), dtype=w.y0.dtype)  # warm up
-    torch_loop.solve(ww.f, ww.y0, ww.t_eval, method=ww.method, controller=ctrl)
+    ww = to.workloads.make(w.name, batch=min(B, {"reaction_diffusion": 8, "mlp": 256}.get(w.name, 2048)), dtype=w.y0.dtype)
+    ctrl = torch_loop.Controller(**ww.controller)
+    torch_loop.solve(ww.f, ww.y0, ww.t_eval, method=ww.method, controller=ctrl)  # warm up
     t0 = time.perf_counter()
-    ref = torch_loop.solve(wc.f, wc.y0, wc.t_eval, method=wc.method, controller=ctrl)
-    t_torch = time.perf_counter() - t0
-    steps_n = int(ref["n_steps"].sum())
+    torch_loop.solve(ww.f, ww.y0, ww.t_eval, method=ww.method, controller=ctrl)
+    per_sample = (time.perf_counter() - t0) / ww.y0.shape[0]
+    # the loop's cost per iteration has a fixed part, so small batches overestimate the cost per
+    # sample: the sample below is sized generously and the time actually taken is reported
+    n = int(min(B, max(ww.y0.shape[0], 2 * args.cpu_baseline_seconds / per_sample)))
+    wc = to.workloads.make(w.name, batch=n, dtype=w.y0.dtype)
+    t_torch, steps_n, solves = 0.0, 0, 0
+    while solves == 0 or (t_torch < 0.8 * args.cpu_baseline_seconds and solves < 64):  # whole workload too short: repeat it
+        t0 = time.perf_counter()
+        ref = torch_loop.solve(wc.f, wc.y0, wc.t_eval, method=wc.method, controller=ctrl)
+        t_torch += time.perf_counter() - t0
+        steps_n += int(ref["n_steps"].sum())
+        solves += 1
 
     first = {
         "cpu_baseline": {
@@ -201,14 +226,14 @@ def cpu_baselines(args, w, sol):
             "unit": "sample-steps/s",
             "cores": cores,
             "kind": "port",
-            "sample": f"first {n} samples of the workload, one eager solve of the ATen-op restatement (torch {torch.__version__})",
+            "sample": f"first {n} of {B} samples of the workload, {solves} eager solve(s) of the ATen-op restatement (torch {torch.__version__})",
             "seconds": t_torch,
         }
     }
     if w.name not in c_oracle.TERMS:
         return first
     name = w.name
-    nc = min(B, 65536)
+    nc = min(B, 262144)
     wc2 = to.workloads.make(w.name, batch=nc, dtype=w.y0.dtype)
     cfg = c_oracle.make_config(method=wc2.method, term=name, nthreads=cores, **wc2.controller)
     c_oracle.solve(cfg, ww.f.builtin_params(), ww.y0, ww.t_eval)
@@ -222,7 +247,7 @@ def cpu_baselines(args, w, sol):
             "unit": "sample-steps/s",
             "cores": cores,
             "kind": "port",
-            "sample": f"first {nc} samples, one solve of the scalar C oracle (OpenMP over samples)",
+            "sample": f"first {nc} of {B} samples, one solve of the scalar C oracle (OpenMP over samples)",
             "seconds": t_c,
         },
     }

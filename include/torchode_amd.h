@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 5
+#define TODE_ABI_VERSION 6
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -185,6 +185,23 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
  */
 int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                             int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream);
+
+/*
+ * tode_solve_builtin_fast for a caller that needs the flag block on the host at
+ * once, as the reference's loop does (its stats["n_f_evals"] is a CPU tensor,
+ * terms.py:41-63, and adjoints.py:197-201 synchronises on the loop's state):
+ * the same kernels, but `args->flags` is not used (may be null).  The kernel
+ * works on flag words the library owns (allocated once per device, on the
+ * first call), its last workgroup stores them into pinned host memory, and
+ * this call returns when they have arrived there, with the TODE_FLAG_WORDS
+ * values in the host array `flags_out`.  That saves the launch that resets the
+ * flag block and the device-to-host copy.  ys and the four stat arrays are
+ * complete in stream order as before (here: when the call returns).  Safe to
+ * call from several host threads and on several streams at once.
+ */
+int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
+                                 int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream,
+                                 int32_t *flags_out);
 
 /* ------------------------------------------------------------------------- */
 /* Per-step kernels around a right-hand side that lives outside the library   */

@@ -308,3 +308,75 @@ def test_gpu_matches_golden_fixture(path, fast):
     ys = sol.ys.cpu()
     assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
     assert float(ys.double().abs().max()).hex() == g["ys_max_abs"]
+
+
+# ---------------------------------------------------------------------------------------------
+# the two forms of the fast entry point, called through the C ABI directly
+# ---------------------------------------------------------------------------------------------
+
+
+def _fast_call(w, sync: bool):
+    """One call of tode_solve_builtin_fast[_sync] on workload `w` (tensors on the GPU)."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    B, F = w.y0.shape
+    E = w.t_eval.shape[1]
+    params = w.f.builtin_params()
+    ys = torch.full((B, E, F), float("nan"), dtype=w.y0.dtype, device="cuda")
+    out = torch.full((4, B), -7, dtype=torch.int64, device="cuda")
+    spec = dict(w.controller)
+    kind = spec.pop("kind")
+    ctrl = (to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)).c_struct()
+    a = _lib.SolveArgs()
+    a.dtype, a.method, a.term = _lib.DTYPES[w.y0.dtype], {"dopri5": 0, "tsit5": 1}[w.method], w.f.builtin_kind
+    a.n_features, a.n_eval, a.n_params, a.batch, a.max_steps, a.iteration_cap = F, E, params.shape[1], B, -1, -1
+    scal = list(getattr(w.f, "builtin_scalars", lambda: ())()) + [0.0] * 4
+    a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
+    a.y0, a.t_start, a.t_end, a.t_eval = w.y0.data_ptr(), w.t_eval[:, 0].data_ptr(), w.t_eval[:, -1].data_ptr(), w.t_eval.data_ptr()
+    a.t_start_stride = a.t_end_stride = E
+    a.params, a.ys = params.data_ptr(), ys.data_ptr()
+    stream = _lib.stream_of(w.y0)
+    if sync:
+        fl = (_lib.C.c_int32 * _lib.FLAG_WORDS)(-1, -1, -1, -1)
+        rc = lib.tode_solve_builtin_fast_sync(_lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream, fl)
+        flags = list(fl)  # no synchronisation of ours: the call itself has waited for the flags
+    else:
+        dev_flags = torch.full((_lib.FLAG_WORDS,), -1, dtype=torch.int32, device="cuda")
+        a.flags = dev_flags.data_ptr()
+        rc = lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream)
+        flags = dev_flags.tolist()
+    _lib.check(rc, "tode_solve_builtin_fast")
+    torch.cuda.synchronize()
+    return ys, out, flags
+
+
+@pytest.mark.parametrize("name,dtype,sizes", [("vdp", F32, (5000, 100, 64)), ("vdp", F64, (777, 3000)), ("lorenz", F32, (300000, 4096, 1))])
+def test_fast_entry_point_with_flags_on_the_host_equals_the_plain_one(name, dtype, sizes):
+    for batch in sizes:  # in a row: the flag words the library keeps must come back to their start values
+        w = to.workloads.make(name, batch=batch, dtype=dtype, device="cuda")
+        ys_a, out_a, flags_a = _fast_call(w, sync=False)
+        ys_b, out_b, flags_b = _fast_call(w, sync=True)
+        assert flags_a == flags_b and flags_a[0] == int(out_a[0].max()) and flags_a[3] == 0
+        assert torch.equal(ys_a, ys_b) and torch.equal(out_a, out_b) and not torch.isnan(ys_a).any()
+        if batch <= 5000:
+            wc = to.workloads.make(name, batch=batch, dtype=dtype)
+            ref = c_oracle_solve(wc.f, wc.y0, wc.t_eval, wc.method, wc.controller)
+            assert torch.equal(ys_b.cpu(), ref["ys"]) and torch.equal(out_b[0].cpu(), ref["n_steps"])
+
+
+def test_flags_on_the_host_over_more_calls_than_there_are_slots_and_when_the_batch_needs_the_general_kernel():
+    w = to.workloads.make("vdp", batch=200, dtype=F32, device="cuda")
+    first = _fast_call(w, sync=True)
+    for _ in range(150):
+        ys, out, flags = _fast_call(w, sync=True)
+        assert flags == first[2]
+    assert torch.equal(ys, first[0]) and torch.equal(out, first[1])
+    # a t_eval row that is not monotone: the kernel asks for the general one; the next call is clean again
+    bad = to.workloads.make("vdp", batch=200, dtype=F32, device="cuda")
+    bad.t_eval[17, 5] = bad.t_eval[17, 3]
+    assert _fast_call(bad, sync=True)[2][3] == 1 and _fast_call(bad, sync=False)[2][3] == 1
+    assert _fast_call(w, sync=True)[2] == first[2]
+    # empty batch: nothing is launched, the start values come back
+    empty = w._replace(f=to.VanDerPol(w.f.mu[:0]), y0=w.y0[:0], t_eval=w.t_eval[:0])
+    assert _fast_call(empty, sync=True)[2] == [0, 2**31 - 1, 0, 0]

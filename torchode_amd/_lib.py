@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -31,6 +31,7 @@ EXPORTS = (
     "tode_last_error",
     "tode_solve_builtin",
     "tode_solve_builtin_fast",
+    "tode_solve_builtin_fast_sync",
     "tode_step_begin",
     "tode_step_stage",
     "tode_step_finish",
@@ -220,6 +221,8 @@ def load():
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
         lib.tode_solve_builtin_fast.restype = C.c_int
         lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
+        lib.tode_solve_builtin_fast_sync.restype = C.c_int
+        lib.tode_solve_builtin_fast_sync.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.POINTER(C.c_int32)]
         lib.tode_step_begin.restype = C.c_int
         lib.tode_step_begin.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p, C.c_int, C.c_void_p]
         lib.tode_step_stage.restype = C.c_int

@@ -26,10 +26,13 @@ def _f_evals(count: int, batch: int) -> torch.Tensor:
     return torch.tensor(count, dtype=torch.long).expand(batch)
 
 
+_PROTOCOL_NAME_SET = frozenset(_PROTOCOL_NAMES)
+
+
 def _library_object(obj, classes) -> bool:
     """True if ``obj`` is exactly one of the library's classes with no protocol method replaced on
     the instance; only then may a fused kernel stand in for the calls the loop would make."""
-    return type(obj) in classes and not any(name in vars(obj) for name in _PROTOCOL_NAMES)
+    return type(obj) in classes and _PROTOCOL_NAME_SET.isdisjoint(vars(obj))
 
 
 class AutoDiffAdjoint(nn.Module):
@@ -69,8 +72,12 @@ class AutoDiffAdjoint(nn.Module):
         term_ = term if term is not None else getattr(self.step_method, "term", None)
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
-        if torch.is_grad_enabled() and any(
-            t is not None and t.requires_grad for t in (problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
+        if torch.is_grad_enabled() and (
+            problem.y0.requires_grad
+            or problem.t_start.requires_grad
+            or problem.t_end.requires_grad
+            or (problem.t_eval is not None and problem.t_eval.requires_grad)
+            or (dt0 is not None and dt0.requires_grad)
         ):
             raise RuntimeError(
                 "torchode_amd's solve loop is forward-only; call it under torch.no_grad() or detach the inputs"
@@ -93,7 +100,8 @@ class AutoDiffAdjoint(nn.Module):
             and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
             and type(term).vf is ODETerm.vf
             and type(term).init is ODETerm.init
-            and not any(name in vars(term) for name in ("vf", "init"))
+            and "vf" not in vars(term)
+            and "init" not in vars(term)
             and problem.data_dtype == problem.time_dtype
             and problem.data_dtype in _lib.DTYPES
         )
@@ -334,28 +342,19 @@ class AutoDiffAdjoint(nn.Module):
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
         y_idle = torch.empty((B, F), dtype=dtype, device=dev) if E == 0 else None
-        flags = torch.empty(_lib.FLAG_WORDS, dtype=torch.int32, device=dev)
         ctrl = self.step_size_controller.c_struct()
         stream = _lib.stream_of(y0)
         scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
 
-        a = _lib.SolveArgs()
-        a.dtype, a.method, a.term = _lib.DTYPES[dtype], self.step_method.method_id, f.builtin_kind
-        a.n_features, a.n_eval, a.n_params, a.batch = F, E, params.shape[1], B
-        a.max_steps = -1 if self.max_steps is None else int(self.max_steps)
-        a.iteration_cap = -1
-        a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
-        a.y0, a.t_start, a.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
-        a.t_start_stride, a.t_end_stride = t_start.stride(0), t_end.stride(0)
-        a.t_eval = None if t_eval is None else t_eval.data_ptr()
-        a.dt0 = None if dt0_ is None else dt0_.data_ptr()
-        a.params = params.data_ptr() if params.numel() else None
-        a.shared_params = None if shared is None else shared.data_ptr()
-        a.n_shared_params = 0 if shared is None else shared.numel()
-        a.ys = ys.data_ptr()
-        a.y_idle = None if y_idle is None else y_idle.data_ptr()
-        a.pending = None
-        a.flags = flags.data_ptr()
+        a = _lib.SolveArgs(  # positional, in the order of struct tode_solve_args
+            _lib.DTYPES[dtype], self.step_method.method_id, f.builtin_kind, F, E, params.shape[1], B,
+            -1 if self.max_steps is None else int(self.max_steps), -1, (_lib.C.c_double * 4)(*scal[:4]),
+            y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0),
+            None if t_eval is None else t_eval.data_ptr(), None if dt0_ is None else dt0_.data_ptr(),
+            params.data_ptr() if params.numel() else None,
+            None if shared is None else shared.data_ptr(), 0 if shared is None else shared.numel(),
+            ys.data_ptr(), None if y_idle is None else y_idle.data_ptr(),
+        )  # fmt: skip  (pending, the five int32 outputs and flags stay null: set below where they are used)
 
         stats: Dict[str, Any] = {}
         n_init_evals = 2 if dt0 is None else 1
@@ -377,20 +376,24 @@ class AutoDiffAdjoint(nn.Module):
                 return None  # no whole-solve kernel for this case: the caller takes the protocol path
         if fast_ok:
             out = torch.empty((4, B), dtype=torch.int64, device=dev)
-            rc = lib.tode_solve_builtin_fast(
-                _lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream
-            )
-            _lib.check(rc, "tode_solve_builtin_fast")
-            fl = flags.tolist()  # the one host synchronisation of the solve
+            o0, row = out.data_ptr(), 8 * B
+            fl = (_lib.C.c_int32 * _lib.FLAG_WORDS)()
+            rc = lib.tode_solve_builtin_fast_sync(
+                _lib.C.byref(a), _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, stream, fl
+            )  # returns when the kernel has published the flag block: the one host synchronisation of the solve
+            if rc:
+                _lib.check(rc, "tode_solve_builtin_fast_sync")
             if fl[_lib.FLAG_NEEDS_GENERAL] and not has_general:
                 return None
             if not fl[_lib.FLAG_NEEDS_GENERAL]:
                 if term.with_stats:
                     last = fl[_lib.FLAG_MAX_ITERATIONS]
                     stats["n_f_evals"] = _f_evals(n_init_evals + 6 * last, B)
-                stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
-                return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+                stats["n_steps"], stats["n_accepted"], stats["n_initialized"], status = out.unbind(0)
+                return Solution(ts=ts, ys=ys, stats=stats, status=status)
 
+        flags = torch.empty(_lib.FLAG_WORDS, dtype=torch.int32, device=dev)
+        a.flags = flags.data_ptr()
         counters = torch.empty((5, B), dtype=torch.int32, device=dev)
         a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
 

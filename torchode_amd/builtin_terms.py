@@ -138,5 +138,11 @@ class MLPField(BuiltinTerm):
         return torch.empty((0, 0), dtype=self.W1.dtype, device=self.W1.device)
 
     def builtin_shared(self) -> torch.Tensor:
-        """W1 | b1 | W2 | b2, row-major and concatenated: the layout the whole-solve kernel reads."""
-        return torch.cat([self.W1.reshape(-1), self.b1.reshape(-1), self.W2.reshape(-1), self.b2.reshape(-1)]).contiguous()
+        """W1 | b1 | W2 | b2, row-major and concatenated: the layout the whole-solve kernel reads.
+        Packed once and again whenever a weight tensor has been replaced or written in place."""
+        weights = (self.W1, self.b1, self.W2, self.b2)
+        key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights)
+        if getattr(self, "_packed_key", None) != key:
+            self._packed = torch.cat([w.reshape(-1) for w in weights]).contiguous()
+            self._packed_key = key
+        return self._packed

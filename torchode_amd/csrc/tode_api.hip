@@ -1,8 +1,12 @@
 // extern "C" surface of libtorchode_amd: argument validation, error reporting
 // and the small finalisation kernel.
 #include <hip/hip_runtime.h>
+#include <limits.h>
 #include <stdarg.h>
 #include <stdio.h>
+
+#include <atomic>
+#include <mutex>
 
 #include "../../include/torchode_amd.h"
 #include "tode_internal.h"
@@ -45,6 +49,78 @@ void timing_after(hipStream_t s) {
     if (!g_timing) return;
     (void)hipEventRecord(g_ev[1], s);
     g_timed = true;
+}
+
+// ---- flag slots of tode_solve_builtin_fast_sync -------------------------------------------------
+// Per device: FLAG_SLOTS blocks of FLAG_SLOT_WORDS int32 in device memory (four flag words at their
+// start values and a count of finished workgroups, put back by the kernel that used them) and as
+// many in pinned, coherent host memory (the published flags and a sequence number).  A call takes a
+// free slot, so calls from several host threads or on several streams do not share words.
+constexpr int FLAG_SLOTS = 64, FLAG_SLOT_WORDS = 8, FLAG_DEVICES = 64;
+
+struct FlagPool {
+    int32_t *dev = nullptr;
+    int32_t *host = nullptr;
+    int32_t *host_as_seen_by_device = nullptr;
+    std::atomic<int> busy[FLAG_SLOTS];
+    int32_t sequence[FLAG_SLOTS];
+    std::atomic<unsigned> next;
+};
+static FlagPool g_flag_pools[FLAG_DEVICES];  // static storage: zero-initialised
+static std::mutex g_flag_mutex;
+static thread_local const FlagTarget *g_flag_target = nullptr;
+
+const FlagTarget *flag_target() { return g_flag_target; }
+
+static int flag_pool(hipStream_t s, FlagPool **out) {
+    int device = 0;
+    int rc = check_hip(s ? hipStreamGetDevice(s, &device) : hipGetDevice(&device), "device of the stream");
+    if (rc) return rc;
+    if (device < 0 || device >= FLAG_DEVICES) return fail(TODE_E_UNSUPPORTED, "device index %d", device);
+    FlagPool &pool = g_flag_pools[device];
+    std::lock_guard<std::mutex> lock(g_flag_mutex);
+    if (!pool.dev) {
+        int current = 0;
+        if ((rc = check_hip(hipGetDevice(&current), "hipGetDevice"))) return rc;
+        if (current != device && (rc = check_hip(hipSetDevice(device), "hipSetDevice"))) return rc;
+        const size_t bytes = (size_t)FLAG_SLOTS * FLAG_SLOT_WORDS * sizeof(int32_t);
+        int32_t start[FLAG_SLOTS * FLAG_SLOT_WORDS] = {};
+        for (int i = 0; i < FLAG_SLOTS; ++i) start[i * FLAG_SLOT_WORDS + TODE_FLAG_FIRST_FAILURE] = INT_MAX;
+        int32_t *dev = nullptr, *host = nullptr, *host_dev = nullptr;
+        hipError_t err = hipMalloc((void **)&dev, bytes);
+        if (err == hipSuccess) err = hipMemcpy(dev, start, bytes, hipMemcpyHostToDevice);
+        if (err == hipSuccess) err = hipHostMalloc((void **)&host, bytes, hipHostMallocPortable | hipHostMallocMapped | hipHostMallocCoherent);
+        if (err == hipSuccess) err = hipHostGetDevicePointer((void **)&host_dev, host, 0);
+        if (current != device) (void)hipSetDevice(current);
+        if (err != hipSuccess) {
+            if (dev) (void)hipFree(dev);
+            if (host) (void)hipHostFree(host);
+            return check_hip(err, "allocating the flag slots");
+        }
+        for (int i = 0; i < FLAG_SLOTS * FLAG_SLOT_WORDS; ++i) host[i] = 0;
+        pool.host = host;
+        pool.host_as_seen_by_device = host_dev;
+        pool.dev = dev;
+    }
+    *out = &pool;
+    return TODE_OK;
+}
+
+// Spins on the slot's sequence word; looks at the stream now and then, so that a kernel that never
+// ran (or a failed device) ends the wait with an error instead of a hang.
+static int wait_for_flags(const int32_t *slot, int32_t sequence, hipStream_t s) {
+    for (unsigned spin = 1;; ++spin) {
+        if (__atomic_load_n(&slot[TODE_FLAG_WORDS], __ATOMIC_ACQUIRE) == sequence) return TODE_OK;
+        if ((spin & 0x3FFF) == 0) {
+            const hipError_t q = hipStreamQuery(s);
+            if (q == hipSuccess) {
+                if (__atomic_load_n(&slot[TODE_FLAG_WORDS], __ATOMIC_ACQUIRE) == sequence) return TODE_OK;
+                return fail(TODE_E_HIP, "the stream is idle but the solve kernel has not published its flags");
+            }
+            if (q != hipErrorNotReady) return check_hip(q, "hipStreamQuery while waiting for the solve kernel");
+        }
+        __builtin_ia32_pause();
+    }
 }
 
 template <typename T>
@@ -151,6 +227,45 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     }
     if (a->dtype == TODE_F32) return solve_fast_f32(*a, *c, ns, na, ni, st, s);
     return solve_fast_f64(*a, *c, ns, na, ni, st, s);
+}
+
+int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,
+                                 int64_t *st, void *stream, int32_t *flags_out) {
+    using namespace tode;
+    if (!a || !c || !flags_out) return fail(TODE_E_INVALID, "null argument");
+    hipStream_t s = (hipStream_t)stream;
+    FlagPool *pool = nullptr;
+    int rc = flag_pool(s, &pool);
+    if (rc) return rc;
+    int slot = -1;
+    const unsigned first = pool->next.fetch_add(1, std::memory_order_relaxed);
+    for (int i = 0; i < FLAG_SLOTS && slot < 0; ++i) {
+        const int candidate = (int)((first + i) % FLAG_SLOTS);
+        if (pool->busy[candidate].exchange(1, std::memory_order_acquire) == 0) slot = candidate;
+    }
+    if (slot < 0) return fail(TODE_E_UNSUPPORTED, "all %d flag slots of this device are in use by calls that have not returned", FLAG_SLOTS);
+
+    // sequence numbers 1, 2, ... INT_MAX, 1, ...: never the 0 the host words start with
+    const int32_t sequence = pool->sequence[slot] = pool->sequence[slot] == INT_MAX ? 1 : pool->sequence[slot] + 1;
+    const FlagTarget target = {pool->dev + slot * FLAG_SLOT_WORDS, pool->host_as_seen_by_device + slot * FLAG_SLOT_WORDS, sequence};
+    tode_solve_args b = *a;
+    b.flags = target.dev;
+    g_flag_target = &target;
+    rc = tode_solve_builtin_fast(&b, c, ns, na, ni, st, stream);
+    g_flag_target = nullptr;
+    if (rc == TODE_OK && a->batch == 0) {  // nothing was launched
+        flags_out[TODE_FLAG_MAX_ITERATIONS] = 0;
+        flags_out[TODE_FLAG_FIRST_FAILURE] = INT_MAX;
+        flags_out[TODE_FLAG_NON_MONOTONE] = flags_out[TODE_FLAG_NEEDS_GENERAL] = 0;
+    } else if (rc == TODE_OK) {
+        const int32_t *host = pool->host + slot * FLAG_SLOT_WORDS;
+        rc = wait_for_flags(host, sequence, s);
+        if (rc == TODE_OK)
+            for (int i = 0; i < TODE_FLAG_WORDS; ++i) flags_out[i] = host[i];
+    }
+    // (after a failed wait the slot's words may be anything: the slot stays out of use)
+    if (rc == TODE_OK || rc == TODE_E_INVALID || rc == TODE_E_UNSUPPORTED) pool->busy[slot].store(0, std::memory_order_release);
+    return rc;
 }
 
 int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,

@@ -251,6 +251,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         if (my_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], my_steps);
         if (my_bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
     }
+    publish_flags(p);
 }
 
 // LDS bytes per workgroup: evaluation times [E][64], plus the staged output [E*F][65].
@@ -262,7 +263,7 @@ template <typename T, int METHOD, int CTRL, typename Term>
 static int launch_fast(const tode_solve_args &a, const tode_controller &c, const FastOut<T> &o, hipStream_t stream) {
     SolveParams<T> p = make_params<T>(a, c);
     const long long blocks = (a.batch + 63) / 64;
-    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    reset_flags(a.flags, stream);
     if (blocks == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
     // Occupancy target: enough workgroups per CU to give every SIMD its share of the batch, up
     // to 4 per SIMD; LDS (160 KiB per CU) is spent on staging only while that target holds.

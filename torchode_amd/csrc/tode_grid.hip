@@ -262,11 +262,12 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
         if (n_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], n_steps);
         if (bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
     }
+    publish_flags(p);
 }
 
 template <int METHOD, int CTRL, int N> static int launch_grid(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t stream) {
     SolveParams<float> p = make_params<float>(a, c);
-    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
     const size_t lds = (size_t)a.n_eval * sizeof(float);
     timing_before(stream, "tode::solve_grid_kernel");

@@ -27,6 +27,16 @@ int fail(int code, const char *fmt, ...);
 // Maps a HIP error to TODE_E_HIP (recording its string) or returns TODE_OK.
 int check_hip(hipError_t err, const char *what);
 
+// Set on the calling thread while tode_solve_builtin_fast_sync runs: the solve kernel then works on
+// the library's own, self-resetting flag words `dev` (no reset launch in front of it) and its last
+// workgroup stores the result, followed by `sequence`, into the pinned host words `host`.
+struct FlagTarget {
+    int32_t *dev;
+    int32_t *host;
+    int32_t sequence;
+};
+const FlagTarget *flag_target();
+
 // Event pair around the solve kernel, active only while timing is enabled on this thread.
 void timing_before(hipStream_t s, const char *kernel_name);
 void timing_after(hipStream_t s);

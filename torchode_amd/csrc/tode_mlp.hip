@@ -352,11 +352,12 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
         if (most > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], most);
         if (bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
     }
+    publish_flags(p);
 }
 
 template <int METHOD, int CTRL> static int launch_mlp(const tode_solve_args &a, const tode_controller &c, const MlpOut &o, hipStream_t stream) {
     SolveParams<float> p = make_params<float>(a, c);
-    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
     const size_t lds = (size_t)MLP_TILE * a.n_eval * sizeof(float);
     const unsigned blocks = (unsigned)((a.batch + MLP_TILE - 1) / MLP_TILE);

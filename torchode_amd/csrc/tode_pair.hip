@@ -270,6 +270,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
         for (int off = 32; off > 0; off >>= 1) my_bail = max(my_bail, __shfl_xor(my_bail, off));
         if (lane == 0 && my_bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
     }
+    publish_flags(p);
 }
 
 template <typename T, int METHOD, int CTRL, typename Term>
@@ -288,7 +289,7 @@ static int launch_pair(const tode_solve_args &a, const tode_controller &c, const
     SolveParams<T> p = make_params<T>(a, c);
     const int nhist = CTRL == 0 ? 0 : (p.cp.skip3 ? 1 : 2);
     const dim3 grid((unsigned)blocks), block(128);
-    hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
+    reset_flags(a.flags, stream);
     timing_before(stream, "tode::solve_pair_kernel");
 #define TODE_PAIR_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_pair_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
     if (nhist == 0) {

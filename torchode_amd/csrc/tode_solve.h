@@ -74,6 +74,8 @@ template <typename T> struct SolveParams {
     T *ys, *y_idle;
     uint8_t *pending;
     int32_t *n_steps, *n_accepted, *n_initialized, *status_last, *status_idle, *flags;
+    int32_t *host_flags;  // pinned host words the last workgroup publishes the flags to, or null
+    int32_t sequence;     // written behind them, so that the host sees when they have arrived
     long long batch, ts_stride, te_stride;
     int n_eval;
     int max_steps;  // INT_MAX: unlimited
@@ -201,7 +203,10 @@ template <typename T> static SolveParams<T> make_params(const tode_solve_args &a
     p.n_initialized = a.n_initialized;
     p.status_last = a.status_last;
     p.status_idle = a.status_idle;
-    p.flags = a.flags;
+    const FlagTarget *target = flag_target();
+    p.flags = target ? target->dev : a.flags;
+    p.host_flags = target ? target->host : nullptr;
+    p.sequence = target ? target->sequence : 0;
     p.batch = a.batch;
     p.ts_stride = a.t_start_stride;
     p.te_stride = a.t_end_stride;
@@ -213,6 +218,33 @@ template <typename T> static SolveParams<T> make_params(const tode_solve_args &a
     return p;
 }
 
+// End of a whole-solve kernel, reached by every thread of every workgroup after the workgroup's
+// updates of the flag words.  With a host target, word TODE_FLAG_WORDS counts finished workgroups;
+// the last one takes the flag words, puts them back to their start values for the next solve that
+// uses them, and stores them to the host, the sequence number last.
+//
+// Only the flag words themselves need ordering, and they are touched by device-scope atomics alone,
+// which act on the one coherent copy of each word: no release of the workgroup's other writes (it
+// would write back the L2 once per workgroup).  The barrier makes every wavefront wait for its own
+// atomics to complete; the count is incremented after it, so whoever sees the final count issues
+// its exchanges after every update has been performed.
+template <typename T> __device__ __forceinline__ void publish_flags(const SolveParams<T> &p) {
+    if (p.host_flags == nullptr) return;
+    __syncthreads();
+    if (threadIdx.x != 0 || threadIdx.y != 0) return;
+    const int finished = __hip_atomic_fetch_add(&p.flags[TODE_FLAG_WORDS], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (finished != (int)(gridDim.x * gridDim.y) - 1) return;
+    const int32_t start[TODE_FLAG_WORDS] = {0, INT_MAX, 0, 0};
+    int32_t v[TODE_FLAG_WORDS];
+#pragma unroll
+    for (int i = 0; i < TODE_FLAG_WORDS; ++i) v[i] = __hip_atomic_exchange(&p.flags[i], start[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    (void)__hip_atomic_exchange(&p.flags[TODE_FLAG_WORDS], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < TODE_FLAG_WORDS; ++i) __hip_atomic_store(&p.host_flags[i], v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    // (the release also covers the exchanges above: a later kernel finds the words reset)
+    __hip_atomic_store(&p.host_flags[TODE_FLAG_WORDS], p.sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Resets the flag block; launched in front of every solve kernel.
 static __global__ void init_flags_kernel(int32_t *flags) {
     if (threadIdx.x == 0) {
@@ -221,6 +253,12 @@ static __global__ void init_flags_kernel(int32_t *flags) {
         flags[TODE_FLAG_NON_MONOTONE] = 0;
         flags[TODE_FLAG_NEEDS_GENERAL] = 0;
     }
+}
+
+// In front of a fast solve kernel: resets the caller's flag block, unless the kernel works on the
+// library's self-resetting words.
+static inline void reset_flags(int32_t *flags, hipStream_t stream) {
+    if (flag_target() == nullptr) hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, flags);
 }
 
 }  // namespace tode
