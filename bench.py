@@ -57,6 +57,7 @@ def main():
         choices=["auto", "per-step"],
         help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
     )
+    ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
     ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the baseline's sample is sized to")
     ap.add_argument(
         "--calibration-copy-mib",
@@ -82,7 +83,7 @@ def main():
     spec = dict(w.controller)
     kind = spec.pop("kind")
     ctrl = to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
-    solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl)
+    solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl, graph_iterations=args.graph_iterations)
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
     term = to.ODETerm(w.f if args.path == "auto" else (lambda t, y, f=w.f: f(t, y)))
 
@@ -121,6 +122,8 @@ def main():
         # around the torch right-hand side, and the figure below is over the whole solve
         per_step = args.path == "per-step" and F < 64
         kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
+        if per_step and args.graph_iterations:
+            kernel_name += f", {args.graph_iterations} iterations per HIP graph replay"
         kernel_s = wall
     _lib.set_kernel_timing(False)
     achieved = algo_bytes / kernel_s / 1e9

@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 F32, F64 = torch.float32, torch.float64
 
 
-def stepwise_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, calls=None, **extra):
+def stepwise_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt0=None, max_steps=None, calls=None, graph=None, **extra):
     dev = "cuda"
     mv = lambda x: None if x is None else x.to(dev)
     fg = copy.deepcopy(f).to(dev)
@@ -27,7 +27,7 @@ def stepwise_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=Non
             calls.append((t, y))
         return fg(t, y)
 
-    solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **extra), max_steps=max_steps)
+    solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **extra), max_steps=max_steps, graph_iterations=graph)
     problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
     return solver.solve(problem, to.ODETerm(opaque), dt0=mv(dt0))
 
@@ -146,3 +146,41 @@ def test_readme_example():
     assert sol.stats["n_steps"].tolist() == [4, 2] and sol.stats["n_accepted"].tolist() == [4, 2]
     assert sol.stats["n_initialized"].tolist() == [10, 10]
     assert torch.allclose(sol.ys[0, :, 0].cpu(), 1.2 * torch.exp(-0.5 * t_eval[0].cpu()), rtol=2e-3)
+
+
+# ---------------------------------------------------------------------------------------------
+# iterations replayed from a HIP graph
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("name,batch,dtype,n", [("vdp", 512, F32, 3), ("lorenz", 300, F32, 8), ("linear_decay", 256, F64, 1), ("vdp", 200, F64, 5)])
+def test_graph_replay_equals_the_eager_loop_bit_for_bit(name, batch, dtype, n):
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    calls = []
+    for _ in range(3):  # solves in a row, each with a graph of its own, other work in between
+        sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, graph=n, calls=calls)
+        assert_identical(sol, ref)
+        torch.cuda.synchronize()
+        (torch.randn(1000, device="cuda") @ torch.randn(1000, device="cuda")).item()
+    # f was called for the eager iterations and once more for each recorded one, not per replay
+    iterations = (int(ref["n_f_evals"][0]) - 2) // 6
+    assert len(calls) // 3 == 2 + 6 * (4 + n) < 2 + 6 * iterations
+
+
+def test_graph_replay_with_loop_bookkeeping_cases():
+    w = to.workloads.make("vdp", batch=130, dtype=F32)
+    t_eval = w.t_eval.clone()
+    t_eval[5, [3, 7]] = t_eval[5, [7, 3]]  # pending mask
+    assert_identical(stepwise_solve(w.f, w.y0, t_eval, w.method, w.controller, graph=2), c_oracle_solve(w.f, w.y0, t_eval, w.method, w.controller))
+    # max_steps stops some samples early, in the middle of a replayed chunk
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller, max_steps=23)
+    assert (ref["status"] == 3).any()
+    assert_identical(stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, max_steps=23, graph=7), ref)
+    # a solve that ends within the eager iterations never records a graph
+    short = w.t_eval[:, :2] * 1e-3
+    assert_identical(stepwise_solve(w.f, w.y0, short, w.method, w.controller, graph=4), c_oracle_solve(w.f, w.y0, short, w.method, w.controller))
+    # without evaluation points
+    ts, te = w.t_eval[:, 0].contiguous(), w.t_eval[:, -1].contiguous()
+    ref = c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    assert_identical(stepwise_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te, graph=4), ref)

@@ -51,12 +51,21 @@ class AutoDiffAdjoint(nn.Module):
         *,
         max_steps: Optional[int] = None,
         backprop_through_step_size_control: bool = True,
+        graph_iterations: Optional[int] = None,
     ):
         super().__init__()
         self.step_method = step_method
         self.step_size_controller = step_size_controller
         self.max_steps = max_steps
         self.backprop_through_step_size_control = backprop_through_step_size_control
+        # Not in the reference (its counterpart is compiling the loop, docs/jit.ipynb): with a user's
+        # torch right-hand side the loop is bound by kernel launches, about 60 per iteration.  With
+        # graph_iterations = n, a solve runs its first iterations as usual, then records n iterations
+        # (the per-step kernels and whatever f launches) into a HIP graph once and replays it until
+        # the batch has stopped.  Only for an f that is safe to record: same kernels for any input
+        # values, no host synchronisation, no Python side effects it relies on (f is not called
+        # again during replays).
+        self.graph_iterations = graph_iterations
         # Set to False to route built-in terms through the general whole-solve kernel only
         # (same results; used by the tests to compare the two kernels).
         self.use_fast_path = True
@@ -300,18 +309,33 @@ class AutoDiffAdjoint(nn.Module):
             _lib.check(lib.tode_step_begin(sref, cref, _lib.ptr(dt0_), 0, stream), "tode_step_begin")
         s.k[0] = k0.data_ptr()  # from here on the FSAL slot is the state's own buffer
 
-        chunk = self.poll_first
-        while True:
-            for _ in range(chunk):
+        def iterate(n, stream):
+            for _ in range(n):
                 for i in range(1, 7):
                     tt, yy = stage_buffers(i)
                     _lib.check(lib.tode_step_stage(sref, cref, i, stream), "tode_step_stage")
                     evaluate(i, tt, yy)
                 _lib.check(lib.tode_step_finish(sref, cref, stream), "tode_step_finish")
+
+        chunk, graph, replays = self.poll_first, None, 1
+        while True:
+            if graph is None:
+                iterate(chunk, stream)
+            else:
+                for _ in range(replays):
+                    graph.replay()
             fl = flags.tolist()  # host/device synchronisation, once per chunk of iterations
             if fl[_lib.STEP_FLAG_STOPPED]:
                 break
-            chunk = min(2 * chunk, self.poll_max)
+            if self.graph_iterations and graph is None:
+                # (the eager iterations above have also warmed up whatever f uses)
+                graph = self._record(lambda st: iterate(int(self.graph_iterations), st), y0)
+            elif graph is not None:
+                replays = min(2 * replays, max(1, self.poll_max // int(self.graph_iterations)))
+            else:
+                chunk = min(2 * chunk, self.poll_max)
+        keep.clear()
+        del graph  # frees the memory f's intermediate tensors were recorded with
 
         out = new(4, B, dt=torch.int64)
         _lib.check(lib.tode_step_stats(sref, *(_lib.ptr(out[i]) for i in range(4)), stream), "tode_step_stats")
@@ -322,6 +346,22 @@ class AutoDiffAdjoint(nn.Module):
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
         ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
         return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+
+    @staticmethod
+    def _record(body, like: torch.Tensor) -> "torch.cuda.CUDAGraph":
+        """Records ``body(stream)`` into a HIP graph on a side stream; nothing runs until a replay.
+        Kernels after the batch has stopped do nothing, so replaying whole chunks is safe."""
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(device=like.device)  # default priority
+        side.wait_stream(torch.cuda.current_stream(like.device))
+        with torch.cuda.stream(side):
+            graph.capture_begin(capture_error_mode="thread_local")
+            try:
+                body(_lib.stream_of(like))
+            finally:
+                graph.capture_end()
+        torch.cuda.current_stream(like.device).wait_stream(side)
+        return graph
 
     def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
         lib = _lib.load()
@@ -431,5 +471,6 @@ class AutoDiffAdjoint(nn.Module):
         return (
             f"AutoDiffAdjoint(step_method={self.step_method}, "
             f"step_size_controller={self.step_size_controller}, max_steps={self.max_steps}, "
-            f"backprop_through_step_size_control={self.backprop_through_step_size_control})"
+            f"backprop_through_step_size_control={self.backprop_through_step_size_control}"
+            + (f", graph_iterations={self.graph_iterations})" if self.graph_iterations else ")")
         )
