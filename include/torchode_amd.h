@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 6
+#define TODE_ABI_VERSION 7
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -38,8 +38,11 @@ enum {
     TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
                                          float32, tode_solve_builtin_fast only */
     TODE_TERM_MLP = 4                 /* F = 64: tanh([y, t] W1^T + b1) W2^T + b2 with 256 hidden units, weights in
-                                         shared_params; float32, tode_solve_builtin_fast only */
+                                         shared_params as packed by tode_mlp_pack_weights; float32,
+                                         tode_solve_builtin_fast only */
 };
+/* number of float32 values tode_mlp_pack_weights writes */
+#define TODE_MLP_PACKED_SIZE (152 * 256)
 /* per-sample status codes: reference status_codes.py:9-13 */
 enum {
     TODE_SUCCESS = 0,
@@ -202,6 +205,18 @@ int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *
 int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                                  int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream,
                                  int32_t *flags_out);
+
+/*
+ * Weights of TODE_TERM_MLP in the order the solve kernel loads them into
+ * registers (each thread of a workgroup reads its own values, contiguous across
+ * a wavefront).  `raw`: W1 [256 x 65] | b1 [256] | W2 [64 x 256] | b2 [64],
+ * row-major float32 on the device, n_raw = 33088 -- the parameters of the
+ * user's `f` as a torch module holds them (terms.py:13-19 takes any callable).
+ * `packed`: TODE_MLP_PACKED_SIZE float32 on the device; pass it as
+ * shared_params / n_shared_params of the solve.  Pack once per change of the
+ * weights, not per solve.
+ */
+int tode_mlp_pack_weights(const void *raw, int64_t n_raw, void *packed, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Per-step kernels around a right-hand side that lives outside the library   */

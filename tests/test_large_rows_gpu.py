@@ -233,3 +233,40 @@ def test_mlp_kernel_with_tight_tolerances(method, kind):
         assert mixed_error(fused.ys.double().cpu(), proto.ys.double().cpu()) < 2e-5
         work = fused.stats["n_steps"].sum().item() / proto.stats["n_steps"].sum().item()
         assert 0.8 < work < 1.25, work
+
+
+def test_mlp_weight_packing_and_repacking():
+    """tode_mlp_pack_weights against the register map written out with numpy: thread (w, q, c) holds
+    rows 64w + 16 tile + c of W1 at the inputs lane group q feeds, b1 and the columns of W2 for hidden
+    units 64w + 16 tile + 4q + r, and b2 for its own four features."""
+    import numpy as np
+
+    w = to.workloads.make("mlp", batch=32, device="cuda")
+    f = w.f
+    f.b1.copy_(torch.linspace(-1, 1, 256))
+    f.b2.copy_(torch.linspace(2, 3, 64))
+    packed = f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32)
+    assert f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32) is packed
+    got = packed.cpu().numpy().reshape(152, 4, 4, 16)  # [register][w][q][c]
+    W1, b1, W2, b2 = (x.cpu().numpy() for x in (f.W1, f.b1, f.W2, f.b2))
+    wv, qv, cv = np.meshgrid(np.arange(4), np.arange(4), np.arange(16), indexing="ij")
+    for kk in range(17):
+        col = 16 * qv + kk if kk < 16 else 64 + qv
+        for tile in range(4):
+            want = np.where(col <= 64, W1[64 * wv + 16 * tile + cv, np.minimum(col, 64)], 0.0)
+            assert np.array_equal(got[4 * kk + tile], want), (kk, tile)
+    for tile in range(4):
+        for r in range(4):
+            assert np.array_equal(got[68 + 4 * tile + r], b1[64 * wv + 16 * tile + 4 * qv + r])
+            for ft in range(4):
+                assert np.array_equal(got[84 + 16 * ft + 4 * tile + r], W2[16 * ft + cv, 64 * wv + 16 * tile + 4 * qv + r])
+    for r in range(4):
+        assert np.array_equal(got[148 + r], b2[16 * wv + 4 * qv + r])
+
+    # weights written in place are packed again: the solve follows them
+    before, _ = mlp_both_paths(w, w.method, w.controller)
+    f.W2.mul_(-1.0)
+    after, proto = mlp_both_paths(w, w.method, w.controller)
+    assert f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32) is not packed
+    assert mixed_error(before.ys.double().cpu(), after.ys.double().cpu()) > 1e-2
+    assert torch.equal(after.status, proto.status) and mixed_error(after.ys.double().cpu(), proto.ys.double().cpu()) < 1e-2

@@ -13,7 +13,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
+MLP_PACKED_SIZE = 152 * 256
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -32,6 +33,7 @@ EXPORTS = (
     "tode_solve_builtin",
     "tode_solve_builtin_fast",
     "tode_solve_builtin_fast_sync",
+    "tode_mlp_pack_weights",
     "tode_step_begin",
     "tode_step_stage",
     "tode_step_finish",
@@ -221,6 +223,8 @@ def load():
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
         lib.tode_solve_builtin_fast.restype = C.c_int
         lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
+        lib.tode_mlp_pack_weights.restype = C.c_int
+        lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
         lib.tode_solve_builtin_fast_sync.restype = C.c_int
         lib.tode_solve_builtin_fast_sync.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.POINTER(C.c_int32)]
         lib.tode_step_begin.restype = C.c_int

@@ -377,7 +377,10 @@ class AutoDiffAdjoint(nn.Module):
         if params.numel() == 0 and params.shape[0] != B:  # a term without per-sample parameters
             params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
-        shared = f.builtin_shared().to(device=dev, dtype=dtype) if hasattr(f, "builtin_shared") else None
+        mlp = f.builtin_kind == _lib.TERM_MLP
+        if mlp and (dtype != torch.float32 or F != 64 or tuple(f.W1.shape) != (256, 65)):
+            return None  # the matrix-core kernel is built for this shape only: the caller takes the protocol path
+        shared = f.builtin_packed(dev, dtype) if mlp else None
         dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
@@ -411,7 +414,7 @@ class AutoDiffAdjoint(nn.Module):
             if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
                 fast_ok = fast_ok and F in (32 * 32, 64 * 64) and E <= 8192
             else:
-                fast_ok = fast_ok and F == 64 and tuple(f.W1.shape) == (256, 65) and E <= 512
+                fast_ok = fast_ok and E <= 512  # (shape and dtype were checked before the weights were packed)
             if not fast_ok:
                 return None  # no whole-solve kernel for this case: the caller takes the protocol path
         if fast_ok:

@@ -138,11 +138,21 @@ class MLPField(BuiltinTerm):
         return torch.empty((0, 0), dtype=self.W1.dtype, device=self.W1.device)
 
     def builtin_shared(self) -> torch.Tensor:
-        """W1 | b1 | W2 | b2, row-major and concatenated: the layout the whole-solve kernel reads.
-        Packed once and again whenever a weight tensor has been replaced or written in place."""
+        """W1 | b1 | W2 | b2, row-major and concatenated."""
+        return torch.cat([w.reshape(-1) for w in (self.W1, self.b1, self.W2, self.b2)]).contiguous()
+
+    def builtin_packed(self, device, dtype) -> torch.Tensor:
+        """The weights in the order the whole-solve kernel loads them into registers (a device
+        tensor).  Packed once, and again whenever a weight tensor has been replaced or written
+        in place."""
+        from . import _lib
+
         weights = (self.W1, self.b1, self.W2, self.b2)
-        key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights)
+        key = (tuple((w.data_ptr(), w._version) for w in weights), device, dtype)
         if getattr(self, "_packed_key", None) != key:
-            self._packed = torch.cat([w.reshape(-1) for w in weights]).contiguous()
-            self._packed_key = key
+            raw = self.builtin_shared().to(device=device, dtype=dtype)
+            packed = torch.empty(_lib.MLP_PACKED_SIZE, dtype=dtype, device=device)
+            rc = _lib.load().tode_mlp_pack_weights(_lib.ptr(raw), raw.numel(), _lib.ptr(packed), _lib.stream_of(raw))
+            _lib.check(rc, "tode_mlp_pack_weights")
+            self._packed, self._packed_key = packed, key
         return self._packed
