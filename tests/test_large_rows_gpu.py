@@ -247,7 +247,7 @@ def test_mlp_weight_packing_and_repacking():
     f.b2.copy_(torch.linspace(2, 3, 64))
     packed = f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32)
     assert f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32) is packed
-    got = packed.cpu().numpy().reshape(152, 4, 4, 16)  # [register][w][q][c]
+    got = packed.cpu().numpy().reshape(38, 256, 4).transpose(0, 2, 1).reshape(152, 4, 4, 16)  # [register][w][q][c]
     W1, b1, W2, b2 = (x.cpu().numpy() for x in (f.W1, f.b1, f.W2, f.b2))
     wv, qv, cv = np.meshgrid(np.arange(4), np.arange(4), np.arange(16), indexing="ij")
     for kk in range(17):

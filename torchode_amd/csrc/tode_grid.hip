@@ -46,7 +46,7 @@ template <int NW> __device__ __forceinline__ void block_sum2(GridShared<NW> &sh,
         sh.red[slot][wave][0] = a;
         sh.red[slot][wave][1] = b;
     }
-    __syncthreads();
+    lds_barrier();
     A = 0;
     B = 0;
 #pragma unroll
@@ -66,7 +66,7 @@ __device__ __forceinline__ void grid_rhs(GridShared<NW> &sh, int &buf, float D, 
     const int r = t / PER_ROW, c0 = 4 * (t - r * PER_ROW);
     float *x = sh.xch[buf];
     *reinterpret_cast<float4 *>(x + 4 * t) = make_float4(u[0], u[1], u[2], u[3]);
-    __syncthreads();
+    lds_barrier();
     const int ru = (r + N - 1) & (N - 1), rd = (r + 1) & (N - 1);
     const float4 up = *reinterpret_cast<const float4 *>(x + ru * N + c0);
     const float4 dn = *reinterpret_cast<const float4 *>(x + rd * N + c0);

@@ -20,8 +20,9 @@
 //     dense-output coefficients (16-byte accesses to y0 and ys).  Per-sample scalars (t, dt,
 //     error ratio, counters) are carried redundantly by the 16 lanes that share a sample.
 //
-// The weights are read in a packed order (tode_mlp_pack_weights): register j of thread tid at
-// packed[j * 256 + tid], so that the prologue's loads are contiguous across a wavefront.
+// The weights are read in a packed order (tode_mlp_pack_weights): registers 4i..4i+3 of thread
+// tid as one 16-byte value at packed[(i * 256 + tid) * 4], so that the prologue is 38 loads per
+// thread, each contiguous across a wavefront.
 //
 // Same contract as the other fast kernels: the common case only; anything else raises
 // TODE_FLAG_NEEDS_GENERAL and leaves the outputs unspecified.
@@ -46,6 +47,7 @@ struct __align__(16) MlpShared {
     float x[MLP_TILE * MLP_XS];
     float part[4][4][64][4];        // [output tile][wavefront it comes from][lane][4 features]
     float red[2][4][MLP_TILE][2];   // per-wavefront partial sums of up to two per-sample reductions
+    int vote[2][4];                 // per-wavefront bits of the workgroup-wide "or"
 };
 
 struct MlpWeights {
@@ -81,8 +83,23 @@ __host__ __device__ inline long long mlp_packed_source(int j, int tid) {
 static __global__ void mlp_pack_kernel(const float *raw, float *packed) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= MLP_REGS * 256) return;
-    const long long src = mlp_packed_source(i / 256, i % 256);
+    const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
+    const long long src = mlp_packed_source(4 * group + part, tid);
     packed[i] = src < 0 ? 0.0f : raw[src];
+}
+
+// Bitwise "or" of `bits` over the workgroup (four wavefronts).  Consecutive calls alternate between
+// two sets of LDS words, so a wavefront that runs ahead into the next call cannot overwrite what
+// a slower one still has to read.
+__device__ __forceinline__ int block_or(MlpShared &sh, int &vslot, int bits) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) bits |= __shfl_xor(bits, off);
+    if (lane == 0) sh.vote[vslot][w] = bits;
+    lds_barrier();
+    const int all = (sh.vote[vslot][0] | sh.vote[vslot][1]) | (sh.vote[vslot][2] | sh.vote[vslot][3]);
+    vslot ^= 1;
+    return all;
 }
 
 // tanh(x) = 1 - 2 / (exp(2x) + 1) on the hardware exp2 and reciprocal: absolute error about 2e-7
@@ -98,7 +115,7 @@ __device__ __forceinline__ void mlp_rhs(MlpShared &sh, const MlpWeights &W, floa
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, q = lane >> 4, c = lane & 15;
     *reinterpret_cast<float4 *>(sh.x + c * MLP_XS + 16 * w + 4 * q) = make_float4(yi[0], yi[1], yi[2], yi[3]);
     if (w == 0 && q == 0) sh.x[c * MLP_XS + MLP_F] = tn;
-    __syncthreads();
+    lds_barrier();
     // all B operands of the layer into registers first, so that the matrix cores never wait for LDS
     float a1[17];
     {
@@ -134,7 +151,7 @@ __device__ __forceinline__ void mlp_rhs(MlpShared &sh, const MlpWeights &W, floa
             for (int ft = 0; ft < 4; ++ft) acc[ft] = __builtin_amdgcn_mfma_f32_16x16x4f32(W.w2[ft][tile][r], h[tile][r], acc[ft], 0, 0, 0);
 #pragma unroll
     for (int ft = 0; ft < 4; ++ft) *reinterpret_cast<float4 *>(sh.part[ft][w][lane]) = make_float4(acc[ft][0], acc[ft][1], acc[ft][2], acc[ft][3]);
-    __syncthreads();
+    lds_barrier();
     float4 s[4];
 #pragma unroll
     for (int from = 0; from < 4; ++from) s[from] = *reinterpret_cast<const float4 *>(sh.part[w][from][lane]);
@@ -158,7 +175,7 @@ __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (
         sh.red[slot][w][c][0] = u;
         sh.red[slot][w][c][1] = v;
     }
-    __syncthreads();
+    lds_barrier();
     A = (sh.red[slot][0][c][0] + sh.red[slot][1][c][0]) + (sh.red[slot][2][c][0] + sh.red[slot][3][c][0]);
     B = (sh.red[slot][0][c][1] + sh.red[slot][1][c][1]) + (sh.red[slot][2][c][1] + sh.red[slot][3][c][1]);
     slot ^= 1;
@@ -185,17 +202,21 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
     // ---- weights into registers ----
     MlpWeights W;
     {
-        const float *src = packed + tid;
+        const float4 *src = reinterpret_cast<const float4 *>(packed) + tid;
+        float v[MLP_REGS];
 #pragma unroll
-        for (int kk = 0; kk < 17; ++kk)
+        for (int i = 0; i < MLP_REGS / 4; ++i) {
+            const float4 u = src[i * 256];
+            v[4 * i] = u.x, v[4 * i + 1] = u.y, v[4 * i + 2] = u.z, v[4 * i + 3] = u.w;
+        }
 #pragma unroll
-            for (int tile = 0; tile < 4; ++tile) W.w1[kk][tile] = src[(4 * kk + tile) * 256];
+        for (int j = 0; j < 68; ++j) W.w1[j / 4][j % 4] = v[j];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) W.b1[j / 4][j % 4] = src[(68 + j) * 256];
+        for (int j = 0; j < 16; ++j) W.b1[j / 4][j % 4] = v[68 + j];
 #pragma unroll
-        for (int j = 0; j < 64; ++j) W.w2[j / 16][(j / 4) % 4][j % 4] = src[(84 + j) * 256];
+        for (int j = 0; j < 64; ++j) W.w2[j / 16][(j / 4) % 4][j % 4] = v[84 + j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) W.b2[j] = src[(148 + j) * 256];
+        for (int j = 0; j < 4; ++j) W.b2[j] = v[148 + j];
     }
     for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns 65..67
     for (int i = tid; i < rows * E; i += 256) te_s[i] = p.t_eval[b0 * E + i];
@@ -251,9 +272,11 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
         *reinterpret_cast<float4 *>(p.ys + (bs * E) * F + f0) = make_float4(y[0], y[1], y[2], y[3]);
         cursor = 1;
     }
-    bail = __syncthreads_or(bail) != 0;
-
-    while (!bail && __syncthreads_or(active)) {
+    int vslot = 0;
+    // bit 1: some sample needs the general kernel; bit 0: some sample still runs
+    int state = block_or(sh, vslot, (bail ? 2 : 0) | (active ? 1 : 0));
+    bail = (state & 2) != 0;
+    while (state == 1) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
         T y1[4];
@@ -344,7 +367,8 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
         const bool odd = !(t == te) || nonfinite;
         bail = bail || failed || (finished && odd);
         active = active && !failed && running_new;
-        bail = __syncthreads_or(bail) != 0;
+        state = block_or(sh, vslot, (bail ? 2 : 0) | (active ? 1 : 0));
+        bail = (state & 2) != 0;
     }
 
     if (w == 0 && q == 0) {

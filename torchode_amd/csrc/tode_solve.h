@@ -218,6 +218,16 @@ template <typename T> static SolveParams<T> make_params(const tode_solve_args &a
     return p;
 }
 
+// Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for the wavefront's
+// global stores to be acknowledged -- in the whole-solve kernels the dense output, which no thread
+// of the kernel ever reads -- and that wait (a round trip to memory) would sit on the critical path
+// of the next stage.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // End of a whole-solve kernel, reached by every thread of every workgroup after the workgroup's
 // updates of the flag words.  With a host target, word TODE_FLAG_WORDS counts finished workgroups;
 // the last one takes the flag words, puts them back to their start values for the next solve that
