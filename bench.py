@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_FP32_PEAK_TFLOPS = 157.3
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
 MEASURED_TRAFFIC_BYTES = {
@@ -57,6 +58,7 @@ def main():
         choices=["auto", "per-step"],
         help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
     )
+    ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
     ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
     ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the baseline's sample is sized to")
     ap.add_argument(
@@ -78,6 +80,8 @@ def main():
     dtype = {None: None, "f32": torch.float32, "f64": torch.float64}[args.dtype]
     w = to.workloads.make(args.workload, batch=args.batch, dtype=dtype, device="cuda")
     dtype = w.y0.dtype
+    if w.name == "mlp":
+        w.f.matrix_inputs = args.mlp_inputs
     B, F = w.y0.shape
     E = w.t_eval.shape[1]
     spec = dict(w.controller)
@@ -153,14 +157,15 @@ def main():
         flops_f = 2 * (Fin * H + H * F)
         flops = (2 * B + 6 * sample_steps) * flops_f + 5000 * sample_steps
         tflops = flops / kernel_s / 1e12
+        peak = MFMA_FP32_PEAK_TFLOPS if args.mlp_inputs == "float32" else MFMA_BF16_PEAK_TFLOPS
         roofline = {
             "bound": "mfma",
             "kernel": kernel_name,
             "achieved": tflops,
-            "peak": MFMA_FP32_PEAK_TFLOPS,
+            "peak": peak,
             "unit": "TFLOP/s",
-            "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
+            "frac": tflops / peak,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)) if args.mlp_inputs == "float32" else None,
             "algorithmic_flops_per_launch": flops,
             "flops_per_rhs_evaluation_per_sample": flops_f,
             "kernel_ms": kernel_s * 1e3,
@@ -177,7 +182,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {torch.float32: "f32", torch.float64: "f64"}[dtype],
+        "dtype": {torch.float32: "f32", torch.float64: "f64"}[dtype] + (" (bf16 matrix-core inputs)" if w.name == "mlp" and args.mlp_inputs == "bfloat16" else ""),
         "data": "synthetic",
         "config": {
             "workload": f"{w.name} B={B} F={F} E={E} {w.method}+{kind}",

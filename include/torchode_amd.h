@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 7
+#define TODE_ABI_VERSION 8
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -41,8 +41,11 @@ enum {
                                          shared_params as packed by tode_mlp_pack_weights; float32,
                                          tode_solve_builtin_fast only */
 };
-/* number of float32 values tode_mlp_pack_weights writes */
+/* what the matrix cores take as inputs in the MLP kernel; accumulation, biases, tanh and the solver are float32 */
+enum { TODE_MLP_INPUTS_F32 = 0, TODE_MLP_INPUTS_BF16 = 1 };
+/* number of 32-bit words tode_mlp_pack_weights writes for either */
 #define TODE_MLP_PACKED_SIZE (152 * 256)
+#define TODE_MLP_PACKED_SIZE_BF16 (92 * 256)
 /* per-sample status codes: reference status_codes.py:9-13 */
 enum {
     TODE_SUCCESS = 0,
@@ -212,11 +215,16 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_control
  * a wavefront).  `raw`: W1 [256 x 65] | b1 [256] | W2 [64 x 256] | b2 [64],
  * row-major float32 on the device, n_raw = 33088 -- the parameters of the
  * user's `f` as a torch module holds them (terms.py:13-19 takes any callable).
- * `packed`: TODE_MLP_PACKED_SIZE float32 on the device; pass it as
- * shared_params / n_shared_params of the solve.  Pack once per change of the
+ * `packed`: TODE_MLP_PACKED_SIZE (matrix_inputs = TODE_MLP_INPUTS_F32) or
+ * TODE_MLP_PACKED_SIZE_BF16 (TODE_MLP_INPUTS_BF16: W1 and W2 rounded to
+ * bfloat16, two per word) 32-bit words on the device; pass it as shared_params
+ * with that count as n_shared_params, which also selects the kernel.  With
+ * bfloat16 inputs the solve is a reduced-precision variant of its own (the
+ * stage inputs and hidden activations are rounded as well): results differ
+ * from the float32 path at the 1e-3 level.  Pack once per change of the
  * weights, not per solve.
  */
-int tode_mlp_pack_weights(const void *raw, int64_t n_raw, void *packed, void *stream);
+int tode_mlp_pack_weights(const void *raw, int64_t n_raw, int32_t matrix_inputs, void *packed, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Per-step kernels around a right-hand side that lives outside the library   */

@@ -175,13 +175,13 @@ def test_against_the_committed_vectors(name, batch):
 # ---------------------------------------------------------------------------------------------
 
 
-def mlp_both_paths(w, method, ctrl, **kw):
+def mlp_both_paths(w, method, ctrl, kernel="tode::solve_mlp_kernel", **kw):
     from torchode_amd import _lib
 
     lib_m, own_m = {"tsit5": (to.Tsit5, OwnTsit5), "dopri5": (to.Dopri5, OwnDopri5)}[method]
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
     fused = to.AutoDiffAdjoint(lib_m(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f), **kw)
-    assert _lib.last_solve_kernel_name() == "tode::solve_mlp_kernel"
+    assert _lib.last_solve_kernel_name() == kernel
     return fused, to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f), **kw)
 
 
@@ -270,3 +270,29 @@ def test_mlp_weight_packing_and_repacking():
     assert f.builtin_packed(torch.device("cuda", torch.cuda.current_device()), torch.float32) is not packed
     assert mixed_error(before.ys.double().cpu(), after.ys.double().cpu()) > 1e-2
     assert torch.equal(after.status, proto.status) and mixed_error(after.ys.double().cpu(), proto.ys.double().cpu()) < 1e-2
+
+
+def test_mlp_kernel_with_bfloat16_matrix_inputs():
+    """The reduced-precision variant: W1, W2, the stage inputs and the hidden activations rounded to
+    bfloat16 in front of the matrix cores, everything else float32.  MLPField.forward states the same
+    function in torch operations, so the protocol path solves the same problem; the rounding makes f
+    piecewise constant at the 2^-9 level, so the two agree at that level and no better."""
+    w = to.workloads.make("mlp", batch=256, device="cuda")
+    exact, _ = mlp_both_paths(w, w.method, w.controller)
+    w.f.matrix_inputs = "bfloat16"
+    fused, proto = mlp_both_paths(w, w.method, w.controller, kernel="tode::solve_mlp_kernel (bfloat16 matrix inputs)")
+    assert torch.equal(fused.status, proto.status) and (fused.status == 0).all() and (fused.stats["n_initialized"] == 20).all()
+    assert mixed_error(fused.ys.double().cpu(), proto.ys.double().cpu()) < 2e-2
+    against_float32 = mixed_error(fused.ys.double().cpu(), exact.ys.double().cpu())
+    assert 1e-5 < against_float32 < 3e-2, against_float32
+    work = fused.stats["n_steps"].sum().item() / proto.stats["n_steps"].sum().item()
+    assert 0.7 < work < 1.4, work
+    # one evaluation of f, through a problem whose first step size is the whole interval: y(t1) by Euler-sized steps
+    # is dominated by f(t0, y0); checks the operand layout more sharply than a whole solve
+    w2 = to.workloads.make("mlp", batch=64, device="cuda")
+    w2.f.matrix_inputs = "bfloat16"
+    t_eval = torch.stack([torch.zeros(64, device="cuda"), torch.full((64,), 1e-3, device="cuda")], 1)
+    sol = to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-5, 1e-3)).solve(to.InitialValueProblem(w2.y0, t_eval=t_eval), to.ODETerm(w2.f))
+    slope = (sol.ys[:, 1] - sol.ys[:, 0]) / 1e-3
+    want = w2.f(torch.zeros(64, device="cuda"), w2.y0)
+    assert mixed_error(slope.double().cpu(), want.double().cpu()) < 2e-2

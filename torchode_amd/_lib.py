@@ -13,8 +13,9 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 7
-MLP_PACKED_SIZE = 152 * 256
+ABI_VERSION = 8
+MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
+MLP_INPUTS = {"float32": 0, "bfloat16": 1}
 F32, F64 = 0, 1
 DOPRI5, TSIT5 = 0, 1
 CTRL_INTEGRAL, CTRL_PID = 0, 1
@@ -224,7 +225,7 @@ def load():
         lib.tode_solve_builtin_fast.restype = C.c_int
         lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
         lib.tode_mlp_pack_weights.restype = C.c_int
-        lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+        lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         lib.tode_solve_builtin_fast_sync.restype = C.c_int
         lib.tode_solve_builtin_fast_sync.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.POINTER(C.c_int32)]
         lib.tode_step_begin.restype = C.c_int

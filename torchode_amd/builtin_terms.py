@@ -119,19 +119,30 @@ class ReactionDiffusion(BuiltinTerm):
 
 class MLPField(BuiltinTerm):
     """Time-dependent two-layer perceptron shared by the whole batch:
-    ``f(t, y) = tanh(cat([y, t], 1) @ W1.T + b1) @ W2.T + b2`` with ``W1 [H, F+1]``, ``W2 [F, H]``."""
+    ``f(t, y) = tanh(cat([y, t], 1) @ W1.T + b1) @ W2.T + b2`` with ``W1 [H, F+1]``, ``W2 [F, H]``.
+
+    ``matrix_inputs="bfloat16"`` is a reduced-precision variant of the function itself: both matrix
+    products take their two operands rounded to bfloat16 (sums, biases and tanh stay in the working
+    precision), which is what the matrix cores do at eight times the float32 rate."""
 
     builtin_kind = TERM_MLP
 
-    def __init__(self, W1: torch.Tensor, b1: torch.Tensor, W2: torch.Tensor, b2: torch.Tensor):
+    def __init__(self, W1: torch.Tensor, b1: torch.Tensor, W2: torch.Tensor, b2: torch.Tensor, matrix_inputs: str = "float32"):
         super().__init__()
         assert W1.ndim == 2 and W2.ndim == 2 and W1.shape[0] == W2.shape[1] and W1.shape[1] == W2.shape[0] + 1
+        assert matrix_inputs in ("float32", "bfloat16")
         for name, w in (("W1", W1), ("b1", b1), ("W2", W2), ("b2", b2)):
             self.register_buffer(name, w)
         self.n_features = W2.shape[0]
+        self.matrix_inputs = matrix_inputs
 
     def forward(self, t, y):
-        h = torch.tanh(torch.cat([y, t[:, None]], 1) @ self.W1.T + self.b1)
+        x = torch.cat([y, t[:, None]], 1)
+        if self.matrix_inputs == "bfloat16":
+            rounded = lambda z: z.to(torch.bfloat16).to(z.dtype)
+            h = torch.tanh(rounded(x) @ rounded(self.W1).T + self.b1)
+            return rounded(h) @ rounded(self.W2).T + self.b2
+        h = torch.tanh(x @ self.W1.T + self.b1)
         return h @ self.W2.T + self.b2
 
     def builtin_params(self):
@@ -148,11 +159,13 @@ class MLPField(BuiltinTerm):
         from . import _lib
 
         weights = (self.W1, self.b1, self.W2, self.b2)
-        key = (tuple((w.data_ptr(), w._version) for w in weights), device, dtype)
+        key = (tuple((w.data_ptr(), w._version) for w in weights), device, dtype, self.matrix_inputs)
         if getattr(self, "_packed_key", None) != key:
             raw = self.builtin_shared().to(device=device, dtype=dtype)
-            packed = torch.empty(_lib.MLP_PACKED_SIZE, dtype=dtype, device=device)
-            rc = _lib.load().tode_mlp_pack_weights(_lib.ptr(raw), raw.numel(), _lib.ptr(packed), _lib.stream_of(raw))
+            packed = torch.empty(_lib.MLP_PACKED_SIZE[self.matrix_inputs], dtype=dtype, device=device)
+            rc = _lib.load().tode_mlp_pack_weights(
+                _lib.ptr(raw), raw.numel(), _lib.MLP_INPUTS[self.matrix_inputs], _lib.ptr(packed), _lib.stream_of(raw)
+            )
             _lib.check(rc, "tode_mlp_pack_weights")
             self._packed, self._packed_key = packed, key
         return self._packed

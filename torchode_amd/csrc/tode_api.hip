@@ -229,8 +229,8 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     return solve_fast_f64(*a, *c, ns, na, ni, st, s);
 }
 
-int tode_mlp_pack_weights(const void *raw, int64_t n_raw, void *packed, void *stream) {
-    return tode::mlp_pack_weights((const float *)raw, (long long)n_raw, (float *)packed, (hipStream_t)stream);
+int tode_mlp_pack_weights(const void *raw, int64_t n_raw, int32_t matrix_inputs, void *packed, void *stream) {
+    return tode::mlp_pack_weights((const float *)raw, (long long)n_raw, matrix_inputs, (float *)packed, (hipStream_t)stream);
 }
 
 int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,

@@ -39,8 +39,9 @@ struct MlpOut {
 };
 
 constexpr int MLP_F = 64, MLP_H = 256, MLP_TILE = 16;
-constexpr int MLP_XS = 72;  // LDS row of the stage input: 64 features, t, 3 zeros, padding
-constexpr int MLP_REGS = 68 + 16 + 64 + 4;  // packed values per thread: W1, b1, W2, b2
+constexpr int MLP_XS = 84;  // LDS row of the stage input: 64 features, t, zeros up to column 79, padding
+constexpr int MLP_REGS = 68 + 16 + 64 + 4;       // packed values per thread: W1, b1, W2, b2
+constexpr int MLP_REGS_BF16 = 40 + 16 + 32 + 4;  // the same with W1 (80 inputs) and W2 as pairs of bfloat16
 constexpr long long MLP_RAW = (long long)MLP_H * (MLP_F + 1) + MLP_H + (long long)MLP_F * MLP_H + MLP_F;
 
 struct __align__(16) MlpShared {
@@ -55,6 +56,18 @@ struct MlpWeights {
     float b1[4][4];     // b1[64w + 16 tile + 4q + r]
     float w2[4][4][4];  // W2[16 ft + c][64w + 16 tile + 4q + r]
     float b2[4];        // b2[16w + 4q + r]
+};
+
+// The variant with bfloat16 inputs to the matrix cores (v_mfma_f32_16x16x16_bf16: 16 k per
+// instruction, a lane supplies k = 4q..4q+3): float32 accumulation, biases, tanh and solver state.
+typedef __bf16 mlp_bf16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned mlp_u32x2 __attribute__((ext_vector_type(2)));
+
+struct MlpWeightsBf16 {
+    mlp_bf16x4 w1[5][4];  // W1[64w + 16 tile + c][16 ks + 4q + j], inputs 65..79 are zero
+    float b1[4][4];
+    mlp_bf16x4 w2[4][4];  // [ft][tile]: W2[16 ft + c][64w + 16 tile + 4q + j]
+    float b2[4];
 };
 
 // Which input column lane group q feeds at k-step kk of the first layer: 16 features each for
@@ -78,6 +91,49 @@ __host__ __device__ inline long long mlp_packed_source(int j, int tid) {
     }
     j -= 64;
     return o_b2 + 16 * w + 4 * q + j;
+}
+
+// The same for the bfloat16 variant: packed word j of thread tid holds the values of sources
+// (lo, hi) as bfloat16 in its low and high half (words of b1 and b2: one float32, hi = -2).
+__host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, long long &lo, long long &hi) {
+    const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
+    const long long o_b1 = (long long)MLP_H * (MLP_F + 1), o_w2 = o_b1 + MLP_H, o_b2 = o_w2 + (long long)MLP_F * MLP_H;
+    hi = -2;
+    if (j < 40) {
+        const int ks = j / 8, tile = (j / 2) % 4, k = 16 * ks + 4 * q + 2 * (j % 2);
+        const long long row = (long long)(64 * w + 16 * tile + c) * (MLP_F + 1);
+        lo = k <= MLP_F ? row + k : -1;
+        hi = k + 1 <= MLP_F ? row + k + 1 : -1;
+        return;
+    }
+    j -= 40;
+    if (j < 16) {
+        lo = o_b1 + 64 * w + 16 * (j / 4) + 4 * q + (j % 4);
+        return;
+    }
+    j -= 16;
+    if (j < 32) {
+        const int ft = j / 8, tile = (j / 2) % 4;
+        lo = o_w2 + (long long)(16 * ft + c) * MLP_H + 64 * w + 16 * tile + 4 * q + 2 * (j % 2);
+        hi = lo + 1;
+        return;
+    }
+    j -= 32;
+    lo = o_b2 + 16 * w + 4 * q + j;
+}
+
+static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= MLP_REGS_BF16 * 256) return;
+    const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
+    long long lo, hi;
+    mlp_packed_source_bf16(4 * group + part, tid, lo, hi);
+    if (hi == -2) {
+        packed[i] = __float_as_uint(raw[lo]);
+        return;
+    }
+    const __bf16 a = (__bf16)(lo < 0 ? 0.0f : raw[lo]), b = (__bf16)(hi < 0 ? 0.0f : raw[hi]);  // round to nearest even
+    packed[i] = (unsigned)__builtin_bit_cast(unsigned short, a) | ((unsigned)__builtin_bit_cast(unsigned short, b) << 16);
 }
 
 static __global__ void mlp_pack_kernel(const float *raw, float *packed) {
@@ -161,6 +217,89 @@ __device__ __forceinline__ void mlp_rhs(MlpShared &sh, const MlpWeights &W, floa
     out[3] = ((s[0].w + s[1].w) + (s[2].w + s[3].w)) + W.b2[3];
 }
 
+__device__ __forceinline__ void mlp_rhs(MlpShared &sh, const MlpWeightsBf16 &W, float tn, const float (&yi)[4], float (&out)[4]) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, q = lane >> 4, c = lane & 15;
+    *reinterpret_cast<float4 *>(sh.x + c * MLP_XS + 16 * w + 4 * q) = make_float4(yi[0], yi[1], yi[2], yi[3]);
+    if (w == 0 && q == 0) sh.x[c * MLP_XS + MLP_F] = tn;
+    lds_barrier();
+    mlp_bf16x4 a1[5];
+    {
+        const float *row = sh.x + c * MLP_XS + 4 * q;
+#pragma unroll
+        for (int ks = 0; ks < 5; ++ks) {
+            const float4 v = *reinterpret_cast<const float4 *>(row + 16 * ks);
+            a1[ks] = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
+        }
+    }
+    asm volatile("" ::: "memory");
+    mfma_acc h[4];
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile) h[tile] = {W.b1[tile][0], W.b1[tile][1], W.b1[tile][2], W.b1[tile][3]};
+#pragma unroll
+    for (int ks = 0; ks < 5; ++ks) {
+#pragma unroll
+        for (int tile = 0; tile < 4; ++tile) h[tile] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(W.w1[ks][tile], a1[ks], h[tile], 0, 0, 0);
+    }
+    mlp_bf16x4 hb[4];
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile)
+        hb[tile] = {(__bf16)mlp_tanh(h[tile][0]), (__bf16)mlp_tanh(h[tile][1]), (__bf16)mlp_tanh(h[tile][2]), (__bf16)mlp_tanh(h[tile][3])};
+    mfma_acc acc[4];
+#pragma unroll
+    for (int ft = 0; ft < 4; ++ft) acc[ft] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile)
+#pragma unroll
+        for (int ft = 0; ft < 4; ++ft) acc[ft] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(W.w2[ft][tile], hb[tile], acc[ft], 0, 0, 0);
+#pragma unroll
+    for (int ft = 0; ft < 4; ++ft) *reinterpret_cast<float4 *>(sh.part[ft][w][lane]) = make_float4(acc[ft][0], acc[ft][1], acc[ft][2], acc[ft][3]);
+    lds_barrier();
+    float4 s[4];
+#pragma unroll
+    for (int from = 0; from < 4; ++from) s[from] = *reinterpret_cast<const float4 *>(sh.part[w][from][lane]);
+    out[0] = ((s[0].x + s[1].x) + (s[2].x + s[3].x)) + W.b2[0];
+    out[1] = ((s[0].y + s[1].y) + (s[2].y + s[3].y)) + W.b2[1];
+    out[2] = ((s[0].z + s[1].z) + (s[2].z + s[3].z)) + W.b2[2];
+    out[3] = ((s[0].w + s[1].w) + (s[2].w + s[3].w)) + W.b2[3];
+}
+
+// Packed weights (tode_mlp_pack_weights) into the registers of thread tid.
+__device__ __forceinline__ void mlp_load(MlpWeights &W, const float *packed, int tid) {
+    const float4 *src = reinterpret_cast<const float4 *>(packed) + tid;
+    float v[MLP_REGS];
+#pragma unroll
+    for (int i = 0; i < MLP_REGS / 4; ++i) {
+        const float4 u = src[i * 256];
+        v[4 * i] = u.x, v[4 * i + 1] = u.y, v[4 * i + 2] = u.z, v[4 * i + 3] = u.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 68; ++j) W.w1[j / 4][j % 4] = v[j];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) W.b1[j / 4][j % 4] = v[68 + j];
+#pragma unroll
+    for (int j = 0; j < 64; ++j) W.w2[j / 16][(j / 4) % 4][j % 4] = v[84 + j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) W.b2[j] = v[148 + j];
+}
+
+__device__ __forceinline__ void mlp_load(MlpWeightsBf16 &W, const float *packed, int tid) {
+    const uint4 *src = reinterpret_cast<const uint4 *>(packed) + tid;
+    unsigned v[MLP_REGS_BF16];
+#pragma unroll
+    for (int i = 0; i < MLP_REGS_BF16 / 4; ++i) {
+        const uint4 u = src[i * 256];
+        v[4 * i] = u.x, v[4 * i + 1] = u.y, v[4 * i + 2] = u.z, v[4 * i + 3] = u.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 20; ++j) W.w1[j / 4][j % 4] = __builtin_bit_cast(mlp_bf16x4, (mlp_u32x2){v[2 * j], v[2 * j + 1]});
+#pragma unroll
+    for (int j = 0; j < 16; ++j) W.b1[j / 4][j % 4] = __uint_as_float(v[40 + j]);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) W.w2[j / 4][j % 4] = __builtin_bit_cast(mlp_bf16x4, (mlp_u32x2){v[56 + 2 * j], v[56 + 2 * j + 1]});
+#pragma unroll
+    for (int j = 0; j < 4; ++j) W.b2[j] = __uint_as_float(v[88 + j]);
+}
+
 // Per-sample sums over the 64 features of two quantities at once: the lane's four features, the
 // four lane groups of a wavefront by shuffles, the four wavefronts through LDS.
 __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (&a)[4], const float (&b)[4], float &A, float &B) {
@@ -181,7 +320,7 @@ __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (
     slot ^= 1;
 }
 
-template <int METHOD, int CTRL>
+template <int METHOD, int CTRL, typename Weights>
 __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float> p, const float *packed, const MlpOut o) {
     using T = float;
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
@@ -200,25 +339,9 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
     int slot = 0;
 
     // ---- weights into registers ----
-    MlpWeights W;
-    {
-        const float4 *src = reinterpret_cast<const float4 *>(packed) + tid;
-        float v[MLP_REGS];
-#pragma unroll
-        for (int i = 0; i < MLP_REGS / 4; ++i) {
-            const float4 u = src[i * 256];
-            v[4 * i] = u.x, v[4 * i + 1] = u.y, v[4 * i + 2] = u.z, v[4 * i + 3] = u.w;
-        }
-#pragma unroll
-        for (int j = 0; j < 68; ++j) W.w1[j / 4][j % 4] = v[j];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) W.b1[j / 4][j % 4] = v[68 + j];
-#pragma unroll
-        for (int j = 0; j < 64; ++j) W.w2[j / 16][(j / 4) % 4][j % 4] = v[84 + j];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) W.b2[j] = v[148 + j];
-    }
-    for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns 65..67
+    Weights W;
+    mlp_load(W, packed, tid);
+    for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns from 65 on
     for (int i = tid; i < rows * E; i += 256) te_s[i] = p.t_eval[b0 * E + i];
     __syncthreads();
 
@@ -384,39 +507,50 @@ __global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float>
     publish_flags(p);
 }
 
-template <int METHOD, int CTRL> static int launch_mlp(const tode_solve_args &a, const tode_controller &c, const MlpOut &o, hipStream_t stream) {
+template <int METHOD, int CTRL, typename Weights> static int launch_mlp(const tode_solve_args &a, const tode_controller &c, const MlpOut &o, hipStream_t stream) {
     SolveParams<float> p = make_params<float>(a, c);
     reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
     const size_t lds = (size_t)MLP_TILE * a.n_eval * sizeof(float);
     const unsigned blocks = (unsigned)((a.batch + MLP_TILE - 1) / MLP_TILE);
-    timing_before(stream, "tode::solve_mlp_kernel");
-    hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
+    timing_before(stream, std::is_same<Weights, MlpWeightsBf16>::value ? "tode::solve_mlp_kernel (bfloat16 matrix inputs)" : "tode::solve_mlp_kernel");
+    hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }
 
+template <typename Weights> static int solve_mlp_with(const tode_solve_args &a, const tode_controller &c, const MlpOut &o, hipStream_t s) {
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch_mlp<0, 0, Weights>(a, c, o, s);
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch_mlp<0, 1, Weights>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch_mlp<1, 0, Weights>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch_mlp<1, 1, Weights>(a, c, o, s);
+    return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
+}
+
 int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
-    if (a.n_features != MLP_F || a.n_shared_params != (long long)TODE_MLP_PACKED_SIZE)
+    const bool f32 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE, bf16 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE_BF16;
+    if (a.n_features != MLP_F || !(f32 || bf16))
         return fail(TODE_E_UNSUPPORTED,
                     "the MLP kernel is built for 64 features and 256 hidden units, with the weights packed by tode_mlp_pack_weights "
-                    "(%d values); got F=%d and %lld shared parameters", TODE_MLP_PACKED_SIZE, a.n_features, (long long)a.n_shared_params);
+                    "(%d or %d values); got F=%d and %lld shared parameters", TODE_MLP_PACKED_SIZE, TODE_MLP_PACKED_SIZE_BF16, a.n_features,
+                    (long long)a.n_shared_params);
     if (!a.shared_params) return fail(TODE_E_INVALID, "null shared_params");
     if (a.n_eval > 512) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the MLP kernel", a.n_eval);
     if (a.batch > (long long)INT_MAX * MLP_TILE) return fail(TODE_E_UNSUPPORTED, "batch too large");
     MlpOut o{ns, na, ni, st};
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch_mlp<0, 0>(a, c, o, s);
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch_mlp<0, 1>(a, c, o, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch_mlp<1, 0>(a, c, o, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch_mlp<1, 1>(a, c, o, s);
-    return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
+    return f32 ? solve_mlp_with<MlpWeights>(a, c, o, s) : solve_mlp_with<MlpWeightsBf16>(a, c, o, s);
 }
 
-int mlp_pack_weights(const float *raw, long long n_raw, float *packed, hipStream_t s) {
-    static_assert(TODE_MLP_PACKED_SIZE == MLP_REGS * 256, "packed size");
+int mlp_pack_weights(const float *raw, long long n_raw, int matrix_inputs, float *packed, hipStream_t s) {
+    static_assert(TODE_MLP_PACKED_SIZE == MLP_REGS * 256 && TODE_MLP_PACKED_SIZE_BF16 == MLP_REGS_BF16 * 256, "packed sizes");
     if (!raw || !packed) return fail(TODE_E_INVALID, "null pointer");
     if (n_raw != MLP_RAW) return fail(TODE_E_UNSUPPORTED, "expected W1 [256 x 65] | b1 [256] | W2 [64 x 256] | b2 [64] = %lld values, got %lld", MLP_RAW, n_raw);
-    hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed);
+    if (matrix_inputs == TODE_MLP_INPUTS_F32)
+        hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed);
+    else if (matrix_inputs == TODE_MLP_INPUTS_BF16)
+        hipLaunchKernelGGL(mlp_pack_bf16_kernel, dim3((MLP_REGS_BF16 * 256 + 255) / 256), dim3(256), 0, s, raw, reinterpret_cast<unsigned *>(packed));
+    else
+        return fail(TODE_E_INVALID, "unknown matrix input type %d", matrix_inputs);
     return check_hip(hipGetLastError(), "tode_mlp_pack_weights launch");
 }
 
