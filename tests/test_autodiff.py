@@ -1,0 +1,218 @@
+"""Gradients through the solve loop (AutoDiffAdjoint with a y0 or parameters that require grad).
+
+CPU: the differentiable restatement of one loop iteration (torchode_amd/autodiff.py::Replay) is
+driven as a loop of its own and compared with the ATen-op oracle of the whole loop.  GPU: the
+reference's gradcheck cases for this adjoint (tests/adjoint_test.py:400-496, "autodiff"), gradients
+against torch autograd through the closed form y0 expm(A t), and against the backsolve adjoint.
+"""
+import pytest
+import torch
+import torch.nn as nn
+
+import torchode_amd as to
+from oracle import torch_loop
+from torchode_amd.autodiff import Replay, simulate_hits
+
+gpu = pytest.mark.gpu
+A0 = [[-1.4534, -0.3726, -0.7916], [-1.0553, 0.9511, 0.1316], [-1.8320, -0.7707, -1.0867]]
+Y0 = [[0.33, 1.2, -0.4], [0.55, -0.8, 1.23]]
+T_EVAL = [[0.0, 1.77, 3.0], [2.0, 3.5, 6.0]]
+
+
+class LinearDynamics(nn.Module):
+    def __init__(self, A):
+        super().__init__()
+        self.register_parameter("A", A)
+
+    def forward(self, t, y):
+        return y @ self.A
+
+
+class Forced(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.w = nn.Parameter(torch.tensor([[0.3, -1.2], [1.5, 0.1]], dtype=torch.float64))
+
+    def forward(self, t, y):
+        return torch.tanh(y @ self.w) * torch.cos(1.3 * t)[..., None] - 0.2 * y
+
+
+# ---------------------------------------------------------------------------------------------
+# CPU: the restated iteration against the oracle's loop
+# ---------------------------------------------------------------------------------------------
+
+
+def drive(replay: Replay, y0, dt0=None):
+    """The loop of reference adjoints.py:50-311 around Replay.attempt / advance."""
+    B = y0.shape[0]
+    t_start, t_end, t_eval, direction = replay.t_start, replay.t_end, replay.t_eval, replay.direction
+    f0 = replay.f(t_start, y0)
+    dt = replay.first_step(y0, f0) if dt0 is None else dt0
+    dt = torch.minimum(torch.maximum(dt, replay.t_lo - t_start), replay.t_hi - t_start)
+    one = torch.ones(B, dtype=y0.dtype)
+    state = dict(t=t_start, dt=dt, y=y0, k0=f0, prev=one, pprev=one, running=torch.ones(B, dtype=torch.bool))
+    E = t_eval.shape[1]
+    ys = torch.zeros(B, E, y0.shape[1], dtype=y0.dtype)
+    pending = torch.ones(B, E, dtype=torch.bool)
+    at_start = t_eval[:, 0] == t_start
+    ys[at_start, 0] = y0[at_start]
+    pending[:, 0] = ~at_start
+    n_steps, n_acc = torch.zeros(B, dtype=torch.long), torch.zeros(B, dtype=torch.long)
+    while True:
+        attempt = replay.attempt(state)
+        accept = attempt[2] < 1
+        move = accept & state["running"]
+        t_new = torch.where(move, state["t"] + state["dt"], state["t"])
+        running_new = direction * t_new < direction * t_end
+        hit = pending & (direction[:, None] * t_new[:, None] >= direction[:, None] * t_eval)
+        idx = hit.nonzero()
+        (y, k0, t, dt, prev, pprev), values = replay.advance(state, attempt, accept, running_new, (idx[:, 0], idx[:, 1]) if len(idx) else None)
+        if values is not None:
+            ys = ys.index_put((idx[:, 0], idx[:, 1]), values)
+        pending = pending & ~hit
+        n_steps += state["running"]
+        n_acc += move
+        state = dict(t=t, dt=dt, y=y, k0=k0, prev=prev, pprev=pprev, running=running_new)
+        if not running_new.any():
+            return ys, n_steps, n_acc
+
+
+@pytest.mark.parametrize("method,ctrl", [
+    ("dopri5", dict(kind="integral", atol=1e-6, rtol=1e-4)),
+    ("tsit5", dict(kind="pid", atol=1e-7, rtol=1e-5, pcoeff=0.2, icoeff=0.5, dcoeff=0.1)),
+])  # fmt: skip
+def test_restated_iteration_reproduces_the_oracle_loop(method, ctrl):
+    w = to.workloads.make("vdp", batch=40, dtype=torch.float64)
+    w.t_eval[3, 0] = 0.25  # a first evaluation point that is not t_start
+    spec = dict(ctrl)
+    kind = spec.pop("kind")
+    controller = to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
+    problem = to.InitialValueProblem(w.y0, t_start=torch.zeros(40, dtype=torch.float64), t_end=w.t_eval[:, -1], t_eval=w.t_eval)
+    step_method = to.Tsit5() if method == "tsit5" else to.Dopri5()
+    replay = Replay(step_method, controller, to.ODETerm(w.f), None, problem, True)
+    with torch.no_grad():
+        ys, n_steps, n_acc = drive(replay, w.y0)
+    ref = torch_loop.solve(w.f, w.y0, w.t_eval, method=method, controller=torch_loop.Controller(**ctrl), t_start=problem.t_start, t_end=problem.t_end)
+    assert torch.equal(n_steps, ref["n_steps"]) and torch.equal(n_acc, ref["n_accepted"]) and (n_acc < n_steps).any()
+    torch.testing.assert_close(ys, ref["ys"], rtol=1e-7, atol=1e-8)  # same operations, other association: rounding differences grow along stiff samples
+
+
+def test_recorded_times_give_back_the_evaluation_schedule():
+    t_eval = torch.tensor([[0.0, 0.5, 1.0, 2.0], [1.0, 0.6, 0.2, 0.0]])
+    problem = to.InitialValueProblem(torch.zeros(2, 1), t_eval=t_eval)
+    replay = Replay(to.Dopri5(), to.IntegralController(1e-3, 1e-3), to.ODETerm(lambda t, y: y), None, problem, True)
+    times = [[0.0, 1.0], [0.4, 0.7], [0.4, 0.1], [1.2, 0.0], [2.0, 0.0]]  # sample 0 has a rejected step, sample 1 runs backwards
+    hits = simulate_hits(replay, [dict(t=torch.tensor(t)) for t in times], 4)
+    got = [None if h is None else sorted(zip(h[0].tolist(), h[1].tolist())) for h in hits]
+    assert got == [None, [(1, 1), (1, 2)], [(0, 1), (0, 2), (1, 3)], [(0, 3)]]
+    # without evaluation points: the end point, by the last iteration, for every sample
+    none = simulate_hits(replay, [dict(t=torch.tensor(t)) for t in times], 0)
+    assert none[:3] == [None, None, None] and none[3][0].tolist() == [0, 1] and none[3][1] is None
+
+
+# ---------------------------------------------------------------------------------------------
+# GPU
+# ---------------------------------------------------------------------------------------------
+
+
+def closed_form(y0, A, t_eval):
+    dts = t_eval - t_eval[:, :1]
+    return torch.einsum("bf,befg->beg", y0, torch.matrix_exp(A[None, None] * dts[:, :, None, None]))
+
+
+def inputs():
+    y0 = torch.tensor(Y0, dtype=torch.double, device="cuda", requires_grad=True)
+    A = nn.Parameter(torch.tensor(A0, dtype=torch.double, device="cuda"))
+    return y0, A
+
+
+@gpu
+def test_gradients_with_t_eval():
+    """reference tests/adjoint_test.py:401-442, adjoint = "autodiff" """
+    y0, A = inputs()
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+
+    def loss(y0, params):
+        term = to.ODETerm(LinearDynamics(params))
+        adjoint = to.AutoDiffAdjoint(to.Dopri5(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0))
+        return adjoint.solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term).ys.mean()
+
+    assert torch.autograd.gradcheck(loss, (y0, A))
+
+
+@gpu
+def test_gradients_without_t_eval():
+    """reference tests/adjoint_test.py:445-496, adjoint = "autodiff": passes only with the gradient
+    through the step sizes, there as here"""
+    y0, A = inputs()
+    t_start, t_end = torch.tensor([0.0, 2.0], dtype=torch.double, device="cuda"), torch.tensor([3.0, 6.0], dtype=torch.double, device="cuda")
+
+    def loss(through):
+        def fn(y0, params):
+            term = to.ODETerm(LinearDynamics(params))
+            adjoint = to.AutoDiffAdjoint(to.Dopri5(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0), backprop_through_step_size_control=through)
+            return adjoint.solve(to.InitialValueProblem(y0, t_start=t_start, t_end=t_end, t_eval=None), term=term).ys.mean()
+
+        return fn
+
+    assert torch.autograd.gradcheck(loss(True), (y0, A), atol=1e-5)
+    assert torch.autograd.gradcheck(loss(False), (y0, A), atol=1e-2)
+
+
+@gpu
+@pytest.mark.parametrize("method,controller", [
+    (to.Dopri5, lambda: to.IntegralController(1e-10, 1e-10)),
+    (to.Tsit5, lambda: to.PIDController(1e-10, 1e-10, 0.2, 0.5, 0.1)),
+])  # fmt: skip
+def test_gradients_match_the_closed_form(method, controller):
+    y0, A = inputs()
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+    term = to.ODETerm(LinearDynamics(A))
+    solution = to.AutoDiffAdjoint(method(), controller()).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
+    assert solution.ys.requires_grad and (solution.stats["n_accepted"] > 10).all() and solution.stats["n_f_evals"].device.type == "cpu"
+    weights = torch.linspace(0.5, 1.5, solution.ys.numel(), dtype=torch.double, device="cuda").reshape(solution.ys.shape)
+    (solution.ys * weights).sum().backward()
+    y0_ref, A_ref = y0.detach().clone().requires_grad_(), A.detach().clone().requires_grad_()
+    (closed_form(y0_ref, A_ref, t_eval) * weights).sum().backward()
+    torch.testing.assert_close(y0.grad, y0_ref.grad, rtol=1e-7, atol=1e-8)
+    torch.testing.assert_close(A.grad, A_ref.grad, rtol=1e-7, atol=1e-8)
+    # the values are those of the solve without grad
+    with torch.no_grad():
+        plain = to.AutoDiffAdjoint(method(), controller()).solve(to.InitialValueProblem(y0.detach(), t_eval=t_eval), term=term)
+    assert torch.equal(plain.ys, solution.ys.detach()) and torch.equal(plain.stats["n_steps"], solution.stats["n_steps"])
+
+
+@gpu
+def test_parameter_gradients_agree_with_the_backsolve_adjoint_and_float32_runs():
+    torch.manual_seed(1)
+    f = Forced().cuda()
+    y0 = torch.randn(6, 2, dtype=torch.double, device="cuda")  # does not require grad: only the parameters do
+    t_eval = torch.linspace(0, 2, 5, dtype=torch.double, device="cuda").repeat(6, 1) + torch.arange(6, dtype=torch.double, device="cuda")[:, None] * 0.1
+    term = to.ODETerm(f)
+    ctrl = lambda: to.IntegralController(1e-9, 1e-9)
+    to.AutoDiffAdjoint(to.Tsit5(), ctrl()).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term).ys.square().sum().backward()
+    through_loop = f.w.grad.clone()
+    f.w.grad = None
+    to.BacksolveAdjoint(term, to.Tsit5(), ctrl()).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term).ys.square().sum().backward()
+    torch.testing.assert_close(through_loop, f.w.grad, rtol=1e-5, atol=1e-7)
+    # float32, large batch, rejected steps, both directions of time
+    f32 = Forced().cuda().float()
+    y0 = torch.randn(500, 2, device="cuda", requires_grad=True)
+    t_eval = torch.linspace(0, 3, 7, device="cuda").repeat(500, 1)
+    t_eval[::2] = t_eval[::2].flip(1)
+    sol = to.AutoDiffAdjoint(to.Dopri5(), to.PIDController(1e-5, 1e-4, 0.2, 0.5, 0.0)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=to.ODETerm(f32))
+    sol.ys[:, -1].sum().backward()
+    assert torch.isfinite(y0.grad).all() and torch.isfinite(f32.w.grad).all() and (sol.stats["n_accepted"] < sol.stats["n_steps"]).any()
+
+
+@gpu
+def test_what_is_not_differentiated_says_so():
+    y0, A = inputs()
+    term = to.ODETerm(LinearDynamics(A))
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
+    with pytest.raises(RuntimeError, match="times"):
+        to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
+    with pytest.raises(RuntimeError, match="BacksolveAdjoint"):
+        to.AutoDiffAdjoint(to.Heun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
+    with torch.no_grad():  # no graph asked for: any configuration solves
+        to.AutoDiffAdjoint(to.Heun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)

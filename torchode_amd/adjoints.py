@@ -38,10 +38,10 @@ def _library_object(obj, classes) -> bool:
 class AutoDiffAdjoint(nn.Module):
     """Solves a batch of initial value problems with per-sample adaptive steps.
 
-    Same constructor and ``solve`` signature as the reference.  The forward solve
-    runs in HIP kernels; it does not record an autograd graph
-    (``backprop_through_step_size_control`` is accepted for compatibility), and
-    inputs that require grad are rejected rather than silently detached.
+    Same constructor and ``solve`` signature as the reference.  The solve runs in HIP kernels.
+    With a ``y0`` or term parameters that require grad it takes the per-step kernels and records
+    the loop state per iteration, and the result is differentiable (``torchode_amd/autodiff.py``;
+    ``backprop_through_step_size_control`` as in the reference).
     """
 
     def __init__(
@@ -81,20 +81,32 @@ class AutoDiffAdjoint(nn.Module):
         term_ = term if term is not None else getattr(self.step_method, "term", None)
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
-        if torch.is_grad_enabled() and (
-            problem.y0.requires_grad
-            or problem.t_start.requires_grad
+        grad_on = torch.is_grad_enabled()
+        if grad_on and (
+            problem.t_start.requires_grad
             or problem.t_end.requires_grad
             or (problem.t_eval is not None and problem.t_eval.requires_grad)
             or (dt0 is not None and dt0.requires_grad)
         ):
-            raise RuntimeError(
-                "torchode_amd's solve loop is forward-only; call it under torch.no_grad() or detach the inputs"
-            )
-        if self._persistent_ok(problem, term_):
+            raise RuntimeError("torchode_amd differentiates a solve with respect to y0 and the term's parameters; times must not require grad")
+        wants_grad = grad_on and problem.y0.requires_grad
+        if not wants_grad and self._persistent_ok(problem, term_):
             sol = self._solve_persistent(problem, term_, dt0)
             if sol is not None:
                 return sol
+        if grad_on and not wants_grad and isinstance(term_, nn.Module):
+            wants_grad = any(p.requires_grad for p in term_.parameters())
+        if wants_grad:
+            # gradients through the loop: forward in the per-step kernels with a record of the loop
+            # state, backward by a reverse sweep over the record
+            if not self._fused_ok(problem, term_):
+                raise RuntimeError(
+                    "gradients through the loop are built for Dopri5 / Tsit5 with the library's controllers (one dtype); "
+                    "with user-defined plug-ins call solve under torch.no_grad(), or use BacksolveAdjoint"
+                )
+            from . import autodiff
+
+            return autodiff.solve(self, problem, term_, dt0, args)
         if self._stepwise_ok(problem, term_):
             return self._solve_stepwise(problem, term_, dt0, args)
         return self._solve_protocol(problem, term, term_, dt0, args)
@@ -239,7 +251,7 @@ class AutoDiffAdjoint(nn.Module):
     # How many loop iterations are enqueued between two looks at the device flags.
     poll_first, poll_max = 4, 32
 
-    def _solve_stepwise(self, problem: InitialValueProblem, term: ODETerm, dt0, args) -> Solution:
+    def _solve_stepwise(self, problem: InitialValueProblem, term: ODETerm, dt0, args, record=None) -> Solution:
         """Arbitrary Python ``f``: per-step kernels around the user's torch RHS, loop state on the
         device, no host synchronisation per step (the host polls a flag every few iterations)."""
         lib = _lib.load()
@@ -311,6 +323,8 @@ class AutoDiffAdjoint(nn.Module):
 
         def iterate(n, stream):
             for _ in range(n):
+                if record is not None:
+                    record.snapshot(t, dt, y, k0, hist, ints)
                 for i in range(1, 7):
                     tt, yy = stage_buffers(i)
                     _lib.check(lib.tode_step_stage(sref, cref, i, stream), "tode_step_stage")
@@ -327,7 +341,7 @@ class AutoDiffAdjoint(nn.Module):
             fl = flags.tolist()  # host/device synchronisation, once per chunk of iterations
             if fl[_lib.STEP_FLAG_STOPPED]:
                 break
-            if self.graph_iterations and graph is None:
+            if self.graph_iterations and graph is None and record is None:
                 # (the eager iterations above have also warmed up whatever f uses)
                 graph = self._record(lambda st: iterate(int(self.graph_iterations), st), y0)
             elif graph is not None:
@@ -336,6 +350,9 @@ class AutoDiffAdjoint(nn.Module):
                 chunk = min(2 * chunk, self.poll_max)
         keep.clear()
         del graph  # frees the memory f's intermediate tensors were recorded with
+        if record is not None:
+            record.snapshot(t, dt, y, k0, hist, ints)
+            record.iterations = fl[_lib.STEP_FLAG_ITERATIONS]
 
         out = new(4, B, dt=torch.int64)
         _lib.check(lib.tode_step_stats(sref, *(_lib.ptr(out[i]) for i in range(4)), stream), "tode_step_stats")

@@ -1,0 +1,291 @@
+"""Gradients through the solve loop itself (reference adjoints.py:33-40, 111-113, 145-147: the
+reference records every torch operation of its loop; ``backprop_through_step_size_control``
+decides whether the step sizes count as functions of the inputs).
+
+Here the forward pass runs in the per-step HIP kernels and keeps, per loop iteration, a copy of
+the small loop state (t, dt, y, the FSAL derivative, the controller history, two counters).  The
+backward pass walks the iterations in reverse: it restates one iteration as differentiable torch
+operations on the stored state -- same stages, error ratio, step size rule and dense output, with
+the accept / running / evaluation decisions taken from the record -- and pulls the cotangents of
+the next state and of the evaluation points back through it, which evaluates ``f`` and its
+vector-Jacobian products six times per iteration.  Memory: one state copy per iteration instead of
+the reference's whole operation graph.
+
+Gradients flow to ``y0`` and to the parameters of the term; times (``t_start``, ``t_end``,
+``t_eval``) and ``args`` are treated as constants.
+"""
+from math import sqrt
+from typing import Any, List, Optional, Sequence
+
+import torch
+
+from . import _lib
+from .problems import InitialValueProblem
+
+
+class LoopRecord:
+    """State before each iteration (and after the last): what the forward pass hands to the backward pass."""
+
+    FIELDS = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
+
+    def __init__(self):
+        self.states: List[tuple] = []
+        self.iterations = 0  # set by the forward pass when the loop has stopped
+
+    def snapshot(self, t, dt, y, k0, hist, ints):
+        self.states.append((t.clone(), dt.clone(), y.clone(), k0.clone(), hist[0].clone(), hist[1].clone(), ints[0].clone(), ints[3].clone()))
+
+    def trimmed(self, iterations: int) -> List[dict]:
+        """States 0..iterations; iterations enqueued after the batch had stopped changed nothing."""
+        states = self.states[:iterations] + [self.states[-1]]
+        return [dict(zip(self.FIELDS, s)) for s in states]
+
+
+class Replay:
+    """One loop iteration (and the start of the loop) as differentiable torch operations."""
+
+    def __init__(self, method, controller, term, args, problem: InitialValueProblem, through_control: bool):
+        tab = method.tableau
+        self.a = [[float(x) for x in row] for row in tab.a.tolist()]
+        self.c = [float(x) for x in tab.c.tolist()]
+        self.b_err = [float(x) for x in tab.b_err.tolist()]
+        self.b_other = [[float(x) for x in row] for row in tab.b_other.tolist()]
+        self.tsit5 = method.method_id == _lib.TSIT5
+        self.order = float(method.convergence_order())
+        c = controller.c_struct()
+        self.pid = c.kind == _lib.CTRL_PID
+        self.atol, self.rtol = float(c.atol), float(c.rtol)
+        self.safety, self.fmin, self.fmax = float(c.safety), float(c.factor_min), float(c.factor_max)
+        self.dt_min = float(c.dt_min) if c.has_dt_min else None
+        self.dt_max = float(c.dt_max) if c.has_dt_max else None
+        if self.pid:
+            k_i, k_p, k_d = c.icoeff / self.order, c.pcoeff / self.order, c.dcoeff / self.order
+            self.e1, self.e2, self.e3 = -(k_i + k_p + k_d), k_p + 2 * k_d, -k_d
+        else:
+            self.e1, self.e2, self.e3 = -1.0 / self.order, 0.0, 0.0
+        self.term, self.args = term, args
+        self.through_control = through_control
+        self.t_start, self.t_end, self.t_eval = problem.t_start, problem.t_end, problem.t_eval
+        self.t_lo, self.t_hi = torch.minimum(self.t_start, self.t_end), torch.maximum(self.t_start, self.t_end)
+        self.direction = torch.where(self.t_end > self.t_start, 1.0, -1.0).to(self.t_start.dtype)
+
+    def f(self, t, y):
+        return self.term.f(t, y, self.args) if self.term.with_args else self.term.f(t, y)
+
+    def rms(self, x):
+        return torch.linalg.vector_norm(x / sqrt(x.shape[1]), ord=2, dim=1)
+
+    # ---- reference step_size_controllers.py:431-490 / 776-835 ----
+    def first_step(self, y0, f0):
+        inv = 1.0 / (self.atol + self.rtol * y0.abs())
+        d0, d1 = self.rms(y0 * inv), self.rms(f0 * inv)
+        small = (d0 < 1e-5) | (d1 < 1e-5)
+        h0 = torch.where(small, torch.full_like(d0, 1e-6), 0.01 * d0 / torch.where(small, torch.ones_like(d1), d1))
+        h0 = torch.minimum(h0, (self.t_end - self.t_start).abs().to(h0.dtype))
+        step = (self.direction.to(h0.dtype) * h0)
+        f1 = self.f(self.t_start + step.to(self.t_start.dtype), y0 + step[:, None] * f0)
+        d2 = self.rms((f1 - f0) * inv) / h0
+        if not self.pid:
+            d2 = torch.where(h0 == 0, torch.full_like(d2, float("inf")), d2)
+        m = torch.maximum(d1, d2)
+        tiny = m <= 1e-15
+        h1 = torch.where(tiny, torch.clamp_min(h0 * 1e-3, 1e-6), (0.01 / torch.where(tiny, torch.ones_like(m), m)) ** (1.0 / self.order))
+        return (self.direction.to(h0.dtype) * torch.minimum(100 * h0, h1)).to(self.t_start.dtype)
+
+    # ---- reference runge_kutta.py:226-279, step_size_controllers.py:370-429 / 715-774, adjoints.py:150-255 ----
+    def attempt(self, state: dict):
+        """The step from ``state`` and the controller's view of it: stage derivatives, y1, error ratio
+        and the step size it proposes."""
+        t, dt, y, k0, prev, pprev = (state[k] for k in ("t", "dt", "y", "k0", "prev", "pprev"))
+        dtd = dt.to(y.dtype)
+        ks = [k0]
+        yi = y
+        for i in range(1, 7):
+            s = sum(self.a[i][j] * ks[j] for j in range(i) if self.a[i][j] != 0.0)
+            yi = y + dtd[:, None] * s
+            ks.append(self.f(t + self.c[i] * dt, yi))
+        y1 = yi
+        err = dtd[:, None] * sum(self.b_err[s] * ks[s] for s in range(7) if self.b_err[s] != 0.0)
+        scale = self.atol + self.rtol * torch.maximum(y.abs(), y1.abs())
+        ratio = torch.clamp_min(self.rms(err.abs() / scale), 1e-38)
+        factor = self.safety * ratio**self.e1
+        if self.pid:
+            if self.e2 != 0.0:
+                factor = factor * prev**self.e2
+            if self.e3 != 0.0:
+                factor = factor * pprev**self.e3
+        dt_next = dt * factor.clamp(self.fmin, self.fmax).to(dt.dtype)
+        if self.dt_min is not None or self.dt_max is not None:
+            dt_next = torch.sign(dt_next) * dt_next.abs().clamp(self.dt_min, self.dt_max)
+        if not self.through_control:
+            dt_next = dt_next.detach()
+        return ks, y1, ratio, dt_next
+
+    def advance(self, state: dict, attempt, accept, running_new, hits):
+        """The loop's update with the decisions given: the next state's differentiable part, and the
+        dense-output values at ``hits`` = (samples, points)."""
+        t, dt, y, k0, prev, pprev, running = (state[k] for k in ("t", "dt", "y", "k0", "prev", "pprev", "running"))
+        ks, y1, ratio, dt_next = attempt
+        move = accept & running
+        y_new = torch.where(move[:, None], y1, y)
+        k0_new = torch.where(move[:, None], ks[6], k0)
+        t_new = torch.where(move, t + dt, t)
+        dt_new = torch.where(running_new, dt_next, dt)
+        dt_new = torch.minimum(torch.maximum(dt_new, self.t_lo - t_new), self.t_hi - t_new)
+        keep = running_new & accept
+        prev_new, pprev_new = (torch.where(keep, ratio, prev), torch.where(keep, prev, pprev)) if self.pid else (prev, pprev)
+
+        values = None
+        if hits is not None:
+            rows, points = hits
+            at = self.t_eval[rows, points] if points is not None else self.t_end[rows]
+            values = self.dense(t[rows], dt[rows], y[rows], y1[rows], [k[rows] for k in ks], at)
+        return (y_new, k0_new, t_new, dt_new, prev_new, pprev_new), values
+
+    def iteration(self, state: dict, accept, running_new, hits):
+        return self.advance(state, self.attempt(state), accept, running_new, hits)
+
+    # ---- reference tsit5.py:123-139, dopri5.py:53-60, interpolation.py:25-40, 138-170 ----
+    def dense(self, t0, dt, y0, y1, ks, at):
+        h = dt.to(y0.dtype)[:, None]
+        weighted = lambda w: h * sum(w[s] * ks[s] for s in range(7) if w[s] != 0.0)
+        if self.tsit5:
+            q = [y0, h * ks[0], weighted(self.b_other[0]), weighted(self.b_other[1]), weighted(self.b_other[2])]
+        else:
+            f0, f1, mid = h * ks[0], h * ks[6], y0 + weighted(self.b_other[0])
+            q = [
+                y0,
+                f0,
+                f1 - 4 * f0 - 11 * y0 - 5 * y1 + 16 * mid,
+                5 * f0 - 3 * f1 + 18 * y0 + 14 * y1 - 32 * mid,
+                2 * (f1 - f0) - 8 * (y1 + y0) + 16 * mid,
+            ]
+        den = (t0 + dt) - t0
+        den = torch.where(den.abs() > 0, den, torch.ones_like(den))
+        x = ((at - t0) / den).to(y0.dtype)[:, None]
+        out = q[4]
+        for p in (3, 2, 1, 0):
+            out = out * x + q[p]
+        return out
+
+
+def simulate_hits(replay: Replay, states: Sequence[dict], n_eval: int):
+    """Which evaluation points each iteration wrote (adjoints.py:215-234), from the recorded times:
+    a list of (samples, points) index pairs, None where an iteration wrote nothing."""
+    if n_eval == 0:
+        return [None] * (len(states) - 2) + [(torch.arange(states[0]["t"].shape[0], device=states[0]["t"].device), None)]
+    t_eval, direction = replay.t_eval, replay.direction
+    pending = torch.ones_like(t_eval, dtype=torch.bool)
+    pending[:, 0] = t_eval[:, 0] != replay.t_start
+    hits = []
+    for n in range(len(states) - 1):
+        t_new = states[n + 1]["t"]
+        passed = direction[:, None] * t_new[:, None] >= direction[:, None] * t_eval
+        hit = pending & passed
+        pending = pending & ~hit
+        idx = hit.nonzero()
+        hits.append((idx[:, 0], idx[:, 1]) if idx.shape[0] > 0 else None)
+    return hits
+
+
+class SolveThroughLoop(torch.autograd.Function):
+    """Forward: the per-step kernels with a record.  Backward: the reverse sweep over it."""
+
+    @staticmethod
+    def forward(ctx, adjoint, problem, term, dt0, args, y0, *params):
+        record = LoopRecord()
+        detached = lambda x: None if x is None else x.detach()
+        plain = InitialValueProblem(y0.detach(), detached(problem.t_start), detached(problem.t_end), detached(problem.t_eval))
+        with torch.no_grad():
+            solution = adjoint._solve_stepwise(plain, term, detached(dt0), args, record=record)
+        ctx.adjoint, ctx.problem, ctx.term, ctx.dt0, ctx.args = adjoint, plain, term, dt0, args
+        ctx.record, ctx.params = record, params
+        stats = solution.stats
+        n_f_evals = stats["n_f_evals"] if "n_f_evals" in stats else torch.empty(0, dtype=torch.long)
+        outs = (solution.ys, solution.status, stats["n_steps"], stats["n_accepted"], stats["n_initialized"], n_f_evals)
+        ctx.mark_non_differentiable(*outs[1:])
+        return outs
+
+    @staticmethod
+    def backward(ctx, grad_ys, *unused):
+        adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
+        replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, ctx.args, problem, adjoint.backprop_through_step_size_control)
+        states = ctx.record.trimmed(ctx.record.iterations)
+        E = problem.n_evaluation_points
+        hits = simulate_hits(replay, states, E)
+        y0 = problem.y0
+        names = ("y", "k0", "t", "dt", "prev", "pprev")
+        adj = {k: None for k in names}
+        grad_params = [None] * len(params)
+
+        def add(total, part):
+            return part if total is None else (total if part is None else total + part)
+
+        for n in range(len(states) - 2, -1, -1):
+            now, then = states[n], states[n + 1]
+            accept = (then["n_accepted"] - now["n_accepted"]) > 0
+            live = dict(now, running=now["running"] != 0)
+            with torch.enable_grad():
+                for k in names:
+                    live[k] = now[k].detach().requires_grad_()
+                outs, values = replay.iteration(live, accept, then["running"] != 0, hits[n])
+                targets, cotangents = [], []
+                for k, out in zip(names, outs):
+                    if adj[k] is not None and out.requires_grad:
+                        targets.append(out)
+                        cotangents.append(adj[k])
+                if values is not None:
+                    rows, points = hits[n]
+                    targets.append(values)
+                    cotangents.append(grad_ys[rows, points] if points is not None else grad_ys[rows, 0])
+                if not targets:
+                    adj = {k: None for k in names}
+                    continue
+                wrt = [live[k] for k in names] + params
+                grads = torch.autograd.grad(targets, wrt, cotangents, allow_unused=True)
+            adj = dict(zip(names, grads[: len(names)]))
+            for i, g in enumerate(grads[len(names) :]):
+                grad_params[i] = add(grad_params[i], g)
+
+        # ---- the start of the loop: y = y0, k0 = f(t_start, y0), dt from the start step rule or dt0 ----
+        with torch.enable_grad():
+            y_in = y0.detach().requires_grad_()
+            targets, cotangents = [], []
+            if adj["y"] is not None:
+                targets.append(y_in * 1.0)
+                cotangents.append(adj["y"])
+            need_f0 = adj["k0"] is not None or (adj["dt"] is not None and ctx.dt0 is None and replay.through_control)
+            if need_f0:
+                f0 = replay.f(problem.t_start, y_in)
+                if adj["k0"] is not None:
+                    targets.append(f0)
+                    cotangents.append(adj["k0"])
+                if adj["dt"] is not None and ctx.dt0 is None and replay.through_control:
+                    dt_first = replay.first_step(y_in, f0)
+                    dt_first = torch.minimum(torch.maximum(dt_first, replay.t_lo - problem.t_start), replay.t_hi - problem.t_start)
+                    if dt_first.requires_grad:
+                        targets.append(dt_first)
+                        cotangents.append(adj["dt"])
+            grad_y0 = None
+            if targets:
+                grads = torch.autograd.grad(targets, [y_in] + params, cotangents, allow_unused=True)
+                grad_y0 = grads[0]
+                for i, g in enumerate(grads[1:]):
+                    grad_params[i] = add(grad_params[i], g)
+        if E > 0:
+            at_start = problem.t_eval[:, 0] == problem.t_start
+            first = torch.where(at_start[:, None], grad_ys[:, 0], torch.zeros_like(grad_ys[:, 0]))
+            grad_y0 = add(grad_y0, first)
+        return (None, None, None, None, None, grad_y0, *grad_params)
+
+
+def solve(adjoint, problem: InitialValueProblem, term, dt0: Optional[torch.Tensor], args: Any):
+    """``AutoDiffAdjoint.solve`` for a ``y0`` or term parameters that require grad."""
+    from .solution import Solution
+
+    params = [p for p in term.parameters() if p.requires_grad]
+    ys, status, n_steps, n_accepted, n_initialized, n_f_evals = SolveThroughLoop.apply(adjoint, problem, term, dt0, args, problem.y0, *params)
+    stats = {"n_f_evals": n_f_evals} if term.with_stats else {}
+    stats.update(n_steps=n_steps, n_accepted=n_accepted, n_initialized=n_initialized)
+    ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+    return Solution(ts=ts, ys=ys, stats=stats, status=status)
