@@ -380,3 +380,71 @@ def test_flags_on_the_host_over_more_calls_than_there_are_slots_and_when_the_bat
     # empty batch: nothing is launched, the start values come back
     empty = w._replace(f=to.VanDerPol(w.f.mu[:0]), y0=w.y0[:0], t_eval=w.t_eval[:0])
     assert _fast_call(empty, sync=True)[2] == [0, 2**31 - 1, 0, 0]
+
+
+def test_flags_on_the_host_from_several_threads_and_streams_at_once():
+    """Every call takes a flag slot of its own: concurrent solves must not see each other's flags."""
+    import threading
+
+    sizes = [64, 1000, 3000, 129, 2048, 700]
+    works = [to.workloads.make("vdp", batch=n, dtype=F32, device="cuda") for n in sizes]
+    torch.cuda.synchronize()
+    want = [_fast_call(w, sync=False) for w in works]
+    errors = []
+
+    def run(i):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for _ in range(40):
+                    ys, out, flags = _fast_call(works[i], sync=True)
+                    assert flags == want[i][2], (i, flags, want[i][2])
+                assert torch.equal(ys, want[i][0]) and torch.equal(out, want[i][1])
+        except Exception as e:  # surfaced below: an exception in a thread does not fail the test by itself
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(len(sizes))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
+def test_plain_fast_entry_point_in_a_hip_graph():
+    """The entry point without host synchronisation can be recorded: the graph is replayed several times,
+    with other work and synchronisations in between, and every replay is checked against the eager result."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    w = to.workloads.make("vdp", batch=5000, dtype=F32, device="cuda")
+    ys_want, out_want, flags_want = _fast_call(w, sync=False)
+    B, F = w.y0.shape
+    E = w.t_eval.shape[1]
+    params = w.f.builtin_params()
+    ys = torch.zeros((B, E, F), device="cuda")
+    out = torch.zeros((4, B), dtype=torch.int64, device="cuda")
+    flags = torch.zeros(_lib.FLAG_WORDS, dtype=torch.int32, device="cuda")
+    spec = dict(w.controller)
+    spec.pop("kind")
+    ctrl = to.PIDController(**spec).c_struct()
+    a = _lib.SolveArgs()
+    a.dtype, a.method, a.term, a.n_features, a.n_eval, a.n_params, a.batch, a.max_steps, a.iteration_cap = 0, 1, w.f.builtin_kind, F, E, 1, B, -1, -1
+    a.y0, a.t_start, a.t_end, a.t_eval = w.y0.data_ptr(), w.t_eval[:, 0].data_ptr(), w.t_eval[:, -1].data_ptr(), w.t_eval.data_ptr()
+    a.t_start_stride = a.t_end_stride = E
+    a.params, a.ys, a.flags = params.data_ptr(), ys.data_ptr(), flags.data_ptr()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        rc = lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), _lib.stream_of(w.y0))
+        graph.capture_end()
+    _lib.check(rc, "tode_solve_builtin_fast under capture")
+    torch.cuda.current_stream().wait_stream(side)
+    assert not ys.any()  # recording runs nothing
+    for i in range(4):
+        ys.zero_(), out.zero_(), flags.zero_()
+        (torch.randn(500, 500, device="cuda") @ torch.randn(500, 500, device="cuda")).sum().item()  # other work, a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ys, ys_want) and torch.equal(out, out_want) and flags.tolist() == flags_want, i
