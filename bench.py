@@ -124,7 +124,7 @@ def main():
     except RuntimeError:
         # no whole-solve kernel for this workload: the solve is a sequence of per-call kernels
         # around the torch right-hand side, and the figure below is over the whole solve
-        per_step = args.path == "per-step" and F < 64
+        per_step = args.path == "per-step"
         kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
         if per_step and args.graph_iterations:
             kernel_name += f", {args.graph_iterations} iterations per HIP graph replay"

@@ -296,3 +296,56 @@ def test_mlp_kernel_with_bfloat16_matrix_inputs():
     slope = (sol.ys[:, 1] - sol.ys[:, 0]) / 1e-3
     want = w2.f(torch.zeros(64, device="cuda"), w2.y0)
     assert mixed_error(slope.double().cpu(), want.double().cpu()) < 2e-2
+
+
+# ---------------------------------------------------------------------------------------------
+# the per-step path on long rows (one wavefront per sample) against the protocol path
+# ---------------------------------------------------------------------------------------------
+
+
+def per_step_and_protocol(f, y0, t_eval, method, ctrl, t_start=None, t_end=None, **kw):
+    """Library method and controller around a plain callable: per-step kernels.  The same with a
+    subclass of the method: protocol path.  Both form every sum in the same fixed order."""
+    lib_m, own_m = {"tsit5": (to.Tsit5, OwnTsit5), "dopri5": (to.Dopri5, OwnDopri5)}[method]
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
+    opaque = lambda t, y: f(t, y)
+    a = to.AutoDiffAdjoint(lib_m(), make_controller(ctrl), max_steps=kw.pop("max_steps", None)).solve(problem, to.ODETerm(opaque), **kw)
+    b = to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(opaque), **kw)
+    return a, b
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("features", [64, 100, 300, 1024])
+def test_per_step_path_on_long_rows_equals_the_protocol_path(features, dtype):
+    g = torch.Generator().manual_seed(features)
+    B, E = 37, 9
+    W = (torch.randn((features, features), generator=g, dtype=torch.float64) / features**0.5).to(dtype).cuda()
+    y0 = torch.randn((B, features), generator=g, dtype=torch.float64).to(dtype).cuda()
+    t1 = (1.0 + 2.0 * torch.rand(B, generator=g, dtype=torch.float64)).to(dtype)
+    t_eval = (t1[:, None] * torch.linspace(0, 1, E, dtype=dtype)[None, :]).cuda()
+    t_eval[::3] = t_eval[::3].flip(1)  # every third sample runs backwards
+    f = lambda t, y: torch.tanh(y @ W) * torch.cos(t)[:, None] - 0.5 * y
+    for method, ctrl in (("tsit5", dict(kind="pid", atol=1e-7, rtol=1e-5, pcoeff=0.2, icoeff=0.5, dcoeff=0.1)), ("dopri5", dict(kind="integral", atol=1e-6, rtol=1e-4))):
+        a, b = per_step_and_protocol(f, y0, t_eval, method, ctrl)
+        assert_same(a, b)
+        assert (a.stats["n_steps"] >= 3).all() and (a.stats["n_initialized"] == E).all() and (a.status == 0).all()
+
+
+def test_per_step_path_on_long_rows_bookkeeping_cases():
+    f, y0, t_eval = rd_problem(9, n=32, E=7, t1=4.0, d_max=0.5)
+    ctrl = dict(kind="pid", atol=1e-6, rtol=1e-4, pcoeff=0.3, icoeff=0.4, dcoeff=0.0)
+    # evaluation times out of order, a first point that is not t_start, points beyond t_end
+    t_odd = t_eval.clone()
+    t_odd[:, [2, 5]] = t_odd[:, [5, 2]]
+    t_odd[3, 0] = 0.1
+    t_start, t_end = torch.zeros(9, device="cuda"), t_eval[:, -1] * 0.9
+    a, b = per_step_and_protocol(f, y0, t_odd, "tsit5", ctrl, t_start=t_start, t_end=t_end)
+    assert_same(a, b)
+    assert (a.stats["n_initialized"] < 7).any()
+    # no evaluation points; a given first step; max_steps
+    assert_same(*per_step_and_protocol(f, y0, None, "dopri5", ctrl, t_start=t_start, t_end=t_end))
+    assert_same(*per_step_and_protocol(f, y0, t_eval, "dopri5", ctrl, dt0=torch.full((9,), 0.02, device="cuda")))
+    a = to.AutoDiffAdjoint(to.Tsit5(), make_controller(ctrl), max_steps=3).solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(lambda t, y: f(t, y)))
+    b = to.AutoDiffAdjoint(OwnTsit5(), make_controller(ctrl), max_steps=3).solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(lambda t, y: f(t, y)))
+    assert a.status.tolist() == [3] * 9
+    assert_same(a, b)

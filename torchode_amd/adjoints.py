@@ -132,8 +132,7 @@ class AutoDiffAdjoint(nn.Module):
         return self._fused_ok(problem, term) and isinstance(f, BuiltinTerm) and f.builtin_kind in _lib.PERSISTENT_TERMS and not term.with_args
 
     def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        # the per-step kernels walk a sample's row in one thread: small rows only
-        return self._fused_ok(problem, term) and problem.n_features < 64
+        return self._fused_ok(problem, term)
 
     # ------------------------------------------------------------------ #
     def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args) -> Solution:

@@ -6,7 +6,7 @@
 // registers for the whole solve.  Only the stage input travels through LDS, double
 // buffered, so that the five-point stencil can read its neighbours: one barrier per
 // right-hand side evaluation.  Norms over the row are block reductions in a fixed
-// order (the order of wave_row_norm in tode_ops.hip: per-thread chain over its four
+// order (the order of wave_row_norm in tode_solve.h: per-thread chain over its four
 // values, butterfly over the wavefront, wavefront sums added in order), so that this
 // kernel and the per-call operators produce the same bits.  Every thread of the
 // workgroup carries the same scalar state (t, dt, error ratio, counters), computed

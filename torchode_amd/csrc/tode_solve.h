@@ -218,6 +218,39 @@ template <typename T> static SolveParams<T> make_params(const tode_solve_args &a
     return p;
 }
 
+// One wavefront reduces one row (F >= 64).  The order of summation is fixed, so that every kernel
+// that forms such a norm gets the same bits: the row is cut into chunks of 256 values; within a
+// chunk lane l accumulates values 4l..4l+3 in order (fused multiply-add from zero), the 64 partial
+// sums are combined by a butterfly (xor 32, 16, .., 1), and the chunk sums are added in order.
+template <typename T, int NORM, typename Load> __device__ __forceinline__ T wave_row_norm(int F, Load load) {
+    const int lane = threadIdx.x & 63;
+    const T sf = (T)__builtin_sqrt((double)F);
+    T total = 0;
+    for (int base = 0; base < F; base += 256) {
+        T p = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int f = base + 4 * lane + j;
+            if (f < F) {
+                const T v = load(f);
+                if (NORM == TODE_NORM_MAX)
+                    p = tmax(p, abs_(v));
+                else {
+                    const T x = v / sf;
+                    p = fma_(x, x, p);
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const T o = __shfl_xor(p, off);
+            p = NORM == TODE_NORM_MAX ? tmax(p, o) : p + o;
+        }
+        total = NORM == TODE_NORM_MAX ? tmax(total, p) : total + p;
+    }
+    return NORM == TODE_NORM_MAX ? total : sqrt_(total);
+}
+
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for the wavefront's
 // global stores to be acknowledged -- in the whole-solve kernels the dense output, which no thread
 // of the kernel ever reads -- and that wait (a round trip to memory) would sit on the critical path

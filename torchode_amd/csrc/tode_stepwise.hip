@@ -5,10 +5,11 @@
 // iterations.  Once the loop has ended on the device, kernels of iterations
 // that were enqueued speculatively return immediately.
 //
-// One thread per sample; features are walked with run-time loops in the same
-// order as a scalar evaluation (this path is meant for small F, where a
-// sample's row is a few contiguous values; the stage arrays necessarily go
-// through HBM because f is external).
+// Rows of fewer than 64 features: one thread per sample, features walked with run-time
+// loops in the same order as a scalar evaluation.  Longer rows: one wavefront per sample,
+// lanes strided over the features, norms in the fixed order of wave_row_norm (the stage
+// kernel is per element either way).  The stage arrays necessarily go through HBM because
+// f is external.
 #include "tode_solve.h"
 
 namespace tode {
@@ -296,6 +297,208 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     if (status != 0) p.flags[TODE_STEP_FLAG_ANY_FAILURE] = 1;
 }
 
+// ------------------------------------------------------------------------------------------
+// The same three kernels for long rows: one wavefront per sample, four samples per workgroup.
+// Per-sample scalars are computed by every lane; lane 0 stores them.
+// ------------------------------------------------------------------------------------------
+
+template <typename T> __global__ void __launch_bounds__(256) init_a_wave_kernel(const StepParams<T> p) {
+    const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= p.batch) return;
+    const int F = p.F, lane = threadIdx.x & 63;
+    const CtrlParams<T> &cp = p.cp;
+    const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
+    const T d0 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return y0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
+    const T d1 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return f0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
+    h0 = tmin(h0, abs_(te - ts));
+    const T dh = dir * h0;
+    T *y1 = p.ystage[1] + b * F;
+    for (int f = lane; f < F; f += 64) y1[f] = fma_(dh, f0[f], y0[f]);
+    if (lane == 0) {
+        p.tnode[b] = fma_(dir, h0, ts);
+        p.dt[b] = h0;
+    }
+}
+
+template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<T> p, const T *dt0) {
+    const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= p.batch) return;
+    const int F = p.F, E = p.E, lane = threadIdx.x & 63;
+    const CtrlParams<T> &cp = p.cp;
+    const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    T dt;
+    if (FROM_F1) {
+        const T *f1 = p.k[1] + b * F;
+        const T d1 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return f0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
+        const T d2n = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
+            const T df = f1[f] - f0[f];
+            return df * inv_scale(cp.atol, cp.rtol, y0[f]);
+        });
+        dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, p.dt[b], d1, d2n);
+    } else {
+        dt = dt0[b];
+    }
+    for (int f = lane; f < F; f += 64) {
+        p.y[b * F + f] = y0[f];
+        p.k0[b * F + f] = f0[f];
+    }
+    bool ordered = true;
+    int cursor = 0;
+    if (E > 0) {
+        const T *tev = p.t_eval + b * E;
+        for (int e = lane; e < E; e += 64) {
+            if (e > 0 && !(dir > 0 ? tev[e] >= tev[e - 1] : tev[e] <= tev[e - 1])) ordered = false;
+            p.pending[b * E + e] = (e == 0 && tev[0] == ts) ? 0 : 1;
+        }
+        if (tev[0] == ts) {
+            for (int f = lane; f < F; f += 64) p.ys[(b * E) * F + f] = y0[f];
+            cursor = 1;
+        }
+    }
+    ordered = !__any(!ordered);
+    if (lane == 0) {
+        const T tlo = tmin(ts, te), thi = tmax(te, ts);
+        p.t[b] = ts;
+        p.dt[b] = tclamp(dt, tlo - ts, thi - ts);
+        p.ratio_prev[b] = (T)1;
+        p.ratio_pprev[b] = (T)1;
+        p.running[b] = 1;
+        p.n_steps[b] = 0;
+        p.n_accepted[b] = 0;
+        p.status[b] = 0;
+        p.cursor[b] = cursor;
+        p.monotone[b] = ordered ? 1 : 0;
+    }
+}
+
+template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<T> p) {
+    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
+    const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= p.batch) return;
+    const int F = p.F, E = p.E, lane = threadIdx.x & 63;
+    const CtrlParams<T> &cp = p.cp;
+    const bool fused = F >= 58;
+    const T t0 = p.t[b], dt = p.dt[b];
+    const T ts = p.t_start[b], te = p.t_end[b];
+    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
+
+    // ---- error estimate and error ratio ----
+    const T norm = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
+        T err = 0;
+#pragma unroll
+        for (int s = 0; s < 7; ++s) {
+            const T ps = dt * (T)Tab::b_err[s], ks = p.k[s][b * F + f];
+            if (fused)
+                err = fma_(ps, ks, err);
+            else {
+                const T pk = ps * ks;
+                err = err + pk;
+            }
+        }
+        const T m = tmax(abs_(y[f]), abs_(y1[f]));
+        return abs_(err) / fma_(cp.rtol, m, cp.atol);
+    });
+    const T ratio = tmax(norm, (T)1e-38);
+    const bool accept = ratio < (T)1;
+
+    // ---- step size proposal ----
+    const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
+    T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
+    int status = limit_dt<T>(cp, ratio, dt_next);
+
+    const bool running = p.running[b] != 0;
+    const bool move = accept && running;
+    const T t_new = move ? (t0 + dt) : t0;
+    const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+    const int n_steps = p.n_steps[b] + (running ? 1 : 0);
+    if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
+    if (status == 0 && n_steps >= TODE_HARD_STEP_LIMIT) status = TODE_GENERAL_ERROR;
+
+    // ---- dense output with the interpolant of the attempted step: the quartic of a feature is
+    // built once, when the first evaluation point turns out to have been passed ----
+    if (E > 0) {
+        const T *tev = p.t_eval + b * E;
+        T *ys = p.ys + b * (long long)E * F;
+        uint8_t *pend = p.pending + b * (long long)E;
+        const bool mono = p.monotone[b] != 0;
+        const int cursor = p.cursor[b];
+        for (int f = lane; f < F; f += 64) {
+            T q[5][1];
+            bool built = false;
+            for (int e = mono ? cursor : 0; e < E; ++e) {
+                if (!pend[e]) continue;
+                const T te_e = tev[e];
+                const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+                if (!passed) {
+                    if (mono) break;
+                    continue;
+                }
+                if (!built) {
+                    T ks[7];
+#pragma unroll
+                    for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+                    quartic_elem<T, METHOD>(dt, y[f], y1[f], ks, fused, q);
+                    built = true;
+                }
+                T out[1];
+                quartic_eval<T, 1>(q, t0, dt, te_e, out);
+                ys[(long long)e * F + f] = out[0];
+            }
+        }
+        // (every lane has finished reading the pending marks: the wavefront runs in lock step)
+        int first_pending = E;
+        for (int e = lane; e < E; e += 64) {
+            if (!pend[e]) continue;
+            const T te_e = tev[e];
+            const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+            const bool taken = passed && (!mono || e >= cursor);
+            if (taken) pend[e] = 0;
+            else first_pending = min(first_pending, e);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) first_pending = min(first_pending, __shfl_xor(first_pending, off));
+        if (lane == 0) p.cursor[b] = first_pending;
+    } else {
+        for (int f = lane; f < F; f += 64) {
+            T ks[7];
+#pragma unroll
+            for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+            p.ys[b * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+        }
+    }
+
+    // ---- state update ----
+    if (move) {
+        for (int f = lane; f < F; f += 64) {
+            p.y[b * F + f] = y1[f];
+            p.k0[b * F + f] = p.k[6][b * F + f];
+        }
+    }
+    if (lane == 0) {
+        p.n_steps[b] = n_steps;
+        if (move) p.n_accepted[b] += 1;
+        p.status[b] = status;
+        p.t[b] = t_new;
+        const T tlo = tmin(ts, te), thi = tmax(te, ts);
+        const T dtn = running_new ? dt_next : dt;
+        p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
+        if (CTRL == 1 && running_new && accept) {
+            p.ratio_pprev[b] = prev;
+            p.ratio_prev[b] = ratio;
+        }
+        p.running[b] = running_new ? 1 : 0;
+        if (running_new) p.flags[TODE_STEP_FLAG_ANY_RUNNING] = 1;
+        if (status != 0) p.flags[TODE_STEP_FLAG_ANY_FAILURE] = 1;
+    }
+}
+
 // One thread: closes the iteration.  The loop goes on iff some sample is still running and
 // every status is SUCCESS (adjoints.py:186-190).
 static __global__ void loop_control_kernel(int32_t *flags) {
@@ -389,7 +592,8 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
     int rc = check_state(s, c);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned blocks = (unsigned)((s->batch + 255) / 256);
+    const bool wide = s->n_features >= 64;  // one wavefront per sample
+    const unsigned blocks = wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
     if (phase == 0) {
         hipLaunchKernelGGL(step_flags_init_kernel, dim3(1), dim3(64), 0, st, s->flags);
         if (blocks == 0) return check_hip(hipGetLastError(), "tode_step_begin");
@@ -397,7 +601,9 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
             if (!s->k[0]) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
             TODE_DISPATCH_T(s->dtype, {
                 auto p = make_step_params<T>(*s, *c);
-                if (c->kind == TODE_CTRL_INTEGRAL)
+                if (wide)
+                    hipLaunchKernelGGL((init_b_wave_kernel<T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);  // (CTRL is unused here)
+                else if (c->kind == TODE_CTRL_INTEGRAL)
                     hipLaunchKernelGGL((init_b_kernel<T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
                 else
                     hipLaunchKernelGGL((init_b_kernel<T, 1, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
@@ -406,7 +612,10 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
             if (!s->k[0] || !s->ystage[1]) return fail(TODE_E_INVALID, "k[0] or ystage[1] is null");
             TODE_DISPATCH_T(s->dtype, {
                 auto p = make_step_params<T>(*s, *c);
-                hipLaunchKernelGGL(init_a_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
+                if (wide)
+                    hipLaunchKernelGGL(init_a_wave_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
+                else
+                    hipLaunchKernelGGL(init_a_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
             });
         }
     } else {
@@ -414,7 +623,11 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
         if (!s->k[0] || !s->k[1]) return fail(TODE_E_INVALID, "k[0] or k[1] is null");
         TODE_DISPATCH_T(s->dtype, {
             auto p = make_step_params<T>(*s, *c);
-            if (c->kind == TODE_CTRL_INTEGRAL)
+            if (wide && c->kind == TODE_CTRL_INTEGRAL)
+                hipLaunchKernelGGL((init_b_wave_kernel<T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+            else if (wide)
+                hipLaunchKernelGGL((init_b_wave_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+            else if (c->kind == TODE_CTRL_INTEGRAL)
                 hipLaunchKernelGGL((init_b_kernel<T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
             else
                 hipLaunchKernelGGL((init_b_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
@@ -460,7 +673,8 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
     int rc = check_state(s, c);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned blocks = (unsigned)((s->batch + 255) / 256);
+    const bool wide = s->n_features >= 64;
+    const unsigned blocks = wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
     if (blocks > 0) {
         for (int j = 0; j < 7; ++j)
             if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
@@ -468,7 +682,19 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
         TODE_DISPATCH_T(s->dtype, {
             auto p = make_step_params<T>(*s, *c);
             const bool pid = c->kind == TODE_CTRL_PID;
-            if (s->method == TODE_TSIT5) {
+            if (wide) {
+                if (s->method == TODE_TSIT5) {
+                    if (pid)
+                        hipLaunchKernelGGL((finish_wave_kernel<T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
+                    else
+                        hipLaunchKernelGGL((finish_wave_kernel<T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
+                } else {
+                    if (pid)
+                        hipLaunchKernelGGL((finish_wave_kernel<T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
+                    else
+                        hipLaunchKernelGGL((finish_wave_kernel<T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
+                }
+            } else if (s->method == TODE_TSIT5) {
                 if (pid)
                     hipLaunchKernelGGL((finish_kernel<T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
                 else
