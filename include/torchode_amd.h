@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 8
+#define TODE_ABI_VERSION 9
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -255,8 +255,8 @@ enum {
  *   [ k[1] <- f(tnode, ystage[1]);  tode_step_begin(phase 1) ]      only when dt0 == NULL
  *   repeat:  for s = 1..6:  tode_step_stage(s);  k[s] <- f(tnode, ystage[s])
  *            tode_step_finish()
- *   The caller reads `flags` whenever it likes; after TODE_STEP_FLAG_STOPPED is
- *   set, further stage/finish calls are no-ops.  tode_step_stats converts the
+ *   The caller reads `flags` (a synchronisation) or `host_flags` (none) whenever it
+ *   likes; after TODE_STEP_FLAG_STOPPED is set, further stage/finish calls are no-ops.  tode_step_stats converts the
  *   counters.  k[0] must point at k0 from the first stage call on (begin
  *   copies f(t_start, y0) there).
  */
@@ -289,6 +289,10 @@ typedef struct tode_step_state {
     void *ystage[7];     /* [B,F] each: input of stage s (index 0 unused); ystage[6] is y1 */
     const void *k[7];    /* [B,F] each: f at stage s, written by the caller; k[0] == k0   */
     void *tnode;         /* [B] time of the stage that was just prepared */
+    int32_t *host_flags; /* NULL, or two int32 in pinned host memory that the device can write: every
+                            tode_step_finish leaves there TODE_STEP_FLAG_STOPPED and
+                            TODE_STEP_FLAG_ITERATIONS as of its iteration, so that the host can see the loop
+                            end by reading its own memory, without a synchronisation */
 } tode_step_state;
 
 /*

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
 F32, F64 = 0, 1
@@ -164,6 +164,7 @@ class StepState(C.Structure):
         ("ystage", C.c_void_p * 7),
         ("k", C.c_void_p * 7),
         ("tnode", C.c_void_p),
+        ("host_flags", C.c_void_p),
     ]
 
 

@@ -247,8 +247,9 @@ class AutoDiffAdjoint(nn.Module):
             stats["n_initialized"] = torch.ones(B, dtype=torch.long, device=dev)
             return Solution(ts=problem.t_end[:, None], ys=y_end[:, None], stats=stats, status=status)
 
-    # How many loop iterations are enqueued between two looks at the device flags.
-    poll_first, poll_max = 4, 32
+    # Graph replay: how many loop iterations are enqueued between two synchronising looks at the
+    # device flags.  Eager iterations: how many iterations the host may be ahead of the device.
+    poll_first, poll_max, run_ahead = 4, 32, 2
 
     def _solve_stepwise(self, problem: InitialValueProblem, term: ODETerm, dt0, args, record=None) -> Solution:
         """Arbitrary Python ``f``: per-step kernels around the user's torch RHS, loop state on the
@@ -283,6 +284,12 @@ class AutoDiffAdjoint(nn.Module):
         s.ratio_prev, s.ratio_pprev = hist[0].data_ptr(), hist[1].data_ptr()
         s.running, s.cursor, s.n_steps, s.n_accepted, s.status, s.monotone = (ints[i].data_ptr() for i in range(6))
         s.pending, s.ys, s.flags = pending.data_ptr(), ys.data_ptr(), flags.data_ptr()
+        # two words in pinned host memory that the device keeps up to date: the host sees the loop end
+        # by reading its own memory, after every iteration and without a synchronisation
+        mirror = torch.empty(2, dtype=torch.int32, pin_memory=True)
+        s.host_flags = mirror.data_ptr()
+        stopped_on_device = mirror.numpy()
+        stopped_on_device[:] = 0  # (on the host: torch.zeros on pinned memory costs 0.2 ms)
         sref, cref = _lib.C.byref(s), _lib.C.byref(ctrl)
 
         f, with_args = term.f, term.with_args
@@ -330,23 +337,37 @@ class AutoDiffAdjoint(nn.Module):
                     evaluate(i, tt, yy)
                 _lib.check(lib.tode_step_finish(sref, cref, stream), "tode_step_finish")
 
-        chunk, graph, replays = self.poll_first, None, 1
+        use_graph = bool(self.graph_iterations) and record is None
+        chunk, graph, replays, enqueued, spins = self.poll_first, None, 1, 0, 0
         while True:
-            if graph is None:
-                iterate(chunk, stream)
-            else:
+            if graph is not None:
                 for _ in range(replays):
                     graph.replay()
-            fl = flags.tolist()  # host/device synchronisation, once per chunk of iterations
+            elif use_graph or not self.run_ahead:
+                iterate(chunk, stream)
+                if not use_graph:
+                    chunk = min(2 * chunk, self.poll_max)
+            else:
+                # Eager iterations: the host looks at the device's stop word (in its own memory) after
+                # every iteration it has enqueued.  It runs ahead of the device, so a few iterations
+                # are still enqueued after the loop has ended there; their kernels do nothing.
+                while not stopped_on_device[0]:
+                    if enqueued - int(stopped_on_device[1]) < self.run_ahead:
+                        iterate(1, stream)
+                        enqueued += 1
+                        spins = 0
+                    else:  # the device is the slower side: let it finish an iteration before enqueuing more
+                        spins += 1
+                        if spins > 1_000_000:
+                            break  # (no news for long: synchronise below and look again)
+            fl = flags.tolist()  # host/device synchronisation
             if fl[_lib.STEP_FLAG_STOPPED]:
                 break
-            if self.graph_iterations and graph is None and record is None:
+            if use_graph and graph is None:
                 # (the eager iterations above have also warmed up whatever f uses)
                 graph = self._record(lambda st: iterate(int(self.graph_iterations), st), y0)
             elif graph is not None:
                 replays = min(2 * replays, max(1, self.poll_max // int(self.graph_iterations)))
-            else:
-                chunk = min(2 * chunk, self.poll_max)
         keep.clear()
         del graph  # frees the memory f's intermediate tensors were recorded with
         if record is not None:

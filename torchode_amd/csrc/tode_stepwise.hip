@@ -501,15 +501,22 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
 
 // One thread: closes the iteration.  The loop goes on iff some sample is still running and
 // every status is SUCCESS (adjoints.py:186-190).
-static __global__ void loop_control_kernel(int32_t *flags) {
+static __global__ void loop_control_kernel(int32_t *flags, int32_t *host_flags) {
     if (threadIdx.x != 0 || flags[TODE_STEP_FLAG_STOPPED]) return;
-    flags[TODE_STEP_FLAG_ITERATIONS] += 1;
-    if (!flags[TODE_STEP_FLAG_ANY_RUNNING] || flags[TODE_STEP_FLAG_ANY_FAILURE]) flags[TODE_STEP_FLAG_STOPPED] = 1;
+    const int iterations = flags[TODE_STEP_FLAG_ITERATIONS] + 1;
+    const int stopped = (!flags[TODE_STEP_FLAG_ANY_RUNNING] || flags[TODE_STEP_FLAG_ANY_FAILURE]) ? 1 : 0;
+    flags[TODE_STEP_FLAG_ITERATIONS] = iterations;
+    flags[TODE_STEP_FLAG_STOPPED] = stopped;
     flags[TODE_STEP_FLAG_ANY_RUNNING] = 0;
+    if (host_flags) {  // the count first: a host that sees "stopped" also sees the final count
+        __hip_atomic_store(&host_flags[1], iterations, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(&host_flags[0], stopped, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
-static __global__ void step_flags_init_kernel(int32_t *flags) {
+static __global__ void step_flags_init_kernel(int32_t *flags, int32_t *host_flags) {
     if (threadIdx.x < TODE_STEP_FLAG_WORDS) flags[threadIdx.x] = 0;
+    if (host_flags && threadIdx.x < 2) __hip_atomic_store(&host_flags[threadIdx.x], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // int32 device state -> the reference's int64 stats (adjoints.py:267-292)
@@ -595,7 +602,7 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
     const bool wide = s->n_features >= 64;  // one wavefront per sample
     const unsigned blocks = wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
     if (phase == 0) {
-        hipLaunchKernelGGL(step_flags_init_kernel, dim3(1), dim3(64), 0, st, s->flags);
+        hipLaunchKernelGGL(step_flags_init_kernel, dim3(1), dim3(64), 0, st, s->flags, s->host_flags);
         if (blocks == 0) return check_hip(hipGetLastError(), "tode_step_begin");
         if (dt0) {
             if (!s->k[0]) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
@@ -707,7 +714,7 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
             }
         });
     }
-    hipLaunchKernelGGL(loop_control_kernel, dim3(1), dim3(64), 0, st, s->flags);
+    hipLaunchKernelGGL(loop_control_kernel, dim3(1), dim3(64), 0, st, s->flags, s->host_flags);
     return check_hip(hipGetLastError(), "tode_step_finish");
 }
 
