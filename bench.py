@@ -32,11 +32,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6869.1 KiB x 2.000 + 32540.4 KiB x 1.000) x 1024
-    ("vdp", "torch.float32", 65536): 47.39e6,
-    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (77468.9 KiB x 2.000 + 895940 KiB x 1.000) x 1024
-    ("lorenz", "torch.float32", 1048576): 1076.1e6,
-    # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4363 KiB x 2.000 + 819284 KiB x 1.000) x 1024
+    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6873.0 KiB x 2.000 + 32671.0 KiB x 1.000) x 1024
+    ("vdp", "torch.float32", 65536): 47.53e6,
+    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (77710 KiB x 2.000 + 870500 KiB x 1.000) x 1024
+    ("lorenz", "torch.float32", 1048576): 1050.5e6,
+    # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4370 KiB x 2.000 + 819300 KiB x 1.000) x 1024
     ("reaction_diffusion", "torch.float32", 512): 847.9e6,
     # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1498 KiB x 2.000 + 20624 KiB x 1.000) x 1024
     ("mlp", "torch.float32", 4096): 24.19e6,
