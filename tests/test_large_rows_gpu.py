@@ -1,6 +1,7 @@
 """GPU tests of the workloads with long rows (reaction-diffusion F = 4096, MLP F = 64): the
-solve runs through the protocol path (one kernel per protocol call, one wavefront per row in the
-norms) around torch right-hand sides on the device.
+whole-solve kernels for both, the per-step path with one wavefront per sample, and the protocol
+path (one kernel per protocol call, one wavefront per row in the norms) around torch right-hand
+sides on the device.
 
 The checker is the ATen-op oracle evaluated live on this host's CPU.  Bit-level agreement is not
 asked for here: ATen's order of summation in a 4096-element norm and in its matrix products
