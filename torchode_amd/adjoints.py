@@ -19,11 +19,19 @@ _PROTOCOL_NAMES = (
 )  # fmt: skip
 
 
+_F_EVAL_VALUES: Dict[int, torch.Tensor] = {}  # count -> 0-dim int64 tensor (never written to)
+
+
 def _f_evals(count: int, batch: int) -> torch.Tensor:
     """``stats["n_f_evals"]``: int64 ``[B]`` on the CPU, every sample carrying the same count (the
     reference counts evaluations of ``f`` on the whole batch, terms.py:41-63).  One stored value
     viewed ``B`` times: filling half a megabyte per solve costs more than the kernel launch."""
-    return torch.tensor(count, dtype=torch.long).expand(batch)
+    value = _F_EVAL_VALUES.get(count)
+    if value is None:
+        if len(_F_EVAL_VALUES) > 4096:
+            _F_EVAL_VALUES.clear()
+        value = _F_EVAL_VALUES[count] = torch.tensor(count, dtype=torch.long)
+    return value.expand(batch)
 
 
 _PROTOCOL_NAME_SET = frozenset(_PROTOCOL_NAMES)
@@ -403,13 +411,21 @@ class AutoDiffAdjoint(nn.Module):
     def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
         lib = _lib.load()
         f: BuiltinTerm = term.f
-        y0 = problem.y0.contiguous()
-        dev, dtype = y0.device, y0.dtype
-        B, F = y0.shape
-        E = problem.n_evaluation_points
-        # t_start / t_end are usually columns of t_eval: hand them over with their stride
-        t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
-        t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
+        # What depends on the problem's tensors alone is worked out once per problem object and kept on it
+        # (checked by identity: the attributes of a problem may be reassigned).
+        tensors = (problem.y0, problem.t_start, problem.t_end, problem.t_eval)
+        plan = getattr(problem, "_launch_plan", None)
+        if plan is None or any(a is not b for a, b in zip(plan[0], tensors)):
+            y0 = problem.y0.contiguous()
+            # t_start / t_end are usually columns of t_eval: hand them over with their stride
+            t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
+            t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
+            ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+            plan = (tensors, y0, t_start, t_end, t_eval, ts, y0.device, y0.dtype, y0.shape[0], y0.shape[1], problem.n_evaluation_points,
+                    y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0),
+                    None if t_eval is None else t_eval.data_ptr())  # fmt: skip
+            problem._launch_plan = plan
+        _, y0, t_start, t_end, t_eval, ts, dev, dtype, B, F, E, y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr = plan
         params = f.builtin_params().to(device=dev, dtype=dtype)
         if params.numel() == 0 and params.shape[0] != B:  # a term without per-sample parameters
             params = y0.new_empty((B, 0))
@@ -429,8 +445,7 @@ class AutoDiffAdjoint(nn.Module):
         a = _lib.SolveArgs(  # positional, in the order of struct tode_solve_args
             _lib.DTYPES[dtype], self.step_method.method_id, f.builtin_kind, F, E, params.shape[1], B,
             -1 if self.max_steps is None else int(self.max_steps), -1, (_lib.C.c_double * 4)(*scal[:4]),
-            y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0),
-            None if t_eval is None else t_eval.data_ptr(), None if dt0_ is None else dt0_.data_ptr(),
+            y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, None if dt0_ is None else dt0_.data_ptr(),
             params.data_ptr() if params.numel() else None,
             None if shared is None else shared.data_ptr(), 0 if shared is None else shared.numel(),
             ys.data_ptr(), None if y_idle is None else y_idle.data_ptr(),
@@ -438,7 +453,6 @@ class AutoDiffAdjoint(nn.Module):
 
         stats: Dict[str, Any] = {}
         n_init_evals = 2 if dt0 is None else 1
-        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
 
         # Common case first: one kernel, int64 stats written directly.  It reports through the
         # flag block when the batch needs the general kernel (which handles every case).

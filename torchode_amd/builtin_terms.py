@@ -62,7 +62,11 @@ class VanDerPol(BuiltinTerm):
         return torch.stack((v, dv), dim=1)
 
     def builtin_params(self):
-        return self.mu.reshape(-1, 1).contiguous()
+        mu = self.mu
+        cached = self.__dict__.get("_params_view")
+        if cached is None or cached[0] is not mu or cached[1] != mu._version:
+            cached = self.__dict__["_params_view"] = (mu, mu._version, mu.reshape(-1, 1).contiguous())
+        return cached[2]
 
 
 class Lorenz63(BuiltinTerm):
