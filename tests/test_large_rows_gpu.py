@@ -350,3 +350,25 @@ def test_per_step_path_on_long_rows_bookkeeping_cases():
     b = to.AutoDiffAdjoint(OwnTsit5(), make_controller(ctrl), max_steps=3).solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(lambda t, y: f(t, y)))
     assert a.status.tolist() == [3] * 9
     assert_same(a, b)
+
+
+def test_mlp_kernel_backwards_in_time_mixed_directions_and_few_points():
+    w = to.workloads.make("mlp", batch=90, device="cuda")
+    t_eval = w.t_eval.clone()
+    t_eval[::2] = t_eval[::2].flip(1)  # every other sample runs from 1 to 0
+    mixed = w._replace(t_eval=t_eval)
+    for method, ctrl in (("dopri5", w.controller), ("tsit5", dict(kind="pid", atol=1e-6, rtol=1e-4, pcoeff=0.2, icoeff=0.5, dcoeff=0.0))):
+        fused, proto = mlp_both_paths(mixed, method, ctrl)
+        assert (fused.status == 0).all() and (fused.stats["n_initialized"] == 20).all()
+        assert_close_solutions(fused, proto, min_agree=0.9)
+        assert torch.equal(fused.ys[:, 0], w.y0)  # the first evaluation point is t_start: y0 itself
+    two = w._replace(t_eval=w.t_eval[:, [0, -1]].contiguous())
+    fused, proto = mlp_both_paths(two, w.method, w.controller)
+    assert fused.ys.shape == (90, 2, 64)
+    assert_close_solutions(fused, proto, min_agree=0.9)
+    # a first evaluation point after t_start
+    late = w._replace(t_eval=(w.t_eval * 0.5 + 0.25).contiguous())
+    problem = to.InitialValueProblem(w.y0, t_start=torch.zeros(90, device="cuda"), t_end=torch.ones(90, device="cuda"), t_eval=late.t_eval)
+    a = to.AutoDiffAdjoint(to.Dopri5(), make_controller(w.controller)).solve(problem, to.ODETerm(w.f))
+    b = to.AutoDiffAdjoint(OwnDopri5(), make_controller(w.controller)).solve(problem, to.ODETerm(w.f))
+    assert_close_solutions(a, b, min_agree=0.9)
