@@ -180,3 +180,15 @@ def test_mlp_weights_in_one_row_major_block():
     assert raw.shape == (256 * 65 + 256 + 64 * 256 + 64,)
     assert torch.equal(raw[: 256 * 65], f.W1.reshape(-1)) and torch.equal(raw[256 * 65 : 256 * 65 + 256], f.b1)
     assert torch.equal(raw[256 * 65 + 256 : -64], f.W2.reshape(-1)) and torch.equal(raw[-64:], f.b2)
+
+
+def test_torch_compile_wrapper_hands_out_the_solvers_own_solve():
+    """torch.compile(solver) wraps the module; `.solve` on the wrapper is the wrapped solver's bound
+    method, so the idiom of the reference's README and tests/torch_script_test.py:17-21 runs this
+    library's solve unchanged."""
+    term = to.ODETerm(torch.nn.Linear(2, 2))
+    for cls in (to.AutoDiffAdjoint, to.BacksolveAdjoint, to.JointBacksolveAdjoint):
+        args = (to.Tsit5(), to.IntegralController(1e-3, 1e-3))
+        solver = cls(*args) if cls is to.AutoDiffAdjoint else cls(term, *args)
+        wrapped = torch.compile(solver)
+        assert wrapped.solve.__self__ is solver and wrapped.solve.__func__ is cls.solve

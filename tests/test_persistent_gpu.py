@@ -448,3 +448,57 @@ def test_plain_fast_entry_point_in_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(ys, ys_want) and torch.equal(out, out_want) and flags.tolist() == flags_want, i
+
+
+def _random_case(seed):
+    """One seeded configuration: term, shapes, time spans, evaluation points, tolerances and controller
+    coefficients all drawn at random, inside the ranges where every sample still succeeds."""
+    g = torch.Generator().manual_seed(seed)
+    u = lambda lo, hi, *shape: lo + (hi - lo) * torch.rand(*shape, generator=g, dtype=torch.float64)
+    pick = lambda seq: seq[int(torch.randint(len(seq), (1,), generator=g))]
+    dtype = pick([F32, F64])
+    batch = int(torch.randint(1, 700, (1,), generator=g))
+    n_eval = int(torch.randint(1, 71, (1,), generator=g))
+    term = pick(["linear_decay", "vdp", "lorenz"])
+    if term == "linear_decay":
+        n_features = int(torch.randint(1, 5, (1,), generator=g))
+        f = to.LinearDecay(u(0.1, 6.0, batch, n_features).to(dtype))
+        y0, span = u(-2.0, 2.0, batch, n_features), 3.0
+    elif term == "vdp":
+        f = to.VanDerPol(u(0.2, 8.0, batch).to(dtype))
+        y0, span = u(-2.5, 2.5, batch, 2), 6.0
+    else:
+        f = to.Lorenz63(u(20.0, 35.0, batch).to(dtype))
+        y0, span = u(-10.0, 10.0, batch, 3) + torch.tensor([0.0, 0.0, 20.0], dtype=torch.float64), 1.5
+    # per-sample spans, some samples backwards in time; evaluation points sorted in the sample's direction,
+    # drawn from an interval a little larger than [t_start, t_end] so that some fall outside it
+    t_start = u(-1.0, 1.0, batch)
+    length = u(0.3, 1.0, batch) * span
+    # (only the linear system is solved backwards here: the other two blow up in reverse time)
+    backwards = (torch.rand(batch, generator=g) < 0.3) & (term == "linear_decay")
+    t_end = torch.where(backwards, t_start - length, t_start + length)
+    frac = u(-0.05, 1.05, batch, n_eval).sort(dim=1).values
+    if pick([True, False]):
+        frac[:, 0] = 0.0  # first point exactly at t_start
+    if pick([True, False]):
+        frac[:, -1] = 1.0
+    t_eval = t_start[:, None] + frac * (t_end - t_start)[:, None]
+    rtol = 10.0 ** float(u(-7.0, -2.5, 1)) if dtype == F64 else 10.0 ** float(u(-5.0, -2.5, 1))
+    atol = rtol * 10.0 ** float(u(-3.0, 0.0, 1))
+    kind = pick(["integral", "pid", "pid", "pid"])
+    controller = dict(kind=kind, atol=atol, rtol=rtol)
+    if kind == "pid":
+        controller.update(pcoeff=float(u(0.0, 0.4, 1)), icoeff=float(u(0.3, 1.0, 1)), dcoeff=pick([0.0, float(u(0.0, 0.1, 1))]))
+    method = pick(["dopri5", "tsit5"])
+    return f, y0.to(dtype), t_eval.to(dtype), t_start.to(dtype), t_end.to(dtype), method, controller
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configurations_match_oracle_bit_for_bit(seed):
+    f, y0, t_eval, t_start, t_end, method, controller = _random_case(1000 + seed)
+    kw = dict(t_start=t_start, t_end=t_end, max_steps=4000)
+    ref = c_oracle_solve(f, y0, t_eval, method, controller, **kw)
+    assert (ref["status"] == 0).all() and 2 <= int(ref["n_steps"].max()) < 4000
+    print(f"seed {seed}: {type(f).__name__} {tuple(y0.shape)} E={t_eval.shape[1]} {y0.dtype} {method} {controller}", flush=True)
+    for fast in ("one", False, "two"):
+        assert_identical(gpu_solve(f, y0, t_eval, method, controller, fast=fast, **kw), ref)

@@ -776,3 +776,41 @@ def test_heun_keeps_time_and_data_dtypes_apart(time_dtype, data_dtype):
     t_eval = torch.tensor([[0.0, 1.77, 3.0]], dtype=time_dtype, device=DEV)
     sol = to.AutoDiffAdjoint(to.Heun(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0)).solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(rhs))
     assert sol.stats["n_steps"].item() > 3 and sol.ts.dtype == time_dtype and sol.ys.dtype == data_dtype
+
+
+# ---------------------------------------------------------------------------------------------
+# part six: the solver object inside torch.compile's wrapper (reference tests/torch_script_test.py)
+# ---------------------------------------------------------------------------------------------
+
+COMPILE_METHODS = [to.Dopri5, to.Heun, to.Tsit5, to.Euler]
+
+
+def sine_case():
+    t_eval = dev([[0.1, 0.15, 1.0], [1.0, 1.9, 2.0]])
+    return to.ODETerm(sine_dynamics), to.InitialValueProblem(sine_solution(t_eval[:, 0]), t_eval=t_eval)
+
+
+@pytest.mark.parametrize("method", COMPILE_METHODS)
+def test_wrapped_by_torch_compile_gives_the_same_solution(method):
+    """reference tests/torch_script_test.py:12-24"""
+    term, problem = sine_case()
+    adjoint = to.AutoDiffAdjoint(method(term), to.IntegralController(1e-3, 1e-3, term=term))
+    wrapped = torch.compile(adjoint)
+    dt0 = dev([0.01, 0.01]) if method is to.Euler else None
+    sol, sol_w = adjoint.solve(problem, dt0=dt0), wrapped.solve(problem, dt0=dt0)
+    assert sol.status.tolist() == [OK, OK] and torch.equal(sol.ts, sol_w.ts)
+    assert torch.equal(sol.ys, sol_w.ys) and torch.equal(sol.stats["n_steps"], sol_w.stats["n_steps"])
+    if method is not to.Euler:
+        assert torch.allclose(sol.ys, sine_solution(problem.t_eval), rtol=2e-2)
+
+
+@pytest.mark.parametrize("method", COMPILE_METHODS)
+def test_term_passed_to_solve_equals_term_fixed_at_construction(method):
+    """reference tests/torch_script_test.py:35-50"""
+    term, problem = sine_case()
+    dt0 = dev([0.01, 0.01]) if method is to.Euler else None
+    sol = to.AutoDiffAdjoint(method(None), to.IntegralController(1e-3, 1e-3)).solve(problem, term, dt0=dt0)
+    fixed = to.AutoDiffAdjoint(method(term), to.IntegralController(1e-3, 1e-3, term=term))
+    sol_f = torch.compile(fixed).solve(problem, dt0=dt0)
+    assert torch.equal(sol.ts, sol_f.ts) and torch.equal(sol.ys, sol_f.ys)
+    assert torch.equal(sol.stats["n_steps"], sol_f.stats["n_steps"])
