@@ -206,6 +206,38 @@ def test_parameter_gradients_agree_with_the_backsolve_adjoint_and_float32_runs()
 
 
 @gpu
+def test_gradients_reach_tensors_inside_args():
+    """The reference's loop is torch operations, so a tensor handed to `f` through `args` gets its
+    gradient like any other input (adjoints.py:42-48, terms.py: `f(t, y, args)`).  Here: the system
+    matrix and a scale as a dict in `args`, one of them not a leaf, no parameters on the term."""
+    y0, A = inputs()
+    A = A.detach().clone().requires_grad_()
+    log_scale = torch.tensor(0.25, dtype=torch.double, device="cuda", requires_grad=True)
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+    term = to.ODETerm(lambda t, y, args: (y @ args["A"]) * args["more"][0], with_args=True)
+    args = {"A": A, "more": (log_scale.exp(), "a string", 3)}
+    solution = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-10, 1e-10)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term, args=args)
+    assert solution.ys.requires_grad
+    weights = torch.linspace(0.5, 1.5, solution.ys.numel(), dtype=torch.double, device="cuda").reshape(solution.ys.shape)
+    (solution.ys * weights).sum().backward()
+    y0_ref, A_ref, ls_ref = (x.detach().clone().requires_grad_() for x in (y0, A, log_scale))
+    (closed_form(y0_ref, A_ref * ls_ref.exp(), t_eval) * weights).sum().backward()
+    torch.testing.assert_close(y0.grad, y0_ref.grad, rtol=1e-7, atol=1e-8)
+    torch.testing.assert_close(A.grad, A_ref.grad, rtol=1e-7, atol=1e-8)
+    torch.testing.assert_close(log_scale.grad, ls_ref.grad, rtol=1e-7, atol=1e-8)
+    # only a tensor in args requires grad: still the differentiable path
+    y0_plain = y0.detach()
+    A2 = A.detach().clone().requires_grad_()
+    sol = to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-10, 1e-10)).solve(
+        to.InitialValueProblem(y0_plain, t_eval=t_eval), term=to.ODETerm(lambda t, y, a: y @ a, with_args=True), args=A2
+    )
+    (sol.ys * weights).sum().backward()
+    A_ref2 = A.detach().clone().requires_grad_()
+    (closed_form(y0_plain, A_ref2, t_eval) * weights).sum().backward()
+    torch.testing.assert_close(A2.grad, A_ref2.grad, rtol=1e-7, atol=1e-8)
+
+
+@gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))

@@ -96,7 +96,7 @@ class AutoDiffAdjoint(nn.Module):
             or (problem.t_eval is not None and problem.t_eval.requires_grad)
             or (dt0 is not None and dt0.requires_grad)
         ):
-            raise RuntimeError("torchode_amd differentiates a solve with respect to y0 and the term's parameters; times must not require grad")
+            raise RuntimeError("torchode_amd differentiates a solve with respect to y0, the term's parameters and tensors in args; times must not require grad")
         wants_grad = grad_on and problem.y0.requires_grad
         if not wants_grad and self._persistent_ok(problem, term_):
             sol = self._solve_persistent(problem, term_, dt0)
@@ -104,6 +104,10 @@ class AutoDiffAdjoint(nn.Module):
                 return sol
         if grad_on and not wants_grad and isinstance(term_, nn.Module):
             wants_grad = any(p.requires_grad for p in term_.parameters())
+        if grad_on and not wants_grad and args is not None:
+            from .autodiff import tensor_leaves
+
+            wants_grad = any(a.requires_grad for a in tensor_leaves(args))
         if wants_grad:
             # gradients through the loop: forward in the per-step kernels with a record of the loop
             # state, backward by a reverse sweep over the record

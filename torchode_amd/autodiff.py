@@ -11,8 +11,9 @@ the next state and of the evaluation points back through it, which evaluates ``f
 vector-Jacobian products six times per iteration.  Memory: one state copy per iteration instead of
 the reference's whole operation graph.
 
-Gradients flow to ``y0`` and to the parameters of the term; times (``t_start``, ``t_end``,
-``t_eval``) and ``args`` are treated as constants.
+Gradients flow to ``y0``, to the parameters of the term and to the tensors inside ``args`` (a
+tensor, or tuples / lists / dicts of them); times (``t_start``, ``t_end``, ``t_eval``) are
+treated as constants.
 """
 from math import sqrt
 from typing import Any, List, Optional, Sequence
@@ -21,6 +22,17 @@ import torch
 
 from . import _lib
 from .problems import InitialValueProblem
+
+
+def tensor_leaves(obj) -> List[torch.Tensor]:
+    """The tensors inside ``obj``: a tensor itself, or tuples, lists and dicts (by value) of such."""
+    if isinstance(obj, torch.Tensor):
+        return [obj]
+    if isinstance(obj, (tuple, list)):
+        return [t for item in obj for t in tensor_leaves(item)]
+    if isinstance(obj, dict):
+        return [t for item in obj.values() for t in tensor_leaves(item)]
+    return []
 
 
 class LoopRecord:
@@ -280,10 +292,11 @@ class SolveThroughLoop(torch.autograd.Function):
 
 
 def solve(adjoint, problem: InitialValueProblem, term, dt0: Optional[torch.Tensor], args: Any):
-    """``AutoDiffAdjoint.solve`` for a ``y0`` or term parameters that require grad."""
+    """``AutoDiffAdjoint.solve`` for a ``y0``, term parameters or tensors in ``args`` that require grad."""
     from .solution import Solution
 
     params = [p for p in term.parameters() if p.requires_grad]
+    params += [a for a in tensor_leaves(args) if a.requires_grad and not any(a is p for p in params)]
     ys, status, n_steps, n_accepted, n_initialized, n_f_evals = SolveThroughLoop.apply(adjoint, problem, term, dt0, args, problem.y0, *params)
     stats = {"n_f_evals": n_f_evals} if term.with_stats else {}
     stats.update(n_steps=n_steps, n_accepted=n_accepted, n_initialized=n_initialized)
