@@ -3,8 +3,8 @@
 // MI355X: 256 CUs x 4 SIMDs x 64 lanes).
 //
 // A single in-order wavefront cannot keep a SIMD busy: every instruction costs an
-// issue slot and every dependent result is waited for (measured: 5.75 cycles per
-// dependent fp32 FMA with one wave per SIMD, 3.7 per SIMD with two).  The solve
+// issue slot and every dependent result is waited for (measured: one dependent fp32
+// FMA every 7.7 cycles with one wave per SIMD, one every 5.3 per SIMD with two).  The solve
 // loop has exactly one piece of work that the next step does not depend on -- the
 // dense output -- so each group of 64 samples gets two wavefronts:
 //   * the STEPPER runs the adaptive loop (stages, error ratio, step size control,
