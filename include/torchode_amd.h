@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 9
+#define TODE_ABI_VERSION 10
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -186,9 +186,19 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
  * past t_end); every output is then unspecified and the caller must repeat the
  * solve with tode_solve_builtin.  Results are bit-identical to
  * tode_solve_builtin + tode_finalize_stats whenever the flag stays 0.
- * Returns TODE_E_UNSUPPORTED for n_eval == 0, dt_min / dt_max, or n_eval too
- * large for on-chip staging.
+ * Returns TODE_E_UNSUPPORTED for dt_min / dt_max, or n_eval too large for
+ * on-chip staging.
+ *
+ * n_eval == 0 (the reference's t_eval=None, adjoints.py:296-311: the end point
+ * alone, ys of shape [B,1,F]) is covered for the small systems (linear decay,
+ * Van der Pol, Lorenz) and batches of up to TODE_END_ONLY_MAX_BATCH samples;
+ * otherwise TODE_E_UNSUPPORTED.  `t_eval` may then be null and `y_idle` [B,F]
+ * must be given: the kernel leaves in ys[b] the dense output of sample b's last
+ * step at t_end and in y_idle[b] its final state, and the caller, once it has
+ * read the flags, finishes with tode_select_end_point(...,
+ * flags[TODE_FLAG_MAX_ITERATIONS], ...).
  */
+#define TODE_END_ONLY_MAX_BATCH (2048 * 64)
 int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                             int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream);
 
@@ -203,11 +213,23 @@ int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *
  * values in the host array `flags_out`.  That saves the launch that resets the
  * flag block and the device-to-host copy.  ys and the four stat arrays are
  * complete in stream order as before (here: when the call returns).  Safe to
- * call from several host threads and on several streams at once.
+ * call from several host threads and on several streams at once.  With
+ * n_eval == 0 this call also enqueues tode_select_end_point.
  */
 int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                                  int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream,
                                  int32_t *flags_out);
+
+/*
+ * Last step of a solve without evaluation points through tode_solve_builtin_fast
+ * (adjoints.py:296-311): the reference evaluates the interpolant of the batch's
+ * LAST iteration at t_end, and a sample that had finished earlier took a
+ * zero-length step in that iteration, whose interpolant is its final state.
+ * ys[b] = y_idle[b] for every sample with n_steps[b] < last_iteration; the
+ * others keep the dense output of their last step.
+ */
+int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int64_t last_iteration, const int64_t *n_steps, void *ys,
+                          const void *y_idle, void *stream);
 
 /*
  * Weights of TODE_TERM_MLP in the order the solve kernel loads them into

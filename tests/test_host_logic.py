@@ -104,7 +104,18 @@ def test_abi_argument_validation_without_a_gpu():
         setattr(a, name, _lib.C.addressof(dummy))
     assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1  # strides left at zero
     assert b"stride" in lib.tode_last_error()
-    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -2  # n_eval == 0
+    # n_eval == 0 through the fast entry point: the small systems only, and y_idle is needed
+    a.term = _lib.TERM_MLP
+    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -2
+    assert b"small systems" in lib.tode_last_error()
+    a.term, a.y_idle = 1, None
+    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -1
+    assert b"y_idle" in lib.tode_last_error()
+    a.y_idle = _lib.C.addressof(dummy)
+    assert lib.tode_select_end_point(4, 2, 7, 3, _lib.C.addressof(dummy), _lib.C.addressof(dummy), _lib.C.addressof(dummy), None) == -1
+    assert b"dtype" in lib.tode_last_error()
+    assert lib.tode_select_end_point(4, 2, 0, 3, None, _lib.C.addressof(dummy), _lib.C.addressof(dummy), None) == -1
+    assert lib.tode_select_end_point(0, 2, 0, 3, None, None, None, None) == 0
     a.n_features = 0
     assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1
     assert b"bad sizes" in lib.tode_last_error()

@@ -99,6 +99,74 @@ def test_no_t_eval_reports_end_point():
     assert (sol.stats["n_initialized"] == 1).all()
 
 
+@pytest.mark.parametrize("name,batch,dtype", [("vdp", 4096, F32), ("lorenz", 1000, F64), ("linear_decay", 70, F32), ("vdp", 1, F64)])
+def test_no_t_eval_through_the_fast_and_the_general_kernel(name, batch, dtype):
+    """reference adjoints.py:296-311: the interpolant of the batch's LAST iteration at t_end -- the dense
+    output of the last step for the samples that were still running then, the final state for the others."""
+    from torchode_amd import _lib
+
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    ts, te = w.t_eval[:, 0].contiguous(), w.t_eval[:, -1].contiguous()
+    if batch > 8:
+        ts[::3], te[::3] = te[::3].clone(), ts[::3].clone()  # every third sample backwards in time
+        if name != "linear_decay":
+            te[::3] = ts[::3] - 0.01 * (ts[::3] - te[::3])  # (the other two blow up in reverse time: a short way only)
+    ref = c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    fast = gpu_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    assert _lib.last_solve_kernel_name() == "tode::solve_pair_kernel"
+    general = gpu_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te, fast=False)
+    assert _lib.last_solve_kernel_name() == "tode::solve_kernel"
+    for sol in (fast, general):
+        assert sol.ys.shape == (batch, 1, w.y0.shape[1]) and torch.equal(sol.ts.cpu(), te[:, None])
+        assert_identical(sol, ref)
+        assert (sol.stats["n_initialized"] == 1).all()
+    if batch > 8:
+        slowest = ref["n_steps"] == ref["n_steps"].max()
+        assert 0 < slowest.sum() < batch  # both kinds of sample are in the batch
+    # a sample that needs the general kernel (max_steps) is handed over
+    capped = gpu_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te, max_steps=3)
+    assert_identical(capped, c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te, max_steps=3))
+
+
+def test_plain_fast_entry_point_without_evaluation_points_and_the_select_call():
+    """tode_solve_builtin_fast with n_eval == 0 leaves the last step's dense output in ys and the final
+    state in y_idle; tode_select_end_point, given the iteration count from the flags, makes the reference's
+    result of them."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    w = to.workloads.make("lorenz", batch=333, dtype=F32)
+    ts, te = w.t_eval[:, 0].contiguous(), w.t_eval[:, -1].contiguous()
+    ref = c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    y0, tsd, ted, params = w.y0.cuda(), ts.cuda(), te.cuda(), w.f.builtin_params().cuda()
+    B, F = y0.shape
+    ys = torch.full((B, 1, F), float("nan"), device="cuda")
+    y_idle = torch.full((B, F), float("nan"), device="cuda")
+    out = torch.full((4, B), -7, dtype=torch.int64, device="cuda")
+    flags = torch.full((_lib.FLAG_WORDS,), -1, dtype=torch.int32, device="cuda")
+    spec = dict(w.controller)
+    spec.pop("kind")
+    ctrl = to.IntegralController(**spec).c_struct()
+    a = _lib.SolveArgs()
+    a.dtype, a.method, a.term = _lib.F32, _lib.DOPRI5, w.f.builtin_kind
+    a.n_features, a.n_eval, a.n_params, a.batch, a.max_steps, a.iteration_cap = F, 0, 1, B, -1, -1
+    a.term_scalars = (_lib.C.c_double * 4)(*(list(w.f.builtin_scalars()) + [0.0] * 4)[:4])
+    a.y0, a.t_start, a.t_end, a.t_start_stride, a.t_end_stride = y0.data_ptr(), tsd.data_ptr(), ted.data_ptr(), 1, 1
+    a.params, a.ys, a.y_idle, a.flags = params.data_ptr(), ys.data_ptr(), y_idle.data_ptr(), flags.data_ptr()
+    stream = _lib.stream_of(y0)
+    _lib.check(lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream), "fast")
+    fl = flags.tolist()
+    assert fl[_lib.FLAG_NEEDS_GENERAL] == 0 and fl[_lib.FLAG_MAX_ITERATIONS] == int(ref["n_steps"].max())
+    at_last = ref["n_steps"] == ref["n_steps"].max()
+    assert torch.equal(ys.cpu()[at_last], ref["ys"][at_last]) and not torch.equal(ys.cpu()[~at_last], ref["ys"][~at_last])
+    _lib.check(lib.tode_select_end_point(B, F, _lib.F32, fl[_lib.FLAG_MAX_ITERATIONS], _lib.ptr(out[0]), _lib.ptr(ys), _lib.ptr(y_idle), stream), "select")
+    assert torch.equal(ys.cpu(), ref["ys"]) and torch.equal(out[0].cpu(), ref["n_steps"]) and (out[2] == 1).all() and (out[3] == 0).all()
+    # too many samples for this form: the caller is told so
+    a.batch = _lib.END_ONLY_MAX_BATCH + 1
+    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(ctrl), *(_lib.ptr(out[i]) for i in range(4)), stream) == -2
+    assert b"up to" in lib.tode_last_error()
+
+
 def test_user_dt0_skips_start_step():
     w = to.workloads.make("lorenz", batch=256, dtype=F32)
     dt0 = torch.full((256,), 0.01, dtype=F32)

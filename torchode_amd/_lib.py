@@ -13,7 +13,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
+END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
 F32, F64 = 0, 1
@@ -35,6 +36,7 @@ EXPORTS = (
     "tode_solve_builtin_fast",
     "tode_solve_builtin_fast_sync",
     "tode_mlp_pack_weights",
+    "tode_select_end_point",
     "tode_step_begin",
     "tode_step_stage",
     "tode_step_finish",
@@ -225,6 +227,8 @@ def load():
         lib.tode_solve_builtin.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.c_void_p]
         lib.tode_solve_builtin_fast.restype = C.c_int
         lib.tode_solve_builtin_fast.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5
+        lib.tode_select_end_point.restype = C.c_int
+        lib.tode_select_end_point.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.tode_mlp_pack_weights.restype = C.c_int
         lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         lib.tode_solve_builtin_fast_sync.restype = C.c_int

@@ -461,11 +461,12 @@ class AutoDiffAdjoint(nn.Module):
         # Common case first: one kernel, int64 stats written directly.  It reports through the
         # flag block when the batch needs the general kernel (which handles every case).
         has_general = f.builtin_kind in _lib.GENERAL_TERMS
-        fast_ok = E > 0 and not ctrl.has_dt_min and not ctrl.has_dt_max
+        fast_ok = not ctrl.has_dt_min and not ctrl.has_dt_max
         if has_general:
-            fast_ok = fast_ok and self.use_fast_path and E * y0.element_size() <= 1024
+            # (without evaluation points: the end point alone, built for batches that leave SIMDs to spare)
+            fast_ok = fast_ok and self.use_fast_path and E * y0.element_size() <= 1024 and (E > 0 or 0 < B <= _lib.END_ONLY_MAX_BATCH)
         else:
-            fast_ok = fast_ok and dtype == torch.float32
+            fast_ok = fast_ok and E > 0 and dtype == torch.float32
             if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
                 fast_ok = fast_ok and F in (32 * 32, 64 * 64) and E <= 8192
             else:

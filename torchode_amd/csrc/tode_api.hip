@@ -141,6 +141,12 @@ __global__ void finalize_kernel(long long batch, int last_iteration, const int32
     }
 }
 
+template <typename T>
+__global__ void select_end_point_kernel(long long n, int F, long long last, const int64_t *n_steps, T *ys, const T *y_idle) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && n_steps[i / F] < last) ys[i] = y_idle[i];
+}
+
 }  // namespace tode
 
 extern "C" {
@@ -199,11 +205,14 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (!a || !c) return fail(TODE_E_INVALID, "null argument struct");
     if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
         return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
-    if (a->n_eval == 0) return fail(TODE_E_UNSUPPORTED, "the fast entry point needs evaluation points");
+    const bool end_only = a->n_eval == 0;
+    if (end_only && (a->term == TODE_TERM_REACTION_DIFFUSION || a->term == TODE_TERM_MLP))
+        return fail(TODE_E_UNSUPPORTED, "without evaluation points the fast entry point covers the small systems only");
+    if (end_only && a->batch > 0 && !a->y_idle) return fail(TODE_E_INVALID, "n_eval == 0 needs y_idle");
     if (c->has_dt_min || c->has_dt_max) return fail(TODE_E_UNSUPPORTED, "the fast entry point does not take dt_min / dt_max");
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (!a->flags) return fail(TODE_E_INVALID, "null flags pointer");
-    if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || !a->t_eval || !a->ys || (a->n_params > 0 && !a->params) || !ns || !na || !ni || !st))
+    if (a->batch > 0 && (!a->y0 || !a->t_start || !a->t_end || (!end_only && !a->t_eval) || !a->ys || (a->n_params > 0 && !a->params) || !ns || !na || !ni || !st))
         return fail(TODE_E_INVALID, "null pointer");
     if (a->t_start_stride < 1 || a->t_end_stride < 1)
         return fail(TODE_E_INVALID, "t_start_stride / t_end_stride must be >= 1 (got %lld, %lld)", (long long)a->t_start_stride, (long long)a->t_end_stride);
@@ -225,6 +234,8 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         if (rc || used) return rc;
         if (g_fast_variant == 2) return fail(TODE_E_UNSUPPORTED, "the two-wavefront kernel does not cover this problem size");
     }
+    if (end_only)
+        return fail(TODE_E_UNSUPPORTED, "without evaluation points the fast entry point covers batches of up to %d samples", TODE_END_ONLY_MAX_BATCH);
     if (a->dtype == TODE_F32) return solve_fast_f32(*a, *c, ns, na, ni, st, s);
     return solve_fast_f64(*a, *c, ns, na, ni, st, s);
 }
@@ -266,10 +277,30 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller
         rc = wait_for_flags(host, sequence, s);
         if (rc == TODE_OK)
             for (int i = 0; i < TODE_FLAG_WORDS; ++i) flags_out[i] = host[i];
+        if (rc == TODE_OK && a->n_eval == 0 && !flags_out[TODE_FLAG_NEEDS_GENERAL])
+            rc = tode_select_end_point(a->batch, a->n_features, a->dtype, flags_out[TODE_FLAG_MAX_ITERATIONS], ns, a->ys, a->y_idle, stream);
     }
     // (after a failed wait the slot's words may be anything: the slot stays out of use)
     if (rc == TODE_OK || rc == TODE_E_INVALID || rc == TODE_E_UNSUPPORTED) pool->busy[slot].store(0, std::memory_order_release);
     return rc;
+}
+
+int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int64_t last_iteration, const int64_t *n_steps, void *ys,
+                          const void *y_idle, void *stream) {
+    using namespace tode;
+    if (batch < 0 || n_features <= 0) return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d", (long long)batch, n_features);
+    if (batch == 0) return TODE_OK;
+    if (!n_steps || !ys || !y_idle) return fail(TODE_E_INVALID, "null pointer");
+    const long long n = (long long)batch * n_features;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TODE_F32)
+        hipLaunchKernelGGL(select_end_point_kernel<float>, dim3(blocks), dim3(256), 0, s, n, (int)n_features, (long long)last_iteration, n_steps, (float *)ys, (const float *)y_idle);
+    else if (dtype == TODE_F64)
+        hipLaunchKernelGGL(select_end_point_kernel<double>, dim3(blocks), dim3(256), 0, s, n, (int)n_features, (long long)last_iteration, n_steps, (double *)ys, (const double *)y_idle);
+    else
+        return fail(TODE_E_INVALID, "unknown dtype %d", dtype);
+    return check_hip(hipGetLastError(), "tode_select_end_point launch");
 }
 
 int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_steps, const int32_t *n_accepted,

@@ -43,7 +43,13 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
     const bool live = lane < rows;
     const long long bs = live ? b : b0;
     const CtrlParams<T> &cp = p.cp;
-    const int E = p.n_eval;
+    // Without evaluation points the reference reports the end point alone (adjoints.py:296-311): the
+    // interpolant of the batch's last iteration at t_end.  Here: t_end as the one evaluation point of
+    // every sample, and the final state next to it in y_idle; which of the two a sample gets depends on
+    // whether its last step was the batch's last iteration, known only when all samples are done
+    // (tode_select_end_point).
+    const bool end_only = p.n_eval == 0;
+    const int E = end_only ? 1 : p.n_eval;
 
     T *rec = reinterpret_cast<T *>(smem_raw);                // [2][NF][64]
     int *ctl = reinterpret_cast<int *>(rec + 2 * NF * 64);   // [2] "stepper is done" per phase
@@ -175,6 +181,10 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
             o.n_steps[b] = n_steps;
             o.n_accepted[b] = n_acc;
             o.status[b] = 0;
+            if (end_only) {
+#pragma unroll
+                for (int f = 0; f < F; ++f) p.y_idle[b * F + f] = y[f];
+            }
         }
         int my_steps = live ? n_steps : 0, my_bail = (live && bail) ? 1 : 0;
 #pragma unroll
@@ -189,7 +199,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
     } else {
         // ============================== evaluator ==============================
         const T *tev_g = p.t_eval + bs * (long long)E;
-        if (STAGE_TE) {
+        if (STAGE_TE && !end_only) {
             // this group's block of t_eval (rows * E contiguous values), transposed into LDS
             const T *src = p.t_eval + b0 * E;
             const int n = rows * E;
@@ -206,7 +216,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
             }
         }
         // (LDS accesses of one wavefront complete in order; te_s is private to this wave)
-        auto te_at = [&](int e) -> T { return STAGE_TE ? te_s[e * 64 + lane] : tev_g[e]; };
+        auto te_at = [&](int e) -> T { return end_only ? te : (STAGE_TE ? te_s[e * 64 + lane] : tev_g[e]); };
         bool bail = false;
         {
             T prev_te = te_at(0);
