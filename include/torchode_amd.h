@@ -173,11 +173,12 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
 
 /*
  * The same solve as tode_solve_builtin for the common case, in one kernel launch
- * with no finalisation step: evaluation points given (n_eval > 0), no dt_min /
- * dt_max, and a batch in which every sample succeeds.  Uses of `args`: all
- * inputs, `ys` and `flags`; the int32 per-sample outputs, `y_idle`, `pending`
- * and `iteration_cap` are ignored.  The reference's int64 stats and status are
- * written directly (adjoints.py:267-294).
+ * with no finalisation step: evaluation points given (n_eval > 0; for
+ * n_eval == 0 see below), no dt_min / dt_max, and a batch in which every sample
+ * succeeds.  Uses of `args`: all inputs, `ys` and `flags` (and `y_idle` when
+ * n_eval == 0); the int32 per-sample outputs, `pending` and `iteration_cap` are
+ * ignored.  The reference's int64 stats and status are written directly
+ * (adjoints.py:267-294).
  *
  * On return (after stream synchronisation) flags[TODE_FLAG_MAX_ITERATIONS] is
  * the loop's iteration count, and flags[TODE_FLAG_NEEDS_GENERAL] == 1 means the
