@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 10
+#define TODE_ABI_VERSION 11
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -284,7 +284,9 @@ enum {
  *   copies f(t_start, y0) there).
  */
 typedef struct tode_step_state {
-    int32_t dtype;      /* TODE_F32 | TODE_F64 */
+    int32_t dtype;      /* TODE_F32 | TODE_F64: y0, y, k0, ratio_prev/pprev, ys, ystage, k */
+    int32_t time_dtype; /* TODE_F32 | TODE_F64: t_start, t_end, t_eval, t, dt, tnode and a user dt0
+                           (problems.py:44-56: time and data may differ) */
     int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 */
     int32_t n_features; /* F */
     int32_t n_eval;     /* E; 0: report y(t_end) only */

@@ -184,3 +184,86 @@ def test_graph_replay_with_loop_bookkeeping_cases():
     ts, te = w.t_eval[:, 0].contiguous(), w.t_eval[:, -1].contiguous()
     ref = c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
     assert_identical(stepwise_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te, graph=4), ref)
+
+
+# ---------------------------------------------------------------------------------------------
+# time and data in different dtypes (reference problems.py:44-56, tests/dtype_stability_test.py):
+# the per-step kernels against the protocol path (per-call operators), which states the same
+# arithmetic operator by operator -- same bits
+# ---------------------------------------------------------------------------------------------
+
+
+class OperatorTsit5(to.Tsit5):
+    """Not recognised by the fused paths: every protocol call goes through its own kernel."""
+
+
+class OperatorDopri5(to.Dopri5):
+    pass
+
+
+def mixed_case(case, time_dtype, data_dtype):
+    """(f, y0, t_start, t_end, t_eval, dt0, method, controller keywords, max_steps) on the GPU"""
+    dev = "cuda"
+    g = torch.Generator().manual_seed(17)
+    if case == "wide":  # rows of 100 values: one wavefront per sample
+        B, F = 37, 100
+        rate = (0.5 + torch.rand(B, F, generator=g, dtype=torch.float64)).to(data_dtype).to(dev)
+        f = lambda t, y: torch.sin(t).to(y.dtype)[:, None] - rate * y
+        y0 = torch.randn(B, F, generator=g, dtype=torch.float64)
+        t_eval = torch.linspace(0.0, 2.0, 9, dtype=torch.float64).repeat(B, 1) * (0.5 + torch.rand(B, 1, generator=g, dtype=torch.float64))
+        name = "tsit5"
+        ctrl = dict(kind="pid", atol=1e-6, rtol=1e-5, pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    else:
+        w = to.workloads.make("lorenz" if case == "lorenz" else "vdp", batch=200, dtype=torch.float64)
+        fd = copy.deepcopy(w.f).to(data_dtype).to(dev)
+        f = lambda t, y: fd(t, y) + 1e-3 * torch.cos(t).to(y.dtype)[:, None]  # (t matters, in its own dtype)
+        y0, t_eval, name, ctrl = w.y0, w.t_eval.clone(), w.method, dict(w.controller)
+    t_start, t_end, dt0, max_steps = t_eval[:, 0].clone(), t_eval[:, -1].clone(), None, None
+    if case == "backwards":
+        t_eval[::2] = t_eval[::2].flip(1)
+        t_eval[::2] = t_eval[::2, :1] - 0.01 * (t_eval[::2, :1] - t_eval[::2])  # (a short way back: no blow-up)
+        t_start, t_end = t_eval[:, 0].clone(), t_eval[:, -1].clone()
+    if case == "outside":  # first point after t_start, last point beyond t_end, rows not monotone
+        t_start, t_end = t_eval[:, 0] - 0.25, t_eval[:, -2].clone()
+        t_eval[::5, 3], t_eval[::5, 7] = t_eval[::5, 7].clone(), t_eval[::5, 3].clone()
+    if case == "no-t_eval":
+        t_eval = None
+    if case == "dt0":
+        dt0 = torch.full((y0.shape[0],), 1e-3, dtype=torch.float64)
+    if case == "limits":
+        ctrl.update(dt_min=2e-2, dt_max=0.25)
+        max_steps = 60
+    mv = lambda x, dt: None if x is None else x.to(dt).to(dev)
+    return f, mv(y0, data_dtype), mv(t_start, time_dtype), mv(t_end, time_dtype), mv(t_eval, time_dtype), mv(dt0, time_dtype), name, ctrl, max_steps
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", [(F64, F32), (F32, F64)], ids=["t64-y32", "t32-y64"])
+@pytest.mark.parametrize("case", ["vdp", "lorenz", "wide", "backwards", "outside", "no-t_eval", "dt0", "limits"])
+def test_mixed_dtypes_per_step_kernels_equal_the_operator_path(case, time_dtype, data_dtype):
+    f, y0, t_start, t_end, t_eval, dt0, name, ctrl, max_steps = mixed_case(case, time_dtype, data_dtype)
+    seen = []
+
+    def rhs(t, y):
+        seen.append((t.dtype, y.dtype))
+        return f(t, y)
+
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
+    fused_method, operator_method = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[name]
+    fused = to.AutoDiffAdjoint(fused_method(), make_controller(ctrl), max_steps=max_steps).solve(problem, to.ODETerm(rhs), dt0=dt0)
+    assert set(seen) == {(time_dtype, data_dtype)}
+    ops = to.AutoDiffAdjoint(operator_method(), make_controller(ctrl), max_steps=max_steps).solve(problem, to.ODETerm(rhs), dt0=dt0)
+    assert fused.ys.dtype == data_dtype and fused.ts.dtype == time_dtype and fused.ys.shape == ops.ys.shape
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert torch.equal(fused.stats[key], ops.stats[key]), key
+    assert torch.equal(fused.status, ops.status) and torch.equal(fused.stats["n_f_evals"], ops.stats["n_f_evals"])
+    E = fused.ys.shape[1]
+    written = torch.arange(E, device="cuda")[None, :] < ops.stats["n_initialized"][:, None]
+    if case == "outside":  # rows that are not monotone: compare what both wrote (the reference leaves the rest unset)
+        written = written & fused.ys.isfinite().all(dim=2) & ops.ys.isfinite().all(dim=2)
+    a, b = fused.ys[written], ops.ys[written]
+    assert bool(((a == b) | (a.isnan() & b.isnan())).all()), (a - b).abs().nan_to_num().max().item()
+    assert int(fused.stats["n_steps"].max()) >= 3
+    if case == "limits":
+        assert (fused.status != 0).any()  # dt_min reached somewhere (status 2), or max_steps (3)
+    elif case != "outside":
+        assert (fused.status == 0).all()

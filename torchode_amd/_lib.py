@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -139,6 +139,7 @@ class StepState(C.Structure):
 
     _fields_ = [
         ("dtype", C.c_int32),
+        ("time_dtype", C.c_int32),
         ("method", C.c_int32),
         ("n_features", C.c_int32),
         ("n_eval", C.c_int32),

@@ -111,7 +111,7 @@ class AutoDiffAdjoint(nn.Module):
         if wants_grad:
             # gradients through the loop: forward in the per-step kernels with a record of the loop
             # state, backward by a reverse sweep over the record
-            if not self._fused_ok(problem, term_):
+            if not self._fused_ok(problem, term_) or problem.data_dtype != problem.time_dtype:
                 raise RuntimeError(
                     "gradients through the loop are built for Dopri5 / Tsit5 with the library's controllers (one dtype); "
                     "with user-defined plug-ins call solve under torch.no_grad(), or use BacksolveAdjoint"
@@ -135,13 +135,19 @@ class AutoDiffAdjoint(nn.Module):
             and type(term).init is ODETerm.init
             and "vf" not in vars(term)
             and "init" not in vars(term)
-            and problem.data_dtype == problem.time_dtype
             and problem.data_dtype in _lib.DTYPES
+            and problem.time_dtype in _lib.DTYPES
         )
 
     def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
         f = term.f
-        return self._fused_ok(problem, term) and isinstance(f, BuiltinTerm) and f.builtin_kind in _lib.PERSISTENT_TERMS and not term.with_args
+        return (
+            self._fused_ok(problem, term)
+            and problem.data_dtype == problem.time_dtype  # (the whole-solve kernels are built for one dtype)
+            and isinstance(f, BuiltinTerm)
+            and f.builtin_kind in _lib.PERSISTENT_TERMS
+            and not term.with_args
+        )
 
     def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
         return self._fused_ok(problem, term)
@@ -268,18 +274,18 @@ class AutoDiffAdjoint(nn.Module):
         device, no host synchronisation per step (the host polls a flag every few iterations)."""
         lib = _lib.load()
         y0 = problem.y0.contiguous()
-        dev, dtype = y0.device, y0.dtype
+        dev, dtype, ttype = y0.device, y0.dtype, problem.time_dtype  # (time and data may differ, problems.py:44-56)
         B, F = y0.shape
         E = problem.n_evaluation_points
         t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
         t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
-        dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
+        dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()
         ctrl = self.step_size_controller.c_struct()
         stream = _lib.stream_of(y0)
         new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
 
         ys = new(B, max(E, 1), F)
-        t, dt = new(B), new(B)
+        t, dt = new(B, dt=ttype), new(B, dt=ttype)
         y, k0 = new(B, F), new(B, F)
         hist = new(2, B)
         ints = new(6, B, dt=torch.int32)
@@ -287,7 +293,7 @@ class AutoDiffAdjoint(nn.Module):
         flags = new(_lib.STEP_FLAG_WORDS, dt=torch.int32)
 
         s = _lib.StepState()
-        s.dtype, s.method, s.n_features, s.n_eval = _lib.DTYPES[dtype], self.step_method.method_id, F, E
+        s.dtype, s.time_dtype, s.method, s.n_features, s.n_eval = _lib.DTYPES[dtype], _lib.DTYPES[ttype], self.step_method.method_id, F, E
         s.batch = B
         s.max_steps = -1 if self.max_steps is None else int(self.max_steps)
         s.y0, s.t_start, s.t_end = y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr()
@@ -318,7 +324,7 @@ class AutoDiffAdjoint(nn.Module):
         keep = {}
 
         def stage_buffers(i):
-            keep["y", i], keep["t", i] = new(B, F), new(B)
+            keep["y", i], keep["t", i] = new(B, F), new(B, dt=ttype)
             s.ystage[i], s.tnode = keep["y", i].data_ptr(), keep["t", i].data_ptr()
             return keep["t", i], keep["y", i]
 

@@ -10,18 +10,26 @@
 // lanes strided over the features, norms in the fixed order of wave_row_norm (the stage
 // kernel is per element either way).  The stage arrays necessarily go through HBM because
 // f is external.
+//
+// Time and data may have different types (problems.py:44-56): every kernel is a template of the
+// time type TT and the data type T.  Times, steps and their limits are TT; the state, the
+// derivatives, the tolerances, the error ratio and the step factor are T; the step is converted
+// to T where it multiplies derivatives and the factor to TT where it multiplies the step, as in
+// the reference (runge_kutta.py:247, step_size_controllers.py:419, interpolation.py:32).
 #include "tode_solve.h"
 
 namespace tode {
 
-template <typename T> struct StepParams {
+template <typename TT, typename T> struct StepParams {
     // problem
-    const T *y0, *t_start, *t_end, *t_eval;
+    const T *y0;
+    const TT *t_start, *t_end, *t_eval;
     long long batch;
     int F, E;
     int max_steps;
     // loop state (device, owned by the caller for the duration of a solve)
-    T *t, *dt, *y, *k0;          // [B], [B], [B,F], [B,F] (FSAL derivative)
+    TT *t, *dt;                   // [B], [B]
+    T *y, *k0;                    // [B,F], [B,F] (FSAL derivative)
     T *ratio_prev, *ratio_pprev;  // [B] the last two accepted error ratios (PID history)
     int32_t *running, *cursor, *n_steps, *n_accepted, *status, *monotone;
     uint8_t *pending;  // [B,E]
@@ -30,33 +38,51 @@ template <typename T> struct StepParams {
     // per-iteration buffers
     T *ystage[7];    // [B,F] stage inputs; ystage[6] is y1
     const T *k[7];   // [B,F] stage derivatives; k[0] aliases k0
-    T *tnode;        // [B]
+    TT *tnode;       // [B]
     CtrlParams<T> cp;
+    TT dt_min, dt_max;  // limits of the step (step_size_controllers.py:406-422), in the time type
 };
+
+// dt_min / dt_max and the status of a step proposal, limits in the time type
+// (step_size_controllers.py:406-422, 751-767).
+template <typename TT, typename T>
+__device__ __forceinline__ int limit_step(const CtrlParams<T> &cp, TT dt_min, TT dt_max, T ratio, TT &dt_next) {
+    int status = finite_(ratio) ? 0 : 4;
+    if (cp.has_dt_min || cp.has_dt_max) {
+        const TT mag = abs_(dt_next);
+        TT c = mag;
+        if (cp.has_dt_min) c = tmax(c, dt_min);
+        if (cp.has_dt_max) c = tmin(c, dt_max);
+        const TT sg = (dt_next > 0) ? (TT)1 : ((dt_next < 0) ? (TT)-1 : dt_next);
+        dt_next = sg * c;
+        if (cp.has_dt_min && mag < dt_min) status = 2;
+    }
+    return status;
+}
 
 template <typename T> __device__ __forceinline__ T tab_a(int method, int i, int j) {
     return method == 1 ? (T)Tsit5Tab::a[i][j] : (T)Dopri5Tab::a[i][j];
 }
 
 // ystage[s] = fma(dt, sum_j a_sj k_j, y); tnode = fma(c_s, dt, t)   (runge_kutta.py:259-262)
-template <typename T, int METHOD, int S> __global__ void __launch_bounds__(256) stage_kernel(const StepParams<T> p) {
+template <typename TT, typename T, int METHOD, int S> __global__ void __launch_bounds__(256) stage_kernel(const StepParams<TT, T> p) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long n = p.batch * p.F;
     if (i >= n) return;
     const long long b = i / p.F;
-    const T dt = p.dt[b];
+    const T dt = (T)p.dt[b];
     T s = 0;
 #pragma unroll
     for (int j = 0; j < S; ++j) s = fma_((T)Tab::a[S][j], p.k[j][i], s);
     p.ystage[S][i] = fma_(dt, s, p.y[i]);
-    if (i - b * p.F == 0) p.tnode[b] = fma_((T)Tab::c[S], dt, p.t[b]);
+    if (i - b * p.F == 0) p.tnode[b] = fma_((TT)Tab::c[S], p.dt[b], p.t[b]);
 }
 
 // Start step, first half (step_size_controllers.py:459-479): from f0 = f(t0, y0) compute h0,
-// y1 = y0 + dir*h0*f0 -> ystage[1], t1 -> tnode; h0 is parked in dt.
-template <typename T> __global__ void __launch_bounds__(256) init_a_kernel(const StepParams<T> p) {
+// y1 = y0 + dir*h0*f0 -> ystage[1], t1 -> tnode; h0 (data type) is parked in ratio_prev.
+template <typename TT, typename T> __global__ void __launch_bounds__(256) init_a_kernel(const StepParams<TT, T> p) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= p.batch) return;
     const int F = p.F;
@@ -77,32 +103,34 @@ template <typename T> __global__ void __launch_bounds__(256) init_a_kernel(const
         }
     }
     const T d0 = sqrt_(a0), d1 = sqrt_(a1);
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
     T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
-    h0 = tmin(h0, abs_(te - ts));
-    const T dh = dir * h0;
+    h0 = tmin(h0, (T)abs_(te - ts));
+    const T dh = (fwd ? (T)1 : (T)-1) * h0;
     T *y1 = p.ystage[1] + b * F;
     for (int f = 0; f < F; ++f) y1[f] = fma_(dh, f0[f], y0[f]);
-    p.tnode[b] = fma_(dir, h0, ts);
-    p.dt[b] = h0;
+    p.tnode[b] = fma_(fwd ? (TT)1 : (TT)-1, (TT)h0, ts);
+    p.ratio_prev[b] = h0;
 }
 
 // Loop state at t_start; with FROM_F1 also the second half of the start step
 // (step_size_controllers.py:481-490 integral, 826-835 PID) from f1 = k[1].
-template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(256) init_b_kernel(const StepParams<T> p, const T *dt0) {
+template <typename TT, typename T, int CTRL, bool FROM_F1>
+__global__ void __launch_bounds__(256) init_b_kernel(const StepParams<TT, T> p, const TT *dt0) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= p.batch) return;
     const int F = p.F, E = p.E;
     const CtrlParams<T> &cp = p.cp;
     const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
-    T dt;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
+    const T dir = fwd ? (T)1 : (T)-1;
+    TT dt;
     if (FROM_F1) {
         const T *f1 = p.k[1] + b * F;
         const T sf = (T)__builtin_sqrt((double)F);
-        const T h0 = p.dt[b];
+        const T h0 = p.ratio_prev[b];
         T a1 = 0, a2 = 0;
         for (int f = 0; f < F; ++f) {
             T inv = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol);
@@ -129,11 +157,11 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
             T rm = (T)1 / m;
             h1 = rpow<T>(rm * (T)0.01, 1.0 / 5.0);
         }
-        dt = dir * tmin((T)100 * h0, h1);
+        dt = (TT)(dir * tmin((T)100 * h0, h1));
     } else {
         dt = dt0[b];
     }
-    const T tlo = tmin(ts, te), thi = tmax(te, ts);
+    const TT tlo = tmin(ts, te), thi = tmax(te, ts);
     p.t[b] = ts;
     p.dt[b] = tclamp(dt, tlo - ts, thi - ts);
     for (int f = 0; f < F; ++f) {
@@ -148,11 +176,11 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
     p.status[b] = 0;
     int cursor = 0, mono = 1;
     if (E > 0) {
-        const T *tev = p.t_eval + b * E;
-        T prev_te = tev[0];
+        const TT *tev = p.t_eval + b * E;
+        TT prev_te = tev[0];
         for (int e = 0; e < E; ++e) {
-            T cur = tev[e];
-            if (e > 0 && !(dir > 0 ? cur >= prev_te : cur <= prev_te)) mono = 0;
+            TT cur = tev[e];
+            if (e > 0 && !(fwd ? cur >= prev_te : cur <= prev_te)) mono = 0;
             prev_te = cur;
             p.pending[b * E + e] = 1;
         }
@@ -168,12 +196,19 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
 
 // Quartic of the attempted step for one feature, evaluated at time te (tsit5.py:123-139,
 // dopri5.py:53-60, interpolation.py:25-40, 138-175).  ks[s] = k_s[b,f].
-template <typename T, int METHOD> __device__ __forceinline__ T dense_value(T t0, T dt, T y0, T y1, const T (&ks)[7], bool fused, T te) {
+template <typename T> __device__ __forceinline__ T quartic_at(const T (&q)[5][1], T x) {
+    T y = q[4][0];
+    y = fma_(y, x, q[3][0]);
+    y = fma_(y, x, q[2][0]);
+    y = fma_(y, x, q[1][0]);
+    return fma_(y, x, q[0][0]);
+}
+
+template <typename TT, typename T, int METHOD>
+__device__ __forceinline__ T dense_value(TT t0, TT dt, T y0, T y1, const T (&ks)[7], bool fused, TT te) {
     T q[5][1];
-    quartic_elem<T, METHOD>(dt, y0, y1, ks, fused, q);
-    T out[1];
-    quartic_eval<T, 1>(q, t0, dt, te, out);
-    return out[0];
+    quartic_elem<T, METHOD>((T)dt, y0, y1, ks, fused, q);
+    return quartic_at<T>(q, (T)unit_time<TT>(te, t0, t0 + dt));
 }
 
 // Everything after the last stage of one loop iteration, for one sample per thread:
@@ -181,7 +216,7 @@ template <typename T, int METHOD> __device__ __forceinline__ T dense_value(T t0,
 // counters, dense output at the evaluation points the step passed, state update, running
 // flag, dt clamp (runge_kutta.py:265-272, step_size_controllers.py:370-429 / 715-774,
 // adjoints.py:150-255).
-template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<T> p) {
+template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<TT, T> p) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -190,9 +225,10 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     const CtrlParams<T> &cp = p.cp;
     const bool fused = F >= 58;
     const T sf = (T)__builtin_sqrt((double)F);
-    const T t0 = p.t[b], dt = p.dt[b];
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const TT t0 = p.t[b], dt = p.dt[b];
+    const T h = (T)dt;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
     const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
 
     // ---- error estimate and error ratio ----
@@ -201,7 +237,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
         T err = 0;
 #pragma unroll
         for (int s = 0; s < 7; ++s) {
-            T ps = dt * (T)Tab::b_err[s];
+            T ps = h * (T)Tab::b_err[s];
             T ks = p.k[s][b * F + f];
             if (fused)
                 err = fma_(ps, ks, err);
@@ -226,13 +262,13 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
     const T factor0 = dt_factor<T, CTRL>(cp, ratio, prev, pprev);
-    T dt_next = dt * factor0;
-    int status = limit_dt<T>(cp, ratio, dt_next);
+    TT dt_next = dt * (TT)factor0;
+    int status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
 
     const bool running = p.running[b] != 0;
     const bool move = accept && running;
-    const T t_new = move ? (t0 + dt) : t0;
-    const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+    const TT t_new = move ? (t0 + dt) : t0;
+    const bool running_new = fwd ? (t_new < te) : (t_new > te);
     const int n_steps = p.n_steps[b] + (running ? 1 : 0);
     p.n_steps[b] = n_steps;
     if (move) p.n_accepted[b] += 1;
@@ -242,7 +278,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
 
     // ---- dense output with the interpolant of the attempted step ----
     if (E > 0) {
-        const T *tev = p.t_eval + b * E;
+        const TT *tev = p.t_eval + b * E;
         T *ys = p.ys + b * (long long)E * F;
         uint8_t *pend = p.pending + b * (long long)E;
         const bool mono = p.monotone[b] != 0;
@@ -250,8 +286,8 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
         int e = mono ? cursor : 0;
         for (; e < E; ++e) {
             if (!pend[e]) continue;
-            const T te_e = tev[e];
-            const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+            const TT te_e = tev[e];
+            const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
             if (!passed) {
                 if (mono) break;
                 continue;
@@ -260,7 +296,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
                 T ks[7];
 #pragma unroll
                 for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-                ys[(long long)e * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
+                ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
             }
             pend[e] = 0;
         }
@@ -273,7 +309,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
             T ks[7];
 #pragma unroll
             for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-            p.ys[b * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
         }
     }
 
@@ -285,8 +321,8 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
         }
     }
     p.t[b] = t_new;
-    const T tlo = tmin(ts, te), thi = tmax(te, ts);
-    const T dtn = running_new ? dt_next : dt;
+    const TT tlo = tmin(ts, te), thi = tmax(te, ts);
+    const TT dtn = running_new ? dt_next : dt;
     p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
     if (CTRL == 1 && running_new && accept) {
         p.ratio_pprev[b] = prev;
@@ -302,7 +338,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
 // Per-sample scalars are computed by every lane; lane 0 stores them.
 // ------------------------------------------------------------------------------------------
 
-template <typename T> __global__ void __launch_bounds__(256) init_a_wave_kernel(const StepParams<T> p) {
+template <typename TT, typename T> __global__ void __launch_bounds__(256) init_a_wave_kernel(const StepParams<TT, T> p) {
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= p.batch) return;
     const int F = p.F, lane = threadIdx.x & 63;
@@ -310,28 +346,30 @@ template <typename T> __global__ void __launch_bounds__(256) init_a_wave_kernel(
     const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
     const T d0 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return y0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
     const T d1 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return f0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
     T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
-    h0 = tmin(h0, abs_(te - ts));
-    const T dh = dir * h0;
+    h0 = tmin(h0, (T)abs_(te - ts));
+    const T dh = (fwd ? (T)1 : (T)-1) * h0;
     T *y1 = p.ystage[1] + b * F;
     for (int f = lane; f < F; f += 64) y1[f] = fma_(dh, f0[f], y0[f]);
     if (lane == 0) {
-        p.tnode[b] = fma_(dir, h0, ts);
-        p.dt[b] = h0;
+        p.tnode[b] = fma_(fwd ? (TT)1 : (TT)-1, (TT)h0, ts);
+        p.ratio_prev[b] = h0;
     }
 }
 
-template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<T> p, const T *dt0) {
+template <typename TT, typename T, int CTRL, bool FROM_F1>
+__global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T> p, const TT *dt0) {
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= p.batch) return;
     const int F = p.F, E = p.E, lane = threadIdx.x & 63;
     const CtrlParams<T> &cp = p.cp;
     const T *y0 = p.y0 + b * F, *f0 = p.k[0] + b * F;
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
-    T dt;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
+    const T dir = fwd ? (T)1 : (T)-1;
+    TT dt;
     if (FROM_F1) {
         const T *f1 = p.k[1] + b * F;
         const T d1 = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) { return f0[f] * inv_scale(cp.atol, cp.rtol, y0[f]); });
@@ -339,7 +377,7 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
             const T df = f1[f] - f0[f];
             return df * inv_scale(cp.atol, cp.rtol, y0[f]);
         });
-        dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, p.dt[b], d1, d2n);
+        dt = (TT)initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, p.ratio_prev[b], d1, d2n);
     } else {
         dt = dt0[b];
     }
@@ -350,9 +388,9 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
     bool ordered = true;
     int cursor = 0;
     if (E > 0) {
-        const T *tev = p.t_eval + b * E;
+        const TT *tev = p.t_eval + b * E;
         for (int e = lane; e < E; e += 64) {
-            if (e > 0 && !(dir > 0 ? tev[e] >= tev[e - 1] : tev[e] <= tev[e - 1])) ordered = false;
+            if (e > 0 && !(fwd ? tev[e] >= tev[e - 1] : tev[e] <= tev[e - 1])) ordered = false;
             p.pending[b * E + e] = (e == 0 && tev[0] == ts) ? 0 : 1;
         }
         if (tev[0] == ts) {
@@ -362,7 +400,7 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
     }
     ordered = !__any(!ordered);
     if (lane == 0) {
-        const T tlo = tmin(ts, te), thi = tmax(te, ts);
+        const TT tlo = tmin(ts, te), thi = tmax(te, ts);
         p.t[b] = ts;
         p.dt[b] = tclamp(dt, tlo - ts, thi - ts);
         p.ratio_prev[b] = (T)1;
@@ -376,7 +414,7 @@ template <typename T, int CTRL, bool FROM_F1> __global__ void __launch_bounds__(
     }
 }
 
-template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<T> p) {
+template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<TT, T> p) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -384,9 +422,10 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     const int F = p.F, E = p.E, lane = threadIdx.x & 63;
     const CtrlParams<T> &cp = p.cp;
     const bool fused = F >= 58;
-    const T t0 = p.t[b], dt = p.dt[b];
-    const T ts = p.t_start[b], te = p.t_end[b];
-    const T dir = (te > ts) ? (T)1 : (T)-1;
+    const TT t0 = p.t[b], dt = p.dt[b];
+    const T h = (T)dt;
+    const TT ts = p.t_start[b], te = p.t_end[b];
+    const bool fwd = te > ts;
     const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
 
     // ---- error estimate and error ratio ----
@@ -394,7 +433,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
         T err = 0;
 #pragma unroll
         for (int s = 0; s < 7; ++s) {
-            const T ps = dt * (T)Tab::b_err[s], ks = p.k[s][b * F + f];
+            const T ps = h * (T)Tab::b_err[s], ks = p.k[s][b * F + f];
             if (fused)
                 err = fma_(ps, ks, err);
             else {
@@ -410,13 +449,13 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
 
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
-    T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
-    int status = limit_dt<T>(cp, ratio, dt_next);
+    TT dt_next = dt * (TT)dt_factor<T, CTRL>(cp, ratio, prev, pprev);
+    int status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
 
     const bool running = p.running[b] != 0;
     const bool move = accept && running;
-    const T t_new = move ? (t0 + dt) : t0;
-    const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+    const TT t_new = move ? (t0 + dt) : t0;
+    const bool running_new = fwd ? (t_new < te) : (t_new > te);
     const int n_steps = p.n_steps[b] + (running ? 1 : 0);
     if (p.max_steps != INT_MAX && n_steps >= p.max_steps) status = TODE_REACHED_MAX_STEPS;
     if (status == 0 && n_steps >= TODE_HARD_STEP_LIMIT) status = TODE_GENERAL_ERROR;
@@ -424,7 +463,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
     // ---- dense output with the interpolant of the attempted step: the quartic of a feature is
     // built once, when the first evaluation point turns out to have been passed ----
     if (E > 0) {
-        const T *tev = p.t_eval + b * E;
+        const TT *tev = p.t_eval + b * E;
         T *ys = p.ys + b * (long long)E * F;
         uint8_t *pend = p.pending + b * (long long)E;
         const bool mono = p.monotone[b] != 0;
@@ -434,8 +473,8 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
             bool built = false;
             for (int e = mono ? cursor : 0; e < E; ++e) {
                 if (!pend[e]) continue;
-                const T te_e = tev[e];
-                const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+                const TT te_e = tev[e];
+                const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
                 if (!passed) {
                     if (mono) break;
                     continue;
@@ -444,20 +483,18 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
                     T ks[7];
 #pragma unroll
                     for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-                    quartic_elem<T, METHOD>(dt, y[f], y1[f], ks, fused, q);
+                    quartic_elem<T, METHOD>(h, y[f], y1[f], ks, fused, q);
                     built = true;
                 }
-                T out[1];
-                quartic_eval<T, 1>(q, t0, dt, te_e, out);
-                ys[(long long)e * F + f] = out[0];
+                ys[(long long)e * F + f] = quartic_at<T>(q, (T)unit_time<TT>(te_e, t0, t0 + dt));
             }
         }
         // (every lane has finished reading the pending marks: the wavefront runs in lock step)
         int first_pending = E;
         for (int e = lane; e < E; e += 64) {
             if (!pend[e]) continue;
-            const T te_e = tev[e];
-            const bool passed = dir > 0 ? t_new >= te_e : t_new <= te_e;
+            const TT te_e = tev[e];
+            const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
             const bool taken = passed && (!mono || e >= cursor);
             if (taken) pend[e] = 0;
             else first_pending = min(first_pending, e);
@@ -470,7 +507,7 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
             T ks[7];
 #pragma unroll
             for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-            p.ys[b * F + f] = dense_value<T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
         }
     }
 
@@ -486,8 +523,8 @@ template <typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(25
         if (move) p.n_accepted[b] += 1;
         p.status[b] = status;
         p.t[b] = t_new;
-        const T tlo = tmin(ts, te), thi = tmax(te, ts);
-        const T dtn = running_new ? dt_next : dt;
+        const TT tlo = tmin(ts, te), thi = tmax(te, ts);
+        const TT dtn = running_new ? dt_next : dt;
         p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
         if (CTRL == 1 && running_new && accept) {
             p.ratio_pprev[b] = prev;
@@ -531,18 +568,18 @@ static __global__ void step_stats_kernel(long long batch, const int32_t *n_steps
     o_status[b] = status[b];
 }
 
-template <typename T> static StepParams<T> make_step_params(const tode_step_state &s, const tode_controller &c) {
-    StepParams<T> p;
+template <typename TT, typename T> static StepParams<TT, T> make_step_params(const tode_step_state &s, const tode_controller &c) {
+    StepParams<TT, T> p;
     p.y0 = (const T *)s.y0;
-    p.t_start = (const T *)s.t_start;
-    p.t_end = (const T *)s.t_end;
-    p.t_eval = (const T *)s.t_eval;
+    p.t_start = (const TT *)s.t_start;
+    p.t_end = (const TT *)s.t_end;
+    p.t_eval = (const TT *)s.t_eval;
     p.batch = s.batch;
     p.F = s.n_features;
     p.E = s.n_eval;
     p.max_steps = (s.max_steps < 0 || s.max_steps >= INT_MAX) ? INT_MAX : (int)s.max_steps;
-    p.t = (T *)s.t;
-    p.dt = (T *)s.dt;
+    p.t = (TT *)s.t;
+    p.dt = (TT *)s.dt;
     p.y = (T *)s.y;
     p.k0 = (T *)s.k0;
     p.ratio_prev = (T *)s.ratio_prev;
@@ -560,8 +597,10 @@ template <typename T> static StepParams<T> make_step_params(const tode_step_stat
         p.ystage[i] = (T *)s.ystage[i];
         p.k[i] = (const T *)s.k[i];
     }
-    p.tnode = (T *)s.tnode;
+    p.tnode = (TT *)s.tnode;
     p.cp = make_ctrl<T>(c);
+    p.dt_min = (TT)c.dt_min;
+    p.dt_max = (TT)c.dt_max;
     return p;
 }
 
@@ -569,6 +608,7 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     if (!s || !c) return fail(TODE_E_INVALID, "null argument struct");
     if (s->batch < 0 || s->n_features <= 0 || s->n_eval < 0) return fail(TODE_E_INVALID, "bad sizes");
     if (s->dtype != TODE_F32 && s->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", s->dtype);
+    if (s->time_dtype != TODE_F32 && s->time_dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown time dtype %d", s->time_dtype);
     if (s->method != TODE_DOPRI5 && s->method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", s->method);
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (!s->flags) return fail(TODE_E_INVALID, "null flags pointer");
@@ -579,15 +619,26 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     return TODE_OK;
 }
 
-#define TODE_DISPATCH_T(dtype, EXPR)    \
-    do {                                \
-        if ((dtype) == TODE_F32) {      \
-            using T = float;            \
-            EXPR;                       \
-        } else {                        \
-            using T = double;           \
-            EXPR;                       \
-        }                               \
+// The statements given, with TT = the state's time type and T = its data type
+#define TODE_DISPATCH_T(state, ...)                                        \
+    do {                                                                   \
+        if ((state)->time_dtype == TODE_F32 && (state)->dtype == TODE_F32) {  \
+            using TT = float;                                              \
+            using T = float;                                               \
+            __VA_ARGS__;                                                   \
+        } else if ((state)->time_dtype == TODE_F64 && (state)->dtype == TODE_F64) { \
+            using TT = double;                                             \
+            using T = double;                                              \
+            __VA_ARGS__;                                                   \
+        } else if ((state)->time_dtype == TODE_F64) {                      \
+            using TT = double;                                             \
+            using T = float;                                               \
+            __VA_ARGS__;                                                   \
+        } else {                                                           \
+            using TT = float;                                              \
+            using T = double;                                              \
+            __VA_ARGS__;                                                   \
+        }                                                                  \
     } while (0)
 
 }  // namespace tode
@@ -606,38 +657,38 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
         if (blocks == 0) return check_hip(hipGetLastError(), "tode_step_begin");
         if (dt0) {
             if (!s->k[0]) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
-            TODE_DISPATCH_T(s->dtype, {
-                auto p = make_step_params<T>(*s, *c);
+            TODE_DISPATCH_T(s, {
+                auto p = make_step_params<TT, T>(*s, *c);
                 if (wide)
-                    hipLaunchKernelGGL((init_b_wave_kernel<T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);  // (CTRL is unused here)
+                    hipLaunchKernelGGL((init_b_wave_kernel<TT, T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);  // (CTRL is unused here)
                 else if (c->kind == TODE_CTRL_INTEGRAL)
-                    hipLaunchKernelGGL((init_b_kernel<T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
+                    hipLaunchKernelGGL((init_b_kernel<TT, T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);
                 else
-                    hipLaunchKernelGGL((init_b_kernel<T, 1, false>), dim3(blocks), dim3(256), 0, st, p, (const T *)dt0);
+                    hipLaunchKernelGGL((init_b_kernel<TT, T, 1, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);
             });
         } else {
             if (!s->k[0] || !s->ystage[1]) return fail(TODE_E_INVALID, "k[0] or ystage[1] is null");
-            TODE_DISPATCH_T(s->dtype, {
-                auto p = make_step_params<T>(*s, *c);
+            TODE_DISPATCH_T(s, {
+                auto p = make_step_params<TT, T>(*s, *c);
                 if (wide)
-                    hipLaunchKernelGGL(init_a_wave_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((init_a_wave_kernel<TT, T>), dim3(blocks), dim3(256), 0, st, p);
                 else
-                    hipLaunchKernelGGL(init_a_kernel<T>, dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((init_a_kernel<TT, T>), dim3(blocks), dim3(256), 0, st, p);
             });
         }
     } else {
         if (blocks == 0) return TODE_OK;
         if (!s->k[0] || !s->k[1]) return fail(TODE_E_INVALID, "k[0] or k[1] is null");
-        TODE_DISPATCH_T(s->dtype, {
-            auto p = make_step_params<T>(*s, *c);
+        TODE_DISPATCH_T(s, {
+            auto p = make_step_params<TT, T>(*s, *c);
             if (wide && c->kind == TODE_CTRL_INTEGRAL)
-                hipLaunchKernelGGL((init_b_wave_kernel<T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+                hipLaunchKernelGGL((init_b_wave_kernel<TT, T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const TT *)nullptr);
             else if (wide)
-                hipLaunchKernelGGL((init_b_wave_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+                hipLaunchKernelGGL((init_b_wave_kernel<TT, T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const TT *)nullptr);
             else if (c->kind == TODE_CTRL_INTEGRAL)
-                hipLaunchKernelGGL((init_b_kernel<T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+                hipLaunchKernelGGL((init_b_kernel<TT, T, 0, true>), dim3(blocks), dim3(256), 0, st, p, (const TT *)nullptr);
             else
-                hipLaunchKernelGGL((init_b_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const T *)nullptr);
+                hipLaunchKernelGGL((init_b_kernel<TT, T, 1, true>), dim3(blocks), dim3(256), 0, st, p, (const TT *)nullptr);
         });
     }
     return check_hip(hipGetLastError(), "tode_step_begin");
@@ -656,14 +707,14 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
     hipStream_t st = (hipStream_t)stream;
     const unsigned blocks = (unsigned)((n + 255) / 256);
 #define TODE_STAGE_CASE(M, S) \
-    case S: hipLaunchKernelGGL((stage_kernel<T, M, S>), dim3(blocks), dim3(256), 0, st, p); break;
+    case S: hipLaunchKernelGGL((stage_kernel<TT, T, M, S>), dim3(blocks), dim3(256), 0, st, p); break;
 #define TODE_STAGE_SWITCH(M)                                                                  \
     switch (stage) {                                                                          \
         TODE_STAGE_CASE(M, 1) TODE_STAGE_CASE(M, 2) TODE_STAGE_CASE(M, 3) TODE_STAGE_CASE(M, 4) \
         TODE_STAGE_CASE(M, 5) TODE_STAGE_CASE(M, 6)                                           \
     }
-    TODE_DISPATCH_T(s->dtype, {
-        auto p = make_step_params<T>(*s, *c);
+    TODE_DISPATCH_T(s, {
+        auto p = make_step_params<TT, T>(*s, *c);
         if (s->method == TODE_TSIT5) {
             TODE_STAGE_SWITCH(1)
         } else {
@@ -686,31 +737,31 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
         for (int j = 0; j < 7; ++j)
             if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
         if (!s->ystage[6]) return fail(TODE_E_INVALID, "ystage[6] is null");
-        TODE_DISPATCH_T(s->dtype, {
-            auto p = make_step_params<T>(*s, *c);
+        TODE_DISPATCH_T(s, {
+            auto p = make_step_params<TT, T>(*s, *c);
             const bool pid = c->kind == TODE_CTRL_PID;
             if (wide) {
                 if (s->method == TODE_TSIT5) {
                     if (pid)
-                        hipLaunchKernelGGL((finish_wave_kernel<T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
+                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
                     else
-                        hipLaunchKernelGGL((finish_wave_kernel<T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
+                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
                 } else {
                     if (pid)
-                        hipLaunchKernelGGL((finish_wave_kernel<T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
+                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
                     else
-                        hipLaunchKernelGGL((finish_wave_kernel<T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
+                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
                 }
             } else if (s->method == TODE_TSIT5) {
                 if (pid)
-                    hipLaunchKernelGGL((finish_kernel<T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((finish_kernel<TT, T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
                 else
-                    hipLaunchKernelGGL((finish_kernel<T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((finish_kernel<TT, T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
             } else {
                 if (pid)
-                    hipLaunchKernelGGL((finish_kernel<T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((finish_kernel<TT, T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
                 else
-                    hipLaunchKernelGGL((finish_kernel<T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
+                    hipLaunchKernelGGL((finish_kernel<TT, T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
             }
         });
     }
