@@ -238,6 +238,32 @@ def test_gradients_reach_tensors_inside_args():
 
 
 @gpu
+@pytest.mark.parametrize("time_dtype,data_dtype,tol", [(torch.float32, torch.float64, 2e-5), (torch.float64, torch.float32, 2e-3)], ids=["t32-y64", "t64-y32"])
+def test_gradients_with_time_and_data_in_different_dtypes(time_dtype, data_dtype, tol):
+    """problems.py:44-56 allows the two dtypes to differ; the forward pass keeps them apart in the
+    kernels and the reverse sweep in its torch operations."""
+    y0, A = inputs()
+    y0 = y0.detach().to(data_dtype).requires_grad_()
+    A = nn.Parameter(A.detach().to(data_dtype))
+    t_eval = torch.tensor(T_EVAL, dtype=time_dtype, device="cuda")
+    seen = set()
+
+    class Watched(LinearDynamics):
+        def forward(self, t, y):
+            seen.add((t.dtype, y.dtype))
+            return super().forward(t, y)
+
+    solution = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-7, 1e-7)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=to.ODETerm(Watched(A)))
+    assert solution.ys.dtype == data_dtype and solution.ts.dtype == time_dtype and solution.ys.requires_grad
+    solution.ys.square().sum().backward()
+    assert seen == {(time_dtype, data_dtype)}
+    y0_ref, A_ref = y0.detach().double().requires_grad_(), A.detach().double().requires_grad_()
+    closed_form(y0_ref, A_ref, t_eval.double()).square().sum().backward()
+    torch.testing.assert_close(y0.grad.double(), y0_ref.grad, rtol=tol, atol=tol)
+    torch.testing.assert_close(A.grad.double(), A_ref.grad, rtol=tol, atol=tol)
+
+
+@gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))

@@ -111,9 +111,9 @@ class AutoDiffAdjoint(nn.Module):
         if wants_grad:
             # gradients through the loop: forward in the per-step kernels with a record of the loop
             # state, backward by a reverse sweep over the record
-            if not self._fused_ok(problem, term_) or problem.data_dtype != problem.time_dtype:
+            if not self._fused_ok(problem, term_):
                 raise RuntimeError(
-                    "gradients through the loop are built for Dopri5 / Tsit5 with the library's controllers (one dtype); "
+                    "gradients through the loop are built for Dopri5 / Tsit5 with the library's controllers; "
                     "with user-defined plug-ins call solve under torch.no_grad(), or use BacksolveAdjoint"
                 )
             from . import autodiff
