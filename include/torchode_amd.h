@@ -22,14 +22,14 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 11
+#define TODE_ABI_VERSION 12
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
 /* single step methods: reference single_step_methods/dopri5.py, tsit5.py */
 enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1 };
 /* step size controllers: reference step_size_controllers.py:260 (integral), :554 (PID) */
-enum { TODE_CTRL_INTEGRAL = 0, TODE_CTRL_PID = 1 };
+enum { TODE_CTRL_INTEGRAL = 0, TODE_CTRL_PID = 1, TODE_CTRL_FIXED = 2 /* per-step entry points only */ };
 /* right-hand sides the persistent kernel evaluates itself */
 enum {
     TODE_TERM_LINEAR_DECAY = 0,       /* dy/dt = -k y, k [B,F] */
@@ -318,6 +318,9 @@ typedef struct tode_step_state {
                             tode_step_finish leaves there TODE_STEP_FLAG_STOPPED and
                             TODE_STEP_FLAG_ITERATIONS as of its iteration, so that the host can see the loop
                             end by reading its own memory, without a synchronisation */
+    const void *fixed_dt; /* [B] time dtype, TODE_CTRL_FIXED only: the step every running sample takes
+                             (step_size_controllers.py:116-167: every step is accepted and the next step
+                             is dt0 again, whatever the last one was clamped to) */
 } tode_step_state;
 
 /*

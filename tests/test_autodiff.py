@@ -264,6 +264,25 @@ def test_gradients_with_time_and_data_in_different_dtypes(time_dtype, data_dtype
 
 
 @gpu
+@pytest.mark.parametrize("method", [to.Dopri5, to.Tsit5])
+def test_gradients_with_fixed_steps(method):
+    """Fixed steps (step_size_controllers.py:116-167) through the loop: the step sizes are constants, the
+    gradient is that of the Runge-Kutta map itself and agrees with the closed form to the method's error."""
+    y0, A = inputs()
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+    dt0 = torch.tensor([0.013, 0.017], dtype=torch.double, device="cuda")
+    solution = to.AutoDiffAdjoint(method(), to.FixedStepController()).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=to.ODETerm(LinearDynamics(A)), dt0=dt0)
+    n = solution.stats["n_steps"].tolist()  # 3 / 0.013 and 4 / 0.017 steps, one more where the sums of the steps fall short of t_end
+    assert solution.ys.requires_grad and n[0] in (231, 232) and n[1] in (236, 237) and (solution.status == 0).all()
+    weights = torch.linspace(0.5, 1.5, solution.ys.numel(), dtype=torch.double, device="cuda").reshape(solution.ys.shape)
+    (solution.ys * weights).sum().backward()
+    y0_ref, A_ref = y0.detach().clone().requires_grad_(), A.detach().clone().requires_grad_()
+    (closed_form(y0_ref, A_ref, t_eval) * weights).sum().backward()
+    torch.testing.assert_close(y0.grad, y0_ref.grad, rtol=1e-8, atol=1e-9)
+    torch.testing.assert_close(A.grad, A_ref.grad, rtol=1e-8, atol=1e-9)
+
+
+@gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))

@@ -267,3 +267,39 @@ def test_mixed_dtypes_per_step_kernels_equal_the_operator_path(case, time_dtype,
         assert (fused.status != 0).any()  # dt_min reached somewhere (status 2), or max_steps (3)
     elif case != "outside":
         assert (fused.status == 0).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# fixed steps (reference step_size_controllers.py:116-167, tests/fixed_step_controller_test.py):
+# Dopri5 / Tsit5 with the library's FixedStepController run in the per-step kernels; a subclass of
+# the method sends the same solve through the operator path
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", [(F32, F32), (F64, F64), (F64, F32)], ids=["f32", "f64", "t64-y32"])
+@pytest.mark.parametrize("case", ["vdp", "wide", "backwards", "no-t_eval", "outside"])
+def test_fixed_steps_in_the_per_step_kernels_equal_the_operator_path(case, time_dtype, data_dtype):
+    f, y0, t_start, t_end, t_eval, _, name, _, _ = mixed_case(case, time_dtype, data_dtype)
+    B = y0.shape[0]
+    span = (t_end - t_start).double()
+    dt0 = (span / (40.0 + torch.arange(B, device="cuda", dtype=torch.float64) % 7 + 0.37)).to(time_dtype)  # 41 to 47 steps, the last one cut
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
+    fused_method, operator_method = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[name]
+    fused = to.AutoDiffAdjoint(fused_method(), to.FixedStepController(), max_steps=44 if case == "outside" else None).solve(problem, to.ODETerm(f), dt0=dt0)
+    ops = to.AutoDiffAdjoint(operator_method(), to.FixedStepController(), max_steps=44 if case == "outside" else None).solve(problem, to.ODETerm(f), dt0=dt0)
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert torch.equal(fused.stats[key], ops.stats[key]), key
+    assert torch.equal(fused.status, ops.status) and torch.equal(fused.stats["n_f_evals"], ops.stats["n_f_evals"])
+    assert torch.equal(fused.stats["n_steps"], fused.stats["n_accepted"]) and 38 <= int(fused.stats["n_steps"].min()) <= int(fused.stats["n_steps"].max()) <= 48
+    E = fused.ys.shape[1]
+    written = torch.arange(E, device="cuda")[None, :] < ops.stats["n_initialized"][:, None]
+    if case == "outside":
+        written = written & fused.ys.isfinite().all(dim=2) & ops.ys.isfinite().all(dim=2)
+        assert (fused.status == 3).any()  # max_steps cuts the slower samples short
+    else:
+        assert (fused.status == 0).all()
+    a, b = fused.ys[written], ops.ys[written]
+    assert bool(((a == b) | (a.isnan() & b.isnan())).all()), (a - b).abs().nan_to_num().max().item()
+    assert a.isfinite().float().mean().item() > 0.5  # (some of the stiffer samples blow up at these step sizes, in both paths alike)
+    with pytest.raises(AssertionError, match="dt0"):
+        to.AutoDiffAdjoint(fused_method(), to.FixedStepController()).solve(problem, to.ODETerm(f))

@@ -10,7 +10,7 @@ from .problems import InitialValueProblem
 from .interpolation import _PolynomialInterpolation
 from .single_step_methods import Dopri5, Tsit5
 from .solution import Solution
-from .step_size_controllers import IntegralController, PIDController
+from .step_size_controllers import FixedStepController, IntegralController, PIDController
 from .terms import ODETerm
 
 _PROTOCOL_NAMES = (
@@ -128,7 +128,7 @@ class AutoDiffAdjoint(nn.Module):
         m, c = self.step_method, self.step_size_controller
         return (
             _library_object(m, (Dopri5, Tsit5))
-            and _library_object(c, (IntegralController, PIDController))
+            and _library_object(c, (IntegralController, PIDController, FixedStepController))
             and c.fusable
             and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
             and type(term).vf is ODETerm.vf
@@ -144,6 +144,7 @@ class AutoDiffAdjoint(nn.Module):
         return (
             self._fused_ok(problem, term)
             and problem.data_dtype == problem.time_dtype  # (the whole-solve kernels are built for one dtype)
+            and type(self.step_size_controller) is not FixedStepController
             and isinstance(f, BuiltinTerm)
             and f.builtin_kind in _lib.PERSISTENT_TERMS
             and not term.with_args
@@ -280,6 +281,8 @@ class AutoDiffAdjoint(nn.Module):
         t_start, t_end = problem.t_start.contiguous(), problem.t_end.contiguous()
         t_eval = None if problem.t_eval is None else problem.t_eval.contiguous()
         dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()
+        fixed = type(self.step_size_controller) is FixedStepController
+        assert not fixed or dt0_ is not None, "Fixed step size solving requires you to configure dt0"
         ctrl = self.step_size_controller.c_struct()
         stream = _lib.stream_of(y0)
         new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
@@ -306,6 +309,7 @@ class AutoDiffAdjoint(nn.Module):
         # by reading its own memory, after every iteration and without a synchronisation
         mirror = torch.empty(2, dtype=torch.int32, pin_memory=True)
         s.host_flags = mirror.data_ptr()
+        s.fixed_dt = dt0_.data_ptr() if fixed else None
         stopped_on_device = mirror.numpy()
         stopped_on_device[:] = 0  # (on the host: torch.zeros on pinned memory costs 0.2 ms)
         sref, cref = _lib.C.byref(s), _lib.C.byref(ctrl)

@@ -56,7 +56,7 @@ class LoopRecord:
 class Replay:
     """One loop iteration (and the start of the loop) as differentiable torch operations."""
 
-    def __init__(self, method, controller, term, args, problem: InitialValueProblem, through_control: bool):
+    def __init__(self, method, controller, term, args, problem: InitialValueProblem, through_control: bool, dt0=None):
         tab = method.tableau
         self.a = [[float(x) for x in row] for row in tab.a.tolist()]
         self.c = [float(x) for x in tab.c.tolist()]
@@ -66,6 +66,8 @@ class Replay:
         self.order = float(method.convergence_order())
         c = controller.c_struct()
         self.pid = c.kind == _lib.CTRL_PID
+        # fixed steps (reference step_size_controllers.py:116-167): every step accepted, the next step is dt0 again
+        self.fixed_dt = dt0.detach().to(problem.t_start.dtype) if c.kind == _lib.CTRL_FIXED else None
         self.atol, self.rtol = float(c.atol), float(c.rtol)
         self.safety, self.fmin, self.fmax = float(c.safety), float(c.factor_min), float(c.factor_max)
         self.dt_min = float(c.dt_min) if c.has_dt_min else None
@@ -117,6 +119,8 @@ class Replay:
             yi = y + dtd[:, None] * s
             ks.append(self.f(t + self.c[i] * dt, yi))
         y1 = yi
+        if self.fixed_dt is not None:
+            return ks, y1, torch.zeros_like(dtd), self.fixed_dt
         err = dtd[:, None] * sum(self.b_err[s] * ks[s] for s in range(7) if self.b_err[s] != 0.0)
         scale = self.atol + self.rtol * torch.maximum(y.abs(), y1.abs())
         ratio = torch.clamp_min(self.rms(err.abs() / scale), 1e-38)
@@ -221,7 +225,7 @@ class SolveThroughLoop(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_ys, *unused):
         adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
-        replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, ctx.args, problem, adjoint.backprop_through_step_size_control)
+        replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, ctx.args, problem, adjoint.backprop_through_step_size_control, ctx.dt0)
         states = ctx.record.trimmed(ctx.record.iterations)
         E = problem.n_evaluation_points
         hits = simulate_hits(replay, states, E)

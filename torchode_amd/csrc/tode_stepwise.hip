@@ -41,6 +41,7 @@ template <typename TT, typename T> struct StepParams {
     TT *tnode;       // [B]
     CtrlParams<T> cp;
     TT dt_min, dt_max;  // limits of the step (step_size_controllers.py:406-422), in the time type
+    const TT *fixed_dt;  // [B] CTRL == 2: the fixed step (step_size_controllers.py:116-167)
 };
 
 // dt_min / dt_max and the status of a step proposal, limits in the time type
@@ -231,9 +232,9 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     const bool fwd = te > ts;
     const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
 
-    // ---- error estimate and error ratio ----
+    // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
     T acc = 0;
-    for (int f = 0; f < F; ++f) {
+    for (int f = 0; CTRL != 2 && f < F; ++f) {
         T err = 0;
 #pragma unroll
         for (int s = 0; s < 7; ++s) {
@@ -257,13 +258,18 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         }
     }
     const T ratio = tmax(sqrt_(acc), (T)1e-38);
-    const bool accept = ratio < (T)1;
+    const bool accept = CTRL == 2 || ratio < (T)1;
 
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
-    const T factor0 = dt_factor<T, CTRL>(cp, ratio, prev, pprev);
-    TT dt_next = dt * (TT)factor0;
-    int status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
+    TT dt_next;
+    int status = 0;
+    if (CTRL == 2) {
+        dt_next = p.fixed_dt[b];
+    } else {
+        dt_next = dt * (TT)dt_factor<T, (CTRL == 2 ? 0 : CTRL)>(cp, ratio, prev, pprev);
+        status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
+    }
 
     const bool running = p.running[b] != 0;
     const bool move = accept && running;
@@ -428,8 +434,8 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     const bool fwd = te > ts;
     const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
 
-    // ---- error estimate and error ratio ----
-    const T norm = wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
+    // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
+    const T norm = CTRL == 2 ? (T)0 : wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
         T err = 0;
 #pragma unroll
         for (int s = 0; s < 7; ++s) {
@@ -445,12 +451,18 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         return abs_(err) / fma_(cp.rtol, m, cp.atol);
     });
     const T ratio = tmax(norm, (T)1e-38);
-    const bool accept = ratio < (T)1;
+    const bool accept = CTRL == 2 || ratio < (T)1;
 
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
-    TT dt_next = dt * (TT)dt_factor<T, CTRL>(cp, ratio, prev, pprev);
-    int status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
+    TT dt_next;
+    int status = 0;
+    if (CTRL == 2) {
+        dt_next = p.fixed_dt[b];
+    } else {
+        dt_next = dt * (TT)dt_factor<T, (CTRL == 2 ? 0 : CTRL)>(cp, ratio, prev, pprev);
+        status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
+    }
 
     const bool running = p.running[b] != 0;
     const bool move = accept && running;
@@ -601,6 +613,7 @@ template <typename TT, typename T> static StepParams<TT, T> make_step_params(con
     p.cp = make_ctrl<T>(c);
     p.dt_min = (TT)c.dt_min;
     p.dt_max = (TT)c.dt_max;
+    p.fixed_dt = (const TT *)s.fixed_dt;
     return p;
 }
 
@@ -610,7 +623,9 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     if (s->dtype != TODE_F32 && s->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", s->dtype);
     if (s->time_dtype != TODE_F32 && s->time_dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown time dtype %d", s->time_dtype);
     if (s->method != TODE_DOPRI5 && s->method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", s->method);
-    if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
+    if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID && c->kind != TODE_CTRL_FIXED)
+        return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
+    if (c->kind == TODE_CTRL_FIXED && s->batch > 0 && !s->fixed_dt) return fail(TODE_E_INVALID, "the fixed-step controller needs fixed_dt");
     if (!s->flags) return fail(TODE_E_INVALID, "null flags pointer");
     if (s->batch > 0 && (!s->y0 || !s->t_start || !s->t_end || !s->t || !s->dt || !s->y || !s->k0 || !s->ratio_prev || !s->ratio_pprev ||
                          !s->running || !s->cursor || !s->n_steps || !s->n_accepted || !s->status || !s->monotone || !s->ys || !s->tnode))
@@ -661,12 +676,13 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
                 auto p = make_step_params<TT, T>(*s, *c);
                 if (wide)
                     hipLaunchKernelGGL((init_b_wave_kernel<TT, T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);  // (CTRL is unused here)
-                else if (c->kind == TODE_CTRL_INTEGRAL)
+                else if (c->kind != TODE_CTRL_PID)  // (CTRL is unused here as well)
                     hipLaunchKernelGGL((init_b_kernel<TT, T, 0, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);
                 else
                     hipLaunchKernelGGL((init_b_kernel<TT, T, 1, false>), dim3(blocks), dim3(256), 0, st, p, (const TT *)dt0);
             });
         } else {
+            if (c->kind == TODE_CTRL_FIXED) return fail(TODE_E_INVALID, "the fixed-step controller needs dt0");
             if (!s->k[0] || !s->ystage[1]) return fail(TODE_E_INVALID, "k[0] or ystage[1] is null");
             TODE_DISPATCH_T(s, {
                 auto p = make_step_params<TT, T>(*s, *c);
@@ -677,6 +693,7 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
             });
         }
     } else {
+        if (c->kind == TODE_CTRL_FIXED) return fail(TODE_E_INVALID, "the fixed-step controller has no second phase");
         if (blocks == 0) return TODE_OK;
         if (!s->k[0] || !s->k[1]) return fail(TODE_E_INVALID, "k[0] or k[1] is null");
         TODE_DISPATCH_T(s, {
@@ -726,6 +743,14 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
     return check_hip(hipGetLastError(), "tode_step_stage");
 }
 
+#define TODE_FINISH(KERNEL, M, C) hipLaunchKernelGGL((KERNEL<TT, T, M, C>), dim3(blocks), dim3(256), 0, st, p)
+#define TODE_FINISH_CTRL(KERNEL, M)                                     \
+    do {                                                                \
+        if (c->kind == TODE_CTRL_PID) TODE_FINISH(KERNEL, M, 1);        \
+        else if (c->kind == TODE_CTRL_FIXED) TODE_FINISH(KERNEL, M, 2); \
+        else TODE_FINISH(KERNEL, M, 0);                                 \
+    } while (0)
+
 int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *stream) {
     using namespace tode;
     int rc = check_state(s, c);
@@ -739,35 +764,21 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
         if (!s->ystage[6]) return fail(TODE_E_INVALID, "ystage[6] is null");
         TODE_DISPATCH_T(s, {
             auto p = make_step_params<TT, T>(*s, *c);
-            const bool pid = c->kind == TODE_CTRL_PID;
+            const bool tsit5 = s->method == TODE_TSIT5;
             if (wide) {
-                if (s->method == TODE_TSIT5) {
-                    if (pid)
-                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
-                    else
-                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
-                } else {
-                    if (pid)
-                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
-                    else
-                        hipLaunchKernelGGL((finish_wave_kernel<TT, T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
-                }
-            } else if (s->method == TODE_TSIT5) {
-                if (pid)
-                    hipLaunchKernelGGL((finish_kernel<TT, T, 1, 1>), dim3(blocks), dim3(256), 0, st, p);
-                else
-                    hipLaunchKernelGGL((finish_kernel<TT, T, 1, 0>), dim3(blocks), dim3(256), 0, st, p);
+                if (tsit5) TODE_FINISH_CTRL(finish_wave_kernel, 1);
+                else TODE_FINISH_CTRL(finish_wave_kernel, 0);
             } else {
-                if (pid)
-                    hipLaunchKernelGGL((finish_kernel<TT, T, 0, 1>), dim3(blocks), dim3(256), 0, st, p);
-                else
-                    hipLaunchKernelGGL((finish_kernel<TT, T, 0, 0>), dim3(blocks), dim3(256), 0, st, p);
+                if (tsit5) TODE_FINISH_CTRL(finish_kernel, 1);
+                else TODE_FINISH_CTRL(finish_kernel, 0);
             }
         });
     }
     hipLaunchKernelGGL(loop_control_kernel, dim3(1), dim3(64), 0, st, s->flags, s->host_flags);
     return check_hip(hipGetLastError(), "tode_step_finish");
 }
+#undef TODE_FINISH_CTRL
+#undef TODE_FINISH
 
 int tode_step_stats(const tode_step_state *s, int64_t *n_steps, int64_t *n_accepted, int64_t *n_initialized, int64_t *status, void *stream) {
     using namespace tode;

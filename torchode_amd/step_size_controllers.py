@@ -53,6 +53,12 @@ class FixedStepState(NamedTuple):
 class FixedStepController(StepSizeController):
     """Accepts every step and keeps the step size (reference step_size_controllers.py:116-167)."""
 
+    fusable = True  # the per-step kernels know this controller (it has no whole-solve kernel)
+
+    def c_struct(self, limits=None) -> "_lib.Controller":
+        """``struct tode_controller`` of kind TODE_CTRL_FIXED; no other field is looked at."""
+        return _lib.Controller(_lib.CTRL_FIXED, False, False, 0, 0.0, 0.0, 0.0, 1.0, 0.0, 0.9, 0.2, 10.0, 0.0, 0.0)
+
     def init(self, term, problem, method_order, dt0, *, stats, args):
         assert dt0 is not None, "Fixed step size solving requires you to configure dt0"
         accept_all = torch.ones(problem.batch_size, device=problem.device, dtype=torch.bool)
