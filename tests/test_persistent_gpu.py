@@ -99,6 +99,18 @@ def test_no_t_eval_reports_end_point():
     assert (sol.stats["n_initialized"] == 1).all()
 
 
+def test_no_t_eval_where_the_two_wavefront_kernel_does_not_apply():
+    """Four features in float64 need more LDS for the hand-over records than the two-wavefront kernel
+    takes: the solve without evaluation points goes to the general kernel, silently."""
+    from torchode_amd import _lib
+
+    w = to.workloads.make("linear_decay", batch=200, dtype=F64)
+    ts, te = w.t_eval[:, 0].contiguous(), w.t_eval[:, -1].contiguous()
+    sol = gpu_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te)
+    assert _lib.last_solve_kernel_name() == "tode::solve_kernel"
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, None, w.method, w.controller, t_start=ts, t_end=te))
+
+
 @pytest.mark.parametrize("name,batch,dtype", [("vdp", 4096, F32), ("lorenz", 1000, F64), ("linear_decay", 70, F32), ("vdp", 1, F64)])
 def test_no_t_eval_through_the_fast_and_the_general_kernel(name, batch, dtype):
     """reference adjoints.py:296-311: the interpolant of the batch's LAST iteration at t_end -- the dense
