@@ -283,12 +283,63 @@ def test_gradients_with_fixed_steps(method):
 
 
 @gpu
+@pytest.mark.parametrize("method,controller", [
+    (to.Dopri5, lambda: to.IntegralController(1e-10, 1e-10)),
+    (to.Tsit5, lambda: to.PIDController(1e-10, 1e-10, 0.2, 0.5, 0.1)),
+])  # fmt: skip
+def test_gradients_with_respect_to_the_times_match_the_closed_form(method, controller):
+    """The reference's loop is torch operations on t_start, t_end and t_eval too.  y(t_eval) = y0 expm(A (t_eval -
+    t_start)): the derivative with respect to an evaluation time is f there, with respect to t_start its negative sum,
+    and t_end only decides where the last step stops."""
+    y0, A = inputs()
+    t_start = torch.tensor([0.0, 2.0], dtype=torch.double, device="cuda", requires_grad=True)
+    t_end = torch.tensor([3.0, 6.0], dtype=torch.double, device="cuda", requires_grad=True)
+    t_eval = torch.tensor([[0.4, 1.77, 2.9], [2.5, 3.5, 5.2]], dtype=torch.double, device="cuda", requires_grad=True)
+    solution = to.AutoDiffAdjoint(method(), controller()).solve(to.InitialValueProblem(y0, t_start, t_end, t_eval), term=to.ODETerm(LinearDynamics(A)))
+    weights = torch.linspace(0.5, 1.5, solution.ys.numel(), dtype=torch.double, device="cuda").reshape(solution.ys.shape)
+    (solution.ys * weights).sum().backward()
+    ref = [x.detach().clone().requires_grad_() for x in (y0, A, t_start, t_eval)]
+    dts = ref[3] - ref[2][:, None]
+    (torch.einsum("bf,befg->beg", ref[0], torch.matrix_exp(ref[1][None, None] * dts[:, :, None, None])) * weights).sum().backward()
+    for got, want in zip((y0, A, t_start, t_eval), ref):
+        torch.testing.assert_close(got.grad, want.grad, rtol=1e-7, atol=1e-8)
+    assert t_end.grad is not None and t_end.grad.abs().max().item() < 1e-7  # the solution at earlier times does not depend on it
+    assert t_eval.grad.abs().min().item() > 1e-3
+
+
+@gpu
+def test_gradcheck_with_respect_to_the_times_and_the_first_step():
+    """Every time input at once, the evaluation times as one tensor from which t_start and t_end are cut (the usual
+    construction: the sweep must not count the shared tensor twice), and a user's first step."""
+    y0, A = inputs()
+    term = to.ODETerm(LinearDynamics(A))
+
+    def through_t_eval(t_eval, dt0):
+        adjoint = to.AutoDiffAdjoint(to.Dopri5(), to.PIDController(1e-6, 0.0, 0.3, 0.6, 0.0))
+        return adjoint.solve(to.InitialValueProblem(y0.detach(), t_eval=t_eval), term=term, dt0=dt0).ys[:, 1:].mean()
+
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
+    dt0 = torch.tensor([0.05, 0.08], dtype=torch.double, device="cuda", requires_grad=True)
+    assert torch.autograd.gradcheck(through_t_eval, (t_eval, dt0), atol=1e-5)
+
+    def without_t_eval(t_start, t_end):
+        adjoint = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-7, 1e-7))
+        return adjoint.solve(to.InitialValueProblem(y0.detach(), t_start, t_end), term=term).ys.mean()
+
+    t_start = torch.tensor([0.0, 2.0], dtype=torch.double, device="cuda", requires_grad=True)
+    t_end = torch.tensor([3.0, 1.0], dtype=torch.double, device="cuda", requires_grad=True)  # the second sample backwards
+    assert torch.autograd.gradcheck(without_t_eval, (t_start, t_end), atol=1e-5)
+    # the end state moves with t_end by f(t_end, y(t_end)), and against t_start by the transported f(t_start, y0)
+    ys = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-10, 1e-10)).solve(to.InitialValueProblem(y0.detach(), t_start, t_end), term=term).ys
+    (g_end,) = torch.autograd.grad(ys.sum(), t_end)
+    torch.testing.assert_close(g_end, (ys[:, 0].detach() @ A.detach()).sum(dim=1), rtol=1e-6, atol=1e-8)
+
+
+@gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))
     t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
-    with pytest.raises(RuntimeError, match="times"):
-        to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
     with pytest.raises(RuntimeError, match="BacksolveAdjoint"):
         to.AutoDiffAdjoint(to.Heun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
     with torch.no_grad():  # no graph asked for: any configuration solves

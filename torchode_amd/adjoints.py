@@ -90,14 +90,13 @@ class AutoDiffAdjoint(nn.Module):
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
         grad_on = torch.is_grad_enabled()
-        if grad_on and (
-            problem.t_start.requires_grad
+        wants_grad = grad_on and (
+            problem.y0.requires_grad
+            or problem.t_start.requires_grad
             or problem.t_end.requires_grad
             or (problem.t_eval is not None and problem.t_eval.requires_grad)
             or (dt0 is not None and dt0.requires_grad)
-        ):
-            raise RuntimeError("torchode_amd differentiates a solve with respect to y0, the term's parameters and tensors in args; times must not require grad")
-        wants_grad = grad_on and problem.y0.requires_grad
+        )
         if not wants_grad and self._persistent_ok(problem, term_):
             sol = self._solve_persistent(problem, term_, dt0)
             if sol is not None:

@@ -11,9 +11,11 @@ the next state and of the evaluation points back through it, which evaluates ``f
 vector-Jacobian products six times per iteration.  Memory: one state copy per iteration instead of
 the reference's whole operation graph.
 
-Gradients flow to ``y0``, to the parameters of the term and to the tensors inside ``args`` (a
-tensor, or tuples / lists / dicts of them); times (``t_start``, ``t_end``, ``t_eval``) are
-treated as constants.
+Gradients flow to ``y0``, to the parameters of the term, to the tensors inside ``args`` (a
+tensor, or tuples / lists / dicts of them) and to the times (``t_start``, ``t_end``, ``t_eval``,
+a user's ``dt0``): the start of the loop, the clamp of every step to the time range and the
+position of an evaluation point inside its step are functions of them, as in the reference,
+while which step passes which point is a recorded decision.
 """
 from math import sqrt
 from typing import Any, List, Optional, Sequence
@@ -33,6 +35,19 @@ def tensor_leaves(obj) -> List[torch.Tensor]:
     if isinstance(obj, dict):
         return [t for item in obj.values() for t in tensor_leaves(item)]
     return []
+
+
+def map_tensors(obj, fn):
+    """``obj`` with ``fn`` applied to the tensors that ``tensor_leaves`` finds; containers are rebuilt."""
+    if isinstance(obj, torch.Tensor):
+        return fn(obj)
+    if isinstance(obj, tuple):
+        return tuple(map_tensors(item, fn) for item in obj)
+    if isinstance(obj, list):
+        return [map_tensors(item, fn) for item in obj]
+    if isinstance(obj, dict):
+        return {key: map_tensors(item, fn) for key, item in obj.items()}
+    return obj
 
 
 class LoopRecord:
@@ -80,8 +95,17 @@ class Replay:
         self.term, self.args = term, args
         self.through_control = through_control
         self.t_start, self.t_end, self.t_eval = problem.t_start, problem.t_end, problem.t_eval
-        self.t_lo, self.t_hi = torch.minimum(self.t_start, self.t_end), torch.maximum(self.t_start, self.t_end)
         self.direction = torch.where(self.t_end > self.t_start, 1.0, -1.0).to(self.t_start.dtype)
+
+    # the ends of the time range are functions of t_start and t_end: formed where they are used, so that every
+    # iteration of the reverse sweep differentiates a graph of its own
+    @property
+    def t_lo(self):
+        return torch.minimum(self.t_start, self.t_end)
+
+    @property
+    def t_hi(self):
+        return torch.maximum(self.t_start, self.t_end)
 
     def f(self, t, y):
         return self.term.f(t, y, self.args) if self.term.with_args else self.term.f(t, y)
@@ -215,6 +239,8 @@ class SolveThroughLoop(torch.autograd.Function):
         with torch.no_grad():
             solution = adjoint._solve_stepwise(plain, term, detached(dt0), args, record=record)
         ctx.adjoint, ctx.problem, ctx.term, ctx.dt0, ctx.args = adjoint, plain, term, dt0, args
+        # the times as the caller gave them: those that require grad are among `params`
+        ctx.times = InitialValueProblem(plain.y0, problem.t_start, problem.t_end, problem.t_eval)
         ctx.record, ctx.params = record, params
         stats = solution.stats
         n_f_evals = stats["n_f_evals"] if "n_f_evals" in stats else torch.empty(0, dtype=torch.long)
@@ -225,7 +251,23 @@ class SolveThroughLoop(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_ys, *unused):
         adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
-        replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, ctx.args, problem, adjoint.backprop_through_step_size_control, ctx.dt0)
+        # The sweep works on leaves of its own for the times and the tensors in args: one of them may be computed
+        # from another (t_start is usually a column of t_eval), and a gradient taken with respect to both would
+        # reach the first one twice, once here and once when autograd carries the second one's gradient on.
+        stand_in = {}
+
+        def leaf(x):
+            if x is None or not x.requires_grad or isinstance(x, torch.nn.Parameter):
+                return x
+            if id(x) not in stand_in:
+                stand_in[id(x)] = x.detach().requires_grad_()
+            return stand_in[id(x)]
+
+        times = InitialValueProblem(problem.y0, leaf(ctx.times.t_start), leaf(ctx.times.t_end), leaf(ctx.times.t_eval))
+        dt0 = leaf(ctx.dt0)
+        args = map_tensors(ctx.args, leaf)
+        params = [stand_in.get(id(p), p) for p in params]
+        replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, args, times, adjoint.backprop_through_step_size_control, dt0)
         states = ctx.record.trimmed(ctx.record.iterations)
         E = problem.n_evaluation_points
         hits = simulate_hits(replay, states, E)
@@ -270,18 +312,21 @@ class SolveThroughLoop(torch.autograd.Function):
             if adj["y"] is not None:
                 targets.append(y_in * 1.0)
                 cotangents.append(adj["y"])
+            if adj["t"] is not None and replay.t_start.requires_grad:
+                targets.append(replay.t_start * 1.0)
+                cotangents.append(adj["t"])
             need_f0 = adj["k0"] is not None or (adj["dt"] is not None and ctx.dt0 is None and replay.through_control)
             if need_f0:
-                f0 = replay.f(problem.t_start, y_in)
+                f0 = replay.f(replay.t_start, y_in)
                 if adj["k0"] is not None:
                     targets.append(f0)
                     cotangents.append(adj["k0"])
-                if adj["dt"] is not None and ctx.dt0 is None and replay.through_control:
-                    dt_first = replay.first_step(y_in, f0)
-                    dt_first = torch.minimum(torch.maximum(dt_first, replay.t_lo - problem.t_start), replay.t_hi - problem.t_start)
-                    if dt_first.requires_grad:
-                        targets.append(dt_first)
-                        cotangents.append(adj["dt"])
+            if adj["dt"] is not None and replay.through_control:
+                dt_first = replay.first_step(y_in, f0) if dt0 is None else dt0.to(replay.t_start.dtype)
+                dt_first = torch.minimum(torch.maximum(dt_first, replay.t_lo - replay.t_start), replay.t_hi - replay.t_start)
+                if dt_first.requires_grad:
+                    targets.append(dt_first)
+                    cotangents.append(adj["dt"])
             grad_y0 = None
             if targets:
                 grads = torch.autograd.grad(targets, [y_in] + params, cotangents, allow_unused=True)
@@ -300,7 +345,9 @@ def solve(adjoint, problem: InitialValueProblem, term, dt0: Optional[torch.Tenso
     from .solution import Solution
 
     params = [p for p in term.parameters() if p.requires_grad]
-    params += [a for a in tensor_leaves(args) if a.requires_grad and not any(a is p for p in params)]
+    for extra in tensor_leaves(args) + [problem.t_start, problem.t_end, problem.t_eval, dt0]:
+        if extra is not None and extra.requires_grad and not any(extra is p for p in params):
+            params.append(extra)
     ys, status, n_steps, n_accepted, n_initialized, n_f_evals = SolveThroughLoop.apply(adjoint, problem, term, dt0, args, problem.y0, *params)
     stats = {"n_f_evals": n_f_evals} if term.with_stats else {}
     stats.update(n_steps=n_steps, n_accepted=n_accepted, n_initialized=n_initialized)
