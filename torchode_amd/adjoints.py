@@ -47,9 +47,10 @@ class AutoDiffAdjoint(nn.Module):
     """Solves a batch of initial value problems with per-sample adaptive steps.
 
     Same constructor and ``solve`` signature as the reference.  The solve runs in HIP kernels.
-    With a ``y0`` or term parameters that require grad it takes the per-step kernels and records
-    the loop state per iteration, and the result is differentiable (``torchode_amd/autodiff.py``;
-    ``backprop_through_step_size_control`` as in the reference).
+    When ``y0``, a parameter of the term, a tensor in ``args`` or one of the times requires grad it
+    takes the per-step kernels and records the loop state per iteration, and the result is
+    differentiable (``torchode_amd/autodiff.py``; ``backprop_through_step_size_control`` as in the
+    reference).
     """
 
     def __init__(
