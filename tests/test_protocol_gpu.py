@@ -814,3 +814,14 @@ def test_term_passed_to_solve_equals_term_fixed_at_construction(method):
     sol_f = torch.compile(fixed).solve(problem, dt0=dt0)
     assert torch.equal(sol.ts, sol_f.ts) and torch.equal(sol.ys, sol_f.ys)
     assert torch.equal(sol.stats["n_steps"], sol_f.stats["n_steps"])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_configurations_match_oracle_bit_for_bit(seed):
+    """The seeded random configurations of the whole-solve suite through the operator path."""
+    from test_persistent_gpu import _random_case
+
+    f, y0, t_eval, t_start, t_end, method, controller = _random_case(3000 + seed)
+    ref = c_oracle_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000)
+    assert (ref["status"] == 0).all() and 2 <= int(ref["n_steps"].max()) < 4000
+    assert_identical(protocol_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000), ref)

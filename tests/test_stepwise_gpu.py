@@ -303,3 +303,16 @@ def test_fixed_steps_in_the_per_step_kernels_equal_the_operator_path(case, time_
     assert a.isfinite().float().mean().item() > 0.5  # (some of the stiffer samples blow up at these step sizes, in both paths alike)
     with pytest.raises(AssertionError, match="dt0"):
         to.AutoDiffAdjoint(fused_method(), to.FixedStepController()).solve(problem, to.ODETerm(f))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations_match_oracle_bit_for_bit(seed):
+    """The seeded random configurations of the whole-solve suite (term, shapes, time spans, evaluation points,
+    tolerances, controller coefficients) through the per-step kernels."""
+    from test_persistent_gpu import _random_case
+
+    f, y0, t_eval, t_start, t_end, method, controller = _random_case(2000 + seed)
+    ref = c_oracle_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000)
+    assert (ref["status"] == 0).all() and 2 <= int(ref["n_steps"].max()) < 4000
+    sol = stepwise_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000)
+    assert_identical(sol, ref)
