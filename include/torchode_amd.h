@@ -215,9 +215,11 @@ int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *
  * flag block and the device-to-host copy.  ys and the four stat arrays are
  * complete in stream order as before (here: when the call returns).  Safe to
  * call from several host threads and on several streams at once.  With
- * n_eval == 0 this call also enqueues tode_select_end_point; where
- * tode_solve_builtin_fast would refuse such a batch for its size, this call
- * launches nothing and reports flags_out[TODE_FLAG_NEEDS_GENERAL] = 1.
+ * n_eval == 0 this call also enqueues tode_select_end_point.  Where
+ * tode_solve_builtin_fast would refuse a small system for its shape (n_eval
+ * == 0 or n_eval too large, in a batch that the two-wavefront kernel does not
+ * take), this call launches no kernel and reports
+ * flags_out[TODE_FLAG_NEEDS_GENERAL] = 1.
  */
 int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                                  int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream,

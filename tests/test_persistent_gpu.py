@@ -179,6 +179,24 @@ def test_plain_fast_entry_point_without_evaluation_points_and_the_select_call():
     assert b"up to" in lib.tode_last_error()
 
 
+@pytest.mark.parametrize("dtype,n_eval", [(F32, 300), (F64, 200)], ids=["f32", "f64"])
+def test_more_evaluation_points_than_fit_on_chip(dtype, n_eval):
+    """The two-wavefront kernel reads t_eval from memory when it does not fit into LDS; the one-wavefront kernel
+    does not take such a problem, and the call hands it to the general kernel."""
+    from torchode_amd import _lib
+
+    w = to.workloads.make("vdp", batch=300, dtype=dtype)
+    t0, t1 = w.t_eval[:, :1].double(), w.t_eval[:, -1:].double()
+    t_eval = (t0 + (t1 - t0) * torch.linspace(0, 1, n_eval, dtype=torch.float64)[None, :]).to(dtype)
+    t_eval[:, -1] = w.t_eval[:, -1]
+    ref = c_oracle_solve(w.f, w.y0, t_eval, w.method, w.controller)
+    assert (ref["n_initialized"] == n_eval).all()
+    assert_identical(gpu_solve(w.f, w.y0, t_eval, w.method, w.controller), ref)
+    assert _lib.last_solve_kernel_name() == "tode::solve_pair_kernel"
+    assert_identical(gpu_solve(w.f, w.y0, t_eval, w.method, w.controller, fast="one"), ref)
+    assert _lib.last_solve_kernel_name() == "tode::solve_kernel"
+
+
 def test_user_dt0_skips_start_step():
     w = to.workloads.make("lorenz", batch=256, dtype=F32)
     dt0 = torch.full((256,), 0.01, dtype=F32)

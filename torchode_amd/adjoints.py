@@ -473,8 +473,8 @@ class AutoDiffAdjoint(nn.Module):
         has_general = f.builtin_kind in _lib.GENERAL_TERMS
         fast_ok = not ctrl.has_dt_min and not ctrl.has_dt_max
         if has_general:
-            # (without evaluation points: the end point alone, built for batches that leave SIMDs to spare)
-            fast_ok = fast_ok and self.use_fast_path and E * y0.element_size() <= 1024 and (E > 0 or 0 < B <= _lib.END_ONLY_MAX_BATCH)
+            # (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
+            fast_ok = fast_ok and self.use_fast_path and (0 < E * y0.element_size() <= 1024 or 0 < B <= _lib.END_ONLY_MAX_BATCH)
         else:
             fast_ok = fast_ok and E > 0 and dtype == torch.float32
             if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
