@@ -1,5 +1,5 @@
-"""One-call interface (mirrors torchode/interface.py)."""
-from typing import Any, Callable, Optional, Tuple, Union
+"""One call from a right-hand side to a solution (reference torchode/interface.py:17-97)."""
+from typing import Any, Callable, Dict, Optional, Tuple, Union
 
 import torch
 
@@ -10,12 +10,18 @@ from .solution import Solution
 from .step_size_controllers import PIDController, StepSizeController
 from .terms import ODETerm
 
-METHODS = {}
+METHODS: Dict[str, Callable[..., SingleStepMethod]] = {}
+DEFAULT_TOLERANCES = dict(atol=1e-7, rtol=1e-7, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)  # interface.py:79-81
 
 
 def register_method(name: str, constructor: Callable[[ODETerm], SingleStepMethod]):
     """Make ``solve_ivp(..., method=name)`` construct the step method with ``constructor(term=term)``."""
     METHODS[name] = constructor
+
+
+def _per_sample(t: torch.Tensor, batch_size: int) -> torch.Tensor:
+    """A scalar time shared by the batch, as ``[B]``."""
+    return t.expand(batch_size) if t.ndim == 0 else t
 
 
 def solve_ivp(
@@ -36,26 +42,14 @@ def solve_ivp(
     ``t_eval`` is ``[B, E]`` or ``[E]`` (shared by the batch); ``t_span`` defaults to the first and
     last evaluation time; ``method`` is a registered name or a step method object; the default
     controller is ``PIDController(atol=1e-7, rtol=1e-7, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)``."""
-    if isinstance(f, ODETerm):
-        term = f
-    else:
-        term = ODETerm(f, with_args=True) if args is not None else ODETerm(f)
-    if not isinstance(method, SingleStepMethod):
-        method = METHODS[method](term=term)
-    if controller is None:
-        controller = PIDController(term=term, atol=1e-7, rtol=1e-7, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)
-    adjoint = AutoDiffAdjoint(method, controller, max_steps=max_steps)
+    term = f if isinstance(f, ODETerm) else ODETerm(f, with_args=args is not None)
+    step_method = method if isinstance(method, SingleStepMethod) else METHODS[method](term=term)
+    step_size_controller = controller if controller is not None else PIDController(term=term, **DEFAULT_TOLERANCES)
 
     batch_size = y0.shape[0]
     if t_eval is not None and t_eval.ndim == 1:
         t_eval = t_eval.expand((batch_size, -1))
-    if t_span is not None:
-        t_start, t_end = t_span
-    else:
-        t_start, t_end = t_eval[:, 0], t_eval[:, -1]
-    if t_start.ndim == 0:
-        t_start = t_start.expand(batch_size)
-    if t_end.ndim == 0:
-        t_end = t_end.expand(batch_size)
-    problem = InitialValueProblem(y0, t_start, t_end, t_eval)
-    return adjoint.solve(problem, term, dt0=dt0, args=args)
+    t_start, t_end = t_span if t_span is not None else (t_eval[:, 0], t_eval[:, -1])
+    problem = InitialValueProblem(y0, _per_sample(t_start, batch_size), _per_sample(t_end, batch_size), t_eval)
+    solver = AutoDiffAdjoint(step_method, step_size_controller, max_steps=max_steps)
+    return solver.solve(problem, term, dt0=dt0, args=args)

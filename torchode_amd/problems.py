@@ -1,11 +1,13 @@
-"""Batch of initial value problems (mirrors torchode/problems.py:6-90)."""
+"""A batch of initial value problems: the container the solvers take (reference torchode/problems.py:6-90)."""
 from typing import Optional
 
 import torch
 
 
-def _same(attr, *tensors):
-    return all(getattr(a, attr) == getattr(b, attr) for a, b in zip(tensors[:-1], tensors[1:]))
+def _agree(what: str, first: torch.Tensor, *others: torch.Tensor) -> bool:
+    """All tensors have the same ``dtype`` / ``device`` / batch size as the first."""
+    read = (lambda x: x.shape[0]) if what == "batch" else (lambda x: getattr(x, what))
+    return all(read(other) == read(first) for other in others)
 
 
 class InitialValueProblem:
@@ -20,62 +22,28 @@ class InitialValueProblem:
     errors, as in the reference (problems.py:44-56).
     """
 
-    def __init__(
-        self,
-        y0: torch.Tensor,
-        t_start: Optional[torch.Tensor] = None,
-        t_end: Optional[torch.Tensor] = None,
-        t_eval: Optional[torch.Tensor] = None,
-    ):
-        self.y0 = y0
-        self.t_eval = t_eval
-        if t_start is None:
-            assert t_eval is not None
-            t_start = t_eval[:, 0]
-        if t_end is None:
-            assert t_eval is not None
-            t_end = t_eval[:, -1]
-        self.t_start = t_start
-        self.t_end = t_end
+    def __init__(self, y0: torch.Tensor, t_start: Optional[torch.Tensor] = None, t_end: Optional[torch.Tensor] = None,
+                 t_eval: Optional[torch.Tensor] = None):  # fmt: skip
+        assert t_eval is not None or (t_start is not None and t_end is not None)  # the range comes from t_eval otherwise
+        self.y0, self.t_eval = y0, t_eval
+        self.t_start = t_eval[:, 0] if t_start is None else t_start
+        self.t_end = t_eval[:, -1] if t_end is None else t_end
         self.time_direction = torch.where(self.t_end > self.t_start, 1, -1)
 
-        assert y0.ndim == 2
-        assert self.t_start.ndim == 1 and self.t_end.ndim == 1
-        assert _same("dtype", self.t_start, self.t_end)
-        assert y0.shape[0] == self.t_start.shape[0] == self.t_end.shape[0]
-        assert _same("device", y0, self.t_start, self.t_end)
-        if t_eval is not None:
-            assert t_eval.ndim == 2
-            assert _same("dtype", self.t_start, t_eval)
-            assert self.t_start.shape[0] == t_eval.shape[0]
-            assert _same("device", self.t_start, t_eval)
+        times = (self.t_start, self.t_end) if t_eval is None else (self.t_start, self.t_end, t_eval)
+        assert y0.ndim == 2 and self.t_start.ndim == 1 and self.t_end.ndim == 1 and (t_eval is None or t_eval.ndim == 2)
+        assert _agree("dtype", *times)
+        assert _agree("batch", y0, *times)
+        assert _agree("device", y0, *times)
 
-    @property
-    def data_dtype(self):
-        return self.y0.dtype
-
-    @property
-    def time_dtype(self):
-        return self.t_start.dtype
-
-    @property
-    def device(self):
-        return self.y0.device
-
-    @property
-    def batch_size(self):
-        return self.y0.shape[0]
-
-    @property
-    def n_features(self):
-        return self.y0.shape[1]
-
-    @property
-    def n_evaluation_points(self):
-        return 0 if self.t_eval is None else self.t_eval.shape[1]
+    # what the solvers ask of a problem
+    data_dtype = property(lambda self: self.y0.dtype)
+    time_dtype = property(lambda self: self.t_start.dtype)
+    device = property(lambda self: self.y0.device)
+    batch_size = property(lambda self: self.y0.shape[0])
+    n_features = property(lambda self: self.y0.shape[1])
+    n_evaluation_points = property(lambda self: 0 if self.t_eval is None else self.t_eval.shape[1])
 
     def __repr__(self):
-        return (
-            f"InitialValueProblem(y0={self.y0}, t_start={self.t_start}, "
-            f"t_end={self.t_end}, t_eval={self.t_eval})"
-        )
+        fields = ", ".join(f"{name}={getattr(self, name)}" for name in ("y0", "t_start", "t_end", "t_eval"))
+        return f"InitialValueProblem({fields})"

@@ -1,7 +1,8 @@
-"""Single step methods (mirror torchode/single_step_methods/__init__.py)."""
+"""Single step methods: the protocol, the explicit Runge-Kutta machinery and the reference's four methods."""
 from .base import SingleStepMethod, StepResult
-from .dopri5 import Dopri5
-from .euler import Euler
-from .heun import Heun
 from .runge_kutta import ButcherTableau, ERKInterpolationData, ERKState, ExplicitRungeKutta
+from .dopri5 import Dopri5
 from .tsit5 import Tsit5
+from .low_order import Euler, Heun
+
+__all__ = ["SingleStepMethod", "StepResult", "ButcherTableau", "ERKInterpolationData", "ERKState", "ExplicitRungeKutta", "Dopri5", "Tsit5", "Euler", "Heun"]

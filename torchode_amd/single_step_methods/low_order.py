@@ -1,12 +1,14 @@
-"""Forward Euler (mirrors torchode/single_step_methods/euler.py)."""
+"""The two low-order methods of the reference: forward Euler (torchode/single_step_methods/euler.py)
+and Heun's method 2(1) (torchode/single_step_methods/heun.py).  Both run through the operator path."""
 from typing import Any, Dict, NamedTuple, Optional
 
 import torch
 
 from .. import _lib
-from ..interpolation import LinearInterpolation
+from ..interpolation import LinearInterpolation, ThirdOrderPolynomialInterpolation
 from ..terms import ODETerm
 from .base import SingleStepMethod, StepResult
+from .runge_kutta import ButcherTableau, ERKInterpolationData, ExplicitRungeKutta
 
 
 class LinearInterpolationData(NamedTuple):
@@ -51,3 +53,26 @@ class Euler(SingleStepMethod):
 
     def build_interpolation(self, data: LinearInterpolationData):
         return LinearInterpolation(data.t0, data.dt, data.y0, data.y1)
+
+
+# Heun 2(1): the trapezoidal rule as the result, the Euler step as the embedded low-order solution.
+_HEUN_NODES = [0.0, 1.0]
+_HEUN_STAGES = [[], [1.0]]
+_HEUN_WEIGHTS, _HEUN_EULER_WEIGHTS = [0.5, 0.5], [1.0, 0.0]
+
+
+class Heun(ExplicitRungeKutta):
+    """Two stages, error estimate against the Euler step, Hermite cubic dense output (stage and sum
+    kernels with this tableau)."""
+
+    TABLEAU = ButcherTableau.from_lists(c=_HEUN_NODES, a=_HEUN_STAGES, b=_HEUN_WEIGHTS, b_low_order=_HEUN_EULER_WEIGHTS)
+
+    def __init__(self, term: Optional[ODETerm] = None):
+        super().__init__(term, type(self).TABLEAU)
+
+    def convergence_order(self) -> int:
+        return 2
+
+    def build_interpolation(self, data: ERKInterpolationData):
+        first_and_last_slopes = data.k
+        return ThirdOrderPolynomialInterpolation.from_k(data.t0, data.dt, data.y0, data.y1, first_and_last_slopes)

@@ -1,4 +1,4 @@
-"""Result container (mirrors torchode/solution.py:6-23)."""
+"""What a solve returns (reference torchode/solution.py:6-23)."""
 from typing import Any, Dict
 
 import torch
@@ -10,11 +10,10 @@ class Solution:
     per-sample ``status`` codes.  Rows of ``ys`` at or beyond ``n_initialized`` hold
     unspecified values after an early stop."""
 
+    FIELDS = ("ts", "ys", "stats", "status")
+
     def __init__(self, ts: torch.Tensor, ys: torch.Tensor, stats: Dict[str, Any], status: torch.Tensor):
-        self.ts = ts
-        self.ys = ys
-        self.stats = stats
-        self.status = status
+        self.ts, self.ys, self.stats, self.status = ts, ys, stats, status
 
     def __repr__(self):
-        return f"Solution(ts={self.ts}, ys={self.ys}, stats={self.stats}, status={self.status})"
+        return "Solution(" + ", ".join(f"{name}={getattr(self, name)}" for name in self.FIELDS) + ")"

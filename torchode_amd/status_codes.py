@@ -7,19 +7,16 @@ sample reports one.
 """
 from enum import Enum
 
-SUCCESS = 0
-GENERAL_ERROR = 1
-REACHED_DT_MIN = 2
-REACHED_MAX_STEPS = 3
-INFINITE_NORM = 4
-
 
 class Status(Enum):
     """User-facing names for the integer status codes."""
 
-    SUCCESS = SUCCESS
-    GENERAL_ERROR = GENERAL_ERROR
-    REACHED_DT_MIN = REACHED_DT_MIN
-    REACHED_MAX_STEPS = REACHED_MAX_STEPS
-    # The error-ratio norm was not finite (NaN or inf in y or in the error estimate).
-    INFINITE_NORM = INFINITE_NORM
+    SUCCESS = 0
+    GENERAL_ERROR = 1
+    REACHED_DT_MIN = 2
+    REACHED_MAX_STEPS = 3
+    INFINITE_NORM = 4  # the error-ratio norm was not finite (NaN or inf in y or in the error estimate)
+
+
+# the plain integers, as the kernels and the status tensors carry them
+SUCCESS, GENERAL_ERROR, REACHED_DT_MIN, REACHED_MAX_STEPS, INFINITE_NORM = (code.value for code in Status)
