@@ -148,12 +148,13 @@ def solve(cfg: Config, params, y0, t_eval=None, *, t_start=None, t_end=None, dt0
     i64 = lambda: torch.zeros(B, dtype=torch.int64)
     n_steps, n_acc, n_init, status = i64(), i64(), i64(), i64()
     n_f = C.c_int64(0)
+    written = torch.ones((B, max(E, 1)), dtype=torch.uint8)  # (without evaluation points: the end point, always)
     trace = torch.zeros((trace_iters, trace_B, 4), dtype=dtype) if trace_iters else None
     fn = getattr(lib(), f"oracle_solve_{_sfx(dtype)}")
     rc = fn(
         C.byref(cfg), C.c_int64(B), C.c_int(F), C.c_int(E), _p(y0), _p(t_start), _p(t_end), _p(t_eval), _p(dt0),
         _p(params), C.c_int(params.shape[1]), _p(ys), _p(n_steps), _p(n_acc), _p(n_init), _p(status), C.byref(n_f),
-        _p(trace), C.c_int64(trace_iters), C.c_int64(trace_B),
+        _p(trace), C.c_int64(trace_iters), C.c_int64(trace_B), _p(written),
     )  # fmt: skip
     assert rc == 0
     out = dict(
@@ -164,6 +165,7 @@ def solve(cfg: Config, params, y0, t_eval=None, *, t_start=None, t_end=None, dt0
         n_steps=n_steps,
         n_accepted=n_acc,
         n_initialized=n_init,
+        written=written.bool(),  # which rows of ys the loop stored (n_initialized is the reference's searchsorted over these marks)
     )
     if trace is not None:
         out["trace"] = trace

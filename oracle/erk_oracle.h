@@ -56,7 +56,8 @@ const oracle_tableau *oracle_get_tableau(int method);
     int oracle_solve_##SFX(const oracle_config *, int64_t B, int F, int E, const REAL *y0, const REAL *t_start,         \
                            const REAL *t_end, const REAL *t_eval, const REAL *dt0, const REAL *params, int P, REAL *ys, \
                            int64_t *n_steps, int64_t *n_accepted, int64_t *n_initialized, int64_t *status,              \
-                           int64_t *n_f_evals, REAL *trace, int64_t trace_iters, int64_t trace_B);
+                           int64_t *n_f_evals, REAL *trace, int64_t trace_iters, int64_t trace_B,                      \
+                           unsigned char *written /* [B,E] or NULL: 1 where the loop stored an evaluation point */);
 
 ORACLE_DECLARE(float, f32)
 ORACLE_DECLARE(double, f64)

@@ -297,7 +297,7 @@ typedef struct {
 int SFX(oracle_solve)(const oracle_config *cfg, int64_t B, int F, int E, const REAL *y0_in, const REAL *t_start,
                       const REAL *t_end, const REAL *t_eval, const REAL *dt0, const REAL *params, int P, REAL *ys,
                       int64_t *n_steps, int64_t *n_accepted, int64_t *n_initialized, int64_t *status_out,
-                      int64_t *n_f_evals, REAL *trace, int64_t trace_iters, int64_t trace_B) {
+                      int64_t *n_f_evals, REAL *trace, int64_t trace_iters, int64_t trace_B, unsigned char *written) {
     const oracle_tableau *tab = oracle_get_tableau(cfg->method);
     if (!tab) return -1;
     int nthreads = cfg->nthreads > 0 ? cfg->nthreads : 1;
@@ -452,9 +452,15 @@ int SFX(oracle_solve)(const oracle_config *cfg, int64_t B, int F, int E, const R
     for (int64_t b = 0; b < B; ++b) {
         status_out[b] = st[b].status;
         if (t_eval) {
-            int64_t e = 0;
-            while (e < E && !pending[b * E + e]) ++e;
-            n_initialized[b] = e;
+            /* adjoints.py:289-292: torch.searchsorted(not_yet_evaluated.int(), 1), i.e. ATen's lower-bound binary
+               search -- the index of the first pending point when the row of marks is sorted (evaluation times
+               monotone in the sample's direction), and whatever the search lands on when it is not */
+            int64_t lo = 0, hi = E;
+            while (lo < hi) {
+                const int64_t mid = lo + ((hi - lo) >> 1);
+                if (!pending[b * E + mid]) lo = mid + 1; else hi = mid;
+            }
+            n_initialized[b] = lo;
         } else {
             n_initialized[b] = 1;
         }
@@ -463,6 +469,8 @@ int SFX(oracle_solve)(const oracle_config *cfg, int64_t B, int F, int E, const R
     free(st);
     free(y);
     free(k0);
+    if (written)
+        for (int64_t i = 0; i < B * (int64_t)E; ++i) written[i] = !pending[i];
     free(pending);
     free(work);
     return 0;

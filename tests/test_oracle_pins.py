@@ -629,3 +629,29 @@ def test_headline_configuration_at_full_size():
     assert torch.equal(a["ys"], c["ys"])
     for key in ("n_steps", "n_accepted", "n_initialized", "status", "n_f_evals"):
         assert torch.equal(a[key], c[key]), key
+
+
+@needs_pinned_aten
+@pytest.mark.parametrize("seed", [1000, 1001, 1002, 1004, 1008, 1010, 1014, 1017, 1019, 1021])
+def test_oracles_agree_on_random_configurations(seed):
+    """The seeded random configurations of the GPU suites (term, shapes, per-sample time spans with evaluation
+    points outside them, tolerances, controller coefficients; linear systems partly backwards in time): scalar C loop
+    against the batched ATen-op loop, on a whole number of 32-sample vector bodies."""
+    from test_persistent_gpu import _random_case
+
+    f, y0, t_eval, t_start, t_end, method, controller = _random_case(seed)
+    n = y0.shape[0] // 32 * 32
+    assert n * y0.shape[1] >= 200, "pick seeds with batches large enough for ATen's fused matrix kernels"
+    f = type(f)(f.builtin_params()[:n].reshape(n, -1) if type(f) is to.LinearDecay else f.builtin_params()[:n, 0])
+    y0, t_eval, t_start, t_end = y0[:n], t_eval[:n], t_start[:n], t_end[:n]
+    a = tl.solve(f, y0, t_eval, method=method, controller=tl.Controller(**controller), t_start=t_start, t_end=t_end, max_steps=4000)
+    from helpers import c_oracle_solve
+
+    c = c_oracle_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000, nthreads=4)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status", "n_f_evals"):
+        assert torch.equal(a[key], c[key]), key
+    # (a point beyond t_end is never written, and where a later point of its row is, the reference's searchsorted
+    # counts it as initialised all the same: compare what was written)
+    written = c["written"]
+    assert torch.equal(a["ys"][written], c["ys"][written]) and not c["ys"][written].isnan().any()
+    assert (~written).float().mean() < 0.1 and c["ys"][~written].isnan().all()

@@ -478,9 +478,7 @@ __global__ void __launch_bounds__(256) loop_begin_kernel(long long batch, int F,
 static __global__ void __launch_bounds__(256) count_initialized_kernel(long long batch, int E, const uint8_t *pending, int64_t *out) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
-    int n = 0;
-    while (n < E && !pending[b * E + n]) ++n;
-    out[b] = n;
+    out[b] = searchsorted_first_pending(pending + b * E, E);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -222,8 +222,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
         int n_init = 1;
         if (tev) {
             if (pend) {
-                n_init = 0;
-                while (n_init < E && !pend[n_init]) ++n_init;
+                n_init = searchsorted_first_pending(pend, E);
             } else {
                 n_init = cursor;
             }

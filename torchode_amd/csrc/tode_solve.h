@@ -147,6 +147,18 @@ template <typename T> __device__ __forceinline__ T initial_finish(int kind, doub
     return dir * tmin((T)100 * h0, h1);
 }
 
+// n_initialized as the reference forms it (adjoints.py:289-292): torch.searchsorted(pending, 1), ATen's
+// lower-bound binary search.  On a sorted row of marks (evaluation times monotone in the sample's direction) this
+// is the index of the first pending point; on any other row it is whatever the search lands on, mirrored here.
+__device__ __forceinline__ int searchsorted_first_pending(const uint8_t *pending, int E) {
+    int lo = 0, hi = E;
+    while (lo < hi) {
+        const int mid = lo + ((hi - lo) >> 1);
+        if (!pending[mid]) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
 // x = (t - t0) / (t1 - t0) with a zero interval mapped to 1 (interpolation.py:8-40)
 template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) {
     T den = t1 - t0;

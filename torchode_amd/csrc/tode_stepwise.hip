@@ -570,13 +570,14 @@ static __global__ void step_flags_init_kernel(int32_t *flags, int32_t *host_flag
 
 // int32 device state -> the reference's int64 stats (adjoints.py:267-292)
 static __global__ void step_stats_kernel(long long batch, const int32_t *n_steps, const int32_t *n_accepted, const int32_t *cursor,
-                                         const int32_t *status, int n_eval, int64_t *o_steps, int64_t *o_acc, int64_t *o_init,
-                                         int64_t *o_status) {
+                                         const int32_t *status, const int32_t *monotone, const uint8_t *pending, int n_eval,
+                                         int64_t *o_steps, int64_t *o_acc, int64_t *o_init, int64_t *o_status) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
     o_steps[b] = n_steps[b];
     o_acc[b] = n_accepted[b];
-    o_init[b] = n_eval > 0 ? cursor[b] : 1;
+    // (a monotone row's marks are sorted: the search of the reference finds the cursor)
+    o_init[b] = n_eval <= 0 ? 1 : (monotone[b] ? cursor[b] : searchsorted_first_pending(pending + b * n_eval, n_eval));
     o_status[b] = status[b];
 }
 
@@ -784,11 +785,12 @@ int tode_step_stats(const tode_step_state *s, int64_t *n_steps, int64_t *n_accep
     using namespace tode;
     if (!s) return fail(TODE_E_INVALID, "null state");
     if (s->batch == 0) return TODE_OK;
-    if (!n_steps || !n_accepted || !n_initialized || !status || !s->n_steps || !s->n_accepted || !s->cursor || !s->status)
+    if (!n_steps || !n_accepted || !n_initialized || !status || !s->n_steps || !s->n_accepted || !s->cursor || !s->status || !s->monotone ||
+        (s->n_eval > 0 && !s->pending))
         return fail(TODE_E_INVALID, "null pointer");
     const unsigned blocks = (unsigned)((s->batch + 255) / 256);
     hipLaunchKernelGGL(step_stats_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (long long)s->batch, s->n_steps, s->n_accepted,
-                       s->cursor, s->status, s->n_eval, n_steps, n_accepted, n_initialized, status);
+                       s->cursor, s->status, s->monotone, s->pending, s->n_eval, n_steps, n_accepted, n_initialized, status);
     return check_hip(hipGetLastError(), "tode_step_stats");
 }
 
