@@ -106,3 +106,49 @@ def aten_host_matches() -> bool:
         ok = ok and torch.equal(torch.einsum("b, s, sbf -> bf", dt, w, k), plain)
         _ATEN_HOST = bool(ok)
     return _ATEN_HOST
+
+
+def wild_case(seed: int):
+    """A seeded configuration from the whole space the loop knows: the three small systems, float32 / float64,
+    per-sample time spans (the linear system partly backwards), evaluation points sorted, shuffled within rows, pinned
+    to the ends of the range or absent, tolerances and controller coefficients at random, dt_min / dt_max, a small
+    max_steps, a user's first step.  Batches are multiples of 32 with B * F >= 200, so that ATen's CPU kernels use
+    their vector bodies and fused matrix kernels throughout and the ATen-op oracle can be compared as well.
+    Returns (f, y0, t_eval, t_start, t_end, method, controller, max_steps, dt0)."""
+    g = torch.Generator().manual_seed(seed)
+    u = lambda lo, hi, *shape: lo + (hi - lo) * torch.rand(*shape, generator=g, dtype=torch.float64)
+    pick = lambda seq: seq[int(torch.randint(len(seq), (1,), generator=g))]
+    dtype = pick([torch.float32, torch.float64])
+    B = 32 * int(torch.randint(4, 12, (1,), generator=g))
+    E = int(torch.randint(1, 40, (1,), generator=g))
+    term = pick(["linear_decay", "vdp", "lorenz"])
+    if term == "linear_decay":
+        f, y0, span = to.LinearDecay(u(0.1, 6.0, B, 3).to(dtype)), u(-2, 2, B, 3), 3.0
+    elif term == "vdp":
+        f, y0, span = to.VanDerPol(u(0.2, pick([8.0, 60.0]), B).to(dtype)), u(-2.5, 2.5, B, 2), 6.0
+    else:
+        f, y0, span = to.Lorenz63(u(20.0, 35.0, B).to(dtype)), u(-10, 10, B, 3) + torch.tensor([0, 0, 20.0], dtype=torch.float64), 1.5
+    t_start, length = u(-1, 1, B), u(0.3, 1.0, B) * span
+    back = (torch.rand(B, generator=g) < 0.3) & (term == "linear_decay")
+    t_end = torch.where(back, t_start - length, t_start + length)
+    frac = u(-0.05, 1.05, B, E).sort(dim=1).values
+    mode = pick(["sorted", "shuffled-rows", "none", "ends"])
+    if mode == "shuffled-rows":
+        rows = torch.rand(B, generator=g) < 0.3
+        frac[rows] = frac[rows][:, torch.randperm(E, generator=g)]
+    if mode == "ends":
+        frac[:, 0], frac[:, -1] = 0.0, 1.0
+    t_eval = None if mode == "none" else (t_start[:, None] + frac * (t_end - t_start)[:, None]).to(dtype)
+    rtol = 10.0 ** float(u(-6, -2.5, 1)) if dtype == torch.float64 else 10.0 ** float(u(-5, -2.5, 1))
+    ctrl = dict(kind=pick(["integral", "pid", "pid"]), atol=rtol * 10.0 ** float(u(-3, 0, 1)), rtol=rtol)
+    if ctrl["kind"] == "pid":
+        ctrl.update(pcoeff=float(u(0, 0.4, 1)), icoeff=float(u(0.3, 1.0, 1)), dcoeff=pick([0.0, float(u(0, 0.1, 1))]))
+    limits = pick(["none", "dt_min", "dt_max", "both"])
+    if limits in ("dt_min", "both"):
+        ctrl["dt_min"] = float(u(1e-3, 5e-2, 1))
+    if limits in ("dt_max", "both"):
+        ctrl["dt_max"] = float(u(0.06, 0.4, 1))
+    max_steps = pick([None, None, 12, 40])
+    dt0 = pick([None, None, u(1e-3, 0.1, B) * torch.where(back, -1.0, 1.0)])
+    method = pick(["dopri5", "tsit5"])
+    return f, y0.to(dtype), t_eval, t_start.to(dtype), t_end.to(dtype), method, ctrl, 3000 if max_steps is None else max_steps, None if dt0 is None else dt0.to(dtype)

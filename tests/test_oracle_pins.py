@@ -655,3 +655,19 @@ def test_oracles_agree_on_random_configurations(seed):
     written = c["written"]
     assert torch.equal(a["ys"][written], c["ys"][written]) and not c["ys"][written].isnan().any()
     assert (~written).float().mean() < 0.1 and c["ys"][~written].isnan().all()
+
+
+@needs_pinned_aten
+@pytest.mark.parametrize("seed", range(24))
+def test_oracles_agree_on_wild_configurations(seed):
+    """Scalar C loop against the batched ATen-op loop over everything the loop knows at once: evaluation points
+    shuffled within rows or absent, dt_min / dt_max, a small max_steps, a user's first step (tests/helpers.py::wild_case)."""
+    from helpers import c_oracle_solve, wild_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = wild_case(seed)
+    a = tl.solve(f, y0, t_eval, method=method, controller=tl.Controller(**ctrl), t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    c = c_oracle_solve(f, y0, t_eval, method, ctrl, t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps, nthreads=4)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status", "n_f_evals"):
+        assert torch.equal(a[key], c[key]), key
+    av, cv = a["ys"][c["written"]], c["ys"][c["written"]]
+    assert bool(((av == cv) | (av.isnan() & cv.isnan())).all())

@@ -600,3 +600,16 @@ def test_random_configurations_match_oracle_bit_for_bit(seed):
     print(f"seed {seed}: {type(f).__name__} {tuple(y0.shape)} E={t_eval.shape[1]} {y0.dtype} {method} {controller}", flush=True)
     for fast in ("one", False, "two"):
         assert_identical(gpu_solve(f, y0, t_eval, method, controller, fast=fast, **kw), ref)
+
+
+@pytest.mark.parametrize("seed", range(100, 130))
+def test_wild_configurations_match_oracle_bit_for_bit(seed):
+    """tests/helpers.py::wild_case: evaluation points shuffled within rows or absent, dt_min / dt_max, a small
+    max_steps, a user's first step -- whatever kernel the dispatch picks, and the general kernel."""
+    from helpers import wild_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = wild_case(seed)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    ref = c_oracle_solve(f, y0, t_eval, method, ctrl, **kw)
+    assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, **kw), ref)
+    assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, fast=False, **kw), ref)

@@ -825,3 +825,13 @@ def test_random_configurations_match_oracle_bit_for_bit(seed):
     ref = c_oracle_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000)
     assert (ref["status"] == 0).all() and 2 <= int(ref["n_steps"].max()) < 4000
     assert_identical(protocol_solve(f, y0, t_eval, method, controller, t_start=t_start, t_end=t_end, max_steps=4000), ref)
+
+
+@pytest.mark.parametrize("seed", range(300, 312))
+def test_wild_configurations_match_oracle_bit_for_bit(seed):
+    """tests/helpers.py::wild_case through the operator path."""
+    from helpers import wild_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = wild_case(seed)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    assert_identical(protocol_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
