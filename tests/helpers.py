@@ -152,3 +152,21 @@ def wild_case(seed: int):
     dt0 = pick([None, None, u(1e-3, 0.1, B) * torch.where(back, -1.0, 1.0)])
     method = pick(["dopri5", "tsit5"])
     return f, y0.to(dtype), t_eval, t_start.to(dtype), t_end.to(dtype), method, ctrl, 3000 if max_steps is None else max_steps, None if dt0 is None else dt0.to(dtype)
+
+
+def poisoned(y0: torch.Tensor, seed: int) -> torch.Tensor:
+    """``y0`` with three samples made NaN, infinite, huge, or large enough to blow up later (by ``seed % 4``): the
+    non-success statuses and the batch-wide stop they cause."""
+    g = torch.Generator().manual_seed(seed + 7)
+    idx = torch.randperm(y0.shape[0], generator=g)[:3]
+    y0 = y0.clone()
+    kind = seed % 4
+    if kind == 0:
+        y0[idx, 0] = float("nan")
+    elif kind == 1:
+        y0[idx, -1] = float("inf")
+    elif kind == 2:
+        y0[idx] = 1e30 if y0.dtype == torch.float32 else 1e200
+    else:
+        y0[idx] = y0[idx] * 1e6
+    return y0

@@ -613,3 +613,15 @@ def test_wild_configurations_match_oracle_bit_for_bit(seed):
     ref = c_oracle_solve(f, y0, t_eval, method, ctrl, **kw)
     assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, **kw), ref)
     assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, fast=False, **kw), ref)
+
+
+@pytest.mark.parametrize("seed", range(400, 416))
+def test_wild_configurations_with_non_finite_samples(seed):
+    """wild_case with three samples NaN, infinite, huge or blowing up later (tests/helpers.py::poisoned): status 4, 2
+    and 3 in every mixture and the batch-wide stop, through whatever kernel the dispatch picks."""
+    from helpers import poisoned, wild_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = wild_case(seed)
+    y0 = poisoned(y0, seed)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=min(max_steps, 400))
+    assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
