@@ -84,6 +84,47 @@ def make(name, batch, dtype):
     }
 
 
+# Time and data in different dtypes (reference problems.py:44-56): vectors of the ATen-op oracle alone (the scalar C
+# oracle is written for one dtype); the per-step kernels and the operator path are compared with them bit for bit.
+MIXED_CASES = [
+    ("vdp", 512, torch.float64, torch.float32),
+    ("vdp", 512, torch.float32, torch.float64),
+    ("lorenz", 256, torch.float64, torch.float32),
+    ("lorenz", 256, torch.float32, torch.float64),
+]
+
+
+def mixed_inputs(name, batch, time_dtype, data_dtype):
+    """The float64 workload with its times rounded to one dtype and its state and parameters to the other."""
+    w = to.workloads.make(name, batch=batch, dtype=torch.float64)
+    params = w.f.builtin_params().to(data_dtype)
+    f = type(w.f)(params[:, 0] if params.shape[1] == 1 else params)
+    return w, f, w.y0.to(data_dtype), w.t_eval.to(time_dtype)
+
+
+def make_mixed(name, batch, time_dtype, data_dtype):
+    w, f, y0, t_eval = mixed_inputs(name, batch, time_dtype, data_dtype)
+    out = torch_loop.solve(f, y0, t_eval, method=w.method, controller=torch_loop.Controller(**w.controller))
+    assert out["ys"].dtype == data_dtype and (out["status"] == 0).all()
+    sub = list(range(0, batch, max(1, batch // 16)))[:16]
+    return {
+        "source": f"oracle/torch_loop.py (ATen CPU ops), torch {torch.__version__}, {torch.backends.cpu.get_cpu_capability()}, "
+        f"opt_einsum {torch.backends.opt_einsum.is_available()}; time and data dtypes differ",
+        "workload": name,
+        "batch": batch,
+        "time_dtype": str(time_dtype).replace("torch.", ""),
+        "data_dtype": str(data_dtype).replace("torch.", ""),
+        "method": w.method,
+        "controller": w.controller,
+        "inputs_sha256": {"y0": sha(y0), "t_eval": sha(t_eval), "params": sha(f.builtin_params())},
+        "n_f_evals": int(out["n_f_evals"][0]),
+        **{key: out[key].tolist() for key in ("n_steps", "n_accepted", "n_initialized", "status")},
+        "ys_sha256": sha(out["ys"]),
+        "subset": sub,
+        "ys_subset": hexlist(out["ys"][sub]),
+    }
+
+
 def make_tolerance(name, batch, dtype):
     w = to.workloads.make(name, batch=batch, dtype=dtype)
     out = torch_loop.solve(w.f, w.y0, w.t_eval, method=w.method, controller=torch_loop.Controller(**w.controller))
@@ -108,6 +149,12 @@ def make_tolerance(name, batch, dtype):
 
 
 if __name__ == "__main__":
+    for name, batch, time_dtype, data_dtype in MIXED_CASES:
+        d = make_mixed(name, batch, time_dtype, data_dtype)
+        path = os.path.join(HERE, f"{name}_t{d['time_dtype'][-2:]}_y{d['data_dtype'][-2:]}_b{batch}_mixed.json")
+        with open(path, "w") as fh:
+            json.dump(d, fh, separators=(",", ":"))
+        print(path, os.path.getsize(path), "bytes")
     for name, batch, dtype in TOLERANCE_CASES:
         d = make_tolerance(name, batch, dtype)
         path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_tolerance.json")

@@ -165,7 +165,7 @@ def test_tolerance_fixture_inputs_and_workload_agree(path):
     assert all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])
 
 
-@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith("_tolerance.json")], ids=os.path.basename)
+@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json"))], ids=os.path.basename)
 def test_oracle_reproduces_golden_fixture(path):
     g = json.load(open(path))
     dtype = getattr(torch, g["dtype"])
@@ -203,3 +203,16 @@ def test_torch_compile_wrapper_hands_out_the_solvers_own_solve():
         solver = cls(*args) if cls is to.AutoDiffAdjoint else cls(term, *args)
         wrapped = torch.compile(solver)
         assert wrapped.solve.__self__ is solver and wrapped.solve.__func__ is cls.solve
+
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if p.endswith("_mixed.json")], ids=os.path.basename)
+def test_mixed_dtype_fixture_is_well_formed(path):
+    """Vectors of the ATen-op oracle with time and data in different dtypes (tests/golden/make_golden.py::make_mixed);
+    the inputs they belong to are the float64 workload rounded to the two dtypes."""
+    g = json.load(open(path))
+    time_dtype, data_dtype = getattr(torch, g["time_dtype"]), getattr(torch, g["data_dtype"])
+    assert time_dtype != data_dtype
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=torch.float64)
+    got = {"y0": _sha(w.y0.to(data_dtype)), "t_eval": _sha(w.t_eval.to(time_dtype)), "params": _sha(w.f.builtin_params().to(data_dtype))}
+    assert got == g["inputs_sha256"]
+    assert len(g["n_steps"]) == g["batch"] and all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])

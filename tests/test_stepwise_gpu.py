@@ -338,3 +338,35 @@ def test_wild_configurations_with_non_finite_samples(seed):
     y0 = poisoned(y0, seed)
     kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=min(max_steps, 400))
     assert_identical(stepwise_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
+
+
+def _mixed_fixtures():
+    import glob
+    import os
+
+    return sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_mixed.json")))
+
+
+@pytest.mark.parametrize("path", _mixed_fixtures(), ids=lambda p: p.split("/")[-1])
+def test_mixed_dtypes_match_the_aten_op_oracle_fixture(path):
+    """tests/golden/*_mixed.json: the reference's loop as ATen CPU operations with time and data in different dtypes,
+    written in the authoring container.  The per-step kernels and the operator path reproduce every bit of them."""
+    import hashlib
+    import json
+
+    g = json.load(open(path))
+    time_dtype, data_dtype = getattr(torch, g["time_dtype"]), getattr(torch, g["data_dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=torch.float64)
+    params = w.f.builtin_params().to(data_dtype)
+    f = type(w.f)(params[:, 0] if params.shape[1] == 1 else params).cuda()
+    problem = to.InitialValueProblem(w.y0.to(data_dtype).cuda(), t_eval=w.t_eval.to(time_dtype).cuda())
+    fused_method, operator_method = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[g["method"]]
+    for method in (fused_method, operator_method):
+        sol = to.AutoDiffAdjoint(method(), make_controller(g["controller"])).solve(problem, to.ODETerm(lambda t, y: f(t, y)))
+        for key in ("n_steps", "n_accepted", "n_initialized"):
+            assert sol.stats[key].tolist() == g[key], (method.__name__, key)
+        assert sol.status.tolist() == g["status"] and int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
+        ys = sol.ys.cpu()
+        assert ys.dtype == data_dtype and sol.ts.dtype == time_dtype
+        assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"], method.__name__
+        assert hashlib.sha256(ys.contiguous().numpy().tobytes()).hexdigest() == g["ys_sha256"], method.__name__
