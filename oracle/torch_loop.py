@@ -231,7 +231,7 @@ class Controller(NamedTuple):
     """Constructor arguments of IntegralController / PIDController
     (step_size_controllers.py:263-287, 566-596)."""
 
-    kind: str  # "integral" | "pid"
+    kind: str  # "integral" | "pid" | "fixed" (FixedStepController, step_size_controllers.py:116-167: needs dt0, other fields unused)
     atol: float
     rtol: float
     pcoeff: float = 0.0
@@ -526,17 +526,22 @@ def solve(
         calls[0] += 1
         return f(t, y)
 
+    fixed = controller.kind == "fixed"
+    assert not fixed or dt0 is not None, "Fixed step size solving requires you to configure dt0"
     if dt0 is None:
         dt, k0 = initial_step(vf, controller, order, t_start, y0, direction_i, (t_end - t_start).abs())
     else:
         dt, k0 = dt0, vf(t_start, y0)
     ones = torch.ones(B, dtype=y0.dtype)
+    accept_all = torch.ones(B, dtype=torch.bool)
 
     def step(running, y, t, dt, k0):
         y1, err, k = erk_step(vf, tab, t, dt, y, k0)
         return y1, (t, dt, y, y1, err, k), k[-1], None
 
     def adapt_(t, dt, y, y1, data, state):
+        if fixed:  # every step accepted, the next step is dt0 again, no status (step_size_controllers.py:153-163)
+            return accept_all, dt0, (state[0], state[1], ones), None
         accept, dt_next, status, ratio, prev_n, prev_prev_n = adapt(controller, order, dt, y, y1, data[4], *state)
         return accept, dt_next, (prev_n, prev_prev_n, ratio), status
 
@@ -559,6 +564,8 @@ def solve(
         y0, t_start, t_end, t_eval, dt, step, adapt_, merge_method, merge_controller, dense, k0, (ones, ones),
         max_steps=max_steps, on_iteration=on_iteration,
     )  # fmt: skip
+    if status is None:  # adjoints.py:266-270: the user always gets a status tensor
+        status = torch.tensor(SUCCESS, dtype=torch.long).expand(B)
     stats = {
         "n_f_evals": torch.full((B,), calls[0], dtype=torch.long),
         "n_steps": n_steps,

@@ -125,6 +125,41 @@ def make_mixed(name, batch, time_dtype, data_dtype):
     }
 
 
+# Fixed steps (reference step_size_controllers.py:116-167) with Dopri5 / Tsit5: vectors of the ATen-op oracle alone.
+FIXED_CASES = [("vdp", 256, torch.float32, "tsit5"), ("lorenz", 256, torch.float64, "dopri5")]
+
+
+def fixed_inputs(name, batch, dtype):
+    """The workload with a per-sample fixed step: the span cut into 60.37 to 66.37 parts (the last step is cut short)."""
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    span = (w.t_eval[:, -1] - w.t_eval[:, 0]).double()
+    dt0 = (span / (60.37 + torch.arange(batch, dtype=torch.float64) % 7)).to(dtype)
+    return w, dt0
+
+
+def make_fixed(name, batch, dtype, method):
+    w, dt0 = fixed_inputs(name, batch, dtype)
+    out = torch_loop.solve(w.f, w.y0, w.t_eval, method=method, controller=torch_loop.Controller("fixed", 0.0, 0.0), dt0=dt0)
+    assert (out["status"] == 0).all() and torch.equal(out["n_steps"], out["n_accepted"]) and 61 <= int(out["n_steps"].min())
+    sub = list(range(0, batch, max(1, batch // 16)))[:16]
+    return {
+        "source": f"oracle/torch_loop.py (ATen CPU ops), torch {torch.__version__}, {torch.backends.cpu.get_cpu_capability()}, "
+        f"opt_einsum {torch.backends.opt_einsum.is_available()}; fixed steps",
+        "workload": name,
+        "batch": batch,
+        "dtype": str(dtype).replace("torch.", ""),
+        "method": method,
+        "inputs_sha256": {"y0": sha(w.y0), "t_eval": sha(w.t_eval), "params": sha(w.f.builtin_params()), "dt0": sha(dt0)},
+        "n_f_evals": int(out["n_f_evals"][0]),
+        **{key: out[key].tolist() for key in ("n_steps", "n_accepted", "n_initialized", "status")},
+        # (some of the stiffer Van der Pol samples blow up at these step sizes: NaN hashed as 0, its bits are not pinned)
+        "ys_sha256_nan_as_zero": sha(out["ys"].nan_to_num(nan=0.0, posinf=float("inf"), neginf=float("-inf"))),
+        "ys_finite_fraction": float(out["ys"].isfinite().double().mean()),
+        "subset": sub,
+        "ys_subset": hexlist(out["ys"][sub]),
+    }
+
+
 def make_tolerance(name, batch, dtype):
     w = to.workloads.make(name, batch=batch, dtype=dtype)
     out = torch_loop.solve(w.f, w.y0, w.t_eval, method=w.method, controller=torch_loop.Controller(**w.controller))
@@ -149,6 +184,12 @@ def make_tolerance(name, batch, dtype):
 
 
 if __name__ == "__main__":
+    for name, batch, dtype, method in FIXED_CASES:
+        d = make_fixed(name, batch, dtype, method)
+        path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_{method}_fixed.json")
+        with open(path, "w") as fh:
+            json.dump(d, fh, separators=(",", ":"))
+        print(path, os.path.getsize(path), "bytes")
     for name, batch, time_dtype, data_dtype in MIXED_CASES:
         d = make_mixed(name, batch, time_dtype, data_dtype)
         path = os.path.join(HERE, f"{name}_t{d['time_dtype'][-2:]}_y{d['data_dtype'][-2:]}_b{batch}_mixed.json")

@@ -165,7 +165,7 @@ def test_tolerance_fixture_inputs_and_workload_agree(path):
     assert all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])
 
 
-@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json"))], ids=os.path.basename)
+@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json"))], ids=os.path.basename)
 def test_oracle_reproduces_golden_fixture(path):
     g = json.load(open(path))
     dtype = getattr(torch, g["dtype"])
@@ -216,3 +216,14 @@ def test_mixed_dtype_fixture_is_well_formed(path):
     got = {"y0": _sha(w.y0.to(data_dtype)), "t_eval": _sha(w.t_eval.to(time_dtype)), "params": _sha(w.f.builtin_params().to(data_dtype))}
     assert got == g["inputs_sha256"]
     assert len(g["n_steps"]) == g["batch"] and all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])
+
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if p.endswith("_fixed.json")], ids=os.path.basename)
+def test_fixed_step_fixture_is_well_formed_and_reproducible_here(path):
+    """Vectors of the ATen-op oracle with the reference's FixedStepController (tests/golden/make_golden.py::make_fixed)."""
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    assert {k: v for k, v in g["inputs_sha256"].items() if k != "dt0"} == {"y0": _sha(w.y0), "t_eval": _sha(w.t_eval), "params": _sha(w.f.builtin_params())}
+    assert g["n_steps"] == g["n_accepted"] and all(61 <= n <= 68 for n in g["n_steps"]) and g["n_f_evals"] == 1 + 6 * max(g["n_steps"])
+    assert all(s == 0 for s in g["status"]) and all(n == 50 or n == 20 for n in g["n_initialized"])

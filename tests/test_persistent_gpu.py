@@ -380,7 +380,7 @@ import glob  # noqa: E402
 import json  # noqa: E402
 import os  # noqa: E402
 
-_GOLDEN = sorted(p for p in glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")) if not p.endswith(("_tolerance.json", "_mixed.json")))
+_GOLDEN = sorted(p for p in glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")) if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json")))
 
 
 @pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])

@@ -370,3 +370,36 @@ def test_mixed_dtypes_match_the_aten_op_oracle_fixture(path):
         assert ys.dtype == data_dtype and sol.ts.dtype == time_dtype
         assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"], method.__name__
         assert hashlib.sha256(ys.contiguous().numpy().tobytes()).hexdigest() == g["ys_sha256"], method.__name__
+
+
+def _fixed_fixtures():
+    import glob
+    import os
+
+    return sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_fixed.json")))
+
+
+@pytest.mark.parametrize("path", _fixed_fixtures(), ids=lambda p: p.split("/")[-1])
+def test_fixed_steps_match_the_aten_op_oracle_fixture(path):
+    """tests/golden/*_fixed.json: the reference's loop with its FixedStepController as ATen CPU operations, written in
+    the authoring container.  The per-step kernels and the operator path reproduce every bit of them."""
+    import hashlib
+    import json
+
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    span = (w.t_eval[:, -1] - w.t_eval[:, 0]).double()
+    dt0 = (span / (60.37 + torch.arange(g["batch"], dtype=torch.float64) % 7)).to(dtype).cuda()
+    f = copy.deepcopy(w.f).cuda()
+    problem = to.InitialValueProblem(w.y0.cuda(), t_eval=w.t_eval.cuda())
+    fused_method, operator_method = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[g["method"]]
+    for method in (fused_method, operator_method):
+        sol = to.AutoDiffAdjoint(method(), to.FixedStepController()).solve(problem, to.ODETerm(lambda t, y: f(t, y)), dt0=dt0)
+        for key in ("n_steps", "n_accepted", "n_initialized"):
+            assert sol.stats[key].tolist() == g[key], (method.__name__, key)
+        assert sol.status.tolist() == g["status"] and int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
+        ys = sol.ys.cpu()
+        assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"], method.__name__
+        clean = ys.nan_to_num(nan=0.0, posinf=float("inf"), neginf=float("-inf"))
+        assert hashlib.sha256(clean.contiguous().numpy().tobytes()).hexdigest() == g["ys_sha256_nan_as_zero"], method.__name__
