@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 12
+#define TODE_ABI_VERSION 13
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -487,14 +487,18 @@ int tode_cubic_build(int32_t dtype, int64_t batch, int32_t n_features, const voi
 
 /* Polynomial evaluation (reference interpolation.py:8-40, 103-106, 172-175): for n = 0..count-1, b = idx[n],
  *   x = (t[n] - t0[b]) / (t1[b] - t0[b])  (denominator 1 where it is 0);  out[n,f] = Horner(coeff[degree..0, b, f], x)
- * coeff is [degree+1,B,F], degree in 1..4. */
-int tode_poly_eval(int32_t dtype, int32_t degree, int64_t batch, int32_t n_features, int64_t count, const void *coeff,
-                   const void *t0, const void *t1, const void *t, const int64_t *idx, void *out, void *stream);
+ * coeff is [degree+1,B,F], degree in 1..4.  With span_is_dt != 0 the operand `t1` holds the step size and is the
+ * denominator as it stands, as in the reference's LinearInterpolation (interpolation.py:56-58), which keeps dt where
+ * the higher-order interpolants keep t1 (interpolation.py:76-77, 132-133). */
+int tode_poly_eval(int32_t dtype, int32_t degree, int32_t span_is_dt, int64_t batch, int32_t n_features, int64_t count,
+                   const void *coeff, const void *t0, const void *t1, const void *t, const int64_t *idx, void *out,
+                   void *stream);
 
 /* The same evaluation for every set entry of a [B,E] byte mask, written to ys[b,e,:]
  * (reference adjoints.py:227-233 without materialising the index list). */
-int tode_poly_eval_masked(int32_t dtype, int32_t degree, int64_t batch, int32_t n_features, int32_t n_eval, const void *coeff,
-                          const void *t0, const void *t1, const void *t_eval, const uint8_t *mask, void *ys, void *stream);
+int tode_poly_eval_masked(int32_t dtype, int32_t degree, int32_t span_is_dt, int64_t batch, int32_t n_features,
+                          int32_t n_eval, const void *coeff, const void *t0, const void *t1, const void *t_eval,
+                          const uint8_t *mask, void *ys, void *stream);
 
 /* out[b,:] = mask[b] ? a[b,:] : b[b,:] for rows of `width` values (merge_states, reference runge_kutta.py:216-224,
  * step_size_controllers.py:628-638). */

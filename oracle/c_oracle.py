@@ -131,6 +131,16 @@ def pow_array(x: torch.Tensor, p: float) -> torch.Tensor:
     return out
 
 
+def pow_tensor_scalar(x: torch.Tensor, p: float) -> torch.Tensor:
+    """``x ** p`` for a Python float ``p`` with ATen's special exponents (0, 1, 0.5, -0.5, -1, 2, 3, -2) computed the
+    way its CPU kernels compute them."""
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    fn = lib().oracle_rpowf_array if x.dtype == torch.float32 else lib().oracle_rpow_array
+    fn(_p(x), C.c_double(p), _p(out), C.c_int64(x.numel()))
+    return out
+
+
 def solve(cfg: Config, params, y0, t_eval=None, *, t_start=None, t_end=None, dt0=None, trace_iters=0, trace_B=0):
     """Whole solve on the CPU.  ``ys`` rows that the loop never wrote are NaN."""
     dtype = y0.dtype

@@ -311,3 +311,7 @@ const oracle_tableau *oracle_get_tableau(int method) {
 #define R_ISFINITE(a) isfinite(a)
 #define R_POW(x, p) oracle_pow((x), (double)(p))
 #include "erk_oracle_impl.h"
+
+/* tensor ** python_float, elementwise (the dispatch of rpow above) */
+void oracle_rpowf_array(const float *x, double p, float *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = rpow_f32(x[i], p); }
+void oracle_rpow_array(const double *x, double p, double *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = rpow_f64(x[i], p); }

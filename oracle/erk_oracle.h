@@ -40,6 +40,8 @@ float oracle_powf(float x, float y);
 double oracle_pow(double x, double y);
 void oracle_powf_array(const float *x, float y, float *out, int64_t n);
 void oracle_pow_array(const double *x, double y, double *out, int64_t n);
+void oracle_rpowf_array(const float *x, double p, float *out, int64_t n);
+void oracle_rpow_array(const double *x, double p, double *out, int64_t n);
 const oracle_tableau *oracle_get_tableau(int method);
 
 #define ORACLE_DECLARE(REAL, SFX)                                                                                      \

@@ -9,9 +9,24 @@ static inline REAL SFX(tmax)(REAL a, REAL b) { return (a != a) ? a : ((b != b) ?
 static inline REAL SFX(tmin)(REAL a, REAL b) { return (a != a) ? a : ((b != b) ? b : (a < b ? a : b)); }
 static inline REAL SFX(tclamp)(REAL x, REAL lo, REAL hi) { return SFX(tmin)(SFX(tmax)(x, lo), hi); }
 
-/* pow in the tensor dtype with the exponent rounded to that dtype first
- * (ATen pow(Tensor, Scalar)). */
-static inline REAL SFX(rpow)(REAL x, double p) { return R_POW(x, (REAL)p); }
+/* tensor ** python_float as ATen's CPU kernels compute it: exponents 0 and 1 are a fill and a copy
+ * (aten/src/ATen/native/Pow.cpp), 0.5, -0.5 and -1 go to the square root, reciprocal square root and reciprocal kernels,
+ * 2, 3 and -2 are multiplications (aten/src/ATen/native/cpu/PowKernel.cpp); every other exponent is rounded to the
+ * tensor dtype and goes through pow.  The first group compares the exponent as the double it is, the second after
+ * rounding to the tensor dtype.  The square roots here are the correctly rounded ones; an ATen build that takes them
+ * from a vector math library can differ from that in the last bit (exponents 0.5 and -0.5 only). */
+static inline REAL SFX(rpow)(REAL x, double p) {
+    if (p == 0.0) return (REAL)1;
+    if (p == 1.0) return x;
+    if (p == 0.5) return R_SQRT(x);
+    if (p == -0.5) return (REAL)1 / R_SQRT(x);
+    if (p == -1.0) return (REAL)1 / x;
+    REAL e = (REAL)p;
+    if (e == (REAL)2) return x * x;
+    if (e == (REAL)3) return (x * x) * x;
+    if (e == (REAL)-2) return (REAL)1 / (x * x);
+    return R_POW(x, e);
+}
 
 /* ---- built-in right-hand sides, canonical op order, every op rounded on its own ---- */
 static void SFX(rhs)(const oracle_config *cfg, const REAL *par, REAL t, const REAL *y, REAL *dy, int F) {

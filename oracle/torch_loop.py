@@ -574,3 +574,146 @@ def solve(
     }
     ts = t_eval if t_eval is not None else t_end[:, None]
     return dict(ts=ts, ys=ys, status=status, **stats)
+
+
+# --------------------------------------------------------------------------- #
+# The two low-order methods: Heun 2(1) and forward Euler                      #
+# --------------------------------------------------------------------------- #
+
+
+def _heun() -> Tableau:
+    """heun.py:10-13: c = (0, 1), a_10 = 1, b = (1/2, 1/2), low-order weights (1, 0);
+    b_err = b - b_low in float64 (runge_kutta.py:84-88).  Neither FSAL nor SSAL."""
+    f64 = torch.float64
+    b, b_low = torch.tensor([0.5, 0.5], dtype=f64), torch.tensor([1.0, 0.0], dtype=f64)
+    return Tableau(torch.tensor([0.0, 1.0], dtype=f64), torch.tensor([[0.0, 0.0], [1.0, 0.0]], dtype=f64), b, b - b_low, torch.zeros((0, 2), dtype=f64), "heun")
+
+
+def erk_step_general(vf, tab: Tableau, t0, dt, y0):
+    """runge_kutta.py:247-272 for a tableau that is neither FSAL nor SSAL: the first stage is evaluated anew in
+    every step and y1 = y0 + sum_s (dt b_s) k_s.  Returns (y1, err, k).
+
+    pinned by: Heun on the linear test equation, y1 = (1 + z + z^2/2) y0 and err = (z^2/2) y0."""
+    dt_d = dt.to(dtype=y0.dtype)
+    S = tab.c.shape[0]
+    k0 = vf(t0, y0)
+    k = k0.new_empty((S, k0.shape[0], k0.shape[1]))
+    k[0] = k0
+    t_nodes = torch.addcmul(t0, tab.c[:, None], dt)
+    for i in range(1, S):
+        y_i = torch.einsum("j, jbf -> bf", tab.a[i, :i], k[:i])
+        y_i = torch.addcmul(y0, dt_d[:, None], y_i)
+        k[i] = vf(t_nodes[i], y_i)
+    y1 = y0 + torch.einsum("b, s, sbf -> bf", dt_d, tab.b, k)
+    err = torch.einsum("b, s, sbf -> bf", dt_d, tab.b_err, k)
+    return y1, err, k
+
+
+def cubic_from_k(dt, y0, y1, k):
+    """interpolation.py:84-106: Hermite cubic through (y0, y1) with end slopes k[0], k[-1]; coefficients (d, c, b, a),
+    lowest power first.
+
+    pinned by: p(0) = y0, p(1) = y1, p'(0) = dt k[0], p'(1) = dt k[-1]."""
+    f0, f1 = k[0], k[-1]
+    dt_d = dt.to(dtype=y0.dtype)
+    y0my1 = y0 - y1
+    a = torch.add(dt_d[:, None] * (f0 + f1), y0my1, alpha=2)
+    b = torch.add(dt_d[:, None] * torch.add(-f1, f0, alpha=-2), y0my1, alpha=-3)
+    c = dt_d[:, None] * f0
+    return y0, c, b, a
+
+
+def cubic_eval(coeff, t0, t1, t, idx):
+    """interpolation.py:8-22, 108-111: Horner on x = (t - t0) / (t1 - t0)."""
+    d, c, b, a = (x[idx] for x in coeff)
+    den = t1[idx] - t0[idx]
+    den = torch.where(den.abs() > 0.0, den, 1.0)
+    x = ((t - t0[idx]) / den)[:, None].to(dtype=a.dtype)
+    y = a
+    y = torch.addcmul(b, y, x)
+    y = torch.addcmul(c, y, x)
+    y = torch.addcmul(d, y, x)
+    return y
+
+
+def linear_eval(t0, dt, y0, y1, t, idx):
+    """interpolation.py:48-62: y0 + (y1 - y0) x with x = (t - t0) / dt (note: dt itself, not (t0 + dt) - t0)."""
+    dy = y1 - y0
+    den = dt[idx]
+    den = torch.where(den.abs() > 0.0, den, 1.0)
+    x = ((t - t0[idx]) / den)[:, None].to(dtype=y0.dtype)
+    return torch.addcmul(y0[idx], dy[idx], x)
+
+
+def solve_low_order(
+    f: Callable,
+    y0: torch.Tensor,
+    t_eval: Optional[torch.Tensor],
+    *,
+    method: str,
+    controller: Controller,
+    t_start: Optional[torch.Tensor] = None,
+    t_end: Optional[torch.Tensor] = None,
+    dt0: Optional[torch.Tensor] = None,
+    max_steps: Optional[int] = None,
+) -> Dict[str, torch.Tensor]:
+    """adjoints.py:50-309 with ``method`` "heun" (heun.py, order 2, error estimate against the Euler step, cubic dense
+    output) or "euler" (euler.py, order 1, no error estimate: an adaptive controller then accepts every step and keeps
+    the step size, step_size_controllers.py:382-391 / 727-736; linear dense output) and any of the three controllers.
+
+    pinned by: the pins of the pieces above; fixed-step accuracy against the analytic solution
+    (tests/fixed_step_controller_test.py:9-19), Euler's step counts [20, 16, 3] (tests/adjoint_test.py:98-118)."""
+    if t_start is None:
+        t_start = t_eval[:, 0]
+    if t_end is None:
+        t_end = t_eval[:, -1]
+    B = y0.shape[0]
+    heun = method == "heun"
+    order = 2 if heun else 1
+    tab = _heun().cast(t_start.dtype, y0.dtype)
+    direction_i = torch.where(t_end > t_start, 1, -1)
+    calls = [0]
+
+    def vf(t, y):
+        calls[0] += 1
+        return f(t, y)
+
+    fixed = controller.kind == "fixed"
+    assert not fixed or dt0 is not None, "Fixed step size solving requires you to configure dt0"
+    # (the controller's start step evaluates f twice; its f0 goes unused: neither method keeps a first-stage value)
+    dt = initial_step(vf, controller, order, t_start, y0, direction_i, (t_end - t_start).abs())[0] if dt0 is None else dt0
+    ones = torch.ones(B, dtype=y0.dtype)
+    accept_all = torch.ones(B, dtype=torch.bool)
+
+    def step(running, y, t, dt, state):
+        if heun:
+            y1, err, k = erk_step_general(vf, tab, t, dt, y)
+            return y1, (t, dt, y, y1, err, k), None, None
+        y1 = torch.addcmul(y, dt.to(dtype=y.dtype)[:, None], vf(t, y))
+        return y1, (t, dt, y, y1, None, None), None, None
+
+    def adapt_(t, dt, y, y1, data, state):
+        if fixed:
+            return accept_all, dt0, (state[0], state[1], ones), None
+        if data[4] is None:  # no error estimate: accepted, step size kept, no status
+            return accept_all, dt, (state[0], state[1], ones), None
+        accept, dt_next, status, ratio, prev_n, prev_prev_n = adapt(controller, order, dt, y, y1, data[4], *state)
+        return accept, dt_next, (prev_n, prev_prev_n, ratio), status
+
+    def dense(data):
+        t0, dt, y, y1, _, k = data
+        if heun:
+            coeff = cubic_from_k(dt, y, y1, k)
+            return lambda tt, idx: cubic_eval(coeff, t0, t0 + dt, tt, idx)
+        return lambda tt, idx: linear_eval(t0, dt, y, y1, tt, idx)
+
+    ys, status, n_steps, n_accepted, n_init, _ = run_loop(
+        y0, t_start, t_end, t_eval, dt, step, adapt_, lambda move, new, old: None,
+        lambda running, new, old: (torch.where(running, new[0], old[0]), torch.where(running, new[1], old[1])),
+        dense, None, (ones, ones), max_steps=max_steps,
+    )  # fmt: skip
+    if status is None:
+        status = torch.tensor(SUCCESS, dtype=torch.long).expand(B)
+    ts = t_eval if t_eval is not None else t_end[:, None]
+    return dict(ts=ts, ys=ys, status=status, n_f_evals=torch.full((B,), calls[0], dtype=torch.long), n_steps=n_steps,
+                n_accepted=n_accepted, n_initialized=n_init)  # fmt: skip

@@ -160,6 +160,55 @@ def make_fixed(name, batch, dtype, method):
     }
 
 
+# Heun and Euler (reference heun.py, euler.py) with the three controllers: vectors of the ATen-op oracle alone.
+#   (workload, batch, dtype, method, controller or None for the workload's own, parts of the span as the first step or None)
+# (Without a first step the reference takes ``x ** (1 / order)`` in its choice of one, which for Heun's order 2 is ATen's
+# square root kernel; that one comes from a vector math library on this host and is not the correctly rounded root for
+# some 0.7 % of arguments.  Such a case is written as a tolerance-level vector: "bit_exact" false.)
+LOW_ORDER_CASES = [
+    ("vdp", 256, torch.float32, "heun", None, 400.37),
+    ("lorenz", 256, torch.float64, "heun", dict(kind="integral", atol=1e-6, rtol=1e-4), 500.37),
+    ("linear_decay", 256, torch.float64, "heun", dict(kind="integral", atol=1e-6, rtol=1e-4), None),
+    ("linear_decay", 256, torch.float64, "heun", dict(kind="fixed", atol=0.0, rtol=0.0), 80.37),
+    ("vdp", 256, torch.float32, "euler", dict(kind="fixed", atol=0.0, rtol=0.0), 200.37),
+    ("linear_decay", 256, torch.float64, "euler", dict(kind="integral", atol=1e-6, rtol=1e-4), 300.37),
+]
+
+
+def low_order_inputs(name, batch, dtype, parts):
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    if parts is None:
+        return w, None
+    span = (w.t_eval[:, -1] - w.t_eval[:, 0]).double()
+    return w, (span / (parts + torch.arange(batch, dtype=torch.float64) % 7)).to(dtype)
+
+
+def make_low_order(name, batch, dtype, method, controller, parts):
+    w, dt0 = low_order_inputs(name, batch, dtype, parts)
+    controller = dict(w.controller) if controller is None else controller
+    out = torch_loop.solve_low_order(w.f, w.y0, w.t_eval, method=method, controller=torch_loop.Controller(**controller), dt0=dt0)
+    assert (out["status"] == 0).all() and (out["n_initialized"] == w.t_eval.shape[1]).all()
+    sub = list(range(0, batch, max(1, batch // 16)))[:16]
+    return {
+        "source": f"oracle/torch_loop.py::solve_low_order (ATen CPU ops), torch {torch.__version__}, {torch.backends.cpu.get_cpu_capability()}, "
+        f"opt_einsum {torch.backends.opt_einsum.is_available()}",
+        "workload": name,
+        "batch": batch,
+        "dtype": str(dtype).replace("torch.", ""),
+        "method": method,
+        "controller": controller,
+        "first_step_parts": parts,
+        "bit_exact": parts is not None,
+        "inputs_sha256": {"y0": sha(w.y0), "t_eval": sha(w.t_eval), "params": sha(w.f.builtin_params())},
+        "n_f_evals": int(out["n_f_evals"][0]),
+        **{key: out[key].tolist() for key in ("n_steps", "n_accepted", "n_initialized", "status")},
+        "ys_sha256_nan_as_zero": sha(out["ys"].nan_to_num(nan=0.0, posinf=float("inf"), neginf=float("-inf"))),
+        "ys_finite_fraction": float(out["ys"].isfinite().double().mean()),
+        "subset": sub,
+        "ys_subset": hexlist(out["ys"][sub]),
+    }
+
+
 def make_tolerance(name, batch, dtype):
     w = to.workloads.make(name, batch=batch, dtype=dtype)
     out = torch_loop.solve(w.f, w.y0, w.t_eval, method=w.method, controller=torch_loop.Controller(**w.controller))
@@ -184,6 +233,12 @@ def make_tolerance(name, batch, dtype):
 
 
 if __name__ == "__main__":
+    for name, batch, dtype, method, controller, parts in LOW_ORDER_CASES:
+        d = make_low_order(name, batch, dtype, method, controller, parts)
+        path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_{method}_{d['controller']['kind']}_low_order.json")
+        with open(path, "w") as fh:
+            json.dump(d, fh, separators=(",", ":"))
+        print(path, os.path.getsize(path), "bytes")
     for name, batch, dtype, method in FIXED_CASES:
         d = make_fixed(name, batch, dtype, method)
         path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_{method}_fixed.json")

@@ -170,3 +170,16 @@ def poisoned(y0: torch.Tensor, seed: int) -> torch.Tensor:
     else:
         y0[idx] = y0[idx] * 1e6
     return y0
+
+
+# PID coefficients (p, i, d) whose exponents for a fifth-order method, -(i+p+d)/5, (p+2d)/5 and -d/5, are ones that
+# ATen does not compute through pow: -1; -2 and 2; -2, 3 and -1; -0.5
+SHORTCUT_PID = [(0.0, 5.0, 0.0), (10.0, 0.0, 0.0), (5.0, 0.0, 5.0), (0.0, 2.5, 0.0)]
+
+
+def shortcut_case(seed):
+    """A wild case whose controller is a PID controller with exponents from SHORTCUT_PID."""
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = wild_case(seed)
+    p, i, d = SHORTCUT_PID[seed % len(SHORTCUT_PID)]
+    ctrl = {k: v for k, v in dict(ctrl, kind="pid", pcoeff=p, icoeff=i, dcoeff=d).items() if k not in ("dt_min", "dt_max")}
+    return f, y0, t_eval, t_start, t_end, method, ctrl, 600, dt0  # (no step limits: the controller runs many times)

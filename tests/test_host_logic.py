@@ -165,7 +165,7 @@ def test_tolerance_fixture_inputs_and_workload_agree(path):
     assert all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])
 
 
-@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json"))], ids=os.path.basename)
+@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json"))], ids=os.path.basename)
 def test_oracle_reproduces_golden_fixture(path):
     g = json.load(open(path))
     dtype = getattr(torch, g["dtype"])
@@ -227,3 +227,21 @@ def test_fixed_step_fixture_is_well_formed_and_reproducible_here(path):
     assert {k: v for k, v in g["inputs_sha256"].items() if k != "dt0"} == {"y0": _sha(w.y0), "t_eval": _sha(w.t_eval), "params": _sha(w.f.builtin_params())}
     assert g["n_steps"] == g["n_accepted"] and all(61 <= n <= 68 for n in g["n_steps"]) and g["n_f_evals"] == 1 + 6 * max(g["n_steps"])
     assert all(s == 0 for s in g["status"]) and all(n == 50 or n == 20 for n in g["n_initialized"])
+
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if p.endswith("_low_order.json")], ids=os.path.basename)
+def test_low_order_fixture_is_well_formed(path):
+    """Vectors of the ATen-op oracle with Heun and Euler (tests/golden/make_golden.py::make_low_order): the inputs are
+    the workload's, every sample finished, and the evaluation count follows from the step count (two per Heun step,
+    one per Euler step, two more where the first step size is chosen automatically)."""
+    g = json.load(open(path))
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=getattr(torch, g["dtype"]))
+    assert g["inputs_sha256"] == {"y0": _sha(w.y0), "t_eval": _sha(w.t_eval), "params": _sha(w.f.builtin_params())}
+    per_step, first = {"heun": 2, "euler": 1}[g["method"]], 2 if g["first_step_parts"] is None else 0
+    assert g["n_f_evals"] == first + per_step * max(g["n_steps"]) and all(s == 0 for s in g["status"])
+    assert all(n == w.t_eval.shape[1] for n in g["n_initialized"]) and g["ys_finite_fraction"] == 1.0
+    assert g["bit_exact"] == (g["first_step_parts"] is not None)  # (the controller's own first step takes x ** 0.5)
+    if g["controller"]["kind"] == "fixed" or g["method"] == "euler":
+        assert g["n_steps"] == g["n_accepted"]  # nothing to reject without an error estimate or with fixed steps
+    else:
+        assert all(a <= n for a, n in zip(g["n_accepted"], g["n_steps"]))

@@ -658,6 +658,23 @@ def test_oracles_agree_on_random_configurations(seed):
 
 
 @needs_pinned_aten
+@pytest.mark.parametrize("seed", range(12))
+def test_oracles_agree_where_the_controller_powers_are_shortcuts(seed):
+    """PID coefficients that make the controller's exponents -1, 2, 3, -2 or -0.5, which ATen computes by reciprocal,
+    products and reciprocal square root instead of pow (tests/helpers.py::shortcut_case)."""
+    from helpers import c_oracle_solve, shortcut_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = shortcut_case(seed)
+    a = tl.solve(f, y0, t_eval, method=method, controller=tl.Controller(**ctrl), t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    c = c_oracle_solve(f, y0, t_eval, method, ctrl, t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps, nthreads=4)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status", "n_f_evals"):
+        assert torch.equal(a[key], c[key]), key
+    av, cv = a["ys"][c["written"]], c["ys"][c["written"]]
+    assert bool(((av == cv) | (av.isnan() & cv.isnan())).all())
+    assert int(c["n_steps"].max()) > 20
+
+
+@needs_pinned_aten
 @pytest.mark.parametrize("seed", range(24))
 def test_oracles_agree_on_wild_configurations(seed):
     """Scalar C loop against the batched ATen-op loop over everything the loop knows at once: evaluation points
@@ -689,3 +706,67 @@ def test_oracles_agree_on_wild_configurations_with_non_finite_samples(seed):
     av, cv = a["ys"][c["written"]], c["ys"][c["written"]]
     assert bool(((av == cv) | (av.isnan() & cv.isnan())).all())
     assert seed % 4 == 3 or (c["status"] != 0).any()  # (a sample that is merely large may solve after all)
+
+
+# --------------------------------------------------------------------------- #
+# the low-order methods of the ATen-op oracle                                 #
+# --------------------------------------------------------------------------- #
+
+
+def test_heun_step_and_hermite_cubic():
+    """Heun on y' = lambda y: y1 = (1 + z + z^2/2) y0 and err = (z^2/2) y0 with z = lambda dt (the second-order
+    stability polynomial against the first-order one); the cubic dense output takes y0, y1 and both end slopes."""
+    lam = torch.tensor([[-0.7, 0.3], [2.0, -5.0]], dtype=F64)
+    y0, t0, dt = torch.tensor([[1.5, -2.0], [0.25, 3.0]], dtype=F64), torch.tensor([0.2, -1.0], dtype=F64), torch.tensor([0.4, -0.05], dtype=F64)
+    y1, err, k = tl.erk_step_general(lambda t, y: lam * y, tl._heun(), t0, dt, y0)
+    z = lam * dt[:, None]
+    assert torch.allclose(y1, (1 + z + z * z / 2) * y0, rtol=1e-14, atol=0) and torch.allclose(err, (z * z / 2) * y0, rtol=1e-13, atol=1e-18)
+    coeff, idx, eps = tl.cubic_from_k(dt, y0, y1, k), torch.arange(2), 1e-6
+    at = lambda x: tl.cubic_eval(coeff, t0, t0 + dt, t0 + x * dt, idx)
+    assert torch.equal(at(0.0), y0) and torch.allclose(at(1.0), y1, rtol=1e-15, atol=0)
+    assert torch.allclose((at(eps) - at(0.0)) / eps, dt[:, None] * k[0], rtol=1e-4) and torch.allclose((at(1.0) - at(1.0 - eps)) / eps, dt[:, None] * k[1], rtol=1e-4)
+    line = lambda x: tl.linear_eval(t0, dt, y0, y1, t0 + x * dt, idx)
+    assert torch.equal(line(0.0), y0) and torch.allclose(line(1.0), y1, rtol=1e-15, atol=0) and torch.allclose(line(0.5), (y0 + y1) / 2, rtol=1e-15, atol=0)
+
+
+def test_low_order_solves_against_the_analytic_solution_and_the_reference_step_counts():
+    """reference tests/fixed_step_controller_test.py:9-19 (analytic solution to 1e-2), tests/adjoint_test.py:98-118
+    (Euler, no evaluation points: n_steps [20, 16, 3]); evaluation counts 2 per Heun step, 1 per Euler step."""
+    w = to.workloads.make("linear_decay", batch=64, dtype=F64)
+    exact = w.y0[:, None] * torch.exp(-w.f.k[:, None] * (w.t_eval - w.t_eval[:, :1])[:, :, None])
+    heun = tl.solve_low_order(w.f, w.y0, w.t_eval, method="heun", controller=tl.Controller("pid", 1e-6, 1e-4, 0.2, 0.5, 0.0))
+    assert (heun["ys"] - exact).abs().max() < 1e-4 and int(heun["n_f_evals"][0]) == 2 + 2 * int(heun["n_steps"].max()) and (heun["n_steps"] > 20).all()
+    dt0 = torch.full((64,), 1e-3, dtype=F64)
+    for method, per_step in (("heun", 2), ("euler", 1)):
+        out = tl.solve_low_order(w.f, w.y0, w.t_eval, method=method, controller=tl.Controller("fixed", 0.0, 0.0), dt0=dt0)
+        assert (out["ys"] - exact).abs().max() < 1e-2 and int(out["n_f_evals"][0]) == per_step * int(out["n_steps"].max())
+    no_estimate = tl.solve_low_order(w.f, w.y0, w.t_eval, method="euler", controller=tl.Controller("integral", 1e-6, 1e-4), dt0=dt0 * 10)
+    assert torch.equal(no_estimate["n_steps"], no_estimate["n_accepted"]) and (no_estimate["status"] == 0).all()  # accepted as is, step kept
+    y0 = torch.tensor([[0.0], [1.0], [2.0]], dtype=F64)
+    t_start, t_end = torch.tensor([0.0, 5.0, 2.0], dtype=F64), torch.tensor([10.0, 9.0, 4.5], dtype=F64)
+    steps = torch.tensor([0.5001, 0.2501, 1.0], dtype=F64)
+    out = tl.solve_low_order(lambda t, y: torch.ones_like(y), y0, None, method="euler", controller=tl.Controller("fixed", 0.0, 0.0), t_start=t_start, t_end=t_end, dt0=steps)
+    assert out["n_steps"].tolist() == [20, 16, 3] and torch.allclose(out["ys"][:, 0], y0 + (t_end - t_start)[:, None], rtol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
+def test_tensor_to_a_python_float_follows_atens_shortcuts(dtype):
+    """``x ** p`` with a Python float ``p`` is not always pow: ATen fills for 0, copies for 1, takes the reciprocal
+    square root, the reciprocal and plain products for -0.5, -1, 2, 3, -2 (step_size_controllers.py:292-293 and 612-617
+    reach these with order-2 methods or unusual PID coefficients).  The oracle's version reproduces each of them bit for
+    bit, special values included; 0.5 is ATen's square root kernel, which on some hosts comes from a vector math library
+    and is then off by one ulp for under 2 % of arguments."""
+    g = torch.Generator().manual_seed(5)
+    n = 1 << 15  # (whole vectors: the scalar tail of ATen's kernels is another implementation)
+    x = torch.rand(n, dtype=dtype, generator=g) * 10 + 1e-3
+    x[:8] = torch.tensor([0.0, 1.0, float("inf"), float("nan"), 1e-30, 1e30, 2.0, 0.25], dtype=dtype)
+    for p in (0.0, 1.0, -1.0, 2.0, 3.0, -2.0, -0.5):
+        got, want = c_oracle.pow_tensor_scalar(x, p), x**p
+        assert torch.equal(got.isnan(), want.isnan()) and torch.equal(got.nan_to_num(nan=0.0), want.nan_to_num(nan=0.0)), p
+        if p not in (0.0, 1.0):
+            generic = c_oracle.pow_array(x, p)
+            assert not torch.equal(generic.nan_to_num(nan=0.0), want.nan_to_num(nan=0.0)), p  # the shortcut is not a no-op
+    got, want = c_oracle.pow_tensor_scalar(x, 0.5), x**0.5
+    assert torch.equal(got.nan_to_num(nan=-1.0), torch.from_numpy(np.sqrt(x.numpy())).nan_to_num(nan=-1.0))
+    off = (got != want) & ~want.isnan()
+    assert off.double().mean() < 0.02 and torch.allclose(got[8:], want[8:], rtol=4 * torch.finfo(dtype).eps, atol=0)

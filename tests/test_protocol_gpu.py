@@ -837,6 +837,16 @@ def test_wild_configurations_match_oracle_bit_for_bit(seed):
     assert_identical(protocol_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
 
 
+@pytest.mark.parametrize("seed", range(740, 748))
+def test_controller_powers_that_are_shortcuts_match_oracle_bit_for_bit(seed):
+    """tests/helpers.py::shortcut_case (controller exponents -1, 2, 3, -2, -0.5) through the operator path."""
+    from helpers import shortcut_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = shortcut_case(seed)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    assert_identical(protocol_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
+
+
 @pytest.mark.parametrize("seed", range(600, 608))
 def test_wild_configurations_with_non_finite_samples(seed):
     """wild_case with three samples NaN, infinite, huge or blowing up later (tests/helpers.py::poisoned): status 4, 2
@@ -847,3 +857,49 @@ def test_wild_configurations_with_non_finite_samples(seed):
     y0 = poisoned(y0, seed)
     kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=min(max_steps, 400))
     assert_identical(protocol_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
+
+
+def _low_order_fixtures():
+    import glob
+    import os
+
+    return sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_low_order.json")))
+
+
+@pytest.mark.parametrize("path", _low_order_fixtures(), ids=lambda p: p.split("/")[-1])
+def test_heun_and_euler_match_the_aten_op_oracle_fixture(path):
+    """tests/golden/*_low_order.json: the reference's loop with Heun / Euler and each of its three controllers as ATen
+    CPU operations (oracle/torch_loop.py::solve_low_order), written in the authoring container.  The operator path
+    reproduces every bit of them.  The one case that leaves the choice of the first step to the controller goes through
+    ATen's square root kernel (``x ** 0.5`` for order 2), which on the authoring host is a vector math library's and not
+    always the correctly rounded root: that case is compared to 1e-10 and in its counts."""
+    import hashlib
+    import json
+
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    dt0 = None
+    if g["first_step_parts"] is not None:
+        span = (w.t_eval[:, -1] - w.t_eval[:, 0]).double()
+        dt0 = (span / (g["first_step_parts"] + torch.arange(g["batch"], dtype=torch.float64) % 7)).to(dtype).to(DEV)
+    spec = dict(g["controller"])
+    controller = to.FixedStepController() if spec["kind"] == "fixed" else make_controller(spec)
+    method = {"heun": to.Heun, "euler": to.Euler}[g["method"]]()
+    f = copy.deepcopy(w.f).to(DEV)
+    sol = to.AutoDiffAdjoint(method, controller).solve(to.InitialValueProblem(w.y0.to(DEV), t_eval=w.t_eval.to(DEV)), to.ODETerm(f), dt0=dt0)
+    ys = sol.ys.cpu()
+    assert sol.status.tolist() == g["status"] and sol.stats["n_initialized"].tolist() == g["n_initialized"]
+    if not g["bit_exact"]:
+        for key in ("n_steps", "n_accepted"):
+            same = (sol.stats[key].cpu() == torch.tensor(g[key])).double().mean().item()
+            assert same >= 0.99, (key, same)
+        want = torch.tensor([float.fromhex(v) for v in g["ys_subset"]], dtype=dtype).reshape(ys[g["subset"]].shape)
+        assert torch.allclose(ys[g["subset"]], want, rtol=1e-10, atol=1e-10)
+        return
+    for key in ("n_steps", "n_accepted"):
+        assert sol.stats[key].tolist() == g[key], key
+    assert int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
+    assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
+    clean = ys.nan_to_num(nan=0.0, posinf=float("inf"), neginf=float("-inf"))
+    assert hashlib.sha256(clean.contiguous().numpy().tobytes()).hexdigest() == g["ys_sha256_nan_as_zero"]

@@ -328,6 +328,16 @@ def test_wild_configurations_match_oracle_bit_for_bit(seed):
     assert_identical(stepwise_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
 
 
+@pytest.mark.parametrize("seed", range(720, 728))
+def test_controller_powers_that_are_shortcuts_match_oracle_bit_for_bit(seed):
+    """tests/helpers.py::shortcut_case (controller exponents -1, 2, 3, -2, -0.5) through the per-step kernels."""
+    from helpers import shortcut_case
+
+    f, y0, t_eval, t_start, t_end, method, ctrl, max_steps, dt0 = shortcut_case(seed)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=max_steps)
+    assert_identical(stepwise_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
+
+
 @pytest.mark.parametrize("seed", range(500, 508))
 def test_wild_configurations_with_non_finite_samples(seed):
     """wild_case with three samples NaN, infinite, huge or blowing up later (tests/helpers.py::poisoned): status 4, 2

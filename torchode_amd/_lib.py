@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -271,8 +271,8 @@ def load():
             "tode_quartic_build": [I32, I32, I64, I32] + [V] * 6,
             "tode_quartic_from_mid": [I32, I64, I32] + [V] * 8,
             "tode_cubic_build": [I32, I64, I32] + [V] * 7,
-            "tode_poly_eval": [I32, I32, I64, I32, I64] + [V] * 7,
-            "tode_poly_eval_masked": [I32, I32, I64, I32, I32] + [V] * 7,
+            "tode_poly_eval": [I32, I32, I32, I64, I32, I64] + [V] * 7,
+            "tode_poly_eval_masked": [I32, I32, I32, I64, I32, I32] + [V] * 7,
             "tode_select_rows": [I32, I64, I32] + [V] * 5,
             "tode_loop_advance": [C.POINTER(LoopArgs), V],
             "tode_loop_begin": [I32, I64, I32, I32] + [V] * 9,

@@ -271,8 +271,9 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller
     if (rc == TODE_E_UNSUPPORTED && (a->n_eval > 0 || a->y_idle) && !c->has_dt_min && !c->has_dt_max &&
         a->term != TODE_TERM_REACTION_DIFFUSION && a->term != TODE_TERM_MLP) {
         // a small system in a shape the fast kernels do not take (no evaluation points, or very many of them, in a
-        // batch too large for the two-wavefront kernel): no kernel was launched, and the caller is sent to the general
-        // kernel like any batch that leaves the common case
+        // batch too large for the two-wavefront kernel) or with a controller exponent that is not computed through pow:
+        // no solve kernel was launched, and the caller is sent to the general kernel like any batch that leaves the
+        // common case
         flags_out[TODE_FLAG_MAX_ITERATIONS] = 0;
         flags_out[TODE_FLAG_FIRST_FAILURE] = INT_MAX;
         flags_out[TODE_FLAG_NON_MONOTONE] = 0;

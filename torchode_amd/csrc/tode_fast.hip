@@ -275,6 +275,7 @@ static int launch_fast(const tode_solve_args &a, const tode_controller &c, const
     const size_t need_all = lds_bytes(a.n_eval, Term::F, sizeof(T), true);
     if (need_te > 64 * 1024) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the fast kernel", a.n_eval);
     const CtrlParams<T> &cp = p.cp;
+    if (cp.shortcut_exponent()) return fail(TODE_E_UNSUPPORTED, "a controller exponent that is not computed through pow: use the general kernel");
     const int nhist = CTRL == 0 ? 0 : (cp.skip3 ? 1 : 2);
     const bool stage = need_all <= budget;
     const size_t lds = stage ? need_all : need_te;

@@ -218,8 +218,30 @@ template <typename T> __device__ __forceinline__ T pow_(T x, T y) {
     return powk<T>(logk(x), y);
 }
 
-// Tensor ** python_float: the exponent is rounded to the tensor dtype first.
-template <typename T> __device__ __forceinline__ T rpow(T x, double p) { return pow_<T>(x, (T)p); }
+// Tensor ** python_float as ATen's CPU kernels compute it: exponents 0 and 1 are a fill and a
+// copy (aten/src/ATen/native/Pow.cpp); 0.5, -0.5 and -1 go to the square root, reciprocal square
+// root and reciprocal kernels and 2, 3 and -2 are multiplications
+// (aten/src/ATen/native/cpu/PowKernel.cpp); every other exponent is rounded to the tensor dtype
+// and goes through pow.  The first group compares the exponent as the double it is, the second
+// after rounding to the tensor dtype.  The square roots are the correctly rounded ones; an ATen
+// build that takes them from a vector math library can differ from that in the last bit
+// (exponents 0.5 and -0.5 only).
+template <typename T> __host__ __device__ __forceinline__ bool special_exponent(double p) {
+    const T e = (T)p;
+    return p == 0.0 || p == 1.0 || p == 0.5 || p == -0.5 || p == -1.0 || e == (T)2 || e == (T)3 || e == (T)-2;
+}
+template <typename T> __device__ __forceinline__ T rpow(T x, double p) {
+    if (p == 0.0) return (T)1;
+    if (p == 1.0) return x;
+    if (p == 0.5) return sqrt_(x);
+    if (p == -0.5) return (T)1 / sqrt_(x);
+    if (p == -1.0) return (T)1 / x;
+    const T e = (T)p;
+    if (e == (T)2) return x * x;
+    if (e == (T)3) return (x * x) * x;
+    if (e == (T)-2) return (T)1 / (x * x);
+    return pow_<T>(x, e);
+}
 
 // ---------------------------------------------------------------------------
 // Butcher tableaux, float64 literals cast to the working type where used
@@ -291,6 +313,11 @@ template <typename T> struct CtrlParams {
     double e1, e2, e3;         // pow exponents: ratio, prev, prev_prev
     int has_dt_min, has_dt_max;
     int skip2, skip3;          // exponent is +-0: the factor is exactly 1
+    // an exponent that ATen does not compute through pow (kernels that share one logarithm
+    // between the powers do not take such a controller)
+    bool shortcut_exponent() const {
+        return special_exponent<T>(e1) && e1 != 0.0 || !skip2 && special_exponent<T>(e2) || !skip3 && special_exponent<T>(e3);
+    }
 };
 
 // rms_norm over F register values (step_size_controllers.py:170-181); ATen's CPU

@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(256) cubic_build_kernel(long long batch, int F
 }
 
 template <typename TT, typename T>
-__global__ void __launch_bounds__(256) poly_eval_kernel(int degree, long long batch, int F, long long count, const T *coeff, const TT *t0, const TT *t1,
+__global__ void __launch_bounds__(256) poly_eval_kernel(int degree, int span_is_dt, long long batch, int F, long long count, const T *coeff, const TT *t0, const TT *t1,
                                                         const TT *t, const int64_t *idx, T *out) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i >= count * F) return;
@@ -360,30 +360,30 @@ __global__ void __launch_bounds__(256) poly_eval_kernel(int degree, long long ba
     const int f = (int)(i - n * F);
     const long long b = idx[n];
     if (b < 0 || b >= batch) return;
-    out[i] = horner(coeff, batch * F, b * F + f, degree, (T)unit_time(t[n], t0[b], t1[b]));
+    out[i] = horner(coeff, batch * F, b * F + f, degree, (T)unit_time_over(t[n], t0[b], span_is_dt ? t1[b] : t1[b] - t0[b]));
 }
 
 // small F: one thread per sample walks its mask row
 template <typename TT, typename T>
-__global__ void __launch_bounds__(256) poly_eval_masked_thread_kernel(int degree, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
+__global__ void __launch_bounds__(256) poly_eval_masked_thread_kernel(int degree, int span_is_dt, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
                                                                       const TT *t_eval, const uint8_t *mask, T *ys) {
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= batch) return;
     for (int e = 0; e < E; ++e) {
         if (!mask[b * E + e]) continue;
-        const T x = (T)unit_time(t_eval[b * E + e], t0[b], t1[b]);
+        const T x = (T)unit_time_over(t_eval[b * E + e], t0[b], span_is_dt ? t1[b] : t1[b] - t0[b]);
         for (int f = 0; f < F; ++f) ys[(b * E + e) * F + f] = horner(coeff, batch * F, b * F + f, degree, x);
     }
 }
 
 // large F: one workgroup per sample, threads over features
 template <typename TT, typename T>
-__global__ void __launch_bounds__(256) poly_eval_masked_block_kernel(int degree, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
+__global__ void __launch_bounds__(256) poly_eval_masked_block_kernel(int degree, int span_is_dt, long long batch, int F, int E, const T *coeff, const TT *t0, const TT *t1,
                                                                      const TT *t_eval, const uint8_t *mask, T *ys) {
     const long long b = blockIdx.x;
     for (int e = 0; e < E; ++e) {
         if (!mask[b * E + e]) continue;  // uniform over the workgroup
-        const T x = (T)unit_time(t_eval[b * E + e], t0[b], t1[b]);
+        const T x = (T)unit_time_over(t_eval[b * E + e], t0[b], span_is_dt ? t1[b] : t1[b] - t0[b]);
         for (int f = threadIdx.x; f < F; f += 256) ys[(b * E + e) * F + f] = horner(coeff, batch * F, b * F + f, degree, x);
     }
 }
@@ -788,21 +788,21 @@ int tode_cubic_build(int32_t dtype, int64_t batch, int32_t F, const void *dt, co
     return done("tode_cubic_build launch");
 }
 
-int tode_poly_eval(int32_t dtype, int32_t degree, int64_t batch, int32_t F, int64_t count, const void *coeff, const void *t0, const void *t1,
-                   const void *t, const int64_t *idx, void *out, void *stream) {
+int tode_poly_eval(int32_t dtype, int32_t degree, int32_t span_is_dt, int64_t batch, int32_t F, int64_t count, const void *coeff, const void *t0,
+                   const void *t1, const void *t, const int64_t *idx, void *out, void *stream) {
     if (int rc = check_common(dtype, batch, F)) return rc;
     if (degree < 1 || degree > 4) return fail(TODE_E_INVALID, "degree %d outside 1..4", degree);
     if (count < 0) return fail(TODE_E_INVALID, "negative count");
     if (count == 0) return TODE_OK;
     if (batch == 0) return fail(TODE_E_INVALID, "evaluation points but an empty batch");
     if (!coeff || !t0 || !t1 || !t || !idx || !out) return fail(TODE_E_INVALID, "null pointer");
-    TODE_TT(dtype, hipLaunchKernelGGL((poly_eval_kernel<TT, T>), dim3(blocks_for(count * F, 256)), dim3(256), 0, (hipStream_t)stream, degree, (long long)batch,
-                                      F, (long long)count, (const T *)coeff, (const TT *)t0, (const TT *)t1, (const TT *)t, idx, (T *)out));
+    TODE_TT(dtype, hipLaunchKernelGGL((poly_eval_kernel<TT, T>), dim3(blocks_for(count * F, 256)), dim3(256), 0, (hipStream_t)stream, degree, span_is_dt != 0,
+                                      (long long)batch, F, (long long)count, (const T *)coeff, (const TT *)t0, (const TT *)t1, (const TT *)t, idx, (T *)out));
     return done("tode_poly_eval launch");
 }
 
-int tode_poly_eval_masked(int32_t dtype, int32_t degree, int64_t batch, int32_t F, int32_t E, const void *coeff, const void *t0, const void *t1,
-                          const void *t_eval, const uint8_t *mask, void *ys, void *stream) {
+int tode_poly_eval_masked(int32_t dtype, int32_t degree, int32_t span_is_dt, int64_t batch, int32_t F, int32_t E, const void *coeff, const void *t0,
+                          const void *t1, const void *t_eval, const uint8_t *mask, void *ys, void *stream) {
     if (int rc = check_common(dtype, batch, F)) return rc;
     if (degree < 1 || degree > 4) return fail(TODE_E_INVALID, "degree %d outside 1..4", degree);
     if (E < 0) return fail(TODE_E_INVALID, "negative n_eval");
@@ -811,10 +811,10 @@ int tode_poly_eval_masked(int32_t dtype, int32_t degree, int64_t batch, int32_t 
     hipStream_t s = (hipStream_t)stream;
     TODE_TT(dtype, {
         if (F < 64)
-            hipLaunchKernelGGL((poly_eval_masked_thread_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, degree, (long long)batch, F, E,
+            hipLaunchKernelGGL((poly_eval_masked_thread_kernel<TT, T>), dim3(blocks_for(batch, 256)), dim3(256), 0, s, degree, span_is_dt != 0, (long long)batch, F, E,
                                (const T *)coeff, (const TT *)t0, (const TT *)t1, (const TT *)t_eval, mask, (T *)ys);
         else
-            hipLaunchKernelGGL((poly_eval_masked_block_kernel<TT, T>), dim3((unsigned)batch), dim3(256), 0, s, degree, (long long)batch, F, E, (const T *)coeff,
+            hipLaunchKernelGGL((poly_eval_masked_block_kernel<TT, T>), dim3((unsigned)batch), dim3(256), 0, s, degree, span_is_dt != 0, (long long)batch, F, E, (const T *)coeff,
                                (const TT *)t0, (const TT *)t1, (const TT *)t_eval, mask, (T *)ys);
     });
     return done("tode_poly_eval_masked launch");

@@ -297,6 +297,7 @@ static int launch_pair(const tode_solve_args &a, const tode_controller &c, const
     const bool stage_te = rec_bytes + te_bytes <= budget;
     const size_t lds = rec_bytes + (stage_te ? te_bytes : 0);
     SolveParams<T> p = make_params<T>(a, c);
+    if (p.cp.shortcut_exponent()) return TODE_OK;  // left to the caller's other kernels
     const int nhist = CTRL == 0 ? 0 : (p.cp.skip3 ? 1 : 2);
     const dim3 grid((unsigned)blocks), block(128);
     reset_flags(a.flags, stream);

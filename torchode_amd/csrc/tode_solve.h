@@ -160,11 +160,11 @@ __device__ __forceinline__ int searchsorted_first_pending(const uint8_t *pending
 }
 
 // x = (t - t0) / (t1 - t0) with a zero interval mapped to 1 (interpolation.py:8-40)
-template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) {
-    T den = t1 - t0;
+template <typename T> __device__ __forceinline__ T unit_time_over(T t, T t0, T den) {
     if (!(abs_(den) > (T)0)) den = (T)1;
     return (t - t0) / den;
 }
+template <typename T> __device__ __forceinline__ T unit_time(T t, T t0, T t1) { return unit_time_over(t, t0, t1 - t0); }
 
 template <typename T> __device__ __forceinline__ T horner(const T *coeff, long long bf, long long at, int degree, T x) {
     T y = coeff[degree * bf + at];

@@ -29,6 +29,7 @@ class _PolynomialInterpolation(LocalInterpolation):
     """Polynomial on [t0, t1] in x = (t - t0) / (t1 - t0); ``coefficients[i]`` belongs to x**i."""
 
     degree = -1
+    span_is_dt = 0  # 1: the second time operand is the step size and divides as it stands
 
     def __init__(self, t0: torch.Tensor, t1: torch.Tensor, coefficients):
         self.t0 = t0
@@ -36,6 +37,9 @@ class _PolynomialInterpolation(LocalInterpolation):
         self._coeff = _stack(coefficients)
         assert self._coeff.ndim == 3 and self._coeff.shape[0] == self.degree + 1
         self.coefficients = tuple(self._coeff.unbind(0))
+
+    def _span(self) -> torch.Tensor:
+        return self.t1
 
     def _code(self, *times) -> int:
         c = self._coeff
@@ -49,10 +53,10 @@ class _PolynomialInterpolation(LocalInterpolation):
         c = self._coeff
         _, B, F = c.shape
         t, idx = t.contiguous(), idx.to(torch.long).contiguous()
-        t0, t1 = self.t0.contiguous(), self.t1.contiguous()
+        t0, t1 = self.t0.contiguous(), self._span().contiguous()
         out = c.new_empty((t.shape[0], F))
         rc = _lib.load().tode_poly_eval(
-            code, self.degree, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
+            code, self.degree, self.span_is_dt, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
             _lib.ptr(idx), _lib.ptr(out), _lib.stream_of(c),
         )  # fmt: skip
         _lib.check(rc, "tode_poly_eval")
@@ -65,9 +69,9 @@ class _PolynomialInterpolation(LocalInterpolation):
         c = self._coeff
         _, B, F = c.shape
         assert t_eval.is_contiguous() and mask.is_contiguous() and ys.is_contiguous() and mask.element_size() == 1
-        t0, t1 = self.t0.contiguous(), self.t1.contiguous()
+        t0, t1 = self.t0.contiguous(), self._span().contiguous()
         rc = _lib.load().tode_poly_eval_masked(
-            code, self.degree, B, F, t_eval.shape[1], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1),
+            code, self.degree, self.span_is_dt, B, F, t_eval.shape[1], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1),
             _lib.ptr(t_eval), _lib.ptr(mask), _lib.ptr(ys), _lib.stream_of(c),
         )  # fmt: skip
         _lib.check(rc, "tode_poly_eval_masked")
@@ -84,15 +88,20 @@ def _build_args(dt, y0, y1, *more):
 
 
 class LinearInterpolation(_PolynomialInterpolation):
-    """y0 + (y1 - y0) x (reference interpolation.py:48-62; x is taken over (t0 + dt) - t0)."""
+    """y0 + (y1 - y0) x with x = (t - t0) / dt: the step size itself divides, not (t0 + dt) - t0, which can differ
+    from it in the last bit (reference interpolation.py:48-62)."""
 
     degree = 1
+    span_is_dt = 1
 
     def __init__(self, t0: torch.Tensor, dt: torch.Tensor, y0: torch.Tensor, y1: torch.Tensor):
-        super().__init__(t0, t0 + dt, (y0, y1 - y0))  # x is taken over (t0 + dt) - t0
         self.dt = dt
+        super().__init__(t0, t0 + dt, (y0, y1 - y0))
         self.y0 = y0
         self.dy = self.coefficients[1]
+
+    def _span(self) -> torch.Tensor:
+        return self.dt
 
 
 class ThirdOrderPolynomialInterpolation(_PolynomialInterpolation):
