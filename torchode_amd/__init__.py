@@ -2,42 +2,27 @@
 
 __version__ = "0.1.0"
 
-from . import builtin_terms, workloads
+# the solve loop and its gradients
 from .adjoints import AutoDiffAdjoint
 from .backsolve import BacksolveAdjoint, JointBacksolveAdjoint
-from .builtin_terms import LinearDecay, Lorenz63, MLPField, ReactionDiffusion, VanDerPol
+
+# what a solve is made of: problem, right-hand side, step method, step size controller; what it returns
 from .problems import InitialValueProblem
-from .interface import register_method, solve_ivp
+from .terms import ODETerm
 from .single_step_methods import Dopri5, Euler, Heun, Tsit5
+from .step_size_controllers import FixedStepController, IntegralController, PIDController
 from .solution import Solution
 from .status_codes import Status
-from .step_size_controllers import FixedStepController, IntegralController, PIDController
-from .terms import ODETerm
 
-register_method("heun", Heun)
-register_method("dopri5", Dopri5)
-register_method("tsit5", Tsit5)
+# right-hand sides the whole-solve kernels know, and the benchmark workloads built from them
+from . import builtin_terms, workloads
+from .builtin_terms import LinearDecay, Lorenz63, MLPField, ReactionDiffusion, VanDerPol
 
-__all__ = [
-    "AutoDiffAdjoint",
-    "BacksolveAdjoint",
-    "JointBacksolveAdjoint",
-    "InitialValueProblem",
-    "register_method",
-    "solve_ivp",
-    "Dopri5",
-    "Euler",
-    "Heun",
-    "Tsit5",
-    "Solution",
-    "Status",
-    "FixedStepController",
-    "IntegralController",
-    "PIDController",
-    "ODETerm",
-    "LinearDecay",
-    "VanDerPol",
-    "Lorenz63",
-    "ReactionDiffusion",
-    "MLPField",
-]
+# the one-call interface and its method names (the reference registers these three)
+from .interface import register_method, solve_ivp
+
+for _name, _method in (("dopri5", Dopri5), ("tsit5", Tsit5), ("heun", Heun)):
+    register_method(_name, _method)
+del _name, _method
+
+__all__ = [name for name, value in list(globals().items()) if not name.startswith("_") and (isinstance(value, type) or name in ("solve_ivp", "register_method"))]

@@ -24,6 +24,12 @@ def _per_sample(t: torch.Tensor, batch_size: int) -> torch.Tensor:
     return t.expand(batch_size) if t.ndim == 0 else t
 
 
+def _time_range(t_span, t_eval, batch_size: int):
+    """``(t_start, t_end)`` as ``[B]`` each: the given span, else the first and last evaluation time."""
+    t_start, t_end = t_span if t_span is not None else (t_eval[:, 0], t_eval[:, -1])
+    return _per_sample(t_start, batch_size), _per_sample(t_end, batch_size)
+
+
 def solve_ivp(
     f: Union[ODETerm, Callable],
     y0: torch.Tensor,
@@ -42,14 +48,14 @@ def solve_ivp(
     ``t_eval`` is ``[B, E]`` or ``[E]`` (shared by the batch); ``t_span`` defaults to the first and
     last evaluation time; ``method`` is a registered name or a step method object; the default
     controller is ``PIDController(atol=1e-7, rtol=1e-7, pcoeff=0.2, icoeff=0.5, dcoeff=0.0)``."""
-    term = f if isinstance(f, ODETerm) else ODETerm(f, with_args=args is not None)
-    step_method = method if isinstance(method, SingleStepMethod) else METHODS[method](term=term)
-    step_size_controller = controller if controller is not None else PIDController(term=term, **DEFAULT_TOLERANCES)
-
     batch_size = y0.shape[0]
     if t_eval is not None and t_eval.ndim == 1:
         t_eval = t_eval.expand((batch_size, -1))
-    t_start, t_end = t_span if t_span is not None else (t_eval[:, 0], t_eval[:, -1])
-    problem = InitialValueProblem(y0, _per_sample(t_start, batch_size), _per_sample(t_end, batch_size), t_eval)
-    solver = AutoDiffAdjoint(step_method, step_size_controller, max_steps=max_steps)
-    return solver.solve(problem, term, dt0=dt0, args=args)
+    problem = InitialValueProblem(y0, *_time_range(t_span, t_eval, batch_size), t_eval)
+
+    term = f if isinstance(f, ODETerm) else ODETerm(f, with_args=args is not None)
+    if isinstance(method, str):
+        method = METHODS[method](term=term)
+    if controller is None:
+        controller = PIDController(term=term, **DEFAULT_TOLERANCES)
+    return AutoDiffAdjoint(method, controller, max_steps=max_steps).solve(problem, term, dt0=dt0, args=args)
