@@ -541,6 +541,48 @@ def test_zero_length_step_does_not_produce_nan():
     assert not torch.isnan(FourthOrderPolynomialInterpolation(t0, t0, torch.rand((5, 1, 2), device=DEV)).evaluate(t0, idx)).any()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+def test_interpolants_match_the_reference_formulas_as_cpu_ops_bit_for_bit(dtype):
+    """Linear, cubic and quartic interpolants against the reference's formulas run as ATen CPU elementwise
+    operations (oracle/torch_loop.py, interpolation.py:8-40, 48-60, 84-106): plain vector operations without matrix
+    products, the same on every host, on whole 32-value vector bodies.  Step sizes are picked so that
+    ``(t0 + dt) - t0 != dt`` for most samples: the linear interpolant divides by ``dt``, the cubic and the quartic by
+    the rounded difference."""
+    from oracle import torch_loop as tl
+
+    g = torch.Generator().manual_seed(11)
+    B, F, N = 64, 4, 256
+    t0 = torch.rand(B, dtype=dtype, generator=g) * 10 + 1
+    dt = (torch.rand(B, dtype=dtype, generator=g) - 0.5) * 1e-2
+    assert ((t0 + dt) - t0 != dt).float().mean() > 0.5
+    y0, y1 = torch.randn(B, F, dtype=dtype, generator=g), torch.randn(B, F, dtype=dtype, generator=g)
+    k = torch.randn(2, B, F, dtype=dtype, generator=g)
+    idx = torch.randint(0, B, (N,), generator=g)
+    t = t0[idx] + torch.rand(N, dtype=dtype, generator=g) * dt[idx]
+    d = lambda x: x.to(DEV)
+
+    got = LinearInterpolation(d(t0), d(dt), d(y0), d(y1)).evaluate(d(t), d(idx)).cpu()
+    assert torch.equal(got, tl.linear_eval(t0, dt, y0, y1, t, idx))
+
+    cubic = ThirdOrderPolynomialInterpolation.from_k(d(t0), d(dt), d(y0), d(y1), d(k))
+    want = tl.cubic_from_k(dt, y0, y1, k)
+    for mine, theirs in zip(cubic.coefficients, want):
+        assert torch.equal(mine.cpu(), theirs)
+    assert torch.equal(cubic.evaluate(d(t), d(idx)).cpu(), tl.cubic_eval(want, t0, t0 + dt, t, idx))
+
+    coeff = torch.randn(5, B, F, dtype=dtype, generator=g)
+    quartic = FourthOrderPolynomialInterpolation(d(t0), d(t0 + dt), d(coeff))
+    assert torch.equal(quartic.evaluate(d(t), d(idx)).cpu(), tl.quartic_eval(tuple(coeff.unbind(0)), t0, t0 + dt, t, idx))
+
+    # the masked form used by the loop: one sample's evaluation points, selected by a byte mask
+    t_eval = t0[:, None] + torch.rand(B, 8, dtype=dtype, generator=g) * dt[:, None]
+    mask = torch.rand(B, 8, generator=g) < 0.5
+    ys = torch.zeros(B, 8, F, dtype=dtype, device=DEV)
+    LinearInterpolation(d(t0), d(dt), d(y0), d(y1)).evaluate_masked(d(t_eval), d(mask.to(torch.uint8)), ys)
+    rows, cols = mask.nonzero(as_tuple=True)
+    assert torch.equal(ys.cpu()[rows, cols], tl.linear_eval(t0, dt, y0, y1, t_eval[rows, cols], rows)) and (ys.cpu()[~mask] == 0).all()
+
+
 def test_cubic_and_quartic_from_stage_derivatives_recover_the_polynomial():
     P = np.polynomial.Polynomial
     t0, dt = np.array([0.3]), np.array([1.9])
