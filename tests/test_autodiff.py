@@ -60,7 +60,7 @@ def drive(replay: Replay, y0, dt0=None):
     n_steps, n_acc = torch.zeros(B, dtype=torch.long), torch.zeros(B, dtype=torch.long)
     while True:
         attempt = replay.attempt(state)
-        accept = attempt[2] < 1
+        accept = attempt[2] < 1 if attempt[2] is not None else torch.ones(B, dtype=torch.bool)  # (no error estimate, or fixed steps)
         move = accept & state["running"]
         t_new = torch.where(move, state["t"] + state["dt"], state["t"])
         running_new = direction * t_new < direction * t_end
@@ -95,6 +95,34 @@ def test_restated_iteration_reproduces_the_oracle_loop(method, ctrl):
     ref = torch_loop.solve(w.f, w.y0, w.t_eval, method=method, controller=torch_loop.Controller(**ctrl), t_start=problem.t_start, t_end=problem.t_end)
     assert torch.equal(n_steps, ref["n_steps"]) and torch.equal(n_acc, ref["n_accepted"]) and (n_acc < n_steps).any()
     torch.testing.assert_close(ys, ref["ys"], rtol=1e-7, atol=1e-8)  # same operations, other association: rounding differences grow along stiff samples
+
+
+@pytest.mark.parametrize("method,ctrl,first_step", [
+    ("heun", dict(kind="pid", atol=1e-6, rtol=1e-4, pcoeff=0.2, icoeff=0.5, dcoeff=0.1), None),
+    ("heun", dict(kind="integral", atol=1e-6, rtol=1e-4), 300.0),
+    ("heun", dict(kind="fixed", atol=0.0, rtol=0.0), 400.0),
+    ("euler", dict(kind="fixed", atol=0.0, rtol=0.0), 500.0),
+    ("euler", dict(kind="integral", atol=1e-6, rtol=1e-4), 450.0),
+])  # fmt: skip
+def test_restated_iteration_reproduces_the_oracle_loop_with_heun_and_euler(method, ctrl, first_step):
+    """A tableau that is neither first-same-as-last nor solution-same-as-last, the Hermite cubic and the linear
+    interpolant, no error estimate (Euler) and fixed steps, against oracle/torch_loop.py::solve_low_order."""
+    w = to.workloads.make("vdp", batch=40, dtype=torch.float64)
+    w.t_eval[3, 0] = 0.25
+    spec = dict(ctrl)
+    kind = spec.pop("kind")
+    controller = {"pid": to.PIDController, "integral": to.IntegralController}[kind](**spec) if kind != "fixed" else to.FixedStepController()
+    t_start = torch.zeros(40, dtype=torch.float64)
+    dt0 = None if first_step is None else (w.t_eval[:, -1] - t_start) / (first_step + torch.arange(40, dtype=torch.float64) % 7)
+    problem = to.InitialValueProblem(w.y0, t_start=t_start, t_end=w.t_eval[:, -1], t_eval=w.t_eval)
+    step_method = to.Heun() if method == "heun" else to.Euler()
+    replay = Replay(step_method, controller, to.ODETerm(w.f), None, problem, True, dt0)
+    with torch.no_grad():
+        ys, n_steps, n_acc = drive(replay, w.y0, dt0)
+    ref = torch_loop.solve_low_order(w.f, w.y0, w.t_eval, method=method, controller=torch_loop.Controller(**ctrl), t_start=t_start, t_end=problem.t_end, dt0=dt0)
+    assert torch.equal(n_steps, ref["n_steps"]) and torch.equal(n_acc, ref["n_accepted"])
+    assert (n_acc < n_steps).any() == (method == "heun" and kind != "fixed")
+    torch.testing.assert_close(ys, ref["ys"], rtol=1e-7, atol=1e-8)
 
 
 def test_recorded_times_give_back_the_evaluation_schedule():
@@ -336,11 +364,41 @@ def test_gradcheck_with_respect_to_the_times_and_the_first_step():
 
 
 @gpu
+@pytest.mark.parametrize("case", ["heun-pid", "heun-integral-end-only", "heun-fixed", "euler-fixed", "euler-integral"])
+def test_gradcheck_through_heun_and_euler(case):
+    """The loop recorded on the operator path (a tableau without first-same-as-last slope, cubic and linear dense
+    output, no error estimate for Euler): y0, the term's parameters, the evaluation times and the first step."""
+    y0, A = inputs()
+    method, kind = case.split("-")[0], case.split("-")[1]
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
+    dt0 = torch.tensor([0.031, 0.047], dtype=torch.double, device="cuda", requires_grad=True)
+
+    def loss(y0, params, t_eval, dt0):
+        term = to.ODETerm(LinearDynamics(params))
+        controller = {"pid": lambda: to.PIDController(1e-4, 0.0, 0.3, 0.6, 0.0), "integral": lambda: to.IntegralController(1e-4, 1e-4),
+                      "fixed": to.FixedStepController}[kind]()  # fmt: skip
+        adjoint = to.AutoDiffAdjoint(to.Heun() if method == "heun" else to.Euler(), controller)
+        if case.endswith("end-only"):
+            problem = to.InitialValueProblem(y0, t_start=t_eval[:, 0], t_end=t_eval[:, -1])
+        else:
+            problem = to.InitialValueProblem(y0, t_eval=t_eval)
+        first = dt0 if kind == "fixed" or method == "euler" else None  # (the adaptive Heun cases choose their own)
+        sol = adjoint.solve(problem, term=term, dt0=first)
+        assert (sol.status == 0).all() and int(sol.stats["n_steps"].max()) > 20
+        return sol.ys.mean()
+
+    assert torch.autograd.gradcheck(loss, (y0, A, t_eval, dt0), atol=1e-5, check_undefined_grad=False)
+
+
+@gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))
     t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
+    class OwnHeun(to.Heun):  # a user's subclass: its protocol methods may do anything
+        pass
+
     with pytest.raises(RuntimeError, match="BacksolveAdjoint"):
-        to.AutoDiffAdjoint(to.Heun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
+        to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
     with torch.no_grad():  # no graph asked for: any configuration solves
-        to.AutoDiffAdjoint(to.Heun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
+        to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)

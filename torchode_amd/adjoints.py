@@ -8,7 +8,7 @@ from . import _lib
 from .builtin_terms import BuiltinTerm
 from .problems import InitialValueProblem
 from .interpolation import _PolynomialInterpolation
-from .single_step_methods import Dopri5, Tsit5
+from .single_step_methods import Dopri5, Euler, Heun, Tsit5
 from .solution import Solution
 from .step_size_controllers import FixedStepController, IntegralController, PIDController
 from .terms import ODETerm
@@ -48,7 +48,7 @@ class AutoDiffAdjoint(nn.Module):
 
     Same constructor and ``solve`` signature as the reference.  The solve runs in HIP kernels.
     When ``y0``, a parameter of the term, a tensor in ``args`` or one of the times requires grad it
-    takes the per-step kernels and records the loop state per iteration, and the result is
+    takes the per-step kernels (Heun, Euler: the operator path) and records the loop state per iteration, and the result is
     differentiable (``torchode_amd/autodiff.py``; ``backprop_through_step_size_control`` as in the
     reference).
     """
@@ -109,11 +109,11 @@ class AutoDiffAdjoint(nn.Module):
 
             wants_grad = any(a.requires_grad for a in tensor_leaves(args))
         if wants_grad:
-            # gradients through the loop: forward in the per-step kernels with a record of the loop
-            # state, backward by a reverse sweep over the record
-            if not self._fused_ok(problem, term_):
+            # gradients through the loop: forward in the per-step kernels (Dopri5, Tsit5) or on the operator
+            # path (Heun, Euler) with a record of the loop state, backward by a reverse sweep over the record
+            if not self._library_setup(problem, term_, (Dopri5, Tsit5, Heun, Euler)):
                 raise RuntimeError(
-                    "gradients through the loop are built for Dopri5 / Tsit5 with the library's controllers; "
+                    "gradients through the loop are built for the library's step methods and controllers; "
                     "with user-defined plug-ins call solve under torch.no_grad(), or use BacksolveAdjoint"
                 )
             from . import autodiff
@@ -125,9 +125,14 @@ class AutoDiffAdjoint(nn.Module):
 
     # ------------------------------------------------------------------ #
     def _fused_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
+        return self._library_setup(problem, term, (Dopri5, Tsit5))
+
+    def _library_setup(self, problem: InitialValueProblem, term: ODETerm, methods) -> bool:
+        """One of ``methods`` and a controller as the library ships them (no overridden protocol method, the RMS
+        norm), a plain term, float32 / float64 tensors."""
         m, c = self.step_method, self.step_size_controller
         return (
-            _library_object(m, (Dopri5, Tsit5))
+            _library_object(m, methods)
             and _library_object(c, (IntegralController, PIDController, FixedStepController))
             and c.fusable
             and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
@@ -154,7 +159,7 @@ class AutoDiffAdjoint(nn.Module):
         return self._fused_ok(problem, term)
 
     # ------------------------------------------------------------------ #
-    def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args) -> Solution:
+    def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args, record=None) -> Solution:
         """The loop of the reference (adjoints.py:50-311) against the plug-in protocols: any step
         method, controller and interpolant, the library's or the user's.  The protocol methods are
         called in the reference's order with the reference's arguments; the bookkeeping between them
@@ -209,6 +214,8 @@ class AutoDiffAdjoint(nn.Module):
         a.flags = flags.data_ptr()
 
         while True:
+            if record is not None:
+                record.snapshot_protocol(t, dt, y, controller_state, running, n_accepted)
             step_result, interp_data, method_state_next, method_status = method.step(
                 term, running, y, t, dt, method_state, stats=stats, args=args
             )
@@ -253,6 +260,9 @@ class AutoDiffAdjoint(nn.Module):
             if fl[_lib.LOOP_ANY_RUNNING] and not fl[_lib.LOOP_ANY_FAILURE]:
                 continue
 
+            if record is not None:
+                record.snapshot_protocol(t, dt, y, controller_state, running, n_accepted)
+                record.iterations = len(record.states) - 1
             if m_status is None and c_status is None and self.max_steps is None:
                 status = torch.tensor(0, dtype=torch.long, device=dev).expand(B)
             stats["n_steps"], stats["n_accepted"] = n_steps, n_accepted

@@ -2,7 +2,8 @@
 reference records every torch operation of its loop; ``backprop_through_step_size_control``
 decides whether the step sizes count as functions of the inputs).
 
-Here the forward pass runs in the per-step HIP kernels and keeps, per loop iteration, a copy of
+Here the forward pass runs in the per-step HIP kernels (Dopri5, Tsit5) or on the operator path
+(Heun, Euler) and keeps, per loop iteration, a copy of
 the small loop state (t, dt, y, the FSAL derivative, the controller history, two counters).  The
 backward pass walks the iterations in reverse: it restates one iteration as differentiable torch
 operations on the stored state -- same stages, error ratio, step size rule and dense output, with
@@ -24,6 +25,7 @@ import torch
 
 from . import _lib
 from .problems import InitialValueProblem
+from .single_step_methods import Euler, Heun
 
 
 def tensor_leaves(obj) -> List[torch.Tensor]:
@@ -62,6 +64,14 @@ class LoopRecord:
     def snapshot(self, t, dt, y, k0, hist, ints):
         self.states.append((t.clone(), dt.clone(), y.clone(), k0.clone(), hist[0].clone(), hist[1].clone(), ints[0].clone(), ints[3].clone()))
 
+    def snapshot_protocol(self, t, dt, y, controller_state, running, n_accepted):
+        """The same record from the operator path: a method without a first-same-as-last slope has nothing to carry
+        (zeros stand in), and only the PID controller carries error ratios."""
+        ones = torch.ones_like(y[:, 0])
+        prev = getattr(controller_state, "prev_error_ratio", ones)
+        pprev = getattr(controller_state, "prev_prev_error_ratio", ones)
+        self.states.append((t.clone(), dt.clone(), y.clone(), torch.zeros_like(y), prev.clone(), pprev.clone(), running.clone(), n_accepted.clone()))
+
     def trimmed(self, iterations: int) -> List[dict]:
         """States 0..iterations; iterations enqueued after the batch had stopped changed nothing."""
         states = self.states[:iterations] + [self.states[-1]]
@@ -72,17 +82,28 @@ class Replay:
     """One loop iteration (and the start of the loop) as differentiable torch operations."""
 
     def __init__(self, method, controller, term, args, problem: InitialValueProblem, through_control: bool, dt0=None):
-        tab = method.tableau
-        self.a = [[float(x) for x in row] for row in tab.a.tolist()]
-        self.c = [float(x) for x in tab.c.tolist()]
-        self.b_err = [float(x) for x in tab.b_err.tolist()]
-        self.b_other = [[float(x) for x in row] for row in tab.b_other.tolist()]
-        self.tsit5 = method.method_id == _lib.TSIT5
+        if isinstance(method, Euler):  # (reference euler.py:29-56: one slope, no error estimate, linear dense output)
+            self.a, self.c, self.b, self.b_err = [[]], [0.0], [1.0], None
+            self.fsal = self.ssal = False
+            self.dense_kind = "linear"
+        else:
+            tab = method.tableau
+            self.a = [[float(x) for x in row] for row in tab.a.tolist()]
+            self.c = [float(x) for x in tab.c.tolist()]
+            self.b = [float(x) for x in tab.b.tolist()]
+            self.b_err = [float(x) for x in tab.b_err.tolist()]
+            self.fsal, self.ssal = bool(tab.fsal), bool(tab.ssal)
+            if isinstance(method, Heun):
+                self.dense_kind = "cubic"
+            else:
+                self.b_other = [[float(x) for x in row] for row in tab.b_other.tolist()]
+                self.dense_kind = "tsit5" if method.method_id == _lib.TSIT5 else "dopri5"
+        self.n_stages = len(self.c)
         self.order = float(method.convergence_order())
         c = controller.c_struct()
         self.pid = c.kind == _lib.CTRL_PID
         # fixed steps (reference step_size_controllers.py:116-167): every step accepted, the next step is dt0 again
-        self.fixed_dt = dt0.detach().to(problem.t_start.dtype) if c.kind == _lib.CTRL_FIXED else None
+        self.fixed, self.dt0 = c.kind == _lib.CTRL_FIXED, dt0
         self.atol, self.rtol = float(c.atol), float(c.rtol)
         self.safety, self.fmin, self.fmax = float(c.safety), float(c.factor_min), float(c.factor_max)
         self.dt_min = float(c.dt_min) if c.has_dt_min else None
@@ -99,6 +120,15 @@ class Replay:
 
     # the ends of the time range are functions of t_start and t_end: formed where they are used, so that every
     # iteration of the reverse sweep differentiates a graph of its own
+    @property
+    def fixed_dt(self):
+        """The step a fixed-step controller hands back every time: the user's ``dt0`` itself, so with
+        ``through_control`` its gradient collects a share from every step."""
+        if not self.fixed:
+            return None
+        dt = self.dt0.to(self.t_start.dtype)
+        return dt if self.through_control else dt.detach()
+
     @property
     def t_lo(self):
         return torch.minimum(self.t_start, self.t_end)
@@ -136,16 +166,19 @@ class Replay:
         and the step size it proposes."""
         t, dt, y, k0, prev, pprev = (state[k] for k in ("t", "dt", "y", "k0", "prev", "pprev"))
         dtd = dt.to(y.dtype)
-        ks = [k0]
+        S = self.n_stages
+        ks = [k0 if self.fsal else self.f(t, y)]
         yi = y
-        for i in range(1, 7):
+        for i in range(1, S):
             s = sum(self.a[i][j] * ks[j] for j in range(i) if self.a[i][j] != 0.0)
             yi = y + dtd[:, None] * s
             ks.append(self.f(t + self.c[i] * dt, yi))
-        y1 = yi
+        y1 = yi if self.ssal else y + dtd[:, None] * sum(self.b[s] * ks[s] for s in range(S) if self.b[s] != 0.0)
         if self.fixed_dt is not None:
-            return ks, y1, torch.zeros_like(dtd), self.fixed_dt
-        err = dtd[:, None] * sum(self.b_err[s] * ks[s] for s in range(7) if self.b_err[s] != 0.0)
+            return ks, y1, None, self.fixed_dt
+        if self.b_err is None:  # no error estimate: the controllers accept and keep the step size
+            return ks, y1, None, dt
+        err = dtd[:, None] * sum(self.b_err[s] * ks[s] for s in range(S) if self.b_err[s] != 0.0)
         scale = self.atol + self.rtol * torch.maximum(y.abs(), y1.abs())
         ratio = torch.clamp_min(self.rms(err.abs() / scale), 1e-38)
         factor = self.safety * ratio**self.e1
@@ -168,12 +201,13 @@ class Replay:
         ks, y1, ratio, dt_next = attempt
         move = accept & running
         y_new = torch.where(move[:, None], y1, y)
-        k0_new = torch.where(move[:, None], ks[6], k0)
+        k0_new = torch.where(move[:, None], ks[-1], k0) if self.fsal else k0
         t_new = torch.where(move, t + dt, t)
         dt_new = torch.where(running_new, dt_next, dt)
         dt_new = torch.minimum(torch.maximum(dt_new, self.t_lo - t_new), self.t_hi - t_new)
         keep = running_new & accept
-        prev_new, pprev_new = (torch.where(keep, ratio, prev), torch.where(keep, prev, pprev)) if self.pid else (prev, pprev)
+        shift = self.pid and ratio is not None
+        prev_new, pprev_new = (torch.where(keep, ratio, prev), torch.where(keep, prev, pprev)) if shift else (prev, pprev)
 
         values = None
         if hits is not None:
@@ -188,8 +222,14 @@ class Replay:
     # ---- reference tsit5.py:123-139, dopri5.py:53-60, interpolation.py:25-40, 138-170 ----
     def dense(self, t0, dt, y0, y1, ks, at):
         h = dt.to(y0.dtype)[:, None]
+        if self.dense_kind == "linear":  # reference interpolation.py:48-60: the step size itself divides
+            den = torch.where(dt.abs() > 0, dt, torch.ones_like(dt))
+            return y0 + (y1 - y0) * ((at - t0) / den).to(y0.dtype)[:, None]
         weighted = lambda w: h * sum(w[s] * ks[s] for s in range(7) if w[s] != 0.0)
-        if self.tsit5:
+        if self.dense_kind == "cubic":  # Hermite cubic from the first and last slope, reference interpolation.py:84-106
+            f0, f1, gap = ks[0], ks[-1], y0 - y1
+            q = [y0, h * f0, h * (-2 * f0 - f1) - 3 * gap, h * (f0 + f1) + 2 * gap]
+        elif self.dense_kind == "tsit5":
             q = [y0, h * ks[0], weighted(self.b_other[0]), weighted(self.b_other[1]), weighted(self.b_other[2])]
         else:
             f0, f1, mid = h * ks[0], h * ks[6], y0 + weighted(self.b_other[0])
@@ -203,8 +243,8 @@ class Replay:
         den = (t0 + dt) - t0
         den = torch.where(den.abs() > 0, den, torch.ones_like(den))
         x = ((at - t0) / den).to(y0.dtype)[:, None]
-        out = q[4]
-        for p in (3, 2, 1, 0):
+        out = q[-1]
+        for p in range(len(q) - 2, -1, -1):
             out = out * x + q[p]
         return out
 
@@ -237,7 +277,10 @@ class SolveThroughLoop(torch.autograd.Function):
         detached = lambda x: None if x is None else x.detach()
         plain = InitialValueProblem(y0.detach(), detached(problem.t_start), detached(problem.t_end), detached(problem.t_eval))
         with torch.no_grad():
-            solution = adjoint._solve_stepwise(plain, term, detached(dt0), args, record=record)
+            if adjoint._fused_ok(plain, term):
+                solution = adjoint._solve_stepwise(plain, term, detached(dt0), args, record=record)
+            else:  # Heun, Euler: the operator path keeps the record
+                solution = adjoint._solve_protocol(plain, term, term, detached(dt0), args, record=record)
         ctx.adjoint, ctx.problem, ctx.term, ctx.dt0, ctx.args = adjoint, plain, term, dt0, args
         # the times as the caller gave them: those that require grad are among `params`
         ctx.times = InitialValueProblem(plain.y0, problem.t_start, problem.t_end, problem.t_eval)
