@@ -245,3 +245,16 @@ def test_low_order_fixture_is_well_formed(path):
         assert g["n_steps"] == g["n_accepted"]  # nothing to reject without an error estimate or with fixed steps
     else:
         assert all(a <= n for a, n in zip(g["n_accepted"], g["n_steps"]))
+
+
+def test_names_the_reference_keeps_in_its_adjoints_and_interpolation_modules():
+    """``from torchode.adjoints import BacksolveAdjoint`` and the like keep working after the switch (reference
+    adjoints.py:15, 322, 510; interpolation.py:8, 25)."""
+    from torchode_amd import adjoints, backsolve, interpolation
+
+    assert adjoints.BacksolveAdjoint is backsolve.BacksolveAdjoint and adjoints.JointBacksolveAdjoint is backsolve.JointBacksolveAdjoint
+    assert callable(interpolation.poly3eval) and callable(interpolation.poly4eval)
+    with pytest.raises(NotImplementedError):
+        adjoints.Adjoint().solve(None)
+    with pytest.raises(AttributeError):
+        adjoints.no_such_name

@@ -583,6 +583,26 @@ def test_interpolants_match_the_reference_formulas_as_cpu_ops_bit_for_bit(dtype)
     assert torch.equal(ys.cpu()[rows, cols], tl.linear_eval(t0, dt, y0, y1, t_eval[rows, cols], rows)) and (ys.cpu()[~mask] == 0).all()
 
 
+def test_poly3eval_and_poly4eval_row_by_row():
+    """The reference's free functions (interpolation.py:8-40): coefficient rows already gathered per evaluation time."""
+    from oracle import torch_loop as tl
+    from torchode_amd.interpolation import poly3eval, poly4eval
+
+    g = torch.Generator().manual_seed(12)
+    N, F = 96, 3
+    coeff = torch.randn(5, N, F, dtype=torch.float64, generator=g)
+    t0 = torch.rand(N, dtype=torch.float64, generator=g)
+    t1 = t0 + torch.rand(N, dtype=torch.float64, generator=g) * 0.1
+    t1[:4] = t0[:4]  # an empty interval divides by one
+    t = t0 + torch.rand(N, dtype=torch.float64, generator=g) * (t1 - t0)
+    d = lambda x: x.to(DEV)
+    rows = torch.arange(N)
+    got = poly4eval(*(d(c) for c in coeff), d(t), d(t0), d(t1)).cpu()
+    assert torch.equal(got, tl.quartic_eval(tuple(coeff.unbind(0)), t0, t1, t, rows))
+    got = poly3eval(*(d(c) for c in coeff[:4]), d(t), d(t0), d(t1)).cpu()
+    assert torch.equal(got, tl.cubic_eval(tuple(coeff[:4].unbind(0)), t0, t1, t, rows))
+
+
 def test_cubic_and_quartic_from_stage_derivatives_recover_the_polynomial():
     P = np.polynomial.Polynomial
     t0, dt = np.array([0.3]), np.array([1.9])

@@ -43,6 +43,22 @@ def _library_object(obj, classes) -> bool:
     return type(obj) in classes and _PROTOCOL_NAME_SET.isdisjoint(vars(obj))
 
 
+class Adjoint:
+    """What every adjoint offers (reference adjoints.py:15-23)."""
+
+    def solve(self, problem: InitialValueProblem, term: Optional[ODETerm] = None, dt0: Optional[torch.Tensor] = None, args: Any = None) -> Solution:
+        raise NotImplementedError()
+
+
+def __getattr__(name):
+    # the reference keeps its backsolve adjoints in this module; here they have one of their own, which imports this one
+    if name in ("BacksolveAdjoint", "JointBacksolveAdjoint"):
+        from . import backsolve
+
+        return getattr(backsolve, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+
+
 class AutoDiffAdjoint(nn.Module):
     """Solves a batch of initial value problems with per-sample adaptive steps.
 

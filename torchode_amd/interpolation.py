@@ -12,6 +12,22 @@ import torch
 from . import _lib
 
 
+def _poly_eval_rows(coefficients, t, t0, t1):
+    """Row n of the coefficient tensors belongs to time ``t[n]`` on ``[t0[n], t1[n]]``."""
+    rows = torch.arange(t.shape[0], device=t.device)
+    return _PolynomialInterpolation._make(len(coefficients) - 1, t0, t1, coefficients).evaluate(t, rows)
+
+
+def poly3eval(d, c, b, a, t, t0, t1):
+    """``d + c x + b x^2 + a x^3`` with ``x = (t - t0) / (t1 - t0)``, row by row (reference interpolation.py:8-22)."""
+    return _poly_eval_rows((d, c, b, a), t, t0, t1)
+
+
+def poly4eval(e, d, c, b, a, t, t0, t1):
+    """The same with five coefficients, constant term first (reference interpolation.py:25-40)."""
+    return _poly_eval_rows((e, d, c, b, a), t, t0, t1)
+
+
 class LocalInterpolation:
     """Protocol (reference interpolation.py:43-45)."""
 
@@ -37,6 +53,11 @@ class _PolynomialInterpolation(LocalInterpolation):
         self._coeff = _stack(coefficients)
         assert self._coeff.ndim == 3 and self._coeff.shape[0] == self.degree + 1
         self.coefficients = tuple(self._coeff.unbind(0))
+
+    @staticmethod
+    def _make(degree: int, t0, t1, coefficients) -> "_PolynomialInterpolation":
+        cls = type("_Polynomial", (_PolynomialInterpolation,), {"degree": degree})
+        return cls(t0, t1, coefficients)
 
     def _span(self) -> torch.Tensor:
         return self.t1
