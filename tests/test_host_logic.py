@@ -254,6 +254,10 @@ def test_names_the_reference_keeps_in_its_adjoints_and_interpolation_modules():
 
     assert adjoints.BacksolveAdjoint is backsolve.BacksolveAdjoint and adjoints.JointBacksolveAdjoint is backsolve.JointBacksolveAdjoint
     assert callable(interpolation.poly3eval) and callable(interpolation.poly4eval)
+    import importlib
+
+    for module, name in (("tsit5", "Tsit5"), ("dopri5", "Dopri5"), ("heun", "Heun"), ("euler", "Euler")):
+        assert getattr(importlib.import_module(f"torchode_amd.single_step_methods.{module}"), name) is getattr(to, name)
     with pytest.raises(NotImplementedError):
         adjoints.Adjoint().solve(None)
     with pytest.raises(AttributeError):

@@ -1,0 +1,2 @@
+"""Import path kept for code written against the reference; the class lives in ``low_order``."""
+from .low_order import Heun  # noqa: F401
