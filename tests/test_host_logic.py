@@ -262,3 +262,15 @@ def test_names_the_reference_keeps_in_its_adjoints_and_interpolation_modules():
         adjoints.Adjoint().solve(None)
     with pytest.raises(AttributeError):
         adjoints.no_such_name
+
+
+def test_typing_names_and_predicates():
+    """reference typing.py:7-36 (the three predicates) and :44-95 (the tensor names, plain ``torch.Tensor`` here)."""
+    from torchode_amd import typing as ty
+
+    a, b, c = torch.zeros(2, 3), torch.zeros(2, 4), torch.zeros(2, 3, dtype=torch.float64)
+    assert ty.same_shape(a, b, dim=0) and not ty.same_shape(a, b) and not ty.same_shape(a, b, dim=1) and ty.same_shape(a, c)
+    assert ty.same_dtype(a, b) and not ty.same_dtype(a, b, c) and ty.same_device(a, b, c) and ty.same_dtype() and ty.same_shape(a)
+    for name in ("DataTensor", "NormTensor", "SolutionDataTensor", "TimeTensor", "EvaluationTimesTensor", "AcceptTensor", "StatusTensor",
+                 "InterpTimeTensor", "InterpDataTensor", "SampleIndexTensor"):  # fmt: skip
+        assert getattr(ty, name) is torch.Tensor
