@@ -13,6 +13,11 @@ from ..terms import ODETerm
 from .base import SingleStepMethod, StepResult
 
 
+# shapes of a tableau's parts, for annotations: c [stages], a [stages, stages], b and b_err [stages], b_other [n, stages]
+# (reference runge_kutta.py:15-28: nodes, nodes x weights, weights, rows x weights)
+CoefficientVector = RungeKuttaMatrix = WeightVector = WeightMatrix = torch.Tensor
+
+
 class ButcherTableau:
     """Coefficients as float64 CPU tensors: nodes ``c``, matrix ``a`` (square, strictly lower
     triangular for explicit methods), weights ``b``, error weights ``b_err`` and optional extra
