@@ -183,3 +183,14 @@ def shortcut_case(seed):
     p, i, d = SHORTCUT_PID[seed % len(SHORTCUT_PID)]
     ctrl = {k: v for k, v in dict(ctrl, kind="pid", pcoeff=p, icoeff=i, dcoeff=d).items() if k not in ("dt_min", "dt_max")}
     return f, y0, t_eval, t_start, t_end, method, ctrl, 600, dt0  # (no step limits: the controller runs many times)
+
+
+def aten_elementwise_fuses() -> bool:
+    """True where this host's ATen computes ``addcmul(c, a, b)`` on whole float64 vectors with one rounding (a fused
+    multiply-add), which is the arithmetic the kernels follow; checked against exact rational arithmetic."""
+    from fractions import Fraction
+
+    g = torch.Generator().manual_seed(3)
+    a, b, c = (torch.randn(64, dtype=torch.float64, generator=g) for _ in range(3))
+    exact = [float(Fraction(x) * Fraction(y) + Fraction(z)) for x, y, z in zip(a.tolist(), b.tolist(), c.tolist())]
+    return torch.addcmul(c, a, b).tolist() == exact
