@@ -263,7 +263,7 @@ static void build_tableaux(void) {
         const double w[3][7] = {
             {-2.763706197274826, 0.13169999999999998, 3.930296236894751, -12.411077166933676, 37.50931341651104,
              -27.896526289197286, 1.5},
-            {2.9132554618219126, -0.2234, -5.941033872131505, 30.33818863028232, -88.1789048947664, 65.09189467479366,
+            {2.9132554618219126, -0.2234, -5.941033872131505, 30.338188630282318, -88.1789048947664, 65.09189467479368,
              -4.0},
             {-1.0530884977290216, 0.1017, 2.490627285651253, -16.548102889244902, 47.37952196281928,
              -34.87065786149661, 2.5},

@@ -32,7 +32,7 @@ so end-to-end trajectories are pinned only through the closed forms, library
 special cases and reference-held examples listed there; ATen's bit-level
 association is inherited, not pinned.
 """
-from fractions import Fraction
+from functools import lru_cache
 from math import sqrt
 from typing import Callable, Dict, NamedTuple, Optional
 
@@ -51,48 +51,42 @@ def _square(rows):
     return [list(r) + [0.0] * (n - len(r)) for r in rows]
 
 
+@lru_cache(maxsize=None)
 def tsit5_dense_weights():
     """theta^2, theta^3, theta^4 monomial coefficients of Tsitouras' seven dense-output
-    basis polynomials (tsit5.py:11-50).  The reference expands the factored
-    polynomials with sympy in floating point; here the factored literals are expanded
-    in exact rational arithmetic and rounded once, which agrees with any float
-    expansion to the last ulp or two.
+    basis polynomials, derived the way the reference derives them (tsit5.py:11-50):
+    the interpolant ``y_0 + dt * sum_s f_s b_s(t)`` is written with the factored basis
+    polynomials as sympy expressions over *floating point* literals, expanded in t,
+    collected by powers of t, and each coefficient converted with ``float``.  The
+    intermediate products are therefore rounded by sympy's float arithmetic, and two of
+    the 21 numbers differ in the last place from an exact expansion rounded once; the
+    reference's solves use these.  The symbol names are the reference's, because
+    sympy's canonical ordering of sums and products goes by name.
 
-    pinned by: brute-force numpy.polynomial product, sum_p W[p][s] == b[s],
-    theta^1 row == (1,0,..,0), quartic-recovery test (tests/interpolation_test.py:105-127).
+    Returns (rows for t^2, t^3, t^4; row for t^1).
+
+    pinned by: literal equality with the kernels' and the C oracle's constants, the
+    brute-force numpy.polynomial product (to 1e-14), sum_p W[p][s] == b[s], t^1 row ==
+    (1,0,..,0) up to one rounding, quartic-recovery test
+    (tests/interpolation_test.py:105-127).
     """
-    F = Fraction
-    one = F(1)
+    import sympy as sp
 
-    def mul(p, q):
-        out = [F(0)] * (len(p) + len(q) - 1)
-        for i, a in enumerate(p):
-            for j, b in enumerate(q):
-                out[i + j] += a * b
-        return out
-
-    def lin(root):  # (t - root), lowest power first
-        return [-F(root), one]
-
-    def quad(p1, p0):  # t^2 - p1 t + p0
-        return [F(p0), -F(p1), one]
-
-    t = [F(0), one]
-    t2 = [F(0), F(0), one]
-
-    def scale(s, p):
-        return [F(s) * x for x in p]
-
+    t, y_0, dt = sp.symbols("t y_0 dt")
+    f = sp.symbols("f_1:8")
+    quad = lambda p1, p0: t**2 - p1 * t + p0
     basis = [
-        scale(-1.0530884977290216, mul(mul(t, lin(1.3299890189751412)), quad(1.4364028541716351, 0.7139816917074209))),
-        scale(0.1017, mul(t2, quad(2.1966568338249754, 1.2949852507374631))),
-        scale(2.490627285651252793, mul(t2, quad(2.38535645472061657, 1.57803468208092486))),
-        scale(-16.54810288924490272, mul(mul(lin(1.21712927295533244), lin(0.61620406037800089)), t2)),
-        scale(47.37952196281928122, mul(mul(lin(1.203071208372362603), lin(0.658047292653547382)), t2)),
-        scale(-34.87065786149660974, mul(mul(lin(1.2), lin(0.666666666666666667)), t2)),
-        scale(2.5, mul(mul(lin(1.0), lin(0.6)), t2)),
+        -1.0530884977290216 * t * (t - 1.3299890189751412) * quad(1.4364028541716351, 0.7139816917074209),
+        0.1017 * t**2 * quad(2.1966568338249754, 1.2949852507374631),
+        2.490627285651252793 * t**2 * quad(2.38535645472061657, 1.57803468208092486),
+        -16.54810288924490272 * (t - 1.21712927295533244) * (t - 0.61620406037800089) * t**2,
+        47.37952196281928122 * (t - 1.203071208372362603) * (t - 0.658047292653547382) * t**2,
+        -34.87065786149660974 * (t - 1.2) * (t - 0.666666666666666667) * t**2,
+        2.5 * (t - 1) * (t - 0.6) * t**2,
     ]
-    return [[float(basis[s][p]) for s in range(7)] for p in (2, 3, 4)], [float(basis[s][1]) for s in range(7)]
+    powers = sp.collect(sp.expand(y_0 + dt * sum(f_s * b_s for f_s, b_s in zip(f, basis)), t), t)
+    row = lambda p: [float(powers.coeff(t, p).coeff(f_s).coeff(dt)) for f_s in f]
+    return [row(p) for p in (2, 3, 4)], row(1)
 
 
 class Tableau(NamedTuple):

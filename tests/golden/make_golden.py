@@ -209,6 +209,46 @@ def make_low_order(name, batch, dtype, method, controller, parts):
     }
 
 
+# Solves without evaluation points that stop early on max_steps (reference adjoints.py:176-181, 296-311): the one value
+# returned per sample is the last step's interpolant evaluated at t_end, far outside the step (theta >> 1), which
+# amplifies the last place of the dense-output weights by many orders of magnitude.  The case that tells the
+# reference's Tsit5 weights (a sympy float expansion, tsit5.py:11-50) from an exact expansion of the same polynomials.
+#   (workload, batch, dtype, max_steps)
+EARLY_STOP_CASES = [("vdp", 256, torch.float64, 20), ("vdp", 256, torch.float32, 12)]
+
+
+def early_stop_inputs(name, batch, dtype):
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    return w, w.t_eval[:, 0].clone(), w.t_eval[:, -1].clone()
+
+
+def make_early_stop(name, batch, dtype, max_steps):
+    w, t_start, t_end = early_stop_inputs(name, batch, dtype)
+    ctrl = torch_loop.Controller(**w.controller)
+    out = torch_loop.solve(w.f, w.y0, None, method=w.method, controller=ctrl, t_start=t_start, t_end=t_end, max_steps=max_steps)
+    cfg = c_oracle.make_config(method=w.method, term=name, nthreads=4, max_steps=max_steps, **w.controller)
+    chk = c_oracle.solve(cfg, w.f.builtin_params(), w.y0, None, t_start=t_start, t_end=t_end)
+    for key in ("ys", "n_steps", "n_accepted", "n_initialized", "status", "n_f_evals"):
+        assert torch.equal(out[key], chk[key]), f"{name} {dtype}: C oracle and ATen-op oracle disagree on {key}"
+    assert out["ys"].shape == (batch, 1, w.y0.shape[1]) and (out["status"] == 3).all() and (out["n_steps"] == max_steps).all()
+    return {
+        "source": f"oracle/torch_loop.py (ATen CPU ops), torch {torch.__version__}, {torch.backends.cpu.get_cpu_capability()}, "
+        f"opt_einsum {torch.backends.opt_einsum.is_available()}; reproduced bit for bit by oracle/erk_oracle.c; no evaluation points, "
+        "every sample stopped by max_steps",
+        "workload": name,
+        "batch": batch,
+        "dtype": str(dtype).replace("torch.", ""),
+        "method": w.method,
+        "controller": w.controller,
+        "max_steps": max_steps,
+        "inputs_sha256": {"y0": sha(w.y0), "t_start": sha(t_start), "t_end": sha(t_end), "params": sha(w.f.builtin_params())},
+        "n_f_evals": int(out["n_f_evals"][0]),
+        **{key: out[key].tolist() for key in ("n_steps", "n_accepted", "n_initialized", "status")},
+        "ys_sha256": sha(out["ys"]),
+        "ys": hexlist(out["ys"]),
+    }
+
+
 def make_tolerance(name, batch, dtype):
     w = to.workloads.make(name, batch=batch, dtype=dtype)
     out = torch_loop.solve(w.f, w.y0, w.t_eval, method=w.method, controller=torch_loop.Controller(**w.controller))
@@ -233,6 +273,12 @@ def make_tolerance(name, batch, dtype):
 
 
 if __name__ == "__main__":
+    for name, batch, dtype, max_steps in EARLY_STOP_CASES:
+        d = make_early_stop(name, batch, dtype, max_steps)
+        path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_early_stop.json")
+        with open(path, "w") as fh:
+            json.dump(d, fh, separators=(",", ":"))
+        print(path, os.path.getsize(path), "bytes")
     for name, batch, dtype, method, controller, parts in LOW_ORDER_CASES:
         d = make_low_order(name, batch, dtype, method, controller, parts)
         path = os.path.join(HERE, f"{name}_{d['dtype']}_b{batch}_{method}_{d['controller']['kind']}_low_order.json")

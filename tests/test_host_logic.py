@@ -165,7 +165,7 @@ def test_tolerance_fixture_inputs_and_workload_agree(path):
     assert all(s == 0 for s in g["status"]) and g["n_f_evals"] == 2 + 6 * max(g["n_steps"])
 
 
-@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json"))], ids=os.path.basename)
+@pytest.mark.parametrize("path", [p for p in GOLDEN if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json", "_early_stop.json"))], ids=os.path.basename)
 def test_oracle_reproduces_golden_fixture(path):
     g = json.load(open(path))
     dtype = getattr(torch, g["dtype"])
@@ -183,6 +183,24 @@ def test_oracle_reproduces_golden_fixture(path):
     got = [float(v).hex() for v in out["ys"][g["subset"]].flatten().tolist()]
     assert got == g["ys_subset"]
     assert float(out["ys"].double().abs().max()).hex() == g["ys_max_abs"]
+
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if p.endswith("_early_stop.json")], ids=os.path.basename)
+def test_oracle_reproduces_early_stop_fixture(path):
+    """No evaluation points and every sample stopped by max_steps (tests/golden/make_golden.py::make_early_stop): the
+    value returned is the last step's interpolant far outside its step, where the last place of Tsit5's dense-output
+    weights shows in the result."""
+    g = json.load(open(path))
+    dtype = getattr(torch, g["dtype"])
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=dtype)
+    t_start, t_end = w.t_eval[:, 0].clone(), w.t_eval[:, -1].clone()
+    assert {"y0": _sha(w.y0), "t_start": _sha(t_start), "t_end": _sha(t_end), "params": _sha(w.f.builtin_params())} == g["inputs_sha256"]
+    cfg = c_oracle.make_config(method=g["method"], term=g["workload"], nthreads=4, max_steps=g["max_steps"], **g["controller"])
+    out = c_oracle.solve(cfg, w.f.builtin_params(), w.y0, None, t_start=t_start, t_end=t_end)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status"):
+        assert out[key].tolist() == g[key], key
+    assert all(s == 3 for s in g["status"]) and int(out["n_f_evals"][0]) == g["n_f_evals"] == 2 + 6 * g["max_steps"]
+    assert [float(v).hex() for v in out["ys"].flatten().tolist()] == g["ys"] and _sha(out["ys"]) == g["ys_sha256"]
 
 
 def test_mlp_weights_in_one_row_major_block():

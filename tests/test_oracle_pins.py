@@ -130,29 +130,61 @@ def test_tsit5_dense_weights_by_brute_force(source):
     assert np.allclose(w.sum(0) + np.eye(7)[0], t["b"], atol=2e-14)
 
 
-def test_tsit5_dense_weights_by_sympy():
+# What tsit5.py:11-50 evaluates to under sympy 1.14: the factored basis polynomials with floating point
+# literals, expanded and collected in t, each coefficient through float().  Two entries of the t^3 row (stages
+# 4 and 6) are one unit in the last place away from the exact expansion rounded once.
+TSIT5_DENSE_WEIGHTS = [
+    [-2.763706197274826, 0.13169999999999998, 3.930296236894751, -12.411077166933676, 37.50931341651104,
+     -27.896526289197286, 1.5],
+    [2.9132554618219126, -0.2234, -5.941033872131505, 30.338188630282318, -88.1789048947664, 65.09189467479368, -4.0],
+    [-1.0530884977290216, 0.1017, 2.490627285651253, -16.548102889244902, 47.37952196281928, -34.87065786149661, 2.5],
+]  # fmt: skip
+
+
+def kernel_tsit5_weights():
+    """The constants compiled into the HIP library (a host-side table read, no GPU needed)."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    c, a, be = (ctypes.c_double * 7)(), (ctypes.c_double * 49)(), (ctypes.c_double * 7)()
+    other, n = (ctypes.c_double * 21)(), ctypes.c_int32(0)
+    tsit5 = 1  # TODE_TSIT5
+    assert lib.tode_tableau(tsit5, c, a, be, other, ctypes.byref(n)) == 0 and n.value == 3
+    return np.array(list(other)).reshape(3, 7)
+
+
+def test_tsit5_dense_weights_are_the_float_derivation_literally():
+    """All 21 weights, in the ATen-op oracle (which runs the sympy float derivation), the C oracle and the
+    kernels: equal as floats, not approximately."""
+    derived, first = tl.tsit5_dense_weights()
+    assert derived == TSIT5_DENSE_WEIGHTS
+    assert first == [0.9999999999999999, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0]
+    assert c_tableau("tsit5")["b_other"].tolist() == TSIT5_DENSE_WEIGHTS
+    assert torch_tableau("tsit5")["b_other"].tolist() == TSIT5_DENSE_WEIGHTS
+    assert kernel_tsit5_weights().tolist() == TSIT5_DENSE_WEIGHTS
+
+
+def test_tsit5_float_derivation_differs_from_the_exact_expansion_in_two_last_places():
+    """Guards the derivation itself: expanding in exact rationals and rounding once gives other last digits
+    in exactly two places, so a derivation that silently went exact (or reordered) would show here."""
     import sympy as sp
 
     th = sp.Symbol("t")
-    lits = [
-        (-1.0530884977290216, [(1.3299890189751412,)], (1.4364028541716351, 0.7139816917074209), 1),
-        (0.1017, [], (2.1966568338249754, 1.2949852507374631), 2),
-        (2.490627285651252793, [], (2.38535645472061657, 1.57803468208092486), 2),
-        (-16.54810288924490272, [(1.21712927295533244,), (0.61620406037800089,)], None, 2),
-        (47.37952196281928122, [(1.203071208372362603,), (0.658047292653547382,)], None, 2),
-        (-34.87065786149660974, [(1.2,), (0.666666666666666667,)], None, 2),
-        (2.5, [(1,), (0.6,)], None, 2),
-    ]
-    w, _ = tl.tsit5_dense_weights()
-    for s, (lead, roots, quad, tpow) in enumerate(lits):
-        e = sp.Rational(Fraction(lead)) * th**tpow
-        for (r,) in roots:
-            e *= th - sp.Rational(Fraction(float(r)))
-        if quad:
-            e *= th**2 - sp.Rational(Fraction(quad[0])) * th + sp.Rational(Fraction(quad[1]))
-        poly = sp.Poly(sp.expand(e), th)
-        for p in (2, 3, 4):
-            assert float(poly.coeff_monomial(th**p)) == pytest.approx(w[p - 2][s], rel=1e-15, abs=1e-300)
+    R = lambda x: sp.Rational(Fraction(float(x)))
+    basis = [
+        R(-1.0530884977290216) * th * (th - R(1.3299890189751412)) * (th**2 - R(1.4364028541716351) * th + R(0.7139816917074209)),
+        R(0.1017) * th**2 * (th**2 - R(2.1966568338249754) * th + R(1.2949852507374631)),
+        R(2.490627285651252793) * th**2 * (th**2 - R(2.38535645472061657) * th + R(1.57803468208092486)),
+        R(-16.54810288924490272) * (th - R(1.21712927295533244)) * (th - R(0.61620406037800089)) * th**2,
+        R(47.37952196281928122) * (th - R(1.203071208372362603)) * (th - R(0.658047292653547382)) * th**2,
+        R(-34.87065786149660974) * (th - R(1.2)) * (th - R(0.666666666666666667)) * th**2,
+        R(2.5) * (th - 1) * (th - R(0.6)) * th**2,
+    ]  # fmt: skip
+    exact = [[float(sp.Poly(sp.expand(b), th).coeff_monomial(th**p)) for b in basis] for p in (2, 3, 4)]
+    differing = [(p, s) for p in range(3) for s in range(7) if exact[p][s] != TSIT5_DENSE_WEIGHTS[p][s]]
+    assert differing == [(1, 3), (1, 5)]
+    for p, s in differing:
+        assert abs(exact[p][s] - TSIT5_DENSE_WEIGHTS[p][s]) <= 2 * np.spacing(abs(exact[p][s]))
 
 
 # --------------------------------------------------------------------------- #

@@ -380,7 +380,7 @@ import glob  # noqa: E402
 import json  # noqa: E402
 import os  # noqa: E402
 
-_GOLDEN = sorted(p for p in glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")) if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json")))
+_GOLDEN = sorted(p for p in glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")) if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json", "_early_stop.json")))
 
 
 @pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])
@@ -406,6 +406,35 @@ def test_gpu_matches_golden_fixture(path, fast):
     ys = sol.ys.cpu()
     assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
     assert float(ys.double().abs().max()).hex() == g["ys_max_abs"]
+
+
+_EARLY_STOP = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_early_stop.json")))
+
+
+@pytest.mark.parametrize("path_kind", ["whole-solve", "general", "per-step", "protocol"])
+@pytest.mark.parametrize("path", _EARLY_STOP, ids=os.path.basename)
+def test_gpu_matches_early_stop_fixture(path, path_kind):
+    """tests/golden/*_early_stop.json: no evaluation points, every sample stopped by max_steps, so the one value per
+    sample is the last step's interpolant evaluated far outside the step -- where the last place of Tsit5's
+    dense-output weights is visible in the result.  Every kernel path reproduces the vectors bit for bit."""
+    g = json.load(open(path))
+    w = to.workloads.make(g["workload"], batch=g["batch"], dtype=getattr(torch, g["dtype"]))
+    kw = dict(t_start=w.t_eval[:, 0].clone(), t_end=w.t_eval[:, -1].clone(), max_steps=g["max_steps"])
+    if path_kind == "per-step":
+        from test_stepwise_gpu import stepwise_solve
+
+        sol = stepwise_solve(w.f, w.y0, None, g["method"], g["controller"], **kw)
+    elif path_kind == "protocol":
+        from test_protocol_gpu import protocol_solve
+
+        sol = protocol_solve(w.f, w.y0, None, g["method"], g["controller"], **kw)
+    else:
+        sol = gpu_solve(w.f, w.y0, None, g["method"], g["controller"], fast=path_kind == "whole-solve", **kw)
+    got = dict(sol.stats, status=sol.status)
+    for key in ("n_steps", "n_accepted", "n_initialized", "status"):
+        assert got[key].cpu().tolist() == g[key], key
+    assert int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]
+    assert [float(v).hex() for v in sol.ys.cpu().flatten().tolist()] == g["ys"]
 
 
 # ---------------------------------------------------------------------------------------------
