@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 13
+#define TODE_ABI_VERSION 14
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -224,6 +224,42 @@ int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *
 int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                                  int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *stream,
                                  int32_t *flags_out);
+
+/*
+ * tode_solve_builtin_fast for a caller that cannot allocate.  No counterpart in
+ * the reference; it is for code under HIP graph capture, tight serving loops
+ * and harnesses that forbid allocation calls: this call performs no hipMalloc /
+ * hipFree / hipHostMalloc and no allocating library routine, now or on its first
+ * use.  The device memory the solve needs beyond its inputs and outputs -- the
+ * working flag words with the count of finished workgroups, and, when n_eval ==
+ * 0, the [B,F] staging area of the final states -- lies in a static device array
+ * of the library (256 + TODE_STATIC_STAGING_BYTES bytes, one copy per GPU the
+ * library runs on, held until the process ends).  `args->flags` and
+ * `args->y_idle` are not used (may be null).  The kernels are those of
+ * tode_solve_builtin_fast and the results are bit-identical to it; the flag
+ * block is written to `flags_out` (DEVICE memory, TODE_FLAG_WORDS int32) and is
+ * valid in stream order, like ys and the stats; the caller reads it when it
+ * likes (flags_out[TODE_FLAG_NEEDS_GENERAL] as for tode_solve_builtin_fast).
+ * With n_eval == 0 the call also enqueues the end point selection
+ * (tode_select_end_point), which reads the iteration count from flags_out on
+ * the device, so ys is final without a host round trip.
+ *
+ * Limit: with n_eval == 0, B * F * sizeof(value) must not exceed
+ * TODE_STATIC_STAGING_BYTES; beyond that the call returns TODE_E_UNSUPPORTED
+ * and launches nothing.  With n_eval > 0 the array sets no limit.  Shapes that
+ * tode_solve_builtin_fast refuses are refused here with the same code.
+ *
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU
+ * (several streams, several host threads) race on it and must be serialised by
+ * the caller.  Calls in a row on one stream need nothing: each call resets the
+ * words it uses by a kernel in front of the solve kernel.  The array's address
+ * is looked up on the first call on a device (hipGetSymbolAddress, not an
+ * allocation); a caller that captures a graph makes one call before capturing.
+ */
+#define TODE_STATIC_STAGING_BYTES (2 << 20)
+int tode_solve_builtin_fast_static(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
+                                   int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,
+                                   int32_t *flags_out, void *stream);
 
 /*
  * Last step of a solve without evaluation points through tode_solve_builtin_fast

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -27,6 +27,8 @@ FLAG_MAX_ITERATIONS, FLAG_FIRST_FAILURE, FLAG_NON_MONOTONE, FLAG_NEEDS_GENERAL, 
 INT32_MAX = 2**31 - 1
 
 DTYPES = {torch.float32: F32, torch.float64: F64}
+E_INVALID, E_UNSUPPORTED, E_HIP = -1, -2, -3  # return codes (TODE_E_*)
+STATIC_STAGING_BYTES = 2 << 20  # TODE_STATIC_STAGING_BYTES
 
 # every symbol include/torchode_amd.h declares
 EXPORTS = (
@@ -35,6 +37,7 @@ EXPORTS = (
     "tode_solve_builtin",
     "tode_solve_builtin_fast",
     "tode_solve_builtin_fast_sync",
+    "tode_solve_builtin_fast_static",
     "tode_mlp_pack_weights",
     "tode_select_end_point",
     "tode_step_begin",
@@ -233,6 +236,8 @@ def load():
         lib.tode_select_end_point.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.tode_mlp_pack_weights.restype = C.c_int
         lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
+        lib.tode_solve_builtin_fast_static.restype = C.c_int
+        lib.tode_solve_builtin_fast_static.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 6
         lib.tode_solve_builtin_fast_sync.restype = C.c_int
         lib.tode_solve_builtin_fast_sync.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.POINTER(C.c_int32)]
         lib.tode_step_begin.restype = C.c_int

@@ -123,6 +123,57 @@ static int wait_for_flags(const int32_t *slot, int32_t sequence, hipStream_t s) 
     }
 }
 
+// ---- static scratch of tode_solve_builtin_fast_static -------------------------------------------
+// Device memory that belongs to the loaded code object, one copy per GPU, held until the process
+// ends: the working flag words of a solve (four flags and the count of finished workgroups) in the
+// first STATIC_FLAG_BYTES, behind them the staging area for the final states of a solve without
+// evaluation points.  Host code never uses the array's name as an address: static_scratch() asks the
+// runtime for the device's copy once and keeps the pointer.
+constexpr size_t STATIC_FLAG_BYTES = 256;
+static __device__ __align__(256) unsigned char scratch[STATIC_FLAG_BYTES + TODE_STATIC_STAGING_BYTES];
+static void *g_scratch_ptr[FLAG_DEVICES];  // static storage: null until asked for
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(hipStream_t s, unsigned char **out) {
+    int device = 0;
+    int rc = check_hip(s ? hipStreamGetDevice(s, &device) : hipGetDevice(&device), "device of the stream");
+    if (rc) return rc;
+    if (device < 0 || device >= FLAG_DEVICES) return fail(TODE_E_UNSUPPORTED, "device index %d", device);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        int current = 0;
+        if ((rc = check_hip(hipGetDevice(&current), "hipGetDevice"))) return rc;
+        if (current != device && (rc = check_hip(hipSetDevice(device), "hipSetDevice"))) return rc;
+        void *ptr = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (current != device) (void)hipSetDevice(current);
+        if (err != hipSuccess) return check_hip(err, "hipGetSymbolAddress of the static scratch array");
+        if (!ptr) return fail(TODE_E_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = (unsigned char *)g_scratch_ptr[device];
+    return TODE_OK;
+}
+
+// The working flag words at their start values, whatever the last call left there.
+static __global__ void static_flags_reset_kernel(int32_t *flags) {
+    if (threadIdx.x <= TODE_FLAG_WORDS) flags[threadIdx.x] = threadIdx.x == TODE_FLAG_FIRST_FAILURE ? INT_MAX : 0;
+}
+
+// Flags of a solve that launched no solve kernel (an empty batch).
+static __global__ void empty_flags_kernel(int32_t *flags_out) {
+    if (threadIdx.x < TODE_FLAG_WORDS) flags_out[threadIdx.x] = threadIdx.x == TODE_FLAG_FIRST_FAILURE ? INT_MAX : 0;
+}
+
+// select_end_point_kernel with the loop's iteration count read from the published flag block
+// instead of passed by the host; does nothing when the batch left the common case.
+template <typename T>
+__global__ void select_end_point_by_flags_kernel(long long n, int F, const int32_t *flags, const int64_t *n_steps, T *ys, const T *y_idle) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n || flags[TODE_FLAG_NEEDS_GENERAL] != 0) return;
+    if (n_steps[i / F] < (long long)flags[TODE_FLAG_MAX_ITERATIONS]) ys[i] = y_idle[i];
+}
+
 template <typename T>
 __global__ void finalize_kernel(long long batch, int last_iteration, const int32_t *n_steps, const int32_t *n_accepted,
                                 const int32_t *n_initialized, const int32_t *status_last, const int32_t *status_idle,
@@ -294,6 +345,48 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller
     // (after a failed wait the slot's words may be anything: the slot stays out of use)
     if (rc == TODE_OK || rc == TODE_E_INVALID || rc == TODE_E_UNSUPPORTED) pool->busy[slot].store(0, std::memory_order_release);
     return rc;
+}
+
+int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,
+                                   int64_t *st, int32_t *flags_out, void *stream) {
+    using namespace tode;
+    if (!a || !c || !flags_out) return fail(TODE_E_INVALID, "null argument");
+    if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0) return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d", (long long)a->batch, a->n_features, a->n_eval);
+    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    const bool end_only = a->n_eval == 0;
+    const size_t value_bytes = a->dtype == TODE_F32 ? 4 : 8;
+    if (end_only && (uint64_t)a->batch * (uint64_t)a->n_features > TODE_STATIC_STAGING_BYTES / value_bytes)
+        return fail(TODE_E_UNSUPPORTED, "without evaluation points the final states of the batch are staged in the static scratch array: "
+                    "%lld x %d values of %zu bytes exceed its %lld bytes", (long long)a->batch, a->n_features, value_bytes, (long long)TODE_STATIC_STAGING_BYTES);
+    hipStream_t s = (hipStream_t)stream;
+    unsigned char *base = nullptr;
+    int rc = static_scratch(s, &base);
+    if (rc) return rc;
+    int32_t *words = (int32_t *)base;
+    void *staging = base + STATIC_FLAG_BYTES;
+
+    tode_solve_args b = *a;
+    b.flags = words;
+    if (end_only) b.y_idle = staging;
+    const FlagTarget target = {words, flags_out, 0};
+    hipLaunchKernelGGL(static_flags_reset_kernel, dim3(1), dim3(64), 0, s, words);
+    g_flag_target = &target;
+    rc = tode_solve_builtin_fast(&b, c, ns, na, ni, st, stream);
+    g_flag_target = nullptr;
+    if (rc) return rc;
+    if (a->batch == 0) {
+        hipLaunchKernelGGL(empty_flags_kernel, dim3(1), dim3(64), 0, s, flags_out);
+        return check_hip(hipGetLastError(), "tode_solve_builtin_fast_static launch");
+    }
+    if (end_only) {
+        const long long n = (long long)a->batch * a->n_features;
+        const unsigned blocks = (unsigned)((n + 255) / 256);
+        if (a->dtype == TODE_F32)
+            hipLaunchKernelGGL(select_end_point_by_flags_kernel<float>, dim3(blocks), dim3(256), 0, s, n, (int)a->n_features, flags_out, ns, (float *)a->ys, (const float *)staging);
+        else
+            hipLaunchKernelGGL(select_end_point_by_flags_kernel<double>, dim3(blocks), dim3(256), 0, s, n, (int)a->n_features, flags_out, ns, (double *)a->ys, (const double *)staging);
+    }
+    return check_hip(hipGetLastError(), "tode_solve_builtin_fast_static launch");
 }
 
 int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int64_t last_iteration, const int64_t *n_steps, void *ys,

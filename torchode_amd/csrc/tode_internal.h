@@ -30,6 +30,9 @@ int check_hip(hipError_t err, const char *what);
 // Set on the calling thread while tode_solve_builtin_fast_sync runs: the solve kernel then works on
 // the library's own, self-resetting flag words `dev` (no reset launch in front of it) and its last
 // workgroup stores the result, followed by `sequence`, into the pinned host words `host`.
+// tode_solve_builtin_fast_static sets it too: `dev` are words of the library's static device array,
+// `host` is the caller's flag block in device memory, and `sequence` is 0 (no word is written
+// behind the flags; the caller reads them in stream order).
 struct FlagTarget {
     int32_t *dev;
     int32_t *host;

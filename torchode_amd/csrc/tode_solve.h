@@ -297,7 +297,8 @@ template <typename T> __device__ __forceinline__ void publish_flags(const SolveP
 #pragma unroll
     for (int i = 0; i < TODE_FLAG_WORDS; ++i) __hip_atomic_store(&p.host_flags[i], v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     // (the release also covers the exchanges above: a later kernel finds the words reset)
-    __hip_atomic_store(&p.host_flags[TODE_FLAG_WORDS], p.sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    // (a target without a sequence number is read in stream order, after the kernel: nothing to announce)
+    if (p.sequence != 0) __hip_atomic_store(&p.host_flags[TODE_FLAG_WORDS], p.sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // Resets the flag block; launched in front of every solve kernel.
