@@ -2,8 +2,10 @@
  * torchode_amd -- C ABI of the MI355X-native batch-parallel adaptive explicit
  * Runge-Kutta solve loop.
  *
- * Every entry point takes plain device pointers, sizes and a HIP stream and
- * allocates nothing.  All pointers are device pointers unless a comment says
+ * Every entry point takes plain device pointers, sizes and a HIP stream.  None
+ * allocates per call; tode_solve_builtin_fast_sync allocates its flag words once
+ * per device on its first call there (see its comment), the others never.  All
+ * pointers are device pointers unless a comment says
  * otherwise; every array is contiguous (row-major) in the layout given.  An
  * entry point returns 0 on success and a negative TODE_E_* code otherwise;
  * tode_last_error() returns a human-readable message for the last failure on
@@ -153,6 +155,11 @@ typedef struct tode_solve_args {
 /* ABI version of the loaded library (== TODE_ABI_VERSION of the header it was built from). */
 int tode_abi_version(void);
 
+/* sha256 (hex, host pointer) of the sources and compiler flags the loaded library was built from, as the build
+ * script computes it; empty for a build that did not pass one.  A loader compares it with the sources it finds
+ * beside the library, so that an edited kernel is never tested through a stale binary. */
+const char *tode_source_hash(void);
+
 /* Message for the most recent non-zero return code on this host thread (host pointer). */
 const char *tode_last_error(void);
 
@@ -212,8 +219,11 @@ int tode_solve_builtin_fast(const tode_solve_args *args, const tode_controller *
  * first call), its last workgroup stores them into pinned host memory, and
  * this call returns when they have arrived there, with the TODE_FLAG_WORDS
  * values in the host array `flags_out`.  That saves the launch that resets the
- * flag block and the device-to-host copy.  ys and the four stat arrays are
- * complete in stream order as before (here: when the call returns).  Safe to
+ * flag block and the device-to-host copy.  Only the flag words are on the host
+ * when the call returns: ys and the four stat arrays are complete in stream
+ * order, as for tode_solve_builtin_fast (work enqueued on `stream` afterwards,
+ * or a stream synchronisation, sees them; the returned call by itself does not
+ * make other workgroups' stores visible to the host or to other streams).  Safe to
  * call from several host threads and on several streams at once.  With
  * n_eval == 0 this call also enqueues tode_select_end_point.  Where
  * tode_solve_builtin_fast would refuse a small system for its shape (n_eval
@@ -305,7 +315,8 @@ enum {
 /*
  * Device-resident state of one solve whose right-hand side f is evaluated by
  * the caller (any framework) between kernels.  The caller owns every buffer
- * for the duration of the solve.  Data and time share one dtype.
+ * for the duration of the solve.  Data and time may have different dtypes
+ * (`dtype` and `time_dtype` below).
  *
  * Replaces the locals of AutoDiffAdjoint.solve (reference adjoints.py:59-126),
  * ERKState / ERKInterpolationData (single_step_methods/runge_kutta.py:161-172)

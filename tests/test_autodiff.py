@@ -265,6 +265,71 @@ def test_gradients_reach_tensors_inside_args():
     torch.testing.assert_close(A2.grad, A_ref2.grad, rtol=1e-7, atol=1e-8)
 
 
+def test_tensors_that_f_closes_over_are_found_from_one_evaluation():
+    """CPU: captured_leaves walks the graph of f(t_start, y0) on detached inputs: a captured leaf, the leaf behind a
+    captured tensor that was computed, a module's parameter and a buffer that requires grad are found; y0, the times
+    and the tensors in args are not (the caller names those)."""
+    from torchode_amd.autodiff import captured_leaves, wants_grad_through_term
+
+    A = torch.tensor(A0, dtype=torch.double, requires_grad=True)
+    raw = torch.tensor(0.3, dtype=torch.double, requires_grad=True)
+    scale = raw.exp()  # not a leaf
+    lin = nn.Linear(3, 3).double()
+    lin.register_buffer("shift", torch.tensor(0.1, dtype=torch.double, requires_grad=True))
+    y0 = torch.tensor(Y0, dtype=torch.double, requires_grad=True)
+    problem = to.InitialValueProblem(y0, t_eval=torch.tensor(T_EVAL, dtype=torch.double))
+    extra = torch.tensor(2.0, dtype=torch.double, requires_grad=True)
+    term = to.ODETerm(lambda t, y, args: (y @ A) * scale + lin(y) + lin.shift + args, with_args=True)
+    found = captured_leaves(term, problem, extra)
+    assert {id(x) for x in found} == {id(A), id(raw), id(lin.weight), id(lin.bias), id(lin.shift)}
+    assert wants_grad_through_term(term, problem, extra.detach())
+    plain = to.ODETerm(lambda t, y: y @ A.detach())
+    assert captured_leaves(plain, problem, None) == [] and not wants_grad_through_term(plain, problem, None)
+    assert wants_grad_through_term(to.ODETerm(to.VanDerPol(torch.ones(2, requires_grad=True))), problem, None)
+    assert not wants_grad_through_term(to.ODETerm(to.VanDerPol(torch.ones(2))), problem, None)
+
+
+@gpu
+def test_gradients_reach_tensors_that_f_closes_over_and_buffers_of_a_built_in_term():
+    """The reference's loop is torch operations, so a tensor that `f` merely closes over, or a buffer behind a module,
+    gets its gradient like a parameter (adjoints.py:135-260).  Here such a solve must neither take a whole-solve
+    kernel (no graph) nor differentiate with respect to y0 alone."""
+    y0, A = inputs()
+    A = A.detach().clone().requires_grad_()
+    raw = torch.tensor(0.25, dtype=torch.double, device="cuda", requires_grad=True)
+    scale = raw.exp()  # captured, and not a leaf
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+    weights = torch.linspace(0.5, 1.5, 2 * 3 * 3, dtype=torch.double, device="cuda").reshape(2, 3, 3)
+    for y_needs_grad in (True, False):
+        for x in (y0, A, raw):
+            x.grad = None
+        y_in = y0 if y_needs_grad else y0.detach()
+        term = to.ODETerm(lambda t, y: (y @ A) * scale)
+        solution = to.AutoDiffAdjoint(to.Tsit5(), to.IntegralController(1e-10, 1e-10)).solve(to.InitialValueProblem(y_in, t_eval=t_eval), term=term)
+        assert solution.ys.requires_grad
+        (solution.ys * weights).sum().backward(retain_graph=True)
+        y0_ref, A_ref, raw_ref = (x.detach().clone().requires_grad_() for x in (y0, A, raw))
+        (closed_form(y0_ref, A_ref * raw_ref.exp(), t_eval) * weights).sum().backward()
+        torch.testing.assert_close(A.grad, A_ref.grad, rtol=1e-7, atol=1e-8)
+        torch.testing.assert_close(raw.grad, raw_ref.grad, rtol=1e-7, atol=1e-8)
+        if y_needs_grad:
+            torch.testing.assert_close(y0.grad, y0_ref.grad, rtol=1e-7, atol=1e-8)
+
+    # a built-in term whose parameter requires grad: dy/dt = -k y, y(t) = y0 exp(-k t), d y / d k = -t y
+    k = torch.tensor([[0.5, 1.0, 2.0], [0.3, 0.7, 1.1]], dtype=torch.double, device="cuda", requires_grad=True)
+    start = y0.detach()
+    sol = to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-11, 1e-11)).solve(to.InitialValueProblem(start, t_eval=t_eval), term=to.ODETerm(to.LinearDecay(k)))
+    assert sol.ys.requires_grad  # (without the check of the buffers this solve ran in the whole-solve kernel)
+    (sol.ys * weights).sum().backward()
+    elapsed = (t_eval - t_eval[:, :1])[:, :, None]
+    expect = (-elapsed * start[:, None, :] * torch.exp(-k.detach()[:, None, :] * elapsed) * weights).sum(1)
+    torch.testing.assert_close(k.grad, expect, rtol=1e-6, atol=1e-8)
+    with torch.no_grad():  # and without grad mode the same term takes the whole-solve kernel, same values to rounding
+        fused = to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-11, 1e-11)).solve(to.InitialValueProblem(start, t_eval=t_eval), term=to.ODETerm(to.LinearDecay(k)))
+    assert not fused.ys.requires_grad
+    torch.testing.assert_close(fused.ys, sol.ys.detach(), rtol=1e-12, atol=1e-13)
+
+
 @gpu
 @pytest.mark.parametrize("time_dtype,data_dtype,tol", [(torch.float32, torch.float64, 2e-5), (torch.float64, torch.float32, 2e-3)], ids=["t32-y64", "t64-y32"])
 def test_gradients_with_time_and_data_in_different_dtypes(time_dtype, data_dtype, tol):

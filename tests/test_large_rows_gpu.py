@@ -27,25 +27,53 @@ def device_solve(w):
     return solver.solve(problem, to.ODETerm(copy.deepcopy(w.f).cuda()))
 
 
-def compare(sol, ref, min_agree):
-    """integer stats equal and ys within 1e-4 (mixed absolute / relative) on at least `min_agree` of the samples"""
+def compare(sol, ref, min_agree, trace=None):
+    """Integer stats equal and ys within 1e-4 (mixed absolute / relative) on at least `min_agree` of the samples.
+    Every differing sample is printed.  With the oracle's per-iteration `trace`, a sample whose integer stats differ
+    must have had a borderline decision: an error ratio within 1e-3 of 1 at some iteration (the accept test is
+    ``ratio < 1``); a sample that merely exceeds 1e-4 in ys with the same steps must stay within 1e-3."""
     assert sol.status.tolist() == ref["status"].tolist()
     B = sol.ys.shape[0]
     ys, rys = sol.ys.cpu().double(), ref["ys"].double()
     d = (ys - rys).abs()
-    good = torch.minimum(d, d / rys.abs().clamp_min(1e-300)).flatten(1).amax(dim=1) < 1e-4
+    err = torch.minimum(d, d / rys.abs().clamp_min(1e-300)).flatten(1).amax(dim=1)
+    same_stats = torch.ones(B, dtype=torch.bool)
     for key in ("n_steps", "n_accepted", "n_initialized"):
-        good &= sol.stats[key].cpu() == ref[key]
-    print(f"{int((~good).sum())} of {B} samples differ in stats or by more than 1e-4")
-    assert int((~good).sum()) <= (1 - min_agree) * B
+        same_stats &= sol.stats[key].cpu() == ref[key]
+    good = same_stats & (err < 1e-4)
+    n_bad = int((~good).sum())
+    print(f"{n_bad} of {B} samples differ in stats or by more than 1e-4 ({100.0 * (B - n_bad) / B:.3f} % agree)")
+    for b in (~good).nonzero().flatten().tolist():
+        line = f"  sample {b}: n_steps {int(sol.stats['n_steps'][b])} / {int(ref['n_steps'][b])}, n_accepted {int(sol.stats['n_accepted'][b])} / {int(ref['n_accepted'][b])}, ys error {err[b].item():.2e}"
+        if trace is not None:
+            ratios = [float(tr["ratio"][b]) for tr in trace if bool(tr["running"][b])]
+            closest = min(abs(r - 1.0) for r in ratios)
+            line += f", error ratios {[f'{r:.3e}' for r in ratios]}, closest to the accept threshold by {closest:.1e}"
+            if not same_stats[b]:
+                assert closest < 1e-3, line
+        if same_stats[b]:
+            assert err[b].item() < 1e-3, line
+        print(line)
+    assert n_bad <= (1 - min_agree) * B
     assert mixed_error(ys, rys) < 1e-2
+    return n_bad
+
+
+def oracle_with_trace(w):
+    """The loop as ATen operations on this host's CPU, with its per-iteration record (t, dt, error ratio, accept)."""
+    from oracle import torch_loop
+
+    trace = []
+    ref = torch_loop.solve(w.f, w.y0, w.t_eval, method=w.method, controller=torch_loop.Controller(**w.controller), trace=trace)
+    return ref, trace
 
 
 def test_reaction_diffusion_against_the_aten_oracle():
     w = to.workloads.make("reaction_diffusion", batch=48)
     sol = device_solve(w)
     assert sol.ys.shape == (48, 100, 4096) and (sol.stats["n_initialized"] == 100).all()
-    compare(sol, torch_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller), 0.999)
+    ref, trace = oracle_with_trace(w)
+    compare(sol, ref, 0.999, trace)
     # mass balance of the periodic stencil: d/dt sum(u) = sum(u (1 - u)) > 0, so the mean grows
     mean = sol.ys.mean(dim=2)
     assert (mean[:, 1:] >= mean[:, :-1]).all()
@@ -55,9 +83,66 @@ def test_mlp_against_the_aten_oracle():
     w = to.workloads.make("mlp", batch=256)
     sol = device_solve(w)
     assert sol.ys.shape == (256, 20, 64)
-    # the device matrix products differ from the host's in the last bits; a sample whose error ratio
-    # sits within that distance of 1 may take one more or one less step
-    compare(sol, torch_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller), 0.98)
+    # the device matrix products differ from the host's in the last bits; at 256 samples the 99.9 % bar leaves no
+    # room, so a differing sample is allowed only with the evidence `compare` demands, and one at most
+    ref, trace = oracle_with_trace(w)
+    compare(sol, ref, 1 - 1.0 / 256, trace)
+
+
+def test_full_size_mlp_against_the_aten_oracle_at_the_stated_bar():
+    """The neural ODE configuration at its full size, B = 4096: ys within 1e-4 and integer stats identical on at
+    least 99.9 % of the samples against the loop as ATen operations on the host; differing samples are counted,
+    printed with their error ratios, and must be borderline accept decisions where their stats differ."""
+    w = to.workloads.make("mlp")
+    assert w.y0.shape == (4096, 64) and w.t_eval.shape == (4096, 20)
+    sol = device_solve(w)
+    from torchode_amd import _lib
+
+    assert _lib.last_solve_kernel_name() == "tode::solve_mlp_kernel"
+    assert (sol.status == 0).all() and (sol.stats["n_initialized"] == 20).all() and torch.isfinite(sol.ys).all()
+    ref, trace = oracle_with_trace(w)
+    assert sol.stats["n_f_evals"].tolist() == ref["n_f_evals"].tolist()
+    compare(sol, ref, 0.999, trace)
+    # batch composition: a strided subset on its own takes the same steps and gives the same bits
+    idx = torch.arange(3, 4096, 37)
+    sub = device_solve(w._replace(y0=w.y0[idx], t_eval=w.t_eval[idx]))
+    assert torch.equal(sub.ys.cpu(), sol.ys.cpu()[idx]) and torch.equal(sub.stats["n_steps"].cpu(), sol.stats["n_steps"].cpu()[idx])
+
+
+def test_full_size_reaction_diffusion():
+    """The reaction-diffusion configuration at its full size, B = 512 (839 MB of ys): size-independent properties on
+    the whole batch; the first 16 samples against the committed ATen-oracle vectors, against the ATen oracle live and
+    bit for bit against the protocol path and against a solve of those 16 samples alone."""
+    import json
+    import os
+
+    w = to.workloads.make("reaction_diffusion")
+    assert w.y0.shape == (512, 4096) and w.t_eval.shape == (512, 100)
+    sol = device_solve(w)
+    from torchode_amd import _lib
+
+    assert _lib.last_solve_kernel_name() == "tode::solve_grid_kernel"
+    assert sol.ys.shape == (512, 100, 4096) and (sol.status == 0).all() and (sol.stats["n_initialized"] == 100).all()
+    assert (sol.stats["n_accepted"] <= sol.stats["n_steps"]).all() and sol.stats["n_f_evals"][0].item() == 2 + 6 * sol.stats["n_steps"].max().item()
+    assert torch.equal(sol.ys[:, 0].cpu(), w.y0) and torch.isfinite(sol.ys).all()
+    mean = sol.ys.mean(dim=2)  # d/dt sum(u) = sum(u (1 - u)) > 0 under the periodic stencil
+    assert (mean[:, 1:] >= mean[:, :-1]).all() and (sol.ys.amin() >= 0) and (sol.ys.amax() <= 1.0 + 1e-5)
+    n = 16
+    head = w._replace(y0=w.y0[:n], t_eval=w.t_eval[:n], f=to.ReactionDiffusion(w.f.D[:n]))
+    alone = device_solve(head)
+    assert torch.equal(alone.ys, sol.ys[:n]) and torch.equal(alone.stats["n_steps"], sol.stats["n_steps"][:n])
+    proto = to.AutoDiffAdjoint(OwnTsit5(), make_controller(w.controller)).solve(
+        to.InitialValueProblem(head.y0.cuda(), t_eval=head.t_eval.cuda()), to.ODETerm(copy.deepcopy(head.f).cuda())
+    )
+    assert_same(alone, proto)
+    ref, trace = oracle_with_trace(head)
+    compare(alone, ref, 0.999, trace)
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reaction_diffusion_float32_b16_tolerance.json")))
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert sol.stats[key][:n].tolist() == gold[key], key
+    pts = torch.tensor(gold["ys_points"])
+    want = torch.tensor([float.fromhex(v) for v in gold["ys_values"]], dtype=torch.float64)
+    assert mixed_error(sol.ys[:n].cpu()[pts[:, 0], pts[:, 1], pts[:, 2]].double(), want) < 1e-4
 
 
 def test_batch_composition_does_not_matter():

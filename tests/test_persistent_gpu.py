@@ -339,6 +339,34 @@ def test_full_size_lorenz_prefix_against_oracle():
     assert torch.equal(sol.stats["n_steps"][:n].cpu(), ref["n_steps"])
 
 
+def test_full_size_vdp_float64_whole_batch_against_the_oracle():
+    """Van der Pol B = 65536 in float64: every ys value and every stat of all samples against the scalar C oracle
+    (OpenMP over the samples), then batch-composition independence on a strided subset."""
+    w = to.workloads.make("vdp", dtype=F64)
+    assert w.y0.shape == (65536, 2) and w.t_eval.shape == (65536, 50)
+    sol = gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert (sol.status == 0).all() and (sol.stats["n_initialized"] == 50).all() and torch.isfinite(sol.ys).all()
+    assert (sol.stats["n_accepted"] <= sol.stats["n_steps"]).all() and torch.equal(sol.ys[:, 0].cpu(), w.y0)
+    ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller, nthreads=16)
+    assert_identical(sol, ref)
+    idx = torch.arange(5, 65536, 101)
+    sub = gpu_solve(to.VanDerPol(w.f.mu[idx]), w.y0[idx], w.t_eval[idx], w.method, w.controller)
+    assert torch.equal(sub.ys.cpu(), sol.ys.cpu()[idx]) and torch.equal(sub.stats["n_steps"].cpu(), sol.stats["n_steps"].cpu()[idx])
+    # the general kernel on the same batch
+    assert_identical(gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller, fast=False), ref)
+
+
+def test_full_size_linear_decay_is_the_reference_configuration():
+    """Linear decay B = 256, F = 4, float64, Dopri5 + integral controller: the configuration the reference runs on
+    its CPU path.  Against the C oracle bit for bit and against the closed form y0 exp(-k t) at the tolerance."""
+    w = to.workloads.make("linear_decay")
+    assert w.y0.shape == (256, 4) and w.y0.dtype == F64 and w.t_eval.shape == (256, 10)
+    sol = gpu_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
+    assert_identical(sol, c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller))
+    exact = w.y0[:, None, :] * torch.exp(-w.f.k[:, None, :] * w.t_eval[:, :, None])
+    assert (sol.ys.cpu() - exact).abs().max().item() < 2e-3 * w.y0.abs().max().item()
+
+
 def test_time_reversal_round_trip():
     # reference tests/adjoint_test.py:322-347: solving back from the end state recovers y0
     w = to.workloads.make("linear_decay", batch=256, dtype=F64)
@@ -406,6 +434,29 @@ def test_gpu_matches_golden_fixture(path, fast):
     ys = sol.ys.cpu()
     assert [float(v).hex() for v in ys[g["subset"]].flatten().tolist()] == g["ys_subset"]
     assert float(ys.double().abs().max()).hex() == g["ys_max_abs"]
+
+
+def test_inputs_updated_in_place_between_two_solves_of_one_problem_object():
+    """A problem object may keep contiguous copies of inputs that are views (an expanded t_eval, a column slice as
+    y0); an in-place update of the original between two solves must reach the second solve."""
+    w = to.workloads.make("vdp", batch=512, dtype=F32, device="cuda")
+    wide = torch.cat([w.y0, torch.zeros_like(w.y0)], dim=1)  # y0 as a strided slice of a wider tensor
+    y0 = wide[:, :2]
+    row = w.t_eval[:1].clone()
+    t_eval = row.expand(512, -1)  # one row of evaluation times for all samples, stride 0
+    assert not y0.is_contiguous() and not t_eval.is_contiguous()
+    spec = dict(w.controller)
+    spec.pop("kind")
+    solver = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(**spec))
+    problem = to.InitialValueProblem(y0, t_eval=t_eval)
+    term = to.ODETerm(w.f)
+    first = solver.solve(problem, term)
+    wide[:, :2] *= 0.5
+    row[:, 1:] *= 0.75
+    second = solver.solve(problem, term)
+    fresh = solver.solve(to.InitialValueProblem(wide[:, :2].clone(), t_eval=row.expand(512, -1).clone()), term)
+    assert torch.equal(second.ys, fresh.ys) and torch.equal(second.stats["n_steps"], fresh.stats["n_steps"])
+    assert not torch.equal(first.ys, second.ys)
 
 
 _EARLY_STOP = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_early_stop.json")))

@@ -159,7 +159,8 @@ def test_graph_replay_equals_the_eager_loop_bit_for_bit(name, batch, dtype, n):
     ref = c_oracle_solve(w.f, w.y0, w.t_eval, w.method, w.controller)
     calls = []
     for _ in range(3):  # solves in a row, each with a graph of its own, other work in between
-        sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, graph=n, calls=calls)
+        with torch.no_grad():  # (under grad mode f is evaluated once more, to look for captured tensors that require grad)
+            sol = stepwise_solve(w.f, w.y0, w.t_eval, w.method, w.controller, graph=n, calls=calls)
         assert_identical(sol, ref)
         torch.cuda.synchronize()
         (torch.randn(1000, device="cuda") @ torch.randn(1000, device="cuda")).item()

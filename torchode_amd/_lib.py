@@ -33,6 +33,7 @@ STATIC_STAGING_BYTES = 2 << 20  # TODE_STATIC_STAGING_BYTES
 # every symbol include/torchode_amd.h declares
 EXPORTS = (
     "tode_abi_version",
+    "tode_source_hash",
     "tode_last_error",
     "tode_solve_builtin",
     "tode_solve_builtin_fast",
@@ -216,16 +217,36 @@ _lib = None
 
 
 def load():
-    """Returns the loaded library, building it first if the file is missing."""
+    """Returns the loaded library.  It is built first if the file is missing, and built again if it was made from
+    other sources than the ones lying next to it (the library carries a hash of its sources): an edited kernel is
+    never run through a stale binary.  Where the sources are absent (an installed copy) the file is taken as it is."""
     global _lib
     with _lock:
         if _lib is not None:
             return _lib
-        if not os.path.exists(LIB_PATH):
-            from . import build
+        from . import build
 
+        if not os.path.exists(LIB_PATH):
             build.build_library(force=True)
         lib = C.CDLL(LIB_PATH)
+        if os.path.isdir(build.CSRC):
+            want = build.source_hash()
+            lib.tode_source_hash.restype = C.c_char_p
+            got = lib.tode_source_hash().decode() if hasattr(lib, "tode_source_hash") else ""
+            if got != want:
+                # (a loaded library cannot be replaced in this process: build, then load the new file under a new name)
+                import shutil
+                import tempfile
+                import warnings
+
+                warnings.warn("libtorchode_amd.so was built from other sources than those in torchode_amd/csrc: rebuilding it")
+                build.build_library(force=True)
+                fresh = os.path.join(tempfile.mkdtemp(prefix="torchode_amd_"), "libtorchode_amd.so")
+                shutil.copy(LIB_PATH, fresh)
+                lib = C.CDLL(fresh)
+                lib.tode_source_hash.restype = C.c_char_p
+                if lib.tode_source_hash().decode() != want:
+                    raise RuntimeError("libtorchode_amd.so does not match its sources even after a rebuild")
         lib.tode_abi_version.restype = C.c_int
         lib.tode_last_error.restype = C.c_char_p
         lib.tode_solve_builtin.restype = C.c_int

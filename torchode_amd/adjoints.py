@@ -114,16 +114,21 @@ class AutoDiffAdjoint(nn.Module):
             or (problem.t_eval is not None and problem.t_eval.requires_grad)
             or (dt0 is not None and dt0.requires_grad)
         )
+        if grad_on and not wants_grad:
+            # a parameter or buffer of the term (the built-in terms keep mu, rho, k, D, the weights as buffers), a
+            # tensor in args, or one that f closes over: the reference's loop of torch operations carries gradients
+            # to all of them, so no kernel path that returns a result without a graph may take such a solve
+            from .autodiff import wants_grad_through_term
+
+            # (f is evaluated once to look for captured tensors, and only where the library's own step methods
+            # would call it: a user-defined method may never evaluate f at all)
+            wants_grad = wants_grad_through_term(term_, problem, args, probe=False)
+            if not wants_grad and not isinstance(getattr(term_, "f", None), BuiltinTerm) and self._library_setup(problem, term_, (Dopri5, Tsit5, Heun, Euler)):
+                wants_grad = wants_grad_through_term(term_, problem, args, probe=True)
         if not wants_grad and self._persistent_ok(problem, term_):
             sol = self._solve_persistent(problem, term_, dt0)
             if sol is not None:
                 return sol
-        if grad_on and not wants_grad and isinstance(term_, nn.Module):
-            wants_grad = any(p.requires_grad for p in term_.parameters())
-        if grad_on and not wants_grad and args is not None:
-            from .autodiff import tensor_leaves
-
-            wants_grad = any(a.requires_grad for a in tensor_leaves(args))
         if wants_grad:
             # gradients through the loop: forward in the per-step kernels (Dopri5, Tsit5) or on the operator
             # path (Heun, Euler) with a record of the loop state, backward by a reverse sweep over the record
@@ -451,11 +456,13 @@ class AutoDiffAdjoint(nn.Module):
     def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
         lib = _lib.load()
         f: BuiltinTerm = term.f
-        # What depends on the problem's tensors alone is worked out once per problem object and kept on it
-        # (checked by identity: the attributes of a problem may be reassigned).
+        # What depends on the problem's tensors alone is worked out once per problem object and kept on it (checked by
+        # identity, since the attributes of a problem may be reassigned, and by the tensors' version counters, since
+        # the plan may hold a contiguous copy of one of them that an in-place update of the original would not reach).
         tensors = (problem.y0, problem.t_start, problem.t_end, problem.t_eval)
+        versions = tuple(-1 if x is None else x._version for x in tensors)
         plan = getattr(problem, "_launch_plan", None)
-        if plan is None or any(a is not b for a, b in zip(plan[0], tensors)):
+        if plan is None or plan[-1] != versions or any(a is not b for a, b in zip(plan[0], tensors)):
             y0 = problem.y0.contiguous()
             # t_start / t_end are usually columns of t_eval: hand them over with their stride
             t_start, t_end = (t if t.stride(0) >= 1 else t.contiguous() for t in (problem.t_start, problem.t_end))
@@ -463,9 +470,9 @@ class AutoDiffAdjoint(nn.Module):
             ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
             plan = (tensors, y0, t_start, t_end, t_eval, ts, y0.device, y0.dtype, y0.shape[0], y0.shape[1], problem.n_evaluation_points,
                     y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0),
-                    None if t_eval is None else t_eval.data_ptr())  # fmt: skip
+                    None if t_eval is None else t_eval.data_ptr(), versions)  # fmt: skip
             problem._launch_plan = plan
-        _, y0, t_start, t_end, t_eval, ts, dev, dtype, B, F, E, y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr = plan
+        _, y0, t_start, t_end, t_eval, ts, dev, dtype, B, F, E, y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, _ = plan
         params = f.builtin_params().to(device=dev, dtype=dtype)
         if params.numel() == 0 and params.shape[0] != B:  # a term without per-sample parameters
             params = y0.new_empty((B, 0))

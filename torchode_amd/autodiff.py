@@ -52,6 +52,54 @@ def map_tensors(obj, fn):
     return obj
 
 
+def captured_leaves(term, problem: InitialValueProblem, args) -> List[torch.Tensor]:
+    """Leaf tensors that require grad and that ``f(t_start, y0)`` depends on without their being an argument of it:
+    what ``f`` closes over, and parameters or buffers of a module behind it (directly, or through tensors computed
+    from them).  Found by evaluating ``f`` once on detached inputs under grad mode and walking the graph of the result.
+    The reference's loop is torch operations throughout, so autograd reaches such tensors by itself
+    (adjoints.py:135-260); here they have to be named as differentiation targets of the reverse sweep."""
+    with torch.enable_grad():
+        y = problem.y0.detach().requires_grad_()
+        t = problem.t_start.detach()
+        # (args reaches f by identity, reference tests/extra_args_test.py:16-22; only tensors in it that require
+        # grad are swapped for detached ones, so that the walk stops at them: the caller names those itself)
+        plain_args = map_tensors(args, lambda a: a.detach()) if any(a.requires_grad for a in tensor_leaves(args)) else args
+        out = term.f(t, y, plain_args) if term.with_args else term.f(t, y)
+    found, seen, stack = [], set(), [getattr(out, "grad_fn", None)]
+    while stack:
+        fn = stack.pop()
+        if fn is None or fn in seen:
+            continue
+        seen.add(fn)
+        var = getattr(fn, "variable", None)  # AccumulateGrad nodes hold the leaf
+        if var is not None and var is not y and var.requires_grad and not any(var is v for v in found):
+            found.append(var)
+        stack.extend(nxt for nxt, _ in fn.next_functions)
+    return found
+
+
+def wants_grad_through_term(term, problem: InitialValueProblem, args, probe: bool = True) -> bool:
+    """True if a solve under grad mode has to be differentiable because of the term alone: a parameter or buffer of
+    it, a tensor in ``args``, or (looked for only with ``probe``, since it takes an evaluation of ``f``) a tensor its
+    ``f`` closes over requires grad."""
+    from .builtin_terms import BuiltinTerm
+
+    f = getattr(term, "f", None)
+    if isinstance(f, BuiltinTerm) and not term._parameters and not term._buffers and len(term._modules) == 1:
+        # the common fast case, without nn.Module's recursive iterators: a plain term around a built-in right-hand
+        # side, which holds all it uses as its own buffers
+        if any(b is not None and b.requires_grad for b in f._buffers.values()) or any(p is not None and p.requires_grad for p in f._parameters.values()):
+            return True
+        return bool(args is not None and any(a.requires_grad for a in tensor_leaves(args)))
+    if isinstance(term, torch.nn.Module) and (any(p.requires_grad for p in term.parameters()) or any(b.requires_grad for b in term.buffers())):
+        return True
+    if any(a.requires_grad for a in tensor_leaves(args)):
+        return True
+    if not probe or f is None or isinstance(f, BuiltinTerm):  # (a built-in term holds all it uses as buffers)
+        return False
+    return bool(captured_leaves(term, problem, args))
+
+
 class LoopRecord:
     """State before each iteration (and after the last): what the forward pass hands to the backward pass."""
 
@@ -343,7 +391,7 @@ class SolveThroughLoop(torch.autograd.Function):
                     adj = {k: None for k in names}
                     continue
                 wrt = [live[k] for k in names] + params
-                grads = torch.autograd.grad(targets, wrt, cotangents, allow_unused=True)
+                grads = torch.autograd.grad(targets, wrt, cotangents, allow_unused=True, retain_graph=True)
             adj = dict(zip(names, grads[: len(names)]))
             for i, g in enumerate(grads[len(names) :]):
                 grad_params[i] = add(grad_params[i], g)
@@ -372,7 +420,7 @@ class SolveThroughLoop(torch.autograd.Function):
                     cotangents.append(adj["dt"])
             grad_y0 = None
             if targets:
-                grads = torch.autograd.grad(targets, [y_in] + params, cotangents, allow_unused=True)
+                grads = torch.autograd.grad(targets, [y_in] + params, cotangents, allow_unused=True, retain_graph=True)
                 grad_y0 = grads[0]
                 for i, g in enumerate(grads[1:]):
                     grad_params[i] = add(grad_params[i], g)
@@ -388,7 +436,9 @@ def solve(adjoint, problem: InitialValueProblem, term, dt0: Optional[torch.Tenso
     from .solution import Solution
 
     params = [p for p in term.parameters() if p.requires_grad]
-    for extra in tensor_leaves(args) + [problem.t_start, problem.t_end, problem.t_eval, dt0]:
+    # buffers that require grad (the built-in terms keep their parameters as buffers) and what f closes over, down
+    # to the leaves they were computed from; then the tensors handed in by the caller
+    for extra in captured_leaves(term, problem, args) + tensor_leaves(args) + [problem.t_start, problem.t_end, problem.t_eval, dt0]:
         if extra is not None and extra.requires_grad and not any(extra is p for p in params):
             params.append(extra)
     ys, status, n_steps, n_accepted, n_initialized, n_f_evals = SolveThroughLoop.apply(adjoint, problem, term, dt0, args, problem.y0, *params)

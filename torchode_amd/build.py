@@ -48,6 +48,23 @@ UNITS = [
 ]
 
 
+def source_hash() -> str:
+    """sha256 over the library's sources (csrc/*, include/torchode_amd.h) and the compiler flags, in a fixed order.
+    Compiled into the library (``tode_source_hash``) so that a loader can tell whether the file it found was built
+    from the sources lying next to it."""
+    import hashlib
+
+    h = hashlib.sha256()
+    files = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith((".hip", ".h")))
+    files.append(os.path.join(os.path.dirname(HERE), "include", "torchode_amd.h"))
+    for path in files:
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    h.update(repr((FLAGS, UNITS)).encode())
+    return h.hexdigest()
+
+
 def _hipcc():
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -71,9 +88,13 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()
 
+    digest = source_hash()
+
     def compile_unit(unit):
         src, obj, defs = unit
         out = os.path.join(OBJ, obj)
+        if src == "tode_api.hip":
+            defs = [*defs, f'-DTODE_SOURCE_HASH="{digest}"']
         msg = _run([hipcc, *FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", out])
         if verbose and msg.strip():
             print(msg, file=sys.stderr)

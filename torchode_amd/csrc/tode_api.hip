@@ -204,6 +204,11 @@ extern "C" {
 
 int tode_abi_version(void) { return TODE_ABI_VERSION; }
 
+#ifndef TODE_SOURCE_HASH
+#define TODE_SOURCE_HASH ""
+#endif
+const char *tode_source_hash(void) { return TODE_SOURCE_HASH; }
+
 const char *tode_last_error(void) { return tode::g_error; }
 
 int tode_set_fast_kernel_variant(int variant) {
