@@ -1,21 +1,32 @@
 #!/usr/bin/env python3
 """Benchmark of the batch-parallel adaptive RK solve loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|f64] [--path auto|per-step]
-                    [--workload vdp|lorenz|linear_decay|reaction_diffusion|mlp]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]                 the headline + every other configuration
+    python bench.py --workload vdp|lorenz|linear_decay|reaction_diffusion|mlp [--dtype f32|f64] [--path auto|per-step] ...
+                                                                         one configuration alone (what the profiles run)
 
 A "step" is one full solve of the workload's batch (start step, adaptive loop,
 dense output, stats) with inputs resident in HBM.  Prints ONE JSON line.
 
-* value        RK sample-steps per second (sum over samples of attempted steps / wall time);
-               `ivps_per_s` and `equiv_hbm_gbps` are the other two figures of the metric.
+* value        RK sample-steps per second (sum over samples of attempted steps / wall time) of the
+               headline configuration, Van der Pol B = 65536 float32 Tsit5 + PID; `ivps_per_s` and
+               `equiv_hbm_gbps` are the other two figures of the metric.
 * roofline     dominant kernel = the persistent solve kernel.  `achieved` = algorithmic bytes
                of one launch (sum_b n_steps[b] * bytes_step + B * bytes_dense) divided by the
                kernel's average duration, measured with HIP events recorded around the kernel
-               on the stream it is launched on.
+               on the stream it is launched on.  The neural ODE is bounded by the matrix cores
+               instead: algorithmic flops per launch over the same duration.
 * cpu_baseline the same loop issued as ATen CPU operations (oracle/torch_loop.py, the closest
-               stand-in for running the reference on the host), all host cores, on a bounded
-               prefix of the batch; `cpu_baseline_scalar_c` is the scalar C oracle with OpenMP.
+               stand-in for running the reference on the host) on the host cores this process
+               may use, on a bounded prefix of the batch; `cpu_baseline_compiled` is the same
+               function under torch.compile (what the reference's README recommends), its compile
+               time reported and not counted; `cpu_baseline_scalar_c` is the scalar C oracle
+               with OpenMP.  Reported baselines, not targets.
+* configs      without --workload: the same measurement (value, roofline, cpu_baseline, ...) for
+               each of the other configurations -- linear decay float64, Van der Pol float64,
+               Lorenz, the neural ODE with float32 and with bfloat16 matrix-core inputs,
+               reaction-diffusion -- each at its full size.  Compiled CPU legs are taken in this
+               order while the run's time budget lasts; one that did not fit says so.
 """
 import argparse
 import json
@@ -29,8 +40,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 MFMA_FP32_PEAK_TFLOPS = 157.3
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch of the solve kernel at the default workload, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
+# HBM bytes per launch of the solve kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); absent (null in the output) where not measured.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6873.0 KiB x 2.000 + 32671.0 KiB x 1.000) x 1024
     ("vdp", "torch.float32", 65536): 47.53e6,
@@ -42,46 +53,30 @@ MEASURED_TRAFFIC_BYTES = {
     ("mlp", "torch.float32", 4096): 24.19e6,
 }
 
+# (workload, dtype flag, matrix-core inputs of the neural ODE) after the headline, in the order their compiled CPU legs are taken
+OTHER_CONFIGS = [
+    ("linear_decay", "f64", "float32"),
+    ("vdp", "f64", "float32"),
+    ("lorenz", "f32", "float32"),
+    ("mlp", "f32", "float32"),
+    ("reaction_diffusion", "f32", "float32"),
+    ("mlp", "f32", "bfloat16"),
+]
+START = time.perf_counter()
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="vdp", choices=["vdp", "lorenz", "linear_decay", "reaction_diffusion", "mlp"])
-    ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
-    ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument(
-        "--path",
-        default="auto",
-        choices=["auto", "per-step"],
-        help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
-    )
-    ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
-    ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
-    ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the baseline's sample is sized to")
-    ap.add_argument(
-        "--calibration-copy-mib",
-        type=int,
-        default=0,
-        help="also run one plain device copy of this many MiB (a known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)",
-    )
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (with more GPUs the batch axis would be split, every GPU solving its own samples)")
 
+def measure(args, name, dtype_flag, mlp_inputs, steps, warmup):
+    """One configuration on the GPU: wall time of `steps` solves, kernel time by HIP events, roofline."""
     import torch
 
     import torchode_amd as to
     from torchode_amd import _lib
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dtype = {None: None, "f32": torch.float32, "f64": torch.float64}[args.dtype]
-    w = to.workloads.make(args.workload, batch=args.batch, dtype=dtype, device="cuda")
+    dtype = {None: None, "f32": torch.float32, "f64": torch.float64}[dtype_flag]
+    w = to.workloads.make(name, batch=args.batch, dtype=dtype, device="cuda")
     dtype = w.y0.dtype
     if w.name == "mlp":
-        w.f.matrix_inputs = args.mlp_inputs
+        w.f.matrix_inputs = mlp_inputs
     B, F = w.y0.shape
     E = w.t_eval.shape[1]
     spec = dict(w.controller)
@@ -91,45 +86,38 @@ def main():
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
     term = to.ODETerm(w.f if args.path == "auto" else (lambda t, y, f=w.f: f(t, y)))
 
-    if args.calibration_copy_mib:
-        src = torch.ones(args.calibration_copy_mib * 2**20 // 4, dtype=torch.float32, device="cuda")
-        dst = torch.empty_like(src)
+    with torch.no_grad():  # a forward solve: nothing here asks for gradients
+        for _ in range(warmup):
+            sol = solver.solve(problem, term)
         torch.cuda.synchronize()
-        dst.copy_(src)  # reads and writes exactly calibration_copy_mib MiB
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            sol = solver.solve(problem, term)
         torch.cuda.synchronize()
-        del src, dst
+        wall = (time.perf_counter() - t0) / steps
 
-    for _ in range(args.warmup):
-        sol = solver.solve(problem, term)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        sol = solver.solve(problem, term)
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / args.steps
+        assert (sol.status == 0).all(), "benchmark solve did not succeed"
+        sample_steps = int(sol.stats["n_steps"].sum().item())
+        algo_bytes = sample_steps * w.bytes_step + B * w.bytes_dense
 
-    assert (sol.status == 0).all(), "benchmark solve did not succeed"
-    sample_steps = int(sol.stats["n_steps"].sum().item())
-    algo_bytes = sample_steps * w.bytes_step + B * w.bytes_dense
-
-    # kernel-only duration: HIP events recorded by the library around the solve kernel
-    _lib.set_kernel_timing(True)
-    kms = []
-    try:
-        for _ in range(max(5, min(args.steps, 20))):
-            solver.solve(problem, term)
-            kms.append(_lib.last_solve_kernel_ms())
-        kernel_name = _lib.last_solve_kernel_name()
-        kernel_s = sum(kms) / len(kms) / 1e3
-    except RuntimeError:
-        # no whole-solve kernel for this workload: the solve is a sequence of per-call kernels
-        # around the torch right-hand side, and the figure below is over the whole solve
-        per_step = args.path == "per-step"
-        kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
-        if per_step and args.graph_iterations:
-            kernel_name += f", {args.graph_iterations} iterations per HIP graph replay"
-        kernel_s = wall
-    _lib.set_kernel_timing(False)
+        # kernel-only duration: HIP events recorded by the library around the solve kernel
+        _lib.set_kernel_timing(True)
+        kms = []
+        try:
+            for _ in range(max(5, min(steps, 20))):
+                solver.solve(problem, term)
+                kms.append(_lib.last_solve_kernel_ms())
+            kernel_name = _lib.last_solve_kernel_name()
+            kernel_s = sum(kms) / len(kms) / 1e3
+        except RuntimeError:
+            # no whole-solve kernel for this workload: the solve is a sequence of per-call kernels
+            # around the torch right-hand side, and the figure below is over the whole solve
+            per_step = args.path == "per-step"
+            kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
+            if per_step and args.graph_iterations:
+                kernel_name += f", {args.graph_iterations} iterations per HIP graph replay"
+            kernel_s = wall
+        _lib.set_kernel_timing(False)
     achieved = algo_bytes / kernel_s / 1e9
     roofline = {
         "bound": "hbm",
@@ -157,7 +145,7 @@ def main():
         flops_f = 2 * (Fin * H + H * F)
         flops = (2 * B + 6 * sample_steps) * flops_f + 5000 * sample_steps
         tflops = flops / kernel_s / 1e12
-        peak = MFMA_FP32_PEAK_TFLOPS if args.mlp_inputs == "float32" else MFMA_BF16_PEAK_TFLOPS
+        peak = MFMA_FP32_PEAK_TFLOPS if mlp_inputs == "float32" else MFMA_BF16_PEAK_TFLOPS
         roofline = {
             "bound": "mfma",
             "kernel": kernel_name,
@@ -165,25 +153,18 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": tflops / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)) if args.mlp_inputs == "float32" else None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)) if mlp_inputs == "float32" else None,
             "algorithmic_flops_per_launch": flops,
             "flops_per_rhs_evaluation_per_sample": flops_f,
             "kernel_ms": kernel_s * 1e3,
         }
-
-    out = {
-        "metric": "RK sample-steps/s (adaptive Tsit5/Dopri5 solve, whole batch)",
+    result = {
         "value": sample_steps / wall,
         "unit": "sample-steps/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": wall * 1e3,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": {torch.float32: "f32", torch.float64: "f64"}[dtype] + (" (bf16 matrix-core inputs)" if w.name == "mlp" and args.mlp_inputs == "bfloat16" else ""),
-        "data": "synthetic",
+        "dtype": {torch.float32: "f32", torch.float64: "f64"}[dtype] + (" (bf16 matrix-core inputs)" if w.name == "mlp" and mlp_inputs == "bfloat16" else ""),
         "config": {
             "workload": f"{w.name} B={B} F={F} E={E} {w.method}+{kind}",
             "controller": w.controller,
@@ -194,23 +175,124 @@ def main():
         "equiv_hbm_gbps": algo_bytes / wall / 1e9,
         "roofline": roofline,
     }
+    del sol, problem, w
+    torch.cuda.empty_cache()
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=None, choices=[None, "vdp", "lorenz", "linear_decay", "reaction_diffusion", "mlp"],
+                    help="measure this configuration alone (default: the headline, Van der Pol float32, and then every other one under 'configs')")  # fmt: skip
+    ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
+    ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-compiled-baseline", action="store_true", help="skip the torch.compile CPU legs (about a minute of compilation each)")
+    ap.add_argument(
+        "--path",
+        default="auto",
+        choices=["auto", "per-step"],
+        help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
+    )
+    ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
+    ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
+    ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the headline's eager baseline is sized to (the other configurations take 0.4 of it)")
+    ap.add_argument("--time-budget", type=float, default=420.0, help="seconds the whole run aims to stay within: a compiled CPU leg is started only while 100 s of it are left")
+    ap.add_argument(
+        "--calibration-copy-mib",
+        type=int,
+        default=0,
+        help="also run one plain device copy of this many MiB (a known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)",
+    )
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (with more GPUs the batch axis would be split, every GPU solving its own samples)")
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+
+    if args.calibration_copy_mib:
+        src = torch.ones(args.calibration_copy_mib * 2**20 // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads and writes exactly calibration_copy_mib MiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    everything = args.workload is None
+    head = ("vdp", "f32", "float32") if everything else (args.workload, args.dtype, args.mlp_inputs)
+    result = measure(args, *head, args.steps, args.warmup)
+    out = {
+        "metric": "RK sample-steps/s (adaptive Tsit5/Dopri5 solve, whole batch)",
+        "value": result.pop("value"),
+        "unit": result.pop("unit"),
+        "n_gpus": 1,
+        "steps": result.pop("steps"),
+        "warmup": result.pop("warmup"),
+        "ms_per_step": result.pop("ms_per_step"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": result.pop("dtype"),
+        "data": "synthetic",
+        **result,
+    }
+    others = []
+    if everything:
+        for name, dtype_flag, mlp_inputs in OTHER_CONFIGS:
+            others.append(measure(args, name, dtype_flag, mlp_inputs, max(5, args.steps // 2), max(2, args.warmup // 2)))
 
     if not args.no_cpu_baseline:
-        out.update(cpu_baselines(args, w, sol))
+        # eager legs of every configuration first (seconds each), then the compiled legs while the budget lasts
+        plans = [(out, *head, args.cpu_baseline_seconds)] + [(o, *c, 0.4 * args.cpu_baseline_seconds) for o, c in zip(others, OTHER_CONFIGS)]
+        for entry, name, dtype_flag, mlp_inputs, seconds in plans:
+            entry.update(cpu_baselines(args, name, dtype_flag, mlp_inputs, seconds))
+        for entry, name, dtype_flag, mlp_inputs, seconds in plans:
+            if args.no_compiled_baseline:
+                entry["cpu_baseline_compiled"] = {"skipped": "--no-compiled-baseline"}
+            elif args.time_budget - (time.perf_counter() - START) < 100.0:
+                entry["cpu_baseline_compiled"] = {"skipped": f"the run's time budget of {args.time_budget:.0f} s leaves no room for another compilation (about a minute each)"}
+            else:
+                entry["cpu_baseline_compiled"] = compiled_baseline(args, name, dtype_flag, mlp_inputs, entry["cpu_baseline"])
+    if everything:
+        out["configs"] = others
+    out["bench_seconds"] = time.perf_counter() - START
     print(json.dumps(out))
 
 
-def cpu_baselines(args, w, sol):
-    """Host-core baselines on a bounded prefix of the same workload."""
+def host_threads():
+    """Threads the CPU legs use: torch's default, which follows OMP_NUM_THREADS / the cores this process may use."""
+    import torch
+
+    return torch.get_num_threads()
+
+
+def cpu_workload(name, dtype_flag, mlp_inputs, batch):
     import torch
 
     import torchode_amd as to
+
+    dtype = {None: None, "f32": torch.float32, "f64": torch.float64}[dtype_flag]
+    w = to.workloads.make(name, batch=batch, dtype=dtype)
+    if name == "mlp":
+        w.f.matrix_inputs = mlp_inputs
+    return w
+
+
+def cpu_baselines(args, name, dtype_flag, mlp_inputs, seconds):
+    """Host-core baselines on a bounded prefix of the same workload."""
+    import torch
+
     from oracle import c_oracle, torch_loop
 
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
-    B = w.y0.shape[0]
-    ww = to.workloads.make(w.name, batch=min(B, {"reaction_diffusion": 8, "mlp": 256}.get(w.name, 2048)), dtype=w.y0.dtype)
+    cores = host_threads()
+    full = cpu_workload(name, dtype_flag, mlp_inputs, args.batch)
+    B = full.y0.shape[0]
+    ww = cpu_workload(name, dtype_flag, mlp_inputs, min(B, {"reaction_diffusion": 8, "mlp": 256}.get(name, 2048)))
     ctrl = torch_loop.Controller(**ww.controller)
     torch_loop.solve(ww.f, ww.y0, ww.t_eval, method=ww.method, controller=ctrl)  # warm up
     t0 = time.perf_counter()
@@ -218,10 +300,10 @@ def cpu_baselines(args, w, sol):
     per_sample = (time.perf_counter() - t0) / ww.y0.shape[0]
     # the loop's cost per iteration has a fixed part, so small batches overestimate the cost per
     # sample: the sample below is sized generously and the time actually taken is reported
-    n = int(min(B, max(ww.y0.shape[0], 2 * args.cpu_baseline_seconds / per_sample)))
-    wc = to.workloads.make(w.name, batch=n, dtype=w.y0.dtype)
+    n = int(min(B, max(ww.y0.shape[0], 2 * seconds / per_sample)))
+    wc = cpu_workload(name, dtype_flag, mlp_inputs, n)
     t_torch, steps_n, solves = 0.0, 0, 0
-    while solves == 0 or (t_torch < 0.8 * args.cpu_baseline_seconds and solves < 64):  # whole workload too short: repeat it
+    while solves == 0 or (t_torch < 0.8 * seconds and solves < 64):  # whole workload too short: repeat it
         t0 = time.perf_counter()
         ref = torch_loop.solve(wc.f, wc.y0, wc.t_eval, method=wc.method, controller=ctrl)
         t_torch += time.perf_counter() - t0
@@ -233,16 +315,17 @@ def cpu_baselines(args, w, sol):
             "value": steps_n / t_torch,
             "unit": "sample-steps/s",
             "cores": cores,
+            "host_cpu_count": os.cpu_count(),
             "kind": "port",
             "sample": f"first {n} of {B} samples of the workload, {solves} eager solve(s) of the ATen-op restatement (torch {torch.__version__})",
+            "sample_batch": n,
             "seconds": t_torch,
         }
     }
-    if w.name not in c_oracle.TERMS:
+    if name not in c_oracle.TERMS:
         return first
-    name = w.name
     nc = min(B, 262144)
-    wc2 = to.workloads.make(w.name, batch=nc, dtype=w.y0.dtype)
+    wc2 = cpu_workload(name, dtype_flag, mlp_inputs, nc)
     cfg = c_oracle.make_config(method=wc2.method, term=name, nthreads=cores, **wc2.controller)
     c_oracle.solve(cfg, ww.f.builtin_params(), ww.y0, ww.t_eval)
     t0 = time.perf_counter()
@@ -258,6 +341,53 @@ def cpu_baselines(args, w, sol):
             "sample": f"first {nc} of {B} samples, one solve of the scalar C oracle (OpenMP over samples)",
             "seconds": t_c,
         },
+    }
+
+
+def compiled_baseline(args, name, dtype_flag, mlp_inputs, eager):
+    """The eager leg's function under torch.compile, on the eager leg's sample.  The reference recommends compiling
+    the solver (its README; its loop has a data-dependent end, so the compiled function is a chain of graphs with a
+    break per iteration).  Compilation happens in the first call and is reported, not counted.  A host on which the
+    compiler cannot run gives {"error": first line of the failure}."""
+    import torch
+
+    from oracle import torch_loop
+
+    wc = cpu_workload(name, dtype_flag, mlp_inputs, eager["sample_batch"])
+    ctrl = torch_loop.Controller(**wc.controller)
+
+    def run(f, y0, t_eval):
+        return torch_loop.solve(f, y0, t_eval, method=wc.method, controller=ctrl)
+
+    try:
+        import torch._dynamo
+
+        torch._dynamo.reset()
+        torch._dynamo.config.cache_size_limit = 64
+        compiled = torch.compile(run)
+        t0 = time.perf_counter()
+        out = compiled(wc.f, wc.y0, wc.t_eval)
+        t_compile = time.perf_counter() - t0
+        want = max(1.0, min(eager["seconds"], 6.0))
+        t_run, steps_n, solves = 0.0, 0, 0
+        while solves == 0 or (t_run < want and solves < 64):
+            t0 = time.perf_counter()
+            out = compiled(wc.f, wc.y0, wc.t_eval)
+            t_run += time.perf_counter() - t0
+            steps_n += int(out["n_steps"].sum())
+            solves += 1
+    except Exception as e:  # noqa: BLE001 -- whatever the compiler stack raises on this host is the result
+        text = str(e).strip().splitlines()
+        return {"error": f"{type(e).__name__}: {text[0][:300] if text else ''}"}
+    return {
+        "value": steps_n / t_run,
+        "unit": "sample-steps/s",
+        "cores": eager["cores"],
+        "kind": "port",
+        "sample": f"first {eager['sample_batch']} samples of the workload, {solves} solve(s) of torch.compile(the ATen-op restatement) after a first call of {t_compile:.0f} s that compiled it",
+        "seconds": t_run,
+        "compile_seconds": t_compile,
+        "speedup_over_eager": (steps_n / t_run) / eager["value"],
     }
 
 
