@@ -204,6 +204,32 @@ template <typename T> __device__ __forceinline__ T powk(DW<T> lg, T y) {
     return (r != r) ? (T)__builtin_huge_val() : r;
 }
 
+// The step factor's powers (step_size_controllers.py:289-294, 598-620) for the kernels that keep
+// the history of accepted error ratios as logarithms: safety * ratio^e1 [* prev^e2 [* prev_prev^e3]],
+// multiplied in this order.  `ratio` is positive and finite.  NHIST = number of history factors.
+template <typename T, int NHIST> struct StepFactor {
+    DW<T> lg, lg_prev, lg_pprev;
+    __device__ __forceinline__ StepFactor() : lg(dw((T)0, (T)0)), lg_prev(dw((T)0, (T)0)), lg_pprev(dw((T)0, (T)0)) {}
+    __device__ __forceinline__ T operator()(T safety, T ratio, T e1, T e2, T e3, bool) {
+        lg = logk(ratio);
+        T factor = safety * powk<T>(lg, e1);
+        if (NHIST >= 1) factor = factor * powk<T>(lg_prev, e2);
+        if (NHIST >= 2) factor = factor * powk<T>(lg_pprev, e3);
+        return factor;
+    }
+    // the ratio just used becomes the previous one where `shift` (an accepted step of a running sample)
+    __device__ __forceinline__ void shift(bool s) {
+        if (NHIST >= 2) {
+            lg_pprev.x = s ? lg_prev.x : lg_pprev.x;
+            lg_pprev.y = s ? lg_prev.y : lg_pprev.y;
+        }
+        if (NHIST >= 1) {
+            lg_prev.x = s ? lg.x : lg_prev.x;
+            lg_prev.y = s ? lg.y : lg_prev.y;
+        }
+    }
+};
+
 // x ** y for x >= 0 or NaN, all special cases included.
 template <typename T> __device__ __forceinline__ T pow_(T x, T y) {
     if (y == (T)0 || x == (T)1) return (T)1;
@@ -342,7 +368,9 @@ template <typename T, int F> __device__ __forceinline__ T rms(const T (&v)[F]) {
 // (einsum "b, s, sbf -> bf" on the small-matrix path, F <= 57).  The weights are
 // row ROW of Tab::w, or Tab::b_err for ROW < 0; they are named by template
 // arguments so that the float64 -> T conversion happens at compile time.
-template <typename T, int F, typename Tab, int ROW>
+// With MAGNITUDE_ONLY the first product is taken as it is instead of being added to zero: the
+// two differ in the sign of a zero sum at most, which a caller that only uses |out| never sees.
+template <typename T, int F, typename Tab, int ROW, bool MAGNITUDE_ONLY = false>
 __device__ __forceinline__ void weighted_k(T dt, const T (&k)[7][F], T (&out)[F]) {
 #pragma unroll
     for (int f = 0; f < F; ++f) out[f] = 0;
@@ -354,7 +382,7 @@ __device__ __forceinline__ void weighted_k(T dt, const T (&k)[7][F], T (&out)[F]
 #pragma unroll
         for (int f = 0; f < F; ++f) {
             T pk = p * k[s][f];
-            out[f] = out[f] + pk;
+            out[f] = (MAGNITUDE_ONLY && s == 0) ? pk : out[f] + pk;
         }
     }
 }
@@ -371,6 +399,79 @@ __device__ __forceinline__ T error_ratio(const CtrlParams<T> &cp, const T (&y0)[
     }
     return tmax(rms<T, F>(q), (T)1e-38);
 }
+
+// x / sqrt(F) as the reference divides (a true division by the rounded square root), in fewer
+// instructions where that is provably the same value: fast() for arguments of at least 2^-100 (or
+// zero), exact() for any.  F == 1 and F == 4 are exact scalings.  For
+// float32 and F == 2, 3 the quotient by the constant c = float(sqrt(F)) is q = x * (1/c) corrected
+// once through the exact remainder: fma(fma(-q, c, x), 1/c, q).  That equals the correctly rounded
+// x / c for every float32 mantissa (verified exhaustively for both constants), provided the
+// remainder is exact, i.e. nothing underflows: arguments below 2^-100 take the division.
+template <typename T, int F> struct DivSqrtFeatures {
+    static constexpr bool corrected = false;
+    static __device__ __forceinline__ T fast(T x) {
+        if (F == 1) return x;
+        if (F == 4) return x * (T)0.5;
+        return x / (T)__builtin_sqrt((double)F);
+    }
+    static __device__ __forceinline__ T exact(T x) { return fast(x); }
+};
+template <int F> struct DivSqrtConstant {};
+template <> struct DivSqrtConstant<2> { static constexpr float c = 1.41421354f, rc = 0x1.6a09e6p-1f; };
+template <> struct DivSqrtConstant<3> { static constexpr float c = 1.73205078f, rc = 0x1.279a74p-1f; };
+template <int F> struct DivSqrtCorrected {
+    static constexpr bool corrected = true;
+    static __device__ __forceinline__ float fast(float x) {
+        const float q = x * DivSqrtConstant<F>::rc;
+        return fma_(fma_(-q, DivSqrtConstant<F>::c, x), DivSqrtConstant<F>::rc, q);
+    }
+    static __device__ __forceinline__ float exact(float x) { return x / DivSqrtConstant<F>::c; }
+};
+template <> struct DivSqrtFeatures<float, 2> : DivSqrtCorrected<2> {};
+template <> struct DivSqrtFeatures<float, 3> : DivSqrtCorrected<3> {};
+
+// Error ratio for the kernels that cover the common case only (and hand every batch with a
+// non-finite value to the general kernel): the same operations as error_ratio() with the
+// hardware's maximum in place of the NaN-propagating one.  The two differ for a NaN operand alone;
+// `unordered` is raised for one (a NaN in y0, y1, err or the sum), and the caller must then leave
+// the common case rather than use the returned value.  An infinite operand takes the same path
+// through both.
+template <typename T, int F>
+__device__ __forceinline__ T error_ratio_common(const CtrlParams<T> &cp, const T (&y0)[F], const T (&y1)[F], const T (&err)[F],
+                                                bool &unordered) {
+    using Div = DivSqrtFeatures<T, F>;
+    T q[F], x[F];
+    bool nan = false, small = false;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        nan = nan || __builtin_isunordered(y0[f], y1[f]);
+        const T m = hwmax(abs_(y0[f]), abs_(y1[f]));
+        const T eb = fma_(cp.rtol, m, cp.atol);
+        q[f] = abs_(err[f]) / eb;
+        x[f] = Div::fast(q[f]);
+        if (Div::corrected) small = small || (q[f] < (T)0x1p-100f && q[f] > (T)0);
+    }
+    if (Div::corrected && __builtin_expect(__any(small), 0)) {  // (one branch for all features, after their divisions)
+#pragma unroll
+        for (int f = 0; f < F; ++f) x[f] = Div::exact(q[f]);
+    }
+    T acc = 0;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        if (F <= 3)
+            acc = fma_(x[f], x[f], acc);
+        else {
+            const T sq = x[f] * x[f];
+            acc = acc + sq;
+        }
+    }
+    const T r = sqrt_(acc);
+    unordered = nan || r != r;
+    return hwmax(r, (T)1e-38);
+}
+
+// clamp(x, lo, hi) for operands that are known not to be NaN.
+template <typename T> __device__ __forceinline__ T clamp_ordered(T x, T lo, T hi) { return hwmin(hwmax(x, lo), hi); }
 
 // dt factor (step_size_controllers.py:289-294, 598-620).
 template <typename T, int CTRL> __device__ __forceinline__ T dt_factor(const CtrlParams<T> &cp, T ratio, T prev, T prev_prev) {

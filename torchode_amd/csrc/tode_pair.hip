@@ -75,10 +75,18 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
             dt = initial_step<T, CTRL, Term>(cp, rhs, ts, y, dir, abs_(te - ts), k[0]);
         }
         dt = tclamp(dt, tlo - t, thi - t);
-        DW<T> lg_prev = dw((T)0, (T)0), lg_pprev = dw((T)0, (T)0);
+        StepFactor<T, NHIST> step_factor;  // with the logarithms of the previous two accepted error ratios (both start at 1)
         const T dte_end = dir * te;
         int n_steps = 0, n_acc = 0;
-        bool active = live, bail = false;
+        // The loop below uses the hardware's minimum and maximum, which is the reference's arithmetic as long as no
+        // operand is NaN: a sample that starts with a NaN or infinite time, step or state goes to the general kernel,
+        // and so does one that produces a non-finite error ratio, step factor or step later.
+        bool odd_start = !finite_(dt) || !finite_(ts) || !finite_(te);
+#pragma unroll
+        for (int f = 0; f < F; ++f) odd_start = odd_start || !finite_(y[f]) || !finite_(k[0][f]);
+        bool bail = live && odd_start;
+        bool active = live && !odd_start;
+        const int step_limit = p.max_steps < TODE_HARD_STEP_LIMIT ? p.max_steps : TODE_HARD_STEP_LIMIT;
         const T e1 = (T)cp.e1, e2 = (T)cp.e2, e3 = (T)cp.e3;
 
         for (int phase = 0;; ++phase) {
@@ -119,17 +127,16 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
 #pragma unroll
                     for (int f = 0; f < F; ++f) r[(4 + 2 * F + s * F + f) * 64] = k[s][f];
 
-                weighted_k<T, F, Tab, -1>(dt, k, err);
+                weighted_k<T, F, Tab, -1, true>(dt, k, err);
 
                 // ---- step size control (step_size_controllers.py:370-429, 715-774) ----
-                const T ratio = error_ratio<T, F>(cp, y, y1, err);
+                bool unordered;
+                const T ratio = error_ratio_common<T, F>(cp, y, y1, err, unordered);
                 const bool accept = ratio < (T)1;
-                const bool sane = ratio > (T)0 && ratio < (T)__builtin_huge_val();
-                const DW<T> lg = logk(sane ? ratio : (T)1);
-                T factor = cp.safety * powk<T>(lg, e1);
-                if (NHIST >= 1) factor = factor * powk<T>(lg_prev, e2);
-                if (NHIST >= 2) factor = factor * powk<T>(lg_pprev, e3);
-                factor = tclamp(factor, cp.fmin, cp.fmax);
+                bool sane = !unordered && ratio < (T)__builtin_huge_val();  // (the ratio is at least 1e-38)
+                T factor = step_factor(cp.safety, sane ? ratio : (T)1, e1, e2, e3, active);
+                sane = sane && factor == factor;  // (a product of an underflowed and an overflowed power)
+                factor = clamp_ordered(factor, cp.fmin, cp.fmax);
                 const T dt_next = dt * factor;
 
                 const bool move = accept && active;
@@ -150,25 +157,22 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                 t = t_new;
                 {
                     const T dtn = running_new ? dt_next : dt;
-                    const T dtc = tclamp(dtn, tlo - t, thi - t);
+                    const T dtc = clamp_ordered(dtn, tlo - t, thi - t);
                     dt = active ? dtc : dt;
                 }
-                if (NHIST >= 1) {
-                    const bool shift = active && running_new && accept;
-                    if (NHIST >= 2) {
-                        lg_pprev.x = shift ? lg_prev.x : lg_pprev.x;
-                        lg_pprev.y = shift ? lg_prev.y : lg_pprev.y;
-                    }
-                    lg_prev.x = shift ? lg.x : lg_prev.x;
-                    lg_prev.y = shift ? lg.y : lg_prev.y;
-                }
+                if (NHIST >= 1) step_factor.shift(active && running_new && accept);
                 {
-                    const bool failed = active && (!sane || n_steps >= p.max_steps || n_steps >= TODE_HARD_STEP_LIMIT);
+                    const bool failed = active && (!sane || n_steps >= step_limit);
                     const bool finished = active && !failed && !running_new;
-                    bool odd = !(t == te);
+                    if (__any(finished)) {
+                        // a sample that lands past t_end, or whose state or derivative at the end is not finite,
+                        // shows up in later iterations of the reference loop
+                        bool odd = !(t == te);
 #pragma unroll
-                    for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
-                    bail = bail || failed || (finished && odd);
+                        for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
+                        bail = bail || (finished && odd);
+                    }
+                    bail = bail || failed;
                     active = active && !failed && running_new;
                 }
             }
