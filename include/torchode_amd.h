@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 14
+#define TODE_ABI_VERSION 15
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -431,6 +431,69 @@ int tode_last_solve_kernel_ms(float *out_ms);
 /* Name of the solve kernel most recently launched by the calling thread ("" if none), e.g.
  * "tode::solve_pair_kernel"; the same for every template instance of a kernel. */
 const char *tode_last_solve_kernel_name(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Reverse of one loop iteration of the per-step kernels (gradients through the loop)
+ * ------------------------------------------------------------------------------------------
+ * Replaces what autograd does for the reference when AutoDiffAdjoint.solve runs under grad mode
+ * (reference adjoints.py:33-40, 111-113, 145-147: the loop is torch operations, recorded as they
+ * run).  The caller keeps the loop state of every iteration during the forward solve, walks the
+ * iterations in reverse and, for each, recomputes the stage values with tode_step_stage and its
+ * own f, then calls
+ *   tode_step_finish_backward        cotangents of the state after the iteration and of the
+ *                                    evaluation points it wrote  ->  g_k[0..6], g_y, g_y1, g_t,
+ *                                    g_dt, g_prev, g_pprev (overwritten) and the time gradients
+ *                                    (accumulated)
+ *   for s = 6 .. 1:
+ *       (g_ystage, g_tnode, ...) = vector-Jacobian product of the caller's f at stage s with g_k[s]
+ *       (for s = 6, g_ystage += g_y1)
+ *       tode_step_stage_backward(s)  adds to g_y, g_k[j < s], g_t, g_dt
+ * after which (g_y, g_k[0], g_t, g_dt, g_prev, g_pprev) are the cotangents of the state before the
+ * iteration.  Rows of fewer than 64 features: one thread per sample; longer rows: one wavefront per sample.
+ */
+typedef struct tode_step_adjoint {
+    int32_t dtype;           /* TODE_F32 | TODE_F64: data (y, k, history, their cotangents, grad_ys) */
+    int32_t time_dtype;      /* TODE_F32 | TODE_F64: times and steps and their cotangents */
+    int32_t method;          /* TODE_DOPRI5 | TODE_TSIT5 */
+    int32_t n_features;      /* F */
+    int32_t n_eval;          /* E; 0: the end point alone */
+    int32_t iteration;       /* index of this loop iteration */
+    int32_t through_control; /* 1: the proposed step is a function of the inputs (AutoDiffAdjoint's
+                                backprop_through_step_size_control, adjoints.py:111-113); 0: a constant */
+    int32_t end_point;       /* n_eval == 0 only: 1 in the loop's last iteration, whose interpolant gives ys */
+    int64_t batch;           /* B */
+    /* the problem and the forward values of the iteration */
+    const void *t_start, *t_end; /* [B] */
+    const void *t_eval;          /* [B,E] or NULL */
+    const void *t, *dt;          /* [B] state before the iteration */
+    const void *y;               /* [B,F] */
+    const void *ratio_prev, *ratio_pprev; /* [B] */
+    const int32_t *running;      /* [B] before the iteration (unused by the kernels, kept for callers' checks; may be NULL) */
+    const int32_t *moved;        /* [B] 1 where the step was accepted for a running sample */
+    const int32_t *running_next; /* [B] running after the iteration */
+    const void *k[7];            /* [B,F] each; k[0] is the state's FSAL derivative */
+    const void *y1;              /* [B,F] input of the last stage = the step's result */
+    const void *fixed_dt;        /* [B] TODE_CTRL_FIXED only */
+    const int32_t *hit_iteration;/* [B,E] iteration that wrote each evaluation point, -1 for none; NULL when E == 0 */
+    const void *grad_ys;         /* [B,max(E,1),F] cotangent of the solve's ys */
+    /* cotangents of the state after the iteration; NULL stands for zeros */
+    const void *a_t, *a_dt;      /* [B] */
+    const void *a_y, *a_k0;      /* [B,F] */
+    const void *a_prev, *a_pprev;/* [B] */
+    /* results, overwritten by tode_step_finish_backward and added to by tode_step_stage_backward */
+    void *g_k[7];                /* [B,F] each */
+    void *g_y, *g_y1;            /* [B,F] */
+    void *g_t, *g_dt;            /* [B] */
+    void *g_prev, *g_pprev;      /* [B] */
+    /* gradients of the problem's times, added to; NULL: not wanted */
+    void *g_t_start, *g_t_end;   /* [B] */
+    void *g_t_eval;              /* [B,E] */
+    void *g_fixed_dt;            /* [B] */
+} tode_step_adjoint;
+
+int tode_step_finish_backward(const tode_step_adjoint *adjoint, const tode_controller *controller, void *stream);
+int tode_step_stage_backward(const tode_step_adjoint *adjoint, const tode_controller *controller, int stage, const void *g_ystage,
+                             const void *g_tnode, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Protocol operators.

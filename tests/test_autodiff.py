@@ -455,6 +455,115 @@ def test_gradcheck_through_heun_and_euler(case):
     assert torch.autograd.gradcheck(loss, (y0, A, t_eval, dt0), atol=1e-5, check_undefined_grad=False)
 
 
+def _gradients(solver, make_inputs, weights_seed=0, **solve_kw):
+    """Gradients of a weighted sum of ys with respect to everything `make_inputs` marks, through `solver`."""
+    problem, term, leaves, extra = make_inputs()
+    sol = solver.solve(problem, term=term, **extra, **solve_kw)
+    g = torch.Generator().manual_seed(weights_seed)
+    weights = torch.randn(sol.ys.shape, generator=g, dtype=torch.float64).to(sol.ys)
+    (sol.ys * weights).sum().backward()
+    return [None if x.grad is None else x.grad.clone() for x in leaves], sol
+
+
+@gpu
+@pytest.mark.parametrize("through_control", [True, False], ids=["through-control", "steps-constant"])
+@pytest.mark.parametrize("case", ["tsit5-pid", "dopri5-integral", "tsit5-pid-limits", "dopri5-fixed", "tsit5-end-only", "dopri5-pid-times", "tsit5-mixed-t32", "dopri5-mixed-t64"])
+def test_reverse_kernels_agree_with_the_sweep_in_torch_operations(case, through_control):
+    """The reverse of an iteration in HIP kernels (tode_step_finish_backward / tode_step_stage_backward) against the
+    same iteration restated as torch operations and differentiated by autograd: gradients with respect to y0, the
+    parameters of f, the evaluation times, the ends of the time range and a fixed step, in both step methods, the
+    three controllers, with step limits, without evaluation points, backwards in time, and with time and data in
+    different dtypes."""
+    from torchode_amd import autodiff
+
+    torch.manual_seed(3)
+    B = 7
+    ydt = torch.float32 if case == "dopri5-mixed-t64" else torch.float64
+    tdt = torch.float32 if case == "tsit5-mixed-t32" else torch.float64
+
+    def make_inputs():
+        torch.manual_seed(11)
+        f = Forced().cuda().to(ydt)
+        y0 = torch.randn(B, 2, dtype=torch.float64, device="cuda").to(ydt).requires_grad_()
+        t_eval = (torch.linspace(0, 2.5, 6, dtype=torch.float64, device="cuda").repeat(B, 1) + torch.arange(B, dtype=torch.float64, device="cuda")[:, None] * 0.1).to(tdt)
+        t_eval[::3] = t_eval[::3].flip(1)  # every third sample runs backwards
+        leaves, extra = [y0, f.w], {}
+        if case == "tsit5-end-only":
+            t_start, t_end = t_eval[:, 0].clone().requires_grad_(), t_eval[:, -1].clone().requires_grad_()
+            problem = to.InitialValueProblem(y0, t_start=t_start, t_end=t_end)
+            leaves += [t_start, t_end]
+        elif case == "dopri5-pid-times":
+            t_eval = t_eval.clone().requires_grad_()
+            problem = to.InitialValueProblem(y0, t_eval=t_eval)
+            leaves += [t_eval]
+        else:
+            problem = to.InitialValueProblem(y0, t_eval=t_eval)
+        if case == "dopri5-fixed":
+            dt0 = ((t_eval[:, -1] - t_eval[:, 0]) / 17.3).detach().requires_grad_()
+            extra["dt0"] = dt0
+            leaves += [dt0]
+        return problem, to.ODETerm(f), leaves, extra
+
+    method = to.Tsit5 if case.startswith("tsit5") else to.Dopri5
+    if "fixed" in case:
+        controller = lambda: to.FixedStepController()
+    elif "limits" in case:
+        controller = lambda: to.PIDController(1e-5, 1e-4, 0.2, 0.5, 0.1, dt_min=1e-3, dt_max=0.2)
+    elif "integral" in case:
+        controller = lambda: to.IntegralController(1e-6, 1e-5)
+    else:
+        controller = lambda: to.PIDController(1e-6, 1e-5, 0.2, 0.5, 0.1)
+    results = {}
+    for kernels in (True, False):
+        solver = to.AutoDiffAdjoint(method(), controller(), backprop_through_step_size_control=through_control)
+        solver.backward_kernels = kernels
+        results[kernels], sol = _gradients(solver, make_inputs)
+        assert autodiff.LAST_SWEEP == ("kernels" if kernels else "torch")
+        assert (sol.stats["n_steps"] >= 3).all()
+    single = ydt == torch.float32 or tdt == torch.float32
+    for a, b in zip(results[True], results[False]):
+        assert (a is None) == (b is None)
+        if a is not None:
+            torch.testing.assert_close(a, b, rtol=5e-3 if single else 1e-9, atol=2e-3 if single else 1e-11)  # (float32: the two sweeps round differently, and the step size control amplifies it)
+            assert torch.isfinite(a).all() and a.abs().max() > 0
+
+
+@gpu
+@pytest.mark.parametrize("features", [64, 100, 300])
+@pytest.mark.parametrize("case", ["tsit5-pid", "dopri5-integral-end-only"])
+def test_reverse_kernels_on_long_rows(features, case):
+    """Rows of 64 features and more: the reverse kernels run one wavefront per sample; same gradients as the sweep in
+    torch operations (y0, the matrix of f, the times)."""
+    from torchode_amd import autodiff
+
+    B = 9
+
+    def make_inputs():
+        g = torch.Generator().manual_seed(features)
+        W = (torch.randn((features, features), generator=g, dtype=torch.float64) / features**0.5).cuda().requires_grad_()
+        y0 = torch.randn((B, features), generator=g, dtype=torch.float64).cuda().requires_grad_()
+        t_eval = (torch.linspace(0, 1.5, 5, dtype=torch.float64).repeat(B, 1) * (1 + 0.1 * torch.arange(B, dtype=torch.float64)[:, None])).cuda()
+        t_eval[1::2] = t_eval[1::2].flip(1)
+        f = lambda t, y: torch.tanh(y @ W) * torch.cos(t)[:, None] - 0.5 * y
+        if case.endswith("end-only"):
+            t_start, t_end = t_eval[:, 0].clone().requires_grad_(), t_eval[:, -1].clone().requires_grad_()
+            return to.InitialValueProblem(y0, t_start=t_start, t_end=t_end), to.ODETerm(f), [y0, W, t_start, t_end], {}
+        t_eval.requires_grad_()
+        return to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(f), [y0, W, t_eval], {}
+
+    method = to.Tsit5 if case.startswith("tsit5") else to.Dopri5
+    controller = (lambda: to.PIDController(1e-7, 1e-6, 0.2, 0.5, 0.1)) if "pid" in case else (lambda: to.IntegralController(1e-7, 1e-6))
+    results = {}
+    for kernels in (True, False):
+        solver = to.AutoDiffAdjoint(method(), controller())
+        solver.backward_kernels = kernels
+        results[kernels], sol = _gradients(solver, make_inputs)
+        assert autodiff.LAST_SWEEP == ("kernels" if kernels else "torch") and (sol.stats["n_steps"] >= 3).all()
+    for a, b in zip(results[True], results[False]):
+        torch.testing.assert_close(a, b, rtol=1e-8, atol=1e-11)
+        assert torch.isfinite(a).all() and a.abs().max() > 0
+
+
 @gpu
 def test_what_is_not_differentiated_says_so():
     y0, A = inputs()

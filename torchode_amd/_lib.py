@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -44,6 +44,8 @@ EXPORTS = (
     "tode_step_begin",
     "tode_step_stage",
     "tode_step_finish",
+    "tode_step_finish_backward",
+    "tode_step_stage_backward",
     "tode_step_stats",
     "tode_finalize_stats",
     "tode_set_fast_kernel_variant",
@@ -176,6 +178,55 @@ class StepState(C.Structure):
     ]
 
 
+class StepAdjoint(C.Structure):
+    """struct tode_step_adjoint"""
+
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("time_dtype", C.c_int32),
+        ("method", C.c_int32),
+        ("n_features", C.c_int32),
+        ("n_eval", C.c_int32),
+        ("iteration", C.c_int32),
+        ("through_control", C.c_int32),
+        ("end_point", C.c_int32),
+        ("batch", C.c_int64),
+        ("t_start", C.c_void_p),
+        ("t_end", C.c_void_p),
+        ("t_eval", C.c_void_p),
+        ("t", C.c_void_p),
+        ("dt", C.c_void_p),
+        ("y", C.c_void_p),
+        ("ratio_prev", C.c_void_p),
+        ("ratio_pprev", C.c_void_p),
+        ("running", C.c_void_p),
+        ("moved", C.c_void_p),
+        ("running_next", C.c_void_p),
+        ("k", C.c_void_p * 7),
+        ("y1", C.c_void_p),
+        ("fixed_dt", C.c_void_p),
+        ("hit_iteration", C.c_void_p),
+        ("grad_ys", C.c_void_p),
+        ("a_t", C.c_void_p),
+        ("a_dt", C.c_void_p),
+        ("a_y", C.c_void_p),
+        ("a_k0", C.c_void_p),
+        ("a_prev", C.c_void_p),
+        ("a_pprev", C.c_void_p),
+        ("g_k", C.c_void_p * 7),
+        ("g_y", C.c_void_p),
+        ("g_y1", C.c_void_p),
+        ("g_t", C.c_void_p),
+        ("g_dt", C.c_void_p),
+        ("g_prev", C.c_void_p),
+        ("g_pprev", C.c_void_p),
+        ("g_t_start", C.c_void_p),
+        ("g_t_end", C.c_void_p),
+        ("g_t_eval", C.c_void_p),
+        ("g_fixed_dt", C.c_void_p),
+    ]
+
+
 class LoopArgs(C.Structure):
     """struct tode_loop_args"""
 
@@ -265,6 +316,10 @@ def load():
         lib.tode_step_begin.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p, C.c_int, C.c_void_p]
         lib.tode_step_stage.restype = C.c_int
         lib.tode_step_stage.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_int, C.c_void_p]
+        lib.tode_step_finish_backward.restype = C.c_int
+        lib.tode_step_finish_backward.argtypes = [C.POINTER(StepAdjoint), C.POINTER(Controller), C.c_void_p]
+        lib.tode_step_stage_backward.restype = C.c_int
+        lib.tode_step_stage_backward.argtypes = [C.POINTER(StepAdjoint), C.POINTER(Controller), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.tode_step_finish.restype = C.c_int
         lib.tode_step_finish.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p]
         lib.tode_step_stats.restype = C.c_int

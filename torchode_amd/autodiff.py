@@ -5,12 +5,16 @@ decides whether the step sizes count as functions of the inputs).
 Here the forward pass runs in the per-step HIP kernels (Dopri5, Tsit5) or on the operator path
 (Heun, Euler) and keeps, per loop iteration, a copy of
 the small loop state (t, dt, y, the FSAL derivative, the controller history, two counters).  The
-backward pass walks the iterations in reverse: it restates one iteration as differentiable torch
-operations on the stored state -- same stages, error ratio, step size rule and dense output, with
-the accept / running / evaluation decisions taken from the record -- and pulls the cotangents of
-the next state and of the evaluation points back through it, which evaluates ``f`` and its
-vector-Jacobian products six times per iteration.  Memory: one state copy per iteration instead of
-the reference's whole operation graph.
+backward pass walks the iterations in reverse and pulls the cotangents of the next state and of
+the evaluation points back through each, with the accept / running / evaluation decisions taken
+from the record.  For Dopri5 / Tsit5 one iteration is reversed by HIP kernels
+(``reverse_sweep_kernels``: the stage values are recomputed by the forward stage kernel and ``f``,
+everything after the stages -- dense output, state update, step clamp, controller, error ratio --
+is one reverse kernel, each stage another; only ``f``'s own vector-Jacobian products are
+autograd's).  ``reverse_sweep_torch`` restates the iteration as differentiable torch operations
+instead (Heun and Euler, and the checker of the kernels in the tests).  Either way ``f`` is
+evaluated six times per iteration again.  Memory: one state copy per iteration instead of the
+reference's whole operation graph.
 
 Gradients flow to ``y0``, to the parameters of the term, to the tensors inside ``args`` (a
 tensor, or tuples / lists / dicts of them) and to the times (``t_start``, ``t_end``, ``t_eval``,
@@ -186,7 +190,8 @@ class Replay:
         return torch.maximum(self.t_start, self.t_end)
 
     def f(self, t, y):
-        return self.term.f(t, y, self.args) if self.term.with_args else self.term.f(t, y)
+        out = self.term.f(t, y, self.args) if self.term.with_args else self.term.f(t, y)
+        return out if out.dtype == y.dtype else out.to(y.dtype)  # (as the forward pass takes what f returns)
 
     def rms(self, x):
         return torch.linalg.vector_norm(x / sqrt(x.shape[1]), ord=2, dim=1)
@@ -252,7 +257,7 @@ class Replay:
         k0_new = torch.where(move[:, None], ks[-1], k0) if self.fsal else k0
         t_new = torch.where(move, t + dt, t)
         dt_new = torch.where(running_new, dt_next, dt)
-        dt_new = torch.minimum(torch.maximum(dt_new, self.t_lo - t_new), self.t_hi - t_new)
+        dt_new = torch.clamp(dt_new, self.t_lo - t_new, self.t_hi - t_new)  # (reference adjoints.py:251; its tie rules differ from minimum / maximum)
         keep = running_new & accept
         shift = self.pid and ratio is not None
         prev_new, pprev_new = (torch.where(keep, ratio, prev), torch.where(keep, prev, pprev)) if shift else (prev, pprev)
@@ -316,6 +321,203 @@ def simulate_hits(replay: Replay, states: Sequence[dict], n_eval: int):
     return hits
 
 
+STATE_NAMES = ("y", "k0", "t", "dt", "prev", "pprev")
+LAST_SWEEP = None  # "kernels" or "torch": what the most recent backward pass went through
+
+
+def _add(total, part):
+    return part if total is None else (total if part is None else total + part)
+
+
+def reverse_sweep_torch(replay: Replay, states, hits, grad_ys, params):
+    """The iterations in reverse, each restated as torch operations (Replay.iteration) and differentiated by
+    autograd.  Returns the cotangents of the state before the first iteration and the gradients of ``params``."""
+    names = STATE_NAMES
+    add = _add
+    adj = {k: None for k in names}
+    grad_params = [None] * len(params)
+    for n in range(len(states) - 2, -1, -1):
+        now, then = states[n], states[n + 1]
+        accept = (then["n_accepted"] - now["n_accepted"]) > 0
+        live = dict(now, running=now["running"] != 0)
+        with torch.enable_grad():
+            for k in names:
+                live[k] = now[k].detach().requires_grad_()
+            outs, values = replay.iteration(live, accept, then["running"] != 0, hits[n])
+            targets, cotangents = [], []
+            for k, out in zip(names, outs):
+                if adj[k] is not None and out.requires_grad:
+                    targets.append(out)
+                    cotangents.append(adj[k])
+            if values is not None:
+                rows, points = hits[n]
+                targets.append(values)
+                cotangents.append(grad_ys[rows, points] if points is not None else grad_ys[rows, 0])
+            if not targets:
+                adj = {k: None for k in names}
+                continue
+            wrt = [live[k] for k in names] + params
+            grads = torch.autograd.grad(targets, wrt, cotangents, allow_unused=True, retain_graph=True)
+        adj = dict(zip(names, grads[: len(names)]))
+        for i, g in enumerate(grads[len(names) :]):
+            grad_params[i] = add(grad_params[i], g)
+
+    return adj, grad_params
+
+
+def reverse_sweep_kernels(adjoint, replay: Replay, term, args, problem, dt0_given, dt0, states, hits, grad_ys, params, params_given):
+    """The iterations in reverse through the library's reverse kernels (tode_step_finish_backward,
+    tode_step_stage_backward): per iteration the stage values are recomputed by the forward stage kernel and ``f``
+    (six evaluations under grad mode, each a small graph of its own), the finish kernel is reversed in one launch,
+    and each stage in one launch after the vector-Jacobian product of ``f`` that autograd supplies.  Same result as
+    ``reverse_sweep_torch`` (the tests compare the two)."""
+    lib = _lib.load()
+    method, controller = adjoint.step_method, adjoint.step_size_controller
+    ctrl = controller.c_struct()
+    cref = _lib.C.byref(ctrl)
+    y0 = problem.y0
+    B, F = y0.shape
+    E = problem.n_evaluation_points
+    dev, dtype, ttype = y0.device, y0.dtype, replay.t_start.dtype
+    stream = _lib.stream_of(y0)
+    new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+    zeros = lambda *shape, dt=dtype: torch.zeros(shape, dtype=dt, device=dev)
+    contiguous = lambda x, dt: x.detach().to(dt).contiguous()
+    t_start, t_end = contiguous(replay.t_start, ttype), contiguous(replay.t_end, ttype)
+    t_eval = None if replay.t_eval is None else contiguous(replay.t_eval, ttype)
+    fixed = ctrl.kind == _lib.CTRL_FIXED
+    fixed_dt = contiguous(dt0, ttype) if fixed else None
+    n_iterations = len(states) - 1
+
+    # which iteration wrote which evaluation point
+    hit_iteration = None
+    if E > 0:
+        hit_iteration = torch.full((B, E), -1, dtype=torch.int32, device=dev)
+        for n, h in enumerate(hits):
+            if h is not None:
+                hit_iteration[h[0], h[1]] = n
+    grad_ys = contiguous(grad_ys, dtype)
+
+    # gradients of the times, collected by the kernels
+    wants = lambda x: x is not None and x.requires_grad
+    g_t_start = zeros(B, dt=ttype) if wants(replay.t_start) else None
+    g_t_end = zeros(B, dt=ttype) if wants(replay.t_end) else None
+    g_t_eval = zeros(B, E, dt=ttype) if (E > 0 and wants(replay.t_eval)) else None
+    g_fixed_dt = zeros(B, dt=ttype) if (fixed and wants(dt0) and replay.through_control) else None
+
+    # a scratch state for the forward stage kernel (it reads t, dt, y and the k's, and writes ystage / tnode)
+    st = _lib.StepState()
+    st.dtype, st.time_dtype, st.method, st.n_features, st.n_eval = _lib.DTYPES[dtype], _lib.DTYPES[ttype], method.method_id, F, 0
+    st.batch, st.max_steps = B, -1
+    clear = zeros(_lib.STEP_FLAG_WORDS, dt=torch.int32)
+    idle = zeros(B, dt=torch.int32)
+    st.flags = clear.data_ptr()
+    st.fixed_dt = _lib.ptr(fixed_dt)
+    st.t_start, st.t_end = t_start.data_ptr(), t_end.data_ptr()
+    for name in ("running", "cursor", "n_steps", "n_accepted", "status", "monotone"):
+        setattr(st, name, idle.data_ptr())
+    sref = _lib.C.byref(st)
+
+    ad = _lib.StepAdjoint()
+    ad.dtype, ad.time_dtype, ad.method, ad.n_features, ad.n_eval = st.dtype, st.time_dtype, st.method, F, E
+    ad.batch, ad.through_control = B, int(bool(replay.through_control))
+    ad.t_start, ad.t_end, ad.t_eval = t_start.data_ptr(), t_end.data_ptr(), _lib.ptr(t_eval)
+    ad.fixed_dt, ad.hit_iteration, ad.grad_ys = _lib.ptr(fixed_dt), _lib.ptr(hit_iteration), grad_ys.data_ptr()
+    ad.g_t_start, ad.g_t_end, ad.g_t_eval, ad.g_fixed_dt = _lib.ptr(g_t_start), _lib.ptr(g_t_end), _lib.ptr(g_t_eval), _lib.ptr(g_fixed_dt)
+    aref = _lib.C.byref(ad)
+
+    g_k = new(7, B, F)
+    g_y, g_y1 = new(B, F), new(B, F)
+    g_t, g_dt = new(B, dt=ttype), new(B, dt=ttype)
+    g_hist = new(2, B)
+    for i in range(7):
+        ad.g_k[i] = g_k[i].data_ptr()
+    ad.g_y, ad.g_y1, ad.g_t, ad.g_dt, ad.g_prev, ad.g_pprev = (x.data_ptr() for x in (g_y, g_y1, g_t, g_dt, g_hist[0], g_hist[1]))
+
+    f, with_args = term.f, term.with_args
+
+    def rhs(tt, yy):
+        out = f(tt, yy, args) if with_args else f(tt, yy)
+        if out.dtype != dtype or not out.is_contiguous() or out.shape != yy.shape:
+            out = out.to(dtype).expand(yy.shape).contiguous()
+        return out
+
+    adj = None  # cotangents of the state after the iteration at hand: (y, k0, t, dt, prev, pprev) or None for zeros
+    grad_params = [None] * len(params)
+    last = n_iterations - 1
+    for n in range(last, -1, -1):
+        has_hits = hits[n] is not None if E > 0 else n == last
+        if adj is None and not has_hits:
+            continue
+        now, then = states[n], states[n + 1]
+        moved = ((then["n_accepted"] - now["n_accepted"]) > 0).to(torch.int32)
+        running_next = (then["running"] != 0).to(torch.int32)
+        # ---- the stages again: forward kernels and f, keeping f's graphs ----
+        st.t, st.dt, st.y, st.k0 = (now[k].data_ptr() for k in ("t", "dt", "y", "k0"))
+        st.y0, st.ys = now["y"].data_ptr(), now["y"].data_ptr()  # (not used by the stage kernel)
+        st.ratio_prev, st.ratio_pprev = now["prev"].data_ptr(), now["pprev"].data_ptr()
+        st.k[0] = now["k0"].data_ptr()
+        ks, inputs = [now["k0"]], [None]
+        for i in range(1, 7):
+            yi, ti = new(B, F), new(B, dt=ttype)
+            st.ystage[i], st.tnode = yi.data_ptr(), ti.data_ptr()
+            _lib.check(lib.tode_step_stage(sref, cref, i, stream), "tode_step_stage")
+            with torch.enable_grad():
+                yi.requires_grad_()
+                ti.requires_grad_()
+                ki = rhs(ti, yi)
+            kd = ki.detach()
+            ks.append(kd)
+            inputs.append((yi, ti, ki))
+            st.k[i] = kd.data_ptr()
+        # ---- everything after the stages, reversed ----
+        ad.iteration, ad.end_point = n, int(E == 0 and n == last)
+        ad.t, ad.dt, ad.y = now["t"].data_ptr(), now["dt"].data_ptr(), now["y"].data_ptr()
+        ad.ratio_prev, ad.ratio_pprev = now["prev"].data_ptr(), now["pprev"].data_ptr()
+        ad.moved, ad.running_next = moved.data_ptr(), running_next.data_ptr()
+        for i in range(7):
+            ad.k[i] = ks[i].data_ptr()
+        ad.y1 = inputs[6][0].data_ptr()
+        names = ("a_y", "a_k0", "a_t", "a_dt", "a_prev", "a_pprev")
+        held = [None if adj is None else adj[j] for j in range(6)]
+        for name, value in zip(names, held):
+            setattr(ad, name, _lib.ptr(value))
+        _lib.check(lib.tode_step_finish_backward(aref, cref, stream), "tode_step_finish_backward")
+        # ---- the stages reversed: f's vector-Jacobian products by autograd, the sums by the kernel ----
+        for i in range(6, 0, -1):
+            yi, ti, ki = inputs[i]
+            if ki.requires_grad:
+                grads = torch.autograd.grad(ki, [yi, ti] + params, g_k[i], allow_unused=True, retain_graph=True)
+            else:
+                grads = [None] * (2 + len(params))
+            g_yi = grads[0] if grads[0] is not None else torch.zeros_like(yi)
+            if i == 6:
+                g_yi = g_yi + g_y1
+            g_ti = None if grads[1] is None else grads[1].to(ttype).contiguous()
+            _lib.check(lib.tode_step_stage_backward(aref, cref, i, g_yi.to(dtype).contiguous().data_ptr(), _lib.ptr(g_ti), stream), "tode_step_stage_backward")
+            for j, g in enumerate(grads[2:]):
+                grad_params[j] = _add(grad_params[j], g)
+        adj = (g_y.clone(), g_k[0].clone(), g_t.clone(), g_dt.clone(), g_hist[0].clone(), g_hist[1].clone())
+
+    # the gradients of the times go to the entries of `params` that stand for them
+    for given, collected in ((problem_time(replay, "t_start"), g_t_start), (problem_time(replay, "t_end"), g_t_end),
+                             (problem_time(replay, "t_eval"), g_t_eval), (dt0 if fixed else None, g_fixed_dt)):
+        if collected is None:
+            continue
+        for j, q in enumerate(params):
+            if q is given:
+                grad_params[j] = _add(grad_params[j], collected.to(q.dtype))
+                break
+    out = {k: None for k in STATE_NAMES}
+    if adj is not None:
+        out = dict(zip(STATE_NAMES, adj))
+    return out, grad_params
+
+
+def problem_time(replay: Replay, name: str):
+    return getattr(replay, name)
+
+
 class SolveThroughLoop(torch.autograd.Function):
     """Forward: the per-step kernels with a record.  Backward: the reverse sweep over it."""
 
@@ -363,38 +565,15 @@ class SolveThroughLoop(torch.autograd.Function):
         E = problem.n_evaluation_points
         hits = simulate_hits(replay, states, E)
         y0 = problem.y0
-        names = ("y", "k0", "t", "dt", "prev", "pprev")
-        adj = {k: None for k in names}
-        grad_params = [None] * len(params)
-
-        def add(total, part):
-            return part if total is None else (total if part is None else total + part)
-
-        for n in range(len(states) - 2, -1, -1):
-            now, then = states[n], states[n + 1]
-            accept = (then["n_accepted"] - now["n_accepted"]) > 0
-            live = dict(now, running=now["running"] != 0)
-            with torch.enable_grad():
-                for k in names:
-                    live[k] = now[k].detach().requires_grad_()
-                outs, values = replay.iteration(live, accept, then["running"] != 0, hits[n])
-                targets, cotangents = [], []
-                for k, out in zip(names, outs):
-                    if adj[k] is not None and out.requires_grad:
-                        targets.append(out)
-                        cotangents.append(adj[k])
-                if values is not None:
-                    rows, points = hits[n]
-                    targets.append(values)
-                    cotangents.append(grad_ys[rows, points] if points is not None else grad_ys[rows, 0])
-                if not targets:
-                    adj = {k: None for k in names}
-                    continue
-                wrt = [live[k] for k in names] + params
-                grads = torch.autograd.grad(targets, wrt, cotangents, allow_unused=True, retain_graph=True)
-            adj = dict(zip(names, grads[: len(names)]))
-            for i, g in enumerate(grads[len(names) :]):
-                grad_params[i] = add(grad_params[i], g)
+        add = _add
+        F = y0.shape[1]
+        use_kernels = getattr(adjoint, "backward_kernels", True) and adjoint._fused_ok(problem, term)
+        global LAST_SWEEP
+        LAST_SWEEP = "kernels" if use_kernels else "torch"  # (looked at by the tests)
+        if use_kernels:
+            adj, grad_params = reverse_sweep_kernels(adjoint, replay, term, args, problem, ctx.dt0, dt0, states, hits, grad_ys, params, list(ctx.params))
+        else:
+            adj, grad_params = reverse_sweep_torch(replay, states, hits, grad_ys, params)
 
         # ---- the start of the loop: y = y0, k0 = f(t_start, y0), dt from the start step rule or dt0 ----
         with torch.enable_grad():
