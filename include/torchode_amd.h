@@ -24,12 +24,12 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 15
+#define TODE_ABI_VERSION 16
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
-/* single step methods: reference single_step_methods/dopri5.py, tsit5.py */
-enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1 };
+/* single step methods: reference single_step_methods/dopri5.py, tsit5.py, heun.py, euler.py */
+enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1, TODE_HEUN = 2, TODE_EULER = 3 /* the last two: per-step entry points only */ };
 /* step size controllers: reference step_size_controllers.py:260 (integral), :554 (PID) */
 enum { TODE_CTRL_INTEGRAL = 0, TODE_CTRL_PID = 1, TODE_CTRL_FIXED = 2 /* per-step entry points only */ };
 /* right-hand sides the persistent kernel evaluates itself */
@@ -329,6 +329,9 @@ enum {
  *   [ k[1] <- f(tnode, ystage[1]);  tode_step_begin(phase 1) ]      only when dt0 == NULL
  *   repeat:  for s = 1..6:  tode_step_stage(s);  k[s] <- f(tnode, ystage[s])
  *            tode_step_finish()
+ *   Heun and Euler keep no derivative from one step to the next (heun.py, euler.py): every iteration starts with
+ *   k[0] <- f(t, y) of the current state, then stage 1 (Heun only), then tode_step_finish; ystage[6] is scratch
+ *   for the step's result.
  *   The caller reads `flags` (a synchronisation) or `host_flags` (none) whenever it
  *   likes; after TODE_STEP_FLAG_STOPPED is set, further stage/finish calls are no-ops.  tode_step_stats converts the
  *   counters.  k[0] must point at k0 from the first stage call on (begin
@@ -338,7 +341,7 @@ typedef struct tode_step_state {
     int32_t dtype;      /* TODE_F32 | TODE_F64: y0, y, k0, ratio_prev/pprev, ys, ystage, k */
     int32_t time_dtype; /* TODE_F32 | TODE_F64: t_start, t_end, t_eval, t, dt, tnode and a user dt0
                            (problems.py:44-56: time and data may differ) */
-    int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 */
+    int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 | TODE_HEUN | TODE_EULER (the last two: F < 64) */
     int32_t n_features; /* F */
     int32_t n_eval;     /* E; 0: report y(t_end) only */
     int64_t batch;      /* B */

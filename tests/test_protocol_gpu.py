@@ -936,11 +936,21 @@ def _low_order_fixtures():
     return sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*_low_order.json")))
 
 
+class OwnHeun(to.Heun):  # a subclass is a user's step method: the loop takes the operator path
+    pass
+
+
+class OwnEuler(to.Euler):
+    pass
+
+
+@pytest.mark.parametrize("kernels", ["per-step kernels", "operator path"])
 @pytest.mark.parametrize("path", _low_order_fixtures(), ids=lambda p: p.split("/")[-1])
-def test_heun_and_euler_match_the_aten_op_oracle_fixture(path):
+def test_heun_and_euler_match_the_aten_op_oracle_fixture(path, kernels):
     """tests/golden/*_low_order.json: the reference's loop with Heun / Euler and each of its three controllers as ATen
-    CPU operations (oracle/torch_loop.py::solve_low_order), written in the authoring container.  The operator path
-    reproduces every bit of them.  The one case that leaves the choice of the first step to the controller goes through
+    CPU operations (oracle/torch_loop.py::solve_low_order), written in the authoring container.  The per-step kernels
+    (the two methods built in, two or three launches per iteration) and the operator path (one launch per operator)
+    both reproduce every bit of them.  The one case that leaves the choice of the first step to the controller goes through
     ATen's square root kernel (``x ** 0.5`` for order 2), which on the authoring host is a vector math library's and not
     always the correctly rounded root: that case is compared to 1e-10 and in its counts."""
     import hashlib
@@ -955,9 +965,14 @@ def test_heun_and_euler_match_the_aten_op_oracle_fixture(path):
         dt0 = (span / (g["first_step_parts"] + torch.arange(g["batch"], dtype=torch.float64) % 7)).to(dtype).to(DEV)
     spec = dict(g["controller"])
     controller = to.FixedStepController() if spec["kind"] == "fixed" else make_controller(spec)
-    method = {"heun": to.Heun, "euler": to.Euler}[g["method"]]()
+    own = kernels == "operator path"
+    method = {"heun": OwnHeun if own else to.Heun, "euler": OwnEuler if own else to.Euler}[g["method"]]()
     f = copy.deepcopy(w.f).to(DEV)
-    sol = to.AutoDiffAdjoint(method, controller).solve(to.InitialValueProblem(w.y0.to(DEV), t_eval=w.t_eval.to(DEV)), to.ODETerm(f), dt0=dt0)
+    solver = to.AutoDiffAdjoint(method, controller)
+    problem = to.InitialValueProblem(w.y0.to(DEV), t_eval=w.t_eval.to(DEV))
+    assert solver._stepwise_ok(problem, to.ODETerm(f)) == (not own)
+    with torch.no_grad():
+        sol = solver.solve(problem, to.ODETerm(f), dt0=dt0)
     ys = sol.ys.cpu()
     assert sol.status.tolist() == g["status"] and sol.stats["n_initialized"].tolist() == g["n_initialized"]
     if not g["bit_exact"]:

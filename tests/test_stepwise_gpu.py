@@ -306,6 +306,118 @@ def test_fixed_steps_in_the_per_step_kernels_equal_the_operator_path(case, time_
         to.AutoDiffAdjoint(fused_method(), to.FixedStepController()).solve(problem, to.ODETerm(f))
 
 
+# ---------------------------------------------------------------------------------------------
+# Heun and Euler (reference single_step_methods/heun.py, euler.py) in the per-step kernels: no
+# derivative carried between steps, the step's result formed in the finish kernel, cubic / linear
+# dense output, controller exponents of order 2 / 1, no error estimate for Euler.  A subclass of
+# the method sends the same solve through the operator path.
+# ---------------------------------------------------------------------------------------------
+
+
+class OperatorHeun(to.Heun):
+    pass
+
+
+class OperatorEuler(to.Euler):
+    pass
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", [(F32, F32), (F64, F64), (F64, F32), (F32, F64)], ids=["f32", "f64", "t64-y32", "t32-y64"])
+@pytest.mark.parametrize("controller", ["integral", "pid", "fixed"])
+@pytest.mark.parametrize("method", ["heun", "euler"])
+@pytest.mark.parametrize("case", ["vdp", "lorenz", "backwards", "outside", "no-t_eval", "dt0", "limits"])
+def test_heun_and_euler_in_the_per_step_kernels_equal_the_operator_path(case, method, controller, time_dtype, data_dtype):
+    f, y0, t_start, t_end, t_eval, dt0, _, ctrl, max_steps = mixed_case(case, time_dtype, data_dtype)
+    B = y0.shape[0]
+    if controller == "fixed" or (method == "euler" and dt0 is None and case != "vdp"):
+        # (Euler under an adaptive controller keeps whatever step it starts with: one case leaves that to the start rule)
+        span = (t_end - t_start).double()
+        dt0 = (span / (40.0 + torch.arange(B, device="cuda", dtype=torch.float64) % 7 + 0.37)).to(time_dtype)
+    if controller == "fixed":
+        make = to.FixedStepController
+    else:
+        spec = dict(kind=controller, atol=1e-3, rtol=1e-2, **{k: ctrl[k] for k in ("dt_min", "dt_max") if k in ctrl})
+        if controller == "pid":
+            spec.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+        make = lambda: make_controller(spec)
+    max_steps = 44 if case in ("outside", "limits") else 400
+    calls = {"kernels": [], "operators": []}
+
+    def rhs(which):
+        def g(t, y):
+            calls[which].append((t, y))
+            return f(t, y)
+
+        return g
+
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
+    fused_method, operator_method = {"heun": (to.Heun, OperatorHeun), "euler": (to.Euler, OperatorEuler)}[method]
+    with torch.no_grad():
+        fused_solver = to.AutoDiffAdjoint(fused_method(), make(), max_steps=max_steps)
+        assert fused_solver._stepwise_ok(problem, to.ODETerm(f))
+        fused = fused_solver.solve(problem, to.ODETerm(rhs("kernels")), dt0=dt0)
+        ops_solver = to.AutoDiffAdjoint(operator_method(), make(), max_steps=max_steps)
+        assert not ops_solver._stepwise_ok(problem, to.ODETerm(f))
+        ops = ops_solver.solve(problem, to.ODETerm(rhs("operators")), dt0=dt0)
+    assert fused.ys.dtype == data_dtype and fused.ts.dtype == time_dtype and fused.ys.shape == ops.ys.shape
+    for key in ("n_steps", "n_accepted", "n_initialized", "n_f_evals"):
+        assert torch.equal(fused.stats[key], ops.stats[key]), key
+    assert torch.equal(fused.status, ops.status)
+    # f is called as often as the counter says (the kernels' loop runs ahead of the device by a few iterations whose
+    # kernels do nothing), with tensors of its own that hold what the operator path's calls held
+    n = int(ops.stats["n_f_evals"][0])
+    assert len(calls["operators"]) == n and len(calls["kernels"]) >= n
+    stages = 2 if method == "heun" else 1
+    for i in sorted({0, 1, 2, stages * 3, n - stages - 1, n - 1} & set(range(n))):
+        (ta, ya), (tb, yb) = calls["kernels"][i], calls["operators"][i]
+        assert ta.dtype == time_dtype and ya.dtype == data_dtype
+        running_rows = torch.isfinite(yb).all(dim=1)
+        if i < n - stages:  # (in the last iteration the finished samples differ: stale in one path, frozen in the other)
+            assert torch.equal(ta, tb) and torch.equal(ya[running_rows], yb[running_rows]), i
+    assert len({x.data_ptr() for pair in calls["kernels"] for x in pair}) == 2 * len(calls["kernels"])
+    E = fused.ys.shape[1]
+    written = torch.arange(E, device="cuda")[None, :] < ops.stats["n_initialized"][:, None]
+    if case == "outside":  # every fifth row is not monotone: what is written there is no prefix of the row (the counts are compared above)
+        written = written & (torch.arange(B, device="cuda") % 5 != 0)[:, None]
+    a, b = fused.ys[written], ops.ys[written]
+    assert bool(((a == b) | (a.isnan() & b.isnan())).all()), (a - b).abs().nan_to_num().max().item()
+    if case == "limits" and method == "heun" and controller != "fixed":
+        assert (fused.status == 2).any()  # the smallest step allowed is too long for these tolerances
+    else:
+        assert int(fused.stats["n_steps"].max()) >= 3
+    if method == "euler" or controller == "fixed":
+        assert torch.equal(fused.stats["n_steps"], fused.stats["n_accepted"])
+    elif case in ("vdp", "lorenz"):
+        assert (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()  # rejected steps are part of the case
+
+
+def test_long_rows_with_heun_and_euler_stay_on_the_operator_path():
+    f, y0, t_start, t_end, t_eval, _, _, ctrl, _ = mixed_case("wide", F32, F32)
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
+    for method in (to.Heun(), to.Euler()):
+        solver = to.AutoDiffAdjoint(method, to.IntegralController(1e-3, 1e-2))
+        assert not solver._stepwise_ok(problem, to.ODETerm(f))
+        with torch.no_grad():
+            sol = solver.solve(problem, to.ODETerm(f), dt0=torch.full((y0.shape[0],), 1e-2, device="cuda"))
+        assert (sol.status == 0).all()
+
+
+@pytest.mark.parametrize("method", ["heun", "euler"])
+def test_graph_replay_with_heun_and_euler(method):
+    w = to.workloads.make("vdp", batch=300, dtype=F32)
+    f = copy.deepcopy(w.f).to("cuda")
+    problem = to.InitialValueProblem(w.y0.to("cuda"), t_eval=w.t_eval.to("cuda"))
+    dt0 = torch.full((300,), 5e-3, device="cuda")
+    m = {"heun": to.Heun, "euler": to.Euler}[method]
+    with torch.no_grad():
+        eager = to.AutoDiffAdjoint(m(), to.IntegralController(1e-3, 1e-2)).solve(problem, to.ODETerm(f), dt0=dt0)
+        replayed = to.AutoDiffAdjoint(m(), to.IntegralController(1e-3, 1e-2), graph_iterations=5).solve(problem, to.ODETerm(f), dt0=dt0)
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert torch.equal(eager.stats[key], replayed.stats[key]), key
+    assert torch.equal(eager.ys, replayed.ys) and torch.equal(eager.status, replayed.status)
+    assert int(eager.stats["n_steps"].max()) > 40
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_random_configurations_match_oracle_bit_for_bit(seed):
     """The seeded random configurations of the whole-solve suite (term, shapes, time spans, evaluation points,

@@ -13,12 +13,12 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
 F32, F64 = 0, 1
-DOPRI5, TSIT5 = 0, 1
+DOPRI5, TSIT5, HEUN, EULER = 0, 1, 2, 3
 CTRL_INTEGRAL, CTRL_PID, CTRL_FIXED = 0, 1, 2
 TERM_REACTION_DIFFUSION, TERM_MLP = 3, 4
 PERSISTENT_TERMS = (0, 1, 2, 3, 4)  # TODE_TERM_* that a whole-solve kernel evaluates itself

@@ -64,7 +64,7 @@ class AutoDiffAdjoint(nn.Module):
 
     Same constructor and ``solve`` signature as the reference.  The solve runs in HIP kernels.
     When ``y0``, a parameter of the term, a tensor in ``args`` or one of the times requires grad it
-    takes the per-step kernels (Heun, Euler: the operator path) and records the loop state per iteration, and the result is
+    takes the per-step kernels (Heun, Euler with gradients: the operator path) and records the loop state per iteration, and the result is
     differentiable (``torchode_amd/autodiff.py``; ``backprop_through_step_size_control`` as in the
     reference).
     """
@@ -177,7 +177,10 @@ class AutoDiffAdjoint(nn.Module):
         )
 
     def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        return self._fused_ok(problem, term)
+        if self._fused_ok(problem, term):
+            return True
+        # Heun and Euler are built into the thread-per-sample kernels (rows of fewer than 64 features)
+        return problem.n_features < 64 and self._library_setup(problem, term, (Heun, Euler))
 
     # ------------------------------------------------------------------ #
     def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args, record=None) -> Solution:
@@ -367,8 +370,15 @@ class AutoDiffAdjoint(nn.Module):
             keep["k", i] = rhs(tt, yy)
             s.k[i] = keep["k", i].data_ptr()
 
-        evaluate(0, t_start, y0)
-        n_init_evals = 1
+        # Dopri5 and Tsit5 carry the last stage's derivative into the next step, so f(t_start, y0) is needed before
+        # the loop whatever sets the first step; Heun and Euler evaluate their first stage anew in every step
+        # (runge_kutta.py:196-212) and see f before the loop only through the controller's start step rule.
+        n_stages = {_lib.DOPRI5: 7, _lib.TSIT5: 7, _lib.HEUN: 2, _lib.EULER: 1}[s.method]
+        carries = n_stages == 7
+        n_init_evals = 0
+        if carries or dt0_ is None:
+            evaluate(0, t_start, y0)
+            n_init_evals = 1
         if dt0_ is None:
             tt, yy = stage_buffers(1)
             _lib.check(lib.tode_step_begin(sref, cref, None, 0, stream), "tode_step_begin")
@@ -378,13 +388,19 @@ class AutoDiffAdjoint(nn.Module):
         else:
             s.tnode = t.data_ptr()  # unused by this phase, but must be a valid pointer
             _lib.check(lib.tode_step_begin(sref, cref, _lib.ptr(dt0_), 0, stream), "tode_step_begin")
-        s.k[0] = k0.data_ptr()  # from here on the FSAL slot is the state's own buffer
+        if carries:
+            s.k[0] = k0.data_ptr()  # from here on the first slot is the state's own buffer
+        else:
+            keep["y1"] = new(B, F)
+            s.ystage[6] = keep["y1"].data_ptr()  # the finish kernel forms the step's result there
 
         def iterate(n, stream):
             for _ in range(n):
                 if record is not None:
                     record.snapshot(t, dt, y, k0, hist, ints)
-                for i in range(1, 7):
+                if not carries:
+                    evaluate(0, t.clone(), y.clone())
+                for i in range(1, n_stages):
                     tt, yy = stage_buffers(i)
                     _lib.check(lib.tode_step_stage(sref, cref, i, stream), "tode_step_stage")
                     evaluate(i, tt, yy)
@@ -421,6 +437,7 @@ class AutoDiffAdjoint(nn.Module):
                 graph = self._record(lambda st: iterate(int(self.graph_iterations), st), y0)
             elif graph is not None:
                 replays = min(2 * replays, max(1, self.poll_max // int(self.graph_iterations)))
+        y1_buffer = keep.pop("y1", None)  # (kernels enqueued after the stop do nothing, but hold the pointer)
         keep.clear()
         del graph  # frees the memory f's intermediate tensors were recorded with
         if record is not None:
@@ -431,7 +448,7 @@ class AutoDiffAdjoint(nn.Module):
         _lib.check(lib.tode_step_stats(sref, *(_lib.ptr(out[i]) for i in range(4)), stream), "tode_step_stats")
         stats: Dict[str, Any] = {}
         if term.with_stats:
-            n = n_init_evals + 6 * fl[_lib.STEP_FLAG_ITERATIONS]
+            n = n_init_evals + (n_stages - 1 if carries else n_stages) * fl[_lib.STEP_FLAG_ITERATIONS]
             stats["n_f_evals"] = _f_evals(n, B)
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
         ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]

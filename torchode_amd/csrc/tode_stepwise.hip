@@ -42,6 +42,8 @@ template <typename TT, typename T> struct StepParams {
     CtrlParams<T> cp;
     TT dt_min, dt_max;  // limits of the step (step_size_controllers.py:406-422), in the time type
     const TT *fixed_dt;  // [B] CTRL == 2: the fixed step (step_size_controllers.py:116-167)
+    double inv_order;    // 1 / convergence order of the step method, the exponent of the start step rule
+    bool carry;          // the method keeps the last stage's derivative as the next step's first (Dopri5, Tsit5)
 };
 
 // dt_min / dt_max and the status of a step proposal, limits in the time type
@@ -61,13 +63,26 @@ __device__ __forceinline__ int limit_step(const CtrlParams<T> &cp, TT dt_min, TT
     return status;
 }
 
-template <typename T> __device__ __forceinline__ T tab_a(int method, int i, int j) {
-    return method == 1 ? (T)Tsit5Tab::a[i][j] : (T)Dopri5Tab::a[i][j];
-}
+// Heun 2(1) (heun.py:10-13): c = (0, 1), a_10 = 1, b = (1/2, 1/2), low-order weights (1, 0), b_err = b - b_low in
+// float64 (runge_kutta.py:84-88).  Neither first-same-as-last nor solution-same-as-last-stage: the first stage is
+// evaluated anew in every step and y1 = y0 + sum_s (dt b_s) k_s.  Euler (euler.py:29-56) has one stage and no tableau.
+struct HeunTab {
+    static constexpr double c[7] = {0.0, 1.0};
+    static constexpr double a[7][7] = {{0}, {1.0}};
+    static constexpr double b[2] = {0.5, 0.5};
+    static constexpr double b_err[2] = {0.5 - 1.0, 0.5 - 0.0};
+};
+template <int METHOD> struct TabOf { using type = Dopri5Tab; };
+template <> struct TabOf<1> { using type = Tsit5Tab; };
+template <> struct TabOf<2> { using type = HeunTab; };
+// stages per step, and the convergence order the controllers divide by (dopri5.py:49-51, tsit5.py:119-121, heun.py,
+// euler.py)
+__host__ __device__ constexpr int stages_of(int method) { return method <= TODE_TSIT5 ? 7 : (method == TODE_HEUN ? 2 : 1); }
+__host__ __device__ constexpr double order_of(int method) { return method <= TODE_TSIT5 ? 5.0 : (method == TODE_HEUN ? 2.0 : 1.0); }
 
 // ystage[s] = fma(dt, sum_j a_sj k_j, y); tnode = fma(c_s, dt, t)   (runge_kutta.py:259-262)
 template <typename TT, typename T, int METHOD, int S> __global__ void __launch_bounds__(256) stage_kernel(const StepParams<TT, T> p) {
-    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    using Tab = typename TabOf<METHOD>::type;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long n = p.batch * p.F;
@@ -156,7 +171,7 @@ __global__ void __launch_bounds__(256) init_b_kernel(const StepParams<TT, T> p, 
             h1 = tmax((T)1e-6, h0 * (T)1e-3);
         } else {
             T rm = (T)1 / m;
-            h1 = rpow<T>(rm * (T)0.01, 1.0 / 5.0);
+            h1 = rpow<T>(rm * (T)0.01, p.inv_order);
         }
         dt = (TT)(dir * tmin((T)100 * h0, h1));
     } else {
@@ -167,7 +182,7 @@ __global__ void __launch_bounds__(256) init_b_kernel(const StepParams<TT, T> p, 
     p.dt[b] = tclamp(dt, tlo - ts, thi - ts);
     for (int f = 0; f < F; ++f) {
         p.y[b * F + f] = y0[f];
-        p.k0[b * F + f] = f0[f];
+        if (p.carry) p.k0[b * F + f] = f0[f];
     }
     p.ratio_prev[b] = (T)1;
     p.ratio_pprev[b] = (T)1;
@@ -207,8 +222,23 @@ template <typename T> __device__ __forceinline__ T quartic_at(const T (&q)[5][1]
 
 template <typename TT, typename T, int METHOD>
 __device__ __forceinline__ T dense_value(TT t0, TT dt, T y0, T y1, const T (&ks)[7], bool fused, TT te) {
+    if (METHOD == TODE_EULER) {
+        // linear (interpolation.py:48-62): the step itself divides, not (t0 + dt) - t0
+        return fma_(y1 - y0, (T)unit_time_over<TT>(te, t0, dt), y0);
+    }
+    if (METHOD == TODE_HEUN) {
+        // Hermite cubic from the first and the last slope (interpolation.py:84-106), ks[1] = f at the step's end
+        const T h = (T)dt, f0 = ks[0], f1 = ks[1], d01 = y0 - y1;
+        const T a = fma_((T)2, d01, h * (f0 + f1));
+        const T b = fma_((T)-3, d01, h * fma_((T)-2, f0, -f1));
+        const T x = (T)unit_time<TT>(te, t0, t0 + dt);
+        T v = a;
+        v = fma_(v, x, b);
+        v = fma_(v, x, h * f0);
+        return fma_(v, x, y0);
+    }
     T q[5][1];
-    quartic_elem<T, METHOD>((T)dt, y0, y1, ks, fused, q);
+    quartic_elem<T, (METHOD == 1 ? 1 : 0)>((T)dt, y0, y1, ks, fused, q);
     return quartic_at<T>(q, (T)unit_time<TT>(te, t0, t0 + dt));
 }
 
@@ -218,7 +248,9 @@ __device__ __forceinline__ T dense_value(TT t0, TT dt, T y0, T y1, const T (&ks)
 // flag, dt clamp (runge_kutta.py:265-272, step_size_controllers.py:370-429 / 715-774,
 // adjoints.py:150-255).
 template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<TT, T> p) {
-    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    using Tab = typename TabOf<METHOD>::type;
+    constexpr int NS = stages_of(METHOD);
+    constexpr bool ESTIMATE = METHOD != TODE_EULER;  // Euler has no error estimate: every step is accepted, the step kept
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= p.batch) return;
@@ -230,14 +262,35 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     const T h = (T)dt;
     const TT ts = p.t_start[b], te = p.t_end[b];
     const bool fwd = te > ts;
-    const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
+    const T *y = p.y + b * F;
+    T *y1 = p.ystage[6] + b * F;
+
+    // ---- the step's result where it is not the input of the last stage (heun.py, euler.py; runge_kutta.py:265-269) ----
+    if (METHOD == TODE_HEUN) {
+        for (int f = 0; f < F; ++f) {
+            T sum = 0;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const T ps = h * (T)HeunTab::b[s], ks = p.k[s][b * F + f];
+                if (fused)
+                    sum = fma_(ps, ks, sum);
+                else {
+                    const T pk = ps * ks;
+                    sum = sum + pk;
+                }
+            }
+            y1[f] = y[f] + sum;
+        }
+    } else if (METHOD == TODE_EULER) {
+        for (int f = 0; f < F; ++f) y1[f] = fma_(h, p.k[0][b * F + f], y[f]);
+    }
 
     // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
     T acc = 0;
-    for (int f = 0; CTRL != 2 && f < F; ++f) {
+    for (int f = 0; ESTIMATE && CTRL != 2 && f < F; ++f) {
         T err = 0;
 #pragma unroll
-        for (int s = 0; s < 7; ++s) {
+        for (int s = 0; s < NS; ++s) {
             T ps = h * (T)Tab::b_err[s];
             T ks = p.k[s][b * F + f];
             if (fused)
@@ -258,7 +311,7 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         }
     }
     const T ratio = tmax(sqrt_(acc), (T)1e-38);
-    const bool accept = CTRL == 2 || ratio < (T)1;
+    const bool accept = CTRL == 2 || !ESTIMATE || ratio < (T)1;
 
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
@@ -266,6 +319,8 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     int status = 0;
     if (CTRL == 2) {
         dt_next = p.fixed_dt[b];
+    } else if (!ESTIMATE) {
+        dt_next = dt;  // (step_size_controllers.py:382-391, 727-736: accepted, step size unchanged, no status)
     } else {
         dt_next = dt * (TT)dt_factor<T, (CTRL == 2 ? 0 : CTRL)>(cp, ratio, prev, pprev);
         status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
@@ -299,9 +354,9 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
                 continue;
             }
             for (int f = 0; f < F; ++f) {
-                T ks[7];
+                T ks[7] = {};
 #pragma unroll
-                for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+                for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
                 ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
             }
             pend[e] = 0;
@@ -312,9 +367,9 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         // no evaluation points: the end-point value of the loop's last interpolant
         // (adjoints.py:295-309); rewritten every iteration, the last one stays
         for (int f = 0; f < F; ++f) {
-            T ks[7];
+            T ks[7] = {};
 #pragma unroll
-            for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
+            for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
             p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
         }
     }
@@ -323,14 +378,14 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     if (move) {
         for (int f = 0; f < F; ++f) {
             p.y[b * F + f] = y1[f];
-            p.k0[b * F + f] = p.k[6][b * F + f];
+            if (NS == 7) p.k0[b * F + f] = p.k[6][b * F + f];  // (first same as last: Dopri5 and Tsit5 only)
         }
     }
     p.t[b] = t_new;
     const TT tlo = tmin(ts, te), thi = tmax(te, ts);
     const TT dtn = running_new ? dt_next : dt;
     p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
-    if (CTRL == 1 && running_new && accept) {
+    if (CTRL == 1 && ESTIMATE && running_new && accept) {
         p.ratio_pprev[b] = prev;
         p.ratio_prev[b] = ratio;
     }
@@ -383,7 +438,7 @@ __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T
             const T df = f1[f] - f0[f];
             return df * inv_scale(cp.atol, cp.rtol, y0[f]);
         });
-        dt = (TT)initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, p.ratio_prev[b], d1, d2n);
+        dt = (TT)initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, p.inv_order, dir, p.ratio_prev[b], d1, d2n);
     } else {
         dt = dt0[b];
     }
@@ -421,7 +476,7 @@ __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T
 }
 
 template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<TT, T> p) {
-    using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
+    using Tab = typename TabOf<METHOD>::type;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= p.batch) return;
@@ -611,10 +666,12 @@ template <typename TT, typename T> static StepParams<TT, T> make_step_params(con
         p.k[i] = (const T *)s.k[i];
     }
     p.tnode = (TT *)s.tnode;
-    p.cp = make_ctrl<T>(c);
+    p.cp = make_ctrl<T>(c, order_of(s.method));
     p.dt_min = (TT)c.dt_min;
     p.dt_max = (TT)c.dt_max;
     p.fixed_dt = (const TT *)s.fixed_dt;
+    p.inv_order = 1.0 / order_of(s.method);
+    p.carry = s.method <= TODE_TSIT5;
     return p;
 }
 
@@ -623,7 +680,9 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     if (s->batch < 0 || s->n_features <= 0 || s->n_eval < 0) return fail(TODE_E_INVALID, "bad sizes");
     if (s->dtype != TODE_F32 && s->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", s->dtype);
     if (s->time_dtype != TODE_F32 && s->time_dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown time dtype %d", s->time_dtype);
-    if (s->method != TODE_DOPRI5 && s->method != TODE_TSIT5) return fail(TODE_E_INVALID, "unknown method %d", s->method);
+    if (s->method < TODE_DOPRI5 || s->method > TODE_EULER) return fail(TODE_E_INVALID, "unknown method %d", s->method);
+    if (s->method > TODE_TSIT5 && s->n_features >= 64)
+        return fail(TODE_E_UNSUPPORTED, "Heun and Euler are built into the per-step kernels for rows of fewer than 64 features (got %d)", s->n_features);
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID && c->kind != TODE_CTRL_FIXED)
         return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (c->kind == TODE_CTRL_FIXED && s->batch > 0 && !s->fixed_dt) return fail(TODE_E_INVALID, "the fixed-step controller needs fixed_dt");
@@ -672,7 +731,7 @@ int tode_step_begin(const tode_step_state *s, const tode_controller *c, const vo
         hipLaunchKernelGGL(step_flags_init_kernel, dim3(1), dim3(64), 0, st, s->flags, s->host_flags);
         if (blocks == 0) return check_hip(hipGetLastError(), "tode_step_begin");
         if (dt0) {
-            if (!s->k[0]) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
+            if (!s->k[0] && s->method <= TODE_TSIT5) return fail(TODE_E_INVALID, "k[0] (f at t_start) is null");
             TODE_DISPATCH_T(s, {
                 auto p = make_step_params<TT, T>(*s, *c);
                 if (wide)
@@ -716,7 +775,8 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
     using namespace tode;
     int rc = check_state(s, c);
     if (rc) return rc;
-    if (stage < 1 || stage > 6) return fail(TODE_E_INVALID, "stage must be 1..6, got %d", stage);
+    const int last_stage = stages_of(s->method) - 1;
+    if (stage < 1 || stage > last_stage) return fail(TODE_E_INVALID, "stage must be 1..%d for this method, got %d", last_stage, stage);
     for (int j = 0; j < stage; ++j)
         if (s->batch > 0 && !s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
     if (s->batch > 0 && !s->ystage[stage]) return fail(TODE_E_INVALID, "ystage[%d] is null", stage);
@@ -733,7 +793,9 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
     }
     TODE_DISPATCH_T(s, {
         auto p = make_step_params<TT, T>(*s, *c);
-        if (s->method == TODE_TSIT5) {
+        if (s->method == TODE_HEUN) {
+            hipLaunchKernelGGL((stage_kernel<TT, T, 2, 1>), dim3(blocks), dim3(256), 0, st, p);
+        } else if (s->method == TODE_TSIT5) {
             TODE_STAGE_SWITCH(1)
         } else {
             TODE_STAGE_SWITCH(0)
@@ -760,13 +822,17 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
     const bool wide = s->n_features >= 64;
     const unsigned blocks = wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
     if (blocks > 0) {
-        for (int j = 0; j < 7; ++j)
+        for (int j = 0; j < stages_of(s->method); ++j)
             if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
         if (!s->ystage[6]) return fail(TODE_E_INVALID, "ystage[6] is null");
         TODE_DISPATCH_T(s, {
             auto p = make_step_params<TT, T>(*s, *c);
             const bool tsit5 = s->method == TODE_TSIT5;
-            if (wide) {
+            if (s->method == TODE_HEUN) {
+                TODE_FINISH_CTRL(finish_kernel, 2);
+            } else if (s->method == TODE_EULER) {
+                TODE_FINISH_CTRL(finish_kernel, 3);
+            } else if (wide) {
                 if (tsit5) TODE_FINISH_CTRL(finish_wave_kernel, 1);
                 else TODE_FINISH_CTRL(finish_wave_kernel, 0);
             } else {

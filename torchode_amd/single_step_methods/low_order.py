@@ -1,5 +1,6 @@
 """The two low-order methods of the reference: forward Euler (torchode/single_step_methods/euler.py)
-and Heun's method 2(1) (torchode/single_step_methods/heun.py).  Both run through the operator path."""
+and Heun's method 2(1) (torchode/single_step_methods/heun.py).  The classes here are the operator
+path; the per-step kernels know the two methods by ``method_id`` (rows of fewer than 64 features)."""
 from typing import Any, Dict, NamedTuple, Optional
 
 import torch
@@ -21,6 +22,8 @@ class LinearInterpolationData(NamedTuple):
 class Euler(SingleStepMethod):
     """``y1 = y0 + dt f(t0, y0)``, no error estimate (a controller then keeps the step size), linear
     dense output."""
+
+    method_id = _lib.EULER
 
     def __init__(self, term: Optional[ODETerm] = None):
         super().__init__()
@@ -65,6 +68,7 @@ class Heun(ExplicitRungeKutta):
     """Two stages, error estimate against the Euler step, Hermite cubic dense output (stage and sum
     kernels with this tableau)."""
 
+    method_id = _lib.HEUN
     TABLEAU = ButcherTableau.from_lists(c=_HEUN_NODES, a=_HEUN_STAGES, b=_HEUN_WEIGHTS, b_low_order=_HEUN_EULER_WEIGHTS)
 
     def __init__(self, term: Optional[ODETerm] = None):
