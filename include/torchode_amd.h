@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 16
+#define TODE_ABI_VERSION 17
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -270,6 +270,38 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_control
 int tode_solve_builtin_fast_static(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
                                    int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status,
                                    int32_t *flags_out, void *stream);
+
+/*
+ * The whole of AutoDiffAdjoint.solve (reference adjoints.py:42-311) for a
+ * built-in term in one call: the one-kernel path where the problem is in its
+ * shape (tode_solve_builtin_fast_sync), else or after it reported
+ * TODE_FLAG_NEEDS_GENERAL the general kernel (tode_solve_builtin, launched
+ * again with a pending mask for rows of evaluation points that are not
+ * monotone, and again with an iteration cap when some sample reported a
+ * non-success status, adjoints.py:229-238), then tode_finalize_stats.  On
+ * return ys and the four int64 [B] outputs hold what the reference returns and
+ * *iterations (HOST memory) the number of loop iterations L, from which the
+ * caller forms stats["n_f_evals"] = (dt0 given ? 1 : 2) + 6 L (terms.py:41-63).
+ *
+ * The call synchronises with the stream (once in the common case), as the
+ * reference's loop does in every iteration.  It allocates nothing: flag words,
+ * int32 counters, the pending mask and the idle end points live in `workspace`,
+ * DEVICE memory of at least tode_solve_workspace_bytes(args) bytes that the
+ * caller provides and may reuse for the next call on the same stream.
+ * args->flags, pending, y_idle, the five int32 outputs and iteration_cap are
+ * not read.  allow_one_kernel = 0 sends the three small systems to the
+ * general kernel directly (same results).
+ *
+ * Returns TODE_E_UNSUPPORTED, with nothing written that the caller may rely
+ * on, where no whole-solve kernel covers the problem (reaction-diffusion and
+ * MLP outside the shapes named at TODE_TERM_*, or a batch of theirs with a
+ * non-success status, non-monotone rows or step size limits): the caller runs
+ * the loop through the per-step or the operator entry points instead.
+ */
+int64_t tode_solve_workspace_bytes(const tode_solve_args *args);
+int tode_solve_builtin_auto(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
+                            int64_t *out_n_accepted, int64_t *out_n_initialized, int64_t *out_status, void *workspace,
+                            int64_t workspace_bytes, int32_t allow_one_kernel, void *stream, int64_t *iterations);
 
 /*
  * Last step of a solve without evaluation points through tode_solve_builtin_fast

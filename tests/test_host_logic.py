@@ -91,6 +91,56 @@ def test_library_exports_every_declared_symbol():
     assert lib.tode_last_error() is not None
 
 
+def test_torch_operators_are_registered_for_the_gpu_only_with_tracing_rules():
+    """libtorchode_amd_ops.so registers torch.ops.torchode_amd.solve_builtin / mlp_pack_weights: no CPU implementation
+    (a call with CPU tensors fails in the dispatcher), and the shapes, dtypes and devices of the results for a tracer."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from torchode_amd import ops
+
+    ops.load()
+    op = torch.ops.torchode_amd.solve_builtin
+    assert "CUDA" in torch._C._dispatch_dump("torchode_amd::solve_builtin") and "CPU:" not in torch._C._dispatch_dump("torchode_amd::solve_builtin")
+    control = [1e-6, 1e-5, 0.0, 1.0, 0.0, 0.9, 0.2, 10.0, float("nan"), float("nan")]
+    with FakeTensorMode():
+        y0, t_eval = torch.empty(8, 3, device="cuda", dtype=torch.float64), torch.empty(8, 5, device="cuda", dtype=torch.float64)
+        out = op(y0, t_eval[:, 0], t_eval[:, -1], t_eval, None, torch.empty(8, 1, device="cuda"), None, 1, 2, [10.0, 8 / 3], 0, control, -1, True)
+        assert [tuple(o.shape) for o in out] == [(8, 5, 3), (8,), (8,), (8,), (8,), ()]
+        assert [o.dtype for o in out] == [torch.float64] + [torch.long] * 5
+        assert [o.device.type for o in out] == ["cuda"] * 5 + ["cpu"]
+        end_only = op(y0, t_eval[:, 0], t_eval[:, -1], None, None, None, None, 1, 2, [10.0, 8 / 3], 0, control, -1, True)
+        assert tuple(end_only[0].shape) == (8, 1, 3)
+        packed = torch.ops.torchode_amd.mlp_pack_weights(torch.empty(256 * 65 + 256 + 64 * 256 + 64, device="cuda"), 1)
+        assert tuple(packed.shape) == (_lib.MLP_PACKED_SIZE["bfloat16"],)
+    y0, t_eval = torch.zeros(8, 3), torch.zeros(8, 5)
+    with pytest.raises(NotImplementedError, match="CPU"):
+        op(y0, t_eval[:, 0], t_eval[:, -1], t_eval, None, torch.zeros(8, 1), None, 1, 2, [10.0, 8 / 3], 0, control, -1, True)
+
+
+def test_solve_workspace_size_and_argument_checks_of_the_one_call_entry_point():
+    lib = _lib.load()
+    a, c = _lib.SolveArgs(), _lib.Controller()
+    assert lib.tode_solve_workspace_bytes(None) == -1
+    a.dtype, a.batch, a.n_features, a.n_eval = _lib.DTYPES[torch.float64], 1000, 3, 0
+    up = lambda n: (n + 255) // 256 * 256
+    assert lib.tode_solve_workspace_bytes(_lib.C.byref(a)) == up(16) + up(5 * 1000 * 4) + up(1000 * 3 * 8)
+    a.n_eval = 7
+    need = lib.tode_solve_workspace_bytes(_lib.C.byref(a))
+    assert need == up(16) + up(5 * 1000 * 4) + up(1000 * 7)
+    it = _lib.C.c_int64(0)
+    dummy = (_lib.C.c_double * 64)()
+    p = _lib.C.addressof(dummy)
+    assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, p, need - 1, 1, None, _lib.C.byref(it)) == _lib.E_INVALID
+    assert b"workspace" in lib.tode_last_error()
+    assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, None, need, 1, None, _lib.C.byref(it)) == _lib.E_INVALID
+    assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, p, need, 1, None, None) == _lib.E_INVALID
+    a.term = 9
+    assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, p, need, 1, None, _lib.C.byref(it)) == _lib.E_INVALID
+    assert b"unknown term" in lib.tode_last_error()
+    a.term, a.dtype = _lib.TERM_MLP, _lib.DTYPES[torch.float64]  # the matrix-core kernel is float32: refused before anything is launched
+    assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, p, need, 1, None, _lib.C.byref(it)) == _lib.E_UNSUPPORTED
+
+
 def test_abi_argument_validation_without_a_gpu():
     """Null / inconsistent arguments are rejected before anything touches a device."""
     lib = _lib.load()

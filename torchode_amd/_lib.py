@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -39,6 +39,8 @@ EXPORTS = (
     "tode_solve_builtin_fast",
     "tode_solve_builtin_fast_sync",
     "tode_solve_builtin_fast_static",
+    "tode_solve_builtin_auto",
+    "tode_solve_workspace_bytes",
     "tode_mlp_pack_weights",
     "tode_select_end_point",
     "tode_step_begin",
@@ -312,6 +314,10 @@ def load():
         lib.tode_solve_builtin_fast_static.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 6
         lib.tode_solve_builtin_fast_sync.restype = C.c_int
         lib.tode_solve_builtin_fast_sync.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.POINTER(C.c_int32)]
+        lib.tode_solve_workspace_bytes.restype = C.c_int64
+        lib.tode_solve_workspace_bytes.argtypes = [C.POINTER(SolveArgs)]
+        lib.tode_solve_builtin_auto.restype = C.c_int
+        lib.tode_solve_builtin_auto.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.c_int64, C.c_int32, C.c_void_p, C.POINTER(C.c_int64)]
         lib.tode_step_begin.restype = C.c_int
         lib.tode_step_begin.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p, C.c_int, C.c_void_p]
         lib.tode_step_stage.restype = C.c_int

@@ -40,7 +40,26 @@ _PROTOCOL_NAME_SET = frozenset(_PROTOCOL_NAMES)
 def _library_object(obj, classes) -> bool:
     """True if ``obj`` is exactly one of the library's classes with no protocol method replaced on
     the instance; only then may a fused kernel stand in for the calls the loop would make."""
-    return type(obj) in classes and _PROTOCOL_NAME_SET.isdisjoint(vars(obj))
+    if type(obj) not in classes:
+        return False
+    if torch.compiler.is_compiling():  # (spelled so that a tracing compiler can follow it)
+        return all(name not in obj.__dict__ for name in _PROTOCOL_NAMES)
+    return _PROTOCOL_NAME_SET.isdisjoint(vars(obj))
+
+
+def _library_plugins(adjoint, term, methods) -> bool:
+    """The part of ``AutoDiffAdjoint._library_setup`` that looks at the plug-in objects only."""
+    m, c = adjoint.step_method, adjoint.step_size_controller
+    return (
+        _library_object(m, methods)
+        and _library_object(c, (IntegralController, PIDController, FixedStepController))
+        and c.fusable
+        and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
+        and type(term).vf is ODETerm.vf
+        and type(term).init is ODETerm.init
+        and "vf" not in term.__dict__
+        and "init" not in term.__dict__
+    )
 
 
 class Adjoint:
@@ -94,6 +113,11 @@ class AutoDiffAdjoint(nn.Module):
         # Set to False to route built-in terms through the general whole-solve kernel only
         # (same results; used by the tests to compare the two kernels).
         self.use_fast_path = True
+        # torch.ops.torchode_amd.*: registered here, where no tracer is looking, so that torch.compile of `solve`
+        # finds the operators and their tracing rules in place
+        from . import ops
+
+        ops.load()
 
     # ------------------------------------------------------------------ #
     def solve(
@@ -103,6 +127,62 @@ class AutoDiffAdjoint(nn.Module):
         dt0: Optional[torch.Tensor] = None,
         args: Any = None,
     ) -> Solution:
+        if torch.compiler.is_compiling():
+            # Under a tracing compiler (torch.compile of this method): a whole solve with a built-in term is one
+            # operator of PyTorch's dispatcher; every other solve leaves the captured program and runs as it does eagerly.
+            return self._solve_traced(problem, term, dt0, args)
+        return self._solve_eager(problem, term, dt0, args)
+
+    def _solve_traced(self, problem: InitialValueProblem, term: Optional[ODETerm], dt0, args) -> Solution:
+        from . import ops
+
+        term_ = term if term is not None else getattr(self.step_method, "term", None)
+        f = getattr(term_, "f", None)
+        tensors = [problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0]
+        if (
+            term_ is None
+            or not isinstance(f, BuiltinTerm)
+            or not self._persistent_ok(problem, term_)
+            or not problem.y0.is_cuda
+            or (torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in [*tensors, *f.buffers(), *f.parameters()]))
+            or not self._whole_solve_shape(problem, f)
+        ):
+            return self._solve_eager_outside_the_trace(problem, term, dt0, args)
+        kind, control = self.step_size_controller.control_values()
+        dtype, B, E = problem.data_dtype, problem.batch_size, problem.n_evaluation_points
+        mlp = f.builtin_kind == _lib.TERM_MLP
+        params = None if mlp else f.builtin_params().to(dtype)
+        shared = ops.mlp_pack_weights(f.builtin_shared().to(dtype), _lib.MLP_INPUTS[f.matrix_inputs]) if mlp else None
+        scalars = [float(x) for x in getattr(f, "builtin_scalars", lambda: ())()]
+        ys, n_steps, n_accepted, n_initialized, status, iterations = ops.solve_builtin(
+            problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0, params, shared, self.step_method.method_id, f.builtin_kind,
+            scalars, kind, control, self.max_steps, self.use_fast_path,
+        )  # fmt: skip
+        stats: Dict[str, Any] = {}
+        if term_.with_stats:
+            stats["n_f_evals"] = ((2 if dt0 is None else 1) + 6 * iterations).expand(B)
+        stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = n_steps, n_accepted, n_initialized
+        ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
+        return Solution(ts=ts, ys=ys, stats=stats, status=status)
+
+    def _whole_solve_shape(self, problem: InitialValueProblem, f: BuiltinTerm) -> bool:
+        """What can be told from shapes and settings alone about whether a whole-solve kernel takes the problem (the
+        library decides for good, tode_solve_builtin_auto; the eager path asks it and goes on to the per-step kernels on
+        a refusal, a captured program cannot)."""
+        if f.builtin_kind in _lib.GENERAL_TERMS:
+            return True
+        c, E, F = self.step_size_controller, problem.n_evaluation_points, problem.n_features
+        if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != torch.float32:
+            return False
+        if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
+            return F in (32 * 32, 64 * 64) and E <= 8192
+        return F == 64 and tuple(f.W1.shape) == (256, 65) and E <= 512
+
+    @torch.compiler.disable
+    def _solve_eager_outside_the_trace(self, problem, term, dt0, args) -> Solution:
+        return self._solve_eager(problem, term, dt0, args)
+
+    def _solve_eager(self, problem: InitialValueProblem, term: Optional[ODETerm], dt0, args) -> Solution:
         term_ = term if term is not None else getattr(self.step_method, "term", None)
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
@@ -151,19 +231,7 @@ class AutoDiffAdjoint(nn.Module):
     def _library_setup(self, problem: InitialValueProblem, term: ODETerm, methods) -> bool:
         """One of ``methods`` and a controller as the library ships them (no overridden protocol method, the RMS
         norm), a plain term, float32 / float64 tensors."""
-        m, c = self.step_method, self.step_size_controller
-        return (
-            _library_object(m, methods)
-            and _library_object(c, (IntegralController, PIDController, FixedStepController))
-            and c.fusable
-            and isinstance(term, ODETerm)  # subclasses that only supply f (the backsolve terms) included
-            and type(term).vf is ODETerm.vf
-            and type(term).init is ODETerm.init
-            and "vf" not in vars(term)
-            and "init" not in vars(term)
-            and problem.data_dtype in _lib.DTYPES
-            and problem.time_dtype in _lib.DTYPES
-        )
+        return _library_plugins(self, term, methods) and problem.data_dtype in _lib.DTYPES and problem.time_dtype in _lib.DTYPES
 
     def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
         f = term.f
@@ -501,7 +569,6 @@ class AutoDiffAdjoint(nn.Module):
         dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
-        y_idle = torch.empty((B, F), dtype=dtype, device=dev) if E == 0 else None
         ctrl = self.step_size_controller.c_struct()
         stream = _lib.stream_of(y0)
         scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
@@ -512,79 +579,28 @@ class AutoDiffAdjoint(nn.Module):
             y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, None if dt0_ is None else dt0_.data_ptr(),
             params.data_ptr() if params.numel() else None,
             None if shared is None else shared.data_ptr(), 0 if shared is None else shared.numel(),
-            ys.data_ptr(), None if y_idle is None else y_idle.data_ptr(),
-        )  # fmt: skip  (pending, the five int32 outputs and flags stay null: set below where they are used)
+            ys.data_ptr(),
+        )  # fmt: skip  (what the general kernel needs besides lives in the workspace)
 
-        stats: Dict[str, Any] = {}
-        n_init_evals = 2 if dt0 is None else 1
-
-        # Common case first: one kernel, int64 stats written directly.  It reports through the
-        # flag block when the batch needs the general kernel (which handles every case).
-        has_general = f.builtin_kind in _lib.GENERAL_TERMS
-        fast_ok = not ctrl.has_dt_min and not ctrl.has_dt_max
-        if has_general:
-            # (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
-            fast_ok = fast_ok and self.use_fast_path and (0 < E * y0.element_size() <= 1024 or 0 < B <= _lib.END_ONLY_MAX_BATCH)
-        else:
-            fast_ok = fast_ok and E > 0 and dtype == torch.float32
-            if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
-                fast_ok = fast_ok and F in (32 * 32, 64 * 64) and E <= 8192
-            else:
-                fast_ok = fast_ok and E <= 512  # (shape and dtype were checked before the weights were packed)
-            if not fast_ok:
-                return None  # no whole-solve kernel for this case: the caller takes the protocol path
-        if fast_ok:
-            out = torch.empty((4, B), dtype=torch.int64, device=dev)
-            o0, row = out.data_ptr(), 8 * B
-            fl = (_lib.C.c_int32 * _lib.FLAG_WORDS)()
-            rc = lib.tode_solve_builtin_fast_sync(
-                _lib.C.byref(a), _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, stream, fl
-            )  # returns when the kernel has published the flag block: the one host synchronisation of the solve
-            if rc:
-                _lib.check(rc, "tode_solve_builtin_fast_sync")
-            if fl[_lib.FLAG_NEEDS_GENERAL] and not has_general:
-                return None
-            if not fl[_lib.FLAG_NEEDS_GENERAL]:
-                if term.with_stats:
-                    last = fl[_lib.FLAG_MAX_ITERATIONS]
-                    stats["n_f_evals"] = _f_evals(n_init_evals + 6 * last, B)
-                stats["n_steps"], stats["n_accepted"], stats["n_initialized"], status = out.unbind(0)
-                return Solution(ts=ts, ys=ys, stats=stats, status=status)
-
-        flags = torch.empty(_lib.FLAG_WORDS, dtype=torch.int32, device=dev)
-        a.flags = flags.data_ptr()
-        counters = torch.empty((5, B), dtype=torch.int32, device=dev)
-        a.n_steps, a.n_accepted, a.n_initialized, a.status_last, a.status_idle = (counters[i].data_ptr() for i in range(5))
-
-        def run():
-            _lib.check(lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
-            return flags.tolist()  # the one host synchronisation of the solve
-
-        fl = run()
-        pending = None
-        if fl[_lib.FLAG_NON_MONOTONE]:
-            # some t_eval row is not monotone in its direction of time: redo with a pending mask
-            pending = torch.empty((B, E), dtype=torch.uint8, device=dev)
-            a.pending = pending.data_ptr()
-            fl = run()
-        max_iter, first_fail = fl[_lib.FLAG_MAX_ITERATIONS], fl[_lib.FLAG_FIRST_FAILURE]
-        last = min(max_iter, first_fail)
-        if last < max_iter:
-            # a non-success status stops the whole batch at iteration `last`
-            a.iteration_cap = last
-            run()
-
+        # One call: the one-kernel path where the batch is in its shape, the general kernel where it is not or where
+        # the first reported that the batch leaves the common case, the int64 stats as the reference returns them.
         out = torch.empty((4, B), dtype=torch.int64, device=dev)
-        rc = lib.tode_finalize_stats(
-            B, last, *(_lib.ptr(counters[i]) for i in range(5)), *(_lib.ptr(out[i]) for i in range(4)),
-            _lib.DTYPES[dtype], F, E, _lib.ptr(ys), _lib.ptr(y_idle), stream,
-        )  # fmt: skip
-        _lib.check(rc, "tode_finalize_stats")
-
+        o0, row = out.data_ptr(), 8 * B
+        workspace = torch.empty(lib.tode_solve_workspace_bytes(_lib.C.byref(a)), dtype=torch.uint8, device=dev)
+        iterations = _lib.C.c_int64(0)
+        rc = lib.tode_solve_builtin_auto(
+            _lib.C.byref(a), _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, workspace.data_ptr(), workspace.numel(),
+            1 if self.use_fast_path else 0, stream, _lib.C.byref(iterations),
+        )  # fmt: skip  (returns after the solve's one host synchronisation)
+        if rc == _lib.E_UNSUPPORTED:
+            return None  # no whole-solve kernel for this case: the caller takes the per-step or the operator path
+        if rc:
+            _lib.check(rc, "tode_solve_builtin_auto")
+        stats: Dict[str, Any] = {}
         if term.with_stats:
-            stats["n_f_evals"] = _f_evals(n_init_evals + 6 * last, B)
-        stats["n_steps"], stats["n_accepted"], stats["n_initialized"] = out[0], out[1], out[2]
-        return Solution(ts=ts, ys=ys, stats=stats, status=out[3])
+            stats["n_f_evals"] = _f_evals((2 if dt0 is None else 1) + 6 * iterations.value, B)
+        stats["n_steps"], stats["n_accepted"], stats["n_initialized"], status = out.unbind(0)
+        return Solution(ts=ts, ys=ys, stats=stats, status=status)
 
     def __repr__(self):
         return (

@@ -16,6 +16,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtorchode_amd.so")
+OPS_LIB = os.path.join(HERE, "libtorchode_amd_ops.so")  # torch.ops.torchode_amd.*: PyTorch operators over the C ABI
 OBJ = os.path.join(HERE, "build")
 
 ARCH = "gfx950"
@@ -55,7 +56,7 @@ def source_hash() -> str:
     import hashlib
 
     h = hashlib.sha256()
-    files = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith((".hip", ".h")))
+    files = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith((".hip", ".h", ".cpp")))
     files.append(os.path.join(os.path.dirname(HERE), "include", "torchode_amd.h"))
     for path in files:
         h.update(os.path.basename(path).encode() + b"\0")
@@ -100,10 +101,38 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
             print(msg, file=sys.stderr)
         return out
 
-    with ThreadPoolExecutor(max_workers=min(8, len(UNITS))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(UNITS) + 1)) as pool:
+        ops_object = pool.submit(compile_ops_object)  # (host code only, done long before the kernels)
         objs = list(pool.map(compile_unit, UNITS))
+        ops_object = ops_object.result()
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-Wno-unused-command-line-argument", "-o", LIB, *objs])
+    link_ops_library(ops_object)
     return LIB
+
+
+def compile_ops_object() -> str:
+    """Compiles csrc/tode_torch_ops.cpp (host code only: PyTorch's headers, no kernel) to an object file."""
+    import torch
+    from torch.utils import cpp_extension
+
+    out = os.path.join(OBJ, "tode_torch_ops.o")
+    includes = [f"-I{p}" for p in cpp_extension.include_paths(device_type="cuda")] + ["-I/opt/rocm/include"]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *includes,
+          "-c", os.path.join(CSRC, "tode_torch_ops.cpp"), "-o", out])  # fmt: skip
+    return out
+
+
+def link_ops_library(obj=None) -> str:
+    """Links the operator library against PyTorch's libraries and against libtorchode_amd.so, which it finds next to itself."""
+    import torch
+
+    if obj is None:
+        obj = compile_ops_object()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    _run(["g++", "-shared", "-fPIC", obj, "-o", OPS_LIB, f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+          f"-L{HERE}", "-l:libtorchode_amd.so", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"])  # fmt: skip
+    return OPS_LIB
 
 
 if __name__ == "__main__":

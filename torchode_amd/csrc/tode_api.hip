@@ -438,4 +438,104 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
     return check_hip(hipGetLastError(), "tode_finalize_stats launch");
 }
 
+namespace tode {
+// Layout of the workspace of tode_solve_builtin_auto: each part starts at a multiple of 256 bytes.
+struct Workspace {
+    int64_t flags, counters, y_idle, pending, bytes;
+};
+static Workspace workspace_layout(const tode_solve_args &a) {
+    auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
+    const int64_t B = a.batch > 0 ? a.batch : 0, elem = a.dtype == TODE_F64 ? 8 : 4;
+    Workspace w;
+    w.flags = 0;
+    w.counters = up(TODE_FLAG_WORDS * 4);
+    w.y_idle = w.counters + up(5 * B * 4);
+    w.pending = w.y_idle + (a.n_eval == 0 ? up(B * a.n_features * elem) : 0);
+    w.bytes = w.pending + up(B * a.n_eval);
+    return w;
+}
+}  // namespace tode
+
+int64_t tode_solve_workspace_bytes(const tode_solve_args *a) {
+    if (!a || a->n_features <= 0 || a->n_eval < 0) return -1;
+    return tode::workspace_layout(*a).bytes;
+}
+
+int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st,
+                            void *workspace, int64_t workspace_bytes, int32_t allow_one_kernel, void *stream, int64_t *iterations) {
+    using namespace tode;
+    if (!a || !c || !iterations) return fail(TODE_E_INVALID, "null argument");
+    if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
+        return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
+    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    const Workspace w = workspace_layout(*a);
+    if (!workspace || workspace_bytes < w.bytes)
+        return fail(TODE_E_INVALID, "the workspace holds %lld bytes, this problem needs %lld (tode_solve_workspace_bytes)", (long long)workspace_bytes, (long long)w.bytes);
+    if (a->batch > 0 && (!ns || !na || !ni || !st)) return fail(TODE_E_INVALID, "null output pointer");
+    hipStream_t s = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)workspace;
+    const int64_t B = a->batch, E = a->n_eval, elem = a->dtype == TODE_F64 ? 8 : 4;
+    const bool small_system = a->term == TODE_TERM_LINEAR_DECAY || a->term == TODE_TERM_VAN_DER_POL || a->term == TODE_TERM_LORENZ63;
+
+    tode_solve_args b = *a;
+    b.iteration_cap = -1;
+    b.pending = nullptr;
+    b.y_idle = E == 0 ? ws + w.y_idle : nullptr;
+
+    // The common case first: one kernel that writes what the reference returns.  It reports through its flag words when the
+    // batch needs the general kernel (rows of evaluation points that are not monotone, a non-success status, non-finite values).
+    bool one_kernel = !c->has_dt_min && !c->has_dt_max;
+    if (small_system) {
+        // (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
+        one_kernel = one_kernel && allow_one_kernel && ((E > 0 && E * elem <= 1024) || (B > 0 && B <= TODE_END_ONLY_MAX_BATCH));
+    } else {
+        one_kernel = one_kernel && E > 0 && a->dtype == TODE_F32;
+        if (a->term == TODE_TERM_REACTION_DIFFUSION)
+            one_kernel = one_kernel && (a->n_features == 32 * 32 || a->n_features == 64 * 64) && E <= 8192;
+        else if (a->term == TODE_TERM_MLP)
+            one_kernel = one_kernel && a->n_features == 64 && E <= 512;
+        else
+            return fail(TODE_E_INVALID, "unknown term %d", a->term);
+        if (!one_kernel) return fail(TODE_E_UNSUPPORTED, "no whole-solve kernel for this term in this shape, dtype or controller setting");
+    }
+    if (one_kernel) {
+        int32_t fl[TODE_FLAG_WORDS];
+        int rc = tode_solve_builtin_fast_sync(&b, c, ns, na, ni, st, stream, fl);
+        if (rc) return rc;
+        if (!fl[TODE_FLAG_NEEDS_GENERAL]) {
+            *iterations = fl[TODE_FLAG_MAX_ITERATIONS];
+            return TODE_OK;
+        }
+        if (!small_system) return fail(TODE_E_UNSUPPORTED, "this batch leaves the case the whole-solve kernel of this term is built for");
+    }
+
+    // The general kernel: every case.  Up to three launches, each followed by a look at its flag words.
+    b.flags = (int32_t *)(ws + w.flags);
+    int32_t *counters = (int32_t *)(ws + w.counters);
+    b.n_steps = counters, b.n_accepted = counters + B, b.n_initialized = counters + 2 * B, b.status_last = counters + 3 * B, b.status_idle = counters + 4 * B;
+    int32_t fl[TODE_FLAG_WORDS] = {0, INT_MAX, 0, 0};
+    auto run = [&]() -> int {
+        int rc = tode_solve_builtin(&b, c, stream);
+        if (rc) return rc;
+        rc = check_hip(hipMemcpyAsync(fl, b.flags, sizeof(fl), hipMemcpyDeviceToHost, s), "tode_solve_builtin_auto: reading the flag words");
+        if (rc) return rc;
+        return check_hip(hipStreamSynchronize(s), "tode_solve_builtin_auto: waiting for the solve");
+    };
+    int rc = run();
+    if (rc) return rc;
+    if (fl[TODE_FLAG_NON_MONOTONE]) {  // some row of evaluation points is not monotone in its direction of time: again, with a mask
+        b.pending = ws + w.pending;
+        if ((rc = run())) return rc;
+    }
+    const int64_t most = fl[TODE_FLAG_MAX_ITERATIONS], first_failure = fl[TODE_FLAG_FIRST_FAILURE];
+    const int64_t last = most < first_failure ? most : first_failure;
+    if (last < most) {  // a non-success status stops the whole batch at iteration `last` (adjoints.py:229-238)
+        b.iteration_cap = last;
+        if ((rc = run())) return rc;
+    }
+    *iterations = last;
+    return tode_finalize_stats(B, last, b.n_steps, b.n_accepted, b.n_initialized, b.status_last, b.status_idle, ns, na, ni, st, a->dtype, a->n_features,
+                               a->n_eval, a->ys, b.y_idle, stream);
+}
+
 }  // extern "C"

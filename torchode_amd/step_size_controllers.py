@@ -171,6 +171,15 @@ class AdaptiveStepSizeController(StepSizeController):
             float(self.factor_min), float(self.factor_max), float(dt_min or 0.0), float(dt_max or 0.0),
         )  # fmt: skip
 
+    def control_values(self):
+        """``(kind, values)``: the same parameters as plain Python numbers, in the order of ``struct tode_controller``
+        with NaN for a step size limit that is not set, as ``torch.ops.torchode_amd.solve_builtin`` takes them."""
+        nan = float("nan")
+        return self._kind, [
+            self._atol_f, self._rtol_f, float(self.pcoeff), float(self.icoeff), float(self.dcoeff), float(self.safety), float(self.factor_min),
+            float(self.factor_max), nan if self.dt_min is None else float(self.dt_min), nan if self.dt_max is None else float(self.dt_max),
+        ]  # fmt: skip
+
     # ------------------------------------------------------------------ #
     def initial_state(self, method_order: int, problem: InitialValueProblem, dt_min, dt_max):
         raise NotImplementedError()
