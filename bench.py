@@ -43,10 +43,12 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the solve kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
 # profiles/); absent (null in the output) where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6873.0 KiB x 2.000 + 32671.0 KiB x 1.000) x 1024
-    ("vdp", "torch.float32", 65536): 47.53e6,
-    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (77710 KiB x 2.000 + 870500 KiB x 1.000) x 1024
-    ("lorenz", "torch.float32", 1048576): 1050.5e6,
+    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6876.0 KiB x 2.000 + 32933.9 KiB x 1.000) x 1024
+    ("vdp", "torch.float32", 65536): 47.81e6,
+    # profiles/solve_pair_kernel_vdp_f64_b65536_hbm_traffic.txt: (25316.5 KiB x 2.000 + 101408.5 KiB x 1.000) x 1024
+    ("vdp", "torch.float64", 65536): 155.69e6,
+    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (78246.4 KiB x 2.000 + 931465.0 KiB x 1.000) x 1024
+    ("lorenz", "torch.float32", 1048576): 1114.07e6,
     # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4370 KiB x 2.000 + 819300 KiB x 1.000) x 1024
     ("reaction_diffusion", "torch.float32", 512): 847.9e6,
     # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1498 KiB x 2.000 + 20624 KiB x 1.000) x 1024
