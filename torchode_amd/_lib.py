@@ -274,6 +274,8 @@ def load():
     other sources than the ones lying next to it (the library carries a hash of its sources): an edited kernel is
     never run through a stale binary.  Where the sources are absent (an installed copy) the file is taken as it is."""
     global _lib
+    if _lib is not None:
+        return _lib
     with _lock:
         if _lib is not None:
             return _lib
@@ -403,7 +405,13 @@ def require_device(*tensors):
             )
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t) -> C.c_void_p:
+    """PyTorch's current stream on the tensor's device, as the handle the C ABI takes."""
+    if _raw_stream is not None:  # (the handle without a Stream object around it: 0.3 instead of 3 microseconds)
+        return C.c_void_p(_raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 

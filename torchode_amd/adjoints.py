@@ -47,9 +47,18 @@ def _library_object(obj, classes) -> bool:
     return _PROTOCOL_NAME_SET.isdisjoint(vars(obj))
 
 
+def _sub(module, name):
+    """``module.name`` for an attribute that usually is a submodule: ``nn.Module`` keeps those in a dict of their own and
+    finds them only through ``__getattr__``, several times the cost of this lookup on a path that runs per solve."""
+    found = module.__dict__.get(name)
+    if found is None and not torch.compiler.is_compiling():
+        found = module._modules.get(name)
+    return getattr(module, name) if found is None else found
+
+
 def _library_plugins(adjoint, term, methods) -> bool:
     """The part of ``AutoDiffAdjoint._library_setup`` that looks at the plug-in objects only."""
-    m, c = adjoint.step_method, adjoint.step_size_controller
+    m, c = _sub(adjoint, "step_method"), _sub(adjoint, "step_size_controller")
     return (
         _library_object(m, methods)
         and _library_object(c, (IntegralController, PIDController, FixedStepController))
@@ -183,7 +192,7 @@ class AutoDiffAdjoint(nn.Module):
         return self._solve_eager(problem, term, dt0, args)
 
     def _solve_eager(self, problem: InitialValueProblem, term: Optional[ODETerm], dt0, args) -> Solution:
-        term_ = term if term is not None else getattr(self.step_method, "term", None)
+        term_ = term if term is not None else getattr(_sub(self, "step_method"), "term", None)
         assert term_ is not None, "no ODE term given, neither to solve() nor to the step method"
         _lib.require_device(problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0)
         grad_on = torch.is_grad_enabled()
@@ -234,12 +243,12 @@ class AutoDiffAdjoint(nn.Module):
         return _library_plugins(self, term, methods) and problem.data_dtype in _lib.DTYPES and problem.time_dtype in _lib.DTYPES
 
     def _persistent_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        f = term.f
+        f = _sub(term, "f")
         return (
-            self._fused_ok(problem, term)
+            isinstance(f, BuiltinTerm)
+            and self._fused_ok(problem, term)
             and problem.data_dtype == problem.time_dtype  # (the whole-solve kernels are built for one dtype)
-            and type(self.step_size_controller) is not FixedStepController
-            and isinstance(f, BuiltinTerm)
+            and type(_sub(self, "step_size_controller")) is not FixedStepController
             and f.builtin_kind in _lib.PERSISTENT_TERMS
             and not term.with_args
         )
@@ -540,7 +549,8 @@ class AutoDiffAdjoint(nn.Module):
 
     def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
         lib = _lib.load()
-        f: BuiltinTerm = term.f
+        f: BuiltinTerm = _sub(term, "f")
+        method_id, controller = _sub(self, "step_method").method_id, _sub(self, "step_size_controller")
         # What depends on the problem's tensors alone is worked out once per problem object and kept on it (checked by
         # identity, since the attributes of a problem may be reassigned, and by the tensors' version counters, since
         # the plan may hold a contiguous copy of one of them that an in-place update of the original would not reach).
@@ -555,10 +565,12 @@ class AutoDiffAdjoint(nn.Module):
             ts = problem.t_eval if problem.t_eval is not None else problem.t_end[:, None]
             plan = (tensors, y0, t_start, t_end, t_eval, ts, y0.device, y0.dtype, y0.shape[0], y0.shape[1], problem.n_evaluation_points,
                     y0.data_ptr(), t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0),
-                    None if t_eval is None else t_eval.data_ptr(), versions)  # fmt: skip
+                    None if t_eval is None else t_eval.data_ptr(), {}, versions)  # fmt: skip
             problem._launch_plan = plan
-        _, y0, t_start, t_end, t_eval, ts, dev, dtype, B, F, E, y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, _ = plan
-        params = f.builtin_params().to(device=dev, dtype=dtype)
+        _, y0, t_start, t_end, t_eval, ts, dev, dtype, B, F, E, y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, _, _ = plan
+        params = f.builtin_params()
+        if params.device != dev or params.dtype != dtype:
+            params = params.to(device=dev, dtype=dtype)
         if params.numel() == 0 and params.shape[0] != B:  # a term without per-sample parameters
             params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
@@ -569,27 +581,40 @@ class AutoDiffAdjoint(nn.Module):
         dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
-        ctrl = self.step_size_controller.c_struct()
+        ctrl = controller.c_struct()
         stream = _lib.stream_of(y0)
-        scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
 
-        a = _lib.SolveArgs(  # positional, in the order of struct tode_solve_args
-            _lib.DTYPES[dtype], self.step_method.method_id, f.builtin_kind, F, E, params.shape[1], B,
-            -1 if self.max_steps is None else int(self.max_steps), -1, (_lib.C.c_double * 4)(*scal[:4]),
-            y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, None if dt0_ is None else dt0_.data_ptr(),
-            params.data_ptr() if params.numel() else None,
-            None if shared is None else shared.data_ptr(), 0 if shared is None else shared.numel(),
-            ys.data_ptr(),
-        )  # fmt: skip  (what the general kernel needs besides lives in the workspace)
+        # The argument struct is kept with the plan and copied from there while it describes the same call (same problem
+        # tensors, parameters, first step, method, term and step limit): only the output pointer changes from solve to solve.
+        key = (method_id, f.builtin_kind, self.max_steps, params.data_ptr(), None if dt0_ is None else dt0_.data_ptr(),
+               None if shared is None else shared.data_ptr())  # fmt: skip
+        held = plan[-2]
+        if held.get("key") != key:
+            scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
+            a = _lib.SolveArgs(  # positional, in the order of struct tode_solve_args
+                _lib.DTYPES[dtype], method_id, f.builtin_kind, F, E, params.shape[1], B,
+                -1 if self.max_steps is None else int(self.max_steps), -1, (_lib.C.c_double * 4)(*scal[:4]),
+                y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, None if dt0_ is None else dt0_.data_ptr(),
+                params.data_ptr() if params.numel() else None,
+                None if shared is None else shared.data_ptr(), 0 if shared is None else shared.numel(),
+            )  # fmt: skip  (what the general kernel needs besides lives in the workspace)
+            held.update(key=key, args=a, workspace_bytes=lib.tode_solve_workspace_bytes(_lib.C.byref(a)), scalars=tuple(scal[:4]),
+                        keep=(params, dt0_, shared))  # fmt: skip
+        elif held["scalars"] != tuple((list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4)[:4]):
+            held.clear()  # (a scalar of the term was reassigned: describe the call anew)
+            return self._solve_persistent(problem, term, dt0)
+        a = _lib.SolveArgs.from_buffer_copy(held["args"])  # (a copy per call: solves of one problem object may overlap in threads)
+        a.ys = ys.data_ptr()
+        a_ref = _lib.C.byref(a)
 
         # One call: the one-kernel path where the batch is in its shape, the general kernel where it is not or where
         # the first reported that the batch leaves the common case, the int64 stats as the reference returns them.
         out = torch.empty((4, B), dtype=torch.int64, device=dev)
         o0, row = out.data_ptr(), 8 * B
-        workspace = torch.empty(lib.tode_solve_workspace_bytes(_lib.C.byref(a)), dtype=torch.uint8, device=dev)
+        workspace = torch.empty(held["workspace_bytes"], dtype=torch.uint8, device=dev)
         iterations = _lib.C.c_int64(0)
         rc = lib.tode_solve_builtin_auto(
-            _lib.C.byref(a), _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, workspace.data_ptr(), workspace.numel(),
+            a_ref, _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, workspace.data_ptr(), held["workspace_bytes"],
             1 if self.use_fast_path else 0, stream, _lib.C.byref(iterations),
         )  # fmt: skip  (returns after the solve's one host synchronisation)
         if rc == _lib.E_UNSUPPORTED:

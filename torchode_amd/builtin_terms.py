@@ -62,9 +62,11 @@ class VanDerPol(BuiltinTerm):
         return torch.stack((v, dv), dim=1)
 
     def builtin_params(self):
-        mu = self.mu
         if torch.compiler.is_compiling():  # (the cache below keys on the tensor's version counter, which a tracer cannot read)
-            return mu.reshape(-1, 1)
+            return self.mu.reshape(-1, 1)
+        mu = self._buffers.get("mu")  # (a dictionary read; `self.mu` goes through nn.Module.__getattr__)
+        if mu is None:
+            mu = self.mu
         cached = self.__dict__.get("_params_view")
         if cached is None or cached[0] is not mu or cached[1] != mu._version:
             cached = self.__dict__["_params_view"] = (mu, mu._version, mu.reshape(-1, 1).contiguous())
