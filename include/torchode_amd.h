@@ -24,10 +24,16 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 17
+#define TODE_ABI_VERSION 18
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
+/* A dtype argument when time and data differ (reference problems.py:44-56, tests/dtype_stability_test.py):
+ * TODE_DTYPES(data, time); a plain TODE_F32 / TODE_F64 means both.  Time: t, dt, t_start, t_end, t_eval, a user's
+ * dt0 and everything derived (node times, next step size, step limits).  Data: y, parameters of the term,
+ * derivatives, coefficients, error norms and ratios, ys. */
+#define TODE_DTYPE_PAIR 0x100
+#define TODE_DTYPES(data, time) (TODE_DTYPE_PAIR | (data) | ((time) << 4))
 /* single step methods: reference single_step_methods/dopri5.py, tsit5.py, heun.py, euler.py */
 enum { TODE_DOPRI5 = 0, TODE_TSIT5 = 1, TODE_HEUN = 2, TODE_EULER = 3 /* the last two: per-step entry points only */ };
 /* step size controllers: reference step_size_controllers.py:260 (integral), :554 (PID) */
@@ -119,7 +125,9 @@ typedef struct tode_controller {
  * tode_finalize_stats.
  */
 typedef struct tode_solve_args {
-    int32_t dtype;  /* TODE_F32 | TODE_F64, for data and time alike */
+    int32_t dtype;  /* TODE_F32 | TODE_F64 for data and time alike; TODE_DTYPES(data, time) where they differ:
+                       tode_solve_builtin and tode_solve_builtin_auto take it for the three small systems (the
+                       general kernel is built for all four pairs), the fast entry points return TODE_E_UNSUPPORTED */
     int32_t method; /* TODE_DOPRI5 | TODE_TSIT5 */
     int32_t term;   /* TODE_TERM_* */
     int32_t n_features;        /* F */
@@ -544,11 +552,7 @@ int tode_step_stage_backward(const tode_step_adjoint *adjoint, const tode_contro
  * host arrays read before the call returns.  Arrays are dense row-major.
  * ------------------------------------------------------------------------------------------ */
 #define TODE_MAX_STAGES 16
-/* dtype argument of the operators when time and data differ: TODE_DTYPES(data, time); a plain
- * TODE_F32 / TODE_F64 means both.  Time: t, dt, t_start, t_end, t_eval and everything derived
- * (node times, next step size).  Data: y, derivatives, coefficients, error norms and ratios. */
-#define TODE_DTYPE_PAIR 0x100
-#define TODE_DTYPES(data, time) (TODE_DTYPE_PAIR | (data) | ((time) << 4))
+/* dtype argument of the operators: TODE_F32, TODE_F64 or TODE_DTYPES(data, time), defined at the top of this file. */
 enum { TODE_NORM_RMS = 0, TODE_NORM_MAX = 1 }; /* reference step_size_controllers.py:170-186 */
 
 /* Coefficients the kernels use for Dopri5 / Tsit5 (reference dopri5.py:11-44, tsit5.py:11-114), as doubles:

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import torchode_amd as to
-from helpers import assert_identical, c_oracle_solve, gpu_solve, mixed_error, torch_oracle_solve
+from helpers import assert_identical, c_oracle_solve, gpu_solve, make_controller, mixed_error, torch_oracle_solve
 
 pytestmark = pytest.mark.gpu
 
@@ -721,3 +721,66 @@ def test_wild_configurations_with_non_finite_samples(seed):
     y0 = poisoned(y0, seed)
     kw = dict(t_start=t_start, t_end=t_end, dt0=dt0, max_steps=min(max_steps, 400))
     assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, **kw), c_oracle_solve(f, y0, t_eval, method, ctrl, **kw))
+
+
+# ---------------------------------------------------------------------------------------------
+# time and data in different dtypes (reference problems.py:44-56, tests/dtype_stability_test.py): the general
+# whole-solve kernel against the per-step kernels (the same term behind a plain callable), which reproduce the
+# ATen-op oracle's mixed-dtype vectors -- same bits, every stat
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("time_dtype,data_dtype", [(torch.float64, torch.float32), (torch.float32, torch.float64)], ids=["t64-y32", "t32-y64"])
+@pytest.mark.parametrize("case", ["vdp", "lorenz", "linear_decay", "backwards", "non-monotone", "no-t_eval", "dt0", "limits", "max_steps", "non-finite", "empty"])
+def test_mixed_dtypes_whole_solve_kernel_equals_the_per_step_kernels(case, time_dtype, data_dtype):
+    name = case if case in ("lorenz", "linear_decay") else "vdp"
+    w = to.workloads.make(name, batch=200, dtype=torch.float64)
+    n = 0 if case == "empty" else 200
+    w = w._replace(y0=w.y0[:n], t_eval=w.t_eval[:n])
+    params = w.f.builtin_params().to(data_dtype)[:n]
+    f = type(w.f)(params[:, 0] if params.shape[1] == 1 and name != "linear_decay" else params).cuda()
+    y0, t_eval = w.y0.clone(), w.t_eval.clone()
+    t_start = t_end = dt0 = None
+    kw, ctrl = {}, dict(w.controller)
+    if case == "backwards":
+        t_eval[::2] = t_eval[::2].flip(1)
+        t_eval[::2] = t_eval[::2, :1] - 0.01 * (t_eval[::2, :1] - t_eval[::2])
+    if case == "non-monotone":
+        t_eval[::5, 3], t_eval[::5, 7] = t_eval[::5, 7].clone(), t_eval[::5, 3].clone()
+    if case == "no-t_eval":
+        t_start, t_end, t_eval = t_eval[:, 0].clone(), t_eval[:, -1].clone(), None
+    if case == "dt0":
+        dt0 = torch.full((y0.shape[0],), 1e-3, dtype=time_dtype, device="cuda")
+    if case == "limits":
+        ctrl.update(dt_min=2e-2, dt_max=0.25)
+    if case == "max_steps":
+        kw["max_steps"] = 25
+    if case == "non-finite":
+        y0[7] = float("inf")
+    mv = lambda x, dt: None if x is None else x.to(dt).cuda()
+    problem = to.InitialValueProblem(mv(y0, data_dtype), mv(t_start, time_dtype), mv(t_end, time_dtype), mv(t_eval, time_dtype))
+    method = {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[w.method]
+    solver = to.AutoDiffAdjoint(method(), make_controller(ctrl), **kw)
+    whole_term, plain_term = to.ODETerm(f), to.ODETerm(lambda t, y: f(t, y))
+    assert solver._persistent_ok(problem, whole_term) and not solver._persistent_ok(problem, plain_term)
+    with torch.no_grad():
+        whole = solver.solve(problem, whole_term, dt0=dt0)
+        steps = solver.solve(problem, plain_term, dt0=dt0)
+    assert whole.ys.dtype == data_dtype and whole.ts.dtype == time_dtype and whole.ys.shape == steps.ys.shape
+    for key in ("n_steps", "n_accepted", "n_initialized", "n_f_evals"):
+        assert torch.equal(whole.stats[key].cpu(), steps.stats[key].cpu()), key
+    assert torch.equal(whole.status, steps.status)
+    E = whole.ys.shape[1]
+    written = torch.arange(E, device="cuda")[None, :] < steps.stats["n_initialized"][:, None]
+    if case == "non-monotone":  # every fifth row: what is written there is no prefix of the row
+        written = written & (torch.arange(y0.shape[0], device="cuda") % 5 != 0)[:, None]
+    a, b = whole.ys[written], steps.ys[written]
+    assert bool(((a == b) | (a.isnan() & b.isnan())).all()), (a - b).abs().nan_to_num().max().item()
+    if case == "limits":
+        assert (whole.status == 2).any()
+    elif case == "max_steps":
+        assert (whole.status == 3).any()
+    elif case == "non-finite":
+        assert (whole.status != 0).any()
+    elif case != "empty":
+        assert (whole.status == 0).all() and int(whole.stats["n_steps"].max()) > 10

@@ -484,8 +484,13 @@ def test_mixed_dtypes_match_the_aten_op_oracle_fixture(path):
     f = type(w.f)(params[:, 0] if params.shape[1] == 1 else params).cuda()
     problem = to.InitialValueProblem(w.y0.to(data_dtype).cuda(), t_eval=w.t_eval.to(time_dtype).cuda())
     fused_method, operator_method = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[g["method"]]
-    for method in (fused_method, operator_method):
-        sol = to.AutoDiffAdjoint(method(), make_controller(g["controller"])).solve(problem, to.ODETerm(lambda t, y: f(t, y)))
+    # the per-step kernels, the operator path, and (the term handed over as it is, not behind a plain callable) the
+    # general whole-solve kernel, which is built for the four (time, data) pairs
+    for method, term in ((fused_method, to.ODETerm(lambda t, y: f(t, y))), (operator_method, to.ODETerm(lambda t, y: f(t, y))), (fused_method, to.ODETerm(f))):
+        solver = to.AutoDiffAdjoint(method(), make_controller(g["controller"]))
+        assert solver._persistent_ok(problem, term) == (term.f is f)
+        with torch.no_grad():
+            sol = solver.solve(problem, term)
         for key in ("n_steps", "n_accepted", "n_initialized"):
             assert sol.stats[key].tolist() == g[key], (method.__name__, key)
         assert sol.status.tolist() == g["status"] and int(sol.stats["n_f_evals"][0]) == g["n_f_evals"]

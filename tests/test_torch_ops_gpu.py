@@ -102,6 +102,22 @@ def test_compiled_solve_is_one_operator_and_equals_the_eager_solve(name, batch, 
         assert (eager.status == 3).any()
 
 
+@pytest.mark.parametrize("time_dtype,data_dtype", [(torch.float64, torch.float32), (torch.float32, torch.float64)], ids=["t64-y32", "t32-y64"])
+def test_compiled_solve_with_time_and_data_in_different_dtypes(time_dtype, data_dtype):
+    torch._dynamo.reset()
+    w = to.workloads.make("lorenz", batch=100, dtype=torch.float64)
+    f = type(w.f)(w.f.builtin_params().to(data_dtype)[:, 0]).to(DEV)
+    problem = to.InitialValueProblem(w.y0.to(data_dtype).to(DEV), t_eval=w.t_eval.to(time_dtype).to(DEV))
+    term, solver = to.ODETerm(f), solver_of(w)
+    with torch.no_grad():
+        eager = solver.solve(problem, term)
+        backend = Captured()
+        traced = torch.compile(solver.solve, backend=backend, fullgraph=True)(problem, term)
+    same_solution(traced, eager)
+    assert traced.ys.dtype == data_dtype and traced.ts.dtype == time_dtype
+    assert [c for c in backend.calls[0] if c.startswith("torchode_amd.")] == ["torchode_amd.solve_builtin"]
+
+
 def test_operator_called_directly_and_its_tracing_rule():
     w, problem, _ = problem_of("vdp", 128, torch.float32)
     term = to.ODETerm(copy.deepcopy(w.f).to(DEV))

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}

@@ -247,7 +247,8 @@ class AutoDiffAdjoint(nn.Module):
         return (
             isinstance(f, BuiltinTerm)
             and self._fused_ok(problem, term)
-            and problem.data_dtype == problem.time_dtype  # (the whole-solve kernels are built for one dtype)
+            # (time and data in different dtypes: the general kernel of the three small systems is built for them)
+            and (problem.data_dtype == problem.time_dtype or f.builtin_kind in _lib.GENERAL_TERMS)
             and type(_sub(self, "step_size_controller")) is not FixedStepController
             and f.builtin_kind in _lib.PERSISTENT_TERMS
             and not term.with_args
@@ -578,7 +579,8 @@ class AutoDiffAdjoint(nn.Module):
         if mlp and (dtype != torch.float32 or F != 64 or tuple(f.W1.shape) != (256, 65)):
             return None  # the matrix-core kernel is built for this shape only: the caller takes the protocol path
         shared = f.builtin_packed(dev, dtype) if mlp else None
-        dt0_ = None if dt0 is None else dt0.to(dtype).contiguous()
+        ttype = t_start.dtype
+        dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()
 
         ys = torch.empty((B, max(E, 1), F), dtype=dtype, device=dev)
         ctrl = controller.c_struct()
@@ -592,7 +594,7 @@ class AutoDiffAdjoint(nn.Module):
         if held.get("key") != key:
             scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
             a = _lib.SolveArgs(  # positional, in the order of struct tode_solve_args
-                _lib.DTYPES[dtype], method_id, f.builtin_kind, F, E, params.shape[1], B,
+                _lib.dtype_code(dtype, ttype), method_id, f.builtin_kind, F, E, params.shape[1], B,
                 -1 if self.max_steps is None else int(self.max_steps), -1, (_lib.C.c_double * 4)(*scal[:4]),
                 y0_ptr, t_start_ptr, t_end_ptr, t_start_stride, t_end_stride, t_eval_ptr, None if dt0_ is None else dt0_.data_ptr(),
                 params.data_ptr() if params.numel() else None,

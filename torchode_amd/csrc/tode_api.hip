@@ -250,9 +250,10 @@ int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void 
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (a->batch > (int64_t)2147483647 * TODE_BLOCK) return fail(TODE_E_UNSUPPORTED, "batch too large");
     hipStream_t s = (hipStream_t)stream;
-    if (a->dtype == TODE_F32) return solve_builtin_f32(*a, *c, s);
-    if (a->dtype == TODE_F64) return solve_builtin_f64(*a, *c, s);
-    return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    const int data = data_type(a->dtype), time = time_type(a->dtype);
+    if (data == time) return data == TODE_F32 ? solve_builtin_f32(*a, *c, s) : solve_builtin_f64(*a, *c, s);
+    return data == TODE_F32 ? solve_builtin_t64_y32(*a, *c, s) : solve_builtin_t32_y64(*a, *c, s);
 }
 
 int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,
@@ -274,7 +275,8 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         return fail(TODE_E_INVALID, "t_start_stride / t_end_stride must be >= 1 (got %lld, %lld)", (long long)a->t_start_stride, (long long)a->t_end_stride);
     if (a->batch > (int64_t)2147483647 * 64) return fail(TODE_E_UNSUPPORTED, "batch too large");
     hipStream_t s = (hipStream_t)stream;
-    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (a->dtype & TODE_DTYPE_PAIR) return fail(TODE_E_UNSUPPORTED, "the fast entry point is built for time and data in one dtype");
     if (a->term == TODE_TERM_REACTION_DIFFUSION) {
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for float32");
         return solve_grid_f32(*a, *c, ns, na, ni, st, s);
@@ -357,7 +359,8 @@ int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controll
     using namespace tode;
     if (!a || !c || !flags_out) return fail(TODE_E_INVALID, "null argument");
     if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0) return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d", (long long)a->batch, a->n_features, a->n_eval);
-    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (a->dtype & TODE_DTYPE_PAIR) return fail(TODE_E_UNSUPPORTED, "the fast entry points are built for time and data in one dtype");
     const bool end_only = a->n_eval == 0;
     const size_t value_bytes = a->dtype == TODE_F32 ? 4 : 8;
     if (end_only && (uint64_t)a->batch * (uint64_t)a->n_features > TODE_STATIC_STAGING_BYTES / value_bytes)
@@ -445,7 +448,7 @@ struct Workspace {
 };
 static Workspace workspace_layout(const tode_solve_args &a) {
     auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
-    const int64_t B = a.batch > 0 ? a.batch : 0, elem = a.dtype == TODE_F64 ? 8 : 4;
+    const int64_t B = a.batch > 0 ? a.batch : 0, elem = data_type(a.dtype) == TODE_F64 ? 8 : 4;
     Workspace w;
     w.flags = 0;
     w.counters = up(TODE_FLAG_WORDS * 4);
@@ -467,14 +470,15 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
     if (!a || !c || !iterations) return fail(TODE_E_INVALID, "null argument");
     if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
         return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
-    if (a->dtype != TODE_F32 && a->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
+    const bool one_dtype = !(a->dtype & TODE_DTYPE_PAIR);  // (time and data in different types: the general kernel)
     const Workspace w = workspace_layout(*a);
     if (!workspace || workspace_bytes < w.bytes)
         return fail(TODE_E_INVALID, "the workspace holds %lld bytes, this problem needs %lld (tode_solve_workspace_bytes)", (long long)workspace_bytes, (long long)w.bytes);
     if (a->batch > 0 && (!ns || !na || !ni || !st)) return fail(TODE_E_INVALID, "null output pointer");
     hipStream_t s = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
-    const int64_t B = a->batch, E = a->n_eval, elem = a->dtype == TODE_F64 ? 8 : 4;
+    const int64_t B = a->batch, E = a->n_eval, elem = data_type(a->dtype) == TODE_F64 ? 8 : 4;
     const bool small_system = a->term == TODE_TERM_LINEAR_DECAY || a->term == TODE_TERM_VAN_DER_POL || a->term == TODE_TERM_LORENZ63;
 
     tode_solve_args b = *a;
@@ -484,7 +488,7 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
 
     // The common case first: one kernel that writes what the reference returns.  It reports through its flag words when the
     // batch needs the general kernel (rows of evaluation points that are not monotone, a non-success status, non-finite values).
-    bool one_kernel = !c->has_dt_min && !c->has_dt_max;
+    bool one_kernel = one_dtype && !c->has_dt_min && !c->has_dt_max;
     if (small_system) {
         // (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
         one_kernel = one_kernel && allow_one_kernel && ((E > 0 && E * elem <= 1024) || (B > 0 && B <= TODE_END_ONLY_MAX_BATCH));
@@ -534,7 +538,7 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
         if ((rc = run())) return rc;
     }
     *iterations = last;
-    return tode_finalize_stats(B, last, b.n_steps, b.n_accepted, b.n_initialized, b.status_last, b.status_idle, ns, na, ni, st, a->dtype, a->n_features,
+    return tode_finalize_stats(B, last, b.n_steps, b.n_accepted, b.n_initialized, b.status_last, b.status_idle, ns, na, ni, st, data_type(a->dtype), a->n_features,
                                a->n_eval, a->ys, b.y_idle, stream);
 }
 

@@ -20,8 +20,22 @@
 #ifndef TODE_INSTANTIATE_F64
 #define TODE_INSTANTIATE_F64 0
 #endif
+#ifndef TODE_INSTANTIATE_T64_Y32
+#define TODE_INSTANTIATE_T64_Y32 0
+#endif
+#ifndef TODE_INSTANTIATE_T32_Y64
+#define TODE_INSTANTIATE_T32_Y64 0
+#endif
 
 namespace tode {
+// The two halves of a dtype argument: a plain TODE_F32 / TODE_F64 means both, TODE_DTYPES(data, time) names each.
+inline int data_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? (dtype & 0xF) : dtype; }
+inline int time_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? ((dtype >> 4) & 0xF) : dtype; }
+inline bool known_dtype(int32_t dtype) {
+    const int d = data_type(dtype), t = time_type(dtype);
+    return (d == TODE_F32 || d == TODE_F64) && (t == TODE_F32 || t == TODE_F64) && !(dtype & ~(TODE_DTYPE_PAIR | 0xFF));
+}
+
 // Records a formatted message for tode_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...);
 // Maps a HIP error to TODE_E_HIP (recording its string) or returns TODE_OK.
@@ -46,6 +60,8 @@ void timing_after(hipStream_t s);
 
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 int solve_pair_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
 int solve_pair_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);

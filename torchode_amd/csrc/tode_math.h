@@ -500,6 +500,23 @@ template <typename T> __device__ __forceinline__ int limit_dt(const CtrlParams<T
     return status;
 }
 
+// dt_min / dt_max and the status of a step proposal, limits in the time type
+// (step_size_controllers.py:406-422, 751-767).
+template <typename TT, typename T>
+__device__ __forceinline__ int limit_step(const CtrlParams<T> &cp, TT dt_min, TT dt_max, T ratio, TT &dt_next) {
+    int status = finite_(ratio) ? 0 : 4;
+    if (cp.has_dt_min || cp.has_dt_max) {
+        const TT mag = abs_(dt_next);
+        TT c = mag;
+        if (cp.has_dt_min) c = tmax(c, dt_min);
+        if (cp.has_dt_max) c = tmin(c, dt_max);
+        const TT sg = (dt_next > 0) ? (TT)1 : ((dt_next < 0) ? (TT)-1 : dt_next);
+        dt_next = sg * c;
+        if (cp.has_dt_min && mag < dt_min) status = 2;
+    }
+    return status;
+}
+
 // Quartic coefficients of the dense output, lowest power first.
 // Tsit5: tsit5.py:123-139.  Dopri5: dopri5.py:53-60 -> interpolation.py:138-170.
 template <typename T, int F, int METHOD>
@@ -544,11 +561,11 @@ __device__ __forceinline__ void quartic(T dt, const T (&y0)[F], const T (&y1)[F]
 }
 
 // Horner on x = (t - t0) / ((t0 + dt) - t0), interpolation.py:25-40.
-template <typename T, int F> __device__ __forceinline__ void quartic_eval(const T (&q)[5][F], T t0, T dt, T t, T (&out)[F]) {
-    T t1 = t0 + dt;
-    T den = t1 - t0;
-    if (!(abs_(den) > (T)0)) den = (T)1;
-    T x = (t - t0) / den;
+template <typename T, int F, typename TT = T> __device__ __forceinline__ void quartic_eval(const T (&q)[5][F], TT t0, TT dt, TT t, T (&out)[F]) {
+    TT t1 = t0 + dt;
+    TT den = t1 - t0;
+    if (!(abs_(den) > (TT)0)) den = (TT)1;
+    T x = (T)((t - t0) / den);  // (formed in the time type, then taken to the data type: interpolation.py:8-40)
 #pragma unroll
     for (int f = 0; f < F; ++f) {
         T y = q[4][f];

@@ -487,8 +487,6 @@ static __global__ void __launch_bounds__(256) count_initialized_kernel(long long
 
 static unsigned blocks_for(long long n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
-static int data_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? (dtype & 0xF) : dtype; }
-static int time_type(int32_t dtype) { return (dtype & TODE_DTYPE_PAIR) ? ((dtype >> 4) & 0xF) : dtype; }
 
 static int check_common(int32_t dtype, int64_t batch, int32_t F) {
     const int d = data_type(dtype), t = time_type(dtype);

@@ -12,8 +12,11 @@
 
 namespace tode {
 
-template <typename T, int METHOD, int CTRL, typename Term>
-__global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> p) {
+// T: data type, TT: time type (the same in the common case; where they differ the conversions stand where the
+// reference's loop of torch operations has them: the step in the data type for stage sums and interpolants, the step
+// factor in the time type for the next step, the position of an evaluation point in its step formed in the time type).
+template <typename T, int METHOD, int CTRL, typename Term, typename TT = T>
+__global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, TT> p) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
     constexpr int P = Term::P;
@@ -30,19 +33,19 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
         T y[F], k[7][F];
 #pragma unroll
         for (int f = 0; f < F; ++f) y[f] = p.y0[b * F + f];
-        const T ts = p.t_start[b * p.ts_stride], te = p.t_end[b * p.te_stride];
+        const TT ts = p.t_start[b * p.ts_stride], te = p.t_end[b * p.te_stride];
         const T dir = (te > ts) ? (T)1 : (T)-1;
-        const T tlo = tmin(ts, te), thi = tmax(te, ts);
-        const T *tev = p.t_eval ? p.t_eval + b * E : nullptr;
+        const TT tlo = tmin(ts, te), thi = tmax(te, ts);
+        const TT *tev = p.t_eval ? p.t_eval + b * E : nullptr;
         T *ys = p.ys + b * (long long)(E > 0 ? E : 1) * F;
 
         // evaluation points: a cursor is equivalent to the reference's pending mask when
         // the row is monotone in the direction of time; otherwise fall back to the mask
         bool use_mask = false;
         if (tev) {
-            T prev_te = tev[0];
+            TT prev_te = tev[0];
             for (int e = 1; e < E; ++e) {
-                T cur = tev[e];
+                TT cur = tev[e];
                 if (!(dir > 0 ? cur >= prev_te : cur <= prev_te)) use_mask = true;
                 prev_te = cur;
             }
@@ -59,12 +62,13 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
             }
         }
 
-        T t = ts, dt;
+        TT t = ts, dt;
         if (p.dt0) {
             dt = p.dt0[b];
-            rhs(ts, y, k[0]);
+            rhs((T)ts, y, k[0]);
         } else {
-            dt = initial_step<T, CTRL, Term>(cp, rhs, ts, y, dir, abs_(te - ts), k[0]);
+            // (the terms built for this kernel do not look at the time they are given)
+            dt = (TT)initial_step<T, CTRL, Term>(cp, rhs, (T)ts, y, dir, (T)abs_(te - ts), k[0]);
         }
         dt = tclamp(dt, tlo - t, thi - t);
         T prev = (T)1, prev_prev = (T)1;
@@ -79,43 +83,44 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
         }
 
         // next pending evaluation time, kept in a register between iterations
-        T te_next = (tev && cursor < E) ? tev[cursor] : (T)0;
+        TT te_next = (tev && cursor < E) ? tev[cursor] : (TT)0;
 
         int n_steps = 0, n_acc = 0, status_last = 0, status_idle = 0;
         bool idle_pass = false;
         bool go = !bail && p.cap > 0;
         while (go) {
             // ---- stages (runge_kutta.py:255-263) ----
-            const T t0 = t;
+            const TT t0 = t;
+            const T h = (T)dt;  // (the step in the data type: runge_kutta.py:246)
             T y1[F], err[F];
 #pragma unroll
             for (int i = 1; i < 7; ++i) {
-                T tn = fma_((T)Tab::c[i], dt, t0);
+                TT tn = fma_((TT)Tab::c[i], dt, t0);
                 T yi[F];
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     T s = 0;
 #pragma unroll
                     for (int j = 0; j < i; ++j) s = fma_((T)Tab::a[i][j], k[j][f], s);
-                    yi[f] = fma_(dt, s, y[f]);
+                    yi[f] = fma_(h, s, y[f]);
                 }
-                rhs(tn, yi, k[i]);
+                rhs((T)tn, yi, k[i]);
                 if (i == 6) {
 #pragma unroll
                     for (int f = 0; f < F; ++f) y1[f] = yi[f];
                 }
             }
-            weighted_k<T, F, Tab, -1>(dt, k, err);
+            weighted_k<T, F, Tab, -1>(h, k, err);
 
             // ---- step size control (step_size_controllers.py:370-429, 715-774) ----
             const T ratio = error_ratio<T, F>(cp, y, y1, err);
             const bool accept = ratio < (T)1;
-            T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, prev_prev);
-            int status = limit_dt<T>(cp, ratio, dt_next);
+            TT dt_next = dt * (TT)dt_factor<T, CTRL>(cp, ratio, prev, prev_prev);
+            int status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
 
             const bool running = !idle_pass;
             const bool move = accept && running;
-            const T t_new = move ? (t0 + dt) : t0;
+            const TT t_new = move ? (t0 + dt) : t0;
             const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
             if (running) {
                 n_steps += 1;
@@ -132,14 +137,14 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
                 if (pend) {
                     for (int e = 0; e < E; ++e) {
                         if (!pend[e]) continue;
-                        T te_e = tev[e];
+                        TT te_e = tev[e];
                         if (dir > 0 ? t_new >= te_e : t_new <= te_e) {
                             if (!have_q) {
-                                quartic<T, F, METHOD>(dt, y, y1, k, q);
+                                quartic<T, F, METHOD>(h, y, y1, k, q);
                                 have_q = true;
                             }
                             T out[F];
-                            quartic_eval<T, F>(q, t0, dt, te_e, out);
+                            quartic_eval<T, F, TT>(q, t0, dt, te_e, out);
 #pragma unroll
                             for (int f = 0; f < F; ++f) ys[(long long)e * F + f] = out[f];
                             pend[e] = 0;
@@ -147,14 +152,14 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
                     }
                 } else {
                     while (cursor < E) {
-                        const T te_e = te_next;
+                        const TT te_e = te_next;
                         if (!(dir > 0 ? t_new >= te_e : t_new <= te_e)) break;
                         if (!have_q) {
-                            quartic<T, F, METHOD>(dt, y, y1, k, q);
+                            quartic<T, F, METHOD>(h, y, y1, k, q);
                             have_q = true;
                         }
                         T out[F];
-                        quartic_eval<T, F>(q, t0, dt, te_e, out);
+                        quartic_eval<T, F, TT>(q, t0, dt, te_e, out);
 #pragma unroll
                         for (int f = 0; f < F; ++f) ys[(long long)cursor * F + f] = out[f];
                         ++cursor;
@@ -164,9 +169,9 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
             } else if (last_own || idle_pass) {
                 // no evaluation points (adjoints.py:295-309): the interpolant of the loop's
                 // last iteration evaluated at t_end
-                quartic<T, F, METHOD>(dt, y, y1, k, q);
+                quartic<T, F, METHOD>(h, y, y1, k, q);
                 T out[F];
-                quartic_eval<T, F>(q, t0, dt, te, out);
+                quartic_eval<T, F, TT>(q, t0, dt, te, out);
                 T *dst = idle_pass ? (p.y_idle + b * F) : ys;
 #pragma unroll
                 for (int f = 0; f < F; ++f) dst[f] = out[f];
@@ -181,7 +186,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
                 }
             }
             t = t_new;
-            const T dtn = running_new ? dt_next : dt;
+            const TT dtn = running_new ? dt_next : dt;
             dt = tclamp(dtn, tlo - t, thi - t);
             if (CTRL == 1 && running_new && accept) {
                 prev_prev = prev;
@@ -249,43 +254,43 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T> 
     }
 }
 
-template <typename T, int METHOD, int CTRL, typename Term>
+template <typename T, int METHOD, int CTRL, typename Term, typename TT>
 static int launch(const tode_solve_args &a, const tode_controller &c, hipStream_t stream) {
-    SolveParams<T> p = make_params<T>(a, c);
+    SolveParams<T, TT> p = make_params<T, TT>(a, c);
     const long long blocks = (a.batch + TODE_BLOCK - 1) / TODE_BLOCK;
     hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
     if (blocks > 0) {
         timing_before(stream, "tode::solve_kernel");
-        hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
+        hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term, TT>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
         timing_after(stream);
     }
     return check_hip(hipGetLastError(), "tode_solve_builtin launch");
 }
 
-template <typename T, typename Term> static int dispatch_mc(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 0, 0, Term>(a, c, s);
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch<T, 0, 1, Term>(a, c, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 1, 0, Term>(a, c, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch<T, 1, 1, Term>(a, c, s);
+template <typename T, typename TT, typename Term> static int dispatch_mc(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 0, 0, Term, TT>(a, c, s);
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch<T, 0, 1, Term, TT>(a, c, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch<T, 1, 0, Term, TT>(a, c, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch<T, 1, 1, Term, TT>(a, c, s);
     return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
 }
 
-template <typename T> static int dispatch_term(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
+template <typename T, typename TT = T> static int dispatch_term(const tode_solve_args &a, const tode_controller &c, hipStream_t s) {
     switch (a.term) {
     case TODE_TERM_VAN_DER_POL:
         if (a.n_features != 2 || a.n_params != 1) return fail(TODE_E_INVALID, "Van der Pol needs F=2, P=1");
-        return dispatch_mc<T, VanDerPolTerm<T>>(a, c, s);
+        return dispatch_mc<T, TT, VanDerPolTerm<T>>(a, c, s);
     case TODE_TERM_LORENZ63:
         if (a.n_features != 3 || a.n_params != 1) return fail(TODE_E_INVALID, "Lorenz-63 needs F=3, P=1");
-        return dispatch_mc<T, Lorenz63Term<T>>(a, c, s);
+        return dispatch_mc<T, TT, Lorenz63Term<T>>(a, c, s);
     case TODE_TERM_LINEAR_DECAY:
         if (a.n_params != a.n_features) return fail(TODE_E_INVALID, "linear decay needs P == F");
         switch (a.n_features) {
-        case 1: return dispatch_mc<T, LinearDecayTerm<T, 1>>(a, c, s);
-        case 2: return dispatch_mc<T, LinearDecayTerm<T, 2>>(a, c, s);
-        case 3: return dispatch_mc<T, LinearDecayTerm<T, 3>>(a, c, s);
-        case 4: return dispatch_mc<T, LinearDecayTerm<T, 4>>(a, c, s);
-        case 8: return dispatch_mc<T, LinearDecayTerm<T, 8>>(a, c, s);
+        case 1: return dispatch_mc<T, TT, LinearDecayTerm<T, 1>>(a, c, s);
+        case 2: return dispatch_mc<T, TT, LinearDecayTerm<T, 2>>(a, c, s);
+        case 3: return dispatch_mc<T, TT, LinearDecayTerm<T, 3>>(a, c, s);
+        case 4: return dispatch_mc<T, TT, LinearDecayTerm<T, 4>>(a, c, s);
+        case 8: return dispatch_mc<T, TT, LinearDecayTerm<T, 8>>(a, c, s);
         default: return fail(TODE_E_UNSUPPORTED, "linear decay is built for F in {1,2,3,4,8}, got %d", a.n_features);
         }
     default:
@@ -295,12 +300,20 @@ template <typename T> static int dispatch_term(const tode_solve_args &a, const t
 
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);  // float64 times, float32 data
+int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 
 #if TODE_INSTANTIATE_F32
 int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float>(a, c, s); }
 #endif
 #if TODE_INSTANTIATE_F64
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double>(a, c, s); }
+#endif
+#if TODE_INSTANTIATE_T64_Y32
+int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float, double>(a, c, s); }
+#endif
+#if TODE_INSTANTIATE_T32_Y64
+int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double, float>(a, c, s); }
 #endif
 
 }  // namespace tode

@@ -69,8 +69,12 @@ template <typename T> struct Lorenz63Term {  // dx=sigma*(y-x); dy=(x*(rho-z))-y
     }
 };
 
-template <typename T> struct SolveParams {
-    const T *y0, *t_start, *t_end, *t_eval, *dt0, *params;
+// T: data type (state, parameters, tolerances, error ratio, step factor, output).  TT: time type (times, steps and
+// their limits; problems.py:44-56 lets the two differ).  Only the general kernel is built for TT != T.
+template <typename T, typename TT = T> struct SolveParams {
+    const T *y0, *params;
+    const TT *t_start, *t_end, *t_eval, *dt0;
+    TT dt_min, dt_max;  // the controller's step limits in the time type
     T *ys, *y_idle;
     uint8_t *pending;
     int32_t *n_steps, *n_accepted, *n_initialized, *status_last, *status_idle, *flags;
@@ -199,13 +203,15 @@ template <typename T> static CtrlParams<T> make_ctrl(const tode_controller &c, d
     return cp;
 }
 
-template <typename T> static SolveParams<T> make_params(const tode_solve_args &a, const tode_controller &c) {
-    SolveParams<T> p;
+template <typename T, typename TT = T> static SolveParams<T, TT> make_params(const tode_solve_args &a, const tode_controller &c) {
+    SolveParams<T, TT> p;
     p.y0 = (const T *)a.y0;
-    p.t_start = (const T *)a.t_start;
-    p.t_end = (const T *)a.t_end;
-    p.t_eval = a.n_eval > 0 ? (const T *)a.t_eval : nullptr;
-    p.dt0 = (const T *)a.dt0;
+    p.t_start = (const TT *)a.t_start;
+    p.t_end = (const TT *)a.t_end;
+    p.t_eval = a.n_eval > 0 ? (const TT *)a.t_eval : nullptr;
+    p.dt0 = (const TT *)a.dt0;
+    p.dt_min = (TT)c.dt_min;
+    p.dt_max = (TT)c.dt_max;
     p.params = (const T *)a.params;
     p.ys = (T *)a.ys;
     p.y_idle = (T *)a.y_idle;
@@ -283,7 +289,7 @@ __device__ __forceinline__ void lds_barrier() {
 // would write back the L2 once per workgroup).  The barrier makes every wavefront wait for its own
 // atomics to complete; the count is incremented after it, so whoever sees the final count issues
 // its exchanges after every update has been performed.
-template <typename T> __device__ __forceinline__ void publish_flags(const SolveParams<T> &p) {
+template <typename T, typename TT> __device__ __forceinline__ void publish_flags(const SolveParams<T, TT> &p) {
     if (p.host_flags == nullptr) return;
     __syncthreads();
     if (threadIdx.x != 0 || threadIdx.y != 0) return;

@@ -46,23 +46,6 @@ template <typename TT, typename T> struct StepParams {
     bool carry;          // the method keeps the last stage's derivative as the next step's first (Dopri5, Tsit5)
 };
 
-// dt_min / dt_max and the status of a step proposal, limits in the time type
-// (step_size_controllers.py:406-422, 751-767).
-template <typename TT, typename T>
-__device__ __forceinline__ int limit_step(const CtrlParams<T> &cp, TT dt_min, TT dt_max, T ratio, TT &dt_next) {
-    int status = finite_(ratio) ? 0 : 4;
-    if (cp.has_dt_min || cp.has_dt_max) {
-        const TT mag = abs_(dt_next);
-        TT c = mag;
-        if (cp.has_dt_min) c = tmax(c, dt_min);
-        if (cp.has_dt_max) c = tmin(c, dt_max);
-        const TT sg = (dt_next > 0) ? (TT)1 : ((dt_next < 0) ? (TT)-1 : dt_next);
-        dt_next = sg * c;
-        if (cp.has_dt_min && mag < dt_min) status = 2;
-    }
-    return status;
-}
-
 // Heun 2(1) (heun.py:10-13): c = (0, 1), a_10 = 1, b = (1/2, 1/2), low-order weights (1, 0), b_err = b - b_low in
 // float64 (runge_kutta.py:84-88).  Neither first-same-as-last nor solution-same-as-last-stage: the first stage is
 // evaluated anew in every step and y1 = y0 + sum_s (dt b_s) k_s.  Euler (euler.py:29-56) has one stage and no tableau.

@@ -37,21 +37,22 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> solve_builtin(const T
     TORCH_CHECK(y0.scalar_type() == at::kFloat || y0.scalar_type() == at::kDouble, "y0 must be float32 or float64");
     TORCH_CHECK(control.size() == 10, "control holds 10 values, got ", control.size());
     TORCH_CHECK(term_scalars.size() <= 4, "at most 4 term scalars");
-    const auto dtype = y0.scalar_type();
+    const auto dtype = y0.scalar_type(), time_dtype = t_start.scalar_type();  // (they may differ: reference problems.py:44-56)
+    TORCH_CHECK(time_dtype == at::kFloat || time_dtype == at::kDouble, "times must be float32 or float64");
     const int64_t B = y0.size(0), F = y0.size(1);
     const bool has_eval = t_eval.has_value() && t_eval->defined();
     const int64_t E = has_eval ? t_eval->size(1) : 0;
     for (const Tensor *t : {&t_start, &t_end}) {
-        TORCH_CHECK(t->dim() == 1 && t->size(0) == B && t->scalar_type() == dtype && t->device() == y0.device(),
-                    "t_start / t_end must be [batch] in y0's dtype on y0's device (the whole-solve kernels compute in one dtype)");
+        TORCH_CHECK(t->dim() == 1 && t->size(0) == B && t->scalar_type() == time_dtype && t->device() == y0.device(),
+                    "t_start / t_end must be [batch], of one dtype, on y0's device");
         TORCH_CHECK(B == 0 || t->stride(0) >= 1, "t_start / t_end must not be expanded views");
     }
     same_device(y0, t_eval, "t_eval"), same_device(y0, dt0, "dt0"), same_device(y0, params, "params"), same_device(y0, shared_params, "shared_params");
-    TORCH_CHECK(!has_eval || (t_eval->dim() == 2 && t_eval->size(0) == B && t_eval->scalar_type() == dtype), "t_eval must be [batch, points] in y0's dtype");
+    TORCH_CHECK(!has_eval || (t_eval->dim() == 2 && t_eval->size(0) == B && t_eval->scalar_type() == time_dtype), "t_eval must be [batch, points] in t_start's dtype");
 
     const Tensor y0_c = y0.contiguous();
     const OptTensor t_eval_c = has_eval ? OptTensor(t_eval->contiguous()) : OptTensor();
-    const OptTensor dt0_c = dt0.has_value() && dt0->defined() ? OptTensor(dt0->to(dtype).contiguous()) : OptTensor();
+    const OptTensor dt0_c = dt0.has_value() && dt0->defined() ? OptTensor(dt0->to(time_dtype).contiguous()) : OptTensor();
     const OptTensor params_c = params.has_value() && params->defined() ? OptTensor(params->to(dtype).contiguous()) : OptTensor();
     const OptTensor shared_c = shared_params.has_value() && shared_params->defined() ? OptTensor(shared_params->contiguous()) : OptTensor();
     TORCH_CHECK(!dt0_c.has_value() || (dt0_c->dim() == 1 && dt0_c->size(0) == B), "dt0 must be [batch]");
@@ -59,7 +60,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> solve_builtin(const T
     TORCH_CHECK(!shared_c.has_value() || shared_c->scalar_type() == dtype, "shared_params must be in y0's dtype");
 
     tode_solve_args a = {};
-    a.dtype = dtype == at::kFloat ? TODE_F32 : TODE_F64;
+    const int data_code = dtype == at::kFloat ? TODE_F32 : TODE_F64, time_code = time_dtype == at::kFloat ? TODE_F32 : TODE_F64;
+    a.dtype = data_code == time_code ? data_code : TODE_DTYPES(data_code, time_code);
     a.method = (int32_t)method, a.term = (int32_t)term;
     a.n_features = (int32_t)F, a.n_eval = (int32_t)E, a.n_params = params_c.has_value() ? (int32_t)params_c->size(1) : 0;
     a.batch = B, a.max_steps = max_steps, a.iteration_cap = -1;
