@@ -371,7 +371,7 @@ enum {
  *            tode_step_finish()
  *   Heun and Euler keep no derivative from one step to the next (heun.py, euler.py): every iteration starts with
  *   k[0] <- f(t, y) of the current state, then stage 1 (Heun only), then tode_step_finish; ystage[6] is scratch
- *   for the step's result.
+ *   for the step's result (rows of fewer than 64 features; longer rows need none).
  *   The caller reads `flags` (a synchronisation) or `host_flags` (none) whenever it
  *   likes; after TODE_STEP_FLAG_STOPPED is set, further stage/finish calls are no-ops.  tode_step_stats converts the
  *   counters.  k[0] must point at k0 from the first stage call on (begin
@@ -381,7 +381,7 @@ typedef struct tode_step_state {
     int32_t dtype;      /* TODE_F32 | TODE_F64: y0, y, k0, ratio_prev/pprev, ys, ystage, k */
     int32_t time_dtype; /* TODE_F32 | TODE_F64: t_start, t_end, t_eval, t, dt, tnode and a user dt0
                            (problems.py:44-56: time and data may differ) */
-    int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 | TODE_HEUN | TODE_EULER (the last two: F < 64) */
+    int32_t method;     /* TODE_DOPRI5 | TODE_TSIT5 | TODE_HEUN | TODE_EULER */
     int32_t n_features; /* F */
     int32_t n_eval;     /* E; 0: report y(t_end) only */
     int64_t batch;      /* B */

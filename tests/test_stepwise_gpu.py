@@ -391,15 +391,41 @@ def test_heun_and_euler_in_the_per_step_kernels_equal_the_operator_path(case, me
         assert (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()  # rejected steps are part of the case
 
 
-def test_long_rows_with_heun_and_euler_stay_on_the_operator_path():
-    f, y0, t_start, t_end, t_eval, _, _, ctrl, _ = mixed_case("wide", F32, F32)
-    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval)
-    for method in (to.Heun(), to.Euler()):
-        solver = to.AutoDiffAdjoint(method, to.IntegralController(1e-3, 1e-2))
-        assert not solver._stepwise_ok(problem, to.ODETerm(f))
-        with torch.no_grad():
-            sol = solver.solve(problem, to.ODETerm(f), dt0=torch.full((y0.shape[0],), 1e-2, device="cuda"))
-        assert (sol.status == 0).all()
+@pytest.mark.parametrize("time_dtype,data_dtype", [(F32, F32), (F64, F64), (F64, F32)], ids=["f32", "f64", "t64-y32"])
+@pytest.mark.parametrize("controller", ["integral", "pid", "fixed"])
+@pytest.mark.parametrize("method", ["heun", "euler"])
+@pytest.mark.parametrize("with_points", [True, False], ids=["t_eval", "end-only"])
+def test_long_rows_with_heun_and_euler_in_the_wavefront_kernels_equal_the_operator_path(with_points, method, controller, time_dtype, data_dtype):
+    """Rows of 100 values: one wavefront per sample in the finish kernel, which for these two methods also forms the
+    step's result (each lane for the features it needs, never through memory another lane has just written)."""
+    f, y0, t_start, t_end, t_eval, _, _, _, _ = mixed_case("wide", time_dtype, data_dtype)
+    B = y0.shape[0]
+    dt0 = None
+    if controller == "fixed" or method == "euler":
+        dt0 = ((t_end - t_start).double() / (40.0 + torch.arange(B, device="cuda", dtype=torch.float64) % 7 + 0.37)).to(time_dtype)
+    if controller == "fixed":
+        make = to.FixedStepController
+    else:
+        spec = dict(kind=controller, atol=1e-3, rtol=1e-2)
+        if controller == "pid":
+            spec.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+        make = lambda: make_controller(spec)
+    problem = to.InitialValueProblem(y0, t_start, t_end, t_eval if with_points else None)
+    fused_method, operator_method = {"heun": (to.Heun, OperatorHeun), "euler": (to.Euler, OperatorEuler)}[method]
+    with torch.no_grad():
+        fused_solver = to.AutoDiffAdjoint(fused_method(), make(), max_steps=300)
+        assert fused_solver._stepwise_ok(problem, to.ODETerm(f))
+        fused = fused_solver.solve(problem, to.ODETerm(f), dt0=dt0)
+        ops_solver = to.AutoDiffAdjoint(operator_method(), make(), max_steps=300)
+        assert not ops_solver._stepwise_ok(problem, to.ODETerm(f))
+        ops = ops_solver.solve(problem, to.ODETerm(f), dt0=dt0)
+    for key in ("n_steps", "n_accepted", "n_initialized", "n_f_evals"):
+        assert torch.equal(fused.stats[key], ops.stats[key]), key
+    assert torch.equal(fused.status, ops.status) and (fused.status == 0).all()
+    assert fused.ys.shape == ops.ys.shape and bool((fused.ys == ops.ys).all()), (fused.ys - ops.ys).abs().max().item()
+    assert int(fused.stats["n_steps"].max()) >= 10
+    if method == "heun" and controller == "integral":
+        assert (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()  # rejected steps are part of the case
 
 
 @pytest.mark.parametrize("method", ["heun", "euler"])

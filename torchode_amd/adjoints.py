@@ -255,10 +255,7 @@ class AutoDiffAdjoint(nn.Module):
         )
 
     def _stepwise_ok(self, problem: InitialValueProblem, term: ODETerm) -> bool:
-        if self._fused_ok(problem, term):
-            return True
-        # Heun and Euler are built into the thread-per-sample kernels (rows of fewer than 64 features)
-        return problem.n_features < 64 and self._library_setup(problem, term, (Heun, Euler))
+        return self._library_setup(problem, term, (Dopri5, Tsit5, Heun, Euler))
 
     # ------------------------------------------------------------------ #
     def _solve_protocol(self, problem: InitialValueProblem, term: Optional[ODETerm], term_: ODETerm, dt0, args, record=None) -> Solution:

@@ -427,7 +427,7 @@ __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T
     }
     for (int f = lane; f < F; f += 64) {
         p.y[b * F + f] = y0[f];
-        p.k0[b * F + f] = f0[f];
+        if (p.carry) p.k0[b * F + f] = f0[f];
     }
     bool ordered = true;
     int cursor = 0;
@@ -460,6 +460,8 @@ __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T
 
 template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<TT, T> p) {
     using Tab = typename TabOf<METHOD>::type;
+    constexpr int NS = stages_of(METHOD);
+    constexpr bool ESTIMATE = METHOD != TODE_EULER;
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= p.batch) return;
@@ -470,13 +472,34 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     const T h = (T)dt;
     const TT ts = p.t_start[b], te = p.t_end[b];
     const bool fwd = te > ts;
-    const T *y = p.y + b * F, *y1 = p.ystage[6] + b * F;
+    const T *y = p.y + b * F;
+    // The step's result: Dopri5 and Tsit5 hand it over as the input of their last stage; for Heun and Euler it is
+    // formed here (heun.py, euler.py; runge_kutta.py:265-269), by whichever lane needs it and as often as it does,
+    // so that no lane reads what another lane of the wavefront has just written.
+    auto y1 = [&](int f) -> T {
+        if (METHOD == TODE_EULER) return fma_(h, p.k[0][b * F + f], y[f]);
+        if (METHOD == TODE_HEUN) {
+            T sum = 0;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const T ps = h * (T)HeunTab::b[s], ks = p.k[s][b * F + f];
+                if (fused)
+                    sum = fma_(ps, ks, sum);
+                else {
+                    const T pk = ps * ks;
+                    sum = sum + pk;
+                }
+            }
+            return y[f] + sum;
+        }
+        return p.ystage[6][b * F + f];
+    };
 
     // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
-    const T norm = CTRL == 2 ? (T)0 : wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
+    const T norm = (CTRL == 2 || !ESTIMATE) ? (T)0 : wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
         T err = 0;
 #pragma unroll
-        for (int s = 0; s < 7; ++s) {
+        for (int s = 0; s < NS; ++s) {
             const T ps = h * (T)Tab::b_err[s], ks = p.k[s][b * F + f];
             if (fused)
                 err = fma_(ps, ks, err);
@@ -485,11 +508,11 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
                 err = err + pk;
             }
         }
-        const T m = tmax(abs_(y[f]), abs_(y1[f]));
+        const T m = tmax(abs_(y[f]), abs_(y1(f)));
         return abs_(err) / fma_(cp.rtol, m, cp.atol);
     });
     const T ratio = tmax(norm, (T)1e-38);
-    const bool accept = CTRL == 2 || ratio < (T)1;
+    const bool accept = CTRL == 2 || !ESTIMATE || ratio < (T)1;
 
     // ---- step size proposal ----
     const T prev = p.ratio_prev[b], pprev = p.ratio_pprev[b];
@@ -497,6 +520,8 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     int status = 0;
     if (CTRL == 2) {
         dt_next = p.fixed_dt[b];
+    } else if (!ESTIMATE) {
+        dt_next = dt;  // (step_size_controllers.py:382-391, 727-736: accepted, step size unchanged, no status)
     } else {
         dt_next = dt * (TT)dt_factor<T, (CTRL == 2 ? 0 : CTRL)>(cp, ratio, prev, pprev);
         status = limit_step<TT, T>(cp, p.dt_min, p.dt_max, ratio, dt_next);
@@ -519,7 +544,8 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         const bool mono = p.monotone[b] != 0;
         const int cursor = p.cursor[b];
         for (int f = lane; f < F; f += 64) {
-            T q[5][1];
+            T q[5][1], ks[7] = {};
+            T y1f = 0;
             bool built = false;
             for (int e = mono ? cursor : 0; e < E; ++e) {
                 if (!pend[e]) continue;
@@ -530,13 +556,16 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
                     continue;
                 }
                 if (!built) {
-                    T ks[7];
 #pragma unroll
-                    for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-                    quartic_elem<T, METHOD>(h, y[f], y1[f], ks, fused, q);
+                    for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
+                    y1f = y1(f);
+                    if (NS == 7) quartic_elem<T, (METHOD == 1 ? 1 : 0)>(h, y[f], y1f, ks, fused, q);
                     built = true;
                 }
-                ys[(long long)e * F + f] = quartic_at<T>(q, (T)unit_time<TT>(te_e, t0, t0 + dt));
+                if (NS == 7)
+                    ys[(long long)e * F + f] = quartic_at<T>(q, (T)unit_time<TT>(te_e, t0, t0 + dt));
+                else  // (Hermite cubic / linear interpolant: cheap enough to form per point)
+                    ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1f, ks, fused, te_e);
             }
         }
         // (every lane has finished reading the pending marks: the wavefront runs in lock step)
@@ -554,18 +583,19 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         if (lane == 0) p.cursor[b] = first_pending;
     } else {
         for (int f = lane; f < F; f += 64) {
-            T ks[7];
+            T ks[7] = {};
 #pragma unroll
-            for (int s = 0; s < 7; ++s) ks[s] = p.k[s][b * F + f];
-            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+            for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
+            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1(f), ks, fused, te);
         }
     }
 
     // ---- state update ----
     if (move) {
         for (int f = lane; f < F; f += 64) {
-            p.y[b * F + f] = y1[f];
-            p.k0[b * F + f] = p.k[6][b * F + f];
+            const T moved = y1(f);  // (read before the write: for Heun and Euler y1 is formed from y)
+            p.y[b * F + f] = moved;
+            if (NS == 7) p.k0[b * F + f] = p.k[6][b * F + f];  // (first same as last: Dopri5 and Tsit5 only)
         }
     }
     if (lane == 0) {
@@ -576,7 +606,7 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         const TT tlo = tmin(ts, te), thi = tmax(te, ts);
         const TT dtn = running_new ? dt_next : dt;
         p.dt[b] = tclamp(dtn, tlo - t_new, thi - t_new);
-        if (CTRL == 1 && running_new && accept) {
+        if (CTRL == 1 && ESTIMATE && running_new && accept) {
             p.ratio_pprev[b] = prev;
             p.ratio_prev[b] = ratio;
         }
@@ -664,8 +694,6 @@ static int check_state(const tode_step_state *s, const tode_controller *c) {
     if (s->dtype != TODE_F32 && s->dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown dtype %d", s->dtype);
     if (s->time_dtype != TODE_F32 && s->time_dtype != TODE_F64) return fail(TODE_E_INVALID, "unknown time dtype %d", s->time_dtype);
     if (s->method < TODE_DOPRI5 || s->method > TODE_EULER) return fail(TODE_E_INVALID, "unknown method %d", s->method);
-    if (s->method > TODE_TSIT5 && s->n_features >= 64)
-        return fail(TODE_E_UNSUPPORTED, "Heun and Euler are built into the per-step kernels for rows of fewer than 64 features (got %d)", s->n_features);
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID && c->kind != TODE_CTRL_FIXED)
         return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
     if (c->kind == TODE_CTRL_FIXED && s->batch > 0 && !s->fixed_dt) return fail(TODE_E_INVALID, "the fixed-step controller needs fixed_dt");
@@ -807,14 +835,16 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
     if (blocks > 0) {
         for (int j = 0; j < stages_of(s->method); ++j)
             if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
-        if (!s->ystage[6]) return fail(TODE_E_INVALID, "ystage[6] is null");
+        if (!s->ystage[6] && !(wide && s->method > TODE_TSIT5)) return fail(TODE_E_INVALID, "ystage[6] is null");
         TODE_DISPATCH_T(s, {
             auto p = make_step_params<TT, T>(*s, *c);
             const bool tsit5 = s->method == TODE_TSIT5;
             if (s->method == TODE_HEUN) {
-                TODE_FINISH_CTRL(finish_kernel, 2);
+                if (wide) TODE_FINISH_CTRL(finish_wave_kernel, 2);
+                else TODE_FINISH_CTRL(finish_kernel, 2);
             } else if (s->method == TODE_EULER) {
-                TODE_FINISH_CTRL(finish_kernel, 3);
+                if (wide) TODE_FINISH_CTRL(finish_wave_kernel, 3);
+                else TODE_FINISH_CTRL(finish_kernel, 3);
             } else if (wide) {
                 if (tsit5) TODE_FINISH_CTRL(finish_wave_kernel, 1);
                 else TODE_FINISH_CTRL(finish_wave_kernel, 0);
