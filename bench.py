@@ -67,8 +67,10 @@ OTHER_CONFIGS = [
 START = time.perf_counter()
 
 
-def measure(args, name, dtype_flag, mlp_inputs, steps, warmup):
+def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_iterations=-1):
     """One configuration on the GPU: wall time of `steps` solves, kernel time by HIP events, roofline."""
+    path = args.path if path is None else path
+    graph_iterations = args.graph_iterations if graph_iterations == -1 else graph_iterations
     import torch
 
     import torchode_amd as to
@@ -84,9 +86,9 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup):
     spec = dict(w.controller)
     kind = spec.pop("kind")
     ctrl = to.PIDController(**spec) if kind == "pid" else to.IntegralController(**spec)
-    solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl, graph_iterations=args.graph_iterations)
+    solver = to.AutoDiffAdjoint(to.Tsit5() if w.method == "tsit5" else to.Dopri5(), ctrl, graph_iterations=graph_iterations)
     problem = to.InitialValueProblem(w.y0, t_eval=w.t_eval)
-    term = to.ODETerm(w.f if args.path == "auto" else (lambda t, y, f=w.f: f(t, y)))
+    term = to.ODETerm(w.f if path == "auto" else (lambda t, y, f=w.f: f(t, y)))
 
     with torch.no_grad():  # a forward solve: nothing here asks for gradients
         for _ in range(warmup):
@@ -114,10 +116,10 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup):
         except RuntimeError:
             # no whole-solve kernel for this workload: the solve is a sequence of per-call kernels
             # around the torch right-hand side, and the figure below is over the whole solve
-            per_step = args.path == "per-step"
+            per_step = path == "per-step"
             kernel_name = ("per-step kernels" if per_step else "protocol path (one kernel per protocol call)") + " + torch right-hand side"
-            if per_step and args.graph_iterations:
-                kernel_name += f", {args.graph_iterations} iterations per HIP graph replay"
+            if per_step and graph_iterations:
+                kernel_name += f", {graph_iterations} iterations per HIP graph replay"
             kernel_s = wall
         _lib.set_kernel_timing(False)
     achieved = algo_bytes / kernel_s / 1e9
@@ -134,7 +136,7 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup):
         "bytes_dense_per_sample": w.bytes_dense,
         "kernel_ms": kernel_s * 1e3,
     }
-    if args.path == "per-step":
+    if path == "per-step":
         # with an external f the stages go through HBM: per sample-step the stage kernels read 27 and
         # write 6 rows, f reads and writes a row six times, the finishing kernel reads 9 and writes 2
         sd = w.y0.element_size()
@@ -262,6 +264,12 @@ def main():
                 entry["cpu_baseline_compiled"] = compiled_baseline(args, name, dtype_flag, mlp_inputs, entry["cpu_baseline"])
     if everything:
         out["configs"] = others
+        # the headline configuration with its right-hand side hidden behind a plain callable, as any user-defined f is:
+        # the per-step kernels around torch's evaluation of f, eager and with iterations replayed from a HIP graph
+        out["user_defined_f"] = [
+            measure(args, "vdp", "f32", "float32", 5, 2, path="per-step", graph_iterations=None),
+            measure(args, "vdp", "f32", "float32", 5, 2, path="per-step", graph_iterations=2),
+        ]
     out["bench_seconds"] = time.perf_counter() - START
     print(json.dumps(out))
 
