@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 18
+#define TODE_ABI_VERSION 19
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -124,6 +124,26 @@ typedef struct tode_controller {
  * caller runs the solve again with iteration_cap = L, then passes L to
  * tode_finalize_stats.
  */
+/*
+ * Optional record of the loop state, written by tode_solve_builtin (the general kernel) when
+ * tode_solve_args.record points to one: entry i holds what the reference's loop variables hold before iteration i
+ * (adjoints.py:135-260: t, dt, y, the first-same-as-last derivative, the PID controller's two previous error
+ * ratios, `running`, `n_accepted`), entry n_steps[b] the sample's final state, and the entries after it that final
+ * state again with running = 0 -- a finished sample keeps its state while the batch goes on.  It is what a reverse
+ * sweep over the iterations starts from (tode_step_finish_backward / tode_step_stage_backward), the counterpart of the
+ * operation graph that torch.autograd keeps for the reference's loop.  All arrays are device memory with
+ * `capacity` entries of the batch each, entry-major: t, dt [capacity, B] in the time type; y, k0 [capacity, B, F] and
+ * prev, pprev [capacity, B] in the data type; running, n_accepted [capacity, B] int32.  capacity must be at least
+ * 1 + the iterations the solve takes (args->iteration_cap + 1 when a cap is set, which is how a caller that has
+ * solved the problem once sizes it); a sample whose steps do not fit stops recording and raises
+ * TODE_FLAG_NEEDS_GENERAL in the flag block.
+ */
+typedef struct tode_solve_record {
+    int64_t capacity;
+    void *t, *dt, *y, *k0, *prev, *pprev;
+    int32_t *running, *n_accepted;
+} tode_solve_record;
+
 typedef struct tode_solve_args {
     int32_t dtype;  /* TODE_F32 | TODE_F64 for data and time alike; TODE_DTYPES(data, time) where they differ:
                        tode_solve_builtin and tode_solve_builtin_auto take it for the three small systems (the
@@ -158,6 +178,8 @@ typedef struct tode_solve_args {
     int32_t *status_last;      /* out [B] status at the sample's last own iteration */
     int32_t *status_idle;      /* out [B] status the sample reports in later iterations */
     int32_t *flags;            /* out [TODE_FLAG_WORDS] */
+    const tode_solve_record *record; /* NULL, or where tode_solve_builtin keeps the loop state of every iteration
+                                        (HOST pointer to the struct; every other entry point ignores it) */
 } tode_solve_args;
 
 /* ABI version of the loaded library (== TODE_ABI_VERSION of the header it was built from). */

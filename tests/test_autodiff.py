@@ -576,3 +576,91 @@ def test_what_is_not_differentiated_says_so():
         to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
     with torch.no_grad():  # no graph asked for: any configuration solves
         to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
+
+
+# ---------------------------------------------------------------------------------------------
+# A differentiable solve with a built-in term: the forward pass stays in the whole-solve kernels, and the general
+# kernel writes the record of the loop state that the reverse sweep starts from.  The per-step kernels' record of the
+# same solve (the term behind a plain callable) is the checker: every entry, every bit.
+# ---------------------------------------------------------------------------------------------
+
+
+@gpu
+@pytest.mark.parametrize("case", ["vdp-f32", "vdp-f64", "lorenz-f32", "linear-decay-f64", "vdp-t64-y32", "vdp-t32-y64", "max-steps", "non-monotone", "dt0",
+                                  "end-only", "backwards", "limits", "non-finite"])  # fmt: skip
+def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
+    from torchode_amd.autodiff import LoopRecord
+
+    name = "lorenz" if case.startswith("lorenz") else ("linear_decay" if case.startswith("linear") else "vdp")
+    data_dtype = torch.float64 if case in ("vdp-f64", "linear-decay-f64", "vdp-t32-y64") else torch.float32
+    time_dtype = {"vdp-t64-y32": torch.float64, "vdp-t32-y64": torch.float32}.get(case, data_dtype)
+    w = to.workloads.make(name, batch=150, dtype=torch.float64)
+    params = w.f.builtin_params().to(data_dtype)
+    f = type(w.f)(params[:, 0] if params.shape[1] == 1 and name != "linear_decay" else params).cuda()
+    y0, t_eval = w.y0.clone(), w.t_eval.clone()
+    t_start = t_end = dt0 = None
+    kw, ctrl = {}, dict(w.controller)
+    if case == "max-steps":
+        kw["max_steps"] = 25
+    if case == "non-monotone":
+        t_eval[::5, 3], t_eval[::5, 7] = t_eval[::5, 7].clone(), t_eval[::5, 3].clone()
+    if case == "dt0":
+        dt0 = torch.full((150,), 1e-3, dtype=time_dtype, device="cuda")
+    if case == "end-only":
+        t_start, t_end, t_eval = t_eval[:, 0].clone(), t_eval[:, -1].clone(), None
+    if case == "backwards":
+        t_eval[::2] = t_eval[::2].flip(1)
+        t_eval[::2] = t_eval[::2, :1] - 0.01 * (t_eval[::2, :1] - t_eval[::2])
+    if case == "limits":
+        ctrl.update(dt_min=2e-2, dt_max=0.25)
+    if case == "non-finite":
+        y0[7] = float("inf")
+    mv = lambda x, dt: None if x is None else x.to(dt).cuda()
+    problem = to.InitialValueProblem(mv(y0, data_dtype), mv(t_start, time_dtype), mv(t_end, time_dtype), mv(t_eval, time_dtype))
+    kind = ctrl.pop("kind")
+    controller = to.PIDController(**ctrl) if kind == "pid" else to.IntegralController(**ctrl)
+    solver = to.AutoDiffAdjoint({"tsit5": to.Tsit5, "dopri5": to.Dopri5}[w.method](), controller, **kw)
+    whole, steps = LoopRecord(), LoopRecord()
+    with torch.no_grad():
+        sol_whole = solver._solve_persistent(problem, to.ODETerm(f), dt0, record=whole)
+        sol_steps = solver._solve_stepwise(problem, to.ODETerm(lambda t, y: f(t, y)), dt0, None, record=steps)
+    assert sol_whole is not None and whole.iterations == steps.iterations
+    assert whole.iterations > 5 or case == "non-finite"  # (an infinite start value stops the whole batch after its first iteration)
+    assert torch.equal(sol_whole.stats["n_steps"], sol_steps.stats["n_steps"]) and torch.equal(sol_whole.status, sol_steps.status)
+    a, b = whole.trimmed(whole.iterations), steps.trimmed(steps.iterations)
+    assert len(a) == len(b) == whole.iterations + 1
+    for i, (sa, sb) in enumerate(zip(a, b)):
+        for key in LoopRecord.FIELDS:
+            x, y = sa[key], sb[key]
+            assert x.dtype == y.dtype and x.shape == y.shape, (i, key)
+            assert bool(((x == y) | ((x != x) & (y != y))).all()), (i, key, (x.double() - y.double()).abs().nan_to_num().max().item())
+    if case == "max-steps":
+        assert (sol_whole.status == 3).any()
+    if case == "non-finite":
+        assert (sol_whole.status != 0).any()
+
+
+@gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float64, 1e-9), (torch.float32, 5e-3)], ids=["f64", "f32"])
+def test_gradients_of_a_built_in_term_with_the_forward_pass_in_the_whole_solve_kernel(dtype, tol):
+    import torchode_amd.autodiff as autodiff
+
+    w = to.workloads.make("vdp", batch=64, dtype=dtype)
+    mu = w.f.builtin_params()[:, 0].cuda().requires_grad_()
+    y0 = w.y0.cuda().requires_grad_()
+    t_eval = w.t_eval.cuda()
+    weights = torch.linspace(0.5, 1.5, t_eval.shape[1] * 2, dtype=dtype, device="cuda").reshape(1, -1, 2)
+    results = {}
+    for in_kernel in (True, False):
+        solver = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(1e-6, 1e-4, 0.2, 0.5, 0.0))
+        solver.record_in_whole_solve_kernel = in_kernel
+        sol = solver.solve(to.InitialValueProblem(y0, t_eval=t_eval), to.ODETerm(to.VanDerPol(mu)))
+        assert sol.ys.requires_grad
+        g_y0, g_mu = torch.autograd.grad((sol.ys * weights).sum(), (y0, mu))
+        results[in_kernel] = (sol.ys.detach(), sol.stats["n_steps"], g_y0, g_mu)
+    assert autodiff.LAST_SWEEP == "kernels"
+    assert torch.equal(results[True][0], results[False][0]) and torch.equal(results[True][1], results[False][1])
+    # (same record, same sweep: the gradients agree to the last bits the atomics-free kernels and autograd's own
+    # accumulation order leave)
+    torch.testing.assert_close(results[True][2], results[False][2], rtol=tol, atol=tol)
+    torch.testing.assert_close(results[True][3], results[False][3], rtol=tol, atol=tol)

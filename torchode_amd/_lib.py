@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -136,7 +136,14 @@ class SolveArgs(C.Structure):
         ("status_last", C.c_void_p),
         ("status_idle", C.c_void_p),
         ("flags", C.c_void_p),
+        ("record", C.c_void_p),
     ]
+
+
+class SolveRecord(C.Structure):
+    """struct tode_solve_record"""
+
+    _fields_ = [("capacity", C.c_int64)] + [(n, C.c_void_p) for n in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")]
 
 
 STEP_FLAG_STOPPED, STEP_FLAG_ITERATIONS, STEP_FLAG_ANY_RUNNING, STEP_FLAG_ANY_FAILURE, STEP_FLAG_WORDS = 0, 1, 2, 3, 4

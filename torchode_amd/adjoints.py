@@ -545,7 +545,9 @@ class AutoDiffAdjoint(nn.Module):
         torch.cuda.current_stream(like.device).wait_stream(side)
         return graph
 
-    def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0) -> Solution:
+    def _solve_persistent(self, problem: InitialValueProblem, term: ODETerm, dt0, record=None) -> Solution:
+        """``record``: a ``LoopRecord`` to fill with the loop state of every iteration (the solve then runs the general
+        kernel once more, limited to the iterations the first pass took, with a record of that many entries)."""
         lib = _lib.load()
         f: BuiltinTerm = _sub(term, "f")
         method_id, controller = _sub(self, "step_method").method_id, _sub(self, "step_size_controller")
@@ -624,6 +626,28 @@ class AutoDiffAdjoint(nn.Module):
         if term.with_stats:
             stats["n_f_evals"] = _f_evals((2 if dt0 is None else 1) + 6 * iterations.value, B)
         stats["n_steps"], stats["n_accepted"], stats["n_initialized"], status = out.unbind(0)
+        if record is not None:
+            # The same solve through the general kernel again, stopped where the first pass stopped, writing the
+            # state before every iteration: entry i of every array is what the per-step kernels' loop holds there.
+            L, n = iterations.value, iterations.value + 1
+            new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+            fields = dict(t=new(n, B, dt=ttype), dt=new(n, B, dt=ttype), y=new(n, B, F), k0=new(n, B, F), prev=new(n, B), pprev=new(n, B),
+                          running=new(n, B, dt=torch.int32), n_accepted=new(n, B, dt=torch.int32))  # fmt: skip
+            rec = _lib.SolveRecord(n, *(fields[k].data_ptr() for k in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")))
+            again = _lib.SolveArgs.from_buffer_copy(a)
+            scratch_ys, y_idle = new(B, max(E, 1), F), new(B, F)
+            counters, flags = new(5, B, dt=torch.int32), new(_lib.FLAG_WORDS, dt=torch.int32)
+            pending = new(B, max(E, 1), dt=torch.uint8)
+            again.ys, again.y_idle, again.pending, again.flags = scratch_ys.data_ptr(), y_idle.data_ptr(), pending.data_ptr(), flags.data_ptr()
+            again.n_steps, again.n_accepted, again.n_initialized, again.status_last, again.status_idle = (counters[i].data_ptr() for i in range(5))
+            again.iteration_cap = L
+            again.record = _lib.C.addressof(rec)
+            _lib.check(lib.tode_solve_builtin(_lib.C.byref(again), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
+            if flags.tolist()[_lib.FLAG_NEEDS_GENERAL]:
+                raise RuntimeError("the record of the loop state was too short for the solve it was sized from")
+            order = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
+            record.states = [tuple(fields[k][i] for k in order) for i in range(n)]
+            record.iterations = L
         return Solution(ts=ts, ys=ys, stats=stats, status=status)
 
     def __repr__(self):

@@ -527,7 +527,13 @@ class SolveThroughLoop(torch.autograd.Function):
         detached = lambda x: None if x is None else x.detach()
         plain = InitialValueProblem(y0.detach(), detached(problem.t_start), detached(problem.t_end), detached(problem.t_eval))
         with torch.no_grad():
-            if adjoint._fused_ok(plain, term):
+            solution = None
+            if getattr(adjoint, "record_in_whole_solve_kernel", True) and adjoint._persistent_ok(plain, term):
+                # a built-in term: the forward pass stays in the whole-solve kernels, and the general one writes the record
+                solution = adjoint._solve_persistent(plain, term, detached(dt0), record=record)
+            if solution is not None:
+                pass
+            elif adjoint._fused_ok(plain, term):
                 solution = adjoint._solve_stepwise(plain, term, detached(dt0), args, record=record)
             else:  # Heun, Euler: the operator path keeps the record
                 solution = adjoint._solve_protocol(plain, term, term, detached(dt0), args, record=record)

@@ -252,6 +252,10 @@ int tode_solve_builtin(const tode_solve_args *a, const tode_controller *c, void 
     hipStream_t s = (hipStream_t)stream;
     if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
     const int data = data_type(a->dtype), time = time_type(a->dtype);
+    if (a->record) {  // the same kernel, keeping the loop state of every iteration
+        if (data == time) return data == TODE_F32 ? solve_builtin_f32_record(*a, *c, s) : solve_builtin_f64_record(*a, *c, s);
+        return data == TODE_F32 ? solve_builtin_t64_y32_record(*a, *c, s) : solve_builtin_t32_y64_record(*a, *c, s);
+    }
     if (data == time) return data == TODE_F32 ? solve_builtin_f32(*a, *c, s) : solve_builtin_f64(*a, *c, s);
     return data == TODE_F32 ? solve_builtin_t64_y32(*a, *c, s) : solve_builtin_t32_y64(*a, *c, s);
 }
@@ -484,6 +488,7 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
     tode_solve_args b = *a;
     b.iteration_cap = -1;
     b.pending = nullptr;
+    b.record = nullptr;
     b.y_idle = E == 0 ? ws + w.y_idle : nullptr;
 
     // The common case first: one kernel that writes what the reference returns.  It reports through its flag words when the

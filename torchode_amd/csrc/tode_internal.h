@@ -26,6 +26,9 @@
 #ifndef TODE_INSTANTIATE_T32_Y64
 #define TODE_INSTANTIATE_T32_Y64 0
 #endif
+#ifndef TODE_INSTANTIATE_RECORD
+#define TODE_INSTANTIATE_RECORD 0
+#endif
 
 namespace tode {
 // The two halves of a dtype argument: a plain TODE_F32 / TODE_F64 means both, TODE_DTYPES(data, time) names each.
@@ -62,6 +65,10 @@ int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStr
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f32_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f64_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t64_y32_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t32_y64_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 int solve_pair_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
 int solve_pair_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);

@@ -15,7 +15,8 @@ namespace tode {
 // T: data type, TT: time type (the same in the common case; where they differ the conversions stand where the
 // reference's loop of torch operations has them: the step in the data type for stage sums and interpolants, the step
 // factor in the time type for the next step, the position of an evaluation point in its step formed in the time type).
-template <typename T, int METHOD, int CTRL, typename Term, typename TT = T>
+// RECORD: the loop state before every iteration goes to p.rec_* (tode_solve_record), for a reverse sweep.
+template <typename T, int METHOD, int CTRL, typename Term, typename TT = T, bool RECORD = false>
 __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, TT> p) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
@@ -25,7 +26,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
     const CtrlParams<T> &cp = p.cp;
     const int E = p.n_eval;
 
-    int my_fail = INT_MAX, my_steps = 0, my_nonmono = 0;
+    int my_fail = INT_MAX, my_steps = 0, my_nonmono = 0, my_overflow = 0;
 
     if (live) {
         Term rhs;
@@ -88,7 +89,22 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
         int n_steps = 0, n_acc = 0, status_last = 0, status_idle = 0;
         bool idle_pass = false;
         bool go = !bail && p.cap > 0;
+        bool still_running = true;  // (RECORD) the sample's `running` after its last own iteration
+        // (RECORD) entry `at` of the record: the state as it is now
+        auto keep = [&](long long at, bool running) {
+            if (at >= p.rec_capacity) {
+                my_overflow = 1;
+                return;
+            }
+            const long long i = at * p.batch + b;
+            p.rec_t[i] = t, p.rec_dt[i] = dt;
+#pragma unroll
+            for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k[0][f];
+            p.rec_prev[i] = prev, p.rec_pprev[i] = prev_prev;
+            p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
+        };
         while (go) {
+            if (RECORD && !idle_pass) keep(n_steps, true);
             // ---- stages (runge_kutta.py:255-263) ----
             const TT t0 = t;
             const T h = (T)dt;  // (the step in the data type: runge_kutta.py:246)
@@ -122,6 +138,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
             const bool move = accept && running;
             const TT t_new = move ? (t0 + dt) : t0;
             const bool running_new = dir > 0 ? (t_new < te) : (t_new > te);
+            if (RECORD && running) still_running = running_new;
             if (running) {
                 n_steps += 1;
                 n_acc += move ? 1 : 0;
@@ -224,6 +241,14 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
             if (n_steps >= p.cap) break;
         }
 
+        if (RECORD) {
+            // the state the sample is left in, and the same for every later iteration of the batch (a sample that never
+            // started -- rows that need the pending mask and have none -- records nothing: the solve is repeated)
+            if (!bail) {
+                keep(n_steps, still_running);
+                for (long long at = n_steps + 1; at < p.rec_capacity; ++at) keep(at, false);
+            }
+        }
         int n_init = 1;
         if (tev) {
             if (pend) {
@@ -246,22 +271,30 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
         my_fail = min(my_fail, __shfl_xor(my_fail, off));
         my_steps = max(my_steps, __shfl_xor(my_steps, off));
         my_nonmono = max(my_nonmono, __shfl_xor(my_nonmono, off));
+        my_overflow = max(my_overflow, __shfl_xor(my_overflow, off));
     }
     if ((threadIdx.x & 63) == 0) {
         if (my_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], my_steps);
         if (my_fail != INT_MAX) atomicMin(&p.flags[TODE_FLAG_FIRST_FAILURE], my_fail);
         if (my_nonmono) atomicMax(&p.flags[TODE_FLAG_NON_MONOTONE], 1);
+        if (my_overflow) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);  // (the record was too short)
     }
 }
 
 template <typename T, int METHOD, int CTRL, typename Term, typename TT>
 static int launch(const tode_solve_args &a, const tode_controller &c, hipStream_t stream) {
     SolveParams<T, TT> p = make_params<T, TT>(a, c);
+    if ((TODE_INSTANTIATE_RECORD != 0) != (a.record != nullptr)) return fail(TODE_E_INVALID, "internal: record variant mismatch");
+    if (a.record) {
+        const tode_solve_record &r = *a.record;
+        if (r.capacity < 1 || (a.batch > 0 && (!r.t || !r.dt || !r.y || !r.k0 || !r.prev || !r.pprev || !r.running || !r.n_accepted)))
+            return fail(TODE_E_INVALID, "tode_solve_record: capacity %lld, or a null array", (long long)r.capacity);
+    }
     const long long blocks = (a.batch + TODE_BLOCK - 1) / TODE_BLOCK;
     hipLaunchKernelGGL(init_flags_kernel, dim3(1), dim3(64), 0, stream, a.flags);
     if (blocks > 0) {
         timing_before(stream, "tode::solve_kernel");
-        hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term, TT>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
+        hipLaunchKernelGGL((solve_kernel<T, METHOD, CTRL, Term, TT, TODE_INSTANTIATE_RECORD != 0>), dim3((unsigned)blocks), dim3(TODE_BLOCK), 0, stream, p);
         timing_after(stream);
     }
     return check_hip(hipGetLastError(), "tode_solve_builtin launch");
@@ -302,18 +335,28 @@ int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStr
 int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s);  // float64 times, float32 data
 int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f32_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_f64_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t64_y32_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
+int solve_builtin_t32_y64_record(const tode_solve_args &a, const tode_controller &c, hipStream_t s);
 
+// (each translation unit instantiates one pair of types, with or without the record: TODE_INSTANTIATE_RECORD)
+#if TODE_INSTANTIATE_RECORD
+#define TODE_SOLVE_ENTRY(name) name##_record
+#else
+#define TODE_SOLVE_ENTRY(name) name
+#endif
 #if TODE_INSTANTIATE_F32
-int solve_builtin_f32(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float>(a, c, s); }
+int TODE_SOLVE_ENTRY(solve_builtin_f32)(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float>(a, c, s); }
 #endif
 #if TODE_INSTANTIATE_F64
-int solve_builtin_f64(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double>(a, c, s); }
+int TODE_SOLVE_ENTRY(solve_builtin_f64)(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double>(a, c, s); }
 #endif
 #if TODE_INSTANTIATE_T64_Y32
-int solve_builtin_t64_y32(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float, double>(a, c, s); }
+int TODE_SOLVE_ENTRY(solve_builtin_t64_y32)(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<float, double>(a, c, s); }
 #endif
 #if TODE_INSTANTIATE_T32_Y64
-int solve_builtin_t32_y64(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double, float>(a, c, s); }
+int TODE_SOLVE_ENTRY(solve_builtin_t32_y64)(const tode_solve_args &a, const tode_controller &c, hipStream_t s) { return dispatch_term<double, float>(a, c, s); }
 #endif
 
 }  // namespace tode

@@ -86,6 +86,11 @@ template <typename T, typename TT = T> struct SolveParams {
     int cap;        // INT_MAX: unlimited
     double scalars[4];
     CtrlParams<T> cp;
+    // record of the loop state per iteration (tode_solve_record), null pointers when none is kept
+    long long rec_capacity;
+    TT *rec_t, *rec_dt;
+    T *rec_y, *rec_k0, *rec_prev, *rec_pprev;
+    int32_t *rec_running, *rec_n_accepted;
 };
 
 // Start step (step_size_controllers.py:431-490 integral, 776-835 PID; the integral
@@ -233,6 +238,12 @@ template <typename T, typename TT = T> static SolveParams<T, TT> make_params(con
     p.cap = (a.iteration_cap < 0 || a.iteration_cap >= INT_MAX) ? INT_MAX : (int)a.iteration_cap;
     for (int i = 0; i < 4; ++i) p.scalars[i] = a.term_scalars[i];
     p.cp = make_ctrl<T>(c);
+    const tode_solve_record *r = a.record;
+    p.rec_capacity = r ? r->capacity : 0;
+    p.rec_t = r ? (TT *)r->t : nullptr, p.rec_dt = r ? (TT *)r->dt : nullptr;
+    p.rec_y = r ? (T *)r->y : nullptr, p.rec_k0 = r ? (T *)r->k0 : nullptr;
+    p.rec_prev = r ? (T *)r->prev : nullptr, p.rec_pprev = r ? (T *)r->pprev : nullptr;
+    p.rec_running = r ? r->running : nullptr, p.rec_n_accepted = r ? r->n_accepted : nullptr;
     return p;
 }
 
