@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 19
+#define TODE_ABI_VERSION 20
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -559,6 +559,38 @@ typedef struct tode_step_adjoint {
 int tode_step_finish_backward(const tode_step_adjoint *adjoint, const tode_controller *controller, void *stream);
 int tode_step_stage_backward(const tode_step_adjoint *adjoint, const tode_controller *controller, int stage, const void *g_ystage,
                              const void *g_tnode, void *stream);
+
+/*
+ * The reverse sweep over a whole recorded solve with one of the three small built-in systems, in one kernel (one
+ * thread per sample walks its iterations from the last to the first).  It stands for the backward pass that
+ * torch.autograd runs over the reference's loop (adjoints.py:33-40, 111-113, 135-260), and for the sequence
+ * tode_step_stage / f / tode_step_finish_backward / f's vector-Jacobian product / tode_step_stage_backward per
+ * iteration above, with the right-hand side and its vector-Jacobian product evaluated in the kernel.
+ *
+ * args: the forward problem as for tode_solve_builtin (y0 is not read; t_start / t_end dense; dtype one of TODE_F32 /
+ * TODE_F64; method Dopri5 or Tsit5; controller integral or PID), with args->record pointing to the record the forward
+ * pass wrote.  All pointers below are device memory.  Nothing is allocated; the call only enqueues.
+ */
+typedef struct tode_solve_adjoint {
+    const void *grad_ys;           /* [B, max(E,1), F] cotangent of ys */
+    const int32_t *points_by_iteration; /* [B,E]: each sample's evaluation points ordered by the iteration that wrote them */
+    const int32_t *iterations_sorted;   /* [B,E]: those iterations in the same order, ascending; -1 (first) for a point that
+                                           no iteration wrote.  Both NULL when E == 0 */
+    int64_t iterations;            /* L: iterations of the loop; the record's entries 0..L are read */
+    int32_t through_control;       /* as in tode_step_adjoint */
+    int32_t reserved;
+    void *scratch;                 /* tode_solve_backward_scratch_bytes(args) bytes */
+    int64_t scratch_bytes;
+    /* results: cotangents of the loop state before the first iteration (y, the first-same-as-last derivative
+       f(t_start, y0), t, the first step, the controller's history) ... */
+    void *a_y, *a_k0;              /* [B,F] */
+    void *a_t, *a_dt, *a_prev, *a_pprev; /* [B] */
+    void *g_params;                /* ... and of the term's per-sample parameters [B,P] */
+    void *g_t_start, *g_t_end;     /* [B], added to; NULL: not wanted */
+    void *g_t_eval;                /* [B,E], added to; NULL: not wanted */
+} tode_solve_adjoint;
+int64_t tode_solve_backward_scratch_bytes(const tode_solve_args *args);
+int tode_solve_builtin_backward(const tode_solve_args *args, const tode_controller *controller, const tode_solve_adjoint *adjoint, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Protocol operators.

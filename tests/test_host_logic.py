@@ -141,6 +141,26 @@ def test_solve_workspace_size_and_argument_checks_of_the_one_call_entry_point():
     assert lib.tode_solve_builtin_auto(_lib.C.byref(a), _lib.C.byref(c), p, p, p, p, p, need, 1, None, _lib.C.byref(it)) == _lib.E_UNSUPPORTED
 
 
+def test_whole_reverse_sweep_entry_point_checks_its_arguments_without_a_gpu():
+    lib = _lib.load()
+    a, c, adj = _lib.SolveArgs(), _lib.Controller(), _lib.SolveAdjoint()
+    ref = lambda x: _lib.C.byref(x)
+    assert lib.tode_solve_builtin_backward(None, None, None, None) == _lib.E_INVALID
+    a.dtype, a.batch, a.n_features, a.n_eval, a.n_params, a.term = _lib.DTYPES[torch.float64], 100, 2, 0, 1, 1
+    a.t_start_stride = a.t_end_stride = 1
+    assert lib.tode_solve_backward_scratch_bytes(ref(a)) == (7 * 2 + 7 * 2 + 2 + 2 + 2 * 2 + 4 + 2) * 100 * 8
+    assert lib.tode_solve_builtin_backward(ref(a), ref(c), ref(adj), None) == _lib.E_INVALID and b"record" in lib.tode_last_error()
+    rec = _lib.SolveRecord()
+    rec.capacity = 5
+    a.record = _lib.C.addressof(rec)
+    adj.iterations = 5
+    assert lib.tode_solve_builtin_backward(ref(a), ref(c), ref(adj), None) == _lib.E_INVALID and b"entries" in lib.tode_last_error()
+    adj.iterations = 4
+    assert lib.tode_solve_builtin_backward(ref(a), ref(c), ref(adj), None) == _lib.E_INVALID  # null arrays
+    a.dtype = _lib.dtype_code(torch.float32, torch.float64)
+    assert lib.tode_solve_builtin_backward(ref(a), ref(c), ref(adj), None) == _lib.E_UNSUPPORTED and b"one dtype" in lib.tode_last_error()
+
+
 def test_abi_argument_validation_without_a_gpu():
     """Null / inconsistent arguments are rejected before anything touches a device."""
     lib = _lib.load()

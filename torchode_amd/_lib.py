@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -40,6 +40,8 @@ EXPORTS = (
     "tode_solve_builtin_fast_sync",
     "tode_solve_builtin_fast_static",
     "tode_solve_builtin_auto",
+    "tode_solve_builtin_backward",
+    "tode_solve_backward_scratch_bytes",
     "tode_solve_workspace_bytes",
     "tode_mlp_pack_weights",
     "tode_select_end_point",
@@ -144,6 +146,15 @@ class SolveRecord(C.Structure):
     """struct tode_solve_record"""
 
     _fields_ = [("capacity", C.c_int64)] + [(n, C.c_void_p) for n in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")]
+
+
+class SolveAdjoint(C.Structure):
+    """struct tode_solve_adjoint"""
+
+    _fields_ = [("grad_ys", C.c_void_p), ("points_by_iteration", C.c_void_p), ("iterations_sorted", C.c_void_p), ("iterations", C.c_int64), ("through_control", C.c_int32), ("reserved", C.c_int32),
+                ("scratch", C.c_void_p), ("scratch_bytes", C.c_int64)] + [
+        (n, C.c_void_p) for n in ("a_y", "a_k0", "a_t", "a_dt", "a_prev", "a_pprev", "g_params", "g_t_start", "g_t_end", "g_t_eval")
+    ]  # fmt: skip
 
 
 STEP_FLAG_STOPPED, STEP_FLAG_ITERATIONS, STEP_FLAG_ANY_RUNNING, STEP_FLAG_ANY_FAILURE, STEP_FLAG_WORDS = 0, 1, 2, 3, 4
@@ -327,6 +338,10 @@ def load():
         lib.tode_solve_workspace_bytes.argtypes = [C.POINTER(SolveArgs)]
         lib.tode_solve_builtin_auto.restype = C.c_int
         lib.tode_solve_builtin_auto.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 5 + [C.c_int64, C.c_int32, C.c_void_p, C.POINTER(C.c_int64)]
+        lib.tode_solve_backward_scratch_bytes.restype = C.c_int64
+        lib.tode_solve_backward_scratch_bytes.argtypes = [C.POINTER(SolveArgs)]
+        lib.tode_solve_builtin_backward.restype = C.c_int
+        lib.tode_solve_builtin_backward.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller), C.POINTER(SolveAdjoint), C.c_void_p]
         lib.tode_step_begin.restype = C.c_int
         lib.tode_step_begin.argtypes = [C.POINTER(StepState), C.POINTER(Controller), C.c_void_p, C.c_int, C.c_void_p]
         lib.tode_step_stage.restype = C.c_int

@@ -648,6 +648,7 @@ class AutoDiffAdjoint(nn.Module):
             order = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
             record.states = [tuple(fields[k][i] for k in order) for i in range(n)]
             record.iterations = L
+            record.arrays = fields  # (entry-major arrays: what tode_solve_builtin_backward reads)
         return Solution(ts=ts, ys=ys, stats=stats, status=status)
 
     def __repr__(self):

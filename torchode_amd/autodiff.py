@@ -365,6 +365,92 @@ def reverse_sweep_torch(replay: Replay, states, hits, grad_ys, params):
     return adj, grad_params
 
 
+def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, grad_ys, params):
+    """All iterations in reverse in one kernel (tode_solve_builtin_backward): for a built-in term whose forward pass
+    left its record in entry-major arrays.  The right-hand side and its vector-Jacobian product are evaluated in the
+    kernel; what comes back are the cotangents of the state before the first iteration and of the term's per-sample
+    parameter table, which autograd carries on to the tensors the table was made from."""
+    lib = _lib.load()
+    f = term.f
+    method, controller = adjoint.step_method, adjoint.step_size_controller
+    ctrl = controller.c_struct()
+    y0 = problem.y0
+    B, F = y0.shape
+    E = problem.n_evaluation_points
+    dev, dtype = y0.device, y0.dtype
+    new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+    zeros = lambda *shape, dt=dtype: torch.zeros(shape, dtype=dt, device=dev)
+    contiguous = lambda x: x.detach().to(dtype).contiguous()
+    t_start, t_end = contiguous(replay.t_start), contiguous(replay.t_end)
+    t_eval = None if replay.t_eval is None else contiguous(replay.t_eval)
+    L, arrays = record.iterations, record.arrays
+
+    # which iteration wrote which evaluation point (adjoints.py:215-234): the first whose new time has passed it
+    iterations_sorted = points_by_iteration = None
+    if E > 0:
+        direction = torch.where(t_end > t_start, 1.0, -1.0).to(dtype)
+        reached = (direction[None, :] * arrays["t"][1 : L + 1]).t().contiguous()  # [B, L], ascending
+        hit = torch.searchsorted(reached, direction[:, None] * t_eval) if L > 0 else torch.zeros((B, E), dtype=torch.long, device=dev)
+        hit = torch.where(hit < L, hit, torch.full_like(hit, -1))
+        hit[:, 0] = torch.where(t_eval[:, 0] == t_start, torch.full_like(hit[:, 0], -1), hit[:, 0])
+        # ordered by iteration, so that the kernel, walking the iterations down, finds each one's points at a cursor
+        iterations_sorted, points_by_iteration = torch.sort(hit.to(torch.int32), dim=1, stable=True)
+        iterations_sorted, points_by_iteration = iterations_sorted.contiguous(), points_by_iteration.to(torch.int32).contiguous()
+    wants = lambda x: x is not None and x.requires_grad
+    g_t_start = zeros(B) if wants(replay.t_start) else None
+    g_t_end = zeros(B) if wants(replay.t_end) else None
+    g_t_eval = zeros(B, E) if (E > 0 and wants(replay.t_eval)) else None
+
+    with torch.no_grad():
+        par = f.builtin_params().detach().to(device=dev, dtype=dtype).contiguous()
+    P = par.shape[1]
+    scal = list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4
+    a = _lib.SolveArgs()
+    a.dtype, a.method, a.term, a.n_features, a.n_eval, a.n_params, a.batch = _lib.DTYPES[dtype], method.method_id, f.builtin_kind, F, E, P, B
+    a.max_steps, a.iteration_cap = -1, -1
+    a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
+    a.t_start, a.t_end, a.t_start_stride, a.t_end_stride = t_start.data_ptr(), t_end.data_ptr(), 1, 1
+    a.t_eval, a.params = _lib.ptr(t_eval), (par.data_ptr() if par.numel() else None)
+    names = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
+    rec = _lib.SolveRecord(arrays["t"].shape[0], *(arrays[k].data_ptr() for k in names))
+    a.record = _lib.C.addressof(rec)
+
+    out_y, out_k0 = new(B, F), new(B, F)
+    out_s = new(4, B)
+    g_par = new(B, max(P, 1))
+    grad = grad_ys.detach().to(dtype).contiguous()
+    scratch = torch.empty(max(lib.tode_solve_backward_scratch_bytes(_lib.C.byref(a)), 1), dtype=torch.uint8, device=dev)
+    ad = _lib.SolveAdjoint()
+    ad.grad_ys, ad.iterations, ad.through_control = grad.data_ptr(), L, int(bool(replay.through_control))
+    ad.points_by_iteration, ad.iterations_sorted = _lib.ptr(points_by_iteration), _lib.ptr(iterations_sorted)
+    ad.scratch, ad.scratch_bytes = scratch.data_ptr(), scratch.numel()
+    ad.a_y, ad.a_k0 = out_y.data_ptr(), out_k0.data_ptr()
+    ad.a_t, ad.a_dt, ad.a_prev, ad.a_pprev = (out_s[i].data_ptr() for i in range(4))
+    ad.g_params = g_par.data_ptr()
+    ad.g_t_start, ad.g_t_end, ad.g_t_eval = _lib.ptr(g_t_start), _lib.ptr(g_t_end), _lib.ptr(g_t_eval)
+    _lib.check(lib.tode_solve_builtin_backward(_lib.C.byref(a), _lib.C.byref(ctrl), _lib.C.byref(ad), _lib.stream_of(y0)), "tode_solve_builtin_backward")
+
+    # the parameter table is a function of the term's tensors (a reshape, a negation ...): autograd takes its cotangent on
+    grad_params = [None] * len(params)
+    if params and P > 0:
+        with torch.enable_grad():
+            f.__dict__.pop("_params_view", None)  # (a table kept from a call without grad mode has no graph)
+            table = f.builtin_params()
+            f.__dict__.pop("_params_view", None)
+            if table.requires_grad:
+                grads = torch.autograd.grad(table, params, g_par[:, :P].to(table.dtype), allow_unused=True)
+                grad_params = list(grads)
+    for given, collected in ((replay.t_start, g_t_start), (replay.t_end, g_t_end), (replay.t_eval, g_t_eval)):
+        if collected is None:
+            continue
+        for j, q in enumerate(params):
+            if q is given:
+                grad_params[j] = _add(grad_params[j], collected.to(q.dtype))
+                break
+    adj = dict(y=out_y, k0=out_k0, t=out_s[0], dt=out_s[1], prev=out_s[2], pprev=out_s[3])
+    return adj, grad_params
+
+
 def reverse_sweep_kernels(adjoint, replay: Replay, term, args, problem, dt0_given, dt0, states, hits, grad_ys, params, params_given):
     """The iterations in reverse through the library's reverse kernels (tode_step_finish_backward,
     tode_step_stage_backward): per iteration the stage values are recomputed by the forward stage kernel and ``f``
@@ -567,19 +653,31 @@ class SolveThroughLoop(torch.autograd.Function):
         args = map_tensors(ctx.args, leaf)
         params = [stand_in.get(id(p), p) for p in params]
         replay = Replay(adjoint.step_method, adjoint.step_size_controller, term, args, times, adjoint.backprop_through_step_size_control, dt0)
-        states = ctx.record.trimmed(ctx.record.iterations)
         E = problem.n_evaluation_points
-        hits = simulate_hits(replay, states, E)
         y0 = problem.y0
         add = _add
         F = y0.shape[1]
         use_kernels = getattr(adjoint, "backward_kernels", True) and adjoint._fused_ok(problem, term)
+        # one kernel for the whole sweep: a built-in small system whose forward pass wrote its record in the kernel,
+        # time and data in one dtype, every gradient asked for within the kernel's reach (state, times, the term's table)
+        use_whole = (
+            use_kernels
+            and getattr(adjoint, "backward_whole_kernel", True)
+            and getattr(ctx.record, "arrays", None) is not None
+            and problem.time_dtype == problem.data_dtype
+            and not term.with_args
+        )
         global LAST_SWEEP
-        LAST_SWEEP = "kernels" if use_kernels else "torch"  # (looked at by the tests)
-        if use_kernels:
-            adj, grad_params = reverse_sweep_kernels(adjoint, replay, term, args, problem, ctx.dt0, dt0, states, hits, grad_ys, params, list(ctx.params))
+        LAST_SWEEP = "whole" if use_whole else ("kernels" if use_kernels else "torch")  # (looked at by the tests)
+        if use_whole:
+            adj, grad_params = reverse_sweep_whole(adjoint, replay, term, problem, dt0, ctx.record, grad_ys, params)
         else:
-            adj, grad_params = reverse_sweep_torch(replay, states, hits, grad_ys, params)
+            states = ctx.record.trimmed(ctx.record.iterations)
+            hits = simulate_hits(replay, states, E)
+            if use_kernels:
+                adj, grad_params = reverse_sweep_kernels(adjoint, replay, term, args, problem, ctx.dt0, dt0, states, hits, grad_ys, params, list(ctx.params))
+            else:
+                adj, grad_params = reverse_sweep_torch(replay, states, hits, grad_ys, params)
 
         # ---- the start of the loop: y = y0, k0 = f(t_start, y0), dt from the start step rule or dt0 ----
         with torch.enable_grad():

@@ -49,6 +49,8 @@ UNITS = [
     ("tode_pair.hip", "tode_pair_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_pair.hip", "tode_pair_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
     ("tode_stepwise.hip", "tode_stepwise.o", []),
+    ("tode_backward.hip", "tode_backward_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
+    ("tode_backward.hip", "tode_backward_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
     ("tode_ops.hip", "tode_ops.o", []),
     ("tode_grid.hip", "tode_grid.o", []),
     ("tode_mlp.hip", "tode_mlp.o", []),

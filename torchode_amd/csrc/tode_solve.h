@@ -29,6 +29,14 @@ template <typename T, int F_> struct LinearDecayTerm {  // (-k) * y
 #pragma unroll
         for (int f = 0; f < F; ++f) dy[f] = nk[f] * y[f];
     }
+    // vector-Jacobian product: g is the cotangent of dy; gy receives that of y, gpar is added to that of k
+    __device__ __forceinline__ void vjp(T, const T (&y)[F_], const T (&g)[F_], T (&gy)[F_], T (&gpar)[F_]) const {
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            gy[f] = nk[f] * g[f];
+            gpar[f] -= y[f] * g[f];
+        }
+    }
 };
 
 template <typename T> struct VanDerPolTerm {  // dx = v ; dv = ((mu*(1-(x*x)))*v)-x
@@ -44,6 +52,12 @@ template <typename T> struct VanDerPolTerm {  // dx = v ; dv = ((mu*(1-(x*x)))*v
         T m2 = m1 * v;
         dy[0] = v;
         dy[1] = m2 - x;
+    }
+    __device__ __forceinline__ void vjp(T, const T (&y)[2], const T (&g)[2], T (&gy)[2], T (&gpar)[1]) const {
+        const T x = y[0], v = y[1], om = (T)1 - x * x;
+        gy[0] = g[1] * (mu * ((T)-2 * x) * v - (T)1);
+        gy[1] = g[0] + g[1] * (mu * om);
+        gpar[0] += g[1] * (om * v);
     }
 };
 
@@ -66,6 +80,13 @@ template <typename T> struct Lorenz63Term {  // dx=sigma*(y-x); dy=(x*(rho-z))-y
         dy[0] = sigma * d1;
         dy[1] = xr - yy;
         dy[2] = xy - bz;
+    }
+    __device__ __forceinline__ void vjp(T, const T (&y)[3], const T (&g)[3], T (&gy)[3], T (&gpar)[1]) const {
+        const T x = y[0], yy = y[1], z = y[2];
+        gy[0] = (rho - z) * g[1] + yy * g[2] - sigma * g[0];
+        gy[1] = sigma * g[0] - g[1] + x * g[2];
+        gy[2] = -(x * g[1]) - beta * g[2];
+        gpar[0] += x * g[1];
     }
 };
 
