@@ -642,7 +642,8 @@ def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
 
 @gpu
 @pytest.mark.parametrize("through_control", [True, False], ids=["through-control", "steps-constant"])
-@pytest.mark.parametrize("case", ["vdp-f64", "vdp-f32", "lorenz-f64", "linear-decay-f64", "vdp-dopri5-integral", "end-only", "times", "dt0", "max-steps", "backwards"])
+@pytest.mark.parametrize("case", ["vdp-f64", "vdp-f32", "lorenz-f64", "linear-decay-f64", "vdp-dopri5-integral", "end-only", "times", "dt0", "max-steps", "backwards",
+                                  "non-monotone", "limits"])  # fmt: skip
 def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_sweep(case, through_control):
     """A differentiable solve with a built-in term three ways: the reverse sweep in one kernel (the right-hand side's
     vector-Jacobian product in closed form), the per-iteration reverse kernels with autograd through the term's torch
@@ -659,6 +660,8 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
     if case == "backwards":
         t_eval[::2] = t_eval[::2].flip(1)
         t_eval[::2] = t_eval[::2, :1] - 0.01 * (t_eval[::2, :1] - t_eval[::2])
+    if case == "non-monotone":  # (every fifth row: two points swapped, written by other iterations than their neighbours)
+        t_eval[::5, 3], t_eval[::5, 7] = t_eval[::5, 7].clone(), t_eval[::5, 3].clone()
     if case == "times":
         t_eval.requires_grad_()
     # (a first step large enough for its error estimate to stand above rounding: with 1e-3 even the two older sweeps
@@ -669,6 +672,8 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
     method = {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[w.method]
     if case == "vdp-dopri5-integral":
         method, kind, ctrl = to.Dopri5, "integral", dict(atol=1e-6, rtol=1e-4)
+    if case == "limits":
+        ctrl.update(dt_min=1e-3, dt_max=0.1)
     make_controller = lambda: to.PIDController(**ctrl) if kind == "pid" else to.IntegralController(**ctrl)
     if case == "end-only":
         problem = to.InitialValueProblem(y0, t_eval[:, 0].clone(), t_eval[:, -1].clone())
@@ -686,6 +691,9 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
         sol = solver.solve(problem, to.ODETerm(type(w.f)(leaf)), dt0=dt0)
         assert sol.ys.requires_grad
         written = (torch.arange(max(E, 1), device="cuda")[None, :] < sol.stats["n_initialized"][:, None])[:, :, None]
+        if case == "non-monotone":  # (every point of every row is written here: the solves run to their ends)
+            assert (sol.status == 0).all()
+            written = torch.ones_like(written)
         loss = (torch.where(written, sol.ys, torch.zeros_like(sol.ys)) * weights).sum()
         results[sweep] = torch.autograd.grad(loss, wrt, allow_unused=True)
         assert autodiff.LAST_SWEEP == sweep
