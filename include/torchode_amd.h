@@ -45,7 +45,7 @@ enum {
     TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
     TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
                                          float32, tode_solve_builtin_fast only */
-    TODE_TERM_MLP = 4                 /* F = 64: tanh([y, t] W1^T + b1) W2^T + b2 with 256 hidden units, weights in
+    TODE_TERM_MLP = 4                 /* F = 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units, weights in
                                          shared_params as packed by tode_mlp_pack_weights; float32,
                                          tode_solve_builtin_fast only */
 };
@@ -166,7 +166,7 @@ typedef struct tode_solve_args {
     const void *dt0;           /* [B] user initial step, or NULL to select one */
     const void *params;        /* [B,P] */
     const void *shared_params; /* [n_shared_params] right-hand side parameters shared by the batch, or NULL */
-    int64_t n_shared_params;   /* TODE_TERM_MLP: W1 [256,65] | b1 [256] | W2 [64,256] | b2 [64], row-major, concatenated */
+    int64_t n_shared_params;   /* TODE_TERM_MLP: TODE_MLP_PACKED_SIZE[_BF16], the words tode_mlp_pack_weights wrote */
     void *ys;                  /* out [B,max(E,1),F] */
     void *y_idle;              /* out [B,F], used only when E == 0: value the reference
                                   reports for a sample that finished before iteration L */
@@ -347,9 +347,12 @@ int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int6
 /*
  * Weights of TODE_TERM_MLP in the order the solve kernel loads them into
  * registers (each thread of a workgroup reads its own values, contiguous across
- * a wavefront).  `raw`: W1 [256 x 65] | b1 [256] | W2 [64 x 256] | b2 [64],
- * row-major float32 on the device, n_raw = 33088 -- the parameters of the
- * user's `f` as a torch module holds them (terms.py:13-19 takes any callable).
+ * a wavefront).  `raw`: W1 [H x 65] | b1 [H] | W2 [64 x H] | b2 [64] for a
+ * network of H hidden units, 1 <= H <= 256, row-major float32 on the device,
+ * n_raw = 130 H + 64 (33344 for H = 256) -- the parameters of the user's `f` as
+ * a torch module holds them (terms.py:13-19 takes any callable).  The kernel
+ * always works on 256 units: those from H on are packed with zero weights and
+ * a zero bias and add exact zeros to every sum.
  * `packed`: TODE_MLP_PACKED_SIZE (matrix_inputs = TODE_MLP_INPUTS_F32) or
  * TODE_MLP_PACKED_SIZE_BF16 (TODE_MLP_INPUTS_BF16: W1 and W2 rounded to
  * bfloat16, two per word) 32-bit words on the device; pass it as shared_params

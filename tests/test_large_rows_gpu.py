@@ -303,6 +303,36 @@ def test_mlp_kernel_on_the_benchmark_workload(batch):
     assert_close_solutions(fused, proto)
 
 
+@pytest.mark.parametrize("inputs", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [128, 100, 16, 3])
+def test_mlp_kernel_with_fewer_hidden_units(hidden, inputs):
+    """The kernel works on 256 hidden units; a narrower network is packed with zero weights and a zero bias for the
+    rest, which add exact zeros in the same places: against the protocol path with torch's matrix products of the
+    narrow network itself, and, unit for unit, against the same network written as 256 units of which the last are zero
+    -- same bits."""
+    import torchode_amd.builtin_terms as bt
+
+    w = to.workloads.make("mlp", batch=96, device="cuda")
+    g = torch.Generator().manual_seed(hidden)
+    scale1, scale2 = (6.0 / (65 + hidden)) ** 0.5, (6.0 / (hidden + 64)) ** 0.5
+    W1 = ((torch.rand(hidden, 65, generator=g) * 2 - 1) * scale1).cuda()
+    W2 = ((torch.rand(64, hidden, generator=g) * 2 - 1) * scale2).cuda()
+    b1, b2 = (torch.rand(hidden, generator=g) - 0.5).cuda() * 0.1, (torch.rand(64, generator=g) - 0.5).cuda() * 0.1
+    narrow = bt.MLPField(W1, b1, W2, b2, matrix_inputs=inputs)
+    pad = lambda x, shape: torch.zeros(shape, device="cuda").index_put_(tuple(torch.meshgrid(*(torch.arange(n, device="cuda") for n in x.shape), indexing="ij")), x)
+    wide = bt.MLPField(pad(W1, (256, 65)), pad(b1, (256,)), pad(W2, (64, 256)), b2.clone(), matrix_inputs=inputs)
+    kernel = "tode::solve_mlp_kernel" + ("" if inputs == "float32" else " (bfloat16 matrix inputs)")
+    a, proto = mlp_both_paths(w._replace(f=narrow), w.method, w.controller, kernel=kernel)
+    b, _ = mlp_both_paths(w._replace(f=wide), w.method, w.controller, kernel=kernel)
+    assert torch.equal(a.ys, b.ys) and torch.equal(a.status, b.status)
+    for key in ("n_steps", "n_accepted", "n_initialized"):
+        assert torch.equal(a.stats[key], b.stats[key]), key
+    if inputs == "float32":
+        assert_close_solutions(a, proto, min_agree=0.95, loose=1e-2)
+    else:  # (the rounded right-hand side is piecewise constant at the 2^-9 level: step counts scatter, the solutions agree)
+        assert torch.equal(a.status, proto.status) and mixed_error(a.ys.double().cpu(), proto.ys.double().cpu()) < 5e-2
+
+
 @pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "pid"), ("tsit5", "integral")])
 def test_mlp_kernel_with_tight_tolerances(method, kind):
     """At rtol 1e-6 every error estimate sits at the rounding noise of the float32 matrix products, so

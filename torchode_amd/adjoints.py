@@ -185,7 +185,7 @@ class AutoDiffAdjoint(nn.Module):
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
             return F in (32 * 32, 64 * 64) and E <= 8192
-        return F == 64 and tuple(f.W1.shape) == (256, 65) and E <= 512
+        return F == 64 and f.W1.shape[1] == 65 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable
     def _solve_eager_outside_the_trace(self, problem, term, dt0, args) -> Solution:
@@ -575,8 +575,8 @@ class AutoDiffAdjoint(nn.Module):
             params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
         mlp = f.builtin_kind == _lib.TERM_MLP
-        if mlp and (dtype != torch.float32 or F != 64 or tuple(f.W1.shape) != (256, 65)):
-            return None  # the matrix-core kernel is built for this shape only: the caller takes the protocol path
+        if mlp and (dtype != torch.float32 or F != 64 or f.W1.shape[1] != 65 or not 1 <= f.W1.shape[0] <= 256):
+            return None  # the matrix-core kernel is built for 64 features and up to 256 hidden units: the caller takes another path
         shared = f.builtin_packed(dev, dtype) if mlp else None
         ttype = t_start.dtype
         dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()

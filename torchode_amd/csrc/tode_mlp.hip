@@ -42,7 +42,6 @@ constexpr int MLP_F = 64, MLP_H = 256, MLP_TILE = 16;
 constexpr int MLP_XS = 84;  // LDS row of the stage input: 64 features, t, zeros up to column 79, padding
 constexpr int MLP_REGS = 68 + 16 + 64 + 4;       // packed values per thread: W1, b1, W2, b2
 constexpr int MLP_REGS_BF16 = 40 + 16 + 32 + 4;  // the same with W1 (80 inputs) and W2 as pairs of bfloat16
-constexpr long long MLP_RAW = (long long)MLP_H * (MLP_F + 1) + MLP_H + (long long)MLP_F * MLP_H + MLP_F;
 
 struct __align__(16) MlpShared {
     float x[MLP_TILE * MLP_XS];
@@ -74,20 +73,25 @@ struct MlpWeightsBf16 {
 // the first 16 steps (contiguous in LDS), then t and three zero columns.
 __host__ __device__ __forceinline__ int mlp_input_of(int kk, int q) { return kk < 16 ? 16 * q + kk : 64 + q; }
 
-// Source index (in W1 | b1 | W2 | b2, row-major) of packed value j of thread tid, or -1 for zero.
-__host__ __device__ inline long long mlp_packed_source(int j, int tid) {
+// Source index (in W1 | b1 | W2 | b2, row-major) of packed value j of thread tid, or -1 for zero.  H: hidden units of
+// the network at hand, at most MLP_H; the kernel's units from H on get zero weights and a zero bias, so that they
+// add tanh(0) * 0 = 0 to every sum in the same places as before (a narrower network in the same arithmetic).
+__host__ __device__ inline long long mlp_packed_source(int j, int tid, int H) {
     const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
-    const long long o_b1 = (long long)MLP_H * (MLP_F + 1), o_w2 = o_b1 + MLP_H, o_b2 = o_w2 + (long long)MLP_F * MLP_H;
+    const long long o_b1 = (long long)H * (MLP_F + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)MLP_F * H;
     if (j < 68) {
-        const int kk = j / 4, tile = j % 4, k = mlp_input_of(kk, q);
-        return k <= MLP_F ? (long long)(64 * w + 16 * tile + c) * (MLP_F + 1) + k : -1;
+        const int kk = j / 4, tile = j % 4, k = mlp_input_of(kk, q), unit = 64 * w + 16 * tile + c;
+        return (k <= MLP_F && unit < H) ? (long long)unit * (MLP_F + 1) + k : -1;
     }
     j -= 68;
-    if (j < 16) return o_b1 + 64 * w + 16 * (j / 4) + 4 * q + (j % 4);
+    if (j < 16) {
+        const int unit = 64 * w + 16 * (j / 4) + 4 * q + (j % 4);
+        return unit < H ? o_b1 + unit : -1;
+    }
     j -= 16;
     if (j < 64) {
-        const int ft = j / 16, tile = (j / 4) % 4, r = j % 4;
-        return o_w2 + (long long)(16 * ft + c) * MLP_H + 64 * w + 16 * tile + 4 * q + r;
+        const int ft = j / 16, tile = (j / 4) % 4, r = j % 4, unit = 64 * w + 16 * tile + 4 * q + r;
+        return unit < H ? o_w2 + (long long)(16 * ft + c) * H + unit : -1;
     }
     j -= 64;
     return o_b2 + 16 * w + 4 * q + j;
@@ -95,52 +99,55 @@ __host__ __device__ inline long long mlp_packed_source(int j, int tid) {
 
 // The same for the bfloat16 variant: packed word j of thread tid holds the values of sources
 // (lo, hi) as bfloat16 in its low and high half (words of b1 and b2: one float32, hi = -2).
-__host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, long long &lo, long long &hi) {
+__host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, int H, long long &lo, long long &hi) {
     const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
-    const long long o_b1 = (long long)MLP_H * (MLP_F + 1), o_w2 = o_b1 + MLP_H, o_b2 = o_w2 + (long long)MLP_F * MLP_H;
+    const long long o_b1 = (long long)H * (MLP_F + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)MLP_F * H;
     hi = -2;
     if (j < 40) {
-        const int ks = j / 8, tile = (j / 2) % 4, k = 16 * ks + 4 * q + 2 * (j % 2);
-        const long long row = (long long)(64 * w + 16 * tile + c) * (MLP_F + 1);
-        lo = k <= MLP_F ? row + k : -1;
-        hi = k + 1 <= MLP_F ? row + k + 1 : -1;
+        const int ks = j / 8, tile = (j / 2) % 4, k = 16 * ks + 4 * q + 2 * (j % 2), unit = 64 * w + 16 * tile + c;
+        const long long row = (long long)unit * (MLP_F + 1);
+        lo = (k <= MLP_F && unit < H) ? row + k : -1;
+        hi = (k + 1 <= MLP_F && unit < H) ? row + k + 1 : -1;
         return;
     }
     j -= 40;
     if (j < 16) {
-        lo = o_b1 + 64 * w + 16 * (j / 4) + 4 * q + (j % 4);
+        const int unit = 64 * w + 16 * (j / 4) + 4 * q + (j % 4);
+        lo = unit < H ? o_b1 + unit : -1;
+        hi = -3;  // (one float32 word, zero where lo < 0)
         return;
     }
     j -= 16;
     if (j < 32) {
-        const int ft = j / 8, tile = (j / 2) % 4;
-        lo = o_w2 + (long long)(16 * ft + c) * MLP_H + 64 * w + 16 * tile + 4 * q + 2 * (j % 2);
-        hi = lo + 1;
+        const int ft = j / 8, tile = (j / 2) % 4, unit = 64 * w + 16 * tile + 4 * q + 2 * (j % 2);
+        const long long at = o_w2 + (long long)(16 * ft + c) * H + unit;
+        lo = unit < H ? at : -1;
+        hi = unit + 1 < H ? at + 1 : -1;
         return;
     }
     j -= 32;
     lo = o_b2 + 16 * w + 4 * q + j;
 }
 
-static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed) {
+static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed, int H) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= MLP_REGS_BF16 * 256) return;
     const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
     long long lo, hi;
-    mlp_packed_source_bf16(4 * group + part, tid, lo, hi);
-    if (hi == -2) {
-        packed[i] = __float_as_uint(raw[lo]);
+    mlp_packed_source_bf16(4 * group + part, tid, H, lo, hi);
+    if (hi == -2 || hi == -3) {
+        packed[i] = lo < 0 ? 0u : __float_as_uint(raw[lo]);
         return;
     }
     const __bf16 a = (__bf16)(lo < 0 ? 0.0f : raw[lo]), b = (__bf16)(hi < 0 ? 0.0f : raw[hi]);  // round to nearest even
     packed[i] = (unsigned)__builtin_bit_cast(unsigned short, a) | ((unsigned)__builtin_bit_cast(unsigned short, b) << 16);
 }
 
-static __global__ void mlp_pack_kernel(const float *raw, float *packed) {
+static __global__ void mlp_pack_kernel(const float *raw, float *packed, int H) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= MLP_REGS * 256) return;
     const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
-    const long long src = mlp_packed_source(4 * group + part, tid);
+    const long long src = mlp_packed_source(4 * group + part, tid, H);
     packed[i] = src < 0 ? 0.0f : raw[src];
 }
 
@@ -531,7 +538,7 @@ int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *n
     const bool f32 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE, bf16 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE_BF16;
     if (a.n_features != MLP_F || !(f32 || bf16))
         return fail(TODE_E_UNSUPPORTED,
-                    "the MLP kernel is built for 64 features and 256 hidden units, with the weights packed by tode_mlp_pack_weights "
+                    "the MLP kernel is built for 64 features and up to 256 hidden units, with the weights packed by tode_mlp_pack_weights "
                     "(%d or %d values); got F=%d and %lld shared parameters", TODE_MLP_PACKED_SIZE, TODE_MLP_PACKED_SIZE_BF16, a.n_features,
                     (long long)a.n_shared_params);
     if (!a.shared_params) return fail(TODE_E_INVALID, "null shared_params");
@@ -544,11 +551,14 @@ int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *n
 int mlp_pack_weights(const float *raw, long long n_raw, int matrix_inputs, float *packed, hipStream_t s) {
     static_assert(TODE_MLP_PACKED_SIZE == MLP_REGS * 256 && TODE_MLP_PACKED_SIZE_BF16 == MLP_REGS_BF16 * 256, "packed sizes");
     if (!raw || !packed) return fail(TODE_E_INVALID, "null pointer");
-    if (n_raw != MLP_RAW) return fail(TODE_E_UNSUPPORTED, "expected W1 [256 x 65] | b1 [256] | W2 [64 x 256] | b2 [64] = %lld values, got %lld", MLP_RAW, n_raw);
+    // W1 [H x 65] | b1 [H] | W2 [64 x H] | b2 [64] = 130 H + 64 values for H hidden units, 1 <= H <= 256
+    const long long H = (n_raw - MLP_F) / (2 * MLP_F + 2);
+    if (n_raw < MLP_F || H * (2 * MLP_F + 2) + MLP_F != n_raw || H < 1 || H > MLP_H)
+        return fail(TODE_E_UNSUPPORTED, "expected W1 [H x 65] | b1 [H] | W2 [64 x H] | b2 [64] = 130 H + 64 values with 1 <= H <= %d, got %lld", MLP_H, n_raw);
     if (matrix_inputs == TODE_MLP_INPUTS_F32)
-        hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed);
+        hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed, (int)H);
     else if (matrix_inputs == TODE_MLP_INPUTS_BF16)
-        hipLaunchKernelGGL(mlp_pack_bf16_kernel, dim3((MLP_REGS_BF16 * 256 + 255) / 256), dim3(256), 0, s, raw, reinterpret_cast<unsigned *>(packed));
+        hipLaunchKernelGGL(mlp_pack_bf16_kernel, dim3((MLP_REGS_BF16 * 256 + 255) / 256), dim3(256), 0, s, raw, reinterpret_cast<unsigned *>(packed), (int)H);
     else
         return fail(TODE_E_INVALID, "unknown matrix input type %d", matrix_inputs);
     return check_hip(hipGetLastError(), "tode_mlp_pack_weights launch");
