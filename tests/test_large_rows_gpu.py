@@ -215,6 +215,20 @@ def test_grid_kernel_on_the_benchmark_workload_backwards_and_with_dt0():
     assert_same(*both_paths(f, y0, t_eval, "dopri5", dict(kind="integral", atol=1e-6, rtol=1e-4), dt0=dt0))
 
 
+@pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "integral")])
+def test_grid_kernel_on_a_16_by_16_grid(method, kind):
+    """256 cells: one wavefront per sample, one chunk of the fixed summation order."""
+    ctrl = dict(kind=kind, atol=1e-7, rtol=1e-5)
+    if kind == "pid":
+        ctrl.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    f, y0, t_eval = rd_problem(70, n=16, t1=8.0, d_max=1.0)
+    fused, proto = both_paths(f, y0, t_eval, method, ctrl)
+    assert_same(fused, proto)
+    assert (fused.stats["n_steps"] > 8).all() and (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()
+    f, y0, t_eval = rd_problem(9, n=16, backwards=True)
+    assert_same(*both_paths(f, y0, t_eval, method, ctrl))
+
+
 def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():
     from torchode_amd import _lib
 

@@ -184,7 +184,7 @@ class AutoDiffAdjoint(nn.Module):
         if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != torch.float32:
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
-            return F in (32 * 32, 64 * 64) and E <= 8192
+            return F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192
         return F == 64 and f.W1.shape[1] == 65 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable

@@ -1,5 +1,5 @@
 // Whole-solve kernel for right-hand sides on a periodic N x N grid (reaction-diffusion,
-// F = N*N state values per sample): one workgroup per sample.
+// F = N*N state values per sample, N = 16, 32 or 64): one workgroup of N*N/4 threads per sample.
 //
 // Thread t owns the four consecutive cells 4t..4t+3 of the row-major grid and keeps
 // their state (y, the seven stage derivatives, the dense-output coefficients) in
@@ -291,7 +291,8 @@ int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *
     GridOut o{ns, na, ni, st};
     if (a.n_features == 64 * 64) return grid_mc<64>(a, c, o, s);
     if (a.n_features == 32 * 32) return grid_mc<32>(a, c, o, s);
-    return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 32 x 32 and 64 x 64 grids, got F=%d", a.n_features);
+    if (a.n_features == 16 * 16) return grid_mc<16>(a, c, o, s);  // (one wavefront per sample)
+    return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 16 x 16, 32 x 32 and 64 x 64 grids, got F=%d", a.n_features);
 }
 
 }  // namespace tode
