@@ -428,7 +428,10 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     ad.a_t, ad.a_dt, ad.a_prev, ad.a_pprev = (out_s[i].data_ptr() for i in range(4))
     ad.g_params = g_par.data_ptr()
     ad.g_t_start, ad.g_t_end, ad.g_t_eval = _lib.ptr(g_t_start), _lib.ptr(g_t_end), _lib.ptr(g_t_eval)
-    _lib.check(lib.tode_solve_builtin_backward(_lib.C.byref(a), _lib.C.byref(ctrl), _lib.C.byref(ad), _lib.stream_of(y0)), "tode_solve_builtin_backward")
+    rc = lib.tode_solve_builtin_backward(_lib.C.byref(a), _lib.C.byref(ctrl), _lib.C.byref(ad), _lib.stream_of(y0))
+    if rc == _lib.E_UNSUPPORTED:
+        return None  # (a shape the one-kernel sweep is not built for: the caller takes the per-iteration kernels)
+    _lib.check(rc, "tode_solve_builtin_backward")
 
     # the parameter table is a function of the term's tensors (a reshape, a negation ...): autograd takes its cotangent on
     grad_params = [None] * len(params)
@@ -669,9 +672,11 @@ class SolveThroughLoop(torch.autograd.Function):
         )
         global LAST_SWEEP
         LAST_SWEEP = "whole" if use_whole else ("kernels" if use_kernels else "torch")  # (looked at by the tests)
-        if use_whole:
-            adj, grad_params = reverse_sweep_whole(adjoint, replay, term, problem, dt0, ctx.record, grad_ys, params)
+        swept = reverse_sweep_whole(adjoint, replay, term, problem, dt0, ctx.record, grad_ys, params) if use_whole else None
+        if swept is not None:
+            adj, grad_params = swept
         else:
+            LAST_SWEEP = "kernels" if use_kernels else "torch"
             states = ctx.record.trimmed(ctx.record.iterations)
             hits = simulate_hits(replay, states, E)
             if use_kernels:
