@@ -43,16 +43,16 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the solve kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
 # profiles/); absent (null in the output) where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6876.0 KiB x 2.000 + 32933.9 KiB x 1.000) x 1024
-    ("vdp", "torch.float32", 65536): 47.81e6,
+    # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6871.2 KiB x 2.000 + 32926.0 KiB x 1.000) x 1024
+    ("vdp", "torch.float32", 65536): 47.79e6,
     # profiles/solve_pair_kernel_vdp_f64_b65536_hbm_traffic.txt: (25316.5 KiB x 2.000 + 101408.5 KiB x 1.000) x 1024
     ("vdp", "torch.float64", 65536): 155.69e6,
     # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (78246.4 KiB x 2.000 + 931465.0 KiB x 1.000) x 1024
     ("lorenz", "torch.float32", 1048576): 1114.07e6,
-    # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4370 KiB x 2.000 + 819300 KiB x 1.000) x 1024
-    ("reaction_diffusion", "torch.float32", 512): 847.9e6,
-    # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1498 KiB x 2.000 + 20624 KiB x 1.000) x 1024
-    ("mlp", "torch.float32", 4096): 24.19e6,
+    # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4393 KiB x 2.000 + 819301 KiB x 1.000) x 1024
+    ("reaction_diffusion", "torch.float32", 512): 847.96e6,
+    # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1504 KiB x 2.000 + 20624 KiB x 1.000) x 1024
+    ("mlp", "torch.float32", 4096): 24.20e6,
 }
 
 # (workload, dtype flag, matrix-core inputs of the neural ODE) after the headline, in the order their compiled CPU legs are taken
@@ -184,6 +184,48 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
     return result
 
 
+def measure_gradient(args, steps=10, warmup=3):
+    """A differentiable solve of the headline configuration (Van der Pol float32, y0 and mu requiring grad) and the
+    backward pass of sum(ys): the record of the loop state from the general whole-solve kernel, the reverse sweep in
+    one kernel."""
+    import torch
+
+    import torchode_amd as to
+    from torchode_amd import autodiff
+
+    w = to.workloads.make("vdp", batch=args.batch, dtype=torch.float32, device="cuda")
+    mu = w.f.builtin_params()[:, 0].clone().requires_grad_()
+    y0 = w.y0.clone().requires_grad_()
+    spec = dict(w.controller)
+    spec.pop("kind")
+    solver = to.AutoDiffAdjoint(to.Tsit5(), to.PIDController(**spec))
+    problem, term = to.InitialValueProblem(y0, t_eval=w.t_eval), to.ODETerm(to.VanDerPol(mu))
+    forward = backward = 0.0
+    for i in range(warmup + steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sol = solver.solve(problem, term)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        grads = torch.autograd.grad(sol.ys.sum(), (y0, mu))
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if i >= warmup:
+            forward, backward = forward + (t1 - t0), backward + (t2 - t1)
+    assert all(bool(g.isfinite().all()) for g in grads)
+    sample_steps = int(sol.stats["n_steps"].sum().item())
+    return {
+        "config": {"workload": f"vdp B={y0.shape[0]} F=2 E={w.t_eval.shape[1]} tsit5+pid, gradient of sum(ys) with respect to y0 and mu"},
+        "forward_ms": forward / steps * 1e3,
+        "backward_ms": backward / steps * 1e3,
+        "reverse_sweep": autodiff.LAST_SWEEP,
+        "value": sample_steps / ((forward + backward) / steps),
+        "unit": "sample-steps/s (forward and backward)",
+        "steps": steps,
+        "warmup": warmup,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -202,6 +244,7 @@ def main():
         help="per-step: hide the built-in term behind a plain callable, so that the solve runs through the per-step kernels around the torch right-hand side, as for any user-defined f",
     )
     ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
+    ap.add_argument("--gradient", action="store_true", help="measure the differentiable solve of the headline configuration alone (forward with its record, backward)")
     ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
     ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the headline's eager baseline is sized to (the other configurations take 0.4 of it)")
     ap.add_argument("--time-budget", type=float, default=420.0, help="seconds the whole run aims to stay within: a compiled CPU leg is started only while 100 s of it are left")
@@ -227,6 +270,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.gradient:
+        print(json.dumps(measure_gradient(args, steps=args.steps if args.steps != 50 else 10)))
+        return
     everything = args.workload is None
     head = ("vdp", "f32", "float32") if everything else (args.workload, args.dtype, args.mlp_inputs)
     result = measure(args, *head, args.steps, args.warmup)
@@ -270,6 +316,7 @@ def main():
             measure(args, "vdp", "f32", "float32", 5, 2, path="per-step", graph_iterations=None),
             measure(args, "vdp", "f32", "float32", 5, 2, path="per-step", graph_iterations=2),
         ]
+        out["gradient"] = measure_gradient(args)
     out["bench_seconds"] = time.perf_counter() - START
     print(json.dumps(out))
 
