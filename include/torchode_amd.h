@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 20
+#define TODE_ABI_VERSION 21
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -581,7 +581,14 @@ typedef struct tode_solve_adjoint {
                                            no iteration wrote.  Both NULL when E == 0 */
     int64_t iterations;            /* L: iterations of the loop; the record's entries 0..L are read */
     int32_t through_control;       /* as in tode_step_adjoint */
-    int32_t reserved;
+    int32_t through_start;         /* 0: the results are the cotangents of the loop's first state.  1: the kernel also
+                                      carries them through the start of the loop (y = y0, the first derivative
+                                      f(t_start, y0), and -- with through_control and args->dt0 == NULL -- the first
+                                      step from the start rule, step_size_controllers.py:431-490 / 776-835, clamped to
+                                      the time range): a_y is then the cotangent of y0 and g_params includes the
+                                      start's share.  The times count as constants in that part, so a caller that
+                                      wants g_t_start / g_t_end passes 0 and does the start itself.  args->dt0 is not
+                                      read, only looked at: non-NULL says that the first step was the caller's */
     void *scratch;                 /* tode_solve_backward_scratch_bytes(args) bytes */
     int64_t scratch_bytes;
     /* results: cotangents of the loop state before the first iteration (y, the first-same-as-last derivative

@@ -642,7 +642,7 @@ def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
 
 @gpu
 @pytest.mark.parametrize("through_control", [True, False], ids=["through-control", "steps-constant"])
-@pytest.mark.parametrize("case", ["vdp-f64", "vdp-f32", "lorenz-f64", "linear-decay-f64", "vdp-dopri5-integral", "end-only", "times", "dt0", "max-steps", "backwards",
+@pytest.mark.parametrize("case", ["vdp-f64", "vdp-f32", "lorenz-f64", "linear-decay-f64", "vdp-dopri5-integral", "end-only", "times", "dt0", "dt0-constant", "max-steps", "backwards",
                                   "non-monotone", "limits"])  # fmt: skip
 def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_sweep(case, through_control):
     """A differentiable solve with a built-in term three ways: the reverse sweep in one kernel (the right-hand side's
@@ -666,7 +666,9 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
         t_eval.requires_grad_()
     # (a first step large enough for its error estimate to stand above rounding: with 1e-3 even the two older sweeps
     # differ by 6e-3 in the gradient of the first step)
-    dt0 = torch.full((48,), 5e-2, dtype=dtype, device="cuda", requires_grad=True) if case == "dt0" else None
+    # ("dt0-constant": the first step is given and no time wants a gradient, so the one-kernel sweep also reverses the
+    # start of the loop, where the cotangent of the first step then ends)
+    dt0 = torch.full((48,), 5e-2, dtype=dtype, device="cuda", requires_grad=case == "dt0") if case.startswith("dt0") else None
     ctrl = dict(w.controller)
     kind = ctrl.pop("kind")
     method = {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[w.method]
@@ -681,7 +683,7 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
         problem = to.InitialValueProblem(y0, t_eval=t_eval)
     E = problem.n_evaluation_points
     weights = torch.linspace(0.5, 1.5, max(E, 1) * y0.shape[1], dtype=dtype, device="cuda").reshape(1, max(E, 1), -1)
-    wrt = [y0, leaf] + ([t_eval] if case == "times" else []) + ([dt0] if dt0 is not None else [])
+    wrt = [y0, leaf] + ([t_eval] if case == "times" else []) + ([dt0] if case == "dt0" else [])
     results = {}
     for sweep in ("whole", "kernels", "torch"):
         solver = to.AutoDiffAdjoint(method(), make_controller(), max_steps=30 if case == "max-steps" else None,

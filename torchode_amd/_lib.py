@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -151,7 +151,7 @@ class SolveRecord(C.Structure):
 class SolveAdjoint(C.Structure):
     """struct tode_solve_adjoint"""
 
-    _fields_ = [("grad_ys", C.c_void_p), ("points_by_iteration", C.c_void_p), ("iterations_sorted", C.c_void_p), ("iterations", C.c_int64), ("through_control", C.c_int32), ("reserved", C.c_int32),
+    _fields_ = [("grad_ys", C.c_void_p), ("points_by_iteration", C.c_void_p), ("iterations_sorted", C.c_void_p), ("iterations", C.c_int64), ("through_control", C.c_int32), ("through_start", C.c_int32),
                 ("scratch", C.c_void_p), ("scratch_bytes", C.c_int64)] + [
         (n, C.c_void_p) for n in ("a_y", "a_k0", "a_t", "a_dt", "a_prev", "a_pprev", "g_params", "g_t_start", "g_t_end", "g_t_eval")
     ]  # fmt: skip

@@ -365,6 +365,18 @@ def reverse_sweep_torch(replay: Replay, states, hits, grad_ys, params):
     return adj, grad_params
 
 
+_POINT_NUMBERS = {}
+
+
+def _point_numbers(B: int, E: int, device) -> torch.Tensor:
+    """``[B, E]`` int32, every row ``0 .. E-1`` (kept per shape: the sweep only reads it)."""
+    key = (B, E, str(device))
+    if key not in _POINT_NUMBERS:
+        _POINT_NUMBERS.clear()
+        _POINT_NUMBERS[key] = torch.arange(E, dtype=torch.int32, device=device).expand(B, E).contiguous()
+    return _POINT_NUMBERS[key]
+
+
 def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, grad_ys, params):
     """All iterations in reverse in one kernel (tode_solve_builtin_backward): for a built-in term whose forward pass
     left its record in entry-major arrays.  The right-hand side and its vector-Jacobian product are evaluated in the
@@ -394,8 +406,13 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
         hit = torch.where(hit < L, hit, torch.full_like(hit, -1))
         hit[:, 0] = torch.where(t_eval[:, 0] == t_start, torch.full_like(hit[:, 0], -1), hit[:, 0])
         # ordered by iteration, so that the kernel, walking the iterations down, finds each one's points at a cursor
-        iterations_sorted, points_by_iteration = torch.sort(hit.to(torch.int32), dim=1, stable=True)
-        iterations_sorted, points_by_iteration = iterations_sorted.contiguous(), points_by_iteration.to(torch.int32).contiguous()
+        hit = hit.to(torch.int32)
+        if E == 1 or bool((hit[:, 1:] >= hit[:, :-1]).all()):
+            # evaluation times in the direction of the solve, every one of them reached: already in order
+            iterations_sorted, points_by_iteration = hit.contiguous(), _point_numbers(B, E, dev)
+        else:
+            iterations_sorted, points_by_iteration = torch.sort(hit, dim=1, stable=True)
+            iterations_sorted, points_by_iteration = iterations_sorted.contiguous(), points_by_iteration.to(torch.int32).contiguous()
     wants = lambda x: x is not None and x.requires_grad
     g_t_start = zeros(B) if wants(replay.t_start) else None
     g_t_end = zeros(B) if wants(replay.t_end) else None
@@ -422,6 +439,12 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     scratch = torch.empty(max(lib.tode_solve_backward_scratch_bytes(_lib.C.byref(a)), 1), dtype=torch.uint8, device=dev)
     ad = _lib.SolveAdjoint()
     ad.grad_ys, ad.iterations, ad.through_control = grad.data_ptr(), L, int(bool(replay.through_control))
+    # the start of the loop in the kernel too, unless a time wants a gradient (the kernel takes the times of that part
+    # as constants): what comes back is then the cotangent of y0 itself
+    through_start = getattr(adjoint, "backward_start_in_kernel", True) and not any(wants(x) for x in (replay.t_start, replay.t_end, replay.t_eval, dt0))
+    ad.through_start = int(through_start)
+    if dt0 is not None:
+        a.dt0 = dt0.data_ptr()  # (not read: it says that the first step was given)
     ad.points_by_iteration, ad.iterations_sorted = _lib.ptr(points_by_iteration), _lib.ptr(iterations_sorted)
     ad.scratch, ad.scratch_bytes = scratch.data_ptr(), scratch.numel()
     ad.a_y, ad.a_k0 = out_y.data_ptr(), out_k0.data_ptr()
@@ -450,7 +473,7 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
             if q is given:
                 grad_params[j] = _add(grad_params[j], collected.to(q.dtype))
                 break
-    adj = dict(y=out_y, k0=out_k0, t=out_s[0], dt=out_s[1], prev=out_s[2], pprev=out_s[3])
+    adj = dict(y=out_y, k0=out_k0, t=out_s[0], dt=out_s[1], prev=out_s[2], pprev=out_s[3], through_start=through_start)
     return adj, grad_params
 
 
@@ -685,6 +708,21 @@ class SolveThroughLoop(torch.autograd.Function):
                 adj, grad_params = reverse_sweep_torch(replay, states, hits, grad_ys, params)
 
         # ---- the start of the loop: y = y0, k0 = f(t_start, y0), dt from the start step rule or dt0 ----
+        if adj.get("through_start"):  # (the whole-sweep kernel went through it as well)
+            grad_y0 = adj["y"]
+        else:
+            grad_y0 = SolveThroughLoop.start_backward(ctx, replay, adj, y0, dt0, params, grad_params)
+        if E > 0:
+            at_start = problem.t_eval[:, 0] == problem.t_start
+            first = torch.where(at_start[:, None], grad_ys[:, 0], torch.zeros_like(grad_ys[:, 0]))
+            grad_y0 = add(grad_y0, first)
+        return (None, None, None, None, None, grad_y0, *grad_params)
+
+    @staticmethod
+    def start_backward(ctx, replay, adj, y0, dt0, params, grad_params):
+        """The cotangents of the first loop state carried on to ``y0`` (returned) and to ``params`` (added into
+        ``grad_params``) by autograd over the start of the loop written as torch operations."""
+        add = _add
         with torch.enable_grad():
             y_in = y0.detach().requires_grad_()
             targets, cotangents = [], []
@@ -712,11 +750,7 @@ class SolveThroughLoop(torch.autograd.Function):
                 grad_y0 = grads[0]
                 for i, g in enumerate(grads[1:]):
                     grad_params[i] = add(grad_params[i], g)
-        if E > 0:
-            at_start = problem.t_eval[:, 0] == problem.t_start
-            first = torch.where(at_start[:, None], grad_ys[:, 0], torch.zeros_like(grad_ys[:, 0]))
-            grad_y0 = add(grad_y0, first)
-        return (None, None, None, None, None, grad_y0, *grad_params)
+        return grad_y0
 
 
 def solve(adjoint, problem: InitialValueProblem, term, dt0: Optional[torch.Tensor], args: Any):

@@ -61,12 +61,14 @@ template <bool WAVE, typename T> __device__ __forceinline__ T row_sum(T v) {
 // (the body of finish_backward_kernel for sample b; f_first / f_step: the features this thread walks)
 // points / n_listed: the evaluation points this iteration wrote, where the caller knows them (n_listed >= 0); else
 // every point of the row is looked at and those with hit_iteration == iteration are taken.
-template <typename TT, typename T, int METHOD, int CTRL, bool WAVE>
+// FC: the row length where the caller knows it at compile time (0: p.F).  With FC set, b == 0 and every per-sample
+// array a thread-private one, all indices are constants and the arrays can live in registers.
+template <typename TT, typename T, int METHOD, int CTRL, bool WAVE, int FC = 0>
 __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T> &p, const long long b, const int f_first, const int f_step,
                                                        const int32_t *points = nullptr, const int n_listed = -1) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     const bool scalar_lane = f_first == 0;
-    const int F = p.F, E = p.E;
+    const int F = FC > 0 ? FC : p.F, E = p.E;
     const CtrlParams<T> &cp = p.cp;
     const TT t0 = p.t[b], dt = p.dt[b];
     const T h = (T)dt;
@@ -77,8 +79,10 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
 
     // ---- forward values of the controller ----
     T acc = 0;
+#pragma unroll
     for (int f = f_first; CTRL != 2 && f < F; f += f_step) {
         T err = 0;
+#pragma unroll
         for (int s = 0; s < 7; ++s) err = fma_(h * (T)Tab::b_err[s], p.k[s][b * F + f], err);
         const T m = tmax(abs_(y[f]), abs_(y1[f]));
         const T x = (abs_(err) / fma_(cp.rtol, m, cp.atol)) / sf;
@@ -160,6 +164,7 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
     const T tiny = (T)1e-38;
     const T g_r = r > tiny ? g_ratio : (r == tiny ? g_ratio / (T)2 : (T)0);
     T g_h = 0;  // (this lane's share; summed over the row at the end)
+#pragma unroll
     for (int f = f_first; f < F; f += f_step) {
         const long long i = b * F + f;
         const T a_y = p.a_y ? p.a_y[i] : (T)0, a_k0 = p.a_k0 ? p.a_k0[i] : (T)0;
@@ -167,6 +172,7 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
         T gk[7] = {move ? (T)0 : a_k0, 0, 0, 0, 0, 0, move ? a_k0 : (T)0};
         if (CTRL != 2 && g_r != (T)0 && r > (T)0) {
             T err = 0, bk = 0;
+#pragma unroll
             for (int s = 0; s < 7; ++s) {
                 err = fma_(h * (T)Tab::b_err[s], p.k[s][i], err);
                 bk = fma_((T)Tab::b_err[s], p.k[s][i], bk);
@@ -181,11 +187,13 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
             max_backward<T>(ay, ay1, g_m, ga, gb);
             gy += ga * sign_(y[f]);
             gy1 += gb * sign_(y1[f]);
+#pragma unroll
             for (int s = 0; s < 7; ++s) gk[s] += g_err * (h * (T)Tab::b_err[s]);
             g_h += g_err * bk;
         }
         p.g_y[i] = gy;
         p.g_y1[i] = gy1;
+#pragma unroll
         for (int s = 0; s < 7; ++s) p.g_k[s][i] = gk[s];
     }
 
@@ -201,11 +209,13 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
         const TT at = E > 0 ? p.t_eval[b * E + e] : te;
         const T x = (T)((at - t0) / den);
         T g_x = 0;
+#pragma unroll
         for (int f = f_first; f < F; f += f_step) {
             const long long i = b * F + f;
             const T g = p.grad_ys[(b * (long long)(E > 0 ? E : 1) + e) * F + f];
             if (g == (T)0) continue;
             T ks[7];
+#pragma unroll
             for (int s = 0; s < 7; ++s) ks[s] = p.k[s][i];
             // coefficients (lowest power first) and their cotangents g x^p
             T q[5][1];
@@ -216,6 +226,7 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
                 p.g_y[i] += g0;
                 p.g_k[0][i] += g1 * h;
                 g_h += g1 * ks[0];
+#pragma unroll
                 for (int s = 0; s < 7; ++s) {
                     const T w = g2 * (T)Tsit5Tab::w[0][s] + g3 * (T)Tsit5Tab::w[1][s] + g4 * (T)Tsit5Tab::w[2][s];
                     p.g_k[s][i] += w * h;
@@ -229,6 +240,7 @@ __device__ __forceinline__ void finish_backward_sample(const AdjointParams<TT, T
                 p.g_k[0][i] += g_f0 * h;
                 p.g_k[6][i] += g_f1 * h;
                 g_h += g_f0 * ks[0] + g_f1 * ks[6];
+#pragma unroll
                 for (int s = 0; s < 7; ++s) {
                     p.g_k[s][i] += g_mid * (h * (T)Dopri5Tab::w[0][s]);
                     g_h += g_mid * (T)Dopri5Tab::w[0][s] * ks[s];
@@ -262,20 +274,23 @@ template <typename TT, typename T, int METHOD, int CTRL, bool WAVE> __global__ v
 }
 
 // Stage S reversed.  g_ystage [B,F]: cotangent of the stage input; g_tnode [B] (may be null): of its time.
-template <typename TT, typename T, int METHOD, bool WAVE>
+template <typename TT, typename T, int METHOD, bool WAVE, int FC = 0>
 __device__ __forceinline__ void stage_backward_sample(const AdjointParams<TT, T> &p, const long long b, const int S, const T *g_ystage, const TT *g_tnode,
                                                       const int f_first, const int f_step) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
-    const int F = p.F;
+    const int F = FC > 0 ? FC : p.F;
     const T h = (T)p.dt[b];
     T a[7];
+#pragma unroll
     for (int j = 0; j < 7; ++j) a[j] = j < S ? (T)Tab::a[S][j] : (T)0;
     T g_h = 0;
+#pragma unroll
     for (int f = f_first; f < F; f += f_step) {
         const long long i = b * F + f;
         const T g = g_ystage[i];
         p.g_y[i] += g;
         T s = 0;
+#pragma unroll
         for (int j = 0; j < S; ++j) {
             s = fma_(a[j], p.k[j][i], s);
             p.g_k[j][i] += a[j] * h * g;

@@ -7,16 +7,16 @@
 // cotangents of the state after the iteration and of the evaluation points the iteration wrote through everything
 // after the stages (finish_backward_sample), then through the stages from the last to the first, with the
 // right-hand side's own vector-Jacobian product in closed form where the per-iteration path asks autograd for it.
-// The per-sample arrays that the shared reverse functions read and write (stage derivatives, their cotangents,
-// the cotangents of the state) are rows in LDS that only the sample's own thread touches: the functions index them
-// by the sample's number within its workgroup, and every array in global memory is handed to them moved forward by the
-// workgroup's first sample, so that the same index fits.
+// Everything a sample's thread works on -- stage derivatives, their cotangents, the cotangents of the state -- is an
+// array private to the thread, indexed by constants once the shared reverse functions are inlined with the row length
+// known (registers): those functions get index 0 and every array in global memory moved forward to the thread's sample.
+// The record of the next iteration down is loaded while the current one is worked on.
 #include "tode_adjoint.h"
 
 namespace tode {
 
 template <typename T> struct WholeBackward {
-    AdjointParams<T, T> base;  // problem and controller; the per-iteration fields and the LDS rows are set in the kernel
+    AdjointParams<T, T> base;  // problem and controller; the per-iteration fields and the working arrays are set in the kernel
     long long iterations;      // L: the record holds entries 0..L
     const T *rec_t, *rec_dt, *rec_y, *rec_k0, *rec_prev, *rec_pprev;
     const int32_t *rec_running, *rec_n_accepted;
@@ -27,72 +27,184 @@ template <typename T> struct WholeBackward {
     // the evaluation points of every sample ordered by the iteration that wrote them: [B,E] point indices and, in the
     // same order, the iterations (-1 first: points no iteration wrote)
     const int32_t *points_by_iteration, *iterations_sorted;
+    int through_start;  // also carry the cotangents through the start of the loop (start_backward)
+    int dt0_given;      // the first step was the caller's, not the start rule's
 };
 
-// Elements of T per sample in LDS: k_1..k_6, g_k_0..g_k_6, y1, g_ystage, g_y, g_y1, the cotangents of the state after
-// the iteration (a_y, a_k0) [F each]; g_t, g_dt, g_prev, g_pprev, a_t, a_dt, a_prev, a_pprev, moved, running_next [1 each].
-__host__ __device__ constexpr int backward_row_elements(int F) { return (6 + 7 + 1 + 1 + 2 + 2) * F + 10; }
+template <typename T, int F> struct RecordEntry {
+    T t, dt, prev, pprev, y[F], k0[F];
+    int32_t running, n_accepted;
+};
+
+template <typename T, int F> __device__ __forceinline__ RecordEntry<T, F> load_entry(const WholeBackward<T> &w, long long entry, long long sample) {
+    const long long at = entry * w.base.batch + sample;
+    RecordEntry<T, F> r;
+    r.t = w.rec_t[at], r.dt = w.rec_dt[at], r.prev = w.rec_prev[at], r.pprev = w.rec_pprev[at];
+#pragma unroll
+    for (int f = 0; f < F; ++f) r.y[f] = w.rec_y[at * F + f], r.k0[f] = w.rec_k0[at * F + f];
+    r.running = w.rec_running[at], r.n_accepted = w.rec_n_accepted[at];
+    return r;
+}
+
+// cotangent shares of minimum(a, b) (or maximum with the comparison turned round) for operand a: all of it where a
+// is the one taken, half on a tie (torch.minimum / torch.maximum)
+template <typename T> __device__ __forceinline__ T share_of_min(T a, T b) { return a < b ? (T)1 : (a == b ? (T)0.5 : (T)0); }
+template <typename T> __device__ __forceinline__ T share_of_max(T a, T b) { return a > b ? (T)1 : (a == b ? (T)0.5 : (T)0); }
+
+// cotangent of v given that of rms(v) = |v / sqrt(F)|_2 (zero where the norm is zero, as torch.linalg.vector_norm)
+template <typename T, int F> __device__ __forceinline__ void rms_backward(const T (&v)[F], T norm, T g, T (&gv)[F]) {
+    const T sf = (T)__builtin_sqrt((double)F);
+#pragma unroll
+    for (int f = 0; f < F; ++f) gv[f] = norm != (T)0 ? (g * ((v[f] / sf) / norm)) / sf : (T)0;
+}
+
+// The start of the loop reversed: y = y0, k0 = f(t_start, y0) and, unless the caller gave the first step, the step of
+// the start rule (step_size_controllers.py:431-490 / 776-835, written out in initial_step) clamped to the time range
+// (adjoints.py:86-93).  In: the cotangents a_y, a_k0, a_dt of that first loop state.  Out: a_y becomes the cotangent
+// of y0, gpar gains the right-hand side's parameters' share.  The times are constants here (a caller that wants their
+// gradients takes the first state's cotangents and does this part itself), and the right-hand side does not depend
+// on t (none of the built-in ones does).
+template <typename T, int CTRL, typename Term>
+__device__ __forceinline__ void start_backward(const CtrlParams<T> &cp, const Term &rhs, const bool through_rule, const T ts, const T te,
+                                               const T (&y0)[Term::F], const T (&f0)[Term::F], T (&a_y)[Term::F], const T (&a_k0)[Term::F],
+                                               const T a_dt, T (&gpar)[Term::P]) {
+    constexpr int F = Term::F;
+    T g_y0[F], g_f0[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) g_y0[f] = a_y[f], g_f0[f] = a_k0[f];
+    if (through_rule && a_dt != (T)0) {
+        // ---- forward values (initial_step) ----
+        const T dir = te > ts ? (T)1 : (T)-1, span = abs_(te - ts);
+        T inv[F], u[F], v[F], w[F], y1[F], f1[F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) inv[f] = (T)1 / fma_(cp.rtol, abs_(y0[f]), cp.atol), u[f] = y0[f] * inv[f], v[f] = f0[f] * inv[f];
+        const T d0 = rms<T, F>(u), d1 = rms<T, F>(v);
+        const bool small = d0 < (T)1e-5 || d1 < (T)1e-5;
+        const T h0a = small ? (T)1e-6 : ((T)0.01 * d0) / d1;
+        const T h0 = tmin(h0a, span);
+        const T dh = dir * h0;
+#pragma unroll
+        for (int f = 0; f < F; ++f) y1[f] = fma_(dh, f0[f], y0[f]);
+        const T t1 = fma_(dir, h0, ts);
+        rhs(t1, y1, f1);
+#pragma unroll
+        for (int f = 0; f < F; ++f) w[f] = (f1[f] - f0[f]) * inv[f];
+        const T r2 = rms<T, F>(w);
+        const bool blocked = CTRL == 0 && h0 == (T)0;  // (the integral controller's copy of the rule: d2 = inf)
+        const T d2 = blocked ? (T)__builtin_huge_val() : r2 / h0;
+        const T m = tmax(d1, d2);
+        const bool tiny = m <= (T)1e-15;
+        const T z = ((T)1 / m) * (T)0.01;
+        const T h1 = tiny ? tmax((T)1e-6, h0 * (T)1e-3) : rpow<T>(z, 1.0 / 5.0);
+        const T first = dir * tmin((T)100 * h0, h1);
+        const T lo = tmin(ts, te) - ts, hi = tmax(te, ts) - ts;
+        // ---- reversed ----
+        const T g_first = a_dt * share_of_min<T>(tmax(first, lo), hi) * share_of_max<T>(first, lo);
+        const T g_min = g_first * dir;
+        T g_h0 = (T)100 * (g_min * share_of_min<T>((T)100 * h0, h1));
+        const T g_h1 = g_min * share_of_min<T>(h1, (T)100 * h0);
+        T g_d1 = 0, g_d2 = 0;
+        if (tiny) {
+            g_h0 += (h0 * (T)1e-3 >= (T)1e-6) ? g_h1 * (T)1e-3 : (T)0;
+        } else {
+            const T g_z = g_h1 * ((T)(1.0 / 5.0) * rpow<T>(z, 1.0 / 5.0 - 1.0));
+            const T rm = (T)1 / m;
+            const T g_m = -(g_z * (T)0.01) * rm * rm;
+            g_d1 = g_m * share_of_max<T>(d1, d2);
+            g_d2 = g_m * share_of_max<T>(d2, d1);
+        }
+        T g_inv[F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) g_inv[f] = 0;
+        if (!blocked && g_d2 != (T)0) {
+            const T g_r2 = g_d2 / h0;
+            g_h0 += -g_d2 * r2 / (h0 * h0);
+            T g_w[F], g_f1[F], g_y1[F];
+            rms_backward<T, F>(w, r2, g_r2, g_w);
+#pragma unroll
+            for (int f = 0; f < F; ++f) g_f1[f] = g_w[f] * inv[f], g_f0[f] -= g_w[f] * inv[f], g_inv[f] += g_w[f] * (f1[f] - f0[f]);
+            rhs.vjp(t1, y1, g_f1, g_y1, gpar);
+            T g_step = 0;
+#pragma unroll
+            for (int f = 0; f < F; ++f) g_y0[f] += g_y1[f], g_f0[f] += g_y1[f] * dh, g_step += g_y1[f] * f0[f];
+            g_h0 += g_step * dir;
+        }
+        const T g_h0a = g_h0 * share_of_min<T>(h0a, span);
+        if (!small) {
+            const T q = (T)0.01 * d0;
+            g_d1 += -g_h0a * q / (d1 * d1);
+            const T g_d0 = (T)0.01 * (g_h0a / d1);
+            T g_u[F];
+            rms_backward<T, F>(u, d0, g_d0, g_u);
+#pragma unroll
+            for (int f = 0; f < F; ++f) g_y0[f] += g_u[f] * inv[f], g_inv[f] += g_u[f] * y0[f];
+        }
+        {
+            T g_v[F];
+            rms_backward<T, F>(v, d1, g_d1, g_v);
+#pragma unroll
+            for (int f = 0; f < F; ++f) g_f0[f] += g_v[f] * inv[f], g_inv[f] += g_v[f] * f0[f];
+        }
+#pragma unroll
+        for (int f = 0; f < F; ++f) g_y0[f] += (-g_inv[f] * inv[f] * inv[f]) * cp.rtol * sign_(y0[f]);
+    }
+    T g_from_f0[F];
+    rhs.vjp(ts, y0, g_f0, g_from_f0, gpar);
+#pragma unroll
+    for (int f = 0; f < F; ++f) a_y[f] = g_y0[f] + g_from_f0[f];
+}
 
 template <typename T, int METHOD, int CTRL, typename Term>
-__global__ void __launch_bounds__(256) whole_backward_kernel(const WholeBackward<T> w) {
+__global__ void __launch_bounds__(64) whole_backward_kernel(const WholeBackward<T> w) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F, P = Term::P;
-    extern __shared__ __align__(16) unsigned char lds_raw[];
     const long long B = w.base.batch;
-    const int n = blockDim.x;                        // samples of this workgroup
-    const long long b0 = (long long)blockIdx.x * n;  // its first sample
-    const int b = threadIdx.x;                       // the sample's number within the workgroup: the index the shared functions use
-    if (b0 + b >= B) return;
+    const long long g = (long long)blockIdx.x * 64 + threadIdx.x;  // this thread's sample
+    if (g >= B) return;
     Term rhs;
-    rhs.load(w.params + (b0 + b) * P, w.scalars);
+    rhs.load(w.params + g * P, w.scalars);
     T gpar[P];
 #pragma unroll
     for (int j = 0; j < P; ++j) gpar[j] = 0;
 
-    // ---- the rows in LDS, [n, F] or [n] each ----
-    T *lds = reinterpret_cast<T *>(lds_raw);
-    auto rows = [&](int per_sample) {
-        T *at = lds;
-        lds += per_sample * n;
-        return at;
-    };
-    AdjointParams<T, T> q = w.base;  // (a_* start as null pointers: zeros behind the last iteration)
-    T *k_rows[7];
-    for (int s = 1; s < 7; ++s) k_rows[s] = rows(F), q.k[s] = k_rows[s];
-    for (int s = 0; s < 7; ++s) q.g_k[s] = rows(F);
-    T *y1_row = rows(F), *g_ystage = rows(F);
-    q.y1 = y1_row, q.g_y = rows(F), q.g_y1 = rows(F);
-    T *a_y = rows(F), *a_k0 = rows(F);
-    q.g_t = rows(1), q.g_dt = rows(1), q.g_prev = rows(1), q.g_pprev = rows(1);
-    T *a_t = rows(1), *a_dt = rows(1), *a_prev = rows(1), *a_pprev = rows(1);
-    int32_t *moved = reinterpret_cast<int32_t *>(rows(1)), *running_next = reinterpret_cast<int32_t *>(rows(1));
-    q.moved = moved, q.running_next = running_next;
-    // ---- what lives in global memory, moved forward to the workgroup's first sample ----
+    // ---- the thread's own arrays; the shared functions reach them through q with index 0 ----
+    T k[7][F], g_k[7][F], y[F], y1[F], g_ystage[F], g_y[F], g_y1[F], a_y[F], a_k0[F];
+    T t0 = 0, dt = 0, prev = 1, pprev = 1, g_t = 0, g_dt = 0, g_prev = 0, g_pprev = 0;
+    T a_t = 0, a_dt = 0, a_prev = 0, a_pprev = 0;  // cotangents of the state after the iteration: zeros behind the last one
+    int32_t moved = 0, running_next = 0;
+#pragma unroll
+    for (int f = 0; f < F; ++f) a_y[f] = 0, a_k0[f] = 0;
+    AdjointParams<T, T> q = w.base;
+#pragma unroll
+    for (int s = 0; s < 7; ++s) q.k[s] = k[s], q.g_k[s] = g_k[s];
+    q.t = &t0, q.dt = &dt, q.y = y, q.y1 = y1, q.prev = &prev, q.pprev = &pprev;
+    q.moved = &moved, q.running_next = &running_next;
+    q.g_y = g_y, q.g_y1 = g_y1, q.g_t = &g_t, q.g_dt = &g_dt, q.g_prev = &g_prev, q.g_pprev = &g_pprev;
+    q.a_y = a_y, q.a_k0 = a_k0, q.a_t = &a_t, q.a_dt = &a_dt, q.a_prev = &a_prev, q.a_pprev = &a_pprev;
+    // ---- what lives in global memory, moved forward to this sample ----
     const int E = q.E;
-    q.t_start += b0, q.t_end += b0;
-    if (q.t_eval) q.t_eval += b0 * E;
-    q.grad_ys += b0 * (long long)(E > 0 ? E : 1) * F;
-    if (q.g_t_start) q.g_t_start += b0;
-    if (q.g_t_end) q.g_t_end += b0;
-    if (q.g_t_eval) q.g_t_eval += b0 * E;
-    const int32_t *iterations_sorted = w.iterations_sorted + b0 * E, *points_by_iteration = w.points_by_iteration + b0 * E;
+    q.t_start += g, q.t_end += g;
+    if (q.t_eval) q.t_eval += g * E;
+    q.grad_ys += g * (long long)(E > 0 ? E : 1) * F;
+    if (q.g_t_start) q.g_t_start += g;
+    if (q.g_t_end) q.g_t_end += g;
+    if (q.g_t_eval) q.g_t_eval += g * E;
+    const int32_t *iterations_sorted = w.iterations_sorted + g * E, *points_by_iteration = w.points_by_iteration + g * E;
 
+    const long long L = w.iterations;
     int cursor = E - 1;  // into the sample's points ordered by iteration, walked from the end as the iterations are
-    for (long long i = w.iterations - 1; i >= 0; --i) {
-        const long long at = i * B + b0, next = (i + 1) * B + b0;
+    RecordEntry<T, F> after = load_entry<T, F>(w, L, g), here = load_entry<T, F>(w, L > 0 ? L - 1 : 0, g);
+    for (long long i = L - 1; i >= 0; --i) {
+        const RecordEntry<T, F> before = load_entry<T, F>(w, i > 0 ? i - 1 : 0, g);  // (used by the next pass of this loop)
         q.iteration = (int)i;
-        q.end_point = (E == 0 && i == w.iterations - 1) ? 1 : 0;
-        q.t = w.rec_t + at, q.dt = w.rec_dt + at, q.y = w.rec_y + at * F;
-        q.prev = w.rec_prev + at, q.pprev = w.rec_pprev + at;
-        q.k[0] = w.rec_k0 + at * F;
-        moved[b] = (w.rec_n_accepted[next + b] - w.rec_n_accepted[at + b]) > 0 ? 1 : 0;
-        running_next[b] = w.rec_running[next + b] != 0 ? 1 : 0;
+        q.end_point = (E == 0 && i == L - 1) ? 1 : 0;
+        t0 = here.t, dt = here.dt, prev = here.prev, pprev = here.pprev;
+        moved = (after.n_accepted - here.n_accepted) > 0 ? 1 : 0;
+        running_next = after.running != 0 ? 1 : 0;
 
         // ---- the stages again (runge_kutta.py:255-263) ----
-        const T t0 = q.t[b], dt = q.dt[b];
-        T y[F], k[7][F];
 #pragma unroll
-        for (int f = 0; f < F; ++f) y[f] = q.y[b * F + f], k[0][f] = q.k[0][b * F + f];
+        for (int f = 0; f < F; ++f) y[f] = here.y[f], k[0][f] = here.k0[f];
 #pragma unroll
         for (int s = 1; s < 7; ++s) {
             T yi[F];
@@ -104,49 +216,48 @@ __global__ void __launch_bounds__(256) whole_backward_kernel(const WholeBackward
                 yi[f] = fma_(dt, sum, y[f]);
             }
             rhs(fma_((T)Tab::c[s], dt, t0), yi, k[s]);
-#pragma unroll
-            for (int f = 0; f < F; ++f) k_rows[s][b * F + f] = k[s][f];
             if (s == 6) {
 #pragma unroll
-                for (int f = 0; f < F; ++f) y1_row[b * F + f] = yi[f];
+                for (int f = 0; f < F; ++f) y1[f] = yi[f];
             }
         }
 
         // ---- everything after the stages, reversed ----
         int n_here = 0;
-        while (cursor - n_here >= 0 && iterations_sorted[b * E + cursor - n_here] == (int)i) ++n_here;
+        while (cursor - n_here >= 0 && iterations_sorted[cursor - n_here] == (int)i) ++n_here;
         cursor -= n_here;
-        finish_backward_sample<T, T, METHOD, CTRL, false>(q, b, 0, 1, points_by_iteration + b * E + cursor + 1, n_here);
+        finish_backward_sample<T, T, METHOD, CTRL, false, F>(q, 0, 0, 1, points_by_iteration + cursor + 1, n_here);
 
         // ---- the stages reversed ----
 #pragma unroll
         for (int s = 6; s >= 1; --s) {
-            T yi[F], g[F], gy[F];
+            T yi[F], gk[F], gy[F];
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 T sum = 0;
 #pragma unroll
                 for (int j = 0; j < s; ++j) sum = fma_((T)Tab::a[s][j], k[j][f], sum);
                 yi[f] = fma_(dt, sum, y[f]);
-                g[f] = q.g_k[s][b * F + f];
+                gk[f] = g_k[s][f];
             }
-            rhs.vjp(fma_((T)Tab::c[s], dt, t0), yi, g, gy, gpar);
+            rhs.vjp(fma_((T)Tab::c[s], dt, t0), yi, gk, gy, gpar);
 #pragma unroll
-            for (int f = 0; f < F; ++f) g_ystage[b * F + f] = gy[f] + (s == 6 ? q.g_y1[b * F + f] : (T)0);
-            stage_backward_sample<T, T, METHOD, false>(q, b, s, g_ystage, (const T *)nullptr, 0, 1);
+            for (int f = 0; f < F; ++f) g_ystage[f] = gy[f] + (s == 6 ? g_y1[f] : (T)0);
+            stage_backward_sample<T, T, METHOD, false, F>(q, 0, s, g_ystage, (const T *)nullptr, 0, 1);
         }
 
         // ---- the cotangents of the state before this iteration are those behind the one before it ----
 #pragma unroll
-        for (int f = 0; f < F; ++f) a_y[b * F + f] = q.g_y[b * F + f], a_k0[b * F + f] = q.g_k[0][b * F + f];
-        a_t[b] = q.g_t[b], a_dt[b] = q.g_dt[b], a_prev[b] = q.g_prev[b], a_pprev[b] = q.g_pprev[b];
-        q.a_y = a_y, q.a_k0 = a_k0, q.a_t = a_t, q.a_dt = a_dt, q.a_prev = a_prev, q.a_pprev = a_pprev;
+        for (int f = 0; f < F; ++f) a_y[f] = g_y[f], a_k0[f] = g_k[0][f];
+        a_t = g_t, a_dt = g_dt, a_prev = g_prev, a_pprev = g_pprev;
+        after = here, here = before;
     }
-    const bool any = w.iterations > 0;  // (no iteration: nothing flows back through the loop)
-    const long long g = b0 + b;
+    // (no iteration: nothing flows back through the loop, and the cotangents are still the zeros they started as)
+    if (w.through_start)  // (`here` is the record's first entry now: t_start, y0, f(t_start, y0))
+        start_backward<T, CTRL, Term>(q.cp, rhs, q.through_control && !w.dt0_given, q.t_start[0], q.t_end[0], here.y, here.k0, a_y, a_k0, a_dt, gpar);
 #pragma unroll
-    for (int f = 0; f < F; ++f) w.a_y[g * F + f] = any ? a_y[b * F + f] : (T)0, w.a_k0[g * F + f] = any ? a_k0[b * F + f] : (T)0;
-    w.a_t[g] = any ? a_t[b] : (T)0, w.a_dt[g] = any ? a_dt[b] : (T)0, w.a_prev[g] = any ? a_prev[b] : (T)0, w.a_pprev[g] = any ? a_pprev[b] : (T)0;
+    for (int f = 0; f < F; ++f) w.a_y[g * F + f] = a_y[f], w.a_k0[g * F + f] = a_k0[f];
+    w.a_t[g] = a_t, w.a_dt[g] = a_dt, w.a_prev[g] = a_prev, w.a_pprev[g] = a_pprev;
 #pragma unroll
     for (int j = 0; j < P; ++j) w.g_params[g * P + j] = gpar[j];
 }
@@ -172,14 +283,9 @@ static int launch_backward(const tode_solve_args &a, const tode_controller &c, c
     for (int i = 0; i < 4; ++i) w.scalars[i] = a.term_scalars[i];
     w.g_params = (T *)adj.g_params;
     w.points_by_iteration = adj.points_by_iteration, w.iterations_sorted = adj.iterations_sorted;
+    w.through_start = adj.through_start, w.dt0_given = a.dt0 != nullptr;
     // (the t_start / t_end strides of the forward entry point are not taken here: the caller passes dense arrays)
-    // samples per workgroup: whole wavefronts, as many as 48 KiB of LDS rows hold, at most 256
-    const size_t row_bytes = (size_t)backward_row_elements(F) * sizeof(T);
-    int threads = (int)((48 * 1024) / row_bytes) / 64 * 64;
-    threads = threads > 256 ? 256 : (threads < 64 ? 64 : threads);
-    if ((size_t)threads * row_bytes > 64 * 1024)
-        return fail(TODE_E_UNSUPPORTED, "rows of %d values of %d bytes: one wavefront of samples does not fit the sweep's working rows into 64 KiB of LDS", F, (int)sizeof(T));
-    hipLaunchKernelGGL((whole_backward_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)((B + threads - 1) / threads)), dim3(threads), threads * row_bytes, stream, w);
+    hipLaunchKernelGGL((whole_backward_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)((B + 63) / 64)), dim3(64), 0, stream, w);
     return check_hip(hipGetLastError(), "tode_solve_builtin_backward launch");
 }
 
@@ -230,7 +336,7 @@ extern "C" {
 
 int64_t tode_solve_backward_scratch_bytes(const tode_solve_args *a) {
     if (!a || a->n_features <= 0 || a->batch < 0) return -1;
-    return 0;  // (the sweep's working rows live in LDS)
+    return 0;  // (the sweep's working arrays are the threads' own)
 }
 
 int tode_solve_builtin_backward(const tode_solve_args *a, const tode_controller *c, const tode_solve_adjoint *adj, void *stream) {
