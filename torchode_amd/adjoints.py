@@ -643,10 +643,7 @@ class AutoDiffAdjoint(nn.Module):
             again.iteration_cap = L
             again.record = _lib.C.addressof(rec)
             _lib.check(lib.tode_solve_builtin(_lib.C.byref(again), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
-            if flags.tolist()[_lib.FLAG_NEEDS_GENERAL]:
-                raise RuntimeError("the record of the loop state was too short for the solve it was sized from")
-            order = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
-            record.states = [tuple(fields[k][i] for k in order) for i in range(n)]
+            record.flags = flags  # (looked at when the backward pass starts: no second wait for the GPU here)
             record.iterations = L
             record.arrays = fields  # (entry-major arrays: what tode_solve_builtin_backward reads)
         return Solution(ts=ts, ys=ys, stats=stats, status=status)

@@ -112,6 +112,8 @@ class LoopRecord:
     def __init__(self):
         self.states: List[tuple] = []
         self.iterations = 0  # set by the forward pass when the loop has stopped
+        self.arrays = None  # the same record as entry-major arrays, where the whole-solve kernel wrote it
+        self.flags = None  # that kernel's flag words, still on the device
 
     def snapshot(self, t, dt, y, k0, hist, ints):
         self.states.append((t.clone(), dt.clone(), y.clone(), k0.clone(), hist[0].clone(), hist[1].clone(), ints[0].clone(), ints[3].clone()))
@@ -126,6 +128,8 @@ class LoopRecord:
 
     def trimmed(self, iterations: int) -> List[dict]:
         """States 0..iterations; iterations enqueued after the batch had stopped changed nothing."""
+        if not self.states and self.arrays is not None:  # (views of the arrays, made when a per-iteration sweep asks)
+            self.states = [tuple(self.arrays[k][i] for k in self.FIELDS) for i in range(self.arrays["t"].shape[0])]
         states = self.states[:iterations] + [self.states[-1]]
         return [dict(zip(self.FIELDS, s)) for s in states]
 
@@ -662,6 +666,8 @@ class SolveThroughLoop(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_ys, *unused):
         adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
+        if ctx.record.flags is not None and ctx.record.flags.tolist()[_lib.FLAG_NEEDS_GENERAL]:
+            raise RuntimeError("the record of the loop state was too short for the solve it was sized from")
         # The sweep works on leaves of its own for the times and the tensors in args: one of them may be computed
         # from another (t_start is usually a column of t_eval), and a gradient taken with respect to both would
         # reach the first one twice, once here and once when autograd carries the second one's gradient on.
