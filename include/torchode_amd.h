@@ -125,8 +125,9 @@ typedef struct tode_controller {
  * tode_finalize_stats.
  */
 /*
- * Optional record of the loop state, written by tode_solve_builtin (the general kernel) when
- * tode_solve_args.record points to one: entry i holds what the reference's loop variables hold before iteration i
+ * Optional record of the loop state, written by tode_solve_builtin (the general kernel) and, for the three small
+ * systems with evaluation points, by tode_solve_builtin_fast and its _sync / _static forms (the single-wavefront
+ * kernel: the solve and its record in one launch) when tode_solve_args.record points to one: entry i holds what the reference's loop variables hold before iteration i
  * (adjoints.py:135-260: t, dt, y, the first-same-as-last derivative, the PID controller's two previous error
  * ratios, `running`, `n_accepted`), entry n_steps[b] the sample's final state, and the entries after it that final
  * state again with running = 0 -- a finished sample keeps its state while the batch goes on.  It is what a reverse
@@ -136,7 +137,8 @@ typedef struct tode_controller {
  * prev, pprev [capacity, B] in the data type; running, n_accepted [capacity, B] int32.  capacity must be at least
  * 1 + the iterations the solve takes (args->iteration_cap + 1 when a cap is set, which is how a caller that has
  * solved the problem once sizes it); a sample whose steps do not fit stops recording and raises
- * TODE_FLAG_NEEDS_GENERAL in the flag block.
+ * TODE_FLAG_NEEDS_GENERAL in the flag block.  A caller without that count gives the fast entry point a record sized
+ * from a similar solve and repeats the solve if the flag comes back (TODE_FLAG_MAX_ITERATIONS then says what fits).
  */
 typedef struct tode_solve_record {
     int64_t capacity;
@@ -178,8 +180,9 @@ typedef struct tode_solve_args {
     int32_t *status_last;      /* out [B] status at the sample's last own iteration */
     int32_t *status_idle;      /* out [B] status the sample reports in later iterations */
     int32_t *flags;            /* out [TODE_FLAG_WORDS] */
-    const tode_solve_record *record; /* NULL, or where tode_solve_builtin keeps the loop state of every iteration
-                                        (HOST pointer to the struct; every other entry point ignores it) */
+    const tode_solve_record *record; /* NULL, or where tode_solve_builtin / tode_solve_builtin_fast keep the loop state
+                                        of every iteration (HOST pointer to the struct; tode_solve_builtin_auto
+                                        ignores it) */
 } tode_solve_args;
 
 /* ABI version of the loaded library (== TODE_ABI_VERSION of the header it was built from). */

@@ -627,17 +627,39 @@ def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
     assert sol_whole is not None and whole.iterations == steps.iterations
     assert whole.iterations > 5 or case == "non-finite"  # (an infinite start value stops the whole batch after its first iteration)
     assert torch.equal(sol_whole.stats["n_steps"], sol_steps.stats["n_steps"]) and torch.equal(sol_whole.status, sol_steps.status)
-    a, b = whole.trimmed(whole.iterations), steps.trimmed(steps.iterations)
-    assert len(a) == len(b) == whole.iterations + 1
-    for i, (sa, sb) in enumerate(zip(a, b)):
-        for key in LoopRecord.FIELDS:
-            x, y = sa[key], sb[key]
-            assert x.dtype == y.dtype and x.shape == y.shape, (i, key)
-            assert bool(((x == y) | ((x != x) & (y != y))).all()), (i, key, (x.double() - y.double()).abs().nan_to_num().max().item())
+
+    def same_record(whole):
+        a, b = whole.trimmed(whole.iterations), steps.trimmed(steps.iterations)
+        assert len(a) == len(b) == whole.iterations + 1
+        for i, (sa, sb) in enumerate(zip(a, b)):
+            for key in LoopRecord.FIELDS:
+                x, y = sa[key], sb[key]
+                assert x.dtype == y.dtype and x.shape == y.shape, (i, key)
+                assert bool(((x == y) | ((x != x) & (y != y))).all()), (i, key, (x.double() - y.double()).abs().nan_to_num().max().item())
+
+    same_record(whole)
     if case == "max-steps":
         assert (sol_whole.status == 3).any()
     if case == "non-finite":
         assert (sol_whole.status != 0).any()
+    # The same solver again: it now knows how many entries such a record takes, and where the batch is in the
+    # single-wavefront kernel's case that kernel writes the solve and the record in one launch (no flag words left
+    # behind by a second pass).  Then with a record sized far too short, which sends it the long way again.
+    in_one_kernel_case = case in ("vdp-f32", "vdp-f64", "lorenz-f32", "linear-decay-f64", "dt0", "backwards")
+    for entries, one_kernel in ((None, in_one_kernel_case), (3, False)):
+        if entries is not None:
+            solver._record_entries = entries
+        again = LoopRecord()
+        with torch.no_grad():
+            sol_again = solver._solve_persistent(problem, to.ODETerm(f), dt0, record=again)
+        assert (again.flags is None) == one_kernel, (entries, again.flags)
+        assert again.iterations == steps.iterations
+        E_ = sol_whole.ys.shape[1]
+        written = (torch.arange(E_, device="cuda")[None, :] < sol_whole.stats["n_initialized"][:, None])[:, :, None] if t_eval is not None else True
+        blank = lambda ys: torch.where(written, ys, torch.zeros_like(ys)) if t_eval is not None else ys
+        for x, y in ((blank(sol_again.ys), blank(sol_whole.ys)), (sol_again.status, sol_whole.status)) + tuple((sol_again.stats[k], sol_whole.stats[k]) for k in sol_whole.stats):
+            assert bool(((x == y) | ((x != x) & (y != y))).all())
+        same_record(again)
 
 
 @gpu

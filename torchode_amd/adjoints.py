@@ -603,7 +603,7 @@ class AutoDiffAdjoint(nn.Module):
                         keep=(params, dt0_, shared))  # fmt: skip
         elif held["scalars"] != tuple((list(getattr(f, "builtin_scalars", lambda: ())()) + [0.0] * 4)[:4]):
             held.clear()  # (a scalar of the term was reassigned: describe the call anew)
-            return self._solve_persistent(problem, term, dt0)
+            return self._solve_persistent(problem, term, dt0, record=record)
         a = _lib.SolveArgs.from_buffer_copy(held["args"])  # (a copy per call: solves of one problem object may overlap in threads)
         a.ys = ys.data_ptr()
         a_ref = _lib.C.byref(a)
@@ -612,6 +612,14 @@ class AutoDiffAdjoint(nn.Module):
         # the first reported that the batch leaves the common case, the int64 stats as the reference returns them.
         out = torch.empty((4, B), dtype=torch.int64, device=dev)
         o0, row = out.data_ptr(), 8 * B
+        if record is not None:
+            # Once a recording solve of this solver has told how many iterations such a batch takes: the solve and its
+            # record in one kernel, with a record of a few entries more.  A batch that leaves that kernel's case, or
+            # takes more iterations than the record holds, goes the long way below.
+            solution = self._solve_recording_in_one_kernel(lib, a, ctrl, out, stream, record, dict(
+                B=B, E=E, F=F, dtype=dtype, ttype=ttype, dev=dev, ts=ts, ys=ys, has_dt0=dt0 is not None, with_stats=term.with_stats))  # fmt: skip
+            if solution is not None:
+                return solution
         workspace = torch.empty(held["workspace_bytes"], dtype=torch.uint8, device=dev)
         iterations = _lib.C.c_int64(0)
         rc = lib.tode_solve_builtin_auto(
@@ -631,9 +639,7 @@ class AutoDiffAdjoint(nn.Module):
             # state before every iteration: entry i of every array is what the per-step kernels' loop holds there.
             L, n = iterations.value, iterations.value + 1
             new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
-            fields = dict(t=new(n, B, dt=ttype), dt=new(n, B, dt=ttype), y=new(n, B, F), k0=new(n, B, F), prev=new(n, B), pprev=new(n, B),
-                          running=new(n, B, dt=torch.int32), n_accepted=new(n, B, dt=torch.int32))  # fmt: skip
-            rec = _lib.SolveRecord(n, *(fields[k].data_ptr() for k in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")))
+            fields, rec = self._record_arrays(n, B, F, dtype, ttype, dev)
             again = _lib.SolveArgs.from_buffer_copy(a)
             scratch_ys, y_idle = new(B, max(E, 1), F), new(B, F)
             counters, flags = new(5, B, dt=torch.int32), new(_lib.FLAG_WORDS, dt=torch.int32)
@@ -644,9 +650,47 @@ class AutoDiffAdjoint(nn.Module):
             again.record = _lib.C.addressof(rec)
             _lib.check(lib.tode_solve_builtin(_lib.C.byref(again), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
             record.flags = flags  # (looked at when the backward pass starts: no second wait for the GPU here)
+            self._record_entries = n + 4  # (the next recording solve of a batch like this one tries it in one kernel)
             record.iterations = L
             record.arrays = fields  # (entry-major arrays: what tode_solve_builtin_backward reads)
         return Solution(ts=ts, ys=ys, stats=stats, status=status)
+
+    @staticmethod
+    def _record_arrays(n, B, F, dtype, ttype, dev):
+        new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
+        fields = dict(t=new(n, B, dt=ttype), dt=new(n, B, dt=ttype), y=new(n, B, F), k0=new(n, B, F), prev=new(n, B), pprev=new(n, B),
+                      running=new(n, B, dt=torch.int32), n_accepted=new(n, B, dt=torch.int32))  # fmt: skip
+        return fields, _lib.SolveRecord(n, *(fields[k].data_ptr() for k in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")))
+
+    def _solve_recording_in_one_kernel(self, lib, a, ctrl, out, stream, record, q) -> Optional[Solution]:
+        """The solve with its record from the single-wavefront kernel (``tode_solve_builtin_fast`` with a record), or
+        None where that is not to be had: no earlier recording solve to size the record from, a shape or controller
+        setting outside that kernel's case, a batch that leaves it, or a record that came out too short."""
+        n = getattr(self, "_record_entries", None)
+        if n is None or not getattr(self, "record_in_one_kernel", True) or not self.use_fast_path:
+            return None
+        if q["E"] == 0 or q["dtype"] != q["ttype"] or a.term in (_lib.TERM_REACTION_DIFFUSION, _lib.TERM_MLP):
+            return None
+        B = q["B"]
+        fields, rec = self._record_arrays(n, B, q["F"], q["dtype"], q["ttype"], q["dev"])
+        a.record = _lib.C.addressof(rec)
+        fl = (_lib.C.c_int32 * _lib.FLAG_WORDS)()
+        o0, row = out.data_ptr(), 8 * B
+        rc = lib.tode_solve_builtin_fast_sync(_lib.C.byref(a), _lib.C.byref(ctrl), o0, o0 + row, o0 + 2 * row, o0 + 3 * row, stream, fl)
+        a.record = None
+        if rc == _lib.E_UNSUPPORTED:
+            return None
+        _lib.check(rc, "tode_solve_builtin_fast_sync")
+        if fl[_lib.FLAG_NEEDS_GENERAL]:
+            return None
+        L = fl[_lib.FLAG_MAX_ITERATIONS]
+        record.iterations, record.arrays = L, fields
+        self._record_entries = L + 1 + 4
+        stats: Dict[str, Any] = {}
+        if q["with_stats"]:
+            stats["n_f_evals"] = _f_evals((1 if q["has_dt0"] else 2) + 6 * L, B)
+        stats["n_steps"], stats["n_accepted"], stats["n_initialized"], status = out.unbind(0)
+        return Solution(ts=q["ts"], ys=q["ys"], stats=stats, status=status)
 
     def __repr__(self):
         return (

@@ -130,6 +130,7 @@ class LoopRecord:
         """States 0..iterations; iterations enqueued after the batch had stopped changed nothing."""
         if not self.states and self.arrays is not None:  # (views of the arrays, made when a per-iteration sweep asks)
             self.states = [tuple(self.arrays[k][i] for k in self.FIELDS) for i in range(self.arrays["t"].shape[0])]
+            return [dict(zip(self.FIELDS, s)) for s in self.states[: iterations + 1]]
         states = self.states[:iterations] + [self.states[-1]]
         return [dict(zip(self.FIELDS, s)) for s in states]
 

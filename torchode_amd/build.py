@@ -46,6 +46,8 @@ UNITS = [
     ("tode_persistent.hip", "tode_persistent_t32_y64_record.o", ["-DTODE_INSTANTIATE_T32_Y64=1", "-DTODE_INSTANTIATE_RECORD=1"]),
     ("tode_fast.hip", "tode_fast_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_fast.hip", "tode_fast_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
+    ("tode_fast.hip", "tode_fast_f32_record.o", ["-DTODE_INSTANTIATE_F32=1", "-DTODE_INSTANTIATE_RECORD=1"]),
+    ("tode_fast.hip", "tode_fast_f64_record.o", ["-DTODE_INSTANTIATE_F64=1", "-DTODE_INSTANTIATE_RECORD=1"]),
     ("tode_pair.hip", "tode_pair_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_pair.hip", "tode_pair_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
     ("tode_stepwise.hip", "tode_stepwise.o", []),

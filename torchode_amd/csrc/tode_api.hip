@@ -281,6 +281,8 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     hipStream_t s = (hipStream_t)stream;
     if (!known_dtype(a->dtype)) return fail(TODE_E_INVALID, "unknown dtype %d", a->dtype);
     if (a->dtype & TODE_DTYPE_PAIR) return fail(TODE_E_UNSUPPORTED, "the fast entry point is built for time and data in one dtype");
+    if (a->record && (a->term == TODE_TERM_REACTION_DIFFUSION || a->term == TODE_TERM_MLP))
+        return fail(TODE_E_UNSUPPORTED, "a record of the loop state is written for the small systems only");
     if (a->term == TODE_TERM_REACTION_DIFFUSION) {
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for float32");
         return solve_grid_f32(*a, *c, ns, na, ni, st, s);
@@ -288,6 +290,10 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (a->term == TODE_TERM_MLP) {
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the MLP kernel is built for float32");
         return solve_mlp_f32(*a, *c, ns, na, ni, st, s);
+    }
+    if (a->record) {  // the solve and the record of its loop state in one kernel: the single-wavefront kernel writes it
+        if (end_only) return fail(TODE_E_UNSUPPORTED, "a record from the fast entry point needs evaluation points");
+        return a->dtype == TODE_F32 ? solve_fast_f32_record(*a, *c, ns, na, ni, st, s) : solve_fast_f64_record(*a, *c, ns, na, ni, st, s);
     }
     if (g_fast_variant != 1) {
         // small batches: two wavefronts per group of 64 samples (stepper + dense-output evaluator)

@@ -27,7 +27,10 @@ template <typename T> struct FastOut {
 };
 
 // NHIST: how many history factors the controller multiplies in (0 integral, 1 PI, 2 PID).
-template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_YS>
+// RECORD: the loop state before every iteration of the wavefront goes to p.rec_* (tode_solve_record), as the general
+// kernel writes it: entry i is the state before iteration i; a sample that has finished repeats its last state with
+// `running` 0, up to the record's capacity.  A record that is too short raises TODE_FLAG_NEEDS_GENERAL.
+template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_YS, bool RECORD = false>
 __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, const FastOut<T> o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
@@ -125,7 +128,27 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
     const T e1 = (T)cp.e1, e2 = (T)cp.e2, e3 = (T)cp.e3;
     const int step_limit = p.max_steps < TODE_HARD_STEP_LIMIT ? p.max_steps : TODE_HARD_STEP_LIMIT;
 
+    // (RECORD) iterations of this wavefront so far = the record's next entry; the last two accepted error ratios as
+    // values (the step factor keeps their logarithms)
+    long long iteration = 0;
+    T ratio_prev = 1, ratio_prev_prev = 1;
+    bool record_full = false;
+    auto keep = [&](long long at, bool running) {
+        if (at >= p.rec_capacity) {
+            record_full = true;
+            return;
+        }
+        if (!live) return;
+        const long long i = at * p.batch + b;
+        p.rec_t[i] = t, p.rec_dt[i] = dt;
+#pragma unroll
+        for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k[0][f];
+        p.rec_prev[i] = ratio_prev, p.rec_pprev[i] = ratio_prev_prev;
+        p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
+    };
+
     while (__any(active)) {
+        if (RECORD) keep(iteration++, active);
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
         T y1[F], err[F];
@@ -203,6 +226,11 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
             dt = active ? dtc : dt;
         }
         if (NHIST >= 1) step_factor.shift(active && running_new && accept);
+        if (RECORD && CTRL == 1) {
+            const bool shift = active && running_new && accept;
+            ratio_prev_prev = shift ? ratio_prev : ratio_prev_prev;
+            ratio_prev = shift ? ratio : ratio_prev;
+        }
         {
             // non-finite error ratio or max_steps reached: not the common case
             const bool failed = active && (!sane || n_steps >= step_limit);
@@ -225,6 +253,11 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         o.n_accepted[b] = n_acc;
         o.n_initialized[b] = cursor;
         o.status[b] = 0;
+    }
+    if (RECORD) {  // the state every sample is left in, for every later iteration of the batch
+        for (long long at = iteration; at < p.rec_capacity; ++at) keep(at, false);
+        if (iteration >= p.rec_capacity) record_full = true;
+        bail = bail || record_full;
     }
 
     // ---- dense output: one contiguous block of rows * E * F values per wave ----
@@ -281,11 +314,18 @@ static int launch_fast(const tode_solve_args &a, const tode_controller &c, const
     const CtrlParams<T> &cp = p.cp;
     if (cp.shortcut_exponent()) return fail(TODE_E_UNSUPPORTED, "a controller exponent that is not computed through pow: use the general kernel");
     const int nhist = CTRL == 0 ? 0 : (cp.skip3 ? 1 : 2);
-    const bool stage = need_all <= budget;
+    constexpr bool RECORD = TODE_INSTANTIATE_RECORD != 0;
+    if (RECORD != (a.record != nullptr)) return fail(TODE_E_INVALID, "internal: record variant mismatch");
+    if (a.record) {
+        const tode_solve_record &r = *a.record;
+        if (r.capacity < 1 || !r.t || !r.dt || !r.y || !r.k0 || !r.prev || !r.pprev || !r.running || !r.n_accepted)
+            return fail(TODE_E_INVALID, "tode_solve_record: capacity %lld, or a null array", (long long)r.capacity);
+    }
+    const bool stage = !RECORD && need_all <= budget;  // (the recording variant is built without the staged output)
     const size_t lds = stage ? need_all : need_te;
     const dim3 grid((unsigned)blocks), block(64);
     timing_before(stream, "tode::solve_fast_kernel");
-#define TODE_FAST_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
+#define TODE_FAST_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, (ST) && !RECORD, RECORD>), grid, block, lds, stream, p, o)
     if (nhist == 0) {
         if (stage) TODE_FAST_LAUNCH(0, true); else TODE_FAST_LAUNCH(0, false);
     } else if (nhist == 1) {
@@ -332,13 +372,19 @@ static int fast_term(const tode_solve_args &a, const tode_controller &c, int64_t
     }
 }
 
+// (each translation unit instantiates one type, with or without the record: TODE_INSTANTIATE_RECORD)
+#if TODE_INSTANTIATE_RECORD
+#define TODE_FAST_ENTRY(name) name##_record
+#else
+#define TODE_FAST_ENTRY(name) name
+#endif
 #if TODE_INSTANTIATE_F32
-int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+int TODE_FAST_ENTRY(solve_fast_f32)(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
     return fast_term<float>(a, c, ns, na, ni, st, s);
 }
 #endif
 #if TODE_INSTANTIATE_F64
-int solve_fast_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+int TODE_FAST_ENTRY(solve_fast_f64)(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
     return fast_term<double>(a, c, ns, na, ni, st, s);
 }
 #endif
