@@ -648,7 +648,7 @@ def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
     in_one_kernel_case = case in ("vdp-f32", "vdp-f64", "lorenz-f32", "linear-decay-f64", "dt0", "backwards")
     for entries, one_kernel in ((None, in_one_kernel_case), (3, False)):
         if entries is not None:
-            solver._record_entries = entries
+            solver._record_entries = {shape: entries for shape in solver._record_entries}
         again = LoopRecord()
         with torch.no_grad():
             sol_again = solver._solve_persistent(problem, to.ODETerm(f), dt0, record=again)

@@ -650,10 +650,18 @@ class AutoDiffAdjoint(nn.Module):
             again.record = _lib.C.addressof(rec)
             _lib.check(lib.tode_solve_builtin(_lib.C.byref(again), _lib.C.byref(ctrl), stream), "tode_solve_builtin")
             record.flags = flags  # (looked at when the backward pass starts: no second wait for the GPU here)
-            self._record_entries = n + 4  # (the next recording solve of a batch like this one tries it in one kernel)
+            self._remember_record_entries((B, F, E, dtype, f.builtin_kind), n + 4)  # (the next recording solve of a batch like this one tries it in one kernel)
             record.iterations = L
             record.arrays = fields  # (entry-major arrays: what tode_solve_builtin_backward reads)
         return Solution(ts=ts, ys=ys, stats=stats, status=status)
+
+    def _remember_record_entries(self, shape, entries: int) -> None:
+        """How many entries the record of a solve of this shape (batch, features, evaluation points, dtype, term) took,
+        plus a margin: what the next recording solve of that shape sizes its record from.  A few shapes are kept."""
+        held = self.__dict__.setdefault("_record_entries", {})
+        if shape not in held and len(held) >= 8:
+            held.clear()
+        held[shape] = int(entries)
 
     @staticmethod
     def _record_arrays(n, B, F, dtype, ttype, dev):
@@ -666,7 +674,8 @@ class AutoDiffAdjoint(nn.Module):
         """The solve with its record from the single-wavefront kernel (``tode_solve_builtin_fast`` with a record), or
         None where that is not to be had: no earlier recording solve to size the record from, a shape or controller
         setting outside that kernel's case, a batch that leaves it, or a record that came out too short."""
-        n = getattr(self, "_record_entries", None)
+        shape = (q["B"], q["F"], q["E"], q["dtype"], a.term)
+        n = getattr(self, "_record_entries", {}).get(shape)
         if n is None or not getattr(self, "record_in_one_kernel", True) or not self.use_fast_path:
             return None
         if q["E"] == 0 or q["dtype"] != q["ttype"] or a.term in (_lib.TERM_REACTION_DIFFUSION, _lib.TERM_MLP):
@@ -685,7 +694,7 @@ class AutoDiffAdjoint(nn.Module):
             return None
         L = fl[_lib.FLAG_MAX_ITERATIONS]
         record.iterations, record.arrays = L, fields
-        self._record_entries = L + 1 + 4
+        self._remember_record_entries(shape, L + 1 + 4)
         stats: Dict[str, Any] = {}
         if q["with_stats"]:
             stats["n_f_evals"] = _f_evals((1 if q["has_dt0"] else 2) + 6 * L, B)
