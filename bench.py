@@ -184,6 +184,29 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
     return result
 
 
+def measure_issue_interval():
+    """Nanoseconds per vector operation of one wavefront, and per SIMD (that divided by the wavefronts that share it),
+    for chains of dependent operations: what bounds a kernel that keeps one sample per lane in registers.  Cycles are
+    quoted at the 2.4 GHz the GPU reaches at most."""
+    import torch
+
+    from torchode_amd import _lib
+
+    rows = []
+    for dtype in (torch.float32, torch.float64):
+        for waves in (1, 2, 4, 8):
+            for chains in (1, 2, 4, 8):
+                per_wave = _lib.vector_issue_interval(dtype, "fma", chains, waves)
+                rows.append({"dtype": str(dtype)[6:], "operation": "fma", "wavefronts_per_simd": waves, "chains": chains,
+                             "ns_per_operation_of_a_wavefront": round(per_wave, 3), "ns_per_operation_of_a_simd": round(per_wave / waves, 3),
+                             "cycles_at_2.4_GHz_per_operation_of_a_simd": round(2.4 * per_wave / waves, 2)})  # fmt: skip
+        for op in ("div", "sqrt"):
+            per_wave = _lib.vector_issue_interval(dtype, op, 1, 1)
+            rows.append({"dtype": str(dtype)[6:], "operation": op, "wavefronts_per_simd": 1, "chains": 1, "ns_per_operation_of_a_wavefront": round(per_wave, 2),
+                         "cycles_at_2.4_GHz_per_operation_of_a_wavefront": round(2.4 * per_wave, 1)})  # fmt: skip
+    return {"metric": "vector issue interval", "unit": "ns per operation", "simds": 1024, "rows": rows}
+
+
 def measure_gradient(args, steps=10, warmup=3):
     """A differentiable solve of the headline configuration (Van der Pol float32, y0 and mu requiring grad) and the
     backward pass of sum(ys): the record of the loop state from the general whole-solve kernel, the reverse sweep in
@@ -245,6 +268,7 @@ def main():
     )
     ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
     ap.add_argument("--gradient", action="store_true", help="measure the differentiable solve of the headline configuration alone (forward with its record, backward)")
+    ap.add_argument("--issue-probe", action="store_true", help="measure the vector issue interval of the GPU's SIMDs (chains of dependent multiply-adds, divisions, square roots; 1-8 wavefronts per SIMD) instead of a solve")
     ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
     ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the headline's eager baseline is sized to (the other configurations take 0.4 of it)")
     ap.add_argument("--time-budget", type=float, default=420.0, help="seconds the whole run aims to stay within: a compiled CPU leg is started only while 100 s of it are left")
@@ -270,6 +294,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.issue_probe:
+        print(json.dumps(measure_issue_interval()))
+        return
     if args.gradient:
         print(json.dumps(measure_gradient(args, steps=args.steps if args.steps != 50 else 10)))
         return

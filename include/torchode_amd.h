@@ -503,6 +503,20 @@ int tode_last_solve_kernel_ms(float *out_ms);
  * "tode::solve_pair_kernel"; the same for every template instance of a kernel. */
 const char *tode_last_solve_kernel_name(void);
 
+/*
+ * Measurement aid; no counterpart in the reference.  Runs `wavefronts` wavefronts (one per workgroup; 1024 of them are
+ * one per SIMD of an MI355X, 2048 two, ...), each issuing 16384 vector fused multiply-adds (operation 0), or 2048
+ * correctly rounded divisions (1) or square roots (2), arranged as `chains` (1, 2, 4 or 8) independent dependency
+ * chains, and writes the time from the first wavefront's start to the last one's end divided by the operations of one
+ * wavefront, in nanoseconds (by the GPU-wide constant 100 MHz counter: the shader clock varies with load; at 2.4 GHz a
+ * nanosecond is 2.4 cycles): divided by the wavefronts that share a SIMD, the interval at which a SIMD issues.  It is the rate
+ * the per-step cost of the whole-solve kernels is read against: those are chains of dependent vector instructions,
+ * one sample per lane.  scratch: device memory of tode_probe_scratch_bytes(wavefronts) bytes.  Synchronises `stream`.
+ */
+int64_t tode_probe_scratch_bytes(int32_t wavefronts);
+int tode_probe_vector_issue(int32_t dtype, int32_t operation, int32_t chains, int32_t wavefronts, void *scratch, int64_t scratch_bytes,
+                            double *ns_per_operation, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Reverse of one loop iteration of the per-step kernels (gradients through the loop)
  * ------------------------------------------------------------------------------------------

@@ -56,6 +56,7 @@ UNITS = [
     ("tode_ops.hip", "tode_ops.o", []),
     ("tode_grid.hip", "tode_grid.o", []),
     ("tode_mlp.hip", "tode_mlp.o", []),
+    ("tode_probe.hip", "tode_probe.o", []),
 ]
 
 
