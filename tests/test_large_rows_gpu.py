@@ -445,7 +445,7 @@ def per_step_and_protocol(f, y0, t_eval, method, ctrl, t_start=None, t_end=None,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
-@pytest.mark.parametrize("features", [64, 100, 300, 1024])
+@pytest.mark.parametrize("features", [64, 100, 300, 1024, 2500])  # (from 1024 on: a workgroup per sample in the finish kernel)
 def test_per_step_path_on_long_rows_equals_the_protocol_path(features, dtype):
     g = torch.Generator().manual_seed(features)
     B, E = 37, 9

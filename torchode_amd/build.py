@@ -31,6 +31,7 @@ FLAGS = [
     "-fno-gpu-flush-denormals-to-zero",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-pass-failed",  # (a requested unrolling of a loop whose length only some instantiations know at compile time)
 ]  # fmt: skip
 
 # (source, object name, extra defines)

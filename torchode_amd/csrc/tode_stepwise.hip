@@ -196,6 +196,13 @@ __global__ void __launch_bounds__(256) init_b_kernel(const StepParams<TT, T> p, 
 
 // Quartic of the attempted step for one feature, evaluated at time te (tsit5.py:123-139,
 // dopri5.py:53-60, interpolation.py:25-40, 138-175).  ks[s] = k_s[b,f].
+// The value that lane `src` of the wavefront holds; `src` is the same for all lanes.
+__device__ __forceinline__ float wave_read(float v, int src) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src)); }
+__device__ __forceinline__ double wave_read(double v, int src) {
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), src), hi = __builtin_amdgcn_readlane(__double2hiint(v), src);
+    return __hiloint2double(hi, lo);
+}
+
 template <typename T> __device__ __forceinline__ T quartic_at(const T (&q)[5][1], T x) {
     T y = q[4][0];
     y = fma_(y, x, q[3][0]);
@@ -459,14 +466,51 @@ __global__ void __launch_bounds__(256) init_b_wave_kernel(const StepParams<TT, T
     }
 }
 
-template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<TT, T> p) {
+// The row norm of wave_row_norm with the four wavefronts of a workgroup sharing one row: wavefront w takes the chunks
+// w, w + 4, ..., the chunk sums meet in LDS and every thread adds them in the order of the chunks -- the same sums in
+// the same order, so the same bits as one wavefront walking the whole row.
+constexpr int TODE_BLOCK_ROW_CHUNKS = 1024;  // rows of up to 262144 values
+template <typename T, typename Load> __device__ __forceinline__ T block_row_rms(int F, T *chunk_sums, Load load) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const T sf = (T)__builtin_sqrt((double)F);
+    const int chunks = (F + 255) / 256;
+    for (int c = wave; c < chunks; c += 4) {
+        T part = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int f = c * 256 + 4 * lane + j;
+            if (f < F) {
+                const T x = load(f) / sf;
+                part = fma_(x, x, part);
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part = part + __shfl_xor(part, off);
+        if (lane == 0) chunk_sums[c] = part;
+    }
+    __syncthreads();
+    T total = 0;
+    for (int c = 0; c < chunks; ++c) total = total + chunk_sums[c];
+    return sqrt_(total);
+}
+
+// BLOCK false: one wavefront per sample, four samples per workgroup.  BLOCK true (long rows): the workgroup's four
+// wavefronts share one sample -- each walks every fourth group of 256 features, all four take the same decisions from
+// the same norm, thread 0 stores the sample's scalars.
+template <typename TT, typename T, int METHOD, int CTRL, bool BLOCK = false> __global__ void __launch_bounds__(256) finish_wave_kernel(const StepParams<TT, T> p) {
     using Tab = typename TabOf<METHOD>::type;
     constexpr int NS = stages_of(METHOD);
     constexpr bool ESTIMATE = METHOD != TODE_EULER;
+    __shared__ T chunk_sums[BLOCK ? TODE_BLOCK_ROW_CHUNKS : 1];
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
-    const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long b = BLOCK ? (long long)blockIdx.x : (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= p.batch) return;
     const int F = p.F, E = p.E, lane = threadIdx.x & 63;
+    // a thread's features: `first`, `first + stride`, ...; the dense output walks groups of 256 features, `group_first`
+    // and every `group_stride`-th after it; `scalar_thread` stores what the sample has one of
+    const int first = BLOCK ? (int)threadIdx.x : lane, stride = BLOCK ? 256 : 64;
+    const int group_first = BLOCK ? 256 * (int)(threadIdx.x >> 6) : 0, group_stride = BLOCK ? 1024 : 256;
+    const bool scalar_thread = BLOCK ? threadIdx.x == 0 : lane == 0;
     const CtrlParams<T> &cp = p.cp;
     const bool fused = F >= 58;
     const TT t0 = p.t[b], dt = p.dt[b];
@@ -497,7 +541,7 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     };
 
     // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
-    const T norm = (CTRL == 2 || !ESTIMATE) ? (T)0 : wave_row_norm<T, TODE_NORM_RMS>(F, [&](int f) {
+    auto scaled_error = [&](int f) {
         T err = 0;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -511,7 +555,10 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         }
         const T m = tmax(abs_(y[f]), abs_(y1(f)));
         return abs_(err) / fma_(cp.rtol, m, cp.atol);
-    });
+    };
+    const T norm = (CTRL == 2 || !ESTIMATE) ? (T)0
+                   : BLOCK                  ? block_row_rms<T>(F, chunk_sums, scaled_error)
+                                            : wave_row_norm<T, TODE_NORM_RMS>(F, scaled_error);
     const T ratio = tmax(norm, (T)1e-38);
     const bool accept = CTRL == 2 || !ESTIMATE || ratio < (T)1;
 
@@ -544,46 +591,76 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         uint8_t *pend = p.pending + b * (long long)E;
         const bool mono = p.monotone[b] != 0;
         const int cursor = p.cursor[b];
-        for (int f = lane; f < F; f += 64) {
-            T q[5][1], ks[7] = {};
-            T y1f = 0;
-            bool built = false;
-            for (int e = mono ? cursor : 0; e < E; ++e) {
+        // The pending points are looked at 64 at a time, one per lane: which of them the step has passed (for a
+        // monotone row: those in front of the first one it has not) comes out as a mask that is the same for the whole
+        // wavefront, and each lane keeps its point's position in the step.  Then the row is walked once per such group
+        // of points -- 256 features at a time, so that the loads of four features are in flight together -- and every
+        // feature's interpolant is evaluated at the points of the mask, their positions read from the lanes that hold
+        // them.  Nothing in the inner loops waits for memory but the row itself.
+        for (int e0 = mono ? cursor : 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const bool valid = e < E;
+            const bool pending = valid && pend[e] != 0;
+            const TT te_e = valid ? tev[e] : t0;
+            const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
+            unsigned long long take = __ballot(pending && passed);
+            const unsigned long long blocked = mono ? __ballot(pending && !passed) : 0ull;
+            if (blocked) take &= (blocked & (~blocked + 1ull)) - 1ull;  // (only the points in front of the first one not passed)
+            if (take) {
+                const T x = (T)unit_time<TT>(te_e, t0, t0 + dt);
+                for (int f0 = group_first; f0 < F; f0 += group_stride) {
+                    T q[4][5][1], ks[4][7] = {}, y0f[4] = {}, y1f[4] = {};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int f = f0 + 64 * j + lane;
+                        if (f < F) {
+#pragma unroll
+                            for (int s = 0; s < NS; ++s) ks[j][s] = p.k[s][b * F + f];
+                            y0f[j] = y[f], y1f[j] = y1(f);
+                        }
+                    }
+                    if (NS == 7) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) quartic_elem<T, (METHOD == 1 ? 1 : 0)>(h, y0f[j], y1f[j], ks[j], fused, q[j]);
+                    }
+                    for (unsigned long long m = take; m; m &= m - 1ull) {
+                        const int i = __builtin_ctzll(m);
+                        T *row = ys + (long long)(e0 + i) * F + f0 + lane;
+                        const T xi = wave_read(x, i);
+                        const TT ti = wave_read(te_e, i);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            if (f0 + 64 * j + lane < F) {
+                                if (NS == 7)
+                                    row[64 * j] = quartic_at<T>(q[j], xi);
+                                else  // (Hermite cubic / linear interpolant: cheap enough to form per point)
+                                    row[64 * j] = dense_value<TT, T, METHOD>(t0, dt, y0f[j], y1f[j], ks[j], fused, ti);
+                            }
+                        }
+                    }
+                }
+            }
+            if (blocked) break;
+        }
+        // (every lane has finished reading the pending marks: a wavefront runs in lock step, a workgroup waits here;
+        // the marks are then brought up to date by one wavefront)
+        if (BLOCK) __syncthreads();
+        if (!BLOCK || threadIdx.x < 64) {
+            int first_pending = E;
+            for (int e = lane; e < E; e += 64) {
                 if (!pend[e]) continue;
                 const TT te_e = tev[e];
                 const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
-                if (!passed) {
-                    if (mono) break;
-                    continue;
-                }
-                if (!built) {
-#pragma unroll
-                    for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
-                    y1f = y1(f);
-                    if (NS == 7) quartic_elem<T, (METHOD == 1 ? 1 : 0)>(h, y[f], y1f, ks, fused, q);
-                    built = true;
-                }
-                if (NS == 7)
-                    ys[(long long)e * F + f] = quartic_at<T>(q, (T)unit_time<TT>(te_e, t0, t0 + dt));
-                else  // (Hermite cubic / linear interpolant: cheap enough to form per point)
-                    ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1f, ks, fused, te_e);
+                const bool taken = passed && (!mono || e >= cursor);
+                if (taken) pend[e] = 0;
+                else first_pending = min(first_pending, e);
             }
-        }
-        // (every lane has finished reading the pending marks: the wavefront runs in lock step)
-        int first_pending = E;
-        for (int e = lane; e < E; e += 64) {
-            if (!pend[e]) continue;
-            const TT te_e = tev[e];
-            const bool passed = fwd ? t_new >= te_e : t_new <= te_e;
-            const bool taken = passed && (!mono || e >= cursor);
-            if (taken) pend[e] = 0;
-            else first_pending = min(first_pending, e);
-        }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) first_pending = min(first_pending, __shfl_xor(first_pending, off));
-        if (lane == 0) p.cursor[b] = first_pending;
+            for (int off = 32; off > 0; off >>= 1) first_pending = min(first_pending, __shfl_xor(first_pending, off));
+            if (lane == 0) p.cursor[b] = first_pending;
+        }
     } else {
-        for (int f = lane; f < F; f += 64) {
+        for (int f = first; f < F; f += stride) {
             T ks[7] = {};
 #pragma unroll
             for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
@@ -592,14 +669,15 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     }
 
     // ---- state update ----
+    if (BLOCK) __syncthreads();  // (no thread of the workgroup still reads what is overwritten now)
     if (move) {
-        for (int f = lane; f < F; f += 64) {
+        for (int f = first; f < F; f += stride) {
             const T moved = y1(f);  // (read before the write: for Heun and Euler y1 is formed from y)
             p.y[b * F + f] = moved;
             if (NS == 7) p.k0[b * F + f] = p.k[6][b * F + f];  // (first same as last: Dopri5 and Tsit5 only)
         }
     }
-    if (lane == 0) {
+    if (scalar_thread) {
         p.n_steps[b] = n_steps;
         if (move) p.n_accepted[b] += 1;
         p.status[b] = status;
@@ -819,6 +897,13 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
 }
 
 #define TODE_FINISH(KERNEL, M, C) hipLaunchKernelGGL((KERNEL<TT, T, M, C>), dim3(blocks), dim3(256), 0, st, p)
+// (long rows: the workgroup-per-sample form of the wavefront kernel)
+#define TODE_FINISH_ROWS(M)                                                                                                        \
+    do {                                                                                                                           \
+        if (c->kind == TODE_CTRL_PID) hipLaunchKernelGGL((finish_wave_kernel<TT, T, M, 1, true>), dim3(blocks), dim3(256), 0, st, p);        \
+        else if (c->kind == TODE_CTRL_FIXED) hipLaunchKernelGGL((finish_wave_kernel<TT, T, M, 2, true>), dim3(blocks), dim3(256), 0, st, p); \
+        else hipLaunchKernelGGL((finish_wave_kernel<TT, T, M, 0, true>), dim3(blocks), dim3(256), 0, st, p);                                 \
+    } while (0)
 #define TODE_FINISH_CTRL(KERNEL, M)                                     \
     do {                                                                \
         if (c->kind == TODE_CTRL_PID) TODE_FINISH(KERNEL, M, 1);        \
@@ -832,7 +917,10 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     const bool wide = s->n_features >= 64;
-    const unsigned blocks = wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
+    // rows of 1024 values and more: a workgroup per sample instead of a wavefront (more loads and stores in flight per
+    // sample; the same sums in the same order)
+    const bool rows = s->n_features >= 1024 && (s->n_features + 255) / 256 <= TODE_BLOCK_ROW_CHUNKS && s->batch <= 0x7fffffff;
+    const unsigned blocks = rows ? (unsigned)s->batch : wide ? (unsigned)((s->batch + 3) / 4) : (unsigned)((s->batch + 255) / 256);
     if (blocks > 0) {
         for (int j = 0; j < stages_of(s->method); ++j)
             if (!s->k[j]) return fail(TODE_E_INVALID, "k[%d] is null", j);
@@ -840,7 +928,12 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
         TODE_DISPATCH_T(s, {
             auto p = make_step_params<TT, T>(*s, *c);
             const bool tsit5 = s->method == TODE_TSIT5;
-            if (s->method == TODE_HEUN) {
+            if (rows) {
+                if (s->method == TODE_HEUN) TODE_FINISH_ROWS(2);
+                else if (s->method == TODE_EULER) TODE_FINISH_ROWS(3);
+                else if (tsit5) TODE_FINISH_ROWS(1);
+                else TODE_FINISH_ROWS(0);
+            } else if (s->method == TODE_HEUN) {
                 if (wide) TODE_FINISH_CTRL(finish_wave_kernel, 2);
                 else TODE_FINISH_CTRL(finish_kernel, 2);
             } else if (s->method == TODE_EULER) {
