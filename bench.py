@@ -47,8 +47,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("vdp", "torch.float32", 65536): 47.79e6,
     # profiles/solve_pair_kernel_vdp_f64_b65536_hbm_traffic.txt: (25316.5 KiB x 2.000 + 101408.5 KiB x 1.000) x 1024
     ("vdp", "torch.float64", 65536): 155.69e6,
-    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (78246.4 KiB x 2.000 + 931465.0 KiB x 1.000) x 1024
-    ("lorenz", "torch.float32", 1048576): 1114.07e6,
+    # profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt: (78276.2 KiB x 2.000 + 934960.1 KiB x 1.000) x 1024
+    ("lorenz", "torch.float32", 1048576): 1117.71e6,
     # profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt: (4393 KiB x 2.000 + 819301 KiB x 1.000) x 1024
     ("reaction_diffusion", "torch.float32", 512): 847.96e6,
     # profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt: (1504 KiB x 2.000 + 20624 KiB x 1.000) x 1024
