@@ -587,7 +587,7 @@ int tode_step_stage_backward(const tode_step_adjoint *adjoint, const tode_contro
  * tode_step_stage / f / tode_step_finish_backward / f's vector-Jacobian product / tode_step_stage_backward per
  * iteration above, with the right-hand side and its vector-Jacobian product evaluated in the kernel.
  *
- * args: the forward problem as for tode_solve_builtin (y0 is not read; t_start / t_end dense; dtype one of TODE_F32 /
+ * args: the forward problem as for tode_solve_builtin (y0 is not read; t_start / t_end with their strides; dtype one of TODE_F32 /
  * TODE_F64; method Dopri5 or Tsit5; controller integral or PID), with args->record pointing to the record the forward
  * pass wrote.  All pointers below are device memory.  Nothing is allocated; the call only enqueues.
  */
@@ -595,7 +595,9 @@ typedef struct tode_solve_adjoint {
     const void *grad_ys;           /* [B, max(E,1), F] cotangent of ys */
     const int32_t *points_by_iteration; /* [B,E]: each sample's evaluation points ordered by the iteration that wrote them */
     const int32_t *iterations_sorted;   /* [B,E]: those iterations in the same order, ascending; -1 (first) for a point that
-                                           no iteration wrote.  Both NULL when E == 0 */
+                                           no iteration wrote.  Both NULL when E == 0 -- or to have the library work
+                                           them out from the record's times (a kernel of its own in front of the sweep,
+                                           into `scratch`) */
     int64_t iterations;            /* L: iterations of the loop; the record's entries 0..L are read */
     int32_t through_control;       /* as in tode_step_adjoint */
     int32_t through_start;         /* 0: the results are the cotangents of the loop's first state.  1: the kernel also
@@ -606,7 +608,8 @@ typedef struct tode_solve_adjoint {
                                       start's share.  The times count as constants in that part, so a caller that
                                       wants g_t_start / g_t_end passes 0 and does the start itself.  args->dt0 is not
                                       read, only looked at: non-NULL says that the first step was the caller's */
-    void *scratch;                 /* tode_solve_backward_scratch_bytes(args) bytes */
+    void *scratch;                 /* tode_solve_backward_scratch_bytes(args) bytes (two int32 lists of [B,E]); looked at
+                                      only when the two lists above are NULL and E > 0 */
     int64_t scratch_bytes;
     /* results: cotangents of the loop state before the first iteration (y, the first-same-as-last derivative
        f(t_start, y0), t, the first step, the controller's history) ... */

@@ -148,7 +148,10 @@ def test_whole_reverse_sweep_entry_point_checks_its_arguments_without_a_gpu():
     assert lib.tode_solve_builtin_backward(None, None, None, None) == _lib.E_INVALID
     a.dtype, a.batch, a.n_features, a.n_eval, a.n_params, a.term = _lib.DTYPES[torch.float64], 100, 2, 0, 1, 1
     a.t_start_stride = a.t_end_stride = 1
-    assert lib.tode_solve_backward_scratch_bytes(ref(a)) == 0  # (the working rows live in LDS)
+    assert lib.tode_solve_backward_scratch_bytes(ref(a)) == 0  # (no evaluation points: no lists of them to work out)
+    a.n_eval = 7
+    assert lib.tode_solve_backward_scratch_bytes(ref(a)) == 2 * 100 * 7 * 4  # (two int32 lists [B,E], unless the caller hands them in)
+    a.n_eval = 0
     assert lib.tode_solve_builtin_backward(ref(a), ref(c), ref(adj), None) == _lib.E_INVALID and b"record" in lib.tode_last_error()
     rec = _lib.SolveRecord()
     rec.capacity = 5

@@ -173,7 +173,13 @@ class Replay:
         self.term, self.args = term, args
         self.through_control = through_control
         self.t_start, self.t_end, self.t_eval = problem.t_start, problem.t_end, problem.t_eval
-        self.direction = torch.where(self.t_end > self.t_start, 1.0, -1.0).to(self.t_start.dtype)
+        self._direction = None
+
+    @property
+    def direction(self):
+        if self._direction is None:  # (formed when a sweep in torch operations asks for it)
+            self._direction = torch.where(self.t_end > self.t_start, 1.0, -1.0).to(self.t_start.dtype)
+        return self._direction
 
     # the ends of the time range are functions of t_start and t_end: formed where they are used, so that every
     # iteration of the reverse sweep differentiates a graph of its own
@@ -370,18 +376,6 @@ def reverse_sweep_torch(replay: Replay, states, hits, grad_ys, params):
     return adj, grad_params
 
 
-_POINT_NUMBERS = {}
-
-
-def _point_numbers(B: int, E: int, device) -> torch.Tensor:
-    """``[B, E]`` int32, every row ``0 .. E-1`` (kept per shape: the sweep only reads it)."""
-    key = (B, E, str(device))
-    if key not in _POINT_NUMBERS:
-        _POINT_NUMBERS.clear()
-        _POINT_NUMBERS[key] = torch.arange(E, dtype=torch.int32, device=device).expand(B, E).contiguous()
-    return _POINT_NUMBERS[key]
-
-
 def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, grad_ys, params):
     """All iterations in reverse in one kernel (tode_solve_builtin_backward): for a built-in term whose forward pass
     left its record in entry-major arrays.  The right-hand side and its vector-Jacobian product are evaluated in the
@@ -398,26 +392,14 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     new = lambda *shape, dt=dtype: torch.empty(shape, dtype=dt, device=dev)
     zeros = lambda *shape, dt=dtype: torch.zeros(shape, dtype=dt, device=dev)
     contiguous = lambda x: x.detach().to(dtype).contiguous()
-    t_start, t_end = contiguous(replay.t_start), contiguous(replay.t_end)
+    # (t_start / t_end are usually columns of t_eval: handed over with their strides, unless their gradients are wanted)
+    strided = lambda x: x.detach() if (x.dtype == dtype and x.stride(0) >= 1 and not x.requires_grad) else contiguous(x)
+    t_start, t_end = strided(replay.t_start), strided(replay.t_end)
     t_eval = None if replay.t_eval is None else contiguous(replay.t_eval)
     L, arrays = record.iterations, record.arrays
 
-    # which iteration wrote which evaluation point (adjoints.py:215-234): the first whose new time has passed it
-    iterations_sorted = points_by_iteration = None
-    if E > 0:
-        direction = torch.where(t_end > t_start, 1.0, -1.0).to(dtype)
-        reached = (direction[None, :] * arrays["t"][1 : L + 1]).t().contiguous()  # [B, L], ascending
-        hit = torch.searchsorted(reached, direction[:, None] * t_eval) if L > 0 else torch.zeros((B, E), dtype=torch.long, device=dev)
-        hit = torch.where(hit < L, hit, torch.full_like(hit, -1))
-        hit[:, 0] = torch.where(t_eval[:, 0] == t_start, torch.full_like(hit[:, 0], -1), hit[:, 0])
-        # ordered by iteration, so that the kernel, walking the iterations down, finds each one's points at a cursor
-        hit = hit.to(torch.int32)
-        if E == 1 or bool((hit[:, 1:] >= hit[:, :-1]).all()):
-            # evaluation times in the direction of the solve, every one of them reached: already in order
-            iterations_sorted, points_by_iteration = hit.contiguous(), _point_numbers(B, E, dev)
-        else:
-            iterations_sorted, points_by_iteration = torch.sort(hit, dim=1, stable=True)
-            iterations_sorted, points_by_iteration = iterations_sorted.contiguous(), points_by_iteration.to(torch.int32).contiguous()
+    # (which iteration wrote which evaluation point, and each sample's points ordered by it: worked out by the
+    # library from the record's times, in a kernel in front of the sweep)
     wants = lambda x: x is not None and x.requires_grad
     g_t_start = zeros(B) if wants(replay.t_start) else None
     g_t_end = zeros(B) if wants(replay.t_end) else None
@@ -431,7 +413,7 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     a.dtype, a.method, a.term, a.n_features, a.n_eval, a.n_params, a.batch = _lib.DTYPES[dtype], method.method_id, f.builtin_kind, F, E, P, B
     a.max_steps, a.iteration_cap = -1, -1
     a.term_scalars = (_lib.C.c_double * 4)(*scal[:4])
-    a.t_start, a.t_end, a.t_start_stride, a.t_end_stride = t_start.data_ptr(), t_end.data_ptr(), 1, 1
+    a.t_start, a.t_end, a.t_start_stride, a.t_end_stride = t_start.data_ptr(), t_end.data_ptr(), t_start.stride(0), t_end.stride(0)
     a.t_eval, a.params = _lib.ptr(t_eval), (par.data_ptr() if par.numel() else None)
     names = ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")
     rec = _lib.SolveRecord(arrays["t"].shape[0], *(arrays[k].data_ptr() for k in names))
@@ -450,7 +432,6 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     ad.through_start = int(through_start)
     if dt0 is not None:
         a.dt0 = dt0.data_ptr()  # (not read: it says that the first step was given)
-    ad.points_by_iteration, ad.iterations_sorted = _lib.ptr(points_by_iteration), _lib.ptr(iterations_sorted)
     ad.scratch, ad.scratch_bytes = scratch.data_ptr(), scratch.numel()
     ad.a_y, ad.a_k0 = out_y.data_ptr(), out_k0.data_ptr()
     ad.a_t, ad.a_dt, ad.a_prev, ad.a_pprev = (out_s[i].data_ptr() for i in range(4))

@@ -27,6 +27,7 @@ template <typename T> struct WholeBackward {
     // the evaluation points of every sample ordered by the iteration that wrote them: [B,E] point indices and, in the
     // same order, the iterations (-1 first: points no iteration wrote)
     const int32_t *points_by_iteration, *iterations_sorted;
+    long long ts_stride, te_stride;  // t_start / t_end: sample b at element b * stride
     int through_start;  // also carry the cotangents through the start of the loop (start_backward)
     int dt0_given;      // the first step was the caller's, not the start rule's
 };
@@ -183,7 +184,7 @@ __global__ void __launch_bounds__(64) whole_backward_kernel(const WholeBackward<
     q.a_y = a_y, q.a_k0 = a_k0, q.a_t = &a_t, q.a_dt = &a_dt, q.a_prev = &a_prev, q.a_pprev = &a_pprev;
     // ---- what lives in global memory, moved forward to this sample ----
     const int E = q.E;
-    q.t_start += g, q.t_end += g;
+    q.t_start += g * w.ts_stride, q.t_end += g * w.te_stride;
     if (q.t_eval) q.t_eval += g * E;
     q.grad_ys += g * (long long)(E > 0 ? E : 1) * F;
     if (q.g_t_start) q.g_t_start += g;
@@ -262,6 +263,47 @@ __global__ void __launch_bounds__(64) whole_backward_kernel(const WholeBackward<
     for (int j = 0; j < P; ++j) w.g_params[g * P + j] = gpar[j];
 }
 
+// Which iteration wrote which evaluation point (adjoints.py:215-234: the first whose new time has reached it; none for
+// a point at t_start, which the loop's set-up writes, and for one the solve never reached): one thread per point, a
+// binary search over the sample's recorded times.
+template <typename T> __global__ void __launch_bounds__(256) backward_hits_kernel(long long B, int E, long long L, const T *t_start, long long ts_stride, const T *t_end, long long te_stride,
+                                                                                  const T *t_eval, const T *rec_t, int32_t *iterations_sorted, int32_t *points_by_iteration) {
+    const long long at_point = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (at_point >= B * E) return;
+    const long long b = at_point / E;
+    const int e = (int)(at_point - b * E);
+    const T ts = t_start[b * ts_stride], dir = t_end[b * te_stride] > ts ? (T)1 : (T)-1;
+    const T at = t_eval[at_point], v = dir * at;
+    long long lo = 0, hi = L;
+    while (lo < hi) {
+        const long long mid = (lo + hi) / 2;
+        if (dir * rec_t[(mid + 1) * B + b] < v) lo = mid + 1;
+        else hi = mid;
+    }
+    int32_t hit = lo < L ? (int32_t)lo : -1;
+    if (e == 0 && at == ts) hit = -1;
+    iterations_sorted[at_point] = hit, points_by_iteration[at_point] = e;
+}
+
+// Each sample's points ordered by the iteration that wrote them (stable: points of one iteration stay in their order).
+// One thread per sample.  Rows whose evaluation times run in the direction of the solve are in order already, which a
+// look along the row shows; the others are sorted by insertion.
+// (a template only so that each translation unit that instantiates the sweep has its own copy)
+template <typename T> __global__ void __launch_bounds__(256) backward_order_kernel(long long B, int E, int32_t *iterations_sorted, int32_t *points_by_iteration) {
+    const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= B) return;
+    int32_t *its = iterations_sorted + b * E, *pts = points_by_iteration + b * E;
+    bool ordered = true;
+    for (int e = 1; e < E; ++e) ordered = ordered && its[e - 1] <= its[e];
+    if (ordered) return;
+    for (int e = 1; e < E; ++e) {
+        const int32_t hit = its[e], point = pts[e];
+        int j = e - 1;
+        for (; j >= 0 && its[j] > hit; --j) its[j + 1] = its[j], pts[j + 1] = pts[j];
+        its[j + 1] = hit, pts[j + 1] = point;
+    }
+}
+
 template <typename T, int METHOD, int CTRL, typename Term>
 static int launch_backward(const tode_solve_args &a, const tode_controller &c, const tode_solve_adjoint &adj, hipStream_t stream) {
     const long long B = a.batch;
@@ -283,8 +325,15 @@ static int launch_backward(const tode_solve_args &a, const tode_controller &c, c
     for (int i = 0; i < 4; ++i) w.scalars[i] = a.term_scalars[i];
     w.g_params = (T *)adj.g_params;
     w.points_by_iteration = adj.points_by_iteration, w.iterations_sorted = adj.iterations_sorted;
+    if (a.n_eval > 0 && !adj.points_by_iteration) {  // (not handed in: worked out here, into the caller's scratch)
+        int32_t *lists = (int32_t *)adj.scratch;
+        w.iterations_sorted = lists, w.points_by_iteration = lists + B * a.n_eval;
+        hipLaunchKernelGGL((backward_hits_kernel<T>), dim3((unsigned)((B * a.n_eval + 255) / 256)), dim3(256), 0, stream, B, a.n_eval, (long long)adj.iterations, (const T *)a.t_start,
+                           (long long)a.t_start_stride, (const T *)a.t_end, (long long)a.t_end_stride, (const T *)a.t_eval, (const T *)a.record->t, lists, lists + B * a.n_eval);
+        hipLaunchKernelGGL((backward_order_kernel<T>), dim3((unsigned)((B + 255) / 256)), dim3(256), 0, stream, B, a.n_eval, lists, lists + B * a.n_eval);
+    }
     w.through_start = adj.through_start, w.dt0_given = a.dt0 != nullptr;
-    // (the t_start / t_end strides of the forward entry point are not taken here: the caller passes dense arrays)
+    w.ts_stride = a.t_start_stride, w.te_stride = a.t_end_stride;
     hipLaunchKernelGGL((whole_backward_kernel<T, METHOD, CTRL, Term>), dim3((unsigned)((B + 63) / 64)), dim3(64), 0, stream, w);
     return check_hip(hipGetLastError(), "tode_solve_builtin_backward launch");
 }
@@ -335,8 +384,8 @@ int solve_backward_f64(const tode_solve_args &a, const tode_controller &c, const
 extern "C" {
 
 int64_t tode_solve_backward_scratch_bytes(const tode_solve_args *a) {
-    if (!a || a->n_features <= 0 || a->batch < 0) return -1;
-    return 0;  // (the sweep's working arrays are the threads' own)
+    if (!a || a->n_features <= 0 || a->batch < 0 || a->n_eval < 0) return -1;
+    return 2 * a->batch * a->n_eval * (int64_t)sizeof(int32_t);  // (the two lists of evaluation points, where the caller does not hand them in)
 }
 
 int tode_solve_builtin_backward(const tode_solve_args *a, const tode_controller *c, const tode_solve_adjoint *adj, void *stream) {
@@ -349,15 +398,18 @@ int tode_solve_builtin_backward(const tode_solve_args *a, const tode_controller 
     if (!a->record) return fail(TODE_E_INVALID, "args->record is null: the sweep starts from the record of the forward pass");
     if (adj->iterations < 0 || a->record->capacity < adj->iterations + 1)
         return fail(TODE_E_INVALID, "the record holds %lld entries, %lld iterations need %lld", (long long)a->record->capacity, (long long)adj->iterations, (long long)adj->iterations + 1);
-    if (a->t_start_stride != 1 || a->t_end_stride != 1) return fail(TODE_E_INVALID, "t_start and t_end must be dense arrays here");
+    if (a->t_start_stride < 1 || a->t_end_stride < 1) return fail(TODE_E_INVALID, "t_start_stride / t_end_stride must be >= 1");
+    if ((a->t_start_stride != 1 && adj->g_t_start) || (a->t_end_stride != 1 && adj->g_t_end)) return fail(TODE_E_INVALID, "g_t_start / g_t_end are dense arrays: ask for them with dense t_start / t_end");
     if (a->batch == 0) return TODE_OK;
     const tode_solve_record &r = *a->record;
     if (!r.t || !r.dt || !r.y || !r.k0 || !r.prev || !r.pprev || !r.running || !r.n_accepted) return fail(TODE_E_INVALID, "a null array in the record");
-    if (!a->t_start || !a->t_end || (a->n_eval > 0 && (!a->t_eval || !adj->points_by_iteration || !adj->iterations_sorted)) || (a->n_params > 0 && !a->params) || !adj->grad_ys || !adj->a_y ||
+    if (!a->t_start || !a->t_end || (a->n_eval > 0 && (!a->t_eval || !adj->points_by_iteration != !adj->iterations_sorted)) || (a->n_params > 0 && !a->params) || !adj->grad_ys || !adj->a_y ||
         !adj->a_k0 || !adj->a_t || !adj->a_dt || !adj->a_prev || !adj->a_pprev || !adj->g_params)
         return fail(TODE_E_INVALID, "null pointer");
-    if (adj->scratch_bytes < tode_solve_backward_scratch_bytes(a) || (tode_solve_backward_scratch_bytes(a) > 0 && !adj->scratch))
-        return fail(TODE_E_INVALID, "the scratch buffer holds %lld bytes, this sweep needs %lld (tode_solve_backward_scratch_bytes)", (long long)adj->scratch_bytes,
+    const bool own_lists = a->n_eval > 0 && !adj->points_by_iteration;
+    if (own_lists && (a->batch * (int64_t)a->n_eval + 255) / 256 > 2147483647) return fail(TODE_E_UNSUPPORTED, "too many evaluation points for the library to order them: hand the two lists in");
+    if (own_lists && (!adj->scratch || adj->scratch_bytes < tode_solve_backward_scratch_bytes(a)))
+        return fail(TODE_E_INVALID, "the scratch buffer holds %lld bytes, this sweep needs %lld (tode_solve_backward_scratch_bytes)", (long long)(adj->scratch ? adj->scratch_bytes : 0),
                     (long long)tode_solve_backward_scratch_bytes(a));
     hipStream_t s = (hipStream_t)stream;
     return a->dtype == TODE_F32 ? solve_backward_f32(*a, *c, *adj, s) : solve_backward_f64(*a, *c, *adj, s);

@@ -28,13 +28,20 @@ class InitialValueProblem:
         self.y0, self.t_eval = y0, t_eval
         self.t_start = t_eval[:, 0] if t_start is None else t_start
         self.t_end = t_eval[:, -1] if t_end is None else t_end
-        self.time_direction = torch.where(self.t_end > self.t_start, 1, -1)
+        self._time_direction = None  # (made when first asked for: four small launches that most solves never need)
 
         times = (self.t_start, self.t_end) if t_eval is None else (self.t_start, self.t_end, t_eval)
         assert y0.ndim == 2 and self.t_start.ndim == 1 and self.t_end.ndim == 1 and (t_eval is None or t_eval.ndim == 2)
         assert _agree("dtype", *times)
         assert _agree("batch", y0, *times)
         assert _agree("device", y0, *times)
+
+    @property
+    def time_direction(self) -> torch.Tensor:
+        """``+1`` where ``t_end > t_start``, ``-1`` otherwise (reference problems.py:58-60)."""
+        if self._time_direction is None:
+            self._time_direction = torch.where(self.t_end > self.t_start, 1, -1)
+        return self._time_direction
 
     # what the solvers ask of a problem
     data_dtype = property(lambda self: self.y0.dtype)
