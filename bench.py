@@ -67,7 +67,7 @@ OTHER_CONFIGS = [
 START = time.perf_counter()
 
 
-def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_iterations=-1):
+def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_iterations=-1, batch_copies=None):
     """One configuration on the GPU: wall time of `steps` solves, kernel time by HIP events, roofline."""
     path = args.path if path is None else path
     graph_iterations = args.graph_iterations if graph_iterations == -1 else graph_iterations
@@ -81,6 +81,10 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
     dtype = w.y0.dtype
     if w.name == "mlp":
         w.f.matrix_inputs = mlp_inputs
+    batch_copies = args.batch_copies if batch_copies is None else batch_copies
+    if batch_copies > 1:  # (a larger batch of the same problems: for terms without per-sample parameters)
+        assert w.name == "mlp", "--batch-copies is for the mlp workload (its weights are shared by the batch)"
+        w = w._replace(y0=w.y0.repeat(batch_copies, 1).contiguous(), t_eval=w.t_eval.repeat(batch_copies, 1).contiguous())
     B, F = w.y0.shape
     E = w.t_eval.shape[1]
     spec = dict(w.controller)
@@ -258,6 +262,7 @@ def main():
                     help="measure this configuration alone (default: the headline, Van der Pol float32, and then every other one under 'configs')")  # fmt: skip
     ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
     ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
+    ap.add_argument("--batch-copies", type=int, default=1, help="mlp workload: solve this many copies of the batch at once (B = 4096 x copies), to see the kernel with more than one workgroup per compute unit")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-compiled-baseline", action="store_true", help="skip the torch.compile CPU legs (about a minute of compilation each)")
     ap.add_argument(
@@ -344,6 +349,9 @@ def main():
             measure(args, "vdp", "f32", "float32", 5, 2, path="per-step", graph_iterations=2),
         ]
         out["gradient"] = measure_gradient(args)
+        # the neural ODE at sixteen times its batch (not a BASELINE configuration): two workgroups per compute unit
+        # fill each other's waits for barriers and LDS, which the one workgroup per compute unit of B=4096 cannot
+        out["larger_batch"] = [measure(args, "mlp", "f32", "float32", 10, 2, batch_copies=16)]
     out["bench_seconds"] = time.perf_counter() - START
     print(json.dumps(out))
 

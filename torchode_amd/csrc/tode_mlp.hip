@@ -328,7 +328,7 @@ __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (
 }
 
 template <int METHOD, int CTRL, typename Weights>
-__global__ void __launch_bounds__(256) solve_mlp_kernel(const SolveParams<float> p, const float *packed, const MlpOut o) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) solve_mlp_kernel(const SolveParams<float> p, const float *packed, const MlpOut o) {
     using T = float;
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = MLP_F;
