@@ -398,8 +398,18 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     t_eval = None if replay.t_eval is None else contiguous(replay.t_eval)
     L, arrays = record.iterations, record.arrays
 
-    # (which iteration wrote which evaluation point, and each sample's points ordered by it: worked out by the
-    # library from the record's times, in a kernel in front of the sweep)
+    # Which iteration wrote which evaluation point (adjoints.py:215-234: the first whose new time has passed it), and
+    # each sample's points ordered by it: worked out by the library from the record's times, in two kernels in front
+    # of the sweep.  The same in torch operations, handed in, for the tests to hold against that.
+    iterations_sorted = points_by_iteration = None
+    if E > 0 and getattr(adjoint, "backward_points_in_torch", False):
+        direction = torch.where(t_end > t_start, 1.0, -1.0).to(dtype)
+        reached = (direction[None, :] * arrays["t"][1 : L + 1]).t().contiguous()  # [B, L], ascending
+        hit = torch.searchsorted(reached, direction[:, None] * t_eval) if L > 0 else torch.zeros((B, E), dtype=torch.long, device=dev)
+        hit = torch.where(hit < L, hit, torch.full_like(hit, -1))
+        hit[:, 0] = torch.where(t_eval[:, 0] == t_start, torch.full_like(hit[:, 0], -1), hit[:, 0])
+        iterations_sorted, points_by_iteration = torch.sort(hit.to(torch.int32), dim=1, stable=True)
+        iterations_sorted, points_by_iteration = iterations_sorted.contiguous(), points_by_iteration.to(torch.int32).contiguous()
     wants = lambda x: x is not None and x.requires_grad
     g_t_start = zeros(B) if wants(replay.t_start) else None
     g_t_end = zeros(B) if wants(replay.t_end) else None
@@ -433,6 +443,7 @@ def reverse_sweep_whole(adjoint, replay: Replay, term, problem, dt0, record, gra
     if dt0 is not None:
         a.dt0 = dt0.data_ptr()  # (not read: it says that the first step was given)
     ad.scratch, ad.scratch_bytes = scratch.data_ptr(), scratch.numel()
+    ad.points_by_iteration, ad.iterations_sorted = _lib.ptr(points_by_iteration), _lib.ptr(iterations_sorted)
     ad.a_y, ad.a_k0 = out_y.data_ptr(), out_k0.data_ptr()
     ad.a_t, ad.a_dt, ad.a_prev, ad.a_pprev = (out_s[i].data_ptr() for i in range(4))
     ad.g_params = g_par.data_ptr()
