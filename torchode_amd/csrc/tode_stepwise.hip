@@ -238,14 +238,16 @@ __device__ __forceinline__ T dense_value(TT t0, TT dt, T y0, T y1, const T (&ks)
 // counters, dense output at the evaluation points the step passed, state update, running
 // flag, dt clamp (runge_kutta.py:265-272, step_size_controllers.py:370-429 / 715-774,
 // adjoints.py:150-255).
-template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<TT, T> p) {
+// FC: the row length where the launch knows it at compile time (0: p.F).  With it, and with Dopri5 / Tsit5, the
+// thread loads its sample's rows once, into registers, and everything below works from there.
+template <typename TT, typename T, int METHOD, int CTRL, int FC = 0> __global__ void __launch_bounds__(256) finish_kernel(const StepParams<TT, T> p) {
     using Tab = typename TabOf<METHOD>::type;
     constexpr int NS = stages_of(METHOD);
     constexpr bool ESTIMATE = METHOD != TODE_EULER;  // Euler has no error estimate: every step is accepted, the step kept
     if (p.flags[TODE_STEP_FLAG_STOPPED]) return;
     const long long b = (long long)blockIdx.x * 256 + threadIdx.x;
     if (b >= p.batch) return;
-    const int F = p.F, E = p.E;
+    const int F = FC > 0 ? FC : p.F, E = p.E;
     const CtrlParams<T> &cp = p.cp;
     const bool fused = F >= 58;
     const T sf = (T)__builtin_sqrt((double)F);
@@ -255,6 +257,20 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     const bool fwd = te > ts;
     const T *y = p.y + b * F;
     T *y1 = p.ystage[6] + b * F;
+    constexpr bool REG = FC > 0 && NS == 7;
+    constexpr int FR = REG ? FC : 1;
+    T k_reg[NS][FR], y_reg[FR], y1_reg[FR];
+    if (REG) {
+#pragma unroll
+        for (int f = 0; f < FR; ++f) {
+            y_reg[f] = y[f], y1_reg[f] = y1[f];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) k_reg[s][f] = p.k[s][b * F + f];
+        }
+    }
+    auto K = [&](int s, int f) -> T { return REG ? k_reg[s][REG ? f : 0] : p.k[s][b * F + f]; };
+    auto Y = [&](int f) -> T { return REG ? y_reg[REG ? f : 0] : y[f]; };
+    auto Y1 = [&](int f) -> T { return REG ? y1_reg[REG ? f : 0] : y1[f]; };
 
     // ---- the step's result where it is not the input of the last stage (heun.py, euler.py; runge_kutta.py:265-269) ----
     if (METHOD == TODE_HEUN) {
@@ -278,12 +294,13 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
 
     // ---- error estimate and error ratio (not looked at by the fixed-step controller) ----
     T acc = 0;
+#pragma unroll
     for (int f = 0; ESTIMATE && CTRL != 2 && f < F; ++f) {
         T err = 0;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             T ps = h * (T)Tab::b_err[s];
-            T ks = p.k[s][b * F + f];
+            T ks = K(s, f);
             if (fused)
                 err = fma_(ps, ks, err);
             else {
@@ -291,7 +308,7 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
                 err = err + pk;
             }
         }
-        T m = tmax(abs_(y[f]), abs_(y1[f]));
+        T m = tmax(abs_(Y(f)), abs_(Y1(f)));
         T eb = fma_(cp.rtol, m, cp.atol);
         T x = (abs_(err) / eb) / sf;
         if (F <= 3)
@@ -336,6 +353,8 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
         const bool mono = p.monotone[b] != 0;
         int cursor = p.cursor[b];
         int e = mono ? cursor : 0;
+        T q_reg[FR][5][1];  // (REG: every feature's interpolant, built when the first point turns out to have been passed)
+        bool built = false;
         for (; e < E; ++e) {
             if (!pend[e]) continue;
             const TT te_e = tev[e];
@@ -344,11 +363,27 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
                 if (mono) break;
                 continue;
             }
-            for (int f = 0; f < F; ++f) {
-                T ks[7] = {};
+            if (REG) {
+                if (!built) {
 #pragma unroll
-                for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
-                ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
+                    for (int f = 0; f < FR; ++f) {
+                        T ks[7];
+#pragma unroll
+                        for (int s = 0; s < 7; ++s) ks[s] = K(s, f);
+                        quartic_elem<T, (METHOD == 1 ? 1 : 0)>(h, Y(f), Y1(f), ks, fused, q_reg[f]);
+                    }
+                    built = true;
+                }
+                const T x = (T)unit_time<TT>(te_e, t0, t0 + dt);
+#pragma unroll
+                for (int f = 0; f < FR; ++f) ys[(long long)e * F + f] = quartic_at<T>(q_reg[f], x);
+            } else {
+                for (int f = 0; f < F; ++f) {
+                    T ks[7] = {};
+#pragma unroll
+                    for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
+                    ys[(long long)e * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te_e);
+                }
             }
             pend[e] = 0;
         }
@@ -357,19 +392,21 @@ template <typename TT, typename T, int METHOD, int CTRL> __global__ void __launc
     } else {
         // no evaluation points: the end-point value of the loop's last interpolant
         // (adjoints.py:295-309); rewritten every iteration, the last one stays
+#pragma unroll
         for (int f = 0; f < F; ++f) {
             T ks[7] = {};
 #pragma unroll
-            for (int s = 0; s < NS; ++s) ks[s] = p.k[s][b * F + f];
-            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, y[f], y1[f], ks, fused, te);
+            for (int s = 0; s < NS; ++s) ks[s] = K(s, f);
+            p.ys[b * F + f] = dense_value<TT, T, METHOD>(t0, dt, Y(f), Y1(f), ks, fused, te);
         }
     }
 
     // ---- state update ----
     if (move) {
+#pragma unroll
         for (int f = 0; f < F; ++f) {
-            p.y[b * F + f] = y1[f];
-            if (NS == 7) p.k0[b * F + f] = p.k[6][b * F + f];  // (first same as last: Dopri5 and Tsit5 only)
+            p.y[b * F + f] = Y1(f);
+            if (NS == 7) p.k0[b * F + f] = K(6, f);  // (first same as last: Dopri5 and Tsit5 only)
         }
     }
     p.t[b] = t_new;
@@ -897,6 +934,13 @@ int tode_step_stage(const tode_step_state *s, const tode_controller *c, int stag
 }
 
 #define TODE_FINISH(KERNEL, M, C) hipLaunchKernelGGL((KERNEL<TT, T, M, C>), dim3(blocks), dim3(256), 0, st, p)
+// (rows of 2, 3 or 4 values with Dopri5 / Tsit5: the thread-per-sample kernel with the row length a template argument)
+#define TODE_FINISH_SHORT(M, FCV)                                                                                          \
+    do {                                                                                                                   \
+        if (c->kind == TODE_CTRL_PID) hipLaunchKernelGGL((finish_kernel<TT, T, M, 1, FCV>), dim3(blocks), dim3(256), 0, st, p);        \
+        else if (c->kind == TODE_CTRL_FIXED) hipLaunchKernelGGL((finish_kernel<TT, T, M, 2, FCV>), dim3(blocks), dim3(256), 0, st, p); \
+        else hipLaunchKernelGGL((finish_kernel<TT, T, M, 0, FCV>), dim3(blocks), dim3(256), 0, st, p);                                 \
+    } while (0)
 // (long rows: the workgroup-per-sample form of the wavefront kernel)
 #define TODE_FINISH_ROWS(M)                                                                                                        \
     do {                                                                                                                           \
@@ -942,6 +986,15 @@ int tode_step_finish(const tode_step_state *s, const tode_controller *c, void *s
             } else if (wide) {
                 if (tsit5) TODE_FINISH_CTRL(finish_wave_kernel, 1);
                 else TODE_FINISH_CTRL(finish_wave_kernel, 0);
+            } else if (s->n_features == 2) {
+                if (tsit5) TODE_FINISH_SHORT(1, 2);
+                else TODE_FINISH_SHORT(0, 2);
+            } else if (s->n_features == 3) {
+                if (tsit5) TODE_FINISH_SHORT(1, 3);
+                else TODE_FINISH_SHORT(0, 3);
+            } else if (s->n_features == 4) {
+                if (tsit5) TODE_FINISH_SHORT(1, 4);
+                else TODE_FINISH_SHORT(0, 4);
             } else {
                 if (tsit5) TODE_FINISH_CTRL(finish_kernel, 1);
                 else TODE_FINISH_CTRL(finish_kernel, 0);
