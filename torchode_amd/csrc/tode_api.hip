@@ -29,6 +29,7 @@ int check_hip(hipError_t err, const char *what) {
 }
 
 static thread_local int g_fast_variant = 0;
+bool fast_output_sliced() { return g_fast_variant == 3; }
 static thread_local bool g_timing = false;
 static thread_local bool g_timed = false;
 static thread_local hipEvent_t g_ev[2] = {nullptr, nullptr};
@@ -212,7 +213,8 @@ const char *tode_source_hash(void) { return TODE_SOURCE_HASH; }
 const char *tode_last_error(void) { return tode::g_error; }
 
 int tode_set_fast_kernel_variant(int variant) {
-    if (variant < 0 || variant > 2) return tode::fail(TODE_E_INVALID, "variant must be 0 (auto), 1 (one wavefront) or 2 (two wavefronts)");
+    if (variant < 0 || variant > 3)
+        return tode::fail(TODE_E_INVALID, "variant must be 0 (auto), 1 (one wavefront), 2 (two wavefronts) or 3 (one wavefront, evaluation points stored four at a time)");
     tode::g_fast_variant = variant;
     return TODE_OK;
 }
@@ -295,7 +297,7 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         if (end_only) return fail(TODE_E_UNSUPPORTED, "a record from the fast entry point needs evaluation points");
         return a->dtype == TODE_F32 ? solve_fast_f32_record(*a, *c, ns, na, ni, st, s) : solve_fast_f64_record(*a, *c, ns, na, ni, st, s);
     }
-    if (g_fast_variant != 1) {
+    if (g_fast_variant == 0 || g_fast_variant == 2) {
         // small batches: two wavefronts per group of 64 samples (stepper + dense-output evaluator)
         bool used = false;
         int rc = a->dtype == TODE_F32 ? solve_pair_f32(*a, *c, ns, na, ni, st, s, &used) : solve_pair_f64(*a, *c, ns, na, ni, st, s, &used);
