@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     r[(4 + f) * 64] = y[f];
-                    r[(4 + F + f) * 64] = y1[f];
+                    if (METHOD != 1) r[(4 + F + f) * 64] = y1[f];  // (Tsit5's interpolant does not look at the step's result)
                 }
 #pragma unroll
                 for (int s = 0; s < 7; ++s)
@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
 #pragma unroll
                     for (int f = 0; f < F; ++f) {
                         y[f] = r[(4 + f) * 64];
-                        y1[f] = r[(4 + F + f) * 64];
+                        y1[f] = METHOD != 1 ? r[(4 + F + f) * 64] : (T)0;
                     }
 #pragma unroll
                     for (int s = 0; s < 7; ++s)
