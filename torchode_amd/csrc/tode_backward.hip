@@ -199,6 +199,13 @@ __global__ void __launch_bounds__(64) whole_backward_kernel(const WholeBackward<
         const RecordEntry<T, F> before = load_entry<T, F>(w, i > 0 ? i - 1 : 0, g);  // (used by the next pass of this loop)
         q.iteration = (int)i;
         q.end_point = (E == 0 && i == L - 1) ? 1 : 0;
+        // An iteration that none of the wavefront's samples took part in (all had finished before it) changes nothing for
+        // them -- no move, no point written, the step and the history kept -- so its reverse hands every cotangent on as
+        // it is.  (Without evaluation points the batch's last iteration is the one whose interpolant gives the result.)
+        if (!q.end_point && !__any(here.running != 0)) {
+            after = here, here = before;
+            continue;
+        }
         t0 = here.t, dt = here.dt, prev = here.prev, pprev = here.pprev;
         moved = (after.n_accepted - here.n_accepted) > 0 ? 1 : 0;
         running_next = after.running != 0 ? 1 : 0;
