@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 21
+#define TODE_ABI_VERSION 22
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -45,8 +45,8 @@ enum {
     TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
     TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 16, 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
                                          float32, tode_solve_builtin_fast only */
-    TODE_TERM_MLP = 4                 /* F = 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units, weights in
-                                         shared_params as packed by tode_mlp_pack_weights; float32,
+    TODE_TERM_MLP = 4                 /* F = 4, 8, ..., 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units,
+                                         weights in shared_params as packed by tode_mlp_pack_weights[_for]; float32,
                                          tode_solve_builtin_fast only */
 };
 /* what the matrix cores take as inputs in the MLP kernel; accumulation, biases, tanh and the solver are float32 */
@@ -366,6 +366,19 @@ int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int6
  * weights, not per solve.
  */
 int tode_mlp_pack_weights(const void *raw, int64_t n_raw, int32_t matrix_inputs, void *packed, void *stream);
+
+/*
+ * The same for a network on n_features = 4, 8, ..., 64 state values (the solve
+ * then takes n_features of that size and rows of that many values in y0 and
+ * ys): `raw` is W1 [H x (n_features + 1)] | b1 [H] | W2 [n_features x H] |
+ * b2 [n_features], n_raw = (2 n_features + 2) H + n_features.  The kernel always
+ * works on 64 values per sample: the state values from n_features on are zero,
+ * their weights are packed as zeros, and the root mean squares divide by
+ * n_features, so the sums hold only exact zeros beyond the network's own terms.
+ * `packed` has the same size as for 64 features.
+ * tode_mlp_pack_weights(...) == tode_mlp_pack_weights_for(..., 64, ...).
+ */
+int tode_mlp_pack_weights_for(const void *raw, int64_t n_raw, int32_t n_features, int32_t matrix_inputs, void *packed, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Per-step kernels around a right-hand side that lives outside the library   */

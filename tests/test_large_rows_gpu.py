@@ -347,6 +347,79 @@ def test_mlp_kernel_with_fewer_hidden_units(hidden, inputs):
         assert torch.equal(a.status, proto.status) and mixed_error(a.ys.double().cpu(), proto.ys.double().cpu()) < 5e-2
 
 
+def narrow_mlp_problem(features, hidden, batch, inputs="float32", seed=0):
+    """A two-layer network on `features` state values with its own start values and evaluation points."""
+    import torchode_amd.builtin_terms as bt
+
+    g = torch.Generator().manual_seed(1000 * features + hidden + seed)
+    scale1, scale2 = (6.0 / (features + 1 + hidden)) ** 0.5, (6.0 / (hidden + features)) ** 0.5
+    W1 = ((torch.rand(hidden, features + 1, generator=g) * 2 - 1) * scale1).cuda()
+    W2 = ((torch.rand(features, hidden, generator=g) * 2 - 1) * scale2).cuda()
+    b1, b2 = (torch.rand(hidden, generator=g) - 0.5).cuda() * 0.1, (torch.rand(features, generator=g) - 0.5).cuda() * 0.1
+    w = to.workloads.make("mlp", batch=batch, device="cuda")
+    y0 = (torch.rand(batch, features, generator=g) * 2 - 1).cuda()
+    return w._replace(f=bt.MLPField(W1, b1, W2, b2, matrix_inputs=inputs), y0=y0)
+
+
+@pytest.mark.parametrize("inputs", ["float32", "bfloat16"])
+@pytest.mark.parametrize("features,hidden,batch", [(4, 256, 96), (8, 5, 37), (32, 100, 96), (48, 256, 250), (60, 64, 96)])
+def test_mlp_kernel_with_fewer_features(features, hidden, batch, inputs):
+    """The kernel works on 64 values per sample; a network on 4, 8, ..., 60 of them is packed with zero weights for the
+    rest, whose state stays zero, and the root mean squares divide by the network's own count: against the protocol
+    path with torch's matrix products of the network itself."""
+    w = narrow_mlp_problem(features, hidden, batch, inputs)
+    kernel = "tode::solve_mlp_kernel" + ("" if inputs == "float32" else " (bfloat16 matrix inputs)")
+    tight = dict(kind="pid", atol=1e-6, rtol=1e-4, pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    for method, ctrl in ((w.method, w.controller), ("tsit5", tight)):
+        a, proto = mlp_both_paths(w, method, ctrl, kernel=kernel)
+        assert a.ys.shape == (batch, 20, features) and (a.stats["n_initialized"] == 20).all()
+        assert torch.equal(a.status, proto.status)
+        if inputs == "bfloat16":
+            assert mixed_error(a.ys.double().cpu(), proto.ys.double().cpu()) < 5e-2
+        elif ctrl is tight:
+            # (as with 64 features at this tolerance: up to a tenth of the samples accept or reject differently at the
+            # rounding noise of the matrix products; both pipelines then meet the tolerance with about the same work)
+            assert mixed_error(a.ys.double().cpu(), proto.ys.double().cpu()) < 1e-4
+            assert 0.8 < a.stats["n_steps"].sum().item() / proto.stats["n_steps"].sum().item() < 1.25
+        else:
+            assert_close_solutions(a, proto, min_agree=0.95, loose=1e-2)
+
+
+def test_mlp_weight_packing_with_fewer_features():
+    """tode_mlp_pack_weights_for on an 8-feature network against tode_mlp_pack_weights on the same network written out
+    on 64 features (zero columns and rows for the others, the time in input 64): same words, in both formats.  Sizes
+    that the kernel does not take are refused, by the library and by the choice of path."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    w = narrow_mlp_problem(8, 5, 16)
+    f = w.f
+    W1 = torch.zeros(5, 65, device="cuda")
+    W1[:, :8], W1[:, 64] = f.W1[:, :8], f.W1[:, 8]
+    W2, b2 = torch.zeros(64, 5, device="cuda"), torch.zeros(64, device="cuda")
+    W2[:8], b2[:8] = f.W2, f.b2
+    wide = torch.cat([x.reshape(-1) for x in (W1, f.b1, W2, b2)]).contiguous()
+    raw = f.builtin_shared()
+    for inputs in ("float32", "bfloat16"):
+        n = _lib.MLP_PACKED_SIZE[inputs]
+        a, b = torch.full((n,), 7.0, device="cuda"), torch.full((n,), 9.0, device="cuda")
+        _lib.check(lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel(), 8, _lib.MLP_INPUTS[inputs], _lib.ptr(a), _lib.stream_of(raw)), "pack")
+        _lib.check(lib.tode_mlp_pack_weights(_lib.ptr(wide), wide.numel(), _lib.MLP_INPUTS[inputs], _lib.ptr(b), _lib.stream_of(raw)), "pack")
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), inputs
+    for n_features in (0, 6, 68):
+        assert lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel(), n_features, 0, _lib.ptr(a), _lib.stream_of(raw)) == _lib.E_UNSUPPORTED
+    assert lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel() - 1, 8, 0, _lib.ptr(a), _lib.stream_of(raw)) == _lib.E_UNSUPPORTED
+    # six features: not a size of the matrix-core kernel, the solve takes the per-step kernels and still agrees
+    v = to.workloads.make("vdp", batch=8, device="cuda")  # (another solve first: the library keeps the last kernel's name)
+    to.AutoDiffAdjoint(to.Dopri5(), make_controller(v.controller)).solve(to.InitialValueProblem(v.y0, t_eval=v.t_eval), to.ODETerm(v.f))
+    odd = narrow_mlp_problem(6, 16, 24)
+    problem = to.InitialValueProblem(odd.y0, t_eval=odd.t_eval)
+    got = to.AutoDiffAdjoint(to.Dopri5(), make_controller(odd.controller)).solve(problem, to.ODETerm(odd.f))
+    want = to.AutoDiffAdjoint(OwnDopri5(), make_controller(odd.controller)).solve(problem, to.ODETerm(odd.f))
+    assert not _lib.last_solve_kernel_name().startswith("tode::solve_mlp_kernel")
+    assert_close_solutions(got, want, min_agree=0.95, loose=1e-2)
+
+
 @pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "pid"), ("tsit5", "integral")])
 def test_mlp_kernel_with_tight_tolerances(method, kind):
     """At rtol 1e-6 every error estimate sits at the rounding noise of the float32 matrix products, so

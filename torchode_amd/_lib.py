@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -44,6 +44,7 @@ EXPORTS = (
     "tode_solve_backward_scratch_bytes",
     "tode_solve_workspace_bytes",
     "tode_mlp_pack_weights",
+    "tode_mlp_pack_weights_for",
     "tode_select_end_point",
     "tode_step_begin",
     "tode_step_stage",
@@ -332,6 +333,8 @@ def load():
         lib.tode_select_end_point.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.tode_mlp_pack_weights.restype = C.c_int
         lib.tode_mlp_pack_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
+        lib.tode_mlp_pack_weights_for.restype = C.c_int
+        lib.tode_mlp_pack_weights_for.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
         lib.tode_solve_builtin_fast_static.restype = C.c_int
         lib.tode_solve_builtin_fast_static.argtypes = [C.POINTER(SolveArgs), C.POINTER(Controller)] + [C.c_void_p] * 6
         lib.tode_solve_builtin_fast_sync.restype = C.c_int

@@ -161,7 +161,7 @@ class AutoDiffAdjoint(nn.Module):
         dtype, B, E = problem.data_dtype, problem.batch_size, problem.n_evaluation_points
         mlp = f.builtin_kind == _lib.TERM_MLP
         params = None if mlp else f.builtin_params().to(dtype)
-        shared = ops.mlp_pack_weights(f.builtin_shared().to(dtype), _lib.MLP_INPUTS[f.matrix_inputs]) if mlp else None
+        shared = ops.mlp_pack_weights(f.builtin_shared().to(dtype), _lib.MLP_INPUTS[f.matrix_inputs], problem.n_features) if mlp else None
         scalars = [float(x) for x in getattr(f, "builtin_scalars", lambda: ())()]
         ys, n_steps, n_accepted, n_initialized, status, iterations = ops.solve_builtin(
             problem.y0, problem.t_start, problem.t_end, problem.t_eval, dt0, params, shared, self.step_method.method_id, f.builtin_kind,
@@ -185,7 +185,7 @@ class AutoDiffAdjoint(nn.Module):
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
             return F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192
-        return F == 64 and f.W1.shape[1] == 65 and 1 <= f.W1.shape[0] <= 256 and E <= 512
+        return 4 <= F <= 64 and F % 4 == 0 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable
     def _solve_eager_outside_the_trace(self, problem, term, dt0, args) -> Solution:
@@ -575,8 +575,10 @@ class AutoDiffAdjoint(nn.Module):
             params = y0.new_empty((B, 0))
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
         mlp = f.builtin_kind == _lib.TERM_MLP
-        if mlp and (dtype != torch.float32 or F != 64 or f.W1.shape[1] != 65 or not 1 <= f.W1.shape[0] <= 256):
-            return None  # the matrix-core kernel is built for 64 features and up to 256 hidden units: the caller takes another path
+        if mlp and (
+            dtype != torch.float32 or not 4 <= F <= 64 or F % 4 or f.W1.shape[1] != F + 1 or not 1 <= f.W1.shape[0] <= 256
+        ):
+            return None  # the matrix-core kernel takes 4, 8, ..., 64 features and up to 256 hidden units: the caller takes another path
         shared = f.builtin_packed(dev, dtype) if mlp else None
         ttype = t_start.dtype
         dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()

@@ -171,9 +171,10 @@ class MLPField(BuiltinTerm):
         if getattr(self, "_packed_key", None) != key:
             raw = self.builtin_shared().to(device=device, dtype=dtype)
             packed = torch.empty(_lib.MLP_PACKED_SIZE[self.matrix_inputs], dtype=dtype, device=device)
-            rc = _lib.load().tode_mlp_pack_weights(
-                _lib.ptr(raw), raw.numel(), _lib.MLP_INPUTS[self.matrix_inputs], _lib.ptr(packed), _lib.stream_of(raw)
+            rc = _lib.load().tode_mlp_pack_weights_for(
+                _lib.ptr(raw), raw.numel(), self.W2.shape[0], _lib.MLP_INPUTS[self.matrix_inputs], _lib.ptr(packed),
+                _lib.stream_of(raw),
             )
-            _lib.check(rc, "tode_mlp_pack_weights")
+            _lib.check(rc, "tode_mlp_pack_weights_for")
             self._packed, self._packed_key = packed, key
         return self._packed

@@ -311,7 +311,11 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
 }
 
 int tode_mlp_pack_weights(const void *raw, int64_t n_raw, int32_t matrix_inputs, void *packed, void *stream) {
-    return tode::mlp_pack_weights((const float *)raw, (long long)n_raw, matrix_inputs, (float *)packed, (hipStream_t)stream);
+    return tode::mlp_pack_weights((const float *)raw, (long long)n_raw, 64, matrix_inputs, (float *)packed, (hipStream_t)stream);
+}
+
+int tode_mlp_pack_weights_for(const void *raw, int64_t n_raw, int32_t n_features, int32_t matrix_inputs, void *packed, void *stream) {
+    return tode::mlp_pack_weights((const float *)raw, (long long)n_raw, n_features, matrix_inputs, (float *)packed, (hipStream_t)stream);
 }
 
 int tode_solve_builtin_fast_sync(const tode_solve_args *a, const tode_controller *c, int64_t *ns, int64_t *na, int64_t *ni,
@@ -510,7 +514,7 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
         if (a->term == TODE_TERM_REACTION_DIFFUSION)
             one_kernel = one_kernel && (a->n_features == 16 * 16 || a->n_features == 32 * 32 || a->n_features == 64 * 64) && E <= 8192;
         else if (a->term == TODE_TERM_MLP)
-            one_kernel = one_kernel && a->n_features == 64 && E <= 512;
+            one_kernel = one_kernel && a->n_features >= 4 && a->n_features <= 64 && a->n_features % 4 == 0 && E <= 512;
         else
             return fail(TODE_E_INVALID, "unknown term %d", a->term);
         if (!one_kernel) return fail(TODE_E_UNSUPPORTED, "no whole-solve kernel for this term in this shape, dtype or controller setting");

@@ -36,6 +36,7 @@ typedef float mfma_acc __attribute__((ext_vector_type(4)));
 
 struct MlpOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
+    int n_features;  // features of the problem: a multiple of four, at most 64 (the kernel's others stay zero)
 };
 
 constexpr int MLP_F = 64, MLP_H = 256, MLP_TILE = 16;
@@ -76,12 +77,16 @@ __host__ __device__ __forceinline__ int mlp_input_of(int kk, int q) { return kk 
 // Source index (in W1 | b1 | W2 | b2, row-major) of packed value j of thread tid, or -1 for zero.  H: hidden units of
 // the network at hand, at most MLP_H; the kernel's units from H on get zero weights and a zero bias, so that they
 // add tanh(0) * 0 = 0 to every sum in the same places as before (a narrower network in the same arithmetic).
-__host__ __device__ inline long long mlp_packed_source(int j, int tid, int H) {
+// FR: features of the network at hand (a multiple of four, at most MLP_F): W1 is [H x (FR + 1)] with the time in its last
+// column, W2 [FR x H]; the kernel's features from FR on get zero weights on both sides and stay zero throughout.
+__host__ __device__ inline long long mlp_packed_source(int j, int tid, int H, int FR) {
     const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
-    const long long o_b1 = (long long)H * (MLP_F + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)MLP_F * H;
+    const long long o_b1 = (long long)H * (FR + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)FR * H;
+    // column of W1 for the kernel's input k (features 0..63, then the time at 64), or -1
+    auto w1_column = [&](int k) { return k < FR ? k : (k == MLP_F ? FR : -1); };
     if (j < 68) {
-        const int kk = j / 4, tile = j % 4, k = mlp_input_of(kk, q), unit = 64 * w + 16 * tile + c;
-        return (k <= MLP_F && unit < H) ? (long long)unit * (MLP_F + 1) + k : -1;
+        const int kk = j / 4, tile = j % 4, col = w1_column(mlp_input_of(kk, q)), unit = 64 * w + 16 * tile + c;
+        return (col >= 0 && unit < H) ? (long long)unit * (FR + 1) + col : -1;
     }
     j -= 68;
     if (j < 16) {
@@ -91,23 +96,24 @@ __host__ __device__ inline long long mlp_packed_source(int j, int tid, int H) {
     j -= 16;
     if (j < 64) {
         const int ft = j / 16, tile = (j / 4) % 4, r = j % 4, unit = 64 * w + 16 * tile + 4 * q + r;
-        return unit < H ? o_w2 + (long long)(16 * ft + c) * H + unit : -1;
+        return (unit < H && 16 * ft + c < FR) ? o_w2 + (long long)(16 * ft + c) * H + unit : -1;
     }
     j -= 64;
-    return o_b2 + 16 * w + 4 * q + j;
+    return 16 * w + 4 * q + j < FR ? o_b2 + 16 * w + 4 * q + j : -1;
 }
 
 // The same for the bfloat16 variant: packed word j of thread tid holds the values of sources
 // (lo, hi) as bfloat16 in its low and high half (words of b1 and b2: one float32, hi = -2).
-__host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, int H, long long &lo, long long &hi) {
+__host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, int H, int FR, long long &lo, long long &hi) {
     const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
-    const long long o_b1 = (long long)H * (MLP_F + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)MLP_F * H;
+    const long long o_b1 = (long long)H * (FR + 1), o_w2 = o_b1 + H, o_b2 = o_w2 + (long long)FR * H;
+    auto w1_column = [&](int k) { return k < FR ? k : (k == MLP_F ? FR : -1); };
     hi = -2;
     if (j < 40) {
         const int ks = j / 8, tile = (j / 2) % 4, k = 16 * ks + 4 * q + 2 * (j % 2), unit = 64 * w + 16 * tile + c;
-        const long long row = (long long)unit * (MLP_F + 1);
-        lo = (k <= MLP_F && unit < H) ? row + k : -1;
-        hi = (k + 1 <= MLP_F && unit < H) ? row + k + 1 : -1;
+        const long long row = (long long)unit * (FR + 1);
+        lo = (w1_column(k) >= 0 && unit < H) ? row + w1_column(k) : -1;
+        hi = (w1_column(k + 1) >= 0 && unit < H) ? row + w1_column(k + 1) : -1;
         return;
     }
     j -= 40;
@@ -121,20 +127,20 @@ __host__ __device__ inline void mlp_packed_source_bf16(int j, int tid, int H, lo
     if (j < 32) {
         const int ft = j / 8, tile = (j / 2) % 4, unit = 64 * w + 16 * tile + 4 * q + 2 * (j % 2);
         const long long at = o_w2 + (long long)(16 * ft + c) * H + unit;
-        lo = unit < H ? at : -1;
-        hi = unit + 1 < H ? at + 1 : -1;
+        lo = (unit < H && 16 * ft + c < FR) ? at : -1;
+        hi = (unit + 1 < H && 16 * ft + c < FR) ? at + 1 : -1;
         return;
     }
     j -= 32;
-    lo = o_b2 + 16 * w + 4 * q + j;
+    lo = 16 * w + 4 * q + j < FR ? o_b2 + 16 * w + 4 * q + j : -1;
 }
 
-static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed, int H) {
+static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed, int H, int FR) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= MLP_REGS_BF16 * 256) return;
     const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
     long long lo, hi;
-    mlp_packed_source_bf16(4 * group + part, tid, H, lo, hi);
+    mlp_packed_source_bf16(4 * group + part, tid, H, FR, lo, hi);
     if (hi == -2 || hi == -3) {
         packed[i] = lo < 0 ? 0u : __float_as_uint(raw[lo]);
         return;
@@ -143,11 +149,11 @@ static __global__ void mlp_pack_bf16_kernel(const float *raw, unsigned *packed, 
     packed[i] = (unsigned)__builtin_bit_cast(unsigned short, a) | ((unsigned)__builtin_bit_cast(unsigned short, b) << 16);
 }
 
-static __global__ void mlp_pack_kernel(const float *raw, float *packed, int H) {
+static __global__ void mlp_pack_kernel(const float *raw, float *packed, int H, int FR) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= MLP_REGS * 256) return;
     const int part = i % 4, tid = (i / 4) % 256, group = i / 1024;
-    const long long src = mlp_packed_source(4 * group + part, tid, H);
+    const long long src = mlp_packed_source(4 * group + part, tid, H, FR);
     packed[i] = src < 0 ? 0.0f : raw[src];
 }
 
@@ -341,8 +347,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int rows = (int)min((long long)MLP_TILE, p.batch - b0);
     const int E = p.n_eval;
     const CtrlParams<T> &cp = p.cp;
-    const T sf = (T)__builtin_sqrt((double)F);
+    const int FR = o.n_features;  // the problem's features; the kernel's others (FR .. 63) are zero in every vector
+    const T sf = (T)__builtin_sqrt((double)FR);
     const int f0 = 16 * w + 4 * q;  // the lane's first feature
+    const bool has = f0 < FR;       // (FR is a multiple of four: the lane's four features are the problem's, or none is)
     int slot = 0;
 
     // ---- weights into registers ----
@@ -362,7 +370,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int e = 1; e < E; ++e) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));  // not monotone
     T y[4], k[7][4];
     {
-        const float4 v = *reinterpret_cast<const float4 *>(p.y0 + bs * F + f0);
+        const float4 v = has ? *reinterpret_cast<const float4 *>(p.y0 + bs * FR + f0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         y[0] = v.x, y[1] = v.y, y[2] = v.z, y[3] = v.w;
     }
     T t = ts, dt, prev = 1, pprev = 1;
@@ -399,7 +407,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     dt = tclamp(dt, tlo - t, thi - t);
     bool active = live;
     if (live && E > 0 && tev[0] == ts) {
-        *reinterpret_cast<float4 *>(p.ys + (bs * E) * F + f0) = make_float4(y[0], y[1], y[2], y[3]);
+        if (has) *reinterpret_cast<float4 *>(p.ys + (bs * E) * FR + f0) = make_float4(y[0], y[1], y[2], y[3]);
         cursor = 1;
     }
     int vslot = 0;
@@ -470,7 +478,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
                     for (int pw = 3; pw >= 0; --pw) v[r] = fma_(v[r], x, qc[r][pw][0]);
                 }
-                *reinterpret_cast<float4 *>(p.ys + (bs * E + cursor) * F + f0) = make_float4(v[0], v[1], v[2], v[3]);
+                if (has) *reinterpret_cast<float4 *>(p.ys + (bs * E + cursor) * FR + f0) = make_float4(v[0], v[1], v[2], v[3]);
                 ++cursor;
             } while (cursor < E && fma_(dir, t_new, -dir * tev[cursor]) >= (T)0);
         }
@@ -536,29 +544,32 @@ template <typename Weights> static int solve_mlp_with(const tode_solve_args &a, 
 
 int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
     const bool f32 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE, bf16 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE_BF16;
-    if (a.n_features != MLP_F || !(f32 || bf16))
+    if (a.n_features < 4 || a.n_features > MLP_F || a.n_features % 4 != 0 || !(f32 || bf16))
         return fail(TODE_E_UNSUPPORTED,
-                    "the MLP kernel is built for 64 features and up to 256 hidden units, with the weights packed by tode_mlp_pack_weights "
+                    "the MLP kernel is built for 4, 8, ..., 64 features and up to 256 hidden units, with the weights packed by tode_mlp_pack_weights "
                     "(%d or %d values); got F=%d and %lld shared parameters", TODE_MLP_PACKED_SIZE, TODE_MLP_PACKED_SIZE_BF16, a.n_features,
                     (long long)a.n_shared_params);
     if (!a.shared_params) return fail(TODE_E_INVALID, "null shared_params");
     if (a.n_eval > 512) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the MLP kernel", a.n_eval);
     if (a.batch > (long long)INT_MAX * MLP_TILE) return fail(TODE_E_UNSUPPORTED, "batch too large");
-    MlpOut o{ns, na, ni, st};
+    MlpOut o{ns, na, ni, st, a.n_features};
     return f32 ? solve_mlp_with<MlpWeights>(a, c, o, s) : solve_mlp_with<MlpWeightsBf16>(a, c, o, s);
 }
 
-int mlp_pack_weights(const float *raw, long long n_raw, int matrix_inputs, float *packed, hipStream_t s) {
+int mlp_pack_weights(const float *raw, long long n_raw, int n_features, int matrix_inputs, float *packed, hipStream_t s) {
     static_assert(TODE_MLP_PACKED_SIZE == MLP_REGS * 256 && TODE_MLP_PACKED_SIZE_BF16 == MLP_REGS_BF16 * 256, "packed sizes");
     if (!raw || !packed) return fail(TODE_E_INVALID, "null pointer");
-    // W1 [H x 65] | b1 [H] | W2 [64 x H] | b2 [64] = 130 H + 64 values for H hidden units, 1 <= H <= 256
-    const long long H = (n_raw - MLP_F) / (2 * MLP_F + 2);
-    if (n_raw < MLP_F || H * (2 * MLP_F + 2) + MLP_F != n_raw || H < 1 || H > MLP_H)
-        return fail(TODE_E_UNSUPPORTED, "expected W1 [H x 65] | b1 [H] | W2 [64 x H] | b2 [64] = 130 H + 64 values with 1 <= H <= %d, got %lld", MLP_H, n_raw);
+    const long long FR = n_features;
+    if (FR < 4 || FR > MLP_F || FR % 4 != 0) return fail(TODE_E_UNSUPPORTED, "the MLP kernel takes 4, 8, ..., %d features, got %lld", MLP_F, FR);
+    // W1 [H x (F + 1)] | b1 [H] | W2 [F x H] | b2 [F] = (2 F + 2) H + F values for H hidden units, 1 <= H <= 256
+    const long long H = (n_raw - FR) / (2 * FR + 2);
+    if (n_raw < FR || H * (2 * FR + 2) + FR != n_raw || H < 1 || H > MLP_H)
+        return fail(TODE_E_UNSUPPORTED, "expected W1 [H x %lld] | b1 [H] | W2 [%lld x H] | b2 [%lld] = %lld H + %lld values with 1 <= H <= %d, got %lld", FR + 1, FR, FR,
+                    2 * FR + 2, FR, MLP_H, n_raw);
     if (matrix_inputs == TODE_MLP_INPUTS_F32)
-        hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed, (int)H);
+        hipLaunchKernelGGL(mlp_pack_kernel, dim3((MLP_REGS * 256 + 255) / 256), dim3(256), 0, s, raw, packed, (int)H, (int)FR);
     else if (matrix_inputs == TODE_MLP_INPUTS_BF16)
-        hipLaunchKernelGGL(mlp_pack_bf16_kernel, dim3((MLP_REGS_BF16 * 256 + 255) / 256), dim3(256), 0, s, raw, reinterpret_cast<unsigned *>(packed), (int)H);
+        hipLaunchKernelGGL(mlp_pack_bf16_kernel, dim3((MLP_REGS_BF16 * 256 + 255) / 256), dim3(256), 0, s, raw, reinterpret_cast<unsigned *>(packed), (int)H, (int)FR);
     else
         return fail(TODE_E_INVALID, "unknown matrix input type %d", matrix_inputs);
     return check_hip(hipGetLastError(), "tode_mlp_pack_weights launch");

@@ -97,15 +97,15 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> solve_builtin(const T
     return {ys, n_steps, n_accepted, n_initialized, status, at::scalar_tensor(iterations, at::TensorOptions().dtype(at::kLong))};
 }
 
-// tode_mlp_pack_weights: W1 | b1 | W2 | b2 concatenated -> the order the MLP kernel loads them in.
-Tensor mlp_pack_weights(const Tensor &raw, int64_t matrix_inputs) {
+// tode_mlp_pack_weights_for: W1 | b1 | W2 | b2 concatenated -> the order the MLP kernel loads them in.
+Tensor mlp_pack_weights(const Tensor &raw, int64_t matrix_inputs, int64_t n_features) {
     TORCH_CHECK(raw.is_cuda() && raw.scalar_type() == at::kFloat && raw.dim() == 1, "torchode_amd::mlp_pack_weights takes a float32 vector on the GPU");
     TORCH_CHECK(matrix_inputs == TODE_MLP_INPUTS_F32 || matrix_inputs == TODE_MLP_INPUTS_BF16, "unknown matrix input kind ", matrix_inputs);
     const Tensor raw_c = raw.contiguous();
     const c10::DeviceGuard guard(raw.device());
     Tensor packed = at::empty({matrix_inputs == TODE_MLP_INPUTS_BF16 ? TODE_MLP_PACKED_SIZE_BF16 : TODE_MLP_PACKED_SIZE}, raw.options());
-    const int rc = tode_mlp_pack_weights(raw_c.data_ptr(), raw_c.numel(), (int32_t)matrix_inputs, packed.data_ptr(),
-                                         (void *)c10::hip::getCurrentHIPStream(raw.device().index()).stream());
+    const int rc = tode_mlp_pack_weights_for(raw_c.data_ptr(), raw_c.numel(), (int32_t)n_features, (int32_t)matrix_inputs, packed.data_ptr(),
+                                             (void *)c10::hip::getCurrentHIPStream(raw.device().index()).stream());
     TORCH_CHECK(rc == TODE_OK, "torchode_amd::mlp_pack_weights: ", tode_last_error(), " (code ", rc, ")");
     return packed;
 }
@@ -113,7 +113,7 @@ Tensor mlp_pack_weights(const Tensor &raw, int64_t matrix_inputs) {
 }  // namespace
 
 TORCH_LIBRARY(torchode_amd, m) {
-    m.def("mlp_pack_weights(Tensor raw, int matrix_inputs) -> Tensor");
+    m.def("mlp_pack_weights(Tensor raw, int matrix_inputs, int n_features=64) -> Tensor");
     m.def(
         "solve_builtin(Tensor y0, Tensor t_start, Tensor t_end, Tensor? t_eval, Tensor? dt0, Tensor? params, Tensor? shared_params, int method, int term, "
         "float[] term_scalars, int controller_kind, float[] control, int max_steps, bool allow_one_kernel) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");

@@ -49,7 +49,7 @@ def _load_once() -> None:
             return y0.new_empty((B, E, F)), stat(), stat(), stat(), stat(), torch.empty((), dtype=torch.long, device="cpu")
 
         @torch.library.register_fake("torchode_amd::mlp_pack_weights")
-        def _(raw, matrix_inputs):
+        def _(raw, matrix_inputs, n_features=64):
             return raw.new_empty((_lib.MLP_PACKED_SIZE["bfloat16" if matrix_inputs == _lib.MLP_INPUTS["bfloat16"] else "float32"],))
 
         _loaded = True
@@ -81,6 +81,6 @@ def solve_builtin(
     )  # fmt: skip
 
 
-def mlp_pack_weights(raw: torch.Tensor, matrix_inputs: int) -> torch.Tensor:
+def mlp_pack_weights(raw: torch.Tensor, matrix_inputs: int, n_features: int = 64) -> torch.Tensor:
     load()
-    return torch.ops.torchode_amd.mlp_pack_weights(raw, matrix_inputs)
+    return torch.ops.torchode_amd.mlp_pack_weights(raw, matrix_inputs, n_features)
