@@ -466,6 +466,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
                 T ks[7];
 #pragma unroll
                 for (int s = 0; s < 7; ++s) ks[s] = k[s][r];
+                // (one fused chain per coefficient, ATen's form for rows of 58 values and more; for a shorter row ATen rounds
+                // the products first, a difference at the level of this kernel's matrix products against torch's)
                 quartic_elem<T, METHOD>(dt, y[r], y1[r], ks, true, qc[r]);
             }
             const T t1 = t0 + dt;
