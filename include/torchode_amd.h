@@ -223,9 +223,13 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
  * On return (after stream synchronisation) flags[TODE_FLAG_MAX_ITERATIONS] is
  * the loop's iteration count, and flags[TODE_FLAG_NEEDS_GENERAL] == 1 means the
  * batch left the common case (a non-success status, max_steps reached, a t_eval
- * row that is not monotone in its direction of time, or a sample that ended
- * past t_end); every output is then unspecified and the caller must repeat the
- * solve with tode_solve_builtin.  Results are bit-identical to
+ * row that is not monotone in its direction of time, a sample that ended on a
+ * non-finite state or, with n_eval == 0, past t_end); every output is then
+ * unspecified and the caller must repeat the solve with tode_solve_builtin.
+ * (With evaluation points a sample that lands past t_end, t + (t_end - t)
+ * rounded upwards, stays in the kernel: the reference steps it once more with
+ * the step t_end - t, which shows in that step's status alone, and the kernel
+ * computes that step and looks at its error ratio.)  Results are bit-identical to
  * tode_solve_builtin + tode_finalize_stats whenever the flag stays 0.
  * Returns TODE_E_UNSUPPORTED for dt_min / dt_max, or n_eval too large for
  * on-chip staging.

@@ -247,6 +247,50 @@ def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():
     assert_same(sol, ref)
 
 
+def spans_that_miss_t_end(batch, E, seed, scale=1.0):
+    """Per-sample time spans from t_start in (-2, -1) to a small positive t_end: the last step's length t_end - t is
+    rounded, and t + (t_end - t) lands one unit in the last place past t_end for about a quarter of the samples (a
+    span [0, T] never does that).  Evaluation points evenly spaced from t_start to t_end, both included exactly."""
+    g = torch.Generator().manual_seed(seed)
+    t_start = -(1.0 + torch.rand(batch, generator=g)) * scale
+    t_end = (0.01 + 0.3 * torch.rand(batch, generator=g)) * scale
+    t_eval = t_start[:, None] + (t_end - t_start)[:, None] * torch.linspace(0, 1, E)[None, :]
+    t_eval[:, 0], t_eval[:, -1] = t_start, t_end
+    return t_start, t_end, t_eval
+
+
+def test_grid_and_mlp_kernels_keep_samples_that_land_past_t_end(monkeypatch):
+    """A sample whose last step lands past t_end takes part in the reference's later iterations with the step
+    t_end - t; the whole-solve kernels compute that step once and look at its status instead of giving the batch up
+    (which sent it to the per-step kernels)."""
+    from torchode_amd import _lib
+
+    def no_other_path(*a, **kw):
+        raise AssertionError("the whole-solve kernel gave the batch up")
+
+    monkeypatch.setattr(to.AutoDiffAdjoint, "_solve_stepwise", no_other_path)
+
+    t_start, t_end, t_eval = spans_that_miss_t_end(12, 6, seed=3)
+    f, y0, _ = rd_problem(12, n=32)
+    problem = to.InitialValueProblem(y0, t_start.cuda(), t_end.cuda(), t_eval.cuda())
+    for method, own in ((to.Tsit5, OwnTsit5), (to.Dopri5, OwnDopri5)):
+        fused = to.AutoDiffAdjoint(method(), to.IntegralController(1e-6, 1e-4)).solve(problem, to.ODETerm(f))
+        assert _lib.last_solve_kernel_name() == "tode::solve_grid_kernel"
+        assert_same(fused, to.AutoDiffAdjoint(own(), to.IntegralController(1e-6, 1e-4)).solve(problem, to.ODETerm(f)))
+
+    w = to.workloads.make("mlp", batch=250, device="cuda")
+    t_start, t_end, t_eval = spans_that_miss_t_end(250, 20, seed=4)
+    problem = to.InitialValueProblem(w.y0, t_start.cuda(), t_end.cuda(), t_eval.cuda())
+    fused = to.AutoDiffAdjoint(to.Dopri5(), make_controller(w.controller)).solve(problem, to.ODETerm(w.f))
+    assert _lib.last_solve_kernel_name() == "tode::solve_mlp_kernel"
+    proto = to.AutoDiffAdjoint(OwnDopri5(), make_controller(w.controller)).solve(problem, to.ODETerm(w.f))
+    assert (fused.stats["n_initialized"] == 20).all()
+    # (the two pipelines' step sizes differ in their last bits, so on these spans they also differ in which samples
+    # land on t_end, one unit short of it -- one more step of that length -- or past it: a tenth of the samples)
+    assert_close_solutions(fused, proto, min_agree=0.85)
+    assert ((fused.stats["n_steps"] - proto.stats["n_steps"]).abs() <= 1).all()
+
+
 @pytest.mark.parametrize("name,batch", [("reaction_diffusion", 16), ("mlp", 128)])
 def test_against_the_committed_vectors(name, batch):
     """tests/golden/*_tolerance.json: ATen-op oracle results written in the authoring container."""

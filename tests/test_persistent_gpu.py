@@ -682,6 +682,36 @@ def test_random_configurations_match_oracle_bit_for_bit(seed):
         assert_identical(gpu_solve(f, y0, t_eval, method, controller, fast=fast, **kw), ref)
 
 
+@pytest.mark.parametrize("fast", ["one", "two", "sliced"])
+@pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
+@pytest.mark.parametrize("name", ["vdp", "lorenz", "linear_decay", "linear_decay-backwards"])
+def test_samples_that_land_past_t_end_stay_in_the_fast_kernels(name, dtype, fast):
+    """Time spans from t_start in (-2, -1) to a small t_end of the other sign: the last step's length t_end - t is
+    rounded and t + (t_end - t) lands one unit in the last place past t_end for about a quarter of the samples (a span
+    [0, T] never does that).  Such a sample takes part in the reference's later iterations with the step t_end - t,
+    seen only in that step's status: the fast kernels compute it once instead of handing the batch to the general
+    kernel."""
+    from torchode_amd import _lib
+
+    B, E = 256, 8
+    w = to.workloads.make(name.split("-")[0], batch=B, dtype=dtype)
+    g = torch.Generator().manual_seed(11)
+    sign = -1.0 if name.endswith("backwards") else 1.0
+    t_start = (-sign * (1.0 + torch.rand(B, generator=g, dtype=torch.float64))).to(dtype)
+    t_end = (sign * (0.01 + 0.3 * torch.rand(B, generator=g, dtype=torch.float64))).to(dtype)
+    t_eval = t_start[:, None] + (t_end - t_start)[:, None] * torch.linspace(0, 1, E, dtype=dtype)[None, :]
+    t_eval[:, 0], t_eval[:, -1] = t_start, t_end
+    for method, ctrl in ((w.method, w.controller), ("dopri5", dict(kind="pid", atol=1e-7, rtol=1e-5, pcoeff=0.3, icoeff=0.4, dcoeff=0.1))):
+        kw = dict(t_start=t_start, t_end=t_end)
+        ref = c_oracle_solve(w.f, w.y0, t_eval, method, ctrl, **kw)
+        assert_identical(gpu_solve(w.f, w.y0, t_eval, method, ctrl, fast=fast, **kw), ref)
+        kernel = "tode::solve_pair_kernel" if fast == "two" else "tode::solve_fast_kernel"
+        if fast == "two" and name.startswith("linear_decay") and dtype == F64:
+            kernel = "tode::solve_kernel"  # (four float64 values per sample: the hand-over record does not fit that kernel's share of LDS)
+        assert _lib.last_solve_kernel_name().startswith(kernel)
+        assert (ref["n_initialized"] == E).all() and (ref["status"] == 0).all()
+
+
 @pytest.mark.parametrize("seed", range(100, 130))
 def test_wild_configurations_match_oracle_bit_for_bit(seed):
     """tests/helpers.py::wild_case: evaluation points shuffled within rows or absent, dt_min / dt_max, a small

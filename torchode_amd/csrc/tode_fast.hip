@@ -173,7 +173,12 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
     };
 
-    while (__any(active)) {
+    // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's later
+    // iterations with the clamped step t_end - t: with evaluation points that is seen only in the status of that step,
+    // which is a success unless its error ratio is not finite.  The sample sits through one more iteration here, as
+    // an inactive lane whose error ratio is looked at.
+    bool idle = false;
+    while (__any(active || idle)) {
         if (RECORD) keep(iteration++, active);
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
@@ -203,6 +208,8 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         const bool accept = ratio < (T)1;
         // a NaN or infinite ratio is a non-success status: leave it to the general kernel (the ratio is at least 1e-38)
         bool sane = !unordered && ratio < (T)__builtin_huge_val();
+        bail = bail || (idle && !sane);
+        idle = false;
         T factor = step_factor(cp.safety, sane ? ratio : (T)1, e1, e2, e3, active);
         sane = sane && factor == factor;  // (a product of an underflowed and an overflowed power)
         factor = clamp_ordered(factor, cp.fmin, cp.fmax);
@@ -266,12 +273,13 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
             const bool failed = active && (!sane || n_steps >= step_limit);
             const bool finished = active && !failed && !running_new;
             if (__any(finished)) {
-                // a sample that lands past t_end, or whose state or derivative at the end is not finite,
-                // shows up in later iterations of the reference loop
-                bool odd = !(t == te);
+                // a sample whose state or derivative at the end is not finite shows up in later iterations of the
+                // reference loop with another status; one that landed past t_end is looked at in the next iteration
+                bool odd = false;
 #pragma unroll
                 for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
                 bail = bail || (finished && odd);
+                idle = finished && !odd && !(t == te);
             }
             bail = bail || failed;
             active = active && !failed && running_new;

@@ -156,6 +156,10 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
     }
     T prev = 1, pprev = 1;
 
+    // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's later
+    // iterations with the clamped step t_end - t, which is seen only in the status of that step: the workgroup
+    // computes that step once more and looks at its status.
+    bool idle = false;
     while (!bail) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
@@ -193,6 +197,10 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
         const bool accept = ratio < (T)1;
         T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
         const int status = limit_dt<T>(cp, ratio, dt_next);
+        if (idle) {
+            bail = status != 0;
+            break;
+        }
 
         const T t_new = accept ? (t0 + dt) : t0;
         const bool running_new = fma_(dir, t_new, -dir * te) < (T)0;
@@ -244,13 +252,14 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             break;
         }
         if (!running_new) {
-            // a sample that does not land on t_end, or ends on a non-finite value, shows up in later
-            // iterations of the reference loop: not the common case
-            int odd = !(t == te);
+            // a sample that ends on a non-finite value shows up in later iterations of the reference loop: not the
+            // common case; one that landed past t_end is looked at in one more iteration
+            int odd = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) odd |= !finite_(y[j]) || !finite_(k[0][j]);
             if (__syncthreads_or(odd)) bail = true;
-            break;
+            if (bail || t == te) break;
+            idle = true;
         }
     }
 

@@ -414,6 +414,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // bit 1: some sample needs the general kernel; bit 0: some sample still runs
     int state = block_or(sh, vslot, (bail ? 2 : 0) | (active ? 1 : 0));
     bail = (state & 2) != 0;
+    // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's later
+    // iterations with the clamped step t_end - t, which is seen only in the status of that step: the sample sits
+    // through one more iteration here, inactive, and the status of its step is looked at.
+    bool idle = false;
     while (state == 1) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
@@ -452,6 +456,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         const bool accept = ratio < (T)1;
         T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
         const int status = limit_dt<T>(cp, ratio, dt_next);
+        bail = bail || (idle && status != 0);
+        idle = false;
         const bool move = accept && active;
         const T t_new = move ? (t0 + dt) : t0;
         const bool running_new = fma_(dir, t_new, -dir * te) < (T)0;
@@ -502,12 +508,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         }
         const bool failed = active && (status != 0 || n_steps >= p.max_steps || n_steps >= TODE_HARD_STEP_LIMIT);
         const bool finished = active && !failed && !running_new;
-        // a sample that does not land on t_end, or ends on a non-finite value, shows up in later
-        // iterations of the reference loop: not the common case
-        const bool odd = !(t == te) || nonfinite;
-        bail = bail || failed || (finished && odd);
+        // a sample that ends on a non-finite value shows up in later iterations of the reference loop: not the
+        // common case; one that landed past t_end is looked at in the next iteration
+        bail = bail || failed || (finished && nonfinite);
+        idle = finished && !nonfinite && !(t == te);
         active = active && !failed && running_new;
-        state = block_or(sh, vslot, (bail ? 2 : 0) | (active ? 1 : 0));
+        state = block_or(sh, vslot, (bail ? 2 : 0) | ((active || idle) ? 1 : 0));
         bail = (state & 2) != 0;
     }
 

@@ -89,8 +89,13 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
         const int step_limit = p.max_steps < TODE_HARD_STEP_LIMIT ? p.max_steps : TODE_HARD_STEP_LIMIT;
         const T e1 = (T)cp.e1, e2 = (T)cp.e2, e3 = (T)cp.e3;
 
+        // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's
+        // later iterations with the clamped step t_end - t: with evaluation points that is seen only in the status of
+        // that step, a success unless its error ratio is not finite.  The sample sits through one more iteration here,
+        // as an inactive lane whose error ratio is looked at.
+        bool idle = false;
         for (int phase = 0;; ++phase) {
-            const bool any = __any(active);
+            const bool any = __any(active || idle);
             if (any) {
                 // ---- stages (runge_kutta.py:255-263) ----
                 const T t0 = t;
@@ -134,6 +139,8 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                 const T ratio = error_ratio_common<T, F>(cp, y, y1, err, unordered);
                 const bool accept = ratio < (T)1;
                 bool sane = !unordered && ratio < (T)__builtin_huge_val();  // (the ratio is at least 1e-38)
+                bail = bail || (idle && !sane);
+                idle = false;
                 T factor = step_factor(cp.safety, sane ? ratio : (T)1, e1, e2, e3, active);
                 sane = sane && factor == factor;  // (a product of an underflowed and an overflowed power)
                 factor = clamp_ordered(factor, cp.fmin, cp.fmax);
@@ -165,12 +172,15 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                     const bool failed = active && (!sane || n_steps >= step_limit);
                     const bool finished = active && !failed && !running_new;
                     if (__any(finished)) {
-                        // a sample that lands past t_end, or whose state or derivative at the end is not finite,
-                        // shows up in later iterations of the reference loop
-                        bool odd = !(t == te);
+                        // a sample whose state or derivative at the end is not finite shows up in later iterations of
+                        // the reference loop with another status, and so does, without evaluation points, one that
+                        // landed past t_end (in the interpolant of the batch's last step); with evaluation points
+                        // such a sample is looked at in the next iteration
+                        bool odd = end_only && !(t == te);
 #pragma unroll
                         for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
                         bail = bail || (finished && odd);
+                        idle = finished && !odd && !(t == te);
                     }
                     bail = bail || failed;
                     active = active && !failed && running_new;
