@@ -712,6 +712,36 @@ def test_samples_that_land_past_t_end_stay_in_the_fast_kernels(name, dtype, fast
         assert (ref["n_initialized"] == E).all() and (ref["status"] == 0).all()
 
 
+@pytest.mark.parametrize("fast", [True, "one", "two", False], ids=["auto", "fast1", "fast2", "general"])
+@pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
+@pytest.mark.parametrize("method", ["dopri5", "tsit5"])
+def test_finished_samples_near_the_top_of_the_range(method, dtype, fast):
+    """Growth backwards in time to a final state near the top of the dtype's range: finite, with a finite derivative
+    k * y.  The reference steps a finished sample again in every later iteration of the batch, with dt = 0; the stage
+    sums a_i1 k0 + a_i2 k0 + ... of such a step overflow once k0 is within a factor of about 14 of the largest finite
+    value (0 * inf = NaN, status 4: infinite norm, which also stops the batch).  The first half of this batch ends on
+    either side of that line (in two of the four method / dtype pairs nine samples fail in such a step, having finished;
+    the largest fail in their own last step), the second half well below it.  A kernel that takes a finished sample's
+    later steps for granted must draw the same line."""
+    B = 96
+    top = 85.2 if dtype == F32 else 706.0  # e-foldings to about 1e37 / 1e306
+    folds = torch.full((B,), top, dtype=torch.float64)
+    folds[:48] += torch.linspace(-3.2, -0.6, 48, dtype=torch.float64)
+    folds[48:] -= torch.linspace(4.0, 9.0, 48, dtype=torch.float64)
+    f = to.LinearDecay(torch.full((B, 1), 20.0, dtype=dtype))
+    y0, t_start, t_end = torch.ones(B, 1, dtype=dtype), torch.zeros(B, dtype=dtype), (-folds / 20.0).to(dtype)
+    t_eval = t_end[:, None] * torch.linspace(0, 1, 6, dtype=dtype)[None, :]
+    t_eval[:, -1] = t_end
+    ctrl = dict(kind="integral", atol=1e-6, rtol=1e-4)
+    kw = dict(t_start=t_start, t_end=t_end, dt0=torch.full((B,), -0.01, dtype=dtype))
+    ref = c_oracle_solve(f, y0, t_eval, method, ctrl, **kw)
+    last = (int(ref["n_f_evals"][0]) - 1) // 6  # iterations of the batch
+    failed_after_finishing = (ref["status"] == 4) & (ref["n_steps"] < last)
+    assert int(failed_after_finishing.sum()) == (9 if (method, dtype) in (("tsit5", F32), ("dopri5", F64)) else 0)
+    assert ref["status"][48:].tolist() == [0] * 48 and (ref["status"][:48] == 4).any()
+    assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, fast=fast, **kw), ref)
+
+
 @pytest.mark.parametrize("seed", range(100, 130))
 def test_wild_configurations_match_oracle_bit_for_bit(seed):
     """tests/helpers.py::wild_case: evaluation points shuffled within rows or absent, dt_min / dt_max, a small

@@ -277,7 +277,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
                 // reference loop with another status; one that landed past t_end is looked at in the next iteration
                 bool odd = false;
 #pragma unroll
-                for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
+                for (int f = 0; f < F; ++f) odd = odd || !settles_(y[f], k[0][f]);
                 bail = bail || (finished && odd);
                 idle = finished && !odd && !(t == te);
             }

@@ -256,7 +256,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             // common case; one that landed past t_end is looked at in one more iteration
             int odd = 0;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) odd |= !finite_(y[j]) || !finite_(k[0][j]);
+            for (int j = 0; j < 4; ++j) odd |= !settles_(y[j], k[0][j]);
             if (__syncthreads_or(odd)) bail = true;
             if (bail || t == te) break;
             idle = true;

@@ -28,6 +28,15 @@ template <> __device__ __forceinline__ double abs_<double>(double a) { return __
 
 template <typename T> __device__ __forceinline__ bool finite_(T a) { return abs_(a) < __builtin_huge_val(); }
 
+// A sample that has finished on t_end keeps stepping in the reference's later iterations with dt = 0, which is seen in
+// the status of those steps alone: a success as long as their error ratio is finite.  With dt = 0 every stage is
+// evaluated at y itself, so every stage derivative is k0 again, the stage sums are a_i1 k0 + a_i2 k0 + ..., and the
+// step's result and error estimate are y and 0 -- provided no such sum overflows (0 * inf is NaN).  The tableaus'
+// |a_ij| sum to less than 32 per row: a value and derivative that pass this test cannot produce anything but status 0.
+template <typename T> __device__ __forceinline__ bool settles_(T y, T k0) {
+    return finite_(y) && abs_(k0) <= (T)(sizeof(T) == 4 ? 0x1p+122 : 0x1p+1018);  // (the largest finite value / 64; false for NaN)
+}
+
 // torch.maximum / torch.minimum / torch.clamp: NaN in any operand gives NaN.  Written as
 // max/min plus one unordered-compare select so that it stays straight-line code.
 template <typename T> __device__ __forceinline__ T nan_();

@@ -497,7 +497,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int r = 0; r < 4; ++r) {
             y[r] = move ? y1[r] : y[r];
             k[0][r] = move ? k[6][r] : k[0][r];
-            nonfinite = nonfinite || !finite_(y[r]) || !finite_(k[0][r]);
+            nonfinite = nonfinite || !settles_(y[r], k[0][r]);
         }
         t = t_new;
         const T dtc = tclamp(running_new ? dt_next : dt, tlo - t_new, thi - t_new);

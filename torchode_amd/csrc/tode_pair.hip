@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                         // such a sample is looked at in the next iteration
                         bool odd = end_only && !(t == te);
 #pragma unroll
-                        for (int f = 0; f < F; ++f) odd = odd || !finite_(k[0][f]) || !finite_(y[f]);
+                        for (int f = 0; f < F; ++f) odd = odd || !settles_(y[f], k[0][f]);
                         bail = bail || (finished && odd);
                         idle = finished && !odd && !(t == te);
                     }

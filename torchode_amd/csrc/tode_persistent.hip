@@ -227,7 +227,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
                 // (status 0, value y) unless one of the following holds.
                 bool nontrivial = cp.has_dt_min || !(t == te);
 #pragma unroll
-                for (int f = 0; f < F; ++f) nontrivial = nontrivial || !finite_(k[0][f]) || !finite_(y[f]);
+                for (int f = 0; f < F; ++f) nontrivial = nontrivial || !settles_(y[f], k[0][f]);
                 if (nontrivial) {
                     idle_pass = true;
                     continue;
