@@ -746,3 +746,41 @@ def test_whole_sweep_kernel_agrees_with_the_per_iteration_kernels_and_the_torch_
                 else:
                     torch.testing.assert_close(g / scale, ref / scale, rtol=rtol, atol=atol)
     assert all(g is not None and bool(g.isfinite().all()) for g in results["whole"][:2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("features", [3, 4, 8])
+@pytest.mark.parametrize("method,kind", [(to.Dopri5, "integral"), (to.Dopri5, "pid"), (to.Tsit5, "integral"), (to.Tsit5, "pid")])
+def test_whole_sweep_kernel_when_every_sample_has_used_up_its_points(method, kind, features):
+    """Float64 rows of 3, 4 and 8 values (the kernels under the highest register pressure), evaluation points none of
+    which lies at t_start, few of them: most samples have no point left for most of the reverse sweep.  Four of these
+    instantiations once lost part of the parameter gradient there (a miscompiled divergent region: see
+    torchode_amd/build.py::copies_ahead_of_the_exec_restore).  Against the per-iteration reverse kernels."""
+    import torchode_amd.autodiff as autodiff
+
+    B, dtype = 70, torch.float64
+    g = torch.Generator().manual_seed(5)
+    k = (0.3 + 2.5 * torch.rand(B, features, generator=g, dtype=dtype)).cuda()
+    y0 = (torch.rand(B, features, generator=g, dtype=dtype) * 2 - 1).cuda()
+    t_start = (torch.rand(B, generator=g, dtype=dtype) - 0.5).cuda()
+    t_end = t_start + (1.5 * (0.5 + 0.5 * torch.rand(B, generator=g, dtype=dtype))).cuda()
+    for E in (1, 3):
+        t_eval = t_start[:, None] + (t_end - t_start)[:, None] * torch.linspace(1.0 / E, 1, E, dtype=dtype, device="cuda")[None, :]
+        t_eval[:, -1] = t_end
+        weights = torch.linspace(0.5, 1.5, E * features, dtype=dtype, device="cuda").reshape(1, E, -1)
+        results = {}
+        for sweep in ("whole", "kernels"):
+            leaf, y = k.clone().requires_grad_(), y0.clone().requires_grad_()
+            ctrl = to.IntegralController(1e-6, 1e-4) if kind == "integral" else to.PIDController(1e-6, 1e-4, 0.2, 0.5, 0.05)
+            solver = to.AutoDiffAdjoint(method(), ctrl, backprop_through_step_size_control=False)
+            solver.backward_whole_kernel = sweep == "whole"
+            sol = solver.solve(to.InitialValueProblem(y, t_start, t_end, t_eval), to.ODETerm(to.LinearDecay(leaf)))
+            results[sweep] = torch.autograd.grad((sol.ys * weights).sum(), [y, leaf])
+            assert autodiff.LAST_SWEEP == sweep
+        for got, want in zip(results["whole"], results["kernels"]):
+            torch.testing.assert_close(got, want, rtol=1e-9, atol=1e-9 * float(want.abs().max()))
+        # (and the closed form, y0 exp(-k (t - t_start)), to the solver's own accuracy)
+        span = (t_eval - t_start[:, None])[:, :, None]
+        exact = (weights * -span * y0[:, None, :] * torch.exp(-k[:, None, :] * span)).sum(1)
+        assert float(((results["whole"][1] - exact).abs() / exact.abs().amax(dim=1, keepdim=True)).max()) < 5e-3
+

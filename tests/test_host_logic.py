@@ -365,3 +365,20 @@ def test_typing_names_and_predicates():
     for name in ("DataTensor", "NormTensor", "SolutionDataTensor", "TimeTensor", "EvaluationTimesTensor", "AcceptTensor", "StatusTensor",
                  "InterpTimeTensor", "InterpDataTensor", "SampleIndexTensor"):  # fmt: skip
         assert getattr(ty, name) is torch.Tensor
+
+
+def test_no_register_copy_ahead_of_the_exec_mask_restore(tmp_path):
+    """The device assembly of every translation unit, searched for the one miscompilation met so far: copies of vector
+    registers to accumulation registers placed at the end of a divergent region ahead of the instruction that restores
+    the execution mask, which lanes that skipped the region then miss (torchode_amd/build.py).  Four instantiations of
+    the one-kernel reverse sweep had it -- gradients of the parameters wrong by tens of per cent for samples without an
+    evaluation point left, no error -- until the region was written as a loop the wavefront runs together."""
+    import shutil
+
+    from torchode_amd import build
+
+    if shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"):
+        pytest.skip("no hipcc here")
+    for path in build.emit_assembly(str(tmp_path)):
+        assert build.copies_ahead_of_the_exec_restore(path) == [], path
+

@@ -147,5 +147,52 @@ def link_ops_library(obj=None) -> str:
     return OPS_LIB
 
 
+def emit_assembly(directory: str, units=None) -> list:
+    """The device code of every translation unit (or of ``units``, object names) as assembly text under ``directory``,
+    compiled with the flags of the build.  Returns the paths."""
+    os.makedirs(directory, exist_ok=True)
+    hipcc = _hipcc()
+    chosen = [u for u in UNITS if units is None or u[1] in units]
+
+    def emit(unit):
+        src, obj, defs = unit
+        path = os.path.join(directory, obj[:-2] + ".s")
+        _run([hipcc, *FLAGS, *defs, "-S", "--offload-device-only", os.path.join(CSRC, src), "-o", path])
+        return path
+
+    with ThreadPoolExecutor(max_workers=min(8, len(chosen) + 1)) as pool:
+        return list(pool.map(emit, chosen))
+
+
+def copies_ahead_of_the_exec_restore(assembly_path: str) -> list:
+    """Looks through a unit's device assembly for a block that starts with copies of vector registers into
+    accumulation registers (or spill stores) and only then restores the execution mask (``s_or_b64 exec, exec, ...``
+    at the end of a divergent region).  Such copies run for the lanes that went through the region only, and a lane
+    that skipped it continues with whatever the copy's target held before: wrong values without any error.  This
+    compiler has placed copies like that in kernels under high register pressure.  Returns (kernel, line, count)."""
+    import re
+
+    lines = open(assembly_path).read().split("\n")
+    found, kernel = [], None
+    for n, line in enumerate(lines):
+        name = re.match(r"^(_Z\w+):", line)
+        if name:
+            kernel = name.group(1)
+        if not re.match(r"^\.LBB\d+_\d+:", line):
+            continue
+        copies = 0
+        for text in lines[n + 1 : n + 64]:
+            text = text.strip()
+            if text.startswith((".LBB", "s_branch", "s_endpgm")) or "s_cbranch" in text:
+                break
+            if text.startswith("s_or_b64 exec, exec"):
+                if copies:
+                    found.append((kernel, n + 1, copies))
+                break
+            if text.startswith(("v_accvgpr_write", "scratch_store", "buffer_store")):
+                copies += 1
+    return found
+
+
 if __name__ == "__main__":
     print(build_library(force=True, verbose=True))

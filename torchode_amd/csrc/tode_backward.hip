@@ -231,8 +231,18 @@ __global__ void __launch_bounds__(64) whole_backward_kernel(const WholeBackward<
         }
 
         // ---- everything after the stages, reversed ----
+        // (The points of this iteration are counted in a loop that the whole wavefront runs together, with a clamped
+        // index in place of a guarded load: no lane leaves and rejoins here.  Written as each lane's own loop, this was a
+        // divergent region at whose end the compiler, for four instantiations on long float64 rows, copied registers of
+        // the parameter cotangents to accumulation registers ahead of the instruction that restores the execution mask;
+        // lanes that had no point left skipped the copy and went on with the values of an earlier iteration.)
         int n_here = 0;
-        while (cursor - n_here >= 0 && iterations_sorted[cursor - n_here] == (int)i) ++n_here;
+        while (E > 0) {
+            const int at = cursor - n_here;
+            const bool more = at >= 0 && iterations_sorted[at < 0 ? 0 : at] == (int)i;
+            if (!__any(more)) break;
+            n_here += more ? 1 : 0;
+        }
         cursor -= n_here;
         finish_backward_sample<T, T, METHOD, CTRL, false, F>(q, 0, 0, 1, points_by_iteration + cursor + 1, n_here);
 
