@@ -896,3 +896,44 @@ def test_one_wavefront_kernel_storing_its_points_four_at_a_time(case):
             assert _lib.last_solve_kernel_name() == "tode::solve_fast_kernel" + (" (points stored four at a time)" if four_at_a_time else "")
     finally:
         _lib.set_kernel_timing(False)
+
+
+def test_outputs_of_more_than_two_to_the_31_values():
+    """Lorenz, 8 388 685 samples with 100 evaluation points: 2.5e9 output values, past what a 32-bit index reaches.
+    Batch composition does not matter to any sample, so slices of the large solve -- the first and last thousand
+    samples, and the ones either side of value number 2^31 -- must equal small solves of the same samples bit for bit:
+    the one-wavefront kernel, the general kernel and the per-step kernels (stopped after three steps)."""
+    from torchode_amd import _lib
+
+    if torch.cuda.mem_get_info()[0] < 80e9:
+        pytest.skip("needs 80 GB of free device memory")
+    w = to.workloads.make("lorenz", batch=4096, device="cuda")
+    B, E = 8 * 1024 * 1024 + 77, 100
+    rep = (B + 4095) // 4096
+    y0 = w.y0.repeat(rep, 1)[:B].contiguous()
+    y0 += torch.linspace(0, 1e-3, B, device="cuda")[:, None]  # every sample its own
+    rho = w.f.builtin_params()[:, 0].repeat(rep)[:B].contiguous()
+    t_eval = (w.t_eval[:, -1].repeat(rep)[:B, None] * torch.linspace(0, 1, E, device="cuda")[None, :]).contiguous()
+    assert B * E * 3 > 2**31
+    slices = ((0, 1000), (2**31 // 300 - 250, 2**31 // 300 + 250), (B - 1000, B))
+    method = {"tsit5": to.Tsit5, "dopri5": to.Dopri5}[w.method]
+    hidden = lambda f: (lambda t, y: f(t, y))
+    for path, max_steps in (("one kernel", None), ("general", None), ("per-step", 3)):
+        def solve(lo, hi):
+            f = to.Lorenz63(rho[lo:hi].clone())
+            solver = to.AutoDiffAdjoint(method(), make_controller(w.controller), max_steps=max_steps)
+            solver.use_fast_path = path != "general"
+            problem = to.InitialValueProblem(y0[lo:hi].clone(), t_eval=t_eval[lo:hi].clone())
+            return solver.solve(problem, to.ODETerm(hidden(f) if path == "per-step" else f))
+
+        whole = solve(0, B)
+        if path != "per-step":
+            assert _lib.last_solve_kernel_name() == ("tode::solve_fast_kernel" if path == "one kernel" else "tode::solve_kernel")
+        for lo, hi in slices:
+            part = solve(lo, hi)
+            for key in ("n_steps", "n_accepted", "n_initialized"):
+                assert torch.equal(part.stats[key], whole.stats[key][lo:hi]), (path, lo, key)
+            written = torch.arange(E, device="cuda")[None, :] < part.stats["n_initialized"][:, None]
+            assert torch.equal(part.ys[written], whole.ys[lo:hi][written]) and torch.equal(part.status, whole.status[lo:hi]), (path, lo)
+        del whole
+
