@@ -165,14 +165,14 @@ class OwnDopri5(to.Dopri5):
     pass
 
 
-def rd_problem(batch, n=64, E=12, t1=1.0, seed=7, backwards=False, d_max=0.1):
+def rd_problem(batch, n=64, E=12, t1=1.0, seed=7, backwards=False, d_max=0.1, dtype=torch.float32):
     g = torch.Generator().manual_seed(seed)
-    D = torch.rand(batch, generator=g) * d_max + 0.001
-    y0 = torch.rand((batch, n * n), generator=g)
-    lo, hi = torch.zeros(batch), torch.full((batch,), t1) * (0.5 + torch.rand(batch, generator=g))
+    D = (torch.rand(batch, generator=g) * d_max + 0.001).to(dtype)
+    y0 = torch.rand((batch, n * n), generator=g).to(dtype)
+    lo, hi = torch.zeros(batch, dtype=dtype), (torch.full((batch,), t1) * (0.5 + torch.rand(batch, generator=g))).to(dtype)
     if backwards:
         lo, hi = hi, lo
-    t_eval = lo[:, None] + (hi - lo)[:, None] * torch.linspace(0, 1, E)[None, :]
+    t_eval = lo[:, None] + (hi - lo)[:, None] * torch.linspace(0, 1, E, dtype=dtype)[None, :]
     return to.ReactionDiffusion(D.cuda(), n), y0.cuda(), t_eval.cuda()
 
 
@@ -227,6 +227,30 @@ def test_grid_kernel_on_a_16_by_16_grid(method, kind):
     assert (fused.stats["n_steps"] > 8).all() and (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()
     f, y0, t_eval = rd_problem(9, n=16, backwards=True)
     assert_same(*both_paths(f, y0, t_eval, method, ctrl))
+
+
+@pytest.mark.parametrize("n", [16, 32, 64])
+@pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "integral"), ("tsit5", "integral"), ("dopri5", "pid")])
+def test_grid_kernel_in_float64_equals_the_protocol_path(method, kind, n):
+    """The same kernel compiled for float64 (twice the registers: the 64 x 64 grid, whose workgroup of 1024 threads has
+    128 registers per thread, keeps a few values in scratch memory): same bits as the per-call operators, forwards,
+    backwards, with a first step given, and spans whose last step lands past t_end."""
+    ctrl = dict(kind=kind, atol=1e-9, rtol=1e-7)
+    if kind == "pid":
+        ctrl.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    f, y0, t_eval = rd_problem(10, n=n, t1=8.0, d_max=1.0, dtype=torch.float64)
+    fused, proto = both_paths(f, y0, t_eval, method, ctrl)
+    assert fused.ys.dtype == torch.float64
+    assert_same(fused, proto)
+    assert (fused.stats["n_steps"] > 8).all()
+    f, y0, t_eval = rd_problem(5, n=n, backwards=True, dtype=torch.float64)
+    assert_same(*both_paths(f, y0, t_eval, method, ctrl, dt0=torch.full((5,), -0.01, dtype=torch.float64, device="cuda")))
+    t_start, t_end, t_eval = spans_that_miss_t_end(6, 5, seed=n)
+    f, y0, _ = rd_problem(6, n=n, dtype=torch.float64)
+    problem = to.InitialValueProblem(y0, t_start.double().cuda(), t_end.double().cuda(), t_eval.double().cuda())
+    lib_m, own_m = {"tsit5": (to.Tsit5, OwnTsit5), "dopri5": (to.Dopri5, OwnDopri5)}[method]
+    assert_same(to.AutoDiffAdjoint(lib_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)),
+                to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)))  # fmt: skip
 
 
 def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():

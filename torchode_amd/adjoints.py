@@ -181,11 +181,11 @@ class AutoDiffAdjoint(nn.Module):
         if f.builtin_kind in _lib.GENERAL_TERMS:
             return True
         c, E, F = self.step_size_controller, problem.n_evaluation_points, problem.n_features
-        if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != torch.float32:
+        if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != problem.time_dtype:
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
             return F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192
-        return 4 <= F <= 64 and F % 4 == 0 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
+        return problem.data_dtype == torch.float32 and 4 <= F <= 64 and F % 4 == 0 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable
     def _solve_eager_outside_the_trace(self, problem, term, dt0, args) -> Solution:

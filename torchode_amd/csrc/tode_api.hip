@@ -286,8 +286,7 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (a->record && (a->term == TODE_TERM_REACTION_DIFFUSION || a->term == TODE_TERM_MLP))
         return fail(TODE_E_UNSUPPORTED, "a record of the loop state is written for the small systems only");
     if (a->term == TODE_TERM_REACTION_DIFFUSION) {
-        if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for float32");
-        return solve_grid_f32(*a, *c, ns, na, ni, st, s);
+        return a->dtype == TODE_F32 ? solve_grid_f32(*a, *c, ns, na, ni, st, s) : solve_grid_f64(*a, *c, ns, na, ni, st, s);
     }
     if (a->term == TODE_TERM_MLP) {
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the MLP kernel is built for float32");
@@ -510,11 +509,11 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
         // (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
         one_kernel = one_kernel && allow_one_kernel && ((E > 0 && E * elem <= 1024) || (B > 0 && B <= TODE_END_ONLY_MAX_BATCH));
     } else {
-        one_kernel = one_kernel && E > 0 && a->dtype == TODE_F32;
+        one_kernel = one_kernel && E > 0;
         if (a->term == TODE_TERM_REACTION_DIFFUSION)
             one_kernel = one_kernel && (a->n_features == 16 * 16 || a->n_features == 32 * 32 || a->n_features == 64 * 64) && E <= 8192;
         else if (a->term == TODE_TERM_MLP)
-            one_kernel = one_kernel && a->n_features >= 4 && a->n_features <= 64 && a->n_features % 4 == 0 && E <= 512;
+            one_kernel = one_kernel && a->dtype == TODE_F32 && a->n_features >= 4 && a->n_features <= 64 && a->n_features % 4 == 0 && E <= 512;
         else
             return fail(TODE_E_INVALID, "unknown term %d", a->term);
         if (!one_kernel) return fail(TODE_E_UNSUPPORTED, "no whole-solve kernel for this term in this shape, dtype or controller setting");

@@ -1,5 +1,5 @@
 // Whole-solve kernel for right-hand sides on a periodic N x N grid (reaction-diffusion,
-// F = N*N state values per sample, N = 16, 32 or 64): one workgroup of N*N/4 threads per sample.
+// F = N*N state values per sample, N = 16, 32 or 64, float32 or float64): one workgroup of N*N/4 threads per sample.
 //
 // Thread t owns the four consecutive cells 4t..4t+3 of the row-major grid and keeps
 // their state (y, the seven stage derivatives, the dense-output coefficients) in
@@ -29,13 +29,23 @@ struct GridOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
 };
 
-template <int NW> struct GridShared {
-    float xch[2][NW * 256];  // stage input, double buffered
-    float red[2][NW][2];     // wavefront sums of up to two reductions, double buffered
+template <typename T, int NW> struct GridShared {
+    T xch[2][NW * 256];  // stage input, double buffered
+    T red[2][NW][2];     // wavefront sums of up to two reductions, double buffered
 };
 
+// Four consecutive values, moved with the widest loads and stores their alignment allows.
+template <typename T> struct alignas(4 * sizeof(T)) Four {
+    T x, y, z, w;
+};
+template <typename T> __device__ __forceinline__ void load4(const T *from, T (&v)[4]) {
+    const Four<T> f = *reinterpret_cast<const Four<T> *>(from);
+    v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+}
+template <typename T> __device__ __forceinline__ void store4(T *to, const T (&v)[4]) { *reinterpret_cast<Four<T> *>(to) = Four<T>{v[0], v[1], v[2], v[3]}; }
+
 // Sum over the workgroup of two per-thread partial sums, in the fixed order.
-template <int NW> __device__ __forceinline__ void block_sum2(GridShared<NW> &sh, int &slot, float a, float b, float &A, float &B) {
+template <typename T, int NW> __device__ __forceinline__ void block_sum2(GridShared<T, NW> &sh, int &slot, T a, T b, T &A, T &B) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         a = a + __shfl_xor(a, off);
@@ -59,37 +69,36 @@ template <int NW> __device__ __forceinline__ void block_sum2(GridShared<NW> &sh,
 
 // du/dt = D * lap(u) + u * (1 - u) on the periodic grid; each operation rounds on its own, in the
 // order of the torch expression  (((up + down) + left) + right) - 4u,  D * lap + u * (1 - u).
-template <int N, int NW>
-__device__ __forceinline__ void grid_rhs(GridShared<NW> &sh, int &buf, float D, const float (&u)[4], float (&out)[4]) {
+template <typename T, int N, int NW>
+__device__ __forceinline__ void grid_rhs(GridShared<T, NW> &sh, int &buf, T D, const T (&u)[4], T (&out)[4]) {
     const int t = threadIdx.x;
     constexpr int PER_ROW = N / 4;
     const int r = t / PER_ROW, c0 = 4 * (t - r * PER_ROW);
-    float *x = sh.xch[buf];
-    *reinterpret_cast<float4 *>(x + 4 * t) = make_float4(u[0], u[1], u[2], u[3]);
+    T *x = sh.xch[buf];
+    store4<T>(x + 4 * t, u);
     lds_barrier();
     const int ru = (r + N - 1) & (N - 1), rd = (r + 1) & (N - 1);
-    const float4 up = *reinterpret_cast<const float4 *>(x + ru * N + c0);
-    const float4 dn = *reinterpret_cast<const float4 *>(x + rd * N + c0);
-    const float lf = x[r * N + ((c0 + N - 1) & (N - 1))];
-    const float rt = x[r * N + ((c0 + 4) & (N - 1))];
-    const float ups[4] = {up.x, up.y, up.z, up.w}, dns[4] = {dn.x, dn.y, dn.z, dn.w};
-    const float lfs[4] = {lf, u[0], u[1], u[2]}, rts[4] = {u[1], u[2], u[3], rt};
+    T ups[4], dns[4];
+    load4<T>(x + ru * N + c0, ups);
+    load4<T>(x + rd * N + c0, dns);
+    const T lf = x[r * N + ((c0 + N - 1) & (N - 1))];
+    const T rt = x[r * N + ((c0 + 4) & (N - 1))];
+    const T lfs[4] = {lf, u[0], u[1], u[2]}, rts[4] = {u[1], u[2], u[3], rt};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const float lap = (((ups[j] + dns[j]) + lfs[j]) + rts[j]) - (4.0f * u[j]);
-        const float diff = D * lap;
-        const float react = u[j] * (1.0f - u[j]);
+        const T lap = (((ups[j] + dns[j]) + lfs[j]) + rts[j]) - ((T)4 * u[j]);
+        const T diff = D * lap;
+        const T react = u[j] * ((T)1 - u[j]);
         out[j] = diff + react;
     }
     buf ^= 1;
 }
 
-template <int METHOD, int CTRL, int N>
-__global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<float> p, const GridOut o) {
-    using T = float;
+template <typename T, int METHOD, int CTRL, int N>
+__global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<T> p, const GridOut o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = N * N, NT = F / 4, NW = NT / 64;
-    __shared__ GridShared<NW> sh;
+    __shared__ GridShared<T, NW> sh;
     extern __shared__ __align__(16) unsigned char dyn[];
     T *te_s = reinterpret_cast<T *>(dyn);  // [E] evaluation times of this sample
 
@@ -106,10 +115,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
     const T tlo = tmin(ts, te), thi = tmax(te, ts);
     const T D = p.params[b];
     T y[4], k[7][4];
-    {
-        const float4 v = *reinterpret_cast<const float4 *>(p.y0 + b * F + 4 * tid);
-        y[0] = v.x, y[1] = v.y, y[2] = v.z, y[3] = v.w;
-    }
+    load4<T>(p.y0 + b * F + 4 * tid, y);
     __syncthreads();  // te_s
 
     bool bail = false;
@@ -117,7 +123,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
 
     // ---- first step size (step_size_controllers.py:431-490, 776-835) ----
     T t = ts, dt;
-    grid_rhs<N, NW>(sh, buf, D, y, k[0]);
+    grid_rhs<T, N, NW>(sh, buf, D, y, k[0]);
     if (p.dt0) {
         dt = p.dt0[b];
     } else {
@@ -129,14 +135,14 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             a0 = fma_(x0, x0, a0);
             a1 = fma_(x1, x1, a1);
         }
-        block_sum2<NW>(sh, slot, a0, a1, A0, A1);
+        block_sum2<T, NW>(sh, slot, a0, a1, A0, A1);
         const T d0 = sqrt_(A0), d1 = sqrt_(A1);
         T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
         h0 = tmin(h0, abs_(te - ts));
         T y1[4], f1[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) y1[j] = fma_(dir * h0, k[0][j], y[j]);
-        grid_rhs<N, NW>(sh, buf, D, y1, f1);
+        grid_rhs<T, N, NW>(sh, buf, D, y1, f1);
         T a2 = 0, A2, unused;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -144,14 +150,14 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             const T x2 = (df * inv[j]) / sf;
             a2 = fma_(x2, x2, a2);
         }
-        block_sum2<NW>(sh, slot, a2, (T)0, A2, unused);
+        block_sum2<T, NW>(sh, slot, a2, (T)0, A2, unused);
         dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, h0, d1, sqrt_(A2));
     }
     dt = tclamp(dt, tlo - t, thi - t);
 
     int cursor = 0, n_steps = 0, n_acc = 0;
     if (E > 0 && te_s[0] == ts) {
-        *reinterpret_cast<float4 *>(p.ys + (b * E) * F + 4 * tid) = make_float4(y[0], y[1], y[2], y[3]);
+        store4<T>(p.ys + (b * E) * F + 4 * tid, y);
         cursor = 1;
     }
     T prev = 1, pprev = 1;
@@ -174,7 +180,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
                 for (int jj = 0; jj < i; ++jj) s = fma_((T)Tab::a[i][jj], k[jj][j], s);
                 yi[j] = fma_(dt, s, y[j]);
             }
-            grid_rhs<N, NW>(sh, buf, D, yi, k[i]);
+            grid_rhs<T, N, NW>(sh, buf, D, yi, k[i]);
             if (i == 6) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) y1[j] = yi[j];
@@ -192,7 +198,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             const T x = (abs_(err) / fma_(cp.rtol, m, cp.atol)) / sf;
             part = fma_(x, x, part);
         }
-        block_sum2<NW>(sh, slot, part, (T)0, total, unused);
+        block_sum2<T, NW>(sh, slot, part, (T)0, total, unused);
         const T ratio = tmax(sqrt_(total), (T)1e-38);
         const bool accept = ratio < (T)1;
         T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
@@ -228,7 +234,7 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
                     for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
                     out[j] = v;
                 }
-                *reinterpret_cast<float4 *>(p.ys + (b * E + cursor) * F + 4 * tid) = make_float4(out[0], out[1], out[2], out[3]);
+                store4<T>(p.ys + (b * E + cursor) * F + 4 * tid, out);
                 ++cursor;
             } while (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0);
         }
@@ -274,34 +280,42 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
     publish_flags(p);
 }
 
-template <int METHOD, int CTRL, int N> static int launch_grid(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t stream) {
-    SolveParams<float> p = make_params<float>(a, c);
+template <typename T, int METHOD, int CTRL, int N> static int launch_grid(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t stream) {
+    SolveParams<T> p = make_params<T>(a, c);
     reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
-    const size_t lds = (size_t)a.n_eval * sizeof(float);
+    const size_t lds = (size_t)a.n_eval * sizeof(T);
     timing_before(stream, "tode::solve_grid_kernel");
-    hipLaunchKernelGGL((solve_grid_kernel<METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4), lds, stream, p, o);
+    hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4), lds, stream, p, o);
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }
 
-template <int N> static int grid_mc(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t s) {
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<0, 0, N>(a, c, o, s);
-    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch_grid<0, 1, N>(a, c, o, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<1, 0, N>(a, c, o, s);
-    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch_grid<1, 1, N>(a, c, o, s);
+template <typename T, int N> static int grid_mc(const tode_solve_args &a, const tode_controller &c, const GridOut &o, hipStream_t s) {
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<T, 0, 0, N>(a, c, o, s);
+    if (a.method == TODE_DOPRI5 && c.kind == TODE_CTRL_PID) return launch_grid<T, 0, 1, N>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_INTEGRAL) return launch_grid<T, 1, 0, N>(a, c, o, s);
+    if (a.method == TODE_TSIT5 && c.kind == TODE_CTRL_PID) return launch_grid<T, 1, 1, N>(a, c, o, s);
     return fail(TODE_E_INVALID, "unknown method %d or controller kind %d", a.method, c.kind);
 }
 
-int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+template <typename T> static int solve_grid(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
     if (a.n_params != 1) return fail(TODE_E_INVALID, "reaction-diffusion needs one parameter (the diffusivity) per sample");
     if (a.n_eval > 8192) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the grid kernel", a.n_eval);
     if (a.batch > INT_MAX) return fail(TODE_E_UNSUPPORTED, "batch too large");
     GridOut o{ns, na, ni, st};
-    if (a.n_features == 64 * 64) return grid_mc<64>(a, c, o, s);
-    if (a.n_features == 32 * 32) return grid_mc<32>(a, c, o, s);
-    if (a.n_features == 16 * 16) return grid_mc<16>(a, c, o, s);  // (one wavefront per sample)
+    if (a.n_features == 64 * 64) return grid_mc<T, 64>(a, c, o, s);
+    if (a.n_features == 32 * 32) return grid_mc<T, 32>(a, c, o, s);
+    if (a.n_features == 16 * 16) return grid_mc<T, 16>(a, c, o, s);  // (one wavefront per sample)
     return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 16 x 16, 32 x 32 and 64 x 64 grids, got F=%d", a.n_features);
+}
+
+int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+    return solve_grid<float>(a, c, ns, na, ni, st, s);
+}
+
+int solve_grid_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
+    return solve_grid<double>(a, c, ns, na, ni, st, s);
 }
 
 }  // namespace tode
