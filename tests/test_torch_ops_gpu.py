@@ -76,6 +76,7 @@ CASES = [
     ("lorenz", 200, torch.float64, "plain", dict(dt_max=0.01)),  # step size limits: general kernel only
     ("mlp", 64, torch.float32, "plain", {}),
     ("reaction_diffusion", 4, torch.float32, "plain", {}),
+    ("reaction_diffusion", 3, torch.float64, "plain", {}),
 ]
 
 
