@@ -43,8 +43,8 @@ enum {
     TODE_TERM_LINEAR_DECAY = 0,       /* dy/dt = -k y, k [B,F] */
     TODE_TERM_VAN_DER_POL = 1,        /* F = 2, mu [B] */
     TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
-    TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 16, 32 or 64), du/dt = D lap(u) + u (1 - u), D [B];
-                                         float32 or float64 (time and data alike), tode_solve_builtin_fast only */
+    TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 16, 32 or 64; float32 also 128), du/dt = D lap(u) + u (1 - u),
+                                         D [B]; float32 or float64 (time and data alike), tode_solve_builtin_fast only */
     TODE_TERM_MLP = 4                 /* F = 4, 8, ..., 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units,
                                          weights in shared_params as packed by tode_mlp_pack_weights[_for]; float32,
                                          tode_solve_builtin_fast only */

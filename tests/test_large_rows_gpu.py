@@ -253,6 +253,28 @@ def test_grid_kernel_in_float64_equals_the_protocol_path(method, kind, n):
                 to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)))  # fmt: skip
 
 
+@pytest.mark.parametrize("method,kind", [("tsit5", "pid"), ("dopri5", "integral")])
+def test_grid_kernel_on_a_128_by_128_grid(method, kind):
+    """16 384 cells: 1024 threads with four bands of 32 rows each (16 cells per thread, most of them in scratch memory
+    between uses); the row sums still run over the 64 chunks of 256 cells in order, so the bits are the protocol path's."""
+    ctrl = dict(kind=kind, atol=1e-7, rtol=1e-5)
+    if kind == "pid":
+        ctrl.update(pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
+    f, y0, t_eval = rd_problem(7, n=128, t1=8.0, d_max=1.0)
+    fused, proto = both_paths(f, y0, t_eval, method, ctrl)
+    assert fused.ys.shape == (7, 12, 128 * 128)
+    assert_same(fused, proto)
+    assert (fused.stats["n_steps"] > 8).all() and (fused.stats["n_steps"] > fused.stats["n_accepted"]).any()
+    f, y0, t_eval = rd_problem(3, n=128, backwards=True)
+    assert_same(*both_paths(f, y0, t_eval, method, ctrl, dt0=torch.full((3,), -0.01, device="cuda")))
+    t_start, t_end, t_eval = spans_that_miss_t_end(5, 6, seed=128)
+    f, y0, _ = rd_problem(5, n=128)
+    problem = to.InitialValueProblem(y0, t_start.cuda(), t_end.cuda(), t_eval.cuda())
+    lib_m, own_m = {"tsit5": (to.Tsit5, OwnTsit5), "dopri5": (to.Dopri5, OwnDopri5)}[method]
+    assert_same(to.AutoDiffAdjoint(lib_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)),
+                to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)))  # fmt: skip
+
+
 def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():
     from torchode_amd import _lib
 

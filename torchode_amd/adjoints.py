@@ -184,7 +184,7 @@ class AutoDiffAdjoint(nn.Module):
         if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != problem.time_dtype:
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
-            return F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192
+            return (F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192) or (F == 128 * 128 and problem.data_dtype == torch.float32 and E <= 4096)
         return problem.data_dtype == torch.float32 and 4 <= F <= 64 and F % 4 == 0 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable

@@ -1,7 +1,9 @@
 // Whole-solve kernel for right-hand sides on a periodic N x N grid (reaction-diffusion,
-// F = N*N state values per sample, N = 16, 32 or 64, float32 or float64): one workgroup of N*N/4 threads per sample.
+// F = N*N state values per sample; N = 16, 32 or 64 in float32 or float64, 128 in float32): one workgroup per sample,
+// of N*N/4 threads up to N = 64 and of 1024 threads on the 128 x 128 grid.
 //
-// Thread t owns the four consecutive cells 4t..4t+3 of the row-major grid and keeps
+// Thread t owns the four consecutive cells 4t..4t+3 of the row-major grid (on the 128 x 128 grid: of each of its four
+// bands of 32 rows, so that every wavefront still holds one chunk of 256 consecutive cells per band) and keeps
 // their state (y, the seven stage derivatives, the dense-output coefficients) in
 // registers for the whole solve.  Only the stage input travels through LDS, double
 // buffered, so that the five-point stencil can read its neighbours: one barrier per
@@ -29,9 +31,9 @@ struct GridOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
 };
 
-template <typename T, int NW> struct GridShared {
-    T xch[2][NW * 256];  // stage input, double buffered
-    T red[2][NW][2];     // wavefront sums of up to two reductions, double buffered
+template <typename T, int NW, int R> struct GridShared {
+    T xch[2][R * NW * 256];  // stage input, double buffered
+    T red[2][R][NW][2];      // chunk sums of up to two reductions, double buffered
 };
 
 // Four consecutive values, moved with the widest loads and stores their alignment allows.
@@ -44,61 +46,75 @@ template <typename T> __device__ __forceinline__ void load4(const T *from, T (&v
 }
 template <typename T> __device__ __forceinline__ void store4(T *to, const T (&v)[4]) { *reinterpret_cast<Four<T> *>(to) = Four<T>{v[0], v[1], v[2], v[3]}; }
 
-// Sum over the workgroup of two per-thread partial sums, in the fixed order.
-template <typename T, int NW> __device__ __forceinline__ void block_sum2(GridShared<T, NW> &sh, int &slot, T a, T b, T &A, T &B) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        a = a + __shfl_xor(a, off);
-        b = b + __shfl_xor(b, off);
-    }
+// Sum over the row of two per-thread partial sums per band, in the fixed order: the chunk of 256 cells that wavefront w
+// holds of band r is chunk r * NW + w of the row, and the chunk sums are added in that order.
+template <typename T, int NW, int R> __device__ __forceinline__ void block_sum2(GridShared<T, NW, R> &sh, int &slot, const T (&a)[R], const T (&b)[R], T &A, T &B) {
     const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
-        sh.red[slot][wave][0] = a;
-        sh.red[slot][wave][1] = b;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        T u = a[r], v = b[r];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            u = u + __shfl_xor(u, off);
+            v = v + __shfl_xor(v, off);
+        }
+        if ((threadIdx.x & 63) == 0) {
+            sh.red[slot][r][wave][0] = u;
+            sh.red[slot][r][wave][1] = v;
+        }
     }
     lds_barrier();
     A = 0;
     B = 0;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-        A = A + sh.red[slot][w][0];
-        B = B + sh.red[slot][w][1];
-    }
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            A = A + sh.red[slot][r][w][0];
+            B = B + sh.red[slot][r][w][1];
+        }
     slot ^= 1;
 }
 
 // du/dt = D * lap(u) + u * (1 - u) on the periodic grid; each operation rounds on its own, in the
 // order of the torch expression  (((up + down) + left) + right) - 4u,  D * lap + u * (1 - u).
-template <typename T, int N, int NW>
-__device__ __forceinline__ void grid_rhs(GridShared<T, NW> &sh, int &buf, T D, const T (&u)[4], T (&out)[4]) {
+template <typename T, int N, int NW, int R>
+__device__ __forceinline__ void grid_rhs(GridShared<T, NW, R> &sh, int &buf, T D, const T (&u)[R][4], T (&out)[R][4]) {
     const int t = threadIdx.x;
-    constexpr int PER_ROW = N / 4;
-    const int r = t / PER_ROW, c0 = 4 * (t - r * PER_ROW);
+    constexpr int PER_ROW = N / 4, BAND = N * N / R, BAND_ROWS = N / R;
+    const int rl = t / PER_ROW, c0 = 4 * (t - rl * PER_ROW);
     T *x = sh.xch[buf];
-    store4<T>(x + 4 * t, u);
-    lds_barrier();
-    const int ru = (r + N - 1) & (N - 1), rd = (r + 1) & (N - 1);
-    T ups[4], dns[4];
-    load4<T>(x + ru * N + c0, ups);
-    load4<T>(x + rd * N + c0, dns);
-    const T lf = x[r * N + ((c0 + N - 1) & (N - 1))];
-    const T rt = x[r * N + ((c0 + 4) & (N - 1))];
-    const T lfs[4] = {lf, u[0], u[1], u[2]}, rts[4] = {u[1], u[2], u[3], rt};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const T lap = (((ups[j] + dns[j]) + lfs[j]) + rts[j]) - ((T)4 * u[j]);
-        const T diff = D * lap;
-        const T react = u[j] * ((T)1 - u[j]);
-        out[j] = diff + react;
+    for (int r = 0; r < R; ++r) store4<T>(x + r * BAND + 4 * t, u[r]);
+    lds_barrier();
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = r * BAND_ROWS + rl;
+        const int ru = (row + N - 1) & (N - 1), rd = (row + 1) & (N - 1);
+        T ups[4], dns[4];
+        load4<T>(x + ru * N + c0, ups);
+        load4<T>(x + rd * N + c0, dns);
+        const T lf = x[row * N + ((c0 + N - 1) & (N - 1))];
+        const T rt = x[row * N + ((c0 + 4) & (N - 1))];
+        const T lfs[4] = {lf, u[r][0], u[r][1], u[r][2]}, rts[4] = {u[r][1], u[r][2], u[r][3], rt};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const T lap = (((ups[j] + dns[j]) + lfs[j]) + rts[j]) - ((T)4 * u[r][j]);
+            const T diff = D * lap;
+            const T react = u[r][j] * ((T)1 - u[r][j]);
+            out[r][j] = diff + react;
+        }
     }
     buf ^= 1;
 }
 
+constexpr int grid_bands(int n) { return n * n / 4 > 1024 ? n * n / 4 / 1024 : 1; }
+
 template <typename T, int METHOD, int CTRL, int N>
-__global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<T> p, const GridOut o) {
+__global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(const SolveParams<T> p, const GridOut o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
-    constexpr int F = N * N, NT = F / 4, NW = NT / 64;
-    __shared__ GridShared<T, NW> sh;
+    constexpr int F = N * N, R = grid_bands(N), NT = F / 4 / R, NW = NT / 64, BAND = F / R;
+    __shared__ GridShared<T, NW, R> sh;
     extern __shared__ __align__(16) unsigned char dyn[];
     T *te_s = reinterpret_cast<T *>(dyn);  // [E] evaluation times of this sample
 
@@ -114,8 +130,9 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
     const T dir = (te > ts) ? (T)1 : (T)-1;
     const T tlo = tmin(ts, te), thi = tmax(te, ts);
     const T D = p.params[b];
-    T y[4], k[7][4];
-    load4<T>(p.y0 + b * F + 4 * tid, y);
+    T y[R][4], k[7][R][4];
+#pragma unroll
+    for (int r = 0; r < R; ++r) load4<T>(p.y0 + b * F + r * BAND + 4 * tid, y[r]);
     __syncthreads();  // te_s
 
     bool bail = false;
@@ -123,41 +140,52 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
 
     // ---- first step size (step_size_controllers.py:431-490, 776-835) ----
     T t = ts, dt;
-    grid_rhs<T, N, NW>(sh, buf, D, y, k[0]);
+    grid_rhs<T, N, NW, R>(sh, buf, D, y, k[0]);
     if (p.dt0) {
         dt = p.dt0[b];
     } else {
-        T inv[4], a0 = 0, a1 = 0, A0, A1;
+        T inv[R][4], a0[R], a1[R], A0, A1;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            inv[j] = inv_scale(cp.atol, cp.rtol, y[j]);
-            const T x0 = (y[j] * inv[j]) / sf, x1 = (k[0][j] * inv[j]) / sf;
-            a0 = fma_(x0, x0, a0);
-            a1 = fma_(x1, x1, a1);
+        for (int r = 0; r < R; ++r) {
+            a0[r] = 0, a1[r] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                inv[r][j] = inv_scale(cp.atol, cp.rtol, y[r][j]);
+                const T x0 = (y[r][j] * inv[r][j]) / sf, x1 = (k[0][r][j] * inv[r][j]) / sf;
+                a0[r] = fma_(x0, x0, a0[r]);
+                a1[r] = fma_(x1, x1, a1[r]);
+            }
         }
-        block_sum2<T, NW>(sh, slot, a0, a1, A0, A1);
+        block_sum2<T, NW, R>(sh, slot, a0, a1, A0, A1);
         const T d0 = sqrt_(A0), d1 = sqrt_(A1);
         T h0 = (d0 < (T)1e-5 || d1 < (T)1e-5) ? (T)1e-6 : ((T)0.01 * d0) / d1;
         h0 = tmin(h0, abs_(te - ts));
-        T y1[4], f1[4];
+        T y1[R][4], f1[R][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) y1[j] = fma_(dir * h0, k[0][j], y[j]);
-        grid_rhs<T, N, NW>(sh, buf, D, y1, f1);
-        T a2 = 0, A2, unused;
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const T df = f1[j] - k[0][j];
-            const T x2 = (df * inv[j]) / sf;
-            a2 = fma_(x2, x2, a2);
+            for (int j = 0; j < 4; ++j) y1[r][j] = fma_(dir * h0, k[0][r][j], y[r][j]);
+        grid_rhs<T, N, NW, R>(sh, buf, D, y1, f1);
+        T a2[R], none[R], A2, unused;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            a2[r] = 0, none[r] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const T df = f1[r][j] - k[0][r][j];
+                const T x2 = (df * inv[r][j]) / sf;
+                a2[r] = fma_(x2, x2, a2[r]);
+            }
         }
-        block_sum2<T, NW>(sh, slot, a2, (T)0, A2, unused);
+        block_sum2<T, NW, R>(sh, slot, a2, none, A2, unused);
         dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, h0, d1, sqrt_(A2));
     }
     dt = tclamp(dt, tlo - t, thi - t);
 
     int cursor = 0, n_steps = 0, n_acc = 0;
     if (E > 0 && te_s[0] == ts) {
-        store4<T>(p.ys + (b * E) * F + 4 * tid, y);
+#pragma unroll
+        for (int r = 0; r < R; ++r) store4<T>(p.ys + (b * E) * F + r * BAND + 4 * tid, y[r]);
         cursor = 1;
     }
     T prev = 1, pprev = 1;
@@ -169,36 +197,44 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
     while (!bail) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
-        T y1[4];
+        T y1[R][4];
 #pragma unroll
         for (int i = 1; i < 7; ++i) {
-            T yi[4];
+            T yi[R][4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                T s = 0;
+            for (int r = 0; r < R; ++r)
 #pragma unroll
-                for (int jj = 0; jj < i; ++jj) s = fma_((T)Tab::a[i][jj], k[jj][j], s);
-                yi[j] = fma_(dt, s, y[j]);
-            }
-            grid_rhs<T, N, NW>(sh, buf, D, yi, k[i]);
+                for (int j = 0; j < 4; ++j) {
+                    T s = 0;
+#pragma unroll
+                    for (int jj = 0; jj < i; ++jj) s = fma_((T)Tab::a[i][jj], k[jj][r][j], s);
+                    yi[r][j] = fma_(dt, s, y[r][j]);
+                }
+            grid_rhs<T, N, NW, R>(sh, buf, D, yi, k[i]);
             if (i == 6) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) y1[j] = yi[j];
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) y1[r][j] = yi[r][j];
             }
         }
 
         // ---- error ratio (runge_kutta.py:267, step_size_controllers.py:389-395); long rows: fused sums ----
-        T part = 0, total, unused;
+        T part[R], none[R], total, unused;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            T err = 0;
+        for (int r = 0; r < R; ++r) {
+            part[r] = 0, none[r] = 0;
 #pragma unroll
-            for (int s = 0; s < 7; ++s) err = fma_(dt * (T)Tab::b_err[s], k[s][j], err);
-            const T m = tmax(abs_(y[j]), abs_(y1[j]));
-            const T x = (abs_(err) / fma_(cp.rtol, m, cp.atol)) / sf;
-            part = fma_(x, x, part);
+            for (int j = 0; j < 4; ++j) {
+                T err = 0;
+#pragma unroll
+                for (int s = 0; s < 7; ++s) err = fma_(dt * (T)Tab::b_err[s], k[s][r][j], err);
+                const T m = tmax(abs_(y[r][j]), abs_(y1[r][j]));
+                const T x = (abs_(err) / fma_(cp.rtol, m, cp.atol)) / sf;
+                part[r] = fma_(x, x, part[r]);
+            }
         }
-        block_sum2<T, NW>(sh, slot, part, (T)0, total, unused);
+        block_sum2<T, NW, R>(sh, slot, part, none, total, unused);
         const T ratio = tmax(sqrt_(total), (T)1e-38);
         const bool accept = ratio < (T)1;
         T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
@@ -214,38 +250,48 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
         n_acc += accept ? 1 : 0;
 
         // ---- dense output at the evaluation points this step passed (adjoints.py:215-234) ----
+        // (band by band: the coefficients of one band at a time are alive)
         if (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0) {
-            T q[4][5][1];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                T ks[7];
-#pragma unroll
-                for (int s = 0; s < 7; ++s) ks[s] = k[s][j];
-                quartic_elem<T, METHOD>(dt, y[j], y1[j], ks, true, q[j]);
-            }
             const T t1 = t0 + dt;
-            do {
-                const T x = unit_time(te_s[cursor], t0, t1);
-                T out[4];
+            int reached = cursor;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                T q[4][5][1];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    T v = q[j][4][0];
+                    T ks[7];
 #pragma unroll
-                    for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
-                    out[j] = v;
+                    for (int s = 0; s < 7; ++s) ks[s] = k[s][r][j];
+                    quartic_elem<T, METHOD>(dt, y[r][j], y1[r][j], ks, true, q[j]);
                 }
-                store4<T>(p.ys + (b * E + cursor) * F + 4 * tid, out);
-                ++cursor;
-            } while (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0);
+                int at = cursor;
+                do {
+                    const T x = unit_time(te_s[at], t0, t1);
+                    T out[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        T v = q[j][4][0];
+#pragma unroll
+                        for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
+                        out[j] = v;
+                    }
+                    store4<T>(p.ys + (b * E + at) * F + r * BAND + 4 * tid, out);
+                    ++at;
+                } while (at < E && fma_(dir, t_new, -dir * te_s[at]) >= (T)0);
+                reached = at;
+            }
+            cursor = reached;
         }
 
         // ---- state update (adjoints.py:150-155, 247-255) ----
         if (accept) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                y[j] = y1[j];
-                k[0][j] = k[6][j];
-            }
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    y[r][j] = y1[r][j];
+                    k[0][r][j] = k[6][r][j];
+                }
         }
         t = t_new;
         dt = tclamp(running_new ? dt_next : dt, tlo - t, thi - t);
@@ -262,7 +308,9 @@ __global__ void __launch_bounds__(N *N / 4) solve_grid_kernel(const SolveParams<
             // common case; one that landed past t_end is looked at in one more iteration
             int odd = 0;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) odd |= !settles_(y[j], k[0][j]);
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) odd |= !settles_(y[r][j], k[0][r][j]);
             if (__syncthreads_or(odd)) bail = true;
             if (bail || t == te) break;
             idle = true;
@@ -286,7 +334,7 @@ template <typename T, int METHOD, int CTRL, int N> static int launch_grid(const 
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
     const size_t lds = (size_t)a.n_eval * sizeof(T);
     timing_before(stream, "tode::solve_grid_kernel");
-    hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4), lds, stream, p, o);
+    hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4 / grid_bands(N)), lds, stream, p, o);
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }
@@ -307,7 +355,12 @@ template <typename T> static int solve_grid(const tode_solve_args &a, const tode
     if (a.n_features == 64 * 64) return grid_mc<T, 64>(a, c, o, s);
     if (a.n_features == 32 * 32) return grid_mc<T, 32>(a, c, o, s);
     if (a.n_features == 16 * 16) return grid_mc<T, 16>(a, c, o, s);  // (one wavefront per sample)
-    return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 16 x 16, 32 x 32 and 64 x 64 grids, got F=%d", a.n_features);
+    if (sizeof(T) == 4 && a.n_features == 128 * 128) {
+        // (128 KB of LDS for the double-buffered stage input leave 30 KB for the sample's evaluation times)
+        if (a.n_eval > 4096) return fail(TODE_E_UNSUPPORTED, "n_eval=%d is too large for the grid kernel on the 128 x 128 grid", a.n_eval);
+        return grid_mc<float, 128>(a, c, o, s);
+    }
+    return fail(TODE_E_UNSUPPORTED, "the grid kernel is built for 16 x 16, 32 x 32 and 64 x 64 grids (float32 also 128 x 128), got F=%d", a.n_features);
 }
 
 int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
