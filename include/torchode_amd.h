@@ -45,7 +45,7 @@ enum {
     TODE_TERM_LORENZ63 = 2,           /* F = 3, rho [B]; sigma, beta in term_scalars */
     TODE_TERM_REACTION_DIFFUSION = 3, /* F = N*N periodic grid (N = 16, 32 or 64; float32 also 128), du/dt = D lap(u) + u (1 - u),
                                          D [B]; float32 or float64 (time and data alike), tode_solve_builtin_fast only */
-    TODE_TERM_MLP = 4                 /* F = 4, 8, ..., 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units,
+    TODE_TERM_MLP = 4                 /* F = 1 ... 64: tanh([y, t] W1^T + b1) W2^T + b2 with up to 256 hidden units,
                                          weights in shared_params as packed by tode_mlp_pack_weights[_for]; float32,
                                          tode_solve_builtin_fast only */
 };
@@ -372,14 +372,15 @@ int tode_select_end_point(int64_t batch, int32_t n_features, int32_t dtype, int6
 int tode_mlp_pack_weights(const void *raw, int64_t n_raw, int32_t matrix_inputs, void *packed, void *stream);
 
 /*
- * The same for a network on n_features = 4, 8, ..., 64 state values (the solve
+ * The same for a network on n_features = 1 ... 64 state values (the solve
  * then takes n_features of that size and rows of that many values in y0 and
  * ys): `raw` is W1 [H x (n_features + 1)] | b1 [H] | W2 [n_features x H] |
  * b2 [n_features], n_raw = (2 n_features + 2) H + n_features.  The kernel always
  * works on 64 values per sample: the state values from n_features on are zero,
  * their weights are packed as zeros, and the root mean squares divide by
  * n_features, so the sums hold only exact zeros beyond the network's own terms.
- * `packed` has the same size as for 64 features.
+ * `packed` has the same size as for 64 features.  (Rows of a multiple of four values
+ * are loaded and stored 16 bytes at a time, others value by value.)
  * tode_mlp_pack_weights(...) == tode_mlp_pack_weights_for(..., 64, ...).
  */
 int tode_mlp_pack_weights_for(const void *raw, int64_t n_raw, int32_t n_features, int32_t matrix_inputs, void *packed, void *stream);

@@ -452,11 +452,12 @@ def narrow_mlp_problem(features, hidden, batch, inputs="float32", seed=0):
 
 
 @pytest.mark.parametrize("inputs", ["float32", "bfloat16"])
-@pytest.mark.parametrize("features,hidden,batch", [(4, 256, 96), (8, 5, 37), (32, 100, 96), (48, 256, 250), (60, 64, 96)])
+@pytest.mark.parametrize("features,hidden,batch", [(4, 256, 96), (8, 5, 37), (32, 100, 96), (48, 256, 250), (60, 64, 96), (1, 16, 50), (2, 256, 96), (3, 40, 33), (6, 16, 24), (17, 100, 96), (63, 256, 70)])
 def test_mlp_kernel_with_fewer_features(features, hidden, batch, inputs):
-    """The kernel works on 64 values per sample; a network on 4, 8, ..., 60 of them is packed with zero weights for the
-    rest, whose state stays zero, and the root mean squares divide by the network's own count: against the protocol
-    path with torch's matrix products of the network itself."""
+    """The kernel works on 64 values per sample; a network on fewer of them is packed with zero weights for the rest,
+    whose state stays zero, and the root mean squares divide by the network's own count (rows of a multiple of four
+    values move 16 bytes at a time, others value by value): against the protocol path with torch's matrix products of
+    the network itself."""
     w = narrow_mlp_problem(features, hidden, batch, inputs)
     kernel = "tode::solve_mlp_kernel" + ("" if inputs == "float32" else " (bfloat16 matrix inputs)")
     tight = dict(kind="pid", atol=1e-6, rtol=1e-4, pcoeff=0.2, icoeff=0.5, dcoeff=0.1)
@@ -496,16 +497,17 @@ def test_mlp_weight_packing_with_fewer_features():
         _lib.check(lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel(), 8, _lib.MLP_INPUTS[inputs], _lib.ptr(a), _lib.stream_of(raw)), "pack")
         _lib.check(lib.tode_mlp_pack_weights(_lib.ptr(wide), wide.numel(), _lib.MLP_INPUTS[inputs], _lib.ptr(b), _lib.stream_of(raw)), "pack")
         assert torch.equal(a.view(torch.int32), b.view(torch.int32)), inputs
-    for n_features in (0, 6, 68):
+    for n_features in (0, 65, 68):
         assert lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel(), n_features, 0, _lib.ptr(a), _lib.stream_of(raw)) == _lib.E_UNSUPPORTED
-    assert lib.tode_mlp_pack_weights_for(_lib.ptr(raw), raw.numel() - 1, 8, 0, _lib.ptr(a), _lib.stream_of(raw)) == _lib.E_UNSUPPORTED
-    # six features: not a size of the matrix-core kernel, the solve takes the per-step kernels and still agrees
+    for n_raw in (raw.numel() - 1, raw.numel() + 3):  # (not W1 | b1 | W2 | b2 of any hidden width on 8 features)
+        assert lib.tode_mlp_pack_weights_for(_lib.ptr(raw), n_raw, 8, 0, _lib.ptr(a), _lib.stream_of(raw)) == _lib.E_UNSUPPORTED
+    # 65 features: not a size of the matrix-core kernel, the solve takes the per-step kernels and still agrees
     v = to.workloads.make("vdp", batch=8, device="cuda")  # (another solve first: the library keeps the last kernel's name)
     to.AutoDiffAdjoint(to.Dopri5(), make_controller(v.controller)).solve(to.InitialValueProblem(v.y0, t_eval=v.t_eval), to.ODETerm(v.f))
-    odd = narrow_mlp_problem(6, 16, 24)
-    problem = to.InitialValueProblem(odd.y0, t_eval=odd.t_eval)
-    got = to.AutoDiffAdjoint(to.Dopri5(), make_controller(odd.controller)).solve(problem, to.ODETerm(odd.f))
-    want = to.AutoDiffAdjoint(OwnDopri5(), make_controller(odd.controller)).solve(problem, to.ODETerm(odd.f))
+    wide = narrow_mlp_problem(65, 16, 24)
+    problem = to.InitialValueProblem(wide.y0, t_eval=wide.t_eval)
+    got = to.AutoDiffAdjoint(to.Dopri5(), make_controller(wide.controller)).solve(problem, to.ODETerm(wide.f))
+    want = to.AutoDiffAdjoint(OwnDopri5(), make_controller(wide.controller)).solve(problem, to.ODETerm(wide.f))
     assert not _lib.last_solve_kernel_name().startswith("tode::solve_mlp_kernel")
     assert_close_solutions(got, want, min_agree=0.95, loose=1e-2)
 

@@ -185,7 +185,7 @@ class AutoDiffAdjoint(nn.Module):
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
             return (F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192) or (F == 128 * 128 and problem.data_dtype == torch.float32 and E <= 4096)
-        return problem.data_dtype == torch.float32 and 4 <= F <= 64 and F % 4 == 0 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
+        return problem.data_dtype == torch.float32 and 1 <= F <= 64 and f.W1.shape[1] == F + 1 and 1 <= f.W1.shape[0] <= 256 and E <= 512
 
     @torch.compiler.disable
     def _solve_eager_outside_the_trace(self, problem, term, dt0, args) -> Solution:
@@ -576,9 +576,9 @@ class AutoDiffAdjoint(nn.Module):
         assert params.shape[0] == B, "built-in term parameters do not match the batch size"
         mlp = f.builtin_kind == _lib.TERM_MLP
         if mlp and (
-            dtype != torch.float32 or not 4 <= F <= 64 or F % 4 or f.W1.shape[1] != F + 1 or not 1 <= f.W1.shape[0] <= 256
+            dtype != torch.float32 or not 1 <= F <= 64 or f.W1.shape[1] != F + 1 or not 1 <= f.W1.shape[0] <= 256
         ):
-            return None  # the matrix-core kernel takes 4, 8, ..., 64 features and up to 256 hidden units: the caller takes another path
+            return None  # the matrix-core kernel takes up to 64 features and up to 256 hidden units: the caller takes another path
         shared = f.builtin_packed(dev, dtype) if mlp else None
         ttype = t_start.dtype
         dt0_ = None if dt0 is None else dt0.to(ttype).contiguous()

@@ -514,7 +514,7 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
             one_kernel = one_kernel && ((a->n_features == 16 * 16 || a->n_features == 32 * 32 || a->n_features == 64 * 64) ? E <= 8192
                                                                                                                            : (a->n_features == 128 * 128 && a->dtype == TODE_F32 && E <= 4096));
         else if (a->term == TODE_TERM_MLP)
-            one_kernel = one_kernel && a->dtype == TODE_F32 && a->n_features >= 4 && a->n_features <= 64 && a->n_features % 4 == 0 && E <= 512;
+            one_kernel = one_kernel && a->dtype == TODE_F32 && a->n_features >= 1 && a->n_features <= 64 && E <= 512;
         else
             return fail(TODE_E_INVALID, "unknown term %d", a->term);
         if (!one_kernel) return fail(TODE_E_UNSUPPORTED, "no whole-solve kernel for this term in this shape, dtype or controller setting");

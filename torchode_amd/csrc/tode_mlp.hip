@@ -36,7 +36,7 @@ typedef float mfma_acc __attribute__((ext_vector_type(4)));
 
 struct MlpOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
-    int n_features;  // features of the problem: a multiple of four, at most 64 (the kernel's others stay zero)
+    int n_features;  // features of the problem: at most 64 (the kernel's others stay zero)
 };
 
 constexpr int MLP_F = 64, MLP_H = 256, MLP_TILE = 16;
@@ -77,7 +77,7 @@ __host__ __device__ __forceinline__ int mlp_input_of(int kk, int q) { return kk 
 // Source index (in W1 | b1 | W2 | b2, row-major) of packed value j of thread tid, or -1 for zero.  H: hidden units of
 // the network at hand, at most MLP_H; the kernel's units from H on get zero weights and a zero bias, so that they
 // add tanh(0) * 0 = 0 to every sum in the same places as before (a narrower network in the same arithmetic).
-// FR: features of the network at hand (a multiple of four, at most MLP_F): W1 is [H x (FR + 1)] with the time in its last
+// FR: features of the network at hand (at most MLP_F): W1 is [H x (FR + 1)] with the time in its last
 // column, W2 [FR x H]; the kernel's features from FR on get zero weights on both sides and stay zero throughout.
 __host__ __device__ inline long long mlp_packed_source(int j, int tid, int H, int FR) {
     const int lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
@@ -350,7 +350,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int FR = o.n_features;  // the problem's features; the kernel's others (FR .. 63) are zero in every vector
     const T sf = (T)__builtin_sqrt((double)FR);
     const int f0 = 16 * w + 4 * q;  // the lane's first feature
-    const bool has = f0 < FR;       // (FR is a multiple of four: the lane's four features are the problem's, or none is)
+    const bool has = f0 < FR;       // (some of the lane's four features are the problem's)
+    const bool quads = (FR & 3) == 0;  // rows of whole groups of four: 16-byte loads and stores
+    auto put = [&](T *row, const T (&v)[4]) {  // the lane's share of one row of ys
+        if (quads) {
+            if (has) *reinterpret_cast<float4 *>(row + f0) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (f0 + r < FR) row[f0 + r] = v[r];
+        }
+    };
     int slot = 0;
 
     // ---- weights into registers ----
@@ -370,8 +380,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int e = 1; e < E; ++e) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));  // not monotone
     T y[4], k[7][4];
     {
-        const float4 v = has ? *reinterpret_cast<const float4 *>(p.y0 + bs * FR + f0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        y[0] = v.x, y[1] = v.y, y[2] = v.z, y[3] = v.w;
+        if (quads) {
+            const float4 v = has ? *reinterpret_cast<const float4 *>(p.y0 + bs * FR + f0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            y[0] = v.x, y[1] = v.y, y[2] = v.z, y[3] = v.w;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[r] = f0 + r < FR ? p.y0[bs * FR + f0 + r] : 0.0f;
+        }
     }
     T t = ts, dt, prev = 1, pprev = 1;
     int cursor = 0, n_steps = 0, n_acc = 0;
@@ -407,7 +422,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     dt = tclamp(dt, tlo - t, thi - t);
     bool active = live;
     if (live && E > 0 && tev[0] == ts) {
-        if (has) *reinterpret_cast<float4 *>(p.ys + (bs * E) * FR + f0) = make_float4(y[0], y[1], y[2], y[3]);
+        put(p.ys + (bs * E) * FR, y);
         cursor = 1;
     }
     int vslot = 0;
@@ -486,7 +501,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
                     for (int pw = 3; pw >= 0; --pw) v[r] = fma_(v[r], x, qc[r][pw][0]);
                 }
-                if (has) *reinterpret_cast<float4 *>(p.ys + (bs * E + cursor) * FR + f0) = make_float4(v[0], v[1], v[2], v[3]);
+                put(p.ys + (bs * E + cursor) * FR, v);
                 ++cursor;
             } while (cursor < E && fma_(dir, t_new, -dir * tev[cursor]) >= (T)0);
         }
@@ -552,9 +567,9 @@ template <typename Weights> static int solve_mlp_with(const tode_solve_args &a, 
 
 int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s) {
     const bool f32 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE, bf16 = a.n_shared_params == (long long)TODE_MLP_PACKED_SIZE_BF16;
-    if (a.n_features < 4 || a.n_features > MLP_F || a.n_features % 4 != 0 || !(f32 || bf16))
+    if (a.n_features < 1 || a.n_features > MLP_F || !(f32 || bf16))
         return fail(TODE_E_UNSUPPORTED,
-                    "the MLP kernel is built for 4, 8, ..., 64 features and up to 256 hidden units, with the weights packed by tode_mlp_pack_weights "
+                    "the MLP kernel is built for 1 to 64 features and up to 256 hidden units, with the weights packed by tode_mlp_pack_weights "
                     "(%d or %d values); got F=%d and %lld shared parameters", TODE_MLP_PACKED_SIZE, TODE_MLP_PACKED_SIZE_BF16, a.n_features,
                     (long long)a.n_shared_params);
     if (!a.shared_params) return fail(TODE_E_INVALID, "null shared_params");
@@ -568,7 +583,7 @@ int mlp_pack_weights(const float *raw, long long n_raw, int n_features, int matr
     static_assert(TODE_MLP_PACKED_SIZE == MLP_REGS * 256 && TODE_MLP_PACKED_SIZE_BF16 == MLP_REGS_BF16 * 256, "packed sizes");
     if (!raw || !packed) return fail(TODE_E_INVALID, "null pointer");
     const long long FR = n_features;
-    if (FR < 4 || FR > MLP_F || FR % 4 != 0) return fail(TODE_E_UNSUPPORTED, "the MLP kernel takes 4, 8, ..., %d features, got %lld", MLP_F, FR);
+    if (FR < 1 || FR > MLP_F) return fail(TODE_E_UNSUPPORTED, "the MLP kernel takes 1 to %d features, got %lld", MLP_F, FR);
     // W1 [H x (F + 1)] | b1 [H] | W2 [F x H] | b2 [F] = (2 F + 2) H + F values for H hidden units, 1 <= H <= 256
     const long long H = (n_raw - FR) / (2 * FR + 2);
     if (n_raw < FR || H * (2 * FR + 2) + FR != n_raw || H < 1 || H > MLP_H)
