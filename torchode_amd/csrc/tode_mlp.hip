@@ -333,7 +333,8 @@ __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (
     slot ^= 1;
 }
 
-template <int METHOD, int CTRL, typename Weights>
+// FULL: all 64 state values are the problem's (the feature count is a constant and its tests fold away).
+template <int METHOD, int CTRL, typename Weights, bool FULL>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) solve_mlp_kernel(const SolveParams<float> p, const float *packed, const MlpOut o) {
     using T = float;
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
@@ -347,7 +348,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int rows = (int)min((long long)MLP_TILE, p.batch - b0);
     const int E = p.n_eval;
     const CtrlParams<T> &cp = p.cp;
-    const int FR = o.n_features;  // the problem's features; the kernel's others (FR .. 63) are zero in every vector
+    const int FR = FULL ? MLP_F : o.n_features;  // the problem's features; the kernel's others (FR .. 63) are zero in every vector
     const T sf = (T)__builtin_sqrt((double)FR);
     const int f0 = 16 * w + 4 * q;  // the lane's first feature
     const bool has = f0 < FR;       // (some of the lane's four features are the problem's)
@@ -552,7 +553,10 @@ template <int METHOD, int CTRL, typename Weights> static int launch_mlp(const to
     const size_t lds = (size_t)MLP_TILE * a.n_eval * sizeof(float);
     const unsigned blocks = (unsigned)((a.batch + MLP_TILE - 1) / MLP_TILE);
     timing_before(stream, std::is_same<Weights, MlpWeightsBf16>::value ? "tode::solve_mlp_kernel (bfloat16 matrix inputs)" : "tode::solve_mlp_kernel");
-    hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
+    if (o.n_features == MLP_F)
+        hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights, true>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
+    else
+        hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights, false>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }
