@@ -236,8 +236,8 @@ int tode_finalize_stats(int64_t batch, int64_t last_iteration, const int32_t *n_
  *
  * n_eval == 0 (the reference's t_eval=None, adjoints.py:296-311: the end point
  * alone, ys of shape [B,1,F]) is covered for the small systems (linear decay,
- * Van der Pol, Lorenz) and batches of up to TODE_END_ONLY_MAX_BATCH samples;
- * otherwise TODE_E_UNSUPPORTED.  `t_eval` may then be null and `y_idle` [B,F]
+ * Van der Pol, Lorenz) in batches of up to TODE_END_ONLY_MAX_BATCH samples and
+ * for the grid and MLP terms; otherwise TODE_E_UNSUPPORTED.  `t_eval` may then be null and `y_idle` [B,F]
  * must be given: the kernel leaves in ys[b] the dense output of sample b's last
  * step at t_end and in y_idle[b] its final state, and the caller, once it has
  * read the flags, finishes with tode_select_end_point(...,

@@ -275,6 +275,41 @@ def test_grid_kernel_on_a_128_by_128_grid(method, kind):
                 to.AutoDiffAdjoint(own_m(), make_controller(ctrl)).solve(problem, to.ODETerm(f)))  # fmt: skip
 
 
+def test_grid_and_mlp_kernels_without_evaluation_points(monkeypatch):
+    """t_eval=None (adjoints.py:296-311): the kernels take t_end as the sample's one point and leave the final state
+    next to the dense output of its last step there; which of the two a sample gets depends on whether the batch went
+    on after it (tode_select_end_point).  Spans of different lengths, so that most samples finish before the last."""
+    from torchode_amd import _lib
+
+    def no_other_path(*a, **kw):
+        raise AssertionError("the whole-solve kernel gave the batch up")
+
+    monkeypatch.setattr(to.AutoDiffAdjoint, "_solve_stepwise", no_other_path)
+    for n, dtype in ((32, torch.float32), (64, torch.float64), (128, torch.float32), (16, torch.float32)):
+        f, y0, t_eval = rd_problem(9, n=n, t1=4.0, d_max=1.0, dtype=dtype)
+        problem = to.InitialValueProblem(y0, t_eval[:, 0].clone(), t_eval[:, -1].clone())
+        if n == 16:  # spans whose last step lands past t_end for some samples: their end point is the next step's interpolant
+            t_start, t_end, _ = spans_that_miss_t_end(9, 2, seed=5)
+            problem = to.InitialValueProblem(y0, t_start.cuda(), t_end.cuda())
+        for method, own in ((to.Tsit5, OwnTsit5), (to.Dopri5, OwnDopri5)):
+            ctrl = dict(kind="integral", atol=1e-7, rtol=1e-5)
+            fused = to.AutoDiffAdjoint(method(), make_controller(ctrl)).solve(problem, to.ODETerm(f))
+            assert _lib.last_solve_kernel_name() == "tode::solve_grid_kernel" and fused.ys.shape == (9, 1, n * n)
+            proto = to.AutoDiffAdjoint(own(), make_controller(ctrl)).solve(problem, to.ODETerm(f))
+            assert_same(fused, proto)
+            assert fused.stats["n_steps"].min() < fused.stats["n_steps"].max()
+    for features, hidden in ((64, 256), (10, 33)):
+        w = narrow_mlp_problem(features, hidden, 250)
+        t_end = (0.2 + torch.rand(250, generator=torch.Generator().manual_seed(1))).cuda()
+        problem = to.InitialValueProblem(w.y0, torch.zeros(250, device="cuda"), t_end)
+        ctrl = dict(kind="integral", atol=1e-6, rtol=1e-4)
+        fused = to.AutoDiffAdjoint(to.Dopri5(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f))
+        assert _lib.last_solve_kernel_name() == "tode::solve_mlp_kernel" and fused.ys.shape == (250, 1, features)
+        proto = to.AutoDiffAdjoint(OwnDopri5(), make_controller(ctrl)).solve(problem, to.ODETerm(w.f))
+        assert fused.stats["n_steps"].min() < fused.stats["n_steps"].max()
+        assert_close_solutions(fused, proto, min_agree=0.9)
+
+
 def test_grid_kernel_hands_uncommon_cases_to_the_protocol_path():
     from torchode_amd import _lib
 

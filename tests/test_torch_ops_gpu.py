@@ -77,6 +77,8 @@ CASES = [
     ("mlp", 64, torch.float32, "plain", {}),
     ("reaction_diffusion", 4, torch.float32, "plain", {}),
     ("reaction_diffusion", 3, torch.float64, "plain", {}),
+    ("mlp", 64, torch.float32, "end-only", {}),
+    ("reaction_diffusion", 4, torch.float32, "end-only", {}),
 ]
 
 

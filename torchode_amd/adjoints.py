@@ -181,7 +181,7 @@ class AutoDiffAdjoint(nn.Module):
         if f.builtin_kind in _lib.GENERAL_TERMS:
             return True
         c, E, F = self.step_size_controller, problem.n_evaluation_points, problem.n_features
-        if c.dt_min is not None or c.dt_max is not None or E == 0 or problem.data_dtype != problem.time_dtype:
+        if c.dt_min is not None or c.dt_max is not None or problem.data_dtype != problem.time_dtype:
             return False
         if f.builtin_kind == _lib.TERM_REACTION_DIFFUSION:
             return (F in (16 * 16, 32 * 32, 64 * 64) and E <= 8192) or (F == 128 * 128 and problem.data_dtype == torch.float32 and E <= 4096)

@@ -269,8 +269,6 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
     if (a->batch < 0 || a->n_features <= 0 || a->n_eval < 0 || a->n_params < 0)
         return fail(TODE_E_INVALID, "bad sizes: batch=%lld F=%d E=%d P=%d", (long long)a->batch, a->n_features, a->n_eval, a->n_params);
     const bool end_only = a->n_eval == 0;
-    if (end_only && (a->term == TODE_TERM_REACTION_DIFFUSION || a->term == TODE_TERM_MLP))
-        return fail(TODE_E_UNSUPPORTED, "without evaluation points the fast entry point covers the small systems only");
     if (end_only && a->batch > 0 && !a->y_idle) return fail(TODE_E_INVALID, "n_eval == 0 needs y_idle");
     if (c->has_dt_min || c->has_dt_max) return fail(TODE_E_UNSUPPORTED, "the fast entry point does not take dt_min / dt_max");
     if (c->kind != TODE_CTRL_INTEGRAL && c->kind != TODE_CTRL_PID) return fail(TODE_E_INVALID, "unknown controller kind %d", c->kind);
@@ -509,7 +507,6 @@ int tode_solve_builtin_auto(const tode_solve_args *a, const tode_controller *c, 
         // (no evaluation points, or more than fit on chip: built for batches that leave SIMDs to spare)
         one_kernel = one_kernel && allow_one_kernel && ((E > 0 && E * elem <= 1024) || (B > 0 && B <= TODE_END_ONLY_MAX_BATCH));
     } else {
-        one_kernel = one_kernel && E > 0;
         if (a->term == TODE_TERM_REACTION_DIFFUSION)
             one_kernel = one_kernel && ((a->n_features == 16 * 16 || a->n_features == 32 * 32 || a->n_features == 64 * 64) ? E <= 8192
                                                                                                                            : (a->n_features == 128 * 128 && a->dtype == TODE_F32 && E <= 4096));

@@ -110,7 +110,8 @@ __device__ __forceinline__ void grid_rhs(GridShared<T, NW, R> &sh, int &buf, T D
 
 constexpr int grid_bands(int n) { return n * n / 4 > 1024 ? n * n / 4 / 1024 : 1; }
 
-template <typename T, int METHOD, int CTRL, int N>
+// END_ONLY: no evaluation points (a compile-time constant, so that the usual kernel carries none of that mode's code).
+template <typename T, int METHOD, int CTRL, int N, bool END_ONLY>
 __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(const SolveParams<T> p, const GridOut o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = N * N, R = grid_bands(N), NT = F / 4 / R, NW = NT / 64, BAND = F / R;
@@ -120,12 +121,15 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
 
     const int tid = threadIdx.x;
     const long long b = blockIdx.x;
-    const int E = p.n_eval;
+    // Without evaluation points (the end point alone, adjoints.py:296-311) t_end is the sample's one point: ys takes the
+    // dense output of its last step there and y_idle its final state; the caller picks per sample (tode_select_end_point).
+    constexpr bool end_only = END_ONLY;
+    const int E = end_only ? 1 : p.n_eval;
     const CtrlParams<T> &cp = p.cp;
     const T sf = (T)__builtin_sqrt((double)F);
     int buf = 0, slot = 0;
 
-    for (int e = tid; e < E; e += NT) te_s[e] = p.t_eval[b * E + e];
+    for (int e = tid; e < E; e += NT) te_s[e] = end_only ? p.t_end[b * p.te_stride] : p.t_eval[b * E + e];
     const T ts = p.t_start[b * p.ts_stride], te = p.t_end[b * p.te_stride];
     const T dir = (te > ts) ? (T)1 : (T)-1;
     const T tlo = tmin(ts, te), thi = tmax(te, ts);
@@ -193,7 +197,7 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
     // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's later
     // iterations with the clamped step t_end - t, which is seen only in the status of that step: the workgroup
     // computes that step once more and looks at its status.
-    bool idle = false;
+    bool idle = false, idle_done = false;
     while (!bail) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
@@ -241,6 +245,26 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
         const int status = limit_dt<T>(cp, ratio, dt_next);
         if (idle) {
             bail = status != 0;
+            if (end_only && !bail) {  // the end point of such a sample is this step's interpolant at t_end
+                const T x = unit_time(te, t0, t0 + dt);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    T out[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        T ks[7], q[5][1];
+#pragma unroll
+                        for (int s = 0; s < 7; ++s) ks[s] = k[s][r][j];
+                        quartic_elem<T, METHOD>(dt, y[r][j], y1[r][j], ks, true, q);
+                        T v = q[4][0];
+#pragma unroll
+                        for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[pw][0]);
+                        out[j] = v;
+                    }
+                    store4<T>(p.y_idle + b * F + r * BAND + 4 * tid, out);
+                }
+                idle_done = true;
+            }
             break;
         }
 
@@ -317,6 +341,10 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
         }
     }
 
+    if (end_only && !idle_done) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) store4<T>(p.y_idle + b * F + r * BAND + 4 * tid, y[r]);  // the final state
+    }
     if (tid == 0) {
         o.n_steps[b] = n_steps;
         o.n_accepted[b] = n_acc;
@@ -332,9 +360,12 @@ template <typename T, int METHOD, int CTRL, int N> static int launch_grid(const 
     SolveParams<T> p = make_params<T>(a, c);
     reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
-    const size_t lds = (size_t)a.n_eval * sizeof(T);
+    const size_t lds = (size_t)(a.n_eval > 0 ? a.n_eval : 1) * sizeof(T);
     timing_before(stream, "tode::solve_grid_kernel");
-    hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N>), dim3((unsigned)a.batch), dim3(N * N / 4 / grid_bands(N)), lds, stream, p, o);
+    if (a.n_eval > 0)
+        hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N, false>), dim3((unsigned)a.batch), dim3(N * N / 4 / grid_bands(N)), lds, stream, p, o);
+    else
+        hipLaunchKernelGGL((solve_grid_kernel<T, METHOD, CTRL, N, true>), dim3((unsigned)a.batch), dim3(N * N / 4 / grid_bands(N)), lds, stream, p, o);
     timing_after(stream);
     return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
 }

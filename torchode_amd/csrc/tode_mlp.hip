@@ -333,7 +333,8 @@ __device__ __forceinline__ void mlp_sum2(MlpShared &sh, int &slot, const float (
     slot ^= 1;
 }
 
-// FULL: all 64 state values are the problem's (the feature count is a constant and its tests fold away).
+// FULL: all 64 state values are the problem's and evaluation points are given (the feature count and the end-point mode are
+// constants and their tests fold away).
 template <int METHOD, int CTRL, typename Weights, bool FULL>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) solve_mlp_kernel(const SolveParams<float> p, const float *packed, const MlpOut o) {
     using T = float;
@@ -346,7 +347,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, q = lane >> 4, c = lane & 15;
     const long long b0 = (long long)blockIdx.x * MLP_TILE;
     const int rows = (int)min((long long)MLP_TILE, p.batch - b0);
-    const int E = p.n_eval;
+    // Without evaluation points (the end point alone, adjoints.py:296-311) t_end is every sample's one point: ys takes the
+    // dense output of the sample's last step there and y_idle its final state; the caller picks per sample
+    // (tode_select_end_point).
+    const bool end_only = !FULL && p.n_eval == 0;
+    const int E = end_only ? 1 : p.n_eval;
     const CtrlParams<T> &cp = p.cp;
     const int FR = FULL ? MLP_F : o.n_features;  // the problem's features; the kernel's others (FR .. 63) are zero in every vector
     const T sf = (T)__builtin_sqrt((double)FR);
@@ -368,7 +373,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     Weights W;
     mlp_load(W, packed, tid);
     for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns from 65 on
-    for (int i = tid; i < rows * E; i += 256) te_s[i] = p.t_eval[b0 * E + i];
+    for (int i = tid; i < rows * E; i += 256) te_s[i] = end_only ? p.t_end[(b0 + i) * p.te_stride] : p.t_eval[b0 * E + i];
     __syncthreads();
 
     // ---- state of the lane's sample ----
@@ -433,7 +438,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's later
     // iterations with the clamped step t_end - t, which is seen only in the status of that step: the sample sits
     // through one more iteration here, inactive, and the status of its step is looked at.
-    bool idle = false;
+    bool idle = false, idle_done = false;
     while (state == 1) {
         // ---- stages (runge_kutta.py:255-263) ----
         const T t0 = t;
@@ -473,6 +478,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
         const int status = limit_dt<T>(cp, ratio, dt_next);
         bail = bail || (idle && status != 0);
+        // (without evaluation points the end point of such a sample is this step's interpolant at t_end: below)
+        const bool idle_point = idle && end_only;
         idle = false;
         const bool move = accept && active;
         const T t_new = move ? (t0 + dt) : t0;
@@ -481,7 +488,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         n_acc += move ? 1 : 0;
 
         // ---- dense output at the evaluation points this step passed (adjoints.py:215-234) ----
-        if (active && cursor < E && fma_(dir, t_new, -dir * tev[cursor]) >= (T)0) {
+        if (idle_point || (active && cursor < E && fma_(dir, t_new, -dir * tev[cursor]) >= (T)0)) {
             T qc[4][5][1];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -494,13 +501,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             }
             const T t1 = t0 + dt;
             do {
-                const T x = unit_time(tev[cursor], t0, t1);
+                const T x = unit_time(idle_point ? te : tev[cursor], t0, t1);
                 T v[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     v[r] = qc[r][4][0];
 #pragma unroll
                     for (int pw = 3; pw >= 0; --pw) v[r] = fma_(v[r], x, qc[r][pw][0]);
+                }
+                if (idle_point) {
+                    put(p.y_idle + bs * FR, v);
+                    idle_done = true;
+                    break;
                 }
                 put(p.ys + (bs * E + cursor) * FR, v);
                 ++cursor;
@@ -533,6 +545,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         bail = (state & 2) != 0;
     }
 
+    if (end_only && live && !idle_done) put(p.y_idle + bs * FR, y);  // the final state
     if (w == 0 && q == 0) {
         if (live) {
             o.n_steps[bs] = n_steps;
@@ -550,10 +563,10 @@ template <int METHOD, int CTRL, typename Weights> static int launch_mlp(const to
     SolveParams<float> p = make_params<float>(a, c);
     reset_flags(a.flags, stream);
     if (a.batch == 0) return check_hip(hipGetLastError(), "tode_solve_builtin_fast launch");
-    const size_t lds = (size_t)MLP_TILE * a.n_eval * sizeof(float);
+    const size_t lds = (size_t)MLP_TILE * (a.n_eval > 0 ? a.n_eval : 1) * sizeof(float);
     const unsigned blocks = (unsigned)((a.batch + MLP_TILE - 1) / MLP_TILE);
     timing_before(stream, std::is_same<Weights, MlpWeightsBf16>::value ? "tode::solve_mlp_kernel (bfloat16 matrix inputs)" : "tode::solve_mlp_kernel");
-    if (o.n_features == MLP_F)
+    if (o.n_features == MLP_F && a.n_eval > 0)
         hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights, true>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
     else
         hipLaunchKernelGGL((solve_mlp_kernel<METHOD, CTRL, Weights, false>), dim3(blocks), dim3(256), lds, stream, p, (const float *)a.shared_params, o);
