@@ -177,10 +177,10 @@ def test_abi_argument_validation_without_a_gpu():
         setattr(a, name, _lib.C.addressof(dummy))
     assert lib.tode_solve_builtin(_lib.C.byref(a), _lib.C.byref(c), None) == -1  # strides left at zero
     assert b"stride" in lib.tode_last_error()
-    # n_eval == 0 through the fast entry point: the small systems only, and y_idle is needed
+    # n_eval == 0 through the fast entry point: y_idle is needed (every term takes that case; the next check is the flag block)
     a.term = _lib.TERM_MLP
-    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -2
-    assert b"small systems" in lib.tode_last_error()
+    assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -1
+    assert b"flags" in lib.tode_last_error()
     a.term, a.y_idle = 1, None
     assert lib.tode_solve_builtin_fast(_lib.C.byref(a), _lib.C.byref(c), None, None, None, None, None) == -1
     assert b"y_idle" in lib.tode_last_error()
