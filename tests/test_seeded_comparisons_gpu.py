@@ -2,7 +2,8 @@
 
 * time spans whose ends differ in sign and scale (samples that land one unit in the last place short of or past t_end,
   final states near the top of the dtype's range) through every whole-solve dispatch, against the C oracle: same bits;
-* the reaction-diffusion and MLP kernels against the protocol path (grid: same bits; MLP: the tolerance of its tests);
+* the reaction-diffusion and MLP kernels (grids of 16 to 128 cells a side, 3 to 64 state values, with and without
+  evaluation points) against the protocol path (grid: same bits; MLP: the tolerance of its tests);
 * time and data in different dtypes, general kernel against per-step kernels: same bits;
 * Heun and Euler, per-step kernels against the operator path: same bits;
 * the one-kernel reverse sweep (its record from the recording whole-solve kernel) against the sweep in torch operations.
@@ -107,7 +108,7 @@ def monotone_rows(problem):
     return (d >= 0).all(dim=1)
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(60))
 def test_grid_and_mlp_kernels_against_the_protocol_path(seed):
     from test_large_rows_gpu import narrow_mlp_problem
 
@@ -116,10 +117,10 @@ def test_grid_and_mlp_kernels_against_the_protocol_path(seed):
     ctrl, method = controller_spec(u, pick, F32), pick(["tsit5", "dopri5"])
     B, E = int(torch.randint(1, 40, (1,), generator=g)), int(torch.randint(1, 30, (1,), generator=g))
     if seed % 2 == 0:
-        n = pick([16, 32, 64])
+        n = pick([16, 32, 64, 128])
         f, y0, T1 = to.ReactionDiffusion(u32(0.001, pick([0.1, 1.0]), B).cuda(), n), u32(0, 1, B, n * n).cuda(), pick([0.5, 2.0, 8.0])
     else:
-        w = narrow_mlp_problem(pick([64, 64, 32, 8]), pick([256, 100, 17]), B, seed=seed)
+        w = narrow_mlp_problem(pick([64, 64, 32, 8, 3, 21]), pick([256, 100, 17]), B, seed=seed)
         f, y0, T1 = w.f, w.y0, pick([0.5, 1.0, 3.0])
     sign = torch.where((torch.rand(B, generator=g) < 0.3) & (T1 <= 1.0), -1.0, 1.0)
     t_start = u32(-1, 1, B) * pick([0.0, 1.0])
@@ -131,7 +132,9 @@ def test_grid_and_mlp_kernels_against_the_protocol_path(seed):
     if pick([True, False]):
         t_eval[:, -1] = t_end
     dt0 = pick([None, None, (u32(1e-3, 0.05, B) * sign).cuda()])
-    problem = to.InitialValueProblem(y0, t_start.cuda(), t_end.cuda(), t_eval.cuda())
+    if pick([False, False, False, True]):  # no evaluation points: the end point alone
+        t_eval, E = None, 1
+    problem = to.InitialValueProblem(y0, t_start.cuda(), t_end.cuda(), None if t_eval is None else t_eval.cuda())
     ours, other = {"tsit5": (to.Tsit5, OperatorTsit5), "dopri5": (to.Dopri5, OperatorDopri5)}[method]
     fused = to.AutoDiffAdjoint(ours(), make_controller(ctrl)).solve(problem, to.ODETerm(f), dt0=dt0)
     proto = to.AutoDiffAdjoint(other(), make_controller(ctrl)).solve(problem, to.ODETerm(f), dt0=dt0)
