@@ -784,3 +784,46 @@ def test_whole_sweep_kernel_when_every_sample_has_used_up_its_points(method, kin
         exact = (weights * -span * y0[:, None, :] * torch.exp(-k[:, None, :] * span)).sum(1)
         assert float(((results["whole"][1] - exact).abs() / exact.abs().amax(dim=1, keepdim=True)).max()) < 5e-3
 
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("name", ["mlp", "reaction_diffusion"])
+def test_gradients_with_the_grid_and_mlp_terms(name, dtype):
+    """A differentiable solve with one of the two long-row built-in terms (weights, diffusivities or y0 require grad):
+    their whole-solve kernels write no record of the loop, so the forward pass takes the per-step kernels around the
+    term's torch forward (it used to ask the general kernel, which does not know these terms, for the record).  The
+    reverse kernels against the sweep in torch operations, and the same term hidden behind a plain callable."""
+    import torchode_amd.autodiff as autodiff
+    import torchode_amd.builtin_terms as bt
+
+    g = torch.Generator().manual_seed(3)
+    r = lambda *shape: torch.rand(*shape, generator=g, dtype=torch.float64).to(dtype).cuda()
+    B, E = 6, 5
+    if name == "mlp":
+        F, H = 8, 16
+        leaves = [((r(H, F + 1) - 0.5) * 0.8).requires_grad_(), ((r(F, H) - 0.5) * 0.8).requires_grad_()]
+        b1, b2 = (r(H) - 0.5) * 0.1, (r(F) - 0.5) * 0.1
+        make = lambda: bt.MLPField(leaves[0], b1, leaves[1], b2)
+        y0 = (r(B, F) * 2 - 1).requires_grad_()
+    else:
+        leaves = [(r(B) * 0.3 + 0.01).requires_grad_()]
+        make = lambda: to.ReactionDiffusion(leaves[0], 16)
+        y0 = r(B, 256).requires_grad_()
+    t_eval = (r(B, 1) * 0.5 + 0.5) * torch.linspace(0, 1, E, dtype=dtype, device="cuda")[None, :]
+    weights = torch.linspace(0.5, 1.5, E * y0.shape[1], dtype=dtype, device="cuda").reshape(1, E, -1)
+    results = {}
+    for sweep in ("kernels", "torch", "callable"):
+        f = make()
+        solver = to.AutoDiffAdjoint(to.Dopri5(), to.IntegralController(1e-6, 1e-4))
+        solver.backward_kernels = sweep != "torch"
+        term = to.ODETerm((lambda t, y: f(t, y)) if sweep == "callable" else f)
+        sol = solver.solve(to.InitialValueProblem(y0, t_eval=t_eval), term)
+        assert sol.ys.requires_grad and (sol.status == 0).all()
+        results[sweep] = torch.autograd.grad((sol.ys * weights).sum(), [y0, *leaves])
+        assert autodiff.LAST_SWEEP == ("torch" if sweep == "torch" else "kernels")
+    rtol = 1e-9 if dtype == torch.float64 else 2e-2  # (float32 through the step size rule: the sweeps differ at the level of rounding amplified by it)
+    for other in ("torch", "callable"):
+        for got, want in zip(results["kernels"], results[other]):
+            torch.testing.assert_close(got, want, rtol=rtol, atol=rtol * float(want.abs().max()))
+    assert all(bool(x.isfinite().all()) and float(x.abs().max()) > 0 for x in results["kernels"])
+

@@ -550,6 +550,8 @@ class AutoDiffAdjoint(nn.Module):
         kernel once more, limited to the iterations the first pass took, with a record of that many entries)."""
         lib = _lib.load()
         f: BuiltinTerm = _sub(term, "f")
+        if record is not None and f.builtin_kind not in _lib.GENERAL_TERMS:
+            return None  # (the record is written for the three small systems: the grid and MLP terms record on the per-step path)
         method_id, controller = _sub(self, "step_method").method_id, _sub(self, "step_size_controller")
         # What depends on the problem's tensors alone is worked out once per problem object and kept on it (checked by
         # identity, since the attributes of a problem may be reassigned, and by the tensors' version counters, since
