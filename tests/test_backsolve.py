@@ -326,3 +326,41 @@ def test_forward_values_are_those_of_the_plain_solve_and_large_states_take_the_p
     ys.square().sum().backward()
     torch.testing.assert_close(y0.grad, y0_ref.grad, rtol=1e-6, atol=1e-7)
     torch.testing.assert_close(A.grad, A_ref.grad, rtol=1e-6, atol=1e-7)
+
+
+@gpu
+@pytest.mark.parametrize("name", ["mlp", "vdp"])
+def test_built_in_terms_keep_parameters_as_parameters(name):
+    """A built-in term built from ``nn.Parameter`` tensors holds them as parameters: optimizers find them, and the
+    backsolve adjoints, which differentiate with respect to ``term.parameters()`` (reference adjoints.py:497-539), give
+    about the gradient the loop's own reverse sweep gives (two discretisations of the same derivative).  (The MLP, whose
+    weights the whole batch shares, through ``BacksolveAdjoint``, which calls ``f`` one sample at a time; a term with a
+    parameter per sample through ``JointBacksolveAdjoint``, which calls it on the batch.)"""
+    import torchode_amd.builtin_terms as bt
+
+    torch.manual_seed(0)
+    dtype, B = torch.float64, 12
+    if name == "mlp":
+        F, H = 6, 16
+        leaves = [nn.Parameter(((torch.rand(H, F + 1, dtype=dtype) - 0.5) * 0.8).cuda()), nn.Parameter(((torch.rand(F, H, dtype=dtype) - 0.5) * 0.8).cuda())]
+        f = bt.MLPField(leaves[0], torch.zeros(H, dtype=dtype, device="cuda"), leaves[1], torch.zeros(F, dtype=dtype, device="cuda"))
+        y0 = (torch.rand(B, F, dtype=dtype) * 2 - 1).cuda()
+    else:
+        leaves = [nn.Parameter((0.5 + torch.rand(B, dtype=dtype)).cuda())]
+        f = to.VanDerPol(leaves[0])
+        y0 = (torch.rand(B, 2, dtype=dtype) * 2 - 1).cuda()
+    assert [p is q for p, q in zip(f.parameters(), leaves)] == [True] * len(leaves)
+    t_eval = torch.linspace(0, 1.0, 4, dtype=dtype, device="cuda").expand(B, 4).contiguous()
+    problem = to.InitialValueProblem(y0, t_eval=t_eval)
+    term = to.ODETerm(f)
+    make = lambda: (to.Dopri5(), to.IntegralController(1e-9, 1e-7))
+    grads = {}
+    for kind in ("backsolve", "autodiff"):
+        backsolve = to.BacksolveAdjoint if name == "mlp" else to.JointBacksolveAdjoint
+        solver = backsolve(term, *make()) if kind == "backsolve" else to.AutoDiffAdjoint(*make())
+        sol = solver.solve(problem) if kind == "backsolve" else solver.solve(problem, term)
+        grads[kind] = torch.autograd.grad(sol.ys[:, -1].square().sum(), leaves)
+    for a, b in zip(grads["backsolve"], grads["autodiff"]):
+        assert float(b.abs().max()) > 0
+        torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-5 * float(b.abs().max()))
+

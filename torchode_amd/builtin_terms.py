@@ -26,6 +26,14 @@ class BuiltinTerm(nn.Module):
         """Per-sample parameters as a contiguous ``[B, P]`` tensor in the data dtype."""
         raise NotImplementedError
 
+    def hold(self, name: str, tensor: torch.Tensor) -> None:
+        """Keeps a tensor of the term: an ``nn.Parameter`` as a parameter (so that optimizers and the backsolve adjoints,
+        which differentiate with respect to ``term.parameters()``, find it), any other tensor as a buffer."""
+        if isinstance(tensor, nn.Parameter):
+            self.register_parameter(name, tensor)
+        else:
+            self.register_buffer(name, tensor)
+
 
 class LinearDecay(BuiltinTerm):
     """``dy/dt = (-k) * y`` with one rate per sample and feature, ``k`` of shape ``[B, F]``."""
@@ -35,7 +43,7 @@ class LinearDecay(BuiltinTerm):
     def __init__(self, k: torch.Tensor):
         super().__init__()
         assert k.ndim == 2
-        self.register_buffer("k", k)
+        self.hold("k", k)
         self.n_features = k.shape[1]
 
     def forward(self, t, y):
@@ -54,7 +62,7 @@ class VanDerPol(BuiltinTerm):
     def __init__(self, mu: torch.Tensor):
         super().__init__()
         assert mu.ndim == 1
-        self.register_buffer("mu", mu)
+        self.hold("mu", mu)
 
     def forward(self, t, y):
         x, v = y[:, 0], y[:, 1]
@@ -83,7 +91,7 @@ class Lorenz63(BuiltinTerm):
     def __init__(self, rho: torch.Tensor, sigma: float = 10.0, beta: float = 8.0 / 3.0):
         super().__init__()
         assert rho.ndim == 1
-        self.register_buffer("rho", rho)
+        self.hold("rho", rho)
         self.sigma = float(sigma)
         self.beta = float(beta)
 
@@ -112,7 +120,7 @@ class ReactionDiffusion(BuiltinTerm):
     def __init__(self, D: torch.Tensor, n: int = 64):
         super().__init__()
         assert D.ndim == 1
-        self.register_buffer("D", D)
+        self.hold("D", D)
         self.n = int(n)
         self.n_features = self.n * self.n
 
@@ -140,12 +148,12 @@ class MLPField(BuiltinTerm):
         assert W1.ndim == 2 and W2.ndim == 2 and W1.shape[0] == W2.shape[1] and W1.shape[1] == W2.shape[0] + 1
         assert matrix_inputs in ("float32", "bfloat16")
         for name, w in (("W1", W1), ("b1", b1), ("W2", W2), ("b2", b2)):
-            self.register_buffer(name, w)
+            self.hold(name, w)
         self.n_features = W2.shape[0]
         self.matrix_inputs = matrix_inputs
 
     def forward(self, t, y):
-        x = torch.cat([y, t[:, None]], 1)
+        x = torch.cat([y, t[..., None]], -1)  # (also one sample at a time, as the backsolve adjoint's vmap calls it)
         if self.matrix_inputs == "bfloat16":
             rounded = lambda z: z.to(torch.bfloat16).to(z.dtype)
             h = torch.tanh(rounded(x) @ rounded(self.W1).T + self.b1)
