@@ -565,17 +565,21 @@ def test_reverse_kernels_on_long_rows(features, case):
 
 
 @gpu
-def test_what_is_not_differentiated_says_so():
+def test_a_users_subclass_is_differentiated_on_the_operator_path():
+    """(more in tests/test_protocol_autograd_gpu.py)"""
     y0, A = inputs()
     term = to.ODETerm(LinearDynamics(A))
-    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda", requires_grad=True)
+    t_eval = torch.tensor(T_EVAL, dtype=torch.double, device="cuda")
+
     class OwnHeun(to.Heun):  # a user's subclass: its protocol methods may do anything
         pass
 
-    with pytest.raises(RuntimeError, match="BacksolveAdjoint"):
-        to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
-    with torch.no_grad():  # no graph asked for: any configuration solves
-        to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval.detach()), term=term)
+    solution = to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
+    solution.ys.sum().backward()
+    assert torch.isfinite(y0.grad).all() and torch.isfinite(A.grad).all() and A.grad.abs().max() > 0
+    with torch.no_grad():  # no graph asked for: same values
+        plain = to.AutoDiffAdjoint(OwnHeun(), to.IntegralController(1e-6, 1e-6)).solve(to.InitialValueProblem(y0, t_eval=t_eval), term=term)
+    assert torch.equal(plain.ys, solution.ys.detach())
 
 
 # ---------------------------------------------------------------------------------------------

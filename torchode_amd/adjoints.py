@@ -1,10 +1,11 @@
 """The solve driver (mirrors torchode/adjoints.py:26-319)."""
+from functools import partial
 from typing import Any, Dict, Optional
 
 import torch
 import torch.nn as nn
 
-from . import _lib
+from . import _lib, differentiable
 from .builtin_terms import BuiltinTerm
 from .problems import InitialValueProblem
 from .interpolation import _PolynomialInterpolation
@@ -218,17 +219,15 @@ class AutoDiffAdjoint(nn.Module):
             sol = self._solve_persistent(problem, term_, dt0)
             if sol is not None:
                 return sol
-        if wants_grad:
-            # gradients through the loop: forward in the per-step kernels (Dopri5, Tsit5) or on the operator
-            # path (Heun, Euler) with a record of the loop state, backward by a reverse sweep over the record
-            if not self._library_setup(problem, term_, (Dopri5, Tsit5, Heun, Euler)):
-                raise RuntimeError(
-                    "gradients through the loop are built for the library's step methods and controllers; "
-                    "with user-defined plug-ins call solve under torch.no_grad(), or use BacksolveAdjoint"
-                )
+        if wants_grad and self._library_setup(problem, term_, (Dopri5, Tsit5, Heun, Euler)):
+            # gradients through the loop with the library's own plug-ins: forward in the per-step kernels (Dopri5,
+            # Tsit5) or on the operator path (Heun, Euler) with a record of the loop state, backward by a reverse
+            # sweep over the record
             from . import autodiff
 
             return autodiff.solve(self, problem, term_, dt0, args)
+        # (with a user-defined plug-in a solve that wants gradients takes the operator path below like any other:
+        # its kernels' results carry graph nodes wherever an input requires grad, torchode_amd/differentiable.py)
         if self._stepwise_ok(problem, term_):
             return self._solve_stepwise(problem, term_, dt0, args)
         return self._solve_protocol(problem, term, term_, dt0, args)
@@ -291,12 +290,26 @@ class AutoDiffAdjoint(nn.Module):
 
         ys = new(B, max(E, 1), F)
         pending = new(B, E, dt=torch.uint8) if E > 0 else None
-        dt_in, dt = as_float(dt, (B,), ttype), new(B, dt=ttype)
-        rc = lib.tode_loop_begin(
-            code, B, F, E, _lib.ptr(t_start), _lib.ptr(t_end), _lib.ptr(t_eval), _lib.ptr(y), _lib.ptr(dt_in), _lib.ptr(dt),
-            _lib.ptr(pending), _lib.ptr(ys), stream,
-        )  # fmt: skip
-        _lib.check(rc, "tode_loop_begin")
+        dt_in = as_float(dt, (B,), ttype)
+
+        def begin_kernel():
+            dt = new(B, dt=ttype)
+            rc = lib.tode_loop_begin(
+                code, B, F, E, _lib.ptr(t_start), _lib.ptr(t_end), _lib.ptr(t_eval), _lib.ptr(y), _lib.ptr(dt_in), _lib.ptr(dt),
+                _lib.ptr(pending), _lib.ptr(ys), stream,
+            )  # fmt: skip
+            _lib.check(rc, "tode_loop_begin")
+            return dt
+
+        # Where an input requires grad, every kernel's result carries a graph node that differentiates the same
+        # operation written as torch operations (differentiable.through), so the solve is differentiable for any mix of
+        # the library's and a user's plug-ins, as the reference's loop of torch operations is (adjoints.py:135-260).
+        dt = differentiable.through(begin_kernel, differentiable.loop_begin, t_start, t_end, dt_in)
+        if E > 0 and differentiable.tracked(y):
+            at_start = (t_eval[:, 0] == t_start).nonzero()[:, 0]
+            ys[at_start, 0] = y[at_start]  # (the kernel wrote the same values; this write is the one autograd sees)
+        if not self.backprop_through_step_size_control:
+            dt = dt.detach()
 
         running = torch.ones(B, dtype=torch.bool, device=dev)
         n_steps = torch.zeros(B, dtype=torch.long, device=dev)
@@ -322,23 +335,33 @@ class AutoDiffAdjoint(nn.Module):
                 t, dt, y, step_result, controller_state, stats
             )
 
+            if not self.backprop_through_step_size_control:
+                dt_next = dt_next.detach() if isinstance(dt_next, torch.Tensor) else dt_next
+
             # ---- one kernel: state update, counters, running, status, evaluation mask, next dt ----
             y_new = as_float(step_result.y, (B, F))
             accept_ = torch.as_tensor(accept, device=dev).to(torch.bool).expand((B,)).contiguous()
             dt_next_ = as_float(dt_next, (B,), ttype)
             m_status, c_status = as_status(method_status), as_status(controller_status)
-            t_out, dt_out, y_out = new(B, dt=ttype), new(B, dt=ttype), new(B, F)
             running_out, to_update = new(B, dt=torch.bool), new(B, dt=torch.bool)
             status = new(B, dt=torch.long)
             to_evaluate = new(B, E, dt=torch.uint8) if E > 0 else None
-            a.t, a.dt, a.y, a.running = t.data_ptr(), dt.data_ptr(), y.data_ptr(), running.data_ptr()
-            a.y_new, a.accept, a.dt_next = y_new.data_ptr(), accept_.data_ptr(), dt_next_.data_ptr()
-            a.method_status = None if m_status is None else m_status.data_ptr()
-            a.controller_status = None if c_status is None else c_status.data_ptr()
-            a.t_out, a.dt_out, a.y_out = t_out.data_ptr(), dt_out.data_ptr(), y_out.data_ptr()
-            a.running_out, a.to_update, a.status = running_out.data_ptr(), to_update.data_ptr(), status.data_ptr()
-            a.to_evaluate = None if to_evaluate is None else to_evaluate.data_ptr()
-            _lib.check(lib.tode_loop_advance(_lib.C.byref(a), stream), "tode_loop_advance")
+
+            def advance_kernel(t=t, dt=dt, y=y, y_new=y_new, dt_next_=dt_next_):
+                t_out, dt_out, y_out = new(B, dt=ttype), new(B, dt=ttype), new(B, F)
+                a.t, a.dt, a.y, a.running = t.data_ptr(), dt.data_ptr(), y.data_ptr(), running.data_ptr()
+                a.y_new, a.accept, a.dt_next = y_new.data_ptr(), accept_.data_ptr(), dt_next_.data_ptr()
+                a.method_status = None if m_status is None else m_status.data_ptr()
+                a.controller_status = None if c_status is None else c_status.data_ptr()
+                a.t_out, a.dt_out, a.y_out = t_out.data_ptr(), dt_out.data_ptr(), y_out.data_ptr()
+                a.running_out, a.to_update, a.status = running_out.data_ptr(), to_update.data_ptr(), status.data_ptr()
+                a.to_evaluate = None if to_evaluate is None else to_evaluate.data_ptr()
+                _lib.check(lib.tode_loop_advance(_lib.C.byref(a), stream), "tode_loop_advance")
+                return t_out, dt_out, y_out
+
+            t_out, dt_out, y_out = differentiable.through(
+                advance_kernel, partial(differentiable.loop_advance, to_update, running_out), t_start, t_end, t, dt, y, y_new, dt_next_
+            )
             fl = flags.tolist()  # the iteration's host synchronisation
 
             method_state = method.merge_states(to_update, method_state_next, method_state)
@@ -346,7 +369,8 @@ class AutoDiffAdjoint(nn.Module):
             # ---- dense output at the evaluation points this step passed ----
             if E > 0 and fl[_lib.LOOP_N_TO_EVALUATE] > 0:
                 interpolation = method.build_interpolation(interp_data)
-                if isinstance(interpolation, _PolynomialInterpolation) and type(interpolation).evaluate is _PolynomialInterpolation.evaluate:
+                own = isinstance(interpolation, _PolynomialInterpolation) and type(interpolation).evaluate is _PolynomialInterpolation.evaluate
+                if own and not interpolation.tracked(t_eval):
                     interpolation.evaluate_masked(t_eval, to_evaluate, ys)
                 else:
                     hit = to_evaluate.view(torch.bool).nonzero()

@@ -9,7 +9,7 @@ from typing import Sequence, Union
 
 import torch
 
-from . import _lib
+from . import _lib, differentiable
 
 
 def _poly_eval_rows(coefficients, t, t0, t1):
@@ -68,20 +68,29 @@ class _PolynomialInterpolation(LocalInterpolation):
         assert all(t.dtype == self.t0.dtype for t in (self.t1, *times)), "time tensors of different dtypes"
         return _lib.dtype_code(c.dtype, self.t0.dtype)
 
+    def tracked(self, *times) -> bool:
+        """True if values of this polynomial have to carry a graph (then ``evaluate`` is the way to them)."""
+        return differentiable.tracked(self._coeff, self.t0, self._span(), *times)
+
     def evaluate(self, t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
         """reference interpolation.py:103-106, 172-175"""
         code = self._code(t)
-        c = self._coeff
-        _, B, F = c.shape
-        t, idx = t.contiguous(), idx.to(torch.long).contiguous()
-        t0, t1 = self.t0.contiguous(), self._span().contiguous()
-        out = c.new_empty((t.shape[0], F))
-        rc = _lib.load().tode_poly_eval(
-            code, self.degree, self.span_is_dt, B, F, t.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t),
-            _lib.ptr(idx), _lib.ptr(out), _lib.stream_of(c),
-        )  # fmt: skip
-        _lib.check(rc, "tode_poly_eval")
-        return out
+        idx = idx.to(torch.long).contiguous()
+
+        def kernel():
+            c = self._coeff
+            _, B, F = c.shape
+            t_, t0, t1 = t.contiguous(), self.t0.contiguous(), self._span().contiguous()
+            out = c.new_empty((t_.shape[0], F))
+            rc = _lib.load().tode_poly_eval(
+                code, self.degree, self.span_is_dt, B, F, t_.shape[0], _lib.ptr(c), _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(t_),
+                _lib.ptr(idx), _lib.ptr(out), _lib.stream_of(c),
+            )  # fmt: skip
+            _lib.check(rc, "tode_poly_eval")
+            return out
+
+        formula = lambda c, t0, t1, t_: differentiable.poly_eval(bool(self.span_is_dt), idx, c, t0, t1, t_)
+        return differentiable.through(kernel, formula, self._coeff, self.t0, self._span(), t)
 
     def evaluate_masked(self, t_eval: torch.Tensor, mask: torch.Tensor, ys: torch.Tensor) -> None:
         """``ys[b, e] = p_b(t_eval[b, e])`` wherever ``mask[b, e]`` is set (one byte per entry);
@@ -133,14 +142,20 @@ class ThirdOrderPolynomialInterpolation(_PolynomialInterpolation):
     @staticmethod
     def from_k(t0, dt, y0, y1, k):
         """Hermite cubic from the first and last stage derivative (reference interpolation.py:84-106)."""
-        code, dt_, y0_, y1_, kf, kl = _build_args(dt, y0, y1, k[0], k[-1])
-        B, F = y0_.shape
-        coeff = y0_.new_empty((4, B, F))
-        rc = _lib.load().tode_cubic_build(
-            code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl),
-            _lib.ptr(coeff), _lib.stream_of(y0_),
-        )  # fmt: skip
-        _lib.check(rc, "tode_cubic_build")
+        k_first, k_last = k[0], k[-1]
+
+        def kernel():
+            code, dt_, y0_, y1_, kf, kl = _build_args(dt, y0, y1, k_first, k_last)
+            B, F = y0_.shape
+            coeff = y0_.new_empty((4, B, F))
+            rc = _lib.load().tode_cubic_build(
+                code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl),
+                _lib.ptr(coeff), _lib.stream_of(y0_),
+            )  # fmt: skip
+            _lib.check(rc, "tode_cubic_build")
+            return coeff
+
+        coeff = differentiable.through(kernel, differentiable.cubic_build, dt, y0, y1, k_first, k_last)
         return ThirdOrderPolynomialInterpolation(t0, t0 + dt, coeff)
 
 
@@ -153,33 +168,57 @@ class FourthOrderPolynomialInterpolation(_PolynomialInterpolation):
     def from_k(t0, dt, y0, y1, k, b_mid):
         """Quartic through both end points, their derivatives and the mid-point value
         ``y0 + dt * sum_s b_mid[s] k[s]`` (reference interpolation.py:138-170)."""
-        code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
-        S, B, F = k_.shape
-        lib, stream = _lib.load(), _lib.stream_of(y0_)
         w = [float(x) for x in (b_mid.tolist() if isinstance(b_mid, torch.Tensor) else b_mid)]
-        assert len(w) == S <= _lib.MAX_STAGES
-        y_mid = torch.empty_like(y0_)
-        rc = lib.tode_erk_combine(code, B, F, S, (_lib.C.c_double * S)(*w), _lib.ptr(dt_), _lib.ptr(k_), _lib.ptr(y0_), _lib.ptr(y_mid), stream)
-        _lib.check(rc, "tode_erk_combine")
-        coeff = y0_.new_empty((5, B, F))
-        rc = lib.tode_quartic_from_mid(
-            code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_[0]), _lib.ptr(k_[-1]), _lib.ptr(y_mid),
-            _lib.ptr(coeff), stream,
-        )  # fmt: skip
-        _lib.check(rc, "tode_quartic_from_mid")
+        assert len(w) == k.shape[0] <= _lib.MAX_STAGES
+
+        def mid_kernel():
+            code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+            S, B, F = k_.shape
+            y_mid = torch.empty_like(y0_)
+            rc = _lib.load().tode_erk_combine(code, B, F, S, (_lib.C.c_double * S)(*w), _lib.ptr(dt_), _lib.ptr(k_), _lib.ptr(y0_), _lib.ptr(y_mid), _lib.stream_of(y0_))
+            _lib.check(rc, "tode_erk_combine")
+            return y_mid
+
+        y_mid = differentiable.through(mid_kernel, lambda dt_, y0_, k_: differentiable.combine(w, dt_, y0_, *k_.unbind(0)), dt, y0, k)
+        k_first, k_last = k[0], k[-1]
+
+        def kernel():
+            code, dt_, y0_, y1_, kf, kl, mid = _build_args(dt, y0, y1, k_first, k_last, y_mid)
+            B, F = y0_.shape
+            coeff = y0_.new_empty((5, B, F))
+            rc = _lib.load().tode_quartic_from_mid(
+                code, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(kf), _lib.ptr(kl), _lib.ptr(mid),
+                _lib.ptr(coeff), _lib.stream_of(y0_),
+            )  # fmt: skip
+            _lib.check(rc, "tode_quartic_from_mid")
+            return coeff
+
+        coeff = differentiable.through(kernel, differentiable.quartic_from_mid, dt, y0, y1, k_first, k_last, y_mid)
         return FourthOrderPolynomialInterpolation(t0, t0 + dt, coeff)
 
     @staticmethod
     def from_erk_step(method_id: int, t0, dt, y0, y1, k):
         """Dense output of a Dopri5 / Tsit5 step with the pair's own weights, one kernel
         (reference tsit5.py:123-139, dopri5.py:53-60)."""
-        code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
-        S, B, F = k_.shape
-        assert S == 7
-        coeff = y0_.new_empty((5, B, F))
-        rc = _lib.load().tode_quartic_build(
-            code, method_id, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_), _lib.ptr(coeff),
-            _lib.stream_of(y0_),
-        )  # fmt: skip
-        _lib.check(rc, "tode_quartic_build")
+        assert k.shape[0] == 7
+
+        def kernel():
+            code, dt_, y0_, y1_, k_ = _build_args(dt, y0, y1, k)
+            S, B, F = k_.shape
+            coeff = y0_.new_empty((5, B, F))
+            rc = _lib.load().tode_quartic_build(
+                code, method_id, B, F, _lib.ptr(dt_), _lib.ptr(y0_), _lib.ptr(y1_), _lib.ptr(k_), _lib.ptr(coeff),
+                _lib.stream_of(y0_),
+            )  # fmt: skip
+            _lib.check(rc, "tode_quartic_build")
+            return coeff
+
+        def formula(dt_, y0_, y1_, k_):
+            from .single_step_methods.runge_kutta import library_tableau
+
+            rows = library_tableau(method_id).b_other.tolist()  # Dopri5: the mid-point weights; Tsit5: theta^2 .. theta^4
+            mid, theta = (rows[0], None) if len(rows) == 1 else (None, rows)
+            return differentiable.quartic_build(mid, theta, dt_, y0_, y1_, *k_.unbind(0))
+
+        coeff = differentiable.through(kernel, formula, dt, y0, y1, k)
         return FourthOrderPolynomialInterpolation(t0, t0 + dt, coeff)

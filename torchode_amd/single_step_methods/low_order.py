@@ -5,7 +5,7 @@ from typing import Any, Dict, NamedTuple, Optional
 
 import torch
 
-from .. import _lib
+from .. import _lib, differentiable
 from ..interpolation import LinearInterpolation, ThirdOrderPolynomialInterpolation
 from ..terms import ODETerm
 from .base import SingleStepMethod, StepResult
@@ -39,13 +39,18 @@ class Euler(SingleStepMethod):
         y0, dt = y0.contiguous(), dt.contiguous()
         B, F = y0.shape
         k = term_.vf(t0, y0, stats, args).to(y0.dtype).contiguous()
-        y1 = torch.empty_like(y0)
-        one = (_lib.C.c_double * 1)(1.0)
-        rc = _lib.load().tode_erk_stage(
-            _lib.dtype_code(y0.dtype, dt.dtype), B, F, 1, one, 0.0, None, _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(k), _lib.ptr(y1), None,
-            _lib.stream_of(y0),
-        )  # fmt: skip
-        _lib.check(rc, "tode_erk_stage")
+
+        def kernel():
+            y1 = torch.empty_like(y0)
+            one = (_lib.C.c_double * 1)(1.0)
+            rc = _lib.load().tode_erk_stage(
+                _lib.dtype_code(y0.dtype, dt.dtype), B, F, 1, one, 0.0, None, _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(k), _lib.ptr(y1), None,
+                _lib.stream_of(y0),
+            )  # fmt: skip
+            _lib.check(rc, "tode_erk_stage")
+            return y1
+
+        y1 = differentiable.through(kernel, lambda dt_, y0_, k_: differentiable.stage([1.0], 0.0, None, dt_, y0_, k_), dt, y0, k)
         return StepResult(y1, None), LinearInterpolationData(t0, dt, y0, y1), state, None
 
     def merge_states(self, accept, current, previous):

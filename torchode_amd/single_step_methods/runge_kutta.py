@@ -3,11 +3,12 @@
 The stage inputs, the weighted stage sums and the FSAL merge run as HIP kernels;
 the right-hand side is the caller's torch callable, evaluated between them.
 """
+from functools import partial
 from typing import Any, Dict, List, NamedTuple, Optional
 
 import torch
 
-from .. import _lib
+from .. import _lib, differentiable
 from ..problems import InitialValueProblem
 from ..terms import ODETerm
 from .base import SingleStepMethod, StepResult
@@ -152,13 +153,17 @@ class ExplicitRungeKutta(SingleStepMethod):
         if cur is None or prev is None:
             return current
         _lib.require_device(accept, cur, prev)
-        cur, prev, mask = cur.contiguous(), prev.contiguous(), accept.contiguous()
-        assert mask.element_size() == 1 and cur.dtype == prev.dtype and cur.dtype in _lib.DTYPES
-        out = torch.empty_like(cur)
-        B, F = cur.shape
-        rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], B, F, _lib.ptr(mask), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
-        _lib.check(rc, "tode_select_rows")
-        return ERKState(current.tableau, out)
+        assert accept.element_size() == 1 and cur.dtype == prev.dtype and cur.dtype in _lib.DTYPES
+
+        def kernel():
+            a, b, mask = cur.contiguous(), prev.contiguous(), accept.contiguous()
+            out = torch.empty_like(a)
+            B, F = a.shape
+            rc = _lib.load().tode_select_rows(_lib.DTYPES[a.dtype], B, F, _lib.ptr(mask), _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.stream_of(a))
+            _lib.check(rc, "tode_select_rows")
+            return out
+
+        return ERKState(current.tableau, differentiable.through(kernel, lambda a, b: differentiable.select_rows(accept, a, b), cur, prev))
 
     def step(self, term, running, y0, t0, dt, state: ERKState, *, stats, args):
         term_ = term if term is not None else self.term
@@ -173,26 +178,45 @@ class ExplicitRungeKutta(SingleStepMethod):
         lib, code, stream = _lib.load(), _lib.dtype_code(y0.dtype, t0.dtype), _lib.stream_of(y0)
 
         vf0 = state.prev_vf1 if tab.fsal and state.prev_vf1 is not None else term_.vf(t0, y0, stats, args)
+        # the slopes: one [S, B, F] array for the kernels; beside it, where gradients are wanted, the tensors as f
+        # returned them (the array is filled in place, which autograd could follow only by copying it per stage)
         k = y0.new_empty((S, B, F))
-        k[0].copy_(vf0)
+        vf0 = vf0 if vf0.dtype == y0.dtype else vf0.to(y0.dtype)
+        k[0].copy_(vf0.detach())
+        ks = [vf0]
         y_i = y0
         for i in range(1, S):
-            y_i, t_i = torch.empty_like(y0), torch.empty_like(t0)
-            rc = lib.tode_erk_stage(code, B, F, i, h.a_rows[i], h.c[i], _lib.ptr(t0), _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(k), _lib.ptr(y_i), _lib.ptr(t_i), stream)
-            _lib.check(rc, "tode_erk_stage")
-            k[i].copy_(term_.vf(t_i, y_i, stats, args))
+
+            def stage_kernel(i=i):
+                y_i, t_i = torch.empty_like(y0), torch.empty_like(t0)
+                rc = lib.tode_erk_stage(code, B, F, i, h.a_rows[i], h.c[i], _lib.ptr(t0), _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(k), _lib.ptr(y_i), _lib.ptr(t_i), stream)
+                _lib.check(rc, "tode_erk_stage")
+                return y_i, t_i
+
+            y_i, t_i = differentiable.through(stage_kernel, partial(differentiable.stage, list(h.a_rows[i])[:i], h.c[i]), t0, dt, y0, *ks)
+            k_i = term_.vf(t_i, y_i, stats, args)
+            k_i = k_i if k_i.dtype == y0.dtype else k_i.to(y0.dtype)
+            k[i].copy_(k_i.detach())
+            ks.append(k_i)
+
+        def combine_kernel(weights, base):
+            out = torch.empty_like(y0)
+            _lib.check(lib.tode_erk_combine(code, B, F, S, weights, _lib.ptr(dt), _lib.ptr(k), _lib.ptr(base), _lib.ptr(out), stream), "tode_erk_combine")
+            return out
 
         if tab.ssal:
             y1 = y_i
         else:
-            y1 = torch.empty_like(y0)
-            _lib.check(lib.tode_erk_combine(code, B, F, S, h.b, _lib.ptr(dt), _lib.ptr(k), _lib.ptr(y0), _lib.ptr(y1), stream), "tode_erk_combine")
-        err = torch.empty_like(y0)
-        _lib.check(lib.tode_erk_combine(code, B, F, S, h.b_err, _lib.ptr(dt), _lib.ptr(k), None, _lib.ptr(err), stream), "tode_erk_combine")
+            y1 = differentiable.through(partial(combine_kernel, h.b, y0), partial(differentiable.combine, list(h.b)), dt, y0, *ks)
+        err = differentiable.through(
+            partial(combine_kernel, h.b_err, None), lambda dt_, *ks_: differentiable.combine(list(h.b_err), dt_, None, *ks_), dt, *ks
+        )
 
+        tracked = differentiable.tracked(*ks)
+        slopes = torch.stack(ks) if tracked else k  # (same values; a graph back to every evaluation of f)
         if tab.fsal:
-            state = ERKState(tab, k[-1])
-        return StepResult(y1, err), ERKInterpolationData(tab, t0, dt, y0, y1, k), state, None
+            state = ERKState(tab, ks[-1] if tracked else k[-1])
+        return StepResult(y1, err), ERKInterpolationData(tab, t0, dt, y0, y1, slopes), state, None
 
     def build_interpolation(self, data: ERKInterpolationData):
         raise NotImplementedError()

@@ -6,13 +6,14 @@ kernels: inside the whole-solve kernel when ``AutoDiffAdjoint`` recognises the w
 configuration, and one kernel per protocol call otherwise.  A user-defined controller
 subclasses ``StepSizeController``.
 """
+from functools import partial
 from math import sqrt
 from typing import Any, Callable, Dict, NamedTuple, Optional, Tuple
 
 import torch
 import torch.nn as nn
 
-from . import _lib
+from . import _lib, differentiable
 from .problems import InitialValueProblem
 from .terms import ODETerm
 
@@ -193,34 +194,50 @@ class AdaptiveStepSizeController(StepSizeController):
         _lib.require_device(dt, norm, y0, y1, err)
         data_dtype = data_dtype if y0 is None else y0.dtype
         code = _lib.dtype_code(data_dtype, dt.dtype)
-        dt = dt.contiguous()
         B = dt.shape[0]
         pid = self._kind == _lib.CTRL_PID
-        prev = state.prev_error_ratio.to(data_dtype).contiguous() if pid else None
-        pprev = state.prev_prev_error_ratio.to(data_dtype).contiguous() if pid else None
-        accept = torch.empty(B, dtype=torch.bool, device=dt.device)
-        dt_next, ratio = torch.empty_like(dt), torch.empty(B, dtype=data_dtype, device=dt.device)
-        status = torch.empty(B, dtype=torch.long, device=dt.device)
-        prev_o = torch.empty_like(ratio) if pid else None
-        pprev_o = torch.empty_like(ratio) if pid else None
+        prev = state.prev_error_ratio.to(data_dtype) if pid else None
+        pprev = state.prev_prev_error_ratio.to(data_dtype) if pid else None
         # the limits in force are the state's (reference step_size_controllers.py:406-408)
         c = self.c_struct((_limit(state.dt_min), _limit(state.dt_max)) if limits else (None, None))
-        lib, stream = _lib.load(), _lib.stream_of(dt)
-        tail = (_lib.ptr(prev), _lib.ptr(pprev), _lib.ptr(accept), _lib.ptr(dt_next), _lib.ptr(ratio), _lib.ptr(status),
-                _lib.ptr(prev_o), _lib.ptr(pprev_o), stream)  # fmt: skip
-        if norm is None:
-            y0, y1, err = (x.contiguous() for x in (y0, y1, err))
-            assert y1.dtype == y0.dtype == err.dtype and y0.shape == y1.shape == err.shape
-            rc = lib.tode_adapt_step(
-                code, _lib.C.byref(c), int(state.method_order), self._norm_id(), B, y0.shape[1],
-                _lib.ptr(dt), _lib.ptr(y0), _lib.ptr(y1), _lib.ptr(err), *tail,
+        order = int(state.method_order)
+        decided = {}
+
+        def kernel():
+            dt_ = dt.contiguous()
+            accept = torch.empty(B, dtype=torch.bool, device=dt.device)
+            dt_next, ratio = torch.empty_like(dt_), torch.empty(B, dtype=data_dtype, device=dt.device)
+            status = torch.empty(B, dtype=torch.long, device=dt.device)
+            prev_, pprev_ = (prev.contiguous(), pprev.contiguous()) if pid else (None, None)
+            prev_o = torch.empty_like(ratio) if pid else None
+            pprev_o = torch.empty_like(ratio) if pid else None
+            lib, stream = _lib.load(), _lib.stream_of(dt)
+            tail = (_lib.ptr(prev_), _lib.ptr(pprev_), _lib.ptr(accept), _lib.ptr(dt_next), _lib.ptr(ratio), _lib.ptr(status),
+                    _lib.ptr(prev_o), _lib.ptr(pprev_o), stream)  # fmt: skip
+            if norm is None:
+                a, b, e = (x.contiguous() for x in (y0, y1, err))
+                assert b.dtype == a.dtype == e.dtype and a.shape == b.shape == e.shape
+                rc = lib.tode_adapt_step(code, _lib.C.byref(c), order, self._norm_id(), B, a.shape[1], _lib.ptr(dt_), _lib.ptr(a), _lib.ptr(b), _lib.ptr(e), *tail)
+                _lib.check(rc, "tode_adapt_step")
+            else:
+                n = norm.to(data_dtype).contiguous()
+                rc = lib.tode_control(code, _lib.C.byref(c), order, B, _lib.ptr(n), _lib.ptr(dt_), *tail)
+                _lib.check(rc, "tode_control")
+            decided["accept"] = accept
+            return (accept, dt_next, ratio, status, prev_o, pprev_o) if pid else (accept, dt_next, ratio, status)
+
+        def formula(dt_, norm_, y0_, y1_, err_, prev_, pprev_):
+            k_i, k_p, k_d = float(self.icoeff) / order, float(self.pcoeff) / order, float(self.dcoeff) / order
+            p = dict(
+                atol=self._atol_f, rtol=self._rtol_f, norm={_lib.NORM_RMS: differentiable.rms, _lib.NORM_MAX: differentiable.maximum_norm}.get(self._norm_id()),
+                almost_zero=float(state.almost_zero), safety=float(self.safety), pid=pid, factor_min=float(self.factor_min), factor_max=float(self.factor_max),
+                e1=-(k_i + k_p + k_d) if pid else -1.0 / order, e2=k_p + 2 * k_d, e3=-k_d,
+                dt_min=_limit(state.dt_min) if limits else None, dt_max=_limit(state.dt_max) if limits else None,
             )  # fmt: skip
-            _lib.check(rc, "tode_adapt_step")
-        else:
-            norm = norm.to(data_dtype).contiguous()
-            rc = lib.tode_control(code, _lib.C.byref(c), int(state.method_order), B, _lib.ptr(norm), _lib.ptr(dt), *tail)
-            _lib.check(rc, "tode_control")
-        return accept, dt_next, ratio, status, prev_o, pprev_o
+            return differentiable.decide(p, decided["accept"], dt_, None if norm_ is None else norm_.to(data_dtype), y0_, y1_, err_, prev_, pprev_)
+
+        out = differentiable.through(kernel, formula, dt, norm, y0, y1, err, prev, pprev)
+        return out if pid else (*out, None, None)
 
     def dt_factor(self, state, error_ratio: torch.Tensor) -> torch.Tensor:
         """Growth factor of the step size for a given error ratio, clipped to
@@ -253,16 +270,21 @@ class AdaptiveStepSizeController(StepSizeController):
         else:
             # user-defined norm: scale on the device, call the norm, decide on the device
             _lib.require_device(y0, y1, error_estimate)
-            a, b, e = y0.contiguous(), y1.contiguous(), error_estimate.contiguous()
-            if a.dtype not in _lib.DTYPES or not (a.dtype == b.dtype == e.dtype):
+            if y0.dtype not in _lib.DTYPES or not (y0.dtype == y1.dtype == error_estimate.dtype):
                 raise NotImplementedError("the step size controllers need float32 or float64 data of one dtype")
-            scaled = torch.empty_like(a)
-            rc = _lib.load().tode_error_scale(
-                _lib.DTYPES[a.dtype], a.shape[0], a.shape[1], self._atol_f, self._rtol_f, _lib.ptr(a), _lib.ptr(b), _lib.ptr(e),
-                _lib.ptr(scaled), _lib.stream_of(a),
-            )  # fmt: skip
-            _lib.check(rc, "tode_error_scale")
-            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, norm=self.norm(scaled), data_dtype=a.dtype)
+
+            def scale_kernel():
+                a, b, e = y0.contiguous(), y1.contiguous(), error_estimate.contiguous()
+                scaled = torch.empty_like(a)
+                rc = _lib.load().tode_error_scale(
+                    _lib.DTYPES[a.dtype], a.shape[0], a.shape[1], self._atol_f, self._rtol_f, _lib.ptr(a), _lib.ptr(b), _lib.ptr(e),
+                    _lib.ptr(scaled), _lib.stream_of(a),
+                )  # fmt: skip
+                _lib.check(rc, "tode_error_scale")
+                return scaled
+
+            scaled = differentiable.through(scale_kernel, partial(differentiable.error_scale, self._atol_f, self._rtol_f), y0, y1, error_estimate)
+            accept, dt_next, ratio, status, prev, pprev = self._decide(state, dt, norm=self.norm(scaled), data_dtype=y0.dtype)
         if self._kind == _lib.CTRL_PID and type(self).update_state is PIDController.update_state:
             state = state.update_error_ratios(prev, pprev)  # the decision kernel has already shifted the history
         else:
@@ -280,43 +302,69 @@ class AdaptiveStepSizeController(StepSizeController):
         _lib.require_device(y0, t0, t1)
         B, F = y0.shape
         lib, code, stream = _lib.load(), _lib.dtype_code(y0.dtype, t0.dtype), _lib.stream_of(y0)
+        atol, rtol, order = self._atol_f, self._rtol_f, int(method_order)
+        guards = self._kind == _lib.CTRL_INTEGRAL  # (only the integral controller's copy treats a zero first guess, :481 / :826)
         f0 = term_.vf(t0, y0, stats, args).to(y0.dtype).contiguous()
-        h0, y1, tn = y0.new_empty(B), torch.empty_like(y0), torch.empty_like(t0)
         if norm is None:
             # user-defined norm: its arguments are scaled on the device, it is called three times
             def scaled_norm(v):
-                out = torch.empty_like(y0)
-                rc = lib.tode_tolerance_scale(code, B, F, self._atol_f, self._rtol_f, _lib.ptr(y0), _lib.ptr(v), _lib.ptr(out), stream)
-                _lib.check(rc, "tode_tolerance_scale")
-                return self.norm(out).to(y0.dtype).contiguous()
+                def kernel():
+                    out = torch.empty_like(y0)
+                    rc = lib.tode_tolerance_scale(code, B, F, atol, rtol, _lib.ptr(y0), _lib.ptr(v), _lib.ptr(out), stream)
+                    _lib.check(rc, "tode_tolerance_scale")
+                    return out
+
+                return self.norm(differentiable.through(kernel, partial(differentiable.tolerance_scale, atol, rtol), y0, v)).to(y0.dtype).contiguous()
 
             d0, d1 = scaled_norm(y0), scaled_norm(f0)
-            rc = lib.tode_initial_step_a_norms(
-                code, B, F, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(d0), _lib.ptr(d1), _lib.ptr(h0),
-                _lib.ptr(y1), _lib.ptr(tn), stream,
-            )  # fmt: skip
-            _lib.check(rc, "tode_initial_step_a_norms")
+
+            def probe_kernel():
+                h0, y1, tn = y0.new_empty(B), torch.empty_like(y0), torch.empty_like(t0)
+                rc = lib.tode_initial_step_a_norms(
+                    code, B, F, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(d0), _lib.ptr(d1), _lib.ptr(h0),
+                    _lib.ptr(y1), _lib.ptr(tn), stream,
+                )  # fmt: skip
+                _lib.check(rc, "tode_initial_step_a_norms")
+                return h0, y1, tn
+
+            h0, y1, tn = differentiable.through(probe_kernel, differentiable.initial_step_a_norms, t0, t1, y0, f0, d0, d1)
             f1 = term_.vf(tn, y1, stats, args).to(y0.dtype).contiguous()
             d2n = scaled_norm(f1 - f0)
-            dt0 = torch.empty_like(t0)
-            rc = lib.tode_initial_step_b_norms(
-                code, self._kind, int(method_order), B, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(h0), _lib.ptr(d1), _lib.ptr(d2n),
-                _lib.ptr(dt0), stream,
+
+            def finish_kernel():
+                dt0 = torch.empty_like(t0)
+                rc = lib.tode_initial_step_b_norms(
+                    code, self._kind, order, B, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(h0), _lib.ptr(d1), _lib.ptr(d2n),
+                    _lib.ptr(dt0), stream,
+                )  # fmt: skip
+                _lib.check(rc, "tode_initial_step_b_norms")
+                return dt0
+
+            return differentiable.through(finish_kernel, partial(differentiable.initial_step_b_norms, guards, order), t0, t1, h0, d1, d2n), f0
+        norm_formula = {_lib.NORM_RMS: differentiable.rms, _lib.NORM_MAX: differentiable.maximum_norm}[norm]
+
+        def probe_kernel():
+            h0, y1, tn = y0.new_empty(B), torch.empty_like(y0), torch.empty_like(t0)
+            rc = lib.tode_initial_step_a(
+                code, norm, B, F, atol, rtol, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0),
+                _lib.ptr(h0), _lib.ptr(y1), _lib.ptr(tn), stream,
             )  # fmt: skip
-            _lib.check(rc, "tode_initial_step_b_norms")
-            return dt0, f0
-        rc = lib.tode_initial_step_a(
-            code, norm, B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1), _lib.ptr(y0), _lib.ptr(f0),
-            _lib.ptr(h0), _lib.ptr(y1), _lib.ptr(tn), stream,
-        )  # fmt: skip
-        _lib.check(rc, "tode_initial_step_a")
+            _lib.check(rc, "tode_initial_step_a")
+            return h0, y1, tn
+
+        h0, y1, tn = differentiable.through(probe_kernel, partial(differentiable.initial_step_a, norm_formula, atol, rtol), t0, t1, y0, f0)
         f1 = term_.vf(tn, y1, stats, args).to(y0.dtype).contiguous()
-        dt0 = torch.empty_like(t0)
-        rc = lib.tode_initial_step_b(
-            code, self._kind, norm, int(method_order), B, F, self._atol_f, self._rtol_f, _lib.ptr(t0), _lib.ptr(t1),
-            _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(f1), _lib.ptr(h0), _lib.ptr(dt0), stream,
-        )  # fmt: skip
-        _lib.check(rc, "tode_initial_step_b")
+
+        def finish_kernel():
+            dt0 = torch.empty_like(t0)
+            rc = lib.tode_initial_step_b(
+                code, self._kind, norm, order, B, F, atol, rtol, _lib.ptr(t0), _lib.ptr(t1),
+                _lib.ptr(y0), _lib.ptr(f0), _lib.ptr(f1), _lib.ptr(h0), _lib.ptr(dt0), stream,
+            )  # fmt: skip
+            _lib.check(rc, "tode_initial_step_b")
+            return dt0
+
+        dt0 = differentiable.through(finish_kernel, partial(differentiable.initial_step_b, norm_formula, guards, order, atol, rtol), t0, t1, y0, f0, f1, h0)
         return dt0, f0
 
 
@@ -390,30 +438,28 @@ class PIDController(AdaptiveStepSizeController):
 
     def merge_states(self, running, current: PIDState, previous: PIDState) -> PIDState:
         """reference step_size_controllers.py:628-638"""
-        mask = running.contiguous()
-        assert mask.element_size() == 1
-        outs = []
-        for cur, prev in ((current.prev_error_ratio, previous.prev_error_ratio), (current.prev_prev_error_ratio, previous.prev_prev_error_ratio)):
-            _lib.require_device(cur, prev, mask)
-            cur, prev = cur.contiguous(), prev.contiguous()
-            assert cur.dtype == prev.dtype and cur.dtype in _lib.DTYPES
-            out = torch.empty_like(cur)
-            rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], cur.shape[0], 1, _lib.ptr(mask), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
-            _lib.check(rc, "tode_select_rows")
-            outs.append(out)
-        return current.update_error_ratios(*outs)
+        pairs = ((current.prev_error_ratio, previous.prev_error_ratio), (current.prev_prev_error_ratio, previous.prev_prev_error_ratio))
+        return current.update_error_ratios(*(_select(running, cur, prev) for cur, prev in pairs))
 
     def update_state(self, state: PIDState, y0, dt, error_ratio, accept) -> PIDState:
         """reference step_size_controllers.py:640-671"""
         if error_ratio is None:
             return state.update_error_ratios(prev_error_ratio=y0.new_ones(dt.shape), prev_prev_error_ratio=state.prev_error_ratio)
         assert accept is not None
-        mask = accept.contiguous()
-        outs = []
-        for cur, prev in ((error_ratio, state.prev_error_ratio), (state.prev_error_ratio, state.prev_prev_error_ratio)):
-            cur, prev = cur.contiguous(), prev.contiguous()
-            out = torch.empty_like(cur)
-            rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], cur.shape[0], 1, _lib.ptr(mask), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
-            _lib.check(rc, "tode_select_rows")
-            outs.append(out)
-        return state.update_error_ratios(*outs)
+        pairs = ((error_ratio, state.prev_error_ratio), (state.prev_error_ratio, state.prev_prev_error_ratio))
+        return state.update_error_ratios(*(_select(accept, cur, prev) for cur, prev in pairs))
+
+
+def _select(mask: torch.Tensor, current: torch.Tensor, previous: torch.Tensor) -> torch.Tensor:
+    """``current`` where ``mask`` (one byte per sample), ``previous`` elsewhere."""
+    _lib.require_device(current, previous, mask)
+    assert mask.element_size() == 1 and current.dtype == previous.dtype and current.dtype in _lib.DTYPES
+
+    def kernel():
+        cur, prev, m = current.contiguous(), previous.contiguous(), mask.contiguous()
+        out = torch.empty_like(cur)
+        rc = _lib.load().tode_select_rows(_lib.DTYPES[cur.dtype], cur.shape[0], 1, _lib.ptr(m), _lib.ptr(cur), _lib.ptr(prev), _lib.ptr(out), _lib.stream_of(cur))
+        _lib.check(rc, "tode_select_rows")
+        return out
+
+    return differentiable.through(kernel, lambda cur, prev: differentiable.select_rows(mask, cur, prev), current, previous)
