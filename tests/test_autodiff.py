@@ -11,6 +11,7 @@ import torch.nn as nn
 
 import torchode_amd as to
 from oracle import torch_loop
+from torchode_amd import autodiff
 from torchode_amd.autodiff import Replay, simulate_hits
 
 gpu = pytest.mark.gpu
@@ -831,3 +832,135 @@ def test_gradients_with_the_grid_and_mlp_terms(name, dtype):
             torch.testing.assert_close(got, want, rtol=rtol, atol=rtol * float(want.abs().max()))
     assert all(bool(x.isfinite().all()) and float(x.abs().max()) > 0 for x in results["kernels"])
 
+
+
+# ---------------------------------------------------------------------------------------------
+# Where a gradient is decided by a tie rule.  The reference keeps every step inside the time range with
+# torch.clamp(dt, t_min - t, t_max - t) (adjoints.py:107, 251), whose backward pass leaves the whole cotangent with
+# dt where t_min - t <= dt <= t_max - t, bounds included, and hands it to a bound only where dt lies strictly beyond
+# it (minimum / maximum would halve it on a tie).  And what no operation connects to ys has no gradient at all.
+# ---------------------------------------------------------------------------------------------
+
+
+class OwnHeunForTies(to.Heun):  # (a subclass: the operator path, whose graph nodes run torch.clamp's own backward pass)
+    pass
+
+
+class OwnTsit5ForTies(to.Tsit5):
+    pass
+
+
+def _sweeps(method):
+    """(name, step method, settings of the solver) for every backward pass that takes the method."""
+    if method == "heun":
+        return [("torch", to.Heun, {}), ("operator-path", OwnHeunForTies, {})]
+    return [("kernels", to.Tsit5, dict(backward_kernels=True)), ("torch", to.Tsit5, dict(backward_kernels=False)), ("operator-path", OwnTsit5ForTies, {})]
+
+
+@gpu
+@pytest.mark.parametrize("method", ["heun", "tsit5"])
+def test_a_first_step_that_equals_the_time_range_keeps_its_cotangent(method):
+    """One fixed step dt0 = t_end - t_start exactly: clamp(dt0, lo, hi) meets its upper bound.  By torch.clamp's rule
+    d dt / d dt0 = 1 and d dt / d t_end = 0, so with the step's result y1(dt) read at x = (t_end - t_start) / dt = 1:
+    dL/d dt0 = w . (dy1/ddt - p'(1) / dt), dL/d t_end = w . p'(1) / dt (p' = dt f(t_end, y1): both interpolants take the
+    last slope at their end), dL/d t_start = -dL/d t_end - [dt's part: none].  Written out below with autograd over the
+    step formula and torch.clamp itself; every backward pass of the library has to return the same, element by element."""
+    A = torch.tensor(A0, dtype=torch.double, device="cuda")
+    # (not a linear right-hand side: Heun's dense output of y' = A y depends on dt and x only through their product)
+    f = lambda t, y: torch.tanh(y @ A) * (1.0 + 0.3 * t)[:, None]
+    span = torch.tensor([1.0, -0.75], dtype=torch.double, device="cuda")
+    results = {}
+    for name, cls, settings in _sweeps(method):
+        y0 = torch.tensor(Y0, dtype=torch.double, device="cuda", requires_grad=True)
+        t_start = torch.tensor([0.0, 2.0], dtype=torch.double, device="cuda", requires_grad=True)
+        t_end = (t_start.detach() + span).requires_grad_()
+        dt0 = span.clone().requires_grad_()
+        solver = to.AutoDiffAdjoint(cls(), to.FixedStepController())
+        for key, value in settings.items():
+            setattr(solver, key, value)
+        solution = solver.solve(to.InitialValueProblem(y0, t_start=t_start, t_end=t_end), term=to.ODETerm(f), dt0=dt0)
+        assert solution.stats["n_steps"].tolist() == [1, 1]
+        weights = torch.tensor([[[0.5, 1.0, 1.5]], [[-1.0, 0.25, 2.0]]], dtype=torch.double, device="cuda")
+        results[name] = (solution.ys.detach(), torch.autograd.grad((solution.ys * weights).sum(), [y0, t_start, t_end, dt0]))
+    # by hand: the step as a formula of (y0, t_start, t_end, dt0), the clamp as the reference writes it
+    y0 = torch.tensor(Y0, dtype=torch.double, device="cuda", requires_grad=True)
+    t_start = torch.tensor([0.0, 2.0], dtype=torch.double, device="cuda", requires_grad=True)
+    t_end = (t_start.detach() + span).requires_grad_()
+    dt0 = span.clone().requires_grad_()
+    dt = torch.clamp(dt0, torch.minimum(t_start, t_end) - t_start, torch.maximum(t_end, t_start) - t_start)
+    h = dt[:, None]
+    if method == "heun":
+        k0 = f(t_start, y0)
+        k1 = f(t_start + dt, y0 + h * k0)
+        y1 = y0 + h * (0.5 * k0 + 0.5 * k1)
+        x = ((t_end - t_start) / ((t_start + dt) - t_start))[:, None]
+        gap = y0 - y1
+        value = y0 + x * (h * k0 + x * ((h * (-2 * k0 - k1) - 3 * gap) + x * (h * (k0 + k1) + 2 * gap)))
+    else:
+        tab = to.Tsit5.TABLEAU
+        ks = [f(t_start, y0)]
+        for i in range(1, 7):
+            ks.append(f(t_start + float(tab.c[i]) * dt, y0 + h * sum(float(tab.a[i, j]) * ks[j] for j in range(i))))
+        x = ((t_end - t_start) / ((t_start + dt) - t_start))[:, None]
+        rows = tab.b_other.tolist()
+        value = y0 + x * (h * ks[0] + x * sum(x**p * h * sum(rows[p][s] * ks[s] for s in range(7)) for p in range(3)))
+    by_hand = torch.autograd.grad((value[:, None] * weights).sum(), [y0, t_start, t_end, dt0])
+    for name, (ys, grads) in results.items():
+        torch.testing.assert_close(ys[:, 0], value.detach(), rtol=1e-12, atol=1e-13, msg=name)
+        for got, expected, which in zip(grads, by_hand, ("y0", "t_start", "t_end", "dt0")):
+            torch.testing.assert_close(got, expected, rtol=1e-9, atol=1e-11, msg=f"{name}: {which}")
+    # the rule is visible: the step's own share is not zero (small for the fifth-order pair, still 10^4 times the
+    # tolerance above), and halving it would move both gradients
+    assert by_hand[3].abs().min() > 1e-5
+
+
+@gpu
+@pytest.mark.parametrize("controller", ["integral", "pid"])
+def test_separate_time_tensors_with_equal_values_get_their_own_gradients(controller):
+    """t_eval[:, 0] == t_start and t_eval[:, -1] == t_end as three tensors of their own: the evaluation points get
+    the interpolants' time derivatives, t_start and t_end what the start rule and the clamps hand them.  All four
+    backward passes (one kernel, per-iteration kernels, torch operations, operator-path graph) agree element by element."""
+    results = {}
+    for sweep in ("whole", "kernels", "torch", "operator-path"):
+        mu = torch.tensor([0.7, 1.9, 1.2, 2.4], dtype=torch.double, device="cuda", requires_grad=True)
+        y0 = torch.tensor([[0.5, -0.2], [1.0, 0.3], [-0.8, 0.6], [0.1, 0.9]], dtype=torch.double, device="cuda", requires_grad=True)
+        t_start = torch.tensor([0.0, 0.5, -0.25, 1.0], dtype=torch.double, device="cuda")
+        t_end = t_start + torch.tensor([1.0, -0.8, 1.3, -1.1], dtype=torch.double, device="cuda")
+        t_eval = (t_start[:, None] + (t_end - t_start)[:, None] * torch.tensor([0.0, 0.3, 0.7, 1.0], dtype=torch.double, device="cuda")).clone()
+        t_eval[:, 0], t_eval[:, -1] = t_start, t_end
+        leaves = [x.clone().requires_grad_() for x in (t_start, t_end, t_eval)]
+        ctrl = to.IntegralController(1e-7, 1e-5) if controller == "integral" else to.PIDController(1e-7, 1e-5, 0.2, 0.5, 0.05)
+        solver = to.AutoDiffAdjoint(OwnTsit5ForTies() if sweep == "operator-path" else to.Tsit5(), ctrl)
+        solver.backward_kernels, solver.backward_whole_kernel = sweep in ("whole", "kernels"), sweep == "whole"
+        solution = solver.solve(to.InitialValueProblem(y0, *leaves), to.ODETerm(to.VanDerPol(mu)))
+        weights = torch.linspace(0.5, 1.5, solution.ys.numel(), dtype=torch.double, device="cuda").reshape(solution.ys.shape)
+        results[sweep] = torch.autograd.grad((solution.ys * weights).sum(), [y0, mu, *leaves])
+        if sweep != "operator-path":
+            assert autodiff.LAST_SWEEP == sweep
+    for sweep in ("whole", "kernels", "torch"):
+        for got, expected, which in zip(results[sweep], results["operator-path"], ("y0", "mu", "t_start", "t_end", "t_eval")):
+            torch.testing.assert_close(got, expected, rtol=1e-7, atol=1e-9 * float(expected.abs().max()), msg=f"{sweep}: {which}")
+    assert all(float(g.abs().max()) > 0 for g in results["operator-path"])
+
+
+@gpu
+def test_a_lone_evaluation_point_at_t_start_connects_nothing_but_y0():
+    """t_eval = t_start[:, None]: ys is a copy of y0 (adjoints.py:121-126) and the loop writes nothing, so in the
+    reference's graph the parameters and the times are not connected to ys: autograd reports them unused (None with
+    allow_unused, an error without), and y0 gets the cotangent itself.  The same from every backward pass."""
+    for sweep in ("whole", "kernels", "torch", "operator-path"):
+        mu = torch.tensor([0.7, 1.9], dtype=torch.double, device="cuda", requires_grad=True)
+        y0 = torch.tensor([[0.5, -0.2], [1.0, 0.3]], dtype=torch.double, device="cuda", requires_grad=True)
+        t_start = torch.tensor([0.0, 0.5], dtype=torch.double, device="cuda", requires_grad=True)
+        t_end = torch.tensor([1.0, -0.3], dtype=torch.double, device="cuda", requires_grad=True)
+        t_eval = t_start.detach()[:, None].clone().requires_grad_()
+        solver = to.AutoDiffAdjoint(OwnTsit5ForTies() if sweep == "operator-path" else to.Tsit5(), to.IntegralController(1e-6, 1e-5))
+        solver.backward_kernels, solver.backward_whole_kernel = sweep in ("whole", "kernels"), sweep == "whole"
+        solution = solver.solve(to.InitialValueProblem(y0, t_start, t_end, t_eval), to.ODETerm(to.VanDerPol(mu)))
+        assert torch.equal(solution.ys[:, 0].detach(), y0.detach()) and solution.stats["n_initialized"].tolist() == [1, 1]
+        weights = torch.tensor([[[0.5, 0.7]], [[-1.5, 2.0]]], dtype=torch.double, device="cuda")
+        grads = torch.autograd.grad((solution.ys * weights).sum(), [y0, mu, t_start, t_end, t_eval], allow_unused=True, retain_graph=True)
+        assert torch.equal(grads[0], weights[:, 0]), sweep
+        assert all(g is None for g in grads[1:]), (sweep, grads[1:])
+        with pytest.raises(RuntimeError, match="not have been used"):
+            torch.autograd.grad((solution.ys * weights).sum(), [mu])

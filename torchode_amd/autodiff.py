@@ -126,6 +126,15 @@ class LoopRecord:
         pprev = getattr(controller_state, "prev_prev_error_ratio", ones)
         self.states.append((t.clone(), dt.clone(), y.clone(), torch.zeros_like(y), prev.clone(), pprev.clone(), running.clone(), n_accepted.clone()))
 
+    def any_point_written(self, problem: InitialValueProblem) -> bool:
+        """Whether an iteration of the recorded loop passed an evaluation point that was still to be written
+        (adjoints.py:215-234): the last recorded time against the points, the one at ``t_start`` aside."""
+        t_last = self.arrays["t"][self.iterations] if self.arrays is not None and not self.states else self.states[-1][0]
+        direction = torch.where(problem.t_end > problem.t_start, 1.0, -1.0).to(t_last.dtype)[:, None]
+        passed = direction * t_last[:, None] >= direction * problem.t_eval
+        passed[:, 0] &= problem.t_eval[:, 0] != problem.t_start
+        return bool(passed.any())
+
     def trimmed(self, iterations: int) -> List[dict]:
         """States 0..iterations; iterations enqueued after the batch had stopped changed nothing."""
         if not self.states and self.arrays is not None:  # (views of the arrays, made when a per-iteration sweep asks)
@@ -198,7 +207,7 @@ class Replay:
 
     @property
     def t_hi(self):
-        return torch.maximum(self.t_start, self.t_end)
+        return torch.maximum(self.t_end, self.t_start)
 
     def f(self, t, y):
         out = self.term.f(t, y, self.args) if self.term.with_args else self.term.f(t, y)
@@ -661,6 +670,13 @@ class SolveThroughLoop(torch.autograd.Function):
         adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
         if ctx.record.flags is not None and ctx.record.flags.tolist()[_lib.FLAG_NEEDS_GENERAL]:
             raise RuntimeError("the record of the loop state was too short for the solve it was sized from")
+        if problem.n_evaluation_points > 0 and not ctx.record.any_point_written(problem):
+            # No iteration wrote an evaluation point (every sample's points lie at t_start, or the batch stopped before
+            # one was reached): ys is a copy of y0 where t_eval[:, 0] == t_start and nothing else, so in the reference's
+            # graph no parameter and no time is connected to it: autograd reports them unused, not zero.
+            at_start = problem.t_eval[:, 0] == problem.t_start
+            first = torch.where(at_start[:, None], grad_ys[:, 0], torch.zeros_like(grad_ys[:, 0]))
+            return (None, None, None, None, None, first, *([None] * len(params)))
         # The sweep works on leaves of its own for the times and the tensors in args: one of them may be computed
         # from another (t_start is usually a column of t_eval), and a gradient taken with respect to both would
         # reach the first one twice, once here and once when autograd carries the second one's gradient on.
@@ -739,7 +755,8 @@ class SolveThroughLoop(torch.autograd.Function):
                     cotangents.append(adj["k0"])
             if adj["dt"] is not None and replay.through_control:
                 dt_first = replay.first_step(y_in, f0) if dt0 is None else dt0.to(replay.t_start.dtype)
-                dt_first = torch.minimum(torch.maximum(dt_first, replay.t_lo - replay.t_start), replay.t_hi - replay.t_start)
+                # (torch.clamp as in reference adjoints.py:107: on a tie with a bound the step keeps the cotangent)
+                dt_first = torch.clamp(dt_first, replay.t_lo - replay.t_start, replay.t_hi - replay.t_start)
                 if dt_first.requires_grad:
                     targets.append(dt_first)
                     cotangents.append(adj["dt"])

@@ -100,7 +100,9 @@ __device__ __forceinline__ void start_backward(const CtrlParams<T> &cp, const Te
         const T first = dir * tmin((T)100 * h0, h1);
         const T lo = tmin(ts, te) - ts, hi = tmax(te, ts) - ts;
         // ---- reversed ----
-        const T g_first = a_dt * share_of_min<T>(tmax(first, lo), hi) * share_of_max<T>(first, lo);
+        // torch.clamp(first, lo, hi) (adjoints.py:107): the whole cotangent stays with the step where it lies within
+        // the bounds, the bounds included (another rule than minimum / maximum, which halve it on a tie)
+        const T g_first = (first >= lo && first <= hi) ? a_dt : (T)0;
         const T g_min = g_first * dir;
         T g_h0 = (T)100 * (g_min * share_of_min<T>((T)100 * h0, h1));
         const T g_h1 = g_min * share_of_min<T>(h1, (T)100 * h0);
