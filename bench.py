@@ -40,8 +40,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 MFMA_FP32_PEAK_TFLOPS = 157.3
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch of the solve kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); absent (null in the output) where not measured.
+# HBM bytes per launch of the solve kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (the
+# summaries under profiles/ name their commands).  A counter run is a run of its own, so these are constants read from
+# those summaries, not something this run measures: the output says so (`traffic_source`), and a shape without a
+# summary reports null.
+TRAFFIC_PROFILES = {
+    ("vdp", "torch.float32", 65536): "profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt",
+    ("vdp", "torch.float64", 65536): "profiles/solve_pair_kernel_vdp_f64_b65536_hbm_traffic.txt",
+    ("lorenz", "torch.float32", 1048576): "profiles/solve_fast_kernel_lorenz_f32_b1048576_hbm_traffic.txt",
+    ("reaction_diffusion", "torch.float32", 512): "profiles/solve_grid_kernel_reaction_diffusion_f32_b512_hbm_traffic.txt",
+    ("mlp", "torch.float32", 4096): "profiles/solve_mlp_kernel_mlp_f32_b4096_hbm_traffic.txt",
+}
 MEASURED_TRAFFIC_BYTES = {
     # profiles/solve_pair_kernel_vdp_f32_b65536_hbm_traffic.txt: (6871.2 KiB x 2.000 + 32926.0 KiB x 1.000) x 1024
     ("vdp", "torch.float32", 65536): 47.79e6,
@@ -65,6 +74,12 @@ OTHER_CONFIGS = [
     ("mlp", "f32", "bfloat16"),
 ]
 START = time.perf_counter()
+
+
+def traffic_source(key):
+    if key not in MEASURED_TRAFFIC_BYTES:
+        return None
+    return f"{TRAFFIC_PROFILES[key]}: rocprofv3 --pmc counter runs of this script, read from that summary, not measured in this run"
 
 
 def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_iterations=-1, batch_copies=None):
@@ -135,6 +150,7 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBPS,
         "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)),
+        "traffic_source": traffic_source((w.name, str(dtype), B)),
         "algorithmic_bytes_per_launch": algo_bytes,
         "bytes_per_sample_step": w.bytes_step,
         "bytes_dense_per_sample": w.bytes_dense,
@@ -162,6 +178,7 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
             "unit": "TFLOP/s",
             "frac": tflops / peak,
             "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, str(dtype), B)) if mlp_inputs == "float32" else None,
+            "traffic_source": traffic_source((w.name, str(dtype), B)) if mlp_inputs == "float32" else None,
             "algorithmic_flops_per_launch": flops,
             "flops_per_rhs_evaluation_per_sample": flops_f,
             "kernel_ms": kernel_s * 1e3,
@@ -186,29 +203,6 @@ def measure(args, name, dtype_flag, mlp_inputs, steps, warmup, path=None, graph_
     del sol, problem, w
     torch.cuda.empty_cache()
     return result
-
-
-def measure_issue_interval():
-    """Nanoseconds per vector operation of one wavefront, and per SIMD (that divided by the wavefronts that share it),
-    for chains of dependent operations: what bounds a kernel that keeps one sample per lane in registers.  Cycles are
-    quoted at the 2.4 GHz the GPU reaches at most."""
-    import torch
-
-    from torchode_amd import _lib
-
-    rows = []
-    for dtype in (torch.float32, torch.float64):
-        for waves in (1, 2, 4, 8):
-            for chains in (1, 2, 4, 8):
-                per_wave = _lib.vector_issue_interval(dtype, "fma", chains, waves)
-                rows.append({"dtype": str(dtype)[6:], "operation": "fma", "wavefronts_per_simd": waves, "chains": chains,
-                             "ns_per_operation_of_a_wavefront": round(per_wave, 3), "ns_per_operation_of_a_simd": round(per_wave / waves, 3),
-                             "cycles_at_2.4_GHz_per_operation_of_a_simd": round(2.4 * per_wave / waves, 2)})  # fmt: skip
-        for op in ("div", "sqrt"):
-            per_wave = _lib.vector_issue_interval(dtype, op, 1, 1)
-            rows.append({"dtype": str(dtype)[6:], "operation": op, "wavefronts_per_simd": 1, "chains": 1, "ns_per_operation_of_a_wavefront": round(per_wave, 2),
-                         "cycles_at_2.4_GHz_per_operation_of_a_wavefront": round(2.4 * per_wave, 1)})  # fmt: skip
-    return {"metric": "vector issue interval", "unit": "ns per operation", "simds": 1024, "rows": rows}
 
 
 def measure_gradient(args, steps=10, warmup=3):
@@ -274,7 +268,6 @@ def main():
     )
     ap.add_argument("--mlp-inputs", default="float32", choices=["float32", "bfloat16"], help="mlp workload: what the matrix cores take as inputs (bfloat16: a reduced-precision variant, reported against the bf16 peak)")
     ap.add_argument("--gradient", action="store_true", help="measure the differentiable solve of the headline configuration alone (forward with its record, backward)")
-    ap.add_argument("--issue-probe", action="store_true", help="measure the vector issue interval of the GPU's SIMDs (chains of dependent multiply-adds, divisions, square roots; 1-8 wavefronts per SIMD) instead of a solve")
     ap.add_argument("--graph-iterations", type=int, default=None, help="per-step path: replay this many iterations at a time from a HIP graph")
     ap.add_argument("--cpu-baseline-seconds", type=float, default=10.0, help="CPU work the headline's eager baseline is sized to (the other configurations take 0.4 of it)")
     ap.add_argument("--time-budget", type=float, default=420.0, help="seconds the whole run aims to stay within: a compiled CPU leg is started only while 100 s of it are left")
@@ -300,9 +293,6 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    if args.issue_probe:
-        print(json.dumps(measure_issue_interval()))
-        return
     if args.fast_variant:
         from torchode_amd import _lib
 

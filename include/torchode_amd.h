@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TODE_ABI_VERSION 22
+#define TODE_ABI_VERSION 23
 
 /* floating point type of data (y) and time (t) arrays */
 enum { TODE_F32 = 0, TODE_F64 = 1 };
@@ -296,12 +296,19 @@ int tode_solve_builtin_fast_sync(const tode_solve_args *args, const tode_control
  * and launches nothing.  With n_eval > 0 the array sets no limit.  Shapes that
  * tode_solve_builtin_fast refuses are refused here with the same code.
  *
- * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU
- * (several streams, several host threads) race on it and must be serialised by
- * the caller.  Calls in a row on one stream need nothing: each call resets the
- * words it uses by a kernel in front of the solve kernel.  The array's address
- * is looked up on the first call on a device (hipGetSymbolAddress, not an
- * allocation); a caller that captures a graph makes one call before capturing.
+ * Every call on a GPU uses that GPU's one array, so calls must not overlap on a
+ * GPU.  Calls in a row on one stream need nothing: the stream orders them, and
+ * each call resets the words it uses by a kernel in front of the solve kernel.
+ * Host threads take turns inside the call.  A call on another stream than the
+ * GPU's last call is refused with TODE_E_UNSUPPORTED, and launches nothing,
+ * while that last call's work has not finished (an event recorded behind every
+ * call is looked at, no waiting); the caller synchronises and calls again.
+ * Under stream capture nothing runs at the time of the call, so nothing is
+ * checked: whoever replays the graph keeps the replays apart from other calls
+ * on that GPU.  The array's address is looked up and the event made on the
+ * first call on a device (hipGetSymbolAddress and hipEventCreate: no device
+ * memory is allocated); a caller that captures a graph makes one call before
+ * capturing.
  */
 #define TODE_STATIC_STAGING_BYTES (2 << 20)
 int tode_solve_builtin_fast_static(const tode_solve_args *args, const tode_controller *controller, int64_t *out_n_steps,
@@ -523,20 +530,6 @@ int tode_last_solve_kernel_ms(float *out_ms);
 /* Name of the solve kernel most recently launched by the calling thread ("" if none), e.g.
  * "tode::solve_pair_kernel"; the same for every template instance of a kernel. */
 const char *tode_last_solve_kernel_name(void);
-
-/*
- * Measurement aid; no counterpart in the reference.  Runs `wavefronts` wavefronts (one per workgroup; 1024 of them are
- * one per SIMD of an MI355X, 2048 two, ...), each issuing 16384 vector fused multiply-adds (operation 0), or 2048
- * correctly rounded divisions (1) or square roots (2), arranged as `chains` (1, 2, 4 or 8) independent dependency
- * chains, and writes the time from the first wavefront's start to the last one's end divided by the operations of one
- * wavefront, in nanoseconds (by the GPU-wide constant 100 MHz counter: the shader clock varies with load; at 2.4 GHz a
- * nanosecond is 2.4 cycles): divided by the wavefronts that share a SIMD, the interval at which a SIMD issues.  It is the rate
- * the per-step cost of the whole-solve kernels is read against: those are chains of dependent vector instructions,
- * one sample per lane.  scratch: device memory of tode_probe_scratch_bytes(wavefronts) bytes.  Synchronises `stream`.
- */
-int64_t tode_probe_scratch_bytes(int32_t wavefronts);
-int tode_probe_vector_issue(int32_t dtype, int32_t operation, int32_t chains, int32_t wavefronts, void *scratch, int64_t scratch_bytes,
-                            double *ns_per_operation, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Reverse of one loop iteration of the per-step kernels (gradients through the loop)

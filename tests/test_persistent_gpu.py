@@ -846,28 +846,6 @@ def test_mixed_dtypes_whole_solve_kernel_equals_the_per_step_kernels(case, time_
         assert (whole.status == 0).all() and int(whole.stats["n_steps"].max()) > 10
 
 
-def test_vector_issue_probe_reports_plausible_intervals():
-    """The measurement aid behind the per-step cost figures: a wavefront alone on its SIMD cannot issue dependent
-    multiply-adds faster than one per 4 cycles (16 lanes per cycle: 1.67 ns at 2.4 GHz), more chains or more wavefronts per SIMD bring the
-    SIMD's interval down towards that, and a correctly rounded division is a sequence of a dozen such instructions."""
-    from torchode_amd import _lib
-
-    one = _lib.vector_issue_interval(torch.float32, "fma", chains=1, wavefronts_per_simd=1)
-    eight_chains = _lib.vector_issue_interval(torch.float32, "fma", chains=8, wavefronts_per_simd=1)
-    four_waves = _lib.vector_issue_interval(torch.float32, "fma", chains=1, wavefronts_per_simd=4) / 4
-    division = _lib.vector_issue_interval(torch.float32, "div", chains=1, wavefronts_per_simd=1)
-    # (nanoseconds; 4 cycles at 2.4 GHz are 1.67 ns)
-    assert 1.5 <= eight_chains <= 1.05 * one <= 8.0, (one, eight_chains)
-    assert 1.5 <= four_waves <= one, (four_waves, one)
-    assert division >= 5 * one, (division, one)
-    lib = _lib.load()
-    out = _lib.C.c_double(0.0)
-    scratch = torch.empty(64, dtype=torch.uint8, device="cuda")
-    assert lib.tode_probe_vector_issue(_lib.F32, 0, 3, 1024, scratch.data_ptr(), scratch.numel(), _lib.C.byref(out), None) == _lib.E_INVALID  # (too little scratch)
-    big = torch.empty(lib.tode_probe_scratch_bytes(1024), dtype=torch.uint8, device="cuda")
-    assert lib.tode_probe_vector_issue(_lib.F32, 0, 3, 1024, big.data_ptr(), big.numel(), _lib.C.byref(out), None) == _lib.E_INVALID  # (3 chains)
-
-
 @pytest.mark.parametrize("case", ["lorenz-f32-64-points", "vdp-f64-50-points", "lorenz-f32-41-points", "lorenz-f32-ragged-batch"])
 def test_one_wavefront_kernel_storing_its_points_four_at_a_time(case):
     """Variant 3 of the fast kernel where the whole dense output of a wavefront's samples does not fit into LDS: four

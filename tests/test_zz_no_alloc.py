@@ -151,3 +151,84 @@ def test_sizes_beyond_the_static_array_are_refused_with_a_clear_error():
     same(static_call(at_limit, n_eval_given=False), sync_call(at_limit, n_eval_given=False))
     small = to.workloads.make("vdp", batch=500, dtype=F32, device="cuda")
     same(static_call(small, n_eval_given=False), sync_call(small, n_eval_given=False))
+
+
+def _prepared(w):
+    """A static call with every tensor made beforehand: ``launch(stream)`` only enqueues."""
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    a, ctrl, ys, out, keep = _args(w, True)
+    flags = torch.full((_lib.FLAG_WORDS,), -1, dtype=torch.int32, device="cuda")
+    pointers = [_lib.ptr(out[i]) for i in range(4)]
+
+    def launch(stream):
+        return lib.tode_solve_builtin_fast_static(_lib.C.byref(a), _lib.C.byref(ctrl), *pointers, flags.data_ptr(), stream)
+
+    return launch, ys, out, flags, keep
+
+
+def test_calls_leave_the_free_device_memory_as_it_was_and_record_into_a_graph():
+    """Nothing is allocated: the free device memory reads the same after a row of calls, and a call records into a HIP
+    graph (a capture in the strict mode turns any allocation call into an error); every replay, with eager work and
+    synchronisations in between, gives the bits of tode_solve_builtin_fast_sync."""
+    from torchode_amd import _lib
+
+    w = to.workloads.make("vdp", batch=5000, dtype=F32, device="cuda")
+    want = sync_call(w)
+    launch, ys, out, flags, keep = _prepared(w)
+    current = _lib.stream_of(w.y0)
+    assert launch(current) == 0  # (the first call on the device looks the array's address up)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(20):
+        assert launch(current) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    same((ys, out, flags.tolist()), want)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph.capture_begin(capture_error_mode="global")
+        try:
+            rc = launch(_lib.C.c_void_p(side.cuda_stream))
+        finally:
+            graph.capture_end()
+    assert rc == 0, _lib.load().tode_last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        ys.fill_(float("nan"))
+        out.fill_(-7)
+        flags.fill_(-1)
+        other = to.workloads.make("lorenz", batch=900 + replay, dtype=F32, device="cuda")  # eager work of another shape in between
+        same(static_call(other), sync_call(other))
+        graph.replay()
+        torch.cuda.synchronize()
+        same((ys, out, flags.tolist()), want)
+    assert torch.cuda.mem_get_info()[0] <= free_before  # (the test's own tensors aside, nothing was handed back either)
+
+
+def test_a_call_on_another_stream_is_refused_while_the_last_one_runs():
+    from torchode_amd import _lib
+
+    lib = _lib.load()
+    w = to.workloads.make("vdp", batch=2000, dtype=F32, device="cuda")
+    want = sync_call(w)
+    first, *_ = _prepared(w)
+    second, ys, out, flags, keep = _prepared(w)
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    big = torch.randn(8192, 8192, device="cuda")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(a):
+        for _ in range(8):
+            big = big @ big * 1e-4  # tens of milliseconds of work in front of the first call
+        assert first(_lib.C.c_void_p(a.cuda_stream)) == 0
+    rc = second(_lib.C.c_void_p(b.cuda_stream))
+    assert rc == _lib.E_UNSUPPORTED and b"another stream" in lib.tode_last_error()
+    assert first(_lib.C.c_void_p(a.cuda_stream)) == 0  # the same stream again: ordered by the stream, accepted
+    torch.cuda.synchronize()
+    assert second(_lib.C.c_void_p(b.cuda_stream)) == 0  # the last call has finished: another stream may have the array
+    torch.cuda.synchronize()
+    same((ys, out, flags.tolist()), want)

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtorchode_amd.so")
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 END_ONLY_MAX_BATCH = 2048 * 64  # TODE_END_ONLY_MAX_BATCH
 MLP_PACKED_SIZE = {"float32": 152 * 256, "bfloat16": 92 * 256}
 MLP_INPUTS = {"float32": 0, "bfloat16": 1}
@@ -57,8 +57,6 @@ EXPORTS = (
     "tode_set_kernel_timing",
     "tode_last_solve_kernel_ms",
     "tode_last_solve_kernel_name",
-    "tode_probe_scratch_bytes",
-    "tode_probe_vector_issue",
     "tode_tableau",
     "tode_erk_stage",
     "tode_erk_combine",
@@ -369,10 +367,6 @@ def load():
         lib.tode_last_solve_kernel_name.restype = C.c_char_p
         lib.tode_last_solve_kernel_name.argtypes = []
         lib.tode_last_solve_kernel_ms.argtypes = [C.POINTER(C.c_float)]
-        lib.tode_probe_scratch_bytes.restype = C.c_int64
-        lib.tode_probe_scratch_bytes.argtypes = [C.c_int32]
-        lib.tode_probe_vector_issue.restype = C.c_int
-        lib.tode_probe_vector_issue.argtypes = [C.c_int32] * 4 + [C.c_void_p, C.c_int64, C.POINTER(C.c_double), C.c_void_p]
         V, I32, I64, D = C.c_void_p, C.c_int32, C.c_int64, C.c_double
         DP, CP = C.POINTER(C.c_double), C.POINTER(Controller)
         for name, argtypes in {
@@ -444,18 +438,6 @@ def stream_of(t) -> C.c_void_p:
     if _raw_stream is not None:  # (the handle without a Stream object around it: 0.3 instead of 3 microseconds)
         return C.c_void_p(_raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
-
-
-def vector_issue_interval(dtype: torch.dtype, operation: str = "fma", chains: int = 1, wavefronts_per_simd: int = 1, simds: int = 1024) -> float:
-    """Nanoseconds per vector operation of one wavefront, first start to last end (``tode_probe_vector_issue``), with
-    ``wavefronts_per_simd`` wavefronts on every SIMD, each running ``chains`` independent dependency chains."""
-    lib = load()
-    n = simds * wavefronts_per_simd
-    scratch = torch.empty(lib.tode_probe_scratch_bytes(n), dtype=torch.uint8, device="cuda")
-    out = C.c_double(0.0)
-    check(lib.tode_probe_vector_issue(DTYPES[dtype], {"fma": 0, "div": 1, "sqrt": 2}[operation], chains, n, scratch.data_ptr(), scratch.numel(),
-                                      C.byref(out), stream_of(scratch)), "tode_probe_vector_issue")  # fmt: skip
-    return out.value
 
 
 def set_kernel_timing(enable: bool):

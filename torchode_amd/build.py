@@ -57,7 +57,6 @@ UNITS = [
     ("tode_ops.hip", "tode_ops.o", []),
     ("tode_grid.hip", "tode_grid.o", []),
     ("tode_mlp.hip", "tode_mlp.o", []),
-    ("tode_probe.hip", "tode_probe.o", []),
 ]
 
 
@@ -115,8 +114,10 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
 
     with ThreadPoolExecutor(max_workers=min(8, len(UNITS) + 1)) as pool:
         ops_object = pool.submit(compile_ops_object)  # (host code only, done long before the kernels)
+        checked = pool.submit(check_units_under_register_pressure)
         objs = list(pool.map(compile_unit, UNITS))
         ops_object = ops_object.result()
+        checked.result()
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-Wno-unused-command-line-argument", "-o", LIB, *objs])
     link_ops_library(ops_object)
     return LIB
@@ -162,6 +163,21 @@ def emit_assembly(directory: str, units=None) -> list:
 
     with ThreadPoolExecutor(max_workers=min(8, len(chosen) + 1)) as pool:
         return list(pool.map(emit, chosen))
+
+
+# The units whose kernels keep whole per-sample arrays in registers (up to 256 of them, some in accumulation
+# registers): where the compiler has been seen to place copies ahead of the execution mask's restore.
+UNITS_UNDER_REGISTER_PRESSURE = ("tode_backward_f32.o", "tode_backward_f64.o")
+
+
+def check_units_under_register_pressure() -> None:
+    """Part of every build: the device assembly of those units is searched for the miscompilation described at
+    ``copies_ahead_of_the_exec_restore``; a hit fails the build, since the library would load and run and return
+    wrong gradients without any error."""
+    for path in emit_assembly(os.path.join(OBJ, "asm"), UNITS_UNDER_REGISTER_PRESSURE):
+        hits = copies_ahead_of_the_exec_restore(path)
+        if hits:
+            raise RuntimeError(f"{path}: register copies ahead of the restore of the execution mask (kernel, line, copies): {hits[:5]}")
 
 
 def copies_ahead_of_the_exec_restore(assembly_path: str) -> list:

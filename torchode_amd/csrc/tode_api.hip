@@ -134,22 +134,34 @@ constexpr size_t STATIC_FLAG_BYTES = 256;
 static __device__ __align__(256) unsigned char scratch[STATIC_FLAG_BYTES + TODE_STATIC_STAGING_BYTES];
 static void *g_scratch_ptr[FLAG_DEVICES];  // static storage: null until asked for
 static std::mutex g_scratch_mutex;
+// Who used a device's array last: a call on another stream is refused while that work has not finished (the event
+// behind it has not fired).  The event is made with the array's address, on the first call on the device.
+struct StaticUse {
+    hipEvent_t done = nullptr;
+    hipStream_t stream = nullptr;
+    bool recorded = false;
+};
+static StaticUse g_static_use[FLAG_DEVICES];
 
-static int static_scratch(hipStream_t s, unsigned char **out) {
+// (called with g_scratch_mutex held)
+static int static_scratch(hipStream_t s, unsigned char **out, int *device_out) {
     int device = 0;
     int rc = check_hip(s ? hipStreamGetDevice(s, &device) : hipGetDevice(&device), "device of the stream");
     if (rc) return rc;
     if (device < 0 || device >= FLAG_DEVICES) return fail(TODE_E_UNSUPPORTED, "device index %d", device);
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    *device_out = device;
     if (!g_scratch_ptr[device]) {
         int current = 0;
         if ((rc = check_hip(hipGetDevice(&current), "hipGetDevice"))) return rc;
         if (current != device && (rc = check_hip(hipSetDevice(device), "hipSetDevice"))) return rc;
         void *ptr = nullptr;
-        const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        hipEvent_t done = nullptr;
+        if (err == hipSuccess && ptr) err = hipEventCreateWithFlags(&done, hipEventDisableTiming);
         if (current != device) (void)hipSetDevice(current);
         if (err != hipSuccess) return check_hip(err, "hipGetSymbolAddress of the static scratch array");
         if (!ptr) return fail(TODE_E_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+        g_static_use[device].done = done;
         g_scratch_ptr[device] = ptr;
     }
     *out = (unsigned char *)g_scratch_ptr[device];
@@ -381,8 +393,25 @@ int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controll
                     "%lld x %d values of %zu bytes exceed its %lld bytes", (long long)a->batch, a->n_features, value_bytes, (long long)TODE_STATIC_STAGING_BYTES);
     hipStream_t s = (hipStream_t)stream;
     unsigned char *base = nullptr;
-    int rc = static_scratch(s, &base);
+    // One call at a time enqueues work on a device's array (host threads take turns here), and a call on another
+    // stream than the last one's is refused while the last one's work is still running: on one stream calls are
+    // ordered by the stream, across streams nothing would order them.  A stream under capture launches nothing
+    // now, so there is nothing to look at: the owner of the graph keeps its replays apart from other calls.
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    int device = 0;
+    int rc = static_scratch(s, &base, &device);
     if (rc) return rc;
+    StaticUse &use = g_static_use[device];
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (s && (rc = check_hip(hipStreamIsCapturing(s, &capture), "hipStreamIsCapturing"))) return rc;
+    const bool live = capture == hipStreamCaptureStatusNone;
+    if (live && use.recorded && use.stream != s) {
+        const hipError_t q = hipEventQuery(use.done);
+        if (q == hipErrorNotReady)
+            return fail(TODE_E_UNSUPPORTED, "the static scratch array of this GPU is in use by a call on another stream that has not finished: "
+                        "calls that overlap on one GPU have to be serialised by the caller");
+        if (q != hipSuccess) return check_hip(q, "hipEventQuery of the last static call");
+    }
     int32_t *words = (int32_t *)base;
     void *staging = base + STATIC_FLAG_BYTES;
 
@@ -399,6 +428,14 @@ int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controll
         hipLaunchKernelGGL(empty_flags_kernel, dim3(1), dim3(64), 0, s, flags_out);
         return check_hip(hipGetLastError(), "tode_solve_builtin_fast_static launch");
     }
+    struct MarkUse {  // (whichever way the call leaves from here on: the work enqueued so far is the array's last use)
+        StaticUse &use;
+        hipStream_t s;
+        bool live;
+        ~MarkUse() {
+            if (live && hipEventRecord(use.done, s) == hipSuccess) use.stream = s, use.recorded = true;
+        }
+    } mark{use, s, live};
     if (end_only) {
         const long long n = (long long)a->batch * a->n_features;
         const unsigned blocks = (unsigned)((n + 255) / 256);
