@@ -34,6 +34,8 @@ struct GridOut {
 template <typename T, int NW, int R> struct GridShared {
     T xch[2][R * NW * 256];  // stage input, double buffered
     T red[2][R][NW][2];      // chunk sums of up to two reductions, double buffered
+    T xs[NW * 64];           // positions within the step of the evaluation points it passed (one per thread and round)
+    int passed[NW];          // per wavefront: how many of its threads' candidate points the step passed
 };
 
 // Four consecutive values, moved with the widest loads and stores their alignment allows.
@@ -274,37 +276,52 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
         n_acc += accept ? 1 : 0;
 
         // ---- dense output at the evaluation points this step passed (adjoints.py:215-234) ----
-        // (band by band: the coefficients of one band at a time are alive)
+        // Which points those are and where each lies within the step, x = (t_eval - t0) / (t1 - t0), is the same for
+        // every cell of the sample: worked out once per point (thread i looks at point cursor + i; the evaluation times
+        // are monotone, so the passed ones are the first `count` of them) and handed round in LDS, instead of a division
+        // and a comparison per thread and point.  What every thread then does per point is the polynomial of its four
+        // cells and one 16-byte store.  (Band by band: the coefficients of one band at a time are alive.)
         if (cursor < E && fma_(dir, t_new, -dir * te_s[cursor]) >= (T)0) {
             const T t1 = t0 + dt;
-            int reached = cursor;
+            while (true) {
+                const int mine = cursor + tid;
+                const bool ok = mine < E && fma_(dir, t_new, -dir * te_s[mine]) >= (T)0;
+                if (ok) sh.xs[tid] = unit_time(te_s[mine], t0, t1);
+                const unsigned long long votes = __ballot(ok);
+                if ((tid & 63) == 0) sh.passed[tid >> 6] = __popcll(votes);
+                lds_barrier();
+                int count = 0;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                T q[4][5][1];
+                for (int w = 0; w < NW; ++w) count += sh.passed[w];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    T ks[7];
-#pragma unroll
-                    for (int s = 0; s < 7; ++s) ks[s] = k[s][r][j];
-                    quartic_elem<T, METHOD>(dt, y[r][j], y1[r][j], ks, true, q[j]);
-                }
-                int at = cursor;
-                do {
-                    const T x = unit_time(te_s[at], t0, t1);
-                    T out[4];
+                for (int r = 0; r < R; ++r) {
+                    T q[4][5][1];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        T v = q[j][4][0];
+                        T ks[7];
 #pragma unroll
-                        for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
-                        out[j] = v;
+                        for (int s = 0; s < 7; ++s) ks[s] = k[s][r][j];
+                        quartic_elem<T, METHOD>(dt, y[r][j], y1[r][j], ks, true, q[j]);
                     }
-                    store4<T>(p.ys + (b * E + at) * F + r * BAND + 4 * tid, out);
-                    ++at;
-                } while (at < E && fma_(dir, t_new, -dir * te_s[at]) >= (T)0);
-                reached = at;
+                    T *row = p.ys + (b * E + cursor) * F + r * BAND + 4 * tid;
+#pragma unroll 4
+                    for (int i = 0; i < count; ++i) {
+                        const T x = sh.xs[i];
+                        T out[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            T v = q[j][4][0];
+#pragma unroll
+                            for (int pw = 3; pw >= 0; --pw) v = fma_(v, x, q[j][pw][0]);
+                            out[j] = v;
+                        }
+                        store4<T>(row + (long long)i * F, out);
+                    }
+                }
+                cursor += count;
+                if (count < NT || cursor >= E) break;
+                lds_barrier();  // (a step that passed more points than the workgroup has threads: another round)
             }
-            cursor = reached;
         }
 
         // ---- state update (adjoints.py:150-155, 247-255) ----

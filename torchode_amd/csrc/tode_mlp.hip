@@ -40,7 +40,9 @@ struct MlpOut {
 };
 
 constexpr int MLP_F = 64, MLP_H = 256, MLP_TILE = 16;
-constexpr int MLP_XS = 84;  // LDS row of the stage input: 64 features, t, zeros up to column 79, padding
+// LDS row of the stage input: 64 features, t, zeros up to column 79; padded to 100 values = 4 banks past a multiple of
+// 32, so that the 16-byte reads and writes of eight lanes that differ in their sample fall on 32 different banks
+constexpr int MLP_XS = 100;
 constexpr int MLP_REGS = 68 + 16 + 64 + 4;       // packed values per thread: W1, b1, W2, b2
 constexpr int MLP_REGS_BF16 = 40 + 16 + 32 + 4;  // the same with W1 (80 inputs) and W2 as pairs of bfloat16
 
@@ -369,21 +371,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
     int slot = 0;
 
-    // ---- weights into registers ----
-    Weights W;
-    mlp_load(W, packed, tid);
-    for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns from 65 on
-    for (int i = tid; i < rows * E; i += 256) te_s[i] = end_only ? p.t_end[(b0 + i) * p.te_stride] : p.t_eval[b0 * E + i];
-    __syncthreads();
-
-    // ---- state of the lane's sample ----
+    // ---- state of the lane's sample (asked for first: these loads are on their way while the weights arrive) ----
     const bool live = c < rows;
     const long long bs = b0 + (live ? c : 0);
-    const T *tev = te_s + (live ? c : 0) * E;
     const T ts = p.t_start[bs * p.ts_stride], te = p.t_end[bs * p.te_stride];
-    const T dir = (te > ts) ? (T)1 : (T)-1, tlo = tmin(ts, te), thi = tmax(te, ts);
-    bool bail = false;
-    for (int e = 1; e < E; ++e) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));  // not monotone
     T y[4], k[7][4];
     {
         if (quads) {
@@ -394,6 +385,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             for (int r = 0; r < 4; ++r) y[r] = f0 + r < FR ? p.y0[bs * FR + f0 + r] : 0.0f;
         }
     }
+
+    // ---- weights into registers ----
+    Weights W;
+    mlp_load(W, packed, tid);
+    for (int i = tid; i < MLP_TILE * MLP_XS; i += 256) sh.x[i] = 0.0f;  // also the zero columns from 65 on
+    for (int i = tid; i < rows * E; i += 256) te_s[i] = end_only ? p.t_end[(b0 + i) * p.te_stride] : p.t_eval[b0 * E + i];
+    __syncthreads();
+
+    const T *tev = te_s + (live ? c : 0) * E;
+    const T dir = (te > ts) ? (T)1 : (T)-1, tlo = tmin(ts, te), thi = tmax(te, ts);
+    bool bail = false;
+    for (int e = 1; e < E; ++e) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));  // not monotone
     T t = ts, dt, prev = 1, pprev = 1;
     int cursor = 0, n_steps = 0, n_acc = 0;
 
@@ -546,15 +549,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
 
     if (end_only && live && !idle_done) put(p.y_idle + bs * FR, y);  // the final state
-    if (w == 0 && q == 0) {
-        if (live) {
+    if (w == 0) {
+        if (q == 0 && live) {
             o.n_steps[bs] = n_steps;
             o.n_accepted[bs] = n_acc;
             o.n_initialized[bs] = cursor;
             o.status[bs] = 0;
-            if (n_steps > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], n_steps);
         }
-        if (bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);
+        // one update of each flag word per workgroup: four thousand atomic operations on one address would queue up
+        // behind each other at the end of a kernel whose workgroups all finish together
+        int most = live ? n_steps : 0;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) most = max(most, __shfl_xor(most, off));
+        if (lane == 0) {
+            if (most > 0) atomicMax(&p.flags[TODE_FLAG_MAX_ITERATIONS], most);
+            if (bail) atomicMax(&p.flags[TODE_FLAG_NEEDS_GENERAL], 1);  // (agreed on by the workgroup's last vote)
+        }
     }
     publish_flags(p);
 }
