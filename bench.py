@@ -256,7 +256,6 @@ def main():
                     help="measure this configuration alone (default: the headline, Van der Pol float32, and then every other one under 'configs')")  # fmt: skip
     ap.add_argument("--dtype", default=None, choices=[None, "f32", "f64"])
     ap.add_argument("--batch", type=int, default=None, help="prefix of the workload's batch (default: full size)")
-    ap.add_argument("--fast-variant", type=int, default=0, choices=[0, 1, 2, 3], help="tode_set_fast_kernel_variant: 0 automatic, 1 one wavefront per 64 samples, 2 two wavefronts, 3 one wavefront that stores its evaluation points four at a time")
     ap.add_argument("--batch-copies", type=int, default=1, help="mlp workload: solve this many copies of the batch at once (B = 4096 x copies), to see the kernel with more than one workgroup per compute unit")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-compiled-baseline", action="store_true", help="skip the torch.compile CPU legs (about a minute of compilation each)")
@@ -293,10 +292,6 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    if args.fast_variant:
-        from torchode_amd import _lib
-
-        _lib.set_fast_kernel_variant(args.fast_variant)
     if args.gradient:
         print(json.dumps(measure_gradient(args, steps=args.steps if args.steps != 50 else 10)))
         return

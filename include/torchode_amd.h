@@ -505,14 +505,11 @@ int tode_step_stats(const tode_step_state *state, int64_t *out_n_steps, int64_t 
                     int64_t *out_status, void *stream);
 
 /*
- * Which kernel tode_solve_builtin_fast launches (per host thread); no counterpart in the
- * reference.  0 (default): two wavefronts per 64 samples (a stepper and a dense-output
- * evaluator) while the batch would otherwise leave SIMDs with at most two wavefronts, one
- * wavefront per 64 samples above that; 1: always one wavefront; 2: two wavefronts or
- * TODE_E_UNSUPPORTED; 3: one wavefront that, where the whole dense output of its 64 samples does not fit into LDS,
- * keeps four evaluation points per sample there and stores them together (16-byte stores of complete 4 F values
- * instead of F values per point at the stride of a row: about half the bytes written to HBM on the Lorenz
- * configuration, 4 % more time).  All variants produce identical bits.
+ * Which of its two kernels for the small systems tode_solve_builtin_fast launches (per host thread); no counterpart
+ * in the reference.  A hook for tests and profiles, which have to address each kernel on inputs of their choice.
+ * 0 (default): two wavefronts per 64 samples (a stepper and a dense-output evaluator) while the batch would
+ * otherwise leave SIMDs with at most two wavefronts, one wavefront per 64 samples above that; 1: always one
+ * wavefront; 2: two wavefronts or TODE_E_UNSUPPORTED.  Both kernels produce identical bits.
  */
 int tode_set_fast_kernel_variant(int variant);
 

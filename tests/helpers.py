@@ -26,11 +26,10 @@ def gpu_solve(f, y0, t_eval, method, controller, *, t_start=None, t_end=None, dt
     mv = lambda x: None if x is None else x.to(dev)
     solver = to.AutoDiffAdjoint(make_method(method), make_controller(controller, **ctrl_extra), max_steps=max_steps)
     solver.use_fast_path = bool(fast)
-    # fast=True: automatic choice; fast="one" / "two": force the one- / two-wavefront fast kernel; "sliced": the
-    # one-wavefront kernel storing its evaluation points four at a time
+    # fast=True: automatic choice; fast="one" / "two": force the one- / two-wavefront fast kernel
     from torchode_amd import _lib
 
-    _lib.set_fast_kernel_variant({True: 0, False: 0, "one": 1, "two": 2, "sliced": 3}[fast])
+    _lib.set_fast_kernel_variant({True: 0, False: 0, "one": 1, "two": 2}[fast])
     problem = to.InitialValueProblem(mv(y0), mv(t_start), mv(t_end), mv(t_eval))
     try:
         return solver.solve(problem, to.ODETerm(copy.deepcopy(f).to(dev)), dt0=mv(dt0))

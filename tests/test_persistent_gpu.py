@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 F32, F64 = torch.float32, torch.float64
 
 
-@pytest.mark.parametrize("fast", ["one", "two", "sliced", False], ids=["fast1", "fast2", "fast1-sliced", "general"])
+@pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])
 @pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
 @pytest.mark.parametrize("name,batch", [("linear_decay", 256), ("vdp", 4096), ("lorenz", 4096)])
 def test_workload_matches_oracle_bit_for_bit(name, batch, dtype, fast):
@@ -411,7 +411,7 @@ import os  # noqa: E402
 _GOLDEN = sorted(p for p in glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.json")) if not p.endswith(("_tolerance.json", "_mixed.json", "_fixed.json", "_low_order.json", "_early_stop.json")))
 
 
-@pytest.mark.parametrize("fast", ["one", "two", "sliced", False], ids=["fast1", "fast2", "fast1-sliced", "general"])
+@pytest.mark.parametrize("fast", ["one", "two", False], ids=["fast1", "fast2", "general"])
 @pytest.mark.parametrize("path", _GOLDEN, ids=os.path.basename)
 def test_gpu_matches_golden_fixture(path, fast):
     """Golden vectors of the ATen-op restatement, written in the authoring container."""
@@ -682,7 +682,7 @@ def test_random_configurations_match_oracle_bit_for_bit(seed):
         assert_identical(gpu_solve(f, y0, t_eval, method, controller, fast=fast, **kw), ref)
 
 
-@pytest.mark.parametrize("fast", ["one", "two", "sliced"])
+@pytest.mark.parametrize("fast", ["one", "two"])
 @pytest.mark.parametrize("dtype", [F32, F64], ids=["f32", "f64"])
 @pytest.mark.parametrize("name", ["vdp", "lorenz", "linear_decay", "linear_decay-backwards"])
 def test_samples_that_land_past_t_end_stay_in_the_fast_kernels(name, dtype, fast):
@@ -844,36 +844,6 @@ def test_mixed_dtypes_whole_solve_kernel_equals_the_per_step_kernels(case, time_
         assert (whole.status != 0).any()
     elif case != "empty":
         assert (whole.status == 0).all() and int(whole.stats["n_steps"].max()) > 10
-
-
-@pytest.mark.parametrize("case", ["lorenz-f32-64-points", "vdp-f64-50-points", "lorenz-f32-41-points", "lorenz-f32-ragged-batch"])
-def test_one_wavefront_kernel_storing_its_points_four_at_a_time(case):
-    """Variant 3 of the fast kernel where the whole dense output of a wavefront's samples does not fit into LDS: four
-    points per sample wait there and leave as 16-byte stores.  Against the C oracle, bit for bit; with 41 points of three
-    values a row does not start at a multiple of 16 bytes and the kernel stores point by point as variant 1 does."""
-    name, dtype, E, B = {"lorenz-f32-64-points": ("lorenz", F32, 64, 300), "vdp-f64-50-points": ("vdp", F64, 50, 300),
-                         "lorenz-f32-41-points": ("lorenz", F32, 41, 130), "lorenz-f32-ragged-batch": ("lorenz", F32, 60, 77)}[case]  # fmt: skip
-    w = to.workloads.make(name, batch=B, dtype=dtype)
-    span = w.t_eval[:, -1:] - w.t_eval[:, :1]
-    t_eval = w.t_eval[:, :1] + span * torch.linspace(0, 1, E, dtype=dtype)[None, :]
-    if case == "lorenz-f32-ragged-batch":
-        t_eval[::3, 0] += 0.01  # (a first point after t_start: those samples' rows fill from slot 0, the others' from slot 1)
-        t_start, t_end = w.t_eval[:, 0].clone(), t_eval[:, -1].clone()
-    else:
-        t_start = t_end = None
-    ref = c_oracle_solve(w.f, w.y0, t_eval, w.method, w.controller, t_start=t_start, t_end=t_end)
-    from torchode_amd import _lib
-
-    _lib.set_kernel_timing(True)
-    try:
-        for fast in ("sliced", "one"):
-            sol = gpu_solve(w.f, w.y0, t_eval, w.method, w.controller, t_start=t_start, t_end=t_end, fast=fast)
-            assert_identical(sol, ref)
-            assert (sol.status == 0).all() and (sol.stats["n_initialized"] == E).all()
-            four_at_a_time = fast == "sliced" and case != "lorenz-f32-41-points"
-            assert _lib.last_solve_kernel_name() == "tode::solve_fast_kernel" + (" (points stored four at a time)" if four_at_a_time else "")
-    finally:
-        _lib.set_kernel_timing(False)
 
 
 def test_outputs_of_more_than_two_to_the_31_values():

@@ -70,7 +70,7 @@ def span_case(seed):
 def test_spans_across_zero_through_every_whole_solve_dispatch(seed):
     f, y0, t_eval, method, ctrl, kw = span_case(seed)
     ref = c_oracle_solve(f, y0, t_eval, method, ctrl, **kw)
-    for fast in (True, "one", "two", "sliced", False):
+    for fast in (True, "one", "two", False):
         assert_identical(gpu_solve(f, y0, t_eval, method, ctrl, fast=fast, **kw), ref)
 
 

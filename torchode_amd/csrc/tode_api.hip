@@ -29,7 +29,6 @@ int check_hip(hipError_t err, const char *what) {
 }
 
 static thread_local int g_fast_variant = 0;
-bool fast_output_sliced() { return g_fast_variant == 3; }
 static thread_local bool g_timing = false;
 static thread_local bool g_timed = false;
 static thread_local hipEvent_t g_ev[2] = {nullptr, nullptr};
@@ -225,8 +224,7 @@ const char *tode_source_hash(void) { return TODE_SOURCE_HASH; }
 const char *tode_last_error(void) { return tode::g_error; }
 
 int tode_set_fast_kernel_variant(int variant) {
-    if (variant < 0 || variant > 3)
-        return tode::fail(TODE_E_INVALID, "variant must be 0 (auto), 1 (one wavefront), 2 (two wavefronts) or 3 (one wavefront, evaluation points stored four at a time)");
+    if (variant < 0 || variant > 2) return tode::fail(TODE_E_INVALID, "variant must be 0 (automatic), 1 (one wavefront per 64 samples) or 2 (two wavefronts)");
     tode::g_fast_variant = variant;
     return TODE_OK;
 }

@@ -30,10 +30,7 @@ template <typename T> struct FastOut {
 // RECORD: the loop state before every iteration of the wavefront goes to p.rec_* (tode_solve_record), as the general
 // kernel writes it: entry i is the state before iteration i; a sample that has finished repeats its last state with
 // `running` 0, up to the record's capacity.  A record that is too short raises TODE_FLAG_NEEDS_GENERAL.
-// SLICED (without STAGE_YS): a lane's evaluation points go to memory four at a time -- three more wait in LDS -- as
-// 16-byte stores of 4 F values in a row, instead of F values per point at a stride of the whole row, which leaves
-// every line the lanes touch partly written.
-template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_YS, bool RECORD = false, bool SLICED = false>
+template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_YS, bool RECORD = false>
 __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, const FastOut<T> o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
@@ -50,26 +47,7 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
     const int EF = E * F;
 
     T *te_s = reinterpret_cast<T *>(smem_raw);  // [E][64]
-    T *ys_s = te_s + (size_t)E * 64;            // [E*F][65] when STAGE_YS; [4*F][64] when SLICED
-    // (SLICED) point number `at` of this lane is complete: the four points that end with it leave LDS for memory
-    auto store_point = [&](T *row, int at, const T (&value)[F]) {
-#pragma unroll
-        for (int f = 0; f < F; ++f) ys_s[((at & 3) * F + f) * 64 + lane] = value[f];
-        if ((at & 3) == 3 && live) {
-            constexpr int PER = 16 / sizeof(T);  // values per 16-byte store
-            T *dst = row + (at - 3) * F;
-#pragma unroll
-            for (int j = 0; j < 4 * F; j += PER) {
-                T part[PER];
-#pragma unroll
-                for (int i = 0; i < PER; ++i) part[i] = ys_s[(j + i) * 64 + lane];
-                if (PER == 4)
-                    *reinterpret_cast<float4 *>(dst + j) = *reinterpret_cast<const float4 *>(part);
-                else
-                    *reinterpret_cast<double2 *>(dst + j) = *reinterpret_cast<const double2 *>(part);
-            }
-        }
-    };
+    T *ys_s = te_s + (size_t)E * 64;            // [E*F][65] when STAGE_YS
 
     // ---- stage this wave's block of t_eval (rows * E contiguous values) into LDS ----
     {
@@ -122,16 +100,12 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
     int cursor = 0;
     T *ys_g = p.ys + bs * (long long)EF;
     if (te_s[lane] == ts) {
-        if (SLICED) {
-            store_point(ys_g, 0, y);
-        } else {
 #pragma unroll
-            for (int f = 0; f < F; ++f) {
-                if (STAGE_YS)
-                    ys_s[f * 65 + lane] = y[f];
-                else if (live)
-                    ys_g[f] = y[f];
-            }
+        for (int f = 0; f < F; ++f) {
+            if (STAGE_YS)
+                ys_s[f * 65 + lane] = y[f];
+            else if (live)
+                ys_g[f] = y[f];
         }
         cursor = 1;
     }
@@ -231,16 +205,12 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
                 T out[F];
                 quartic_eval<T, F>(q, t0, dt, dir * dte_next, out);
                 if (hit) {
-                    if (SLICED) {
-                        store_point(ys_g, cursor, out);
-                    } else {
 #pragma unroll
-                        for (int f = 0; f < F; ++f) {
-                            if (STAGE_YS)
-                                ys_s[(cursor * F + f) * 65 + lane] = out[f];
-                            else
-                                ys_g[cursor * F + f] = out[f];
-                        }
+                    for (int f = 0; f < F; ++f) {
+                        if (STAGE_YS)
+                            ys_s[(cursor * F + f) * 65 + lane] = out[f];
+                        else
+                            ys_g[cursor * F + f] = out[f];
                     }
                 }
                 cursor += hit ? 1 : 0;
@@ -291,10 +261,6 @@ __global__ void __launch_bounds__(64) solve_fast_kernel(const SolveParams<T> p, 
         o.n_accepted[b] = n_acc;
         o.n_initialized[b] = cursor;
         o.status[b] = 0;
-    }
-    if (SLICED && live) {  // the points of a last, incomplete group of four
-        const int left = cursor & 3;
-        for (int j = 0; j < left * F; ++j) ys_g[(cursor - left) * F + j] = ys_s[j * 64 + lane];
     }
     if (RECORD) {  // the state every sample is left in, for every later iteration of the batch
         for (long long at = iteration; at < p.rec_capacity; ++at) keep(at, false);
@@ -364,19 +330,10 @@ static int launch_fast(const tode_solve_args &a, const tode_controller &c, const
             return fail(TODE_E_INVALID, "tode_solve_record: capacity %lld, or a null array", (long long)r.capacity);
     }
     const bool stage = !RECORD && need_all <= budget;  // (the recording variant is built without the staged output)
-    // four points of every lane in LDS: where the whole output does not fit, each row starts at a multiple of 16 bytes
-    // and there is room for the slices
-    const size_t need_slices = need_te + (size_t)4 * Term::F * 64 * sizeof(T);
-    const bool sliced = !RECORD && !stage && fast_output_sliced() && ((size_t)a.n_eval * Term::F * sizeof(T)) % 16 == 0 && (reinterpret_cast<uintptr_t>(a.ys) % 16) == 0 &&
-                        need_slices <= 64 * 1024;
-    const size_t lds = stage ? need_all : (sliced ? need_slices : need_te);
+    const size_t lds = stage ? need_all : need_te;
     const dim3 grid((unsigned)blocks), block(64);
-    timing_before(stream, sliced ? "tode::solve_fast_kernel (points stored four at a time)" : "tode::solve_fast_kernel");
-#define TODE_FAST_LAUNCH(NH, ST)                                                                                                          \
-    do {                                                                                                                                  \
-        if (sliced) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, false, false, !RECORD>), grid, block, lds, stream, p, o); \
-        else hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, (ST) && !RECORD, RECORD, false>), grid, block, lds, stream, p, o); \
-    } while (0)
+    timing_before(stream, "tode::solve_fast_kernel");
+#define TODE_FAST_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_fast_kernel<T, METHOD, CTRL, NH, Term, (ST) && !RECORD, RECORD>), grid, block, lds, stream, p, o)
     if (nhist == 0) {
         if (stage) TODE_FAST_LAUNCH(0, true); else TODE_FAST_LAUNCH(0, false);
     } else if (nhist == 1) {

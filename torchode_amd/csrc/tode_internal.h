@@ -57,8 +57,6 @@ struct FlagTarget {
 };
 const FlagTarget *flag_target();
 
-// tode_set_fast_kernel_variant(3) on this thread: the one-wavefront kernel writes its evaluation points in slices of four.
-bool fast_output_sliced();
 
 // Event pair around the solve kernel, active only while timing is enabled on this thread.
 void timing_before(hipStream_t s, const char *kernel_name);
