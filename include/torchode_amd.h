@@ -126,8 +126,9 @@ typedef struct tode_controller {
  */
 /*
  * Optional record of the loop state, written by tode_solve_builtin (the general kernel) and, for the three small
- * systems with evaluation points, by tode_solve_builtin_fast and its _sync / _static forms (the single-wavefront
- * kernel: the solve and its record in one launch) when tode_solve_args.record points to one: entry i holds what the reference's loop variables hold before iteration i
+ * systems with evaluation points, by tode_solve_builtin_fast and its _sync / _static forms (the two-wavefront or the
+ * single-wavefront kernel: the solve and its record in one launch) when tode_solve_args.record points to one: entry i
+ * holds what the reference's loop variables hold before iteration i
  * (adjoints.py:135-260: t, dt, y, the first-same-as-last derivative, the PID controller's two previous error
  * ratios, `running`, `n_accepted`), entry n_steps[b] the sample's final state, and the entries after it that final
  * state again with running = 0 -- a finished sample keeps its state while the batch goes on.  It is what a reverse

@@ -650,14 +650,26 @@ def test_record_of_the_whole_solve_kernel_equals_the_per_step_record(case):
     # The same solver again: it now knows how many entries such a record takes, and where the batch is in the
     # single-wavefront kernel's case that kernel writes the solve and the record in one launch (no flag words left
     # behind by a second pass).  Then with a record sized far too short, which sends it the long way again.
+    # Both kernels that can do so are asked: the two-wavefront kernel's stepper (the choice for a batch of this size) and
+    # the single-wavefront kernel.
+    from torchode_amd import _lib
+
     in_one_kernel_case = case in ("vdp-f32", "vdp-f64", "lorenz-f32", "linear-decay-f64", "dt0", "backwards")
-    for entries, one_kernel in ((None, in_one_kernel_case), (3, False)):
-        if entries is not None:
-            solver._record_entries = {shape: entries for shape in solver._record_entries}
+    # (its hand-over records of four float64 features do not fit the LDS share of a workgroup: the other kernel's case)
+    two_wavefronts = in_one_kernel_case and case != "linear-decay-f64"
+    known = dict(solver._record_entries)
+    for variant, entries, one_kernel in ((0, None, in_one_kernel_case), (1, None, in_one_kernel_case), (2, None, two_wavefronts), (0, 3, False)):
+        solver._record_entries = dict(known) if entries is None else {shape: entries for shape in known}
         again = LoopRecord()
-        with torch.no_grad():
-            sol_again = solver._solve_persistent(problem, to.ODETerm(f), dt0, record=again)
-        assert (again.flags is None) == one_kernel, (entries, again.flags)
+        _lib.set_fast_kernel_variant(variant)
+        try:
+            with torch.no_grad():
+                sol_again = solver._solve_persistent(problem, to.ODETerm(f), dt0, record=again)
+        finally:
+            _lib.set_fast_kernel_variant(0)
+        assert (again.flags is None) == one_kernel, (variant, entries, again.flags)
+        if one_kernel:
+            assert _lib.last_solve_kernel_name() == ("tode::solve_pair_kernel" if variant != 1 and two_wavefronts else "tode::solve_fast_kernel"), variant
         assert again.iterations == steps.iterations
         E_ = sol_whole.ys.shape[1]
         written = (torch.arange(E_, device="cuda")[None, :] < sol_whole.stats["n_initialized"][:, None])[:, :, None] if t_eval is not None else True

@@ -699,7 +699,7 @@ class AutoDiffAdjoint(nn.Module):
         return fields, _lib.SolveRecord(n, *(fields[k].data_ptr() for k in ("t", "dt", "y", "k0", "prev", "pprev", "running", "n_accepted")))
 
     def _solve_recording_in_one_kernel(self, lib, a, ctrl, out, stream, record, q) -> Optional[Solution]:
-        """The solve with its record from the single-wavefront kernel (``tode_solve_builtin_fast`` with a record), or
+        """The solve with its record from one launch of a fast kernel (``tode_solve_builtin_fast`` with a record), or
         None where that is not to be had: no earlier recording solve to size the record from, a shape or controller
         setting outside that kernel's case, a batch that leaves it, or a record that came out too short."""
         shape = (q["B"], q["F"], q["E"], q["dtype"], a.term)

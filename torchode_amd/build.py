@@ -51,6 +51,8 @@ UNITS = [
     ("tode_fast.hip", "tode_fast_f64_record.o", ["-DTODE_INSTANTIATE_F64=1", "-DTODE_INSTANTIATE_RECORD=1"]),
     ("tode_pair.hip", "tode_pair_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_pair.hip", "tode_pair_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),
+    ("tode_pair.hip", "tode_pair_f32_record.o", ["-DTODE_INSTANTIATE_F32=1", "-DTODE_INSTANTIATE_RECORD=1"]),
+    ("tode_pair.hip", "tode_pair_f64_record.o", ["-DTODE_INSTANTIATE_F64=1", "-DTODE_INSTANTIATE_RECORD=1"]),
     ("tode_stepwise.hip", "tode_stepwise.o", []),
     ("tode_backward.hip", "tode_backward_f32.o", ["-DTODE_INSTANTIATE_F32=1"]),
     ("tode_backward.hip", "tode_backward_f64.o", ["-DTODE_INSTANTIATE_F64=1"]),

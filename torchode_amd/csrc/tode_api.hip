@@ -300,8 +300,15 @@ int tode_solve_builtin_fast(const tode_solve_args *a, const tode_controller *c, 
         if (a->dtype != TODE_F32) return fail(TODE_E_UNSUPPORTED, "the MLP kernel is built for float32");
         return solve_mlp_f32(*a, *c, ns, na, ni, st, s);
     }
-    if (a->record) {  // the solve and the record of its loop state in one kernel: the single-wavefront kernel writes it
+    if (a->record) {  // the solve and the record of its loop state in one kernel: the stepper of the two-wavefront kernel
+                      // writes it for small batches, the single-wavefront kernel otherwise
         if (end_only) return fail(TODE_E_UNSUPPORTED, "a record from the fast entry point needs evaluation points");
+        if (g_fast_variant == 0 || g_fast_variant == 2) {
+            bool used = false;
+            int rc = a->dtype == TODE_F32 ? solve_pair_f32_record(*a, *c, ns, na, ni, st, s, &used) : solve_pair_f64_record(*a, *c, ns, na, ni, st, s, &used);
+            if (rc || used) return rc;
+            if (g_fast_variant == 2) return fail(TODE_E_UNSUPPORTED, "the two-wavefront kernel does not cover this problem size");
+        }
         return a->dtype == TODE_F32 ? solve_fast_f32_record(*a, *c, ns, na, ni, st, s) : solve_fast_f64_record(*a, *c, ns, na, ni, st, s);
     }
     if (g_fast_variant == 0 || g_fast_variant == 2) {

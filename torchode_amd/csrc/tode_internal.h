@@ -73,6 +73,8 @@ int solve_builtin_t32_y64_record(const tode_solve_args &a, const tode_controller
 int solve_fast_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 int solve_pair_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
 int solve_pair_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
+int solve_pair_f32_record(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
+int solve_pair_f64_record(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used);
 int solve_mlp_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);
 int mlp_pack_weights(const float *raw, long long n_raw, int n_features, int matrix_inputs, float *packed, hipStream_t s);
 int solve_grid_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s);

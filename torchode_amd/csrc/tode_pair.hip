@@ -19,6 +19,9 @@
 //
 // Same arithmetic, bit for bit, and same contract as tode_fast.hip
 // (TODE_FLAG_NEEDS_GENERAL when the batch leaves the common case).
+//
+// RECORD: the stepper also writes the loop state before every iteration to p.rec_* (tode_solve_record), as
+// tode_fast.hip's recording variant does, for the reverse sweep of a differentiable solve.
 #include "tode_solve.h"
 
 namespace tode {
@@ -27,7 +30,7 @@ template <typename T> struct PairOut {
     int64_t *n_steps, *n_accepted, *n_initialized, *status;
 };
 
-template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_TE>
+template <typename T, int METHOD, int CTRL, int NHIST, typename Term, bool STAGE_TE, bool RECORD = false>
 __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p, const PairOut<T> o) {
     using Tab = typename std::conditional<METHOD == 1, Tsit5Tab, Dopri5Tab>::type;
     constexpr int F = Term::F;
@@ -89,14 +92,33 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
         const int step_limit = p.max_steps < TODE_HARD_STEP_LIMIT ? p.max_steps : TODE_HARD_STEP_LIMIT;
         const T e1 = (T)cp.e1, e2 = (T)cp.e2, e3 = (T)cp.e3;
 
+        // (RECORD) the last two accepted error ratios as values (the step factor keeps their logarithms)
+        T ratio_prev = 1, ratio_prev_prev = 1;
+        bool record_full = false;
+        auto keep = [&](long long at, bool running) {
+            if (at >= p.rec_capacity) {
+                record_full = true;
+                return;
+            }
+            if (!live) return;
+            const long long i = at * p.batch + b;
+            p.rec_t[i] = t, p.rec_dt[i] = dt;
+#pragma unroll
+            for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k[0][f];
+            p.rec_prev[i] = ratio_prev, p.rec_pprev[i] = ratio_prev_prev;
+            p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
+        };
+
         // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's
         // later iterations with the clamped step t_end - t: with evaluation points that is seen only in the status of
         // that step, a success unless its error ratio is not finite.  The sample sits through one more iteration here,
         // as an inactive lane whose error ratio is looked at.
         bool idle = false;
-        for (int phase = 0;; ++phase) {
+        int phase = 0;
+        for (;; ++phase) {
             const bool any = __any(active || idle);
             if (any) {
+                if (RECORD) keep(phase, active);
                 // ---- stages (runge_kutta.py:255-263) ----
                 const T t0 = t;
                 T y1[F], err[F];
@@ -168,6 +190,11 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                     dt = active ? dtc : dt;
                 }
                 if (NHIST >= 1) step_factor.shift(active && running_new && accept);
+                if (RECORD && CTRL == 1) {
+                    const bool shift = active && running_new && accept;
+                    ratio_prev_prev = shift ? ratio_prev : ratio_prev_prev;
+                    ratio_prev = shift ? ratio : ratio_prev;
+                }
                 {
                     const bool failed = active && (!sane || n_steps >= step_limit);
                     const bool finished = active && !failed && !running_new;
@@ -191,6 +218,11 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
             if (!any) break;
         }
 
+        if (RECORD) {  // the state every sample is left in, for every later iteration of the batch
+            for (long long at = phase; at < p.rec_capacity; ++at) keep(at, false);
+            if (phase >= p.rec_capacity) record_full = true;
+            bail = bail || record_full;
+        }
         if (live) {
             o.n_steps[b] = n_steps;
             o.n_accepted[b] = n_acc;
@@ -310,13 +342,15 @@ static int launch_pair(const tode_solve_args &a, const tode_controller &c, const
     if (rec_bytes > budget) return TODE_OK;
     const bool stage_te = rec_bytes + te_bytes <= budget;
     const size_t lds = rec_bytes + (stage_te ? te_bytes : 0);
+    constexpr bool RECORD = TODE_INSTANTIATE_RECORD != 0;
+    if (RECORD != (a.record != nullptr)) return fail(TODE_E_INVALID, "internal: record variant mismatch");
     SolveParams<T> p = make_params<T>(a, c);
     if (p.cp.shortcut_exponent()) return TODE_OK;  // left to the caller's other kernels
     const int nhist = CTRL == 0 ? 0 : (p.cp.skip3 ? 1 : 2);
     const dim3 grid((unsigned)blocks), block(128);
     reset_flags(a.flags, stream);
     timing_before(stream, "tode::solve_pair_kernel");
-#define TODE_PAIR_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_pair_kernel<T, METHOD, CTRL, NH, Term, ST>), grid, block, lds, stream, p, o)
+#define TODE_PAIR_LAUNCH(NH, ST) hipLaunchKernelGGL((solve_pair_kernel<T, METHOD, CTRL, NH, Term, ST, RECORD>), grid, block, lds, stream, p, o)
     if (nhist == 0) {
         if (stage_te) TODE_PAIR_LAUNCH(0, true); else TODE_PAIR_LAUNCH(0, false);
     } else if (nhist == 1) {
@@ -368,13 +402,19 @@ static int pair_term(const tode_solve_args &a, const tode_controller &c, int64_t
     }
 }
 
+// (each translation unit instantiates one type, with or without the record: TODE_INSTANTIATE_RECORD)
+#if TODE_INSTANTIATE_RECORD
+#define TODE_PAIR_ENTRY(name) name##_record
+#else
+#define TODE_PAIR_ENTRY(name) name
+#endif
 #if TODE_INSTANTIATE_F32
-int solve_pair_f32(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used) {
+int TODE_PAIR_ENTRY(solve_pair_f32)(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used) {
     return pair_term<float>(a, c, ns, na, ni, st, s, used);
 }
 #endif
 #if TODE_INSTANTIATE_F64
-int solve_pair_f64(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used) {
+int TODE_PAIR_ENTRY(solve_pair_f64)(const tode_solve_args &a, const tode_controller &c, int64_t *ns, int64_t *na, int64_t *ni, int64_t *st, hipStream_t s, bool *used) {
     return pair_term<double>(a, c, ns, na, ni, st, s, used);
 }
 #endif
