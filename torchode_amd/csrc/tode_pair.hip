@@ -101,12 +101,7 @@ __global__ void __launch_bounds__(128) solve_pair_kernel(const SolveParams<T> p,
                 return;
             }
             if (!live) return;
-            const long long i = at * p.batch + b;
-            p.rec_t[i] = t, p.rec_dt[i] = dt;
-#pragma unroll
-            for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k[0][f];
-            p.rec_prev[i] = ratio_prev, p.rec_pprev[i] = ratio_prev_prev;
-            p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
+            record_entry<T, T, F>(p, at, b, t, dt, y, k[0], ratio_prev, ratio_prev_prev, running, n_acc);
         };
 
         // A sample that has landed past t_end (t + (t_end - t) rounded upwards) keeps stepping in the reference's

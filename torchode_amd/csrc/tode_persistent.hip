@@ -96,12 +96,7 @@ __global__ void __launch_bounds__(TODE_BLOCK) solve_kernel(const SolveParams<T, 
                 my_overflow = 1;
                 return;
             }
-            const long long i = at * p.batch + b;
-            p.rec_t[i] = t, p.rec_dt[i] = dt;
-#pragma unroll
-            for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k[0][f];
-            p.rec_prev[i] = prev, p.rec_pprev[i] = prev_prev;
-            p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_acc;
+            record_entry<T, TT, F>(p, at, b, t, dt, y, k[0], prev, prev_prev, running, n_acc);
         };
         while (go) {
             if (RECORD && !idle_pass) keep(n_steps, true);

@@ -114,6 +114,19 @@ template <typename T, typename TT = T> struct SolveParams {
     int32_t *rec_running, *rec_n_accepted;
 };
 
+// Entry `at` of the record of the loop state (tode_solve_record) for sample b: what the reference's loop variables hold
+// before that iteration (adjoints.py:135-260).  The caller has checked at < p.rec_capacity.
+template <typename T, typename TT, int F>
+__device__ __forceinline__ void record_entry(const SolveParams<T, TT> &p, long long at, long long b, TT t, TT dt, const T (&y)[F], const T (&k0)[F], T prev,
+                                             T prev_prev, bool running, int n_accepted) {
+    const long long i = at * p.batch + b;
+    p.rec_t[i] = t, p.rec_dt[i] = dt;
+#pragma unroll
+    for (int f = 0; f < F; ++f) p.rec_y[i * F + f] = y[f], p.rec_k0[i * F + f] = k0[f];
+    p.rec_prev[i] = prev, p.rec_pprev[i] = prev_prev;
+    p.rec_running[i] = running ? 1 : 0, p.rec_n_accepted[i] = n_accepted;
+}
+
 // Start step (step_size_controllers.py:431-490 integral, 776-835 PID; the integral
 // copy maps h0 == 0 to d2 = inf, the PID copy does not).
 template <typename T, int CTRL, typename Term>
