@@ -659,6 +659,7 @@ class SolveThroughLoop(torch.autograd.Function):
         # the times as the caller gave them: those that require grad are among `params`
         ctx.times = InitialValueProblem(plain.y0, problem.t_start, problem.t_end, problem.t_eval)
         ctx.record, ctx.params = record, params
+        ctx.n_initialized = solution.stats["n_initialized"]
         stats = solution.stats
         n_f_evals = stats["n_f_evals"] if "n_f_evals" in stats else torch.empty(0, dtype=torch.long)
         outs = (solution.ys, solution.status, stats["n_steps"], stats["n_accepted"], stats["n_initialized"], n_f_evals)
@@ -670,7 +671,9 @@ class SolveThroughLoop(torch.autograd.Function):
         adjoint, problem, term, params = ctx.adjoint, ctx.problem, ctx.term, list(ctx.params)
         if ctx.record.flags is not None and ctx.record.flags.tolist()[_lib.FLAG_NEEDS_GENERAL]:
             raise RuntimeError("the record of the loop state was too short for the solve it was sized from")
-        if problem.n_evaluation_points > 0 and not ctx.record.any_point_written(problem):
+        # (a second initialized point of some sample was written by an iteration: the usual case, told by one reduction)
+        some_iteration_wrote = problem.n_evaluation_points > 1 and int(ctx.n_initialized.max()) > 1
+        if problem.n_evaluation_points > 0 and not some_iteration_wrote and not ctx.record.any_point_written(problem):
             # No iteration wrote an evaluation point (every sample's points lie at t_start, or the batch stopped before
             # one was reached): ys is a copy of y0 where t_eval[:, 0] == t_start and nothing else, so in the reference's
             # graph no parameter and no time is connected to it: autograd reports them unused, not zero.
