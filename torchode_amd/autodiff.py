@@ -62,14 +62,27 @@ def captured_leaves(term, problem: InitialValueProblem, args) -> List[torch.Tens
     from them).  Found by evaluating ``f`` once on detached inputs under grad mode and walking the graph of the result.
     The reference's loop is torch operations throughout, so autograd reaches such tensors by itself
     (adjoints.py:135-260); here they have to be named as differentiation targets of the reverse sweep."""
-    with torch.enable_grad():
-        y = problem.y0.detach().requires_grad_()
-        t = problem.t_start.detach()
-        # (args reaches f by identity, reference tests/extra_args_test.py:16-22; only tensors in it that require
-        # grad are swapped for detached ones, so that the walk stops at them: the caller names those itself)
-        plain_args = map_tensors(args, lambda a: a.detach()) if any(a.requires_grad for a in tensor_leaves(args)) else args
-        out = term.f(t, y, plain_args) if term.with_args else term.f(t, y)
-    found, seen, stack = [], set(), [getattr(out, "grad_fn", None)]
+    from .builtin_terms import BuiltinTerm
+
+    f = getattr(term, "f", None)
+    found, y = [], None
+    plain_term = not term._parameters and not term._buffers and len(term._modules) == 1
+    if plain_term and isinstance(f, BuiltinTerm) and type(f).__module__ == BuiltinTerm.__module__ and not f._modules:
+        # a plain term around one of the library's built-in right-hand sides, which compute from their own buffers and
+        # parameters alone: the walk starts at those, without an evaluation of f
+        held = [x for x in list(f._buffers.values()) + list(f._parameters.values()) if x is not None and x.requires_grad]
+        found = [x for x in held if x.is_leaf]
+        stack = [x.grad_fn for x in held if not x.is_leaf]
+    else:
+        with torch.enable_grad():
+            y = problem.y0.detach().requires_grad_()
+            t = problem.t_start.detach()
+            # (args reaches f by identity, reference tests/extra_args_test.py:16-22; only tensors in it that require
+            # grad are swapped for detached ones, so that the walk stops at them: the caller names those itself)
+            plain_args = map_tensors(args, lambda a: a.detach()) if any(a.requires_grad for a in tensor_leaves(args)) else args
+            out = term.f(t, y, plain_args) if term.with_args else term.f(t, y)
+        stack = [getattr(out, "grad_fn", None)]
+    seen = set()
     while stack:
         fn = stack.pop()
         if fn is None or fn in seen:
