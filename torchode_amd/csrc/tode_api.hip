@@ -424,6 +424,14 @@ int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controll
     b.flags = words;
     if (end_only) b.y_idle = staging;
     const FlagTarget target = {words, flags_out, 0};
+    struct MarkUse {  // (whichever way the call leaves from here on: the work enqueued so far is the array's last use)
+        StaticUse &use;
+        hipStream_t s;
+        bool live;
+        ~MarkUse() {
+            if (live && hipEventRecord(use.done, s) == hipSuccess) use.stream = s, use.recorded = true;
+        }
+    } mark{use, s, live};
     hipLaunchKernelGGL(static_flags_reset_kernel, dim3(1), dim3(64), 0, s, words);
     g_flag_target = &target;
     rc = tode_solve_builtin_fast(&b, c, ns, na, ni, st, stream);
@@ -433,14 +441,6 @@ int tode_solve_builtin_fast_static(const tode_solve_args *a, const tode_controll
         hipLaunchKernelGGL(empty_flags_kernel, dim3(1), dim3(64), 0, s, flags_out);
         return check_hip(hipGetLastError(), "tode_solve_builtin_fast_static launch");
     }
-    struct MarkUse {  // (whichever way the call leaves from here on: the work enqueued so far is the array's last use)
-        StaticUse &use;
-        hipStream_t s;
-        bool live;
-        ~MarkUse() {
-            if (live && hipEventRecord(use.done, s) == hipSuccess) use.stream = s, use.recorded = true;
-        }
-    } mark{use, s, live};
     if (end_only) {
         const long long n = (long long)a->batch * a->n_features;
         const unsigned blocks = (unsigned)((n + 255) / 256);
