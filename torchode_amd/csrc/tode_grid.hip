@@ -36,6 +36,7 @@ template <typename T, int NW, int R> struct GridShared {
     T red[2][R][NW][2];      // chunk sums of up to two reductions, double buffered
     T xs[NW * 64];           // positions within the step of the evaluation points it passed (one per thread and round)
     int passed[NW];          // per wavefront: how many of its threads' candidate points the step passed
+    T handed;                // a scalar of the sample that one wavefront worked out for all (by_one_wavefront)
 };
 
 // Four consecutive values, moved with the widest loads and stores their alignment allows.
@@ -76,6 +77,19 @@ template <typename T, int NW, int R> __device__ __forceinline__ void block_sum2(
             B = B + sh.red[slot][r][w][1];
         }
     slot ^= 1;
+}
+
+// A scalar of the sample that takes hundreds of instructions (a power): worked out by the first wavefront alone and
+// handed round in LDS, where otherwise all NW wavefronts would work it out, four to a SIMD one after the other.  Same
+// arithmetic on the same operands: same bits.  (Between two uses lies at least one other barrier of the workgroup, so
+// nobody still reads the word when it is written again.)
+template <typename T, typename Compute> __device__ __forceinline__ T by_one_wavefront(T &word, Compute compute) {
+    if (threadIdx.x < 64) {
+        const T value = compute();
+        if (threadIdx.x == 0) word = value;
+    }
+    lds_barrier();
+    return word;
 }
 
 // du/dt = D * lap(u) + u * (1 - u) on the periodic grid; each operation rounds on its own, in the
@@ -141,8 +155,10 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
     for (int r = 0; r < R; ++r) load4<T>(p.y0 + b * F + r * BAND + 4 * tid, y[r]);
     __syncthreads();  // te_s
 
-    bool bail = false;
-    for (int e = 1; e < E; ++e) bail = bail || !(dir * te_s[e] >= dir * te_s[e - 1]);  // not monotone
+    // evaluation times that are not monotone in the sample's direction: each thread looks at its share of the neighbours
+    int disorder = 0;
+    for (int e = 1 + tid; e < E; e += NT) disorder |= !(dir * te_s[e] >= dir * te_s[e - 1]);
+    bool bail = __syncthreads_or(disorder) != 0;
 
     // ---- first step size (step_size_controllers.py:431-490, 776-835) ----
     T t = ts, dt;
@@ -184,7 +200,7 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
             }
         }
         block_sum2<T, NW, R>(sh, slot, a2, none, A2, unused);
-        dt = initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, h0, d1, sqrt_(A2));
+        dt = by_one_wavefront(sh.handed, [&] { return initial_finish<T>(CTRL == 1 ? TODE_CTRL_PID : TODE_CTRL_INTEGRAL, 1.0 / 5.0, dir, h0, d1, sqrt_(A2)); });
     }
     dt = tclamp(dt, tlo - t, thi - t);
 
@@ -243,7 +259,7 @@ __global__ void __launch_bounds__(N *N / 4 / grid_bands(N)) solve_grid_kernel(co
         block_sum2<T, NW, R>(sh, slot, part, none, total, unused);
         const T ratio = tmax(sqrt_(total), (T)1e-38);
         const bool accept = ratio < (T)1;
-        T dt_next = dt * dt_factor<T, CTRL>(cp, ratio, prev, pprev);
+        T dt_next = dt * by_one_wavefront(sh.handed, [&] { return dt_factor<T, CTRL>(cp, ratio, prev, pprev); });
         const int status = limit_dt<T>(cp, ratio, dt_next);
         if (idle) {
             bail = status != 0;

@@ -396,7 +396,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const T *tev = te_s + (live ? c : 0) * E;
     const T dir = (te > ts) ? (T)1 : (T)-1, tlo = tmin(ts, te), thi = tmax(te, ts);
     bool bail = false;
-    for (int e = 1; e < E; ++e) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));  // not monotone
+    // not monotone: the sixteen threads that share the sample (four lane groups in each of four wavefronts) split its
+    // neighbouring pairs among them; the workgroup's vote below collects what any of them found
+    for (int e = 1 + q + 4 * w; e < E; e += 16) bail = bail || (live && !(dir * tev[e] >= dir * tev[e - 1]));
     T t = ts, dt, prev = 1, pprev = 1;
     int cursor = 0, n_steps = 0, n_acc = 0;
 
