@@ -318,13 +318,15 @@ class Replay:
         elif self.dense_kind == "tsit5":
             q = [y0, h * ks[0], weighted(self.b_other[0]), weighted(self.b_other[1]), weighted(self.b_other[2])]
         else:
+            # (the reference's chains of add(alpha=...), interpolation.py:152-166: one rounding per term, so that where
+            # the terms cancel to the last unit the remainder is the forward pass's)
             f0, f1, mid = h * ks[0], h * ks[6], y0 + weighted(self.b_other[0])
             q = [
                 y0,
                 f0,
-                f1 - 4 * f0 - 11 * y0 - 5 * y1 + 16 * mid,
-                5 * f0 - 3 * f1 + 18 * y0 + 14 * y1 - 32 * mid,
-                2 * (f1 - f0) - 8 * (y1 + y0) + 16 * mid,
+                f1.add(f0, alpha=-4).add(y0, alpha=-11).add(y1, alpha=-5).add(mid, alpha=16),
+                (5 * f0).add(f1, alpha=-3).add(y0, alpha=18).add(y1, alpha=14).add(mid, alpha=-32),
+                (2 * (f1 - f0)).add(y1 + y0, alpha=-8).add(mid, alpha=16),
             ]
         den = (t0 + dt) - t0
         den = torch.where(den.abs() > 0, den, torch.ones_like(den))

@@ -192,9 +192,9 @@ def quartic_from_mid(dt, y0, y1, k_first, k_last, y_mid):
     return torch.stack((
         y0,
         f0,
-        f1 - 4 * f0 - 11 * y0 - 5 * y1 + 16 * y_mid,
-        5 * f0 - 3 * f1 + 18 * y0 + 14 * y1 - 32 * y_mid,
-        2 * (f1 - f0) - 8 * (y1 + y0) + 16 * y_mid,
+        f1.add(f0, alpha=-4).add(y0, alpha=-11).add(y1, alpha=-5).add(y_mid, alpha=16),
+        (5 * f0).add(f1, alpha=-3).add(y0, alpha=18).add(y1, alpha=14).add(y_mid, alpha=-32),
+        (2 * (f1 - f0)).add(y1 + y0, alpha=-8).add(y_mid, alpha=16),
     ))  # fmt: skip
 
 
