@@ -314,7 +314,7 @@ class Replay:
         weighted = lambda w: h * sum(w[s] * ks[s] for s in range(7) if w[s] != 0.0)
         if self.dense_kind == "cubic":  # Hermite cubic from the first and last slope, reference interpolation.py:84-106
             f0, f1, gap = ks[0], ks[-1], y0 - y1
-            q = [y0, h * f0, h * (-2 * f0 - f1) - 3 * gap, h * (f0 + f1) + 2 * gap]
+            q = [y0, h * f0, torch.add(h * torch.add(-f1, f0, alpha=-2), gap, alpha=-3), torch.add(h * (f0 + f1), gap, alpha=2)]
         elif self.dense_kind == "tsit5":
             q = [y0, h * ks[0], weighted(self.b_other[0]), weighted(self.b_other[1]), weighted(self.b_other[2])]
         else:

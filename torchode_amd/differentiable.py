@@ -210,8 +210,10 @@ def quartic_build(mid_weights: Optional[Sequence[float]], theta_weights: Optiona
 def cubic_build(dt, y0, y1, k_first, k_last):
     """reference interpolation.py:84-101: the Hermite cubic of a step."""
     h = dt.to(y0.dtype)[:, None]
-    f0, f1, gap = h * k_first, h * k_last, y0 - y1
-    return torch.stack((y0, f0, -2 * f0 - f1 - 3 * gap, f0 + f1 + 2 * gap))
+    gap = y0 - y1
+    cube = torch.add(h * (k_first + k_last), gap, alpha=2)
+    square = torch.add(h * torch.add(-k_last, k_first, alpha=-2), gap, alpha=-3)
+    return torch.stack((y0, h * k_first, square, cube))
 
 
 def poly_eval(span_is_dt: bool, idx: torch.Tensor, coefficients, t0, t1, t):
