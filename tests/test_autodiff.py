@@ -955,6 +955,57 @@ def test_separate_time_tensors_with_equal_values_get_their_own_gradients(control
     assert all(float(g.abs().max()) > 0 for g in results["operator-path"])
 
 
+class OwnDopri5ForTies(to.Dopri5):
+    """A user's subclass: the solve takes the operator path."""
+
+
+class TanhField(torch.nn.Module):
+    def __init__(self, n, generator):
+        super().__init__()
+        self.A = torch.nn.Parameter(torch.rand(n, n, generator=generator, dtype=torch.float64) - 0.5)
+        self.b = torch.nn.Parameter(torch.rand(n, generator=generator, dtype=torch.float64) - 0.5)
+
+    def forward(self, t, y):
+        return torch.tanh(y @ self.A.T + self.b) - 0.3 * y + 0.1 * torch.sin(t)[:, None]
+
+
+@gpu
+def test_a_last_step_of_one_unit_gives_every_pass_the_same_time_gradients():
+    """In some samples of this seeded batch t + (t_end - t) rounds to one unit in the last place below t_end, so the step
+    that was clamped to reach t_end is followed by a step of 2**-54, and that step writes the point at t_end: the
+    derivative of the point's position multiplies whatever remainder the step's dense-output coefficients carry by
+    2**54.  Dopri5's coefficients cancel to the last unit there (interpolation.py:152-166); a backward pass that does not
+    form them as the forward pass does, the reference's chains of add(alpha=...), puts a rounding term of opposite signs
+    on t_end and t_eval[:, -1] (two tensors here) -- 135.47 on sample 6 with the sums written out term by term."""
+    g = torch.Generator().manual_seed(6188)
+    u = lambda lo, hi, *shape: lo + (hi - lo) * torch.rand(*shape, generator=g, dtype=torch.float64)
+    B, F = 37, 8
+    f = TanhField(F, g).cuda()
+    sign = torch.where(torch.rand(B, generator=g) < 0.3, -1.0, 1.0).to(torch.float64)
+    t_start = u(-1, 1, B)
+    t_end = t_start + sign * u(0.3, 1.5, B)
+    t_eval = torch.stack((t_start, t_end), dim=1)
+    dt0 = u(0.01, 0.05, B) * sign
+    y_first = u(-1, 1, B, F)
+    results, short = {}, None
+    for sweep in ("kernels", "torch", "operator-path"):
+        y0 = y_first.cuda().requires_grad_()
+        leaves = [x.cuda().clone().requires_grad_() for x in (t_start, t_end, t_eval)]
+        solver = to.AutoDiffAdjoint(OwnDopri5ForTies() if sweep == "operator-path" else to.Dopri5(), to.IntegralController(1e-4, 1e-3),
+                                    backprop_through_step_size_control=False)  # fmt: skip
+        solver.backward_kernels = sweep == "kernels"
+        solution = solver.solve(to.InitialValueProblem(y0, *leaves), to.ODETerm(f), dt0=dt0.cuda())
+        weights = torch.linspace(0.5, 1.5, solution.ys[0].numel(), dtype=torch.double, device="cuda").reshape(1, 2, F)
+        results[sweep] = torch.autograd.grad((solution.ys * weights).sum(), [y0, f.A, f.b, *leaves])
+        if sweep != "operator-path":
+            assert autodiff.LAST_SWEEP == sweep
+        short = solution.stats["n_steps"]
+    assert short.min() >= 2 and short.max() == 4  # (the samples with a fourth step took it for one unit)
+    for sweep in ("kernels", "torch"):
+        for got, expected, which in zip(results[sweep], results["operator-path"], ("y0", "A", "b", "t_start", "t_end", "t_eval")):
+            torch.testing.assert_close(got, expected, rtol=1e-9, atol=1e-11 * float(expected.abs().max()), msg=f"{sweep}: {which}")
+
+
 @gpu
 def test_a_lone_evaluation_point_at_t_start_connects_nothing_but_y0():
     """t_eval = t_start[:, None]: ys is a copy of y0 (adjoints.py:121-126) and the loop writes nothing, so in the
